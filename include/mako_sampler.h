@@ -1,0 +1,124 @@
+/*
+ * mako_sampler.h -- C ABI of the MI355X token sampler.
+ *
+ * A batched, device-resident replacement for the reference's C++ class
+ * mako::gen::Sampler (src/gen/sampler.hpp:22-45): fp32 logits in, the
+ * SamplingParams fields, the accept() history, an optional allowed-token
+ * bitmask and one caller-supplied uniform per row in, sampled token ids out.
+ * Row r of a batch behaves exactly like a fresh reference Sampler with row r's
+ * parameters whose accept() was called once per history token and whose
+ * sample() (or verify()) is then called on row r's logits, with the uniform
+ * draws replaced by the caller's u (and u2).
+ *
+ * Every pointer inside mako_sample_desc is a DEVICE pointer; the host-pointer
+ * convenience call stages through context-owned buffers.  The library never
+ * writes the caller's logits, allocates nothing on the sampling path, and
+ * reports failures as negative status codes (the reference throws
+ * std::invalid_argument, src/gen/sampler.cpp:11-12).
+ */
+#ifndef MAKO_SAMPLER_H
+#define MAKO_SAMPLER_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MAKO_OK 0
+#define MAKO_ERR_INVALID_ARG (-1) /* null pointer, n_vocab == 0, sizes beyond the context's */
+#define MAKO_ERR_HIP (-2)         /* a HIP call failed; see mako_sampler_last_error */
+#define MAKO_ERR_NO_MEMORY (-3)
+
+/* Same fields, order, defaults and meaning as SamplingParams,
+ * src/gen/sampler.hpp:11-20 (28 bytes).  temperature <= 0 selects greedy. */
+typedef struct mako_sampling_params {
+    float temperature;
+    uint32_t top_k;
+    float top_p;
+    float min_p;
+    float presence_penalty;
+    float frequency_penalty;
+    float repetition_penalty;
+} mako_sampling_params;
+
+/* How a row was resolved (optional diagnostic output). */
+#define MAKO_PATH_GREEDY 1u   /* argmax of the (masked) raw logits */
+#define MAKO_PATH_FALLBACK 2u /* no candidate survived: most likely token (sampler.cpp:37-38) */
+#define MAKO_PATH_TOPK 3u     /* resolved from the per-slice top-k candidates */
+#define MAKO_PATH_NUCLEUS 4u  /* top_k == 0: nucleus resolved from the per-slice candidates */
+#define MAKO_PATH_GENERAL 5u  /* whole-row sort path */
+
+typedef struct mako_sample_desc {
+    /* ---- inputs (device pointers) ---- */
+    const float* logits;     /* [n_rows][logits_stride], fp32; read-only (sampler.hpp:27 `const float*`) */
+    int64_t logits_stride;   /* elements between rows, >= n_vocab */
+    uint32_t n_rows;
+    uint32_t n_vocab;        /* > 0 (sampler.cpp:11) */
+    const mako_sampling_params* params; /* [n_rows] */
+    const float* u;          /* [n_rows] uniforms in [0,1): the draw of sampler.cpp:66, or of :100 when verifying */
+    const uint32_t* mask;    /* optional [n_rows][mask_stride]: bit (i & 31) of word i >> 5 set = token i allowed;
+                                a cleared bit makes the logit -inf before anything else (no reference counterpart) */
+    int64_t mask_stride;     /* 32-bit words between rows, >= ceil(n_vocab / 32) */
+    const int32_t* hist_tokens; /* optional [n_rows][hist_stride]: the tokens passed to accept(), sampler.cpp:15-18;
+                                   ids outside [0, n_vocab) are ignored */
+    const uint32_t* hist_counts; /* optional, same shape: if non-null entry j counts hist_counts[j] occurrences
+                                    (pre-aggregated (id, count) pairs, the reference's counts_ map) */
+    int64_t hist_stride;
+    const uint32_t* hist_len;   /* [n_rows] valid entries per row (required when hist_tokens is given) */
+    /* speculative verification, sampler.cpp:86-107 (optional: all three or none) */
+    const int32_t* draft;    /* [n_rows] draft token per row */
+    const float* u2;         /* [n_rows] second uniform, consumed by the redraw after a rejection (:106) */
+    uint8_t* out_accepted;   /* [n_rows] 1 = draft accepted */
+    /* ---- outputs (device pointers) ---- */
+    int32_t* out_tokens;     /* [n_rows] sampled token ids */
+    /* optional diagnostics for parity checks; any may be null */
+    uint32_t* out_n_cand;    /* [n_rows] size of the final candidate list (0 for greedy rows) */
+    float* out_total;        /* [n_rows] fp32 total of sampler.cpp:80-82 */
+    float* out_q;            /* [n_rows] unnormalised weight of the returned token; probability = q / total */
+    uint8_t* out_path;       /* [n_rows] MAKO_PATH_* */
+    int32_t* out_cand_idx;   /* [n_rows][cand_cap] first candidates, in candidate order */
+    float* out_cand_q;       /* [n_rows][cand_cap] and their weights */
+    uint32_t cand_cap;
+} mako_sample_desc;
+
+typedef struct mako_sampler_ctx mako_sampler_ctx;
+
+/* Creates a context on HIP device `device` able to serve batches of up to
+ * max_rows x max_vocab with histories of up to max_hist tokens per row; all
+ * device scratch is allocated here.  Replaces Sampler::Sampler
+ * (src/gen/sampler.cpp:9-13) as the owner of the work buffers. */
+int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, uint32_t max_vocab,
+                        uint32_t max_hist);
+void mako_sampler_destroy(mako_sampler_ctx* ctx);
+
+/* Enqueues one batch on `stream` (a hipStream_t, or null for the default
+ * stream) and returns without waiting: Sampler::sample / Sampler::verify
+ * (src/gen/sampler.cpp:75-107) for every row.  One batch at a time per context. */
+int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* desc, void* stream);
+
+/* Host-pointer convenience call with the reference's calling convention
+ * (host logits, src/gen/session.cpp:443): copies the rows to the device,
+ * samples, waits and copies the ids back.  Arrays are host arrays here; mask,
+ * hist_*, draft/u2/accepted may be null.  PCIe-bound, not the measured path. */
+int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t logits_stride, uint32_t n_rows,
+                             uint32_t n_vocab, const mako_sampling_params* params, const float* u,
+                             const uint32_t* mask, int64_t mask_stride, const int32_t* hist_tokens,
+                             const uint32_t* hist_counts, int64_t hist_stride, const uint32_t* hist_len,
+                             const int32_t* draft, const float* u2, uint8_t* out_accepted, int32_t* out_tokens);
+
+/* Text of the last failure on this context (never null). */
+const char* mako_sampler_last_error(const mako_sampler_ctx* ctx);
+
+/* Number of slices a row of n_vocab logits is split into by the scan kernel. */
+uint32_t mako_sampler_slices(uint32_t n_vocab);
+
+/* Device-side self-check hooks used by the parity tests: evaluate the
+ * library's expf (glibc 2.35 bit-exact) and fp32 division on n device values. */
+int mako_sampler_debug_expf(const float* x_dev, float* y_dev, uint32_t n, void* stream);
+int mako_sampler_debug_div(const float* a_dev, const float* b_dev, float* y_dev, uint32_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

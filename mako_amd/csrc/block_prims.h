@@ -1,0 +1,173 @@
+// Workgroup-wide primitives for 1024-thread workgroups of 64-wide wavefronts.
+// Every function must be reached by all threads of the workgroup.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "seqfp.h"
+
+namespace mako {
+
+constexpr int kThreads = 1024;
+constexpr int kWave = 64;
+constexpr int kWaves = kThreads / kWave;
+
+__device__ __forceinline__ int lane_id()
+{
+    return threadIdx.x & (kWave - 1);
+}
+__device__ __forceinline__ int wave_id()
+{
+    return threadIdx.x >> 6;
+}
+
+// Scratch shared by the primitives; one instance per kernel.
+struct BlockScratch {
+    unsigned long long u64[kWaves];
+    double f64[kWaves];
+    seqfp::Step step[kWaves];
+    unsigned long long bcast;
+};
+
+__device__ __forceinline__ uint32_t block_sum_u32(uint32_t v, BlockScratch& s)
+{
+    for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o);
+    if (lane_id() == 0)
+        s.u64[wave_id()] = v;
+    __syncthreads();
+    uint32_t t = 0;
+    for (int w = 0; w < kWaves; ++w)
+        t += (uint32_t)s.u64[w];
+    __syncthreads();
+    return t;
+}
+
+__device__ __forceinline__ uint32_t block_min_u32(uint32_t v, BlockScratch& s)
+{
+    for (int o = 32; o > 0; o >>= 1)
+        v = min(v, (uint32_t)__shfl_xor(v, o));
+    if (lane_id() == 0)
+        s.u64[wave_id()] = v;
+    __syncthreads();
+    uint32_t t = 0xffffffffu;
+    for (int w = 0; w < kWaves; ++w)
+        t = min(t, (uint32_t)s.u64[w]);
+    __syncthreads();
+    return t;
+}
+
+__device__ __forceinline__ unsigned long long block_max_u64(unsigned long long v, BlockScratch& s)
+{
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long t = __shfl_xor(v, o);
+        v = t > v ? t : v;
+    }
+    if (lane_id() == 0)
+        s.u64[wave_id()] = v;
+    __syncthreads();
+    unsigned long long t = 0;
+    for (int w = 0; w < kWaves; ++w)
+        t = s.u64[w] > t ? s.u64[w] : t;
+    __syncthreads();
+    return t;
+}
+
+// Exclusive prefix sum in thread order; `total` receives the workgroup sum.
+__device__ __forceinline__ uint32_t block_excl_scan_u32(uint32_t v, uint32_t& total, BlockScratch& s)
+{
+    uint32_t incl = v;
+    for (int o = 1; o < kWave; o <<= 1) {
+        const uint32_t t = __shfl_up(incl, o);
+        if (lane_id() >= o)
+            incl += t;
+    }
+    if (lane_id() == kWave - 1)
+        s.u64[wave_id()] = incl;
+    __syncthreads();
+    uint32_t pre = 0, tot = 0;
+    for (int w = 0; w < kWaves; ++w) {
+        const uint32_t x = (uint32_t)s.u64[w];
+        if (w < wave_id())
+            pre += x;
+        tot += x;
+    }
+    __syncthreads();
+    total = tot;
+    return pre + incl - v;
+}
+
+// Sum of doubles in a fixed order (lanes by butterfly, then waves in order):
+// the same inputs always give the same bits.
+__device__ __forceinline__ double block_sum_f64(double v, BlockScratch& s)
+{
+    for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o);
+    if (lane_id() == 0)
+        s.f64[wave_id()] = v;
+    __syncthreads();
+    double t = 0;
+    for (int w = 0; w < kWaves; ++w)
+        t += s.f64[w];
+    __syncthreads();
+    return t;
+}
+
+// Inclusive prefix sum of doubles in thread order; fixed association.
+__device__ __forceinline__ double block_incl_scan_f64(double v, double& total, BlockScratch& s)
+{
+    for (int o = 1; o < kWave; o <<= 1) {
+        const double t = __shfl_up(v, o);
+        if (lane_id() >= o)
+            v += t;
+    }
+    if (lane_id() == kWave - 1)
+        s.f64[wave_id()] = v;
+    __syncthreads();
+    double pre = 0, tot = 0;
+    for (int w = 0; w < kWaves; ++w) {
+        const double x = s.f64[w];
+        if (w < wave_id())
+            pre += x;
+        tot += x;
+    }
+    __syncthreads();
+    total = tot;
+    return pre + v;
+}
+
+// Exclusive scan of two-state maps under composition (earlier thread first);
+// `total` receives the composition of all of them.
+__device__ __forceinline__ seqfp::Step block_excl_scan_step(seqfp::Step f, seqfp::Step& total, BlockScratch& s)
+{
+    seqfp::Step incl = f;
+    for (int o = 1; o < kWave; o <<= 1) {
+        seqfp::Step t;
+        t.d0 = __shfl_up(incl.d0, o);
+        t.d1 = __shfl_up(incl.d1, o);
+        if (lane_id() >= o)
+            incl = seqfp::compose(t, incl);
+    }
+    if (lane_id() == kWave - 1)
+        s.step[wave_id()] = incl;
+    // exclusive within the wave: the inclusive value of the previous lane
+    seqfp::Step excl;
+    excl.d0 = __shfl_up(incl.d0, 1);
+    excl.d1 = __shfl_up(incl.d1, 1);
+    if (lane_id() == 0)
+        excl = seqfp::identity();
+    __syncthreads();
+    seqfp::Step pre = seqfp::identity(), tot = seqfp::identity();
+    for (int w = 0; w < kWaves; ++w) {
+        const seqfp::Step x = s.step[w];
+        if (w < wave_id())
+            pre = seqfp::compose(pre, x);
+        tot = seqfp::compose(tot, x);
+    }
+    __syncthreads();
+    total = tot;
+    return seqfp::compose(pre, excl);
+}
+
+} // namespace mako

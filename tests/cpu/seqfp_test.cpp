@@ -1,0 +1,200 @@
+// Host unit test of mako_amd/csrc/seqfp.h: a scan over two-state integer maps must
+// reproduce a sequential fp32 running sum and the sequential fp32 walk bit for bit.
+// The driver below mirrors the kernels' windowed block algorithm with NT
+// virtual threads.  Build: g++ -O2 -std=c++17 -ffp-contract=off.
+#include "../../mako_amd/csrc/seqfp.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+#include <vector>
+
+using namespace seqfp;
+
+static float seq_sum(const std::vector<float>& q)
+{
+    float s = 0;
+    for (float v : q)
+        s += v;
+    return s;
+}
+
+static size_t seq_walk(const std::vector<float>& q, float r)
+{
+    for (size_t i = 0; i < q.size(); ++i) {
+        if (r < q[i])
+            return i;
+        r -= q[i];
+    }
+    return q.size() - 1;
+}
+
+static float emu_sum(const std::vector<float>& q, int NT, int LMAX, long* rounds)
+{
+    const size_t n = q.size();
+    float S = q[0];
+    size_t i0 = 1;
+    int L = 1;
+    while (i0 < n) {
+        ++*rounds;
+        uint32_t M;
+        int e;
+        split(S, M, e);
+        const long long m = M;
+        const size_t W = std::min(n - i0, size_t(NT) * L);
+        std::vector<Step> f(NT, identity());
+        for (int t = 0; t < NT; ++t)
+            for (size_t j = i0 + size_t(t) * L; j < std::min(i0 + size_t(t + 1) * L, i0 + W); ++j)
+                f[t] = compose(f[t], add_step(q[j], e));
+        Step pre = identity();
+        size_t first = SIZE_MAX;
+        long long mm_first = 0, m_end = m;
+        for (int t = 0; t < NT; ++t) {
+            long long mm = m + ((m & 1) ? pre.d1 : pre.d0);
+            size_t j = i0 + size_t(t) * L;
+            const size_t jend = std::min(i0 + size_t(t + 1) * L, i0 + W);
+            for (; j < jend; ++j) {
+                if (add_event(mm, q[j], e))
+                    break;
+                mm = add_apply(mm, q[j], e);
+            }
+            if (j < jend && j < first) {
+                first = j;
+                mm_first = mm;
+            }
+            if (jend > i0 + size_t(t) * L || t == 0)
+                m_end = mm;
+            pre = compose(pre, f[t]);
+        }
+        if (first == SIZE_MAX) {
+            // state after the window: m + total map
+            m_end = m + ((m & 1) ? pre.d1 : pre.d0);
+            S = join(uint32_t(m_end), e);
+            i0 += W;
+            L = std::min(L * 2, LMAX);
+        } else {
+            S = join(uint32_t(mm_first), e) + q[first];
+            i0 = first + 1;
+        }
+    }
+    return S;
+}
+
+static size_t emu_walk(const std::vector<float>& q, float r, int NT, int LMAX)
+{
+    const size_t n = q.size();
+    if (!(r == r) || std::isinf(r))
+        return r < 0 ? 0 : n - 1;
+    if (r < 0)
+        return 0;
+    size_t i0 = 0;
+    int L = 1;
+    for (;;) {
+        if (i0 >= n)
+            return n - 1;
+        uint32_t M;
+        int e;
+        split(r, M, e);
+        const long long m = M;
+        const size_t W = std::min(n - i0, size_t(NT) * L);
+        std::vector<Step> f(NT, identity());
+        for (int t = 0; t < NT; ++t)
+            for (size_t j = i0 + size_t(t) * L; j < std::min(i0 + size_t(t + 1) * L, i0 + W); ++j)
+                f[t] = compose(f[t], sub_step(q[j], e));
+        Step pre = identity();
+        size_t first = SIZE_MAX;
+        long long mm_first = 0;
+        bool stop_first = false;
+        for (int t = 0; t < NT; ++t) {
+            long long mm = m - ((m & 1) ? pre.d1 : pre.d0);
+            size_t j = i0 + size_t(t) * L;
+            const size_t jend = std::min(i0 + size_t(t + 1) * L, i0 + W);
+            bool stop = false;
+            for (; j < jend; ++j) {
+                if (walk_stop(mm, q[j], e)) {
+                    stop = true;
+                    break;
+                }
+                if (sub_event(mm, q[j], e))
+                    break;
+                mm = sub_apply(mm, q[j], e);
+            }
+            if (j < jend && j < first) {
+                first = j;
+                mm_first = mm;
+                stop_first = stop;
+            }
+            pre = compose(pre, f[t]);
+        }
+        if (first == SIZE_MAX) {
+            const long long m_end = m - ((m & 1) ? pre.d1 : pre.d0);
+            r = join(uint32_t(m_end), e);
+            i0 += W;
+            L = std::min(L * 2, LMAX);
+        } else if (stop_first) {
+            return first;
+        } else {
+            r = join(uint32_t(mm_first), e) - q[first];
+            i0 = first + 1;
+        }
+    }
+}
+
+int main()
+{
+    std::mt19937_64 rng(12345);
+    std::uniform_real_distribution<float> U(0.0f, 1.0f);
+    std::normal_distribution<float> N(0.0f, 1.0f);
+    long fails = 0, cases = 0, rounds = 0;
+    for (int it = 0; it < 4000; ++it) {
+        const int kind = it % 8;
+        size_t n = 1 + rng() % (it % 50 == 0 ? 200000 : 3000);
+        std::vector<float> q(n);
+        for (auto& v : q) {
+            switch (kind) {
+            case 0: v = std::exp(3.0f * N(rng)); break;                       // wide
+            case 1: v = std::exp(0.1f * N(rng)); break;                       // near flat
+            case 2: v = seqfp::u2f(uint32_t(rng() % 0x3f800000u) + 1); break; // any exponent incl. subnormal
+            case 3: v = seqfp::u2f(0x3f000000u + uint32_t(rng() % 4) * 0x400000u); break; // many ties
+            case 4: v = U(rng); break;
+            case 5: v = seqfp::u2f(1 + uint32_t(rng() % 64)); break;          // subnormals
+            case 6: v = std::exp(10.0f * N(rng) - 20.0f); break;
+            default: v = float(1 + rng() % 8) * 0.125f; break;
+            }
+            if (!(v > 0))
+                v = 1.0f;
+        }
+        const float mx = *std::max_element(q.begin(), q.end());
+        if (kind != 2 && kind != 5)
+            for (auto& v : q)
+                v = std::min(v / mx, 1.0f);
+        const bool sorted = (it / 8) % 2 == 0;
+        if (sorted)
+            std::sort(q.begin(), q.end(), std::greater<float>());
+        const int NT = (it % 3 == 0) ? 7 : ((it % 3 == 1) ? 64 : 1024);
+        const int LMAX = (it % 5 == 0) ? 1 : 32;
+        const float total = seq_sum(q);
+        const float got = emu_sum(q, NT, LMAX, &rounds);
+        ++cases;
+        if (f2u(total) != f2u(got)) {
+            ++fails;
+            std::printf("SUM mismatch it=%d n=%zu kind=%d sorted=%d want=%a got=%a\n", it, n, kind, sorted, total, got);
+        }
+        for (int d = 0; d < 6; ++d) {
+            float u = U(rng);
+            if (d == 4) u = 0.0f;
+            if (d == 5) u = std::nextafter(1.0f, 0.0f);
+            const float r = u * total;
+            const size_t a = seq_walk(q, r), b = emu_walk(q, r, NT, LMAX);
+            ++cases;
+            if (a != b) {
+                ++fails;
+                std::printf("WALK mismatch it=%d n=%zu kind=%d sorted=%d u=%a want=%zu got=%zu\n", it, n, kind, sorted, u, a, b);
+            }
+        }
+    }
+    std::printf("%ld cases, %ld failures, %ld sum rounds\n", cases, fails, rounds);
+    return fails ? 1 : 0;
+}

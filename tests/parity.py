@@ -1,0 +1,63 @@
+"""Runs a workload through the HIP path (C ABI) and through the CPU oracle and compares them bit for bit."""
+from concurrent.futures import ThreadPoolExecutor
+
+import numpy as np
+
+from mako_amd import api
+from oracle import pyoracle
+
+
+def oracle_rows(w, rows=None, cap=0, order_mode=1, draft=None, u2=None):
+    o = pyoracle.oracle()
+    b = w["logits"].shape[0]
+    rows = range(b) if rows is None else rows
+
+    def one(r):
+        p = pyoracle.params_from_record(w["params"][r])
+        hist = w["hist"][r, : w["hist_len"][r]] if "hist" in w else None
+        mask = w["mask"][r] if "mask" in w else None
+        if draft is not None:
+            t, acc = o.verify(w["logits"][r], p, int(draft[r]), float(w["u"][r]), float(u2[r]), hist, mask, order_mode)
+            return t, dict(accepted=acc)
+        return o.sample(w["logits"][r], p, float(w["u"][r]), hist, mask, order_mode, cap)
+
+    with ThreadPoolExecutor(8) as ex:
+        return list(ex.map(one, rows))
+
+
+def gpu_rows(ctx, w, cap=0, draft=None, u2=None, hist_counts=None):
+    return api.sample(ctx, w["logits"], w["params"], w["u"], mask=w.get("mask"), hist=w.get("hist"),
+                      hist_len=w.get("hist_len"), hist_counts=hist_counts, draft=draft, u2=u2, cand_cap=cap)
+
+
+def assert_parity(ctx, w, cap=256, rel_tol=1e-5):
+    """Token ids, candidate counts, candidate id lists and weights must match the oracle exactly;
+    probabilities q/total within rel_tol (they are in fact bit-identical)."""
+    g = gpu_rows(ctx, w, cap=cap)
+    ref = oracle_rows(w, cap=cap)
+    bad = []
+    for r, (t, tr) in enumerate(ref):
+        greedy = w["params"][r]["temperature"] <= 0
+        if g["tokens"][r] != t:
+            bad.append((r, "token", int(g["tokens"][r]), t))
+            continue
+        if greedy:
+            continue
+        if g["n_cand"][r] != tr["n_cand"]:
+            bad.append((r, "n_cand", int(g["n_cand"][r]), tr["n_cand"]))
+            continue
+        n = min(cap, tr["n_cand"])
+        if not np.array_equal(g["cand_idx"][r, :n], tr["cand_idx"][:n]):
+            bad.append((r, "cand_idx"))
+            continue
+        if not np.array_equal(g["cand_q"][r, :n].view(np.uint32), tr["cand_q"][:n].view(np.uint32)):
+            bad.append((r, "cand_q"))
+            continue
+        if np.float32(g["total"][r]).view(np.uint32) != np.float32(tr["total"]).view(np.uint32):
+            bad.append((r, "total", float(g["total"][r]), float(tr["total"])))
+            continue
+        pg, po = g["q"][r] / g["total"][r], tr["q_chosen"] / tr["total"]
+        if not abs(pg - po) <= rel_tol * abs(po):
+            bad.append((r, "prob", float(pg), float(po)))
+    assert not bad, "%s: %d rows differ from the oracle: %s" % (w.get("name", "?"), len(bad), bad[:8])
+    return g

@@ -1,0 +1,253 @@
+"""GPU parity tests: the HIP sampler, called through the C ABI, against the CPU oracle."""
+import numpy as np
+import pytest
+
+from mako_amd import api, hip, workloads
+from oracle import pyoracle
+from parity import assert_parity, gpu_rows, oracle_rows
+
+pytestmark = pytest.mark.gpu
+
+SAMPLER_TEST_LOGITS = np.array([[2.0, 1.5, 0.3, -0.5, 1.9, -2.0, 0.0, 1.0]], np.float32)  # tests/sampler_test.cpp:56
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def test_device_expf_matches_oracle(gpu_ctx, oracle):
+    """expf on the device equals the glibc restatement on 4M inputs incl. the underflow edge and specials."""
+    rng = np.random.default_rng(7)
+    x = np.concatenate([
+        -np.abs(rng.standard_normal(1 << 21) * 30).astype(np.float32),
+        rng.integers(0, 2**32, 1 << 21, dtype=np.uint64).astype(np.uint32).view(np.float32),
+        np.linspace(-104.5, -102.5, 1 << 16).astype(np.float32),
+        np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 88.0, 88.8, -87.9, -88.0, -103.9, -103.97, -103.98, -104.0, -1e-30, 1e-30,
+                  -150.0], np.float32)])
+    dx = hip.DeviceArray.from_host(x)
+    dy = hip.DeviceArray(x.shape, np.float32)
+    assert gpu_ctx.lib.mako_sampler_debug_expf(dx.ptr, dy.ptr, x.size, None) == 0
+    hip.synchronize()
+    y = dy.download()
+    want = np.array([oracle.expf(v) for v in x[:: 97]], np.float32)
+    got = y[:: 97]
+    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+    assert same.all(), (x[::97][~same][:5], got[~same][:5], want[~same][:5])
+    # and against libm through numpy on the whole array (numpy's exp may differ from libm: use the oracle sample only)
+
+
+def test_device_division_is_ieee(gpu_ctx):
+    rng = np.random.default_rng(8)
+    a = rng.integers(0, 2**32, 1 << 20, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    b = rng.integers(0, 2**32, 1 << 20, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    a[:1000] = (rng.standard_normal(1000) * 5).astype(np.float32)
+    b[:1000] = np.float32(1.1)
+    da, db = hip.DeviceArray.from_host(a), hip.DeviceArray.from_host(b)
+    dy = hip.DeviceArray(a.shape, np.float32)
+    assert gpu_ctx.lib.mako_sampler_debug_div(da.ptr, db.ptr, dy.ptr, a.size, None) == 0
+    hip.synchronize()
+    y = dy.download()
+    with np.errstate(all="ignore"):
+        want = a / b
+    same = (y.view(np.uint32) == want.view(np.uint32)) | (np.isnan(y) & np.isnan(want))
+    assert same.all(), (a[~same][:5], b[~same][:5], y[~same][:5], want[~same][:5])
+
+
+def test_reference_known_answers(gpu_ctx):
+    """The exact checks of tests/sampler_test.cpp:61-67,135-144 and its truncation sets (:91-117)."""
+    lg = SAMPLER_TEST_LOGITS
+    u = np.array([0.3], np.float32)
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 0.0), u)
+    assert r["tokens"][0] == 0
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 0.0), u, draft=np.array([4]), u2=u)
+    assert r["tokens"][0] == 0 and r["accepted"][0] == 0
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 0.0), u, draft=np.array([0]), u2=u)
+    assert r["tokens"][0] == 0 and r["accepted"][0] == 1
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 1e-40), u)
+    assert r["tokens"][0] == 0 and r["path"][0] == api.PATH_FALLBACK
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 1.0, top_k=3), u, cand_cap=8)
+    assert sorted(r["cand_idx"][0, :3].tolist()) == [0, 1, 4] and r["n_cand"][0] == 3
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 1.0, top_p=0.7), u, cand_cap=8)
+    assert r["cand_idx"][0, :3].tolist() == [0, 4, 1] and r["n_cand"][0] == 3
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 1.0, min_p=0.3), u, cand_cap=8)
+    assert sorted(r["cand_idx"][0, :4].tolist()) == [0, 1, 4, 7] and r["n_cand"][0] == 4
+    # presence 0.5 + frequency 0.25, token 0 accepted twice: logit[0] -= 1.0 (:118-126)
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 1.0, presence_penalty=0.5, frequency_penalty=0.25), u,
+                   hist=np.array([[0, 0]], np.int32), cand_cap=8)
+    want = np.exp(np.float32(1.0) - np.float32(1.9))  # token 4 is now the max
+    assert abs(r["cand_q"][0, 0] - want) < 1e-6 and r["cand_idx"][0, 0] == 0
+    # repetition 2.0 with tokens 0 and 5: l0 / 2, l5 * 2 (:127-133)
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 1.0, repetition_penalty=2.0), u, hist=np.array([[0, 5]], np.int32),
+                   cand_cap=8)
+    q = dict(zip(r["cand_idx"][0].tolist(), r["cand_q"][0].tolist()))
+    assert abs(q[0] - np.exp(1.0 - 1.9)) < 1e-6 and abs(q[5] - np.exp(-4.0 - 1.9)) < 1e-7
+    r = api.sample(gpu_ctx, lg, api.make_params(1, 1.0, repetition_penalty=0.0), u, hist=np.array([[0, 4]], np.int32))
+    assert 0 <= r["tokens"][0] < 8
+
+
+def _random_case(rng, v, b):
+    logits = (rng.standard_normal((b, v)) * 3).astype(np.float32)
+    kind = rng.integers(0, 4)
+    if kind == 1:
+        logits = np.round(logits * 2) / 2  # many exact ties
+    if kind == 2:
+        logits = (logits * 0.03).astype(np.float32)  # near-flat: big nuclei
+    p = api.make_params(b)
+    p["temperature"] = rng.choice(np.array([0.0, 0.3, 0.7, 1.0, 1.2, 2.5], np.float32), b)
+    p["top_k"] = rng.choice(np.array([0, 0, 1, 3, 20, 50, 100, 129, 5000, v, v + 7], np.uint32), b)
+    p["top_p"] = rng.choice(np.array([1.0, 0.999, 0.95, 0.9, 0.5, 0.0, 1.5, -1.0], np.float32), b)
+    p["min_p"] = rng.choice(np.array([0.0, 0.0, 0.0, 0.05, 0.5, 1.0, 2.0], np.float32), b)
+    p["presence_penalty"] = rng.choice(np.array([0.0, 0.3, -0.5], np.float32), b)
+    p["frequency_penalty"] = rng.choice(np.array([0.0, 0.2], np.float32), b)
+    p["repetition_penalty"] = rng.choice(np.array([1.0, 1.1, 2.0, 0.5, 0.0], np.float32), b)
+    # the candidate order after top-k alone is the reference library's nth_element order: not compared here
+    both = (p["top_k"] > 0) & ~(p["top_p"] < 1.0)
+    p["top_p"][both] = np.float32(0.97)
+    w = dict(name="random_v%d" % v, logits=logits, params=p, u=rng.random(b).astype(np.float32))
+    hl = int(rng.choice([0, 1, 17, 600]))
+    if hl:
+        w["hist"] = rng.integers(0, v, (b, hl)).astype(np.int32)
+        w["hist"][:, : hl // 2] = w["hist"][:, :1]  # repeats
+        w["hist_len"] = rng.integers(0, hl + 1, b).astype(np.uint32)
+    if rng.integers(0, 3) == 0:
+        w["mask"] = rng.integers(0, 2**32, (b, (v + 31) // 32), dtype=np.uint64).astype(np.uint32)
+    return w
+
+
+@pytest.mark.parametrize("v", [1, 2, 8, 63, 64, 65, 1000, 4096, 16384, 16385, 40000, 129280])
+def test_random_parameters(gpu_ctx, v):
+    """Random parameter mixes (ties, near-flat rows, masks, histories, extreme values) at many vocabulary sizes."""
+    rng = np.random.default_rng(1000 + v)
+    for it in range(3):
+        w = _random_case(rng, v, 24 if v < 100000 else 8)
+        _say("random case v=%d it=%d" % (v, it))
+        assert_parity(gpu_ctx, w, cap=min(v, 512))
+
+
+def test_special_values(gpu_ctx):
+    """NaN/inf logits, all-masked rows, NaN parameters: the fallbacks of src/gen/sampler.cpp:37-38."""
+    v = 5000
+    rng = np.random.default_rng(5)
+    base = (rng.standard_normal((12, v)) * 3).astype(np.float32)
+    base[0, 0] = np.nan
+    base[1, 17] = np.nan
+    base[2, :] = -np.inf
+    base[3, 100] = np.inf
+    base[4, 100] = np.inf
+    base[4, 200] = np.inf
+    base[5, :] = 1.25
+    base[6, :] = 0.0
+    base[6, 7] = -0.0
+    base[7, 1:] = np.nan
+    p = api.make_params(12, 0.8, 0, 0.9)
+    p["temperature"][8] = np.nan
+    p["top_p"][9] = np.nan
+    p["min_p"][10] = np.nan
+    p["temperature"][11] = 1e-40
+    w = dict(name="special", logits=base, params=p, u=rng.random(12).astype(np.float32))
+    assert_parity(gpu_ctx, w)
+    w["params"] = api.make_params(12, 0.0)
+    assert_parity(gpu_ctx, w)
+    mask = np.zeros((12, (v + 31) // 32), np.uint32)
+    mask[1, 3] = 1 << 5
+    w["mask"] = mask
+    w["params"] = p
+    assert_parity(gpu_ctx, w)
+
+
+def test_history_forms_agree(gpu_ctx):
+    """Raw accept() token lists and pre-aggregated (id, count) pairs give identical results."""
+    w = workloads.config3(rows=8, vocab=30000, hist_len=300)
+    g1 = gpu_rows(gpu_ctx, w)
+    hist = np.zeros_like(w["hist"])
+    cnts = np.zeros(w["hist"].shape, np.uint32)
+    lens = np.zeros(8, np.uint32)
+    for r in range(8):
+        ids, c = np.unique(w["hist"][r], return_counts=True)
+        hist[r, : len(ids)], cnts[r, : len(ids)], lens[r] = ids, c, len(ids)
+    w2 = dict(w, hist=hist, hist_len=lens)
+    g2 = gpu_rows(gpu_ctx, w2, hist_counts=cnts)
+    assert np.array_equal(g1["tokens"], g2["tokens"]) and np.array_equal(g1["total"], g2["total"])
+
+
+def test_verify_matches_oracle(gpu_ctx):
+    """Sampler::verify (src/gen/sampler.cpp:86-107): accept/reject and the redraw, against the oracle."""
+    rng = np.random.default_rng(77)
+    v, b = 20000, 48
+    w = _random_case(rng, v, b)
+    w["params"]["temperature"][: b // 2] = 0.9
+    w["params"]["top_k"][: b // 2] = 40
+    w["params"]["top_p"][: b // 2] = 0.95
+    first = oracle_rows(w)
+    draft = np.array([t for t, _ in first], np.int32)
+    draft[::3] = rng.integers(0, v, len(draft[::3]))
+    u2 = rng.random(b).astype(np.float32)
+    g = gpu_rows(gpu_ctx, w, draft=draft, u2=u2)
+    ref = oracle_rows(w, draft=draft, u2=u2)
+    for r, (t, tr) in enumerate(ref):
+        assert g["tokens"][r] == t and bool(g["accepted"][r]) == tr["accepted"], (r, g["tokens"][r], t)
+
+
+def test_config1(gpu_ctx):
+    assert_parity(gpu_ctx, workloads.config1(rows=4))
+
+
+def test_config2(gpu_ctx):
+    assert_parity(gpu_ctx, workloads.config2(rows=2, greedy=True))
+    assert_parity(gpu_ctx, workloads.config2(rows=4, greedy=False), cap=1024)
+
+
+def test_config3_full_batch(gpu_ctx):
+    g = assert_parity(gpu_ctx, workloads.config3())
+    _say("config3 paths: %s" % np.bincount(g["path"], minlength=6).tolist())
+
+
+def test_config4_reduced(gpu_ctx):
+    """16 of the 256 rows (8 heavy-tailed, 8 near-flat with ~133K-token nuclei)."""
+    w = workloads.config4(rows=16)
+    g = assert_parity(gpu_ctx, w, cap=2048)
+    _say("config4 nuclei: %s" % g["n_cand"].tolist())
+
+
+def test_config5_masks(gpu_ctx):
+    for density in (0.01, 0.5):
+        assert_parity(gpu_ctx, workloads.config5(rows=32, density=density))
+
+
+def test_full_size_properties(gpu_ctx):
+    """Size-independent properties at the full benchmark sizes (B=256, V=151552), no oracle:
+    ids inside the allowed set, greedy rows equal numpy's first argmax, u=0 returns the most likely candidate,
+    and the same batch twice gives the same ids."""
+    w = workloads.config4()
+    g1 = gpu_rows(gpu_ctx, w)
+    g2 = gpu_rows(gpu_ctx, w)
+    assert np.array_equal(g1["tokens"], g2["tokens"])
+    assert ((g1["tokens"] >= 0) & (g1["tokens"] < w["logits"].shape[1])).all()
+    w0 = dict(w, u=np.zeros(256, np.float32))
+    g0 = gpu_rows(gpu_ctx, w0)
+    assert np.array_equal(g0["tokens"], w["logits"].argmax(axis=1))
+    wg = dict(w, params=api.make_params(256, 0.0))
+    gg = gpu_rows(gpu_ctx, wg)
+    assert np.array_equal(gg["tokens"], w["logits"].argmax(axis=1))
+    w5 = workloads.config5(density=0.01)
+    g5 = gpu_rows(gpu_ctx, w5)
+    t = g5["tokens"]
+    allowed = (w5["mask"][np.arange(256), t >> 5] >> (t & 31).astype(np.uint32)) & 1
+    assert allowed.all()
+
+
+def test_argument_errors(gpu_ctx):
+    """n_vocab == 0 is the reference's std::invalid_argument (src/gen/sampler.cpp:11-12); other bad arguments too."""
+    b = api.Batch(SAMPLER_TEST_LOGITS, api.make_params(1), np.zeros(1, np.float32))
+    d = b.desc
+    d.n_vocab = 0
+    with pytest.raises(api.MakoError, match="empty vocabulary"):
+        gpu_ctx.sample_batch(d)
+    d.n_vocab = 8
+    d.out_tokens = None
+    with pytest.raises(api.MakoError):
+        gpu_ctx.sample_batch(d)
+    d.out_tokens = b.o_tokens.ptr
+    d.n_rows = 100000
+    with pytest.raises(api.MakoError, match="exceeds"):
+        gpu_ctx.sample_batch(d)
