@@ -1,0 +1,165 @@
+#!/usr/bin/env python3
+"""Headline benchmark: sampled rows/s of the HIP sampler on the decode batch B=64 x V=129280 fp32
+(penalties over 2048-token histories, per-row temperature / top-k / top-p), one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config4|config5|config1|config2b]
+
+A step is one batch through the whole sampling pipeline with every input already resident in HBM.
+The logits are rotated through a pool of copies larger than the 256 MB Infinity Cache so each step
+reads them from HBM.  Prints one JSON line; `roofline` prices the batch's algorithmic bytes against the
+HBM peak using HIP-event time on the launch stream, `cpu_baseline` is the reference CPU sampler timed
+on this host on the same rows.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def make_workload(name):
+    from mako_amd import workloads
+    if name == "config1":
+        return workloads.config1()
+    if name == "config2b":
+        return workloads.config2()
+    if name == "config3":
+        return workloads.config3()
+    if name == "config4":
+        return workloads.config4()
+    if name == "config5":
+        return workloads.config5(density=0.5)
+    raise SystemExit("unknown workload " + name)
+
+
+def cpu_baseline(w, budget_s):
+    """The reference CPU sampler (or, if it was not built, the oracle port) on this host's cores."""
+    from oracle import pyoracle
+    ref = pyoracle.reference()
+    rows = w["logits"].shape[0]
+    cores = max(1, min(os.cpu_count() or 1, 16))
+    if ref is not None:
+        kw = dict(hist=w.get("hist"), hist_len=w.get("hist_len"), mask=w.get("mask"))
+        t1, tok = ref.sample_batch_timed(w["logits"], w["params"], w["seeds"], n_threads=1, **kw)
+        reps, spent, wall = 0, 0.0, 0.0
+        while spent < budget_s and reps < 50:
+            t0 = time.perf_counter()
+            ref.sample_batch_timed(w["logits"], w["params"], w["seeds"], n_threads=cores, **kw)
+            wall += time.perf_counter() - t0
+            spent += wall / (reps + 1)
+            reps += 1
+        return dict(value=rows * reps / wall, unit="rows/s", cores=cores, kind="reference",
+                    value_1thread=rows / t1,
+                    sample="%d x the %d-row %s batch, one fresh Sampler per row, sample() only (history replay and "
+                           "thread start included in the %d-thread wall time)" % (reps, rows, w["name"], cores)), tok
+    o = pyoracle.oracle()
+    t0 = time.perf_counter()
+    tok = []
+    n = min(rows, 16)
+    for r in range(n):
+        p = pyoracle.params_from_record(w["params"][r])
+        hist = w["hist"][r, : w["hist_len"][r]] if "hist" in w else None
+        tok.append(o.sample(w["logits"][r], p, float(w["u"][r]), hist, w["mask"][r] if "mask" in w else None)[0])
+    dt = time.perf_counter() - t0
+    return dict(value=n / dt, unit="rows/s", cores=1, kind="port",
+                sample="first %d rows of the %s batch through the plain-C oracle" % (n, w["name"])), None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--workload", default="config3")
+    ap.add_argument("--pool-mb", type=int, default=640, help="rotate the logits through this many MB of copies")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg (0 = skip)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: rows are independent, a multi-GPU run is a plain batch split "
+                         "(see DESIGN.md); run with --gpus 1")
+
+    from mako_amd import api, hip, workloads
+    from oracle import pyoracle
+    if hip.device_count() < 1:
+        raise SystemExit("bench.py needs an MI355X")
+    hip.set_device(0)
+
+    w = make_workload(a.workload)
+    rows, vocab = w["logits"].shape
+    # the uniforms a reference Sampler seeded with seeds[r] would draw, so both sides consume the same u
+    orc = pyoracle.oracle()
+    w["u"] = np.array([orc.uniforms(int(s), 1)[0] for s in w["seeds"]], np.float32)
+
+    ctx = api.SamplerContext(max_rows=rows, max_vocab=vocab, max_hist=w["hist"].shape[1] if "hist" in w else 0)
+    batch = api.Batch(w["logits"], w["params"], w["u"], mask=w.get("mask"), hist=w.get("hist"),
+                      hist_len=w.get("hist_len"), diagnostics=False)
+    row_bytes = workloads.bytes_per_row(w)
+    batch_bytes = rows * row_bytes
+    n_copies = max(2, -(-a.pool_mb * (1 << 20) // (rows * vocab * 4)))
+    pool = [batch.d_logits] + [hip.DeviceArray.from_host(w["logits"]) for _ in range(n_copies - 1)]
+    stream = hip.Stream()
+
+    def step(i):
+        batch.desc.logits = pool[i % n_copies].ptr
+        ctx.sample_batch(batch.desc, stream)
+
+    for i in range(a.warmup):
+        step(i)
+    stream.synchronize()
+    hip.synchronize()
+    e0, e1 = hip.Event(), hip.Event()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for i in range(a.steps):
+        step(a.warmup + i)
+    e1.record(stream)
+    e1.synchronize()
+    hip.synchronize()
+    wall = time.perf_counter() - t0
+    ms = e0.elapsed_ms(e1)
+    ms_per_step = ms / a.steps
+    tokens = batch.o_tokens.download()
+
+    base, ref_tok = (None, None)
+    if a.cpu_seconds > 0:
+        base, ref_tok = cpu_baseline(w, a.cpu_seconds)
+    parity = None
+    if ref_tok is not None:
+        parity = dict(rows=rows, mismatches=int((np.asarray(ref_tok) != tokens).sum()), against="reference sampler")
+
+    achieved = batch_bytes / (ms_per_step * 1e-3) / 1e9
+    out = {
+        "metric": "sampled rows/sec at B=64xV=129280 fp32; achieved HBM GB/s vs peak",
+        "value": rows * a.steps / (ms * 1e-3),
+        "unit": "rows/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "%s: B=%d x V=%d fp32, full penalty + top-k + top-p pipeline" % (w["name"], rows, vocab),
+                   "rows": rows, "vocab": vocab, "logit_copies_rotated": n_copies,
+                   "host_wall_ms_per_step": wall * 1e3 / a.steps},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "bytes_per_launch": batch_bytes, "kernel": "scan_kernel + finish_kernel (one batch)",
+                     "launch_ms": ms_per_step},
+        "cpu_baseline": base,
+        "parity": parity,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
