@@ -1,0 +1,1018 @@
+// MI355X (gfx950) token sampler kernels.
+//
+// Pipeline per batch (rows are independent, src/gen/session.cpp:416):
+//   scan_kernel    one workgroup per (row, slice): a single coalesced pass over the fp32 logits.  The
+//                  token mask and the history penalties are applied in registers; the slice's maximum
+//                  and its largest logits (a superset of what top-k / the nucleus can need) go to scratch.
+//   finish_kernel  greedy rows: argmax.  top-k rows: the row's candidates are weighted with
+//                  q = expf((w - m) / T), sorted by (q desc, idx asc) in LDS, truncated, and drawn from
+//                  with the reference's exact fp32 rounding order.  top_k == 0 rows first take a second,
+//                  cache-resident pass that sums q exactly over the whole row (all slices in parallel, the
+//                  last one to finish continues).  Whatever the candidate lists cannot certify falls to a
+//                  whole-row sort path that is exact for every parameter combination.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <math.h>
+#include <stdint.h>
+
+#include "../../include/mako_sampler.h"
+#include "block_prims.h"
+#include "device_math.h"
+#include "seqfp.h"
+
+namespace mako {
+
+constexpr uint32_t kNone = 0xffffffffu;
+constexpr uint32_t kSliceMax = 16384; // elements per slice: 16 per thread
+constexpr uint32_t kMaxSlices = 64;
+constexpr uint32_t kCap = 256;       // candidates kept per slice
+constexpr uint32_t kTopKFast = 128;  // largest top_k resolved from the per-slice candidates
+constexpr uint32_t kSortMax = 4096;  // candidates the finisher sorts in LDS
+constexpr uint32_t kDynLds = 65536;  // dynamic LDS of both kernels
+
+constexpr uint32_t kFlagFirstNan = 1u; // element 0 of the row is NaN (slice 0 only)
+constexpr uint32_t kFlagOverflow = 2u; // more than kCap logits reached the slice's threshold
+constexpr uint32_t kFlagComplete = 4u; // every logit above -inf was emitted
+
+struct SliceStat {
+    float wmax;       // max of the slice's penalised logits (-inf if none compares greater)
+    uint32_t argidx;  // first index holding it, kNone if nothing exceeded -inf
+    uint32_t flags;
+    uint32_t n_emit;  // candidates written for this slice
+    uint32_t tau_key; // order key of the emission threshold: every logit with key >= tau_key was emitted
+    uint32_t pad[3];
+};
+
+struct Scratch {
+    SliceStat* stats;  // [max_rows][kMaxSlices]
+    float* cand_w;     // [max_rows][slices_cap][kCap] penalised logits of the slice's candidates
+    uint32_t* cand_i;  // [max_rows][slices_cap][kCap] their token ids
+    double* part_sum;  // [max_rows][kMaxSlices] exact fp64 sum of q over the slice (top_k == 0 rows)
+    uint32_t* part_n;  // [max_rows][kMaxSlices] candidates (q > 0, q >= min_p) in the slice
+    uint32_t* tickets; // [max_rows] arrival counter of the row's slices; all zero between calls
+    float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path
+    uint32_t* cnt;     // [max_rows][vpad] token counts; all zero between calls
+    uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong
+    uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, ping-pong
+    uint64_t vpad;
+    uint32_t slices_cap;
+};
+
+// Total order on floats as unsigned keys: -inf < ... < -0 = +0 < ... < +inf.  Never called on NaN.
+__device__ __forceinline__ uint32_t order_key(float f)
+{
+    const uint32_t b = __float_as_uint(f + 0.0f); // -0 -> +0
+    return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
+}
+__device__ __forceinline__ float order_unkey(uint32_t k)
+{
+    const uint32_t b = (k & 0x80000000u) ? (k ^ 0x80000000u) : ~k;
+    return __uint_as_float(b);
+}
+constexpr uint32_t kKeyNegInf = 0x007fffffu; // order_key(-inf)
+
+enum RowClass { kGreedy = 0, kTopK = 1, kNucleus = 2, kGeneral = 3 };
+
+__device__ __forceinline__ RowClass classify(const mako_sampling_params& p)
+{
+    if (p.temperature <= 0.0f) // Sampler::greedy, src/gen/sampler.hpp:26
+        return kGreedy;
+    if (!(p.top_p < 1.0f)) // no top-p: the candidate order is not the sorted one (sampler.cpp:44)
+        return kGeneral;
+    if (p.top_k == 0)
+        return kNucleus;
+    return p.top_k <= kTopKFast ? kTopK : kGeneral;
+}
+
+__device__ __forceinline__ bool penalties_neutral(const mako_sampling_params& p)
+{
+    return p.repetition_penalty == 1.0f && p.presence_penalty == 0.0f && p.frequency_penalty == 0.0f;
+}
+
+// ---------------------------------------------------------------------------------------------
+// slice loading, shared by both kernels
+// ---------------------------------------------------------------------------------------------
+
+// Thread t of a slice owns 16 logits: for k = 0..3 the four consecutive ones at lo + k * 4096 + 4 * t
+// (VEC), or lo + j * 1024 + t for j = 0..15 (scalar).  Either way a wavefront's loads are contiguous and
+// each logit is read once.
+template <bool VEC>
+__device__ __forceinline__ uint32_t elem_index(uint32_t lo, uint32_t tid, uint32_t j)
+{
+    return VEC ? lo + (j >> 2) * 4096u + tid * 4u + (j & 3u) : lo + j * (uint32_t)kThreads + tid;
+}
+
+// accept() history -> per-token counts for [lo, hi) in LDS (src/gen/sampler.cpp:15-18).
+__device__ __forceinline__ void build_counts(const mako_sample_desc& d, uint32_t row, uint32_t hl, uint32_t lo,
+                                             uint32_t hi, uint32_t slice_len, uint32_t* s_cnt)
+{
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t i = tid; i < slice_len; i += kThreads)
+        s_cnt[i] = 0;
+    __syncthreads();
+    const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
+    const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
+    for (uint32_t h = tid; h < hl; h += kThreads) {
+        const uint32_t t = (uint32_t)ht[h];
+        if (t >= lo && t < hi)
+            atomicAdd(&s_cnt[t - lo], hc ? hc[h] : 1u);
+    }
+    __syncthreads();
+}
+
+// The thread's 16 logits after the mask and the penalties (src/gen/sampler.cpp:22-28); slots past the
+// end of the slice hold NaN, which never wins a comparison and never becomes a candidate.
+template <bool VEC>
+__device__ __forceinline__ void load_slice(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi,
+                                           const mako_sampling_params& P, bool pen, const uint32_t* s_cnt, float (&wv)[16])
+{
+    const uint32_t tid = threadIdx.x;
+    const float* lrow = d.logits + (int64_t)row * d.logits_stride;
+    const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
+    const float nan = __uint_as_float(0x7fc00000u);
+    if (VEC) {
+        float4 v[4];
+        uint32_t bits[4];
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            const uint32_t i = lo + k * 4096u + tid * 4u;
+            bits[k] = 0xfu;
+            if (i < hi) { // hi - lo is a multiple of 4 in this mode
+                v[k] = *reinterpret_cast<const float4*>(lrow + i);
+                if (mrow)
+                    bits[k] = mrow[i >> 5] >> (i & 31u);
+            } else {
+                v[k] = make_float4(nan, nan, nan, nan);
+            }
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            wv[4 * k + 0] = (bits[k] & 1u) ? v[k].x : -INFINITY;
+            wv[4 * k + 1] = (bits[k] & 2u) ? v[k].y : -INFINITY;
+            wv[4 * k + 2] = (bits[k] & 4u) ? v[k].z : -INFINITY;
+            wv[4 * k + 3] = (bits[k] & 8u) ? v[k].w : -INFINITY;
+        }
+    } else {
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) {
+            const uint32_t i = lo + j * (uint32_t)kThreads + tid;
+            float v = nan;
+            if (i < hi) {
+                v = lrow[i];
+                if (mrow && !((mrow[i >> 5] >> (i & 31u)) & 1u))
+                    v = -INFINITY;
+            }
+            wv[j] = v;
+        }
+    }
+    if (pen) {
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) {
+            const uint32_t i = elem_index<VEC>(lo, tid, j);
+            if (i < hi) {
+                const uint32_t n = s_cnt[i - lo];
+                if (n)
+                    wv[j] = penalize(wv[j], n, P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// scan_kernel
+// ---------------------------------------------------------------------------------------------
+
+struct ScanShared {
+    BlockScratch bs;
+    uint32_t sel[2][kWaves][16];
+    uint32_t emit_n;
+    float cw[kCap];
+    uint32_t ci[kCap];
+};
+
+// A key `tau` such that at least K of the workgroup's 1024 keys are >= tau, found by a most-significant-
+// digit-first radix select with 4-bit digits: per round every wavefront counts its keys per digit value
+// with ballots, the counts meet in LDS, and the digit holding the K-th largest key is fixed.  The search
+// stops early once at most 8 surplus keys share the bucket; the bucket's lower edge is returned.
+__device__ __forceinline__ uint32_t select_kth_key(uint32_t key, uint32_t K, ScanShared& sm)
+{
+    const int lane = lane_id(), wave = wave_id();
+    uint32_t prefix = 0, need = K;
+    for (int round = 0; round < 8; ++round) {
+        const int shift = 28 - 4 * round;
+        const bool active = round == 0 || (key >> (shift + 4)) == (prefix >> (shift + 4));
+        const uint32_t dg = (key >> shift) & 15u;
+        uint32_t mine = 0;
+#pragma unroll
+        for (uint32_t dv = 0; dv < 16; ++dv) {
+            const uint32_t c = (uint32_t)__popcll(__ballot(active && dg == dv));
+            if ((uint32_t)lane == dv)
+                mine = c;
+        }
+        if (lane < 16)
+            sm.sel[round & 1][wave][lane] = mine;
+        __syncthreads();
+        uint32_t col = 0;
+        if (lane < 16)
+            for (int w = 0; w < kWaves; ++w)
+                col += sm.sel[round & 1][w][lane];
+        uint32_t suf = col; // keys of this bucket with digit >= lane
+        for (int o = 1; o < 16; o <<= 1) {
+            const uint32_t t = __shfl_down(suf, o);
+            if (lane + o < 16)
+                suf += t;
+        }
+        const unsigned long long bal = __ballot(lane < 16 && suf >= need) & 0xffffull;
+        const int D = 63 - __clzll(bal); // bal != 0: the bucket holds at least `need` keys
+        const uint32_t above = D < 15 ? (uint32_t)__shfl(suf, D + 1) : 0u;
+        const uint32_t in_d = (uint32_t)__shfl(col, D);
+        need -= above;
+        prefix |= (uint32_t)D << shift;
+        if (in_d - need <= 8u)
+            break;
+    }
+    return prefix;
+}
+
+// grid = (slices, rows).
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scratch sc, uint32_t slice_len)
+{
+    extern __shared__ uint32_t s_dyn[]; // [slice_len] token counts when the row has penalties
+    __shared__ ScanShared sm;
+
+    const uint32_t row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
+    const uint32_t lo = slice * slice_len;
+    const uint32_t hi = min(d.n_vocab, lo + slice_len);
+    const mako_sampling_params P = d.params[row];
+    const RowClass cls = classify(P);
+
+    // Greedy rows ignore the penalties (src/gen/sampler.cpp:77-78).
+    const uint32_t hl = (d.hist_tokens && cls != kGreedy) ? d.hist_len[row] : 0u;
+    const bool pen = hl > 0 && !penalties_neutral(P);
+    if (pen)
+        build_counts(d, row, hl, lo, hi, slice_len, s_dyn);
+
+    float wv[16];
+    load_slice<VEC>(d, row, lo, hi, P, pen, s_dyn, wv);
+
+    // first maximum of the thread's logits; its index order is increasing in j
+    float best = -INFINITY;
+    uint32_t bidx = kNone;
+#pragma unroll
+    for (uint32_t j = 0; j < 16; ++j)
+        if (wv[j] > best) {
+            best = wv[j];
+            bidx = elem_index<VEC>(lo, tid, j);
+        }
+    const uint32_t bkey = order_key(best);
+    const unsigned long long top = block_max_u64(((unsigned long long)bkey << 32) | (unsigned long long)(kNone - bidx), sm.bs);
+
+    SliceStat st;
+    st.wmax = order_unkey((uint32_t)(top >> 32));
+    st.argidx = kNone - (uint32_t)top;
+    st.flags = 0;
+    st.n_emit = 0;
+    st.tau_key = 0;
+    st.pad[0] = st.pad[1] = st.pad[2] = 0;
+    if (slice == 0 && tid == 0 && wv[0] != wv[0]) // only thread 0 publishes the record
+        st.flags |= kFlagFirstNan;
+
+    if (cls == kTopK || cls == kNucleus) {
+        // Every logit that can be among the row's K largest is among this slice's K largest, and those are
+        // all >= the K-th largest per-thread maximum.
+        const uint32_t K = cls == kTopK ? P.top_k : kTopKFast;
+        uint32_t tau_key = select_kth_key(bkey, K, sm);
+        if (tau_key <= kKeyNegInf) {
+            tau_key = kKeyNegInf;
+            st.flags |= kFlagComplete;
+        }
+        const float tau = order_unkey(tau_key);
+        if (tid == 0)
+            sm.emit_n = 0;
+        __syncthreads();
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) {
+            const float w = wv[j];
+            if (w >= tau && w > -INFINITY) {
+                const uint32_t pos = atomicAdd(&sm.emit_n, 1u);
+                if (pos < kCap) {
+                    sm.cw[pos] = w;
+                    sm.ci[pos] = elem_index<VEC>(lo, tid, j);
+                }
+            }
+        }
+        __syncthreads();
+        const uint32_t n = sm.emit_n;
+        if (n > kCap)
+            st.flags |= kFlagOverflow;
+        st.n_emit = min(n, kCap);
+        st.tau_key = tau_key;
+        const size_t base = ((size_t)row * sc.slices_cap + slice) * kCap;
+        if (tid < st.n_emit) {
+            sc.cand_w[base + tid] = sm.cw[tid];
+            sc.cand_i[base + tid] = sm.ci[tid];
+        }
+    }
+    if (tid == 0)
+        sc.stats[(size_t)row * kMaxSlices + slice] = st;
+}
+
+// ---------------------------------------------------------------------------------------------
+// finish_kernel
+// ---------------------------------------------------------------------------------------------
+
+struct FinishShared {
+    BlockScratch bs;
+    uint64_t tab[32];
+    uint32_t hist[256];
+    uint32_t run[256];
+    uint32_t flag;
+    uint32_t ticket;
+};
+
+// Views into the 64 KB dynamic LDS block; `cnt` (first pass) overlaps the two others (second pass).
+struct FinishLds {
+    FinishShared* sm;
+    uint32_t* cnt;              // [kSliceMax]
+    unsigned long long* sortk;  // [kSortMax]
+    uint32_t* wcount;           // [kWaves * 256]
+};
+
+// Lanes of this wave whose `digit` equals mine, restricted to `valid` lanes.
+__device__ __forceinline__ unsigned long long match_digit(uint32_t digit, bool valid)
+{
+    unsigned long long m = __ballot(valid);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const bool bit = (digit >> b) & 1u;
+        const unsigned long long bal = __ballot(bit);
+        m &= bit ? bal : ~bal;
+    }
+    return m;
+}
+
+// One stable counting-sort pass on bits [shift, shift + 8) of the keys, ascending.
+// Returns false (and moves nothing) when every key has the same digit.
+__device__ bool radix_pass(const uint32_t* ksrc, const uint32_t* isrc, uint32_t* kdst, uint32_t* idst, uint32_t n,
+                           uint32_t shift, const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    if (tid < 256)
+        sm.hist[tid] = 0;
+    if (tid == 0)
+        sm.flag = 0;
+    __syncthreads();
+    for (uint32_t base = 0; base < n; base += kThreads) {
+        const uint32_t i = base + tid;
+        const bool valid = i < n;
+        const uint32_t dg = valid ? ((ksrc[i] >> shift) & 255u) : 0u;
+        const unsigned long long mm = match_digit(dg, valid);
+        const unsigned long long below = mm & ((1ull << lane_id()) - 1ull);
+        if (valid && below == 0)
+            atomicAdd(&sm.hist[dg], (uint32_t)__popcll(mm));
+    }
+    __syncthreads();
+    const uint32_t mine = tid < 256 ? sm.hist[tid] : 0u;
+    if (mine == n)
+        sm.flag = 1;
+    uint32_t tot;
+    const uint32_t excl = block_excl_scan_u32(mine, tot, sm.bs); // its barriers publish sm.flag
+    if (sm.flag)
+        return false;
+    if (tid < 256)
+        sm.run[tid] = excl;
+    __syncthreads();
+    for (uint32_t base = 0; base < n; base += kThreads) {
+        for (uint32_t j = tid; j < kWaves * 256; j += kThreads)
+            L.wcount[j] = 0;
+        __syncthreads();
+        const uint32_t i = base + tid;
+        const bool valid = i < n;
+        const uint32_t key = valid ? ksrc[i] : 0u;
+        const uint32_t dg = (key >> shift) & 255u;
+        const unsigned long long mm = match_digit(dg, valid);
+        const uint32_t rank = (uint32_t)__popcll(mm & ((1ull << lane_id()) - 1ull));
+        if (valid && rank == 0)
+            L.wcount[wave_id() * 256 + dg] = (uint32_t)__popcll(mm);
+        __syncthreads();
+        if (tid < 256) {
+            uint32_t acc = sm.run[tid];
+            for (int w = 0; w < kWaves; ++w) {
+                const uint32_t t = L.wcount[w * 256 + tid];
+                L.wcount[w * 256 + tid] = acc;
+                acc += t;
+            }
+            sm.run[tid] = acc;
+        }
+        __syncthreads();
+        if (valid) {
+            const uint32_t pos = L.wcount[wave_id() * 256 + dg] + rank;
+            kdst[pos] = key;
+            idst[pos] = isrc[i];
+        }
+        __syncthreads();
+    }
+    return true;
+}
+
+// fp32 running sum of q(0..n) in order, bit-identical to `for (...) total += q` (src/gen/sampler.cpp:80-82).
+template <typename QAt>
+__device__ float emulate_sum(QAt qat, uint32_t n, FinishShared& sm)
+{
+    using namespace seqfp;
+    const uint32_t tid = threadIdx.x;
+    float S = qat(0);
+    uint32_t i0 = 1;
+    uint32_t L = 1;
+    while (i0 < n) {
+        uint32_t M;
+        int e;
+        split(S, M, e);
+        const long long m = M;
+        const uint32_t W = min(n - i0, (uint32_t)kThreads * L);
+        const uint32_t jb = min(i0 + tid * L, i0 + W), je = min(jb + L, i0 + W);
+        Step f = identity();
+        for (uint32_t j = jb; j < je; ++j)
+            f = compose(f, add_step(qat(j), e));
+        Step total;
+        const Step pre = block_excl_scan_step(f, total, sm.bs);
+        long long mm = m + ((m & 1) ? pre.d1 : pre.d0);
+        uint32_t hit = kNone;
+        for (uint32_t j = jb; j < je; ++j) {
+            const float q = qat(j);
+            if (add_event(mm, q, e)) {
+                hit = j;
+                break;
+            }
+            mm = add_apply(mm, q, e);
+        }
+        const uint32_t first = block_min_u32(hit, sm.bs);
+        if (first == kNone) {
+            const long long m_end = m + ((m & 1) ? total.d1 : total.d0);
+            S = join((uint32_t)m_end, e);
+            i0 += W;
+            L = min(L * 2u, 16u);
+        } else {
+            if (hit == first)
+                sm.bs.bcast = (unsigned long long)mm;
+            __syncthreads();
+            const long long mf = (long long)sm.bs.bcast;
+            __syncthreads();
+            S = join((uint32_t)mf, e) + qat(first);
+            i0 = first + 1;
+        }
+    }
+    return S;
+}
+
+// Index returned by the walk of src/gen/sampler.cpp:67-72 started at r, bit-identical to the
+// sequential fp32 `if (r < q) return; r -= q;` loop.
+template <typename QAt>
+__device__ uint32_t emulate_walk(QAt qat, uint32_t n, float r, FinishShared& sm)
+{
+    using namespace seqfp;
+    const uint32_t tid = threadIdx.x;
+    if (r < 0.0f)
+        return 0;
+    if (!(r == r) || r == INFINITY)
+        return n - 1; // never below any q: falls through to the last candidate
+    uint32_t i0 = 0;
+    uint32_t L = 1;
+    for (;;) {
+        if (i0 >= n)
+            return n - 1;
+        uint32_t M;
+        int e;
+        split(r, M, e);
+        const long long m = M;
+        const uint32_t W = min(n - i0, (uint32_t)kThreads * L);
+        const uint32_t jb = min(i0 + tid * L, i0 + W), je = min(jb + L, i0 + W);
+        Step f = identity();
+        for (uint32_t j = jb; j < je; ++j)
+            f = compose(f, sub_step(qat(j), e));
+        Step total;
+        const Step pre = block_excl_scan_step(f, total, sm.bs);
+        long long mm = m - ((m & 1) ? pre.d1 : pre.d0);
+        uint32_t hit = kNone;
+        bool stop = false;
+        for (uint32_t j = jb; j < je; ++j) {
+            const float q = qat(j);
+            if (walk_stop(mm, q, e)) {
+                hit = j;
+                stop = true;
+                break;
+            }
+            if (sub_event(mm, q, e)) {
+                hit = j;
+                break;
+            }
+            mm = sub_apply(mm, q, e);
+        }
+        const uint32_t first = block_min_u32(hit, sm.bs);
+        if (first == kNone) {
+            const long long m_end = m - ((m & 1) ? total.d1 : total.d0);
+            r = join((uint32_t)m_end, e);
+            i0 += W;
+            L = min(L * 2u, 16u);
+        } else {
+            if (hit == first)
+                sm.bs.bcast = ((unsigned long long)mm << 1) | (stop ? 1ull : 0ull);
+            __syncthreads();
+            const unsigned long long bc = sm.bs.bcast;
+            __syncthreads();
+            if (bc & 1ull)
+                return first;
+            r = join((uint32_t)(bc >> 1), e) - qat(first);
+            i0 = first + 1;
+        }
+    }
+}
+
+struct RowOut {
+    int32_t token;
+    uint32_t n_cand;
+    float total;
+    float q;
+    uint32_t path;
+    uint32_t accepted;
+};
+
+__device__ __forceinline__ void write_row(const mako_sample_desc& d, uint32_t row, const RowOut& o)
+{
+    d.out_tokens[row] = o.token;
+    if (d.out_n_cand)
+        d.out_n_cand[row] = o.n_cand;
+    if (d.out_total)
+        d.out_total[row] = o.total;
+    if (d.out_q)
+        d.out_q[row] = o.q;
+    if (d.out_path)
+        d.out_path[row] = (uint8_t)o.path;
+    if (d.out_accepted)
+        d.out_accepted[row] = (uint8_t)o.accepted;
+}
+
+// No candidate survived (src/gen/sampler.cpp:37-38): the single candidate (1.0f, first max).
+__device__ void fallback_row(const mako_sample_desc& d, uint32_t row, uint32_t argidx)
+{
+    if (threadIdx.x != 0)
+        return;
+    RowOut o;
+    o.token = (int32_t)argidx;
+    o.n_cand = 1;
+    o.total = 1.0f;
+    o.q = 1.0f;
+    o.path = MAKO_PATH_FALLBACK;
+    // verifying: u * 1 < 1 accepts the draft iff it is that candidate; otherwise it is the only one left
+    o.accepted = d.draft ? (d.draft[row] == (int32_t)argidx) : 0u;
+    if (d.out_cand_idx && d.out_cand_q && d.cand_cap) {
+        d.out_cand_idx[(size_t)row * d.cand_cap] = (int32_t)argidx;
+        d.out_cand_q[(size_t)row * d.cand_cap] = 1.0f;
+    }
+    write_row(d, row, o);
+}
+
+// The draw (and, when verifying, the accept/reject step) over the final candidate list of n entries with
+// weights qat(i) and token ids idat(i).  src/gen/sampler.cpp:64-73, 79-83, 93-106.
+template <typename QAt, typename IdAt>
+__device__ void draw_from_list(const mako_sample_desc& d, uint32_t row, QAt qat, IdAt idat, uint32_t n, uint32_t path,
+                               FinishShared& sm)
+{
+    const uint32_t tid = threadIdx.x;
+    const float total = emulate_sum(qat, n, sm);
+    const float u = d.u[row];
+    RowOut o;
+    o.n_cand = n;
+    o.total = total;
+    o.path = path;
+    o.accepted = 0;
+    if (d.out_cand_idx && d.out_cand_q)
+        for (uint32_t j = tid; j < n && j < d.cand_cap; j += kThreads) {
+            d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
+            d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
+        }
+    if (!d.draft) {
+        const float span = total - 0.0f;
+        const float prod = u * span;
+        const uint32_t pos = emulate_walk(qat, n, prod + 0.0f, sm);
+        o.token = (int32_t)idat(pos);
+        o.q = qat(pos);
+    } else {
+        // position of the draft in the list, if it survived the truncation
+        const int32_t draft = d.draft[row];
+        uint32_t pd = kNone;
+        for (uint32_t j = tid; j < n; j += kThreads)
+            if ((int32_t)idat(j) == draft)
+                pd = j;
+        pd = block_min_u32(pd, sm.bs);
+        const float q_draft = pd == kNone ? 0.0f : qat(pd);
+        const float span = total - 0.0f;
+        const float prod = u * span;
+        const float r1 = prod + 0.0f;
+        o.accepted = r1 < q_draft;
+        o.token = draft;
+        o.q = q_draft;
+        const uint32_t n2 = pd == kNone ? n : n - 1;
+        if (!o.accepted && n2 > 0) {
+            auto qat2 = [&](uint32_t i) { return qat(i + (i >= pd ? 1u : 0u)); };
+            const float rest = total - q_draft;
+            const float span2 = rest - 0.0f;
+            const float prod2 = d.u2[row] * span2;
+            const uint32_t pos = emulate_walk(qat2, n2, prod2 + 0.0f, sm);
+            const uint32_t at = pos + (pos >= pd ? 1u : 0u);
+            o.token = (int32_t)idat(at);
+            o.q = qat(at);
+        }
+    }
+    if (tid == 0)
+        write_row(d, row, o);
+}
+
+// Whole-row path: exact for every parameter combination.  One workgroup rebuilds the penalised
+// row in scratch, keeps the candidates, sorts them by (q desc, idx asc) when top-k or top-p is
+// active, truncates, and draws.  src/gen/sampler.cpp:20-62.
+__device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
+                            float m, uint32_t argidx, const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t V = d.n_vocab;
+    float* wbuf = sc.wbuf + (size_t)row * sc.vpad;
+    uint32_t* cnt = sc.cnt + (size_t)row * sc.vpad;
+    uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
+    uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
+    uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
+    uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
+    const float* lrow = d.logits + (int64_t)row * d.logits_stride;
+    const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
+
+    // 1. masked copy, then the penalties once per distinct history token
+    for (uint32_t i = tid; i < V; i += kThreads) {
+        float v = lrow[i];
+        if (mrow && !((mrow[i >> 5] >> (i & 31u)) & 1u))
+            v = -INFINITY;
+        wbuf[i] = v;
+    }
+    __syncthreads();
+    const uint32_t hl = d.hist_tokens ? d.hist_len[row] : 0u;
+    if (hl > 0 && !penalties_neutral(P)) {
+        const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
+        const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
+        for (uint32_t h = tid; h < hl; h += kThreads) {
+            const uint32_t t = (uint32_t)ht[h];
+            if (t < V)
+                atomicAdd(&cnt[t], hc ? hc[h] : 1u);
+        }
+        __syncthreads();
+        for (uint32_t h = tid; h < hl; h += kThreads) {
+            const uint32_t t = (uint32_t)ht[h];
+            if (t < V) {
+                const uint32_t c = atomicExch(&cnt[t], 0u); // claims the token and restores the zero
+                if (c)
+                    wbuf[t] = penalize(wbuf[t], c, P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+            }
+        }
+        __syncthreads();
+    }
+
+    // 2. weights and the min_p / q > 0 filter, compacted in index order (sampler.cpp:29-36)
+    const float inv_t = 1.0f / P.temperature;
+    const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p; // std::min(min_p, 1.0f)
+    uint32_t n0 = 0;
+    for (uint32_t base = 0; base < V; base += kThreads * 4u) {
+        const uint32_t i = base + tid * 4u;
+        uint32_t k[4];
+        uint32_t c = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            k[j] = 0;
+            if (i + j < V) {
+                const float q = weight_of(wbuf[i + j], m, inv_t, sm.tab);
+                if (q >= floor_q && q > 0.0f) {
+                    k[j] = __float_as_uint(q);
+                    ++c;
+                }
+            }
+        }
+        uint32_t tot;
+        uint32_t pos = n0 + block_excl_scan_u32(c, tot, sm.bs);
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (k[j]) {
+                key0[pos] = ~k[j];
+                idx0[pos] = i + j;
+                ++pos;
+            }
+        n0 += tot;
+    }
+    __syncthreads();
+
+    if (n0 == 0) {
+        fallback_row(d, row, argidx);
+        return;
+    }
+
+    // 3. order by (q desc, idx asc): stable LSD radix sort of ~bits(q), ascending
+    const bool topk_active = P.top_k > 0 && P.top_k < n0;
+    const bool topp_active = P.top_p < 1.0f;
+    uint32_t *ks = key0, *is = idx0, *kd = key1, *id = idx1;
+    if (topk_active || topp_active) {
+        for (uint32_t shift = 0; shift < 32; shift += 8) {
+            if (radix_pass(ks, is, kd, id, n0, shift, L)) {
+                uint32_t* t = ks;
+                ks = kd;
+                kd = t;
+                t = is;
+                is = id;
+                id = t;
+            }
+            __syncthreads();
+        }
+    }
+    uint32_t n = topk_active ? P.top_k : n0; // sampler.cpp:40-43
+
+    // 4. top-p: shortest sorted prefix whose fp64 running sum reaches top_p * total (sampler.cpp:44-61)
+    if (topp_active) {
+        double part = 0;
+        for (uint32_t i = tid; i < n; i += kThreads)
+            part += (double)__uint_as_float(~ks[i]);
+        const double total64 = block_sum_f64(part, sm.bs);
+        const double want = (double)P.top_p * total64;
+        double carry = 0;
+        uint32_t keep = n;
+        for (uint32_t base = 0; base < n; base += kThreads) {
+            const uint32_t i = base + tid;
+            const double q = i < n ? (double)__uint_as_float(~ks[i]) : 0.0;
+            double tile;
+            const double incl = carry + block_incl_scan_f64(q, tile, sm.bs);
+            const uint32_t hit = (i < n && incl >= want) ? i : kNone;
+            const uint32_t first = block_min_u32(hit, sm.bs);
+            if (first != kNone) {
+                keep = first + 1;
+                break;
+            }
+            carry += tile;
+        }
+        n = keep;
+    }
+
+    const uint32_t* kf = ks;
+    const uint32_t* jf = is;
+    draw_from_list(
+        d, row, [=](uint32_t i) { return __uint_as_float(~kf[i]); }, [=](uint32_t i) { return jf[i]; }, n,
+        MAKO_PATH_GENERAL, sm);
+}
+
+// Bitonic sort of a[0..n), n a power of two, descending.
+__device__ void bitonic_sort_desc(unsigned long long* a, uint32_t n)
+{
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t k = 2; k <= n; k <<= 1)
+        for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+            for (uint32_t t = tid; t < n / 2; t += kThreads) {
+                const uint32_t i = ((t & ~(j - 1u)) << 1) | (t & (j - 1u));
+                const uint32_t p = i | j;
+                const unsigned long long x = a[i], y = a[p];
+                const bool desc = (i & k) == 0;
+                if ((x < y) == desc) {
+                    a[i] = y;
+                    a[p] = x;
+                }
+            }
+            __syncthreads();
+        }
+}
+
+// Exact fp64 sum of q over one slice, and the number of candidates in it (q > 0 and q >= min_p).
+// The summation order is fixed: each thread adds its logits in index order, then lanes, then waves.
+template <bool VEC>
+__device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slice,
+                              uint32_t slice_len, const mako_sampling_params& P, float m, const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t lo = slice * slice_len;
+    const uint32_t hi = min(d.n_vocab, lo + slice_len);
+    const uint32_t hl = d.hist_tokens ? d.hist_len[row] : 0u;
+    const bool pen = hl > 0 && !penalties_neutral(P);
+    if (pen)
+        build_counts(d, row, hl, lo, hi, slice_len, L.cnt);
+    float wv[16];
+    load_slice<VEC>(d, row, lo, hi, P, pen, L.cnt, wv);
+    const float inv_t = 1.0f / P.temperature;
+    const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
+    double sum = 0;
+    uint32_t n = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < 16; ++j) {
+        const float q = weight_of(wv[j], m, inv_t, sm.tab);
+        if (q >= floor_q && q > 0.0f) {
+            sum += (double)q;
+            ++n;
+        }
+    }
+    const double total = block_sum_f64(sum, sm.bs);
+    const uint32_t count = block_sum_u32(n, sm.bs);
+    if (threadIdx.x == 0) {
+        sc.part_sum[(size_t)row * kMaxSlices + slice] = total;
+        sc.part_n[(size_t)row * kMaxSlices + slice] = count;
+    }
+}
+
+// grid = (slices, rows).  Only top_k == 0 rows use more than their first workgroup.
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Scratch sc, uint32_t slices, uint32_t slice_len)
+{
+    extern __shared__ unsigned long long s_dyn64[];
+    __shared__ FinishShared sm;
+    FinishLds L;
+    L.sm = &sm;
+    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
+    L.sortk = s_dyn64;                                             // 32 KB
+    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);    // next 16 KB
+    const uint32_t row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
+    const mako_sampling_params P = d.params[row];
+    const RowClass cls = classify(P);
+    if (cls != kNucleus && slice != 0)
+        return;
+    if (tid < 32)
+        sm.tab[tid] = k_exp2_tab[tid];
+    __syncthreads();
+
+    // first maximum of the row (std::max_element semantics, NaNs never win unless at index 0)
+    unsigned long long top = 0;
+    uint32_t n_cands = 0, any_overflow = 0;
+    for (uint32_t s = 0; s < slices; ++s) {
+        const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
+        const unsigned long long p = ((unsigned long long)order_key(st.wmax) << 32) | (unsigned long long)(kNone - st.argidx);
+        top = p > top ? p : top;
+        n_cands += st.n_emit;
+        any_overflow |= st.flags & kFlagOverflow;
+    }
+    const bool first_nan = sc.stats[(size_t)row * kMaxSlices].flags & kFlagFirstNan;
+    float m = order_unkey((uint32_t)(top >> 32));
+    uint32_t argidx = kNone - (uint32_t)top;
+    if (argidx == kNone)
+        argidx = 0;
+    if (first_nan) {
+        m = __uint_as_float(0x7fc00000u);
+        argidx = 0;
+    }
+
+    if (cls == kGreedy) { // sampler.cpp:77-78, 88-92
+        if (tid == 0) {
+            RowOut o;
+            o.token = (int32_t)argidx;
+            o.n_cand = 0;
+            o.total = 0.0f;
+            o.q = 0.0f;
+            o.path = MAKO_PATH_GREEDY;
+            o.accepted = d.draft ? (d.draft[row] == (int32_t)argidx) : 0u;
+            write_row(d, row, o);
+        }
+        return;
+    }
+
+    if (cls == kNucleus) {
+        // second pass: all slices of the row in parallel; the last one to arrive finishes the row
+        slice_partial<VEC>(d, sc, row, slice, slice_len, P, m, L);
+        if (tid == 0) {
+            __threadfence();
+            sm.ticket = atomicAdd(&sc.tickets[row], 1u);
+        }
+        __syncthreads();
+        if (sm.ticket != slices - 1)
+            return;
+        __threadfence();
+        if (tid == 0)
+            sc.tickets[row] = 0;
+    }
+
+    if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
+        general_row(d, sc, row, P, m, argidx, L);
+        return;
+    }
+
+    // ---- candidate path: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
+    const float inv_t = 1.0f / P.temperature;
+    const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
+    uint32_t npad = 64;
+    while (npad < n_cands)
+        npad <<= 1;
+    // the largest weight a logit that was NOT emitted can have, over all slices (0 if none can be a candidate)
+    float q_bound = 0.0f;
+    {
+        uint32_t off = 0;
+        for (uint32_t s = 0; s < slices; ++s) {
+            const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
+            const size_t base = ((size_t)row * sc.slices_cap + s) * kCap;
+            for (uint32_t c = tid; c < st.n_emit; c += kThreads) {
+                const float q = weight_of(sc.cand_w[base + c], m, inv_t, sm.tab);
+                const uint32_t id = sc.cand_i[base + c];
+                unsigned long long k64 = 0;
+                if (q >= floor_q && q > 0.0f)
+                    k64 = ((unsigned long long)__float_as_uint(q) << 32) | (unsigned long long)(kNone - id);
+                L.sortk[off + c] = k64;
+            }
+            off += st.n_emit;
+            if (!(st.flags & kFlagComplete)) {
+                // everything left behind has an order key below tau_key
+                const float qb = weight_of(order_unkey(st.tau_key - 1u), m, inv_t, sm.tab);
+                if (qb >= floor_q && qb > 0.0f && qb > q_bound)
+                    q_bound = qb;
+            }
+        }
+        for (uint32_t c = n_cands + tid; c < npad; c += kThreads)
+            L.sortk[c] = 0;
+    }
+    __syncthreads();
+    bitonic_sort_desc(L.sortk, npad);
+    uint32_t nv = 0;
+    for (uint32_t c = tid; c < npad; c += kThreads)
+        nv += L.sortk[c] != 0;
+    const uint32_t n_valid = block_sum_u32(nv, sm.bs);
+
+    auto qat = [&](uint32_t i) { return __uint_as_float((uint32_t)(L.sortk[i] >> 32)); };
+    auto idat = [&](uint32_t i) { return kNone - (uint32_t)L.sortk[i]; };
+
+    uint32_t n1;
+    double total64;
+    if (cls == kTopK) {
+        // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
+        const bool ok = n_valid >= P.top_k ? q_bound < qat(P.top_k - 1) : q_bound == 0.0f;
+        if (!ok) {
+            general_row(d, sc, row, P, m, argidx, L);
+            return;
+        }
+        if (n_valid == 0) {
+            fallback_row(d, row, argidx);
+            return;
+        }
+        n1 = min(P.top_k, n_valid); // sampler.cpp:40-43
+        double part = 0;
+        for (uint32_t i = tid; i < n1; i += kThreads)
+            part += (double)qat(i);
+        total64 = block_sum_f64(part, sm.bs);
+    } else {
+        uint32_t n0 = 0;
+        total64 = 0;
+        for (uint32_t s = 0; s < slices; ++s) {
+            total64 += sc.part_sum[(size_t)row * kMaxSlices + s];
+            n0 += sc.part_n[(size_t)row * kMaxSlices + s];
+        }
+        if (n0 == 0) {
+            fallback_row(d, row, argidx);
+            return;
+        }
+        n1 = n_valid;
+    }
+
+    // top-p over the sorted candidates (sampler.cpp:44-61)
+    const double want = (double)P.top_p * total64;
+    double carry = 0;
+    uint32_t keep = kNone;
+    for (uint32_t base = 0; base < n1; base += kThreads) {
+        const uint32_t i = base + tid;
+        const double q = i < n1 ? (double)qat(i) : 0.0;
+        double tile;
+        const double incl = carry + block_incl_scan_f64(q, tile, sm.bs);
+        const uint32_t hit = (i < n1 && incl >= want) ? i : kNone;
+        const uint32_t first = block_min_u32(hit, sm.bs);
+        if (first != kNone) {
+            keep = first + 1;
+            break;
+        }
+        carry += tile;
+    }
+    uint32_t n;
+    if (cls == kTopK) {
+        n = keep == kNone ? n1 : keep;
+    } else {
+        // the nucleus must end inside the candidates, strictly above everything left behind
+        if (keep == kNone || !(q_bound < qat(keep - 1))) {
+            general_row(d, sc, row, P, m, argidx, L);
+            return;
+        }
+        n = keep;
+    }
+    draw_from_list(d, row, qat, idat, n, cls == kTopK ? MAKO_PATH_TOPK : MAKO_PATH_NUCLEUS, sm);
+}
+
+__global__ void debug_expf_kernel(const float* x, float* y, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        y[i] = expf_glibc(x[i], k_exp2_tab);
+}
+
+__global__ void debug_div_kernel(const float* a, const float* b, float* y, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        y[i] = a[i] / b[i];
+}
+
+} // namespace mako
