@@ -156,9 +156,13 @@ static void heap_sift(cand_t* h, long hole, long len, cand_t v)
     h[hole] = v;
 }
 
+static long g_heap_selects; /* times introselect fell back to heap_select (test hook) */
+long or_debug_heap_selects(void) { return g_heap_selects; }
+
 /* libstdc++ 11.4 bits/stl_algo.h __heap_select. */
 static void heap_select(cand_t* a, long middle, long last)
 {
+    ++g_heap_selects;
     if (middle >= 2)
         for (long parent = (middle - 2) / 2;; --parent) {
             heap_sift(a, parent, middle, a[parent]);

@@ -78,6 +78,8 @@ int32_t or_verify(const float* logits, uint32_t n_vocab, const or_params* p,
 /* libstdc++ nth_element restated, exposed for its own pin test:
  * keys are (q, idx) pairs ordered by (q desc, idx asc). */
 void or_nth_element(float* q, int32_t* idx, uint32_t n, uint32_t nth);
+/* Number of times the restated introselect took its heap-select branch (test hook). */
+long or_debug_heap_selects(void);
 
 #ifdef __cplusplus
 }

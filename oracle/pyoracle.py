@@ -94,6 +94,10 @@ class _Oracle:
                                   C.c_uint32, C.POINTER(C.c_uint32), C.c_int32, C.c_float, C.c_float, C.c_int,
                                   C.POINTER(C.c_int), C.POINTER(Trace)]
         lib.or_nth_element.argtypes = [C.POINTER(C.c_float), C.POINTER(C.c_int32), C.c_uint32, C.c_uint32]
+        lib.or_debug_heap_selects.restype = C.c_long
+
+    def heap_selects(self):
+        return self.lib.or_debug_heap_selects()
 
     def expf(self, x):
         return self.lib.or_expf(float(x))
@@ -151,6 +155,8 @@ class _Reference:
         lib.ref_verify.argtypes = [C.POINTER(C.c_float), C.c_uint32, C.POINTER(Params), C.POINTER(C.c_int32),
                                    C.c_uint32, C.POINTER(C.c_uint32), C.c_uint64, C.c_int32, C.POINTER(C.c_int)]
         lib.ref_nth_element.argtypes = [C.POINTER(C.c_float), C.POINTER(C.c_int32), C.c_uint32, C.c_uint32]
+        lib.ref_make_nth_killer.restype = C.c_long
+        lib.ref_make_nth_killer.argtypes = [C.c_uint32, C.c_uint32, C.POINTER(C.c_float)]
         lib.ref_libm_expf.restype = C.c_float
         lib.ref_libm_expf.argtypes = [C.c_float]
         lib.ref_sample_batch_timed.restype = C.c_double
@@ -196,6 +202,11 @@ class _Reference:
         idx = np.array(idx, np.int32)
         self.lib.ref_nth_element(_fp(q), _ip(idx), q.size, nth)
         return q, idx
+
+    def make_nth_killer(self, n, nth):
+        q = np.zeros(n, np.float32)
+        ncmp = self.lib.ref_make_nth_killer(n, nth, _fp(q))
+        return q, ncmp
 
     def libm_expf(self, x):
         return self.lib.ref_libm_expf(float(x))

@@ -114,6 +114,38 @@ void ref_nth_element(float* q, int32_t* idx, uint32_t n, uint32_t nth)
 
 float ref_libm_expf(float x) { return std::exp(x); }
 
+// A worst-case input for libstdc++'s nth_element (McIlroy's adversary, "A Killer Adversary for
+// Quicksort", 1999): the comparator decides the values lazily so that every pivot is bad, which drives
+// __introselect into its depth limit and its heap-select branch.  q_out[i] is the weight of item i such
+// that ordering by (q desc, idx asc) replays the same comparisons.  Returns the comparisons made.
+long ref_make_nth_killer(uint32_t n, uint32_t nth, float* q_out)
+{
+    std::vector<int> val(n, int(n) - 1), items(n);
+    const int gas = int(n) - 1;
+    int nsolid = 0, candidate = 0;
+    long ncmp = 0;
+    for (uint32_t i = 0; i < n; ++i)
+        items[i] = int(i);
+    auto less = [&](int x, int y) {
+        ++ncmp;
+        if (val[x] == gas && val[y] == gas) {
+            if (x == candidate)
+                val[x] = nsolid++;
+            else
+                val[y] = nsolid++;
+        }
+        if (val[x] == gas)
+            candidate = x;
+        else if (val[y] == gas)
+            candidate = y;
+        return val[x] < val[y] || (val[x] == val[y] && x < y);
+    };
+    std::nth_element(items.begin(), items.begin() + nth, items.end(), less);
+    for (uint32_t i = 0; i < n; ++i)
+        q_out[i] = float(int(n) - val[i]);
+    return ncmp;
+}
+
 // Timed CPU baseline: one fresh Sampler per row, history replayed through
 // accept() (untimed), then sample() timed.  Rows are split statically over
 // n_threads threads.  Masks are applied to a private copy before timing.

@@ -1,0 +1,254 @@
+"""CPU tests: the oracle against the reference's own test vectors, against the golden vectors recorded from the
+compiled reference, against libm / libstdc++ behaviour, and against brute force.  No GPU needed."""
+import ctypes
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from oracle import pyoracle
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "golden"))
+
+LOGITS = np.array([2.0, 1.5, 0.3, -0.5, 1.9, -2.0, 0.0, 1.0], np.float32)  # tests/sampler_test.cpp:56
+P = pyoracle.make_params
+
+
+def softmax64(l, t):
+    # the double-precision helper of tests/sampler_test.cpp:23-34
+    x = (np.asarray(l, np.float64) - np.max(l)) / t
+    e = np.exp(x)
+    return e / e.sum()
+
+
+# ---------------------------------------------------------------- the reference's own checks
+
+
+def test_greedy_and_greedy_verify(oracle):
+    # tests/sampler_test.cpp:61-67
+    assert oracle.sample(LOGITS, P(0.0), 0.5)[0] == 0
+    assert oracle.verify(LOGITS, P(0.0), 4, 0.5, 0.5) == (0, False)
+    assert oracle.verify(LOGITS, P(0.0), 0, 0.5, 0.5) == (0, True)
+
+
+def test_truncation_sets(oracle):
+    # tests/sampler_test.cpp:91-117: top_k 3 and top_p 0.7 keep {0, 4, 1}; min_p 0.3 keeps {0, 1, 4, 7}
+    _, tr = oracle.sample(LOGITS, P(1.0, top_k=3), 0.1, cap=8)
+    assert sorted(tr["cand_idx"].tolist()) == [0, 1, 4]
+    _, tr = oracle.sample(LOGITS, P(1.0, top_p=0.7), 0.1, cap=8)
+    assert tr["cand_idx"].tolist() == [0, 4, 1]
+    _, tr = oracle.sample(LOGITS, P(1.0, min_p=0.3), 0.1, cap=8)
+    assert sorted(tr["cand_idx"].tolist()) == [0, 1, 4, 7]
+    # the full distribution against the double-precision softmax of tests/sampler_test.cpp:23-34 (the rounded
+    # figures quoted in the comment at :105 agree with it to 0.007)
+    _, tr = oracle.sample(LOGITS, P(1.0), 0.1, cap=8)
+    p = tr["cand_q"] / tr["cand_q"].sum()
+    assert np.allclose(p, softmax64(LOGITS, 1.0), rtol=1e-5)
+    assert np.allclose(p, [0.297, 0.180, 0.054, 0.024, 0.269, 0.004, 0.040, 0.109], atol=7e-3)
+
+
+def test_penalties_known_answers(oracle):
+    # tests/sampler_test.cpp:118-134
+    _, tr = oracle.sample(LOGITS, P(1.0, presence_penalty=0.5, frequency_penalty=0.25), 0.1, hist=[0, 0], cap=8)
+    pen = LOGITS.copy()
+    pen[0] -= 1.0
+    assert np.allclose(tr["cand_q"] / tr["cand_q"].sum(), softmax64(pen, 1.0), rtol=1e-5)
+    _, tr = oracle.sample(LOGITS, P(1.0, repetition_penalty=2.0), 0.1, hist=[0, 5], cap=8)
+    rp = LOGITS.copy()
+    rp[0] /= 2.0
+    rp[5] *= 2.0
+    assert np.allclose(tr["cand_q"] / tr["cand_q"].sum(), softmax64(rp, 1.0), rtol=1e-5)
+
+
+def test_edge_cases(oracle):
+    # tests/sampler_test.cpp:135-144
+    assert oracle.sample(LOGITS, P(1e-40), 0.9)[0] == 0
+    t, _ = oracle.sample(LOGITS, P(1.0, repetition_penalty=0.0), 0.3, hist=[0, 4])
+    assert 0 <= t < 8
+    # top_p <= 0 keeps one candidate; u = 0 returns the first candidate; u -> 1 the last
+    assert oracle.sample(LOGITS, P(1.0, top_p=0.0), 0.99)[1]["n_cand"] == 1
+    assert oracle.sample(LOGITS, P(1.0, top_p=0.9), 0.0)[0] == 0
+    t, tr = oracle.sample(LOGITS, P(1.0), np.nextafter(np.float32(1), np.float32(0)), cap=8)
+    assert t == 7
+
+
+@pytest.mark.parametrize("t", [1.0, 0.7])
+def test_sample_distribution(oracle, t):
+    # tests/sampler_test.cpp:68-75 with 100k draws: max |hist - softmax| < 0.006
+    rng = np.random.default_rng(3)
+    us = rng.random(100000).astype(np.float32)
+    hist = np.zeros(8)
+    for u in us:
+        hist[oracle.sample(LOGITS, P(t), float(u))[0]] += 1
+    assert np.abs(hist / len(us) - softmax64(LOGITS, t)).max() < 0.006
+
+
+@pytest.mark.parametrize("draft", [0, 4, 5])
+def test_verify_distribution(oracle, draft):
+    # tests/sampler_test.cpp:76-89: verify() reproduces the distribution and accepts at rate p[draft]
+    rng = np.random.default_rng(10 + draft)
+    n = 100000
+    us = rng.random((n, 2)).astype(np.float32)
+    hist = np.zeros(8)
+    acc = 0
+    for u1, u2 in us:
+        tok, a = oracle.verify(LOGITS, P(1.0), draft, float(u1), float(u2))
+        hist[tok] += 1
+        acc += a
+    want = softmax64(LOGITS, 1.0)
+    assert np.abs(hist / n - want).max() < 0.006
+    assert abs(acc / n - want[draft]) < 0.006
+    # a draft outside the top 3 is never accepted (tests/sampler_test.cpp:97-102)
+    for u1, u2 in us[:2000]:
+        assert not oracle.verify(LOGITS, P(1.0, top_k=3), 7, float(u1), float(u2))[1]
+
+
+# ---------------------------------------------------------------- golden vectors from the compiled reference
+
+
+def _golden():
+    with open(os.path.join(HERE, "golden", "reference_vectors.json")) as f:
+        return json.load(f)
+
+
+def test_golden_vectors(oracle):
+    """Every recorded row: same token, same candidate count, same candidate list (ids, weight bits, order) and
+    same fp32 total as the unmodified reference produced."""
+    import make_golden
+    from mako_amd import workloads
+    gold = {c["name"]: c for c in _golden()["cases"]}
+    checked = 0
+    for name, w, rows in make_golden.cases():
+        g = gold[name]
+        assert workloads.input_digest(w) == g["input_digest"], "input generator drifted for " + name
+        v = w["logits"].shape[1]
+        for rec in g["rows"]:
+            r = rec["row"]
+            p = pyoracle.params_from_record(w["params"][r])
+            hist = w["hist"][r, : w["hist_len"][r]] if "hist" in w else None
+            mask = w["mask"][r] if "mask" in w else None
+            u = float(oracle.uniforms(rec["seed"], 1)[0])
+            t, tr = oracle.sample(w["logits"][r], p, u, hist, mask, order_mode=0, cap=v)
+            assert t == rec["token"], (name, r)
+            if p.temperature <= 0:
+                continue
+            assert tr["n_cand"] == rec["n_cand"], (name, r)
+            assert make_golden.list_digest(tr["cand_idx"], tr["cand_q"]) == rec["list_digest"], (name, r)
+            assert int(np.float32(tr["total"]).view(np.uint32)) == rec["total_bits"], (name, r)
+            checked += 1
+    assert checked > 100
+
+
+def test_nth_element_killers(oracle):
+    """Worst-case inputs recorded from libstdc++: the restated introselect must take its heap-select branch and
+    leave exactly the arrangement std::nth_element left."""
+    import make_golden
+    for k in _golden()["nth_killers"]:
+        q = np.array(k["q"], np.float32)
+        before = oracle.heap_selects()
+        rq, ri = oracle.nth_element(q, np.arange(k["n"], dtype=np.int32), k["nth"])
+        assert oracle.heap_selects() == before + 1
+        assert make_golden.list_digest(ri, rq) == k["result_digest"]
+
+
+def test_nth_element_partitions(oracle):
+    """Brute force: after nth_element position nth holds the nth element of the full order and splits the rest."""
+    rng = np.random.default_rng(5)
+    for _ in range(300):
+        n = int(rng.integers(1, 300))
+        nth = int(rng.integers(0, n))
+        q = rng.choice(rng.random(max(1, n // 3)).astype(np.float32), n)
+        idx = rng.permutation(n).astype(np.int32)
+        rq, ri = oracle.nth_element(q, idx, nth)
+        order = sorted(zip((-q).tolist(), idx.tolist()))
+        assert (-rq[nth], ri[nth]) == order[nth]
+        assert sorted(zip((-rq[:nth]).tolist(), ri[:nth].tolist())) == order[:nth]
+
+
+# ---------------------------------------------------------------- third-party arithmetic
+
+
+def test_expf_matches_libm(oracle):
+    """The restated glibc expf equals this host's libm on 3M inputs: the sampler's whole argument range densely,
+    random bit patterns, and the special cases."""
+    libm = ctypes.CDLL("libm.so.6")
+    libm.expf.restype = ctypes.c_float
+    libm.expf.argtypes = [ctypes.c_float]
+    rng = np.random.default_rng(11)
+    xs = np.concatenate([
+        -np.abs(rng.standard_normal(200000) * 30).astype(np.float32),
+        rng.integers(0, 2**32, 200000, dtype=np.uint64).astype(np.uint32).view(np.float32),
+        np.linspace(-104.2, -102.9, 20000).astype(np.float32),
+        np.array([0.0, -0.0, np.inf, -np.inf, 88.0, 88.72, 88.73, -87.9, -103.27, -103.28, -103.97, -103.98, -1e-38,
+                  1e-38, -1e-45], np.float32)])
+    bad = 0
+    for x in xs:
+        a, b = oracle.expf(x), libm.expf(float(x))
+        if not (a == b or (a != a and b != b)):
+            bad += 1
+    assert bad == 0
+    assert oracle.expf(0.0) == 1.0 and oracle.expf(-np.inf) == 0.0 and np.isnan(oracle.expf(np.nan))
+
+
+def test_expf_exhaustive_and_monotone():
+    """All 2^32 inputs against libm, and monotonicity over every negative float (C helper, ~10 s on 8 threads)."""
+    exe = os.path.join(HERE, "cpu", "expf_pin")
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-mfma", "-pthread", "-I", os.path.join(HERE, "..", "oracle"),
+                    os.path.join(HERE, "cpu", "expf_pin.c"), os.path.join(HERE, "..", "oracle", "oracle.c"), "-o", exe,
+                    "-lm"], check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
+    assert "mismatches 0" in out and "non-monotone 0" in out, out
+
+
+def test_uniforms_known_answers(oracle):
+    """mt19937_64: the 10000th output for the default seed is 9981545732273789042 (ISO C++ [rand.predef]); the
+    float mapping is float(x) / 2^64 with 1.0 replaced by the float below it."""
+    u = oracle.uniforms(5489, 10000)
+    first, last = 14514284786278117030, 9981545732273789042
+    assert u[0] == np.float32(first) / np.float32(2.0**64)
+    assert u[-1] == np.float32(last) / np.float32(2.0**64)
+    assert (u >= 0).all() and (u < 1).all()
+
+
+def test_seqfp_host():
+    """The integer-map emulation of sequential fp32 sums and walks (shared with the kernels) against real fp32
+    loops on 28000 random cases."""
+    exe = os.path.join(HERE, "cpu", "seqfp_test")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", os.path.join(HERE, "cpu", "seqfp_test.cpp"), "-o",
+                    exe], check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
+    assert " 0 failures" in out, out
+
+
+# ---------------------------------------------------------------- oracle vs the compiled reference, where built
+
+
+def test_oracle_equals_reference(oracle, reference):
+    rng = np.random.default_rng(1)
+    for seed in [0, 1, 5489, 2**63 + 7, 2**64 - 1]:
+        assert np.array_equal(oracle.uniforms(seed, 700).view(np.uint32), reference.uniforms(seed, 700).view(np.uint32))
+    for it in range(250):
+        v = int(rng.choice([8, 100, 1000, 4096, 20000]))
+        logits = (rng.standard_normal(v) * 3).astype(np.float32)
+        if it % 3 == 0:
+            logits = np.round(logits * 4) / 4
+        p = P(float(rng.choice([0.0, 0.3, 0.7, 1.0, 1.2, 1e-40])), int(rng.choice([0, 0, 1, 3, 20, 50, 100, v, v + 5])),
+              float(rng.choice([1.0, 0.95, 0.9, 0.5, 0.0, 1.5])), float(rng.choice([0.0, 0.0, 0.05, 0.3, 2.0])),
+              float(rng.choice([0, 0.3])), float(rng.choice([0, 0.2])), float(rng.choice([1.0, 1.1, 2.0, 0.0])))
+        hist = rng.integers(0, v, int(rng.choice([0, 5, 512]))).astype(np.int32)
+        mask = rng.integers(0, 2**32, (v + 31) // 32, dtype=np.uint64).astype(np.uint32) if it % 4 == 1 else None
+        seed = int(rng.integers(0, 2**63))
+        u1, u2 = oracle.uniforms(seed, 2)
+        t1, tr1 = oracle.sample(logits, p, float(u1), hist, mask, order_mode=0, cap=v)
+        t2, tr2 = reference.sample(logits, p, seed, hist, mask, cap=v)
+        assert t1 == t2, it
+        if p.temperature > 0:
+            assert tr1["n_cand"] == tr2["n_cand"] and np.array_equal(tr1["cand_idx"], tr2["cand_idx"]), it
+            assert np.array_equal(tr1["cand_q"].view(np.uint32), tr2["cand_q"].view(np.uint32)), it
+        draft = int(rng.integers(0, v)) if it % 2 else t1
+        got = oracle.verify(logits, p, draft, float(u1), float(u2), hist, mask, order_mode=0)
+        assert got == reference.verify(logits, p, seed, draft, hist, mask), it
