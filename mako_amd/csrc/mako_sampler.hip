@@ -107,8 +107,12 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, hipMemset(sc.cnt, 0, rv * sizeof(uint32_t)));
     MAKO_HIP(ctx, hipDeviceSynchronize());
     // both kernels overlay up to 64 KB of dynamic LDS on a few KB of static LDS
-    const void* kernels[] = {(const void*)mako::scan_kernel<true>, (const void*)mako::scan_kernel<false>,
-                             (const void*)mako::finish_kernel<true>, (const void*)mako::finish_kernel<false>};
+    const void* kernels[] = {(const void*)mako::scan_kernel<true, 0>,    (const void*)mako::scan_kernel<false, 0>,
+                             (const void*)mako::scan_kernel<true, 2>,    (const void*)mako::scan_kernel<false, 2>,
+                             (const void*)mako::scan_kernel<true, 8>,    (const void*)mako::scan_kernel<false, 8>,
+                             (const void*)mako::finish_kernel<true, 0>,  (const void*)mako::finish_kernel<false, 0>,
+                             (const void*)mako::finish_kernel<true, 2>,  (const void*)mako::finish_kernel<false, 2>,
+                             (const void*)mako::finish_kernel<true, 8>,  (const void*)mako::finish_kernel<false, 8>};
     for (const void* k : kernels)
         MAKO_HIP(ctx, hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)mako::kDynLds));
     return MAKO_OK;
@@ -165,16 +169,27 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     const bool vec = d.n_vocab % 4 == 0 && d.logits_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(d.logits) & 15u) == 0;
     const size_t lds = d.hist_tokens ? (size_t)slice_len * sizeof(uint32_t) : 0;
     const dim3 grid(slices, d.n_rows);
-    if (vec)
-        hipLaunchKernelGGL(mako::scan_kernel<true>, grid, dim3(mako::kThreads), lds, st, d, ctx->sc, slice_len);
+    // histories of up to 2 (8) entries per thread stay in registers; longer ones take the generic route
+    const int kh = !d.hist_tokens ? 2 : (d.hist_stride <= 2 * mako::kThreads ? 2 : (d.hist_stride <= 8 * mako::kThreads ? 8 : 0));
+#define MAKO_LAUNCH(V, K)                                                                                          \
+    do {                                                                                                           \
+        hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc, slice_len); \
+        hipLaunchKernelGGL((mako::finish_kernel<V, K>), grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc, \
+                           slices, slice_len);                                                                     \
+    } while (0)
+    if (vec && kh == 2)
+        MAKO_LAUNCH(true, 2);
+    else if (vec && kh == 8)
+        MAKO_LAUNCH(true, 8);
+    else if (vec)
+        MAKO_LAUNCH(true, 0);
+    else if (kh == 2)
+        MAKO_LAUNCH(false, 2);
+    else if (kh == 8)
+        MAKO_LAUNCH(false, 8);
     else
-        hipLaunchKernelGGL(mako::scan_kernel<false>, grid, dim3(mako::kThreads), lds, st, d, ctx->sc, slice_len);
-    if (vec)
-        hipLaunchKernelGGL(mako::finish_kernel<true>, grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc, slices,
-                           slice_len);
-    else
-        hipLaunchKernelGGL(mako::finish_kernel<false>, grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc, slices,
-                           slice_len);
+        MAKO_LAUNCH(false, 0);
+#undef MAKO_LAUNCH
     MAKO_HIP(ctx, hipGetLastError());
     return MAKO_OK;
 }

@@ -27,7 +27,7 @@ namespace mako {
 constexpr uint32_t kNone = 0xffffffffu;
 constexpr uint32_t kSliceMax = 16384; // elements per slice: 16 per thread
 constexpr uint32_t kMaxSlices = 64;
-constexpr uint32_t kCap = 256;       // candidates kept per slice
+constexpr uint32_t kCap = 512;       // candidates kept per slice
 constexpr uint32_t kTopKFast = 128;  // largest top_k resolved from the per-slice candidates
 constexpr uint32_t kSortMax = 4096;  // candidates the finisher sorts in LDS
 constexpr uint32_t kDynLds = 65536;  // dynamic LDS of both kernels
@@ -104,13 +104,15 @@ __device__ __forceinline__ uint32_t elem_index(uint32_t lo, uint32_t tid, uint32
     return VEC ? lo + (j >> 2) * 4096u + tid * 4u + (j & 3u) : lo + j * (uint32_t)kThreads + tid;
 }
 
-// accept() history -> per-token counts for [lo, hi) in LDS (src/gen/sampler.cpp:15-18).
+// accept() history -> per-token counts for [lo, hi) in LDS (src/gen/sampler.cpp:15-18); generic form used
+// when a row's history is too long for the register-resident scheme of load_penalised().
 __device__ __forceinline__ void build_counts(const mako_sample_desc& d, uint32_t row, uint32_t hl, uint32_t lo,
                                              uint32_t hi, uint32_t slice_len, uint32_t* s_cnt)
 {
     const uint32_t tid = threadIdx.x;
-    for (uint32_t i = tid; i < slice_len; i += kThreads)
-        s_cnt[i] = 0;
+    uint4* z = reinterpret_cast<uint4*>(s_cnt); // slice_len is a multiple of 4
+    for (uint32_t i = tid; i < slice_len / 4; i += kThreads)
+        z[i] = make_uint4(0, 0, 0, 0);
     __syncthreads();
     const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
     const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
@@ -122,60 +124,224 @@ __device__ __forceinline__ void build_counts(const mako_sample_desc& d, uint32_t
     __syncthreads();
 }
 
-// The thread's 16 logits after the mask and the penalties (src/gen/sampler.cpp:22-28); slots past the
-// end of the slice hold NaN, which never wins a comparison and never becomes a candidate.
+// The thread's 16 logits, raw, plus the mask bits of each group of four (VEC) or of each logit (scalar).
+// Issued before anything else so that the HBM latency overlaps the LDS work that follows.
 template <bool VEC>
-__device__ __forceinline__ void load_slice(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi,
-                                           const mako_sampling_params& P, bool pen, const uint32_t* s_cnt, float (&wv)[16])
+struct RawSlice {
+    float4 v[4];
+    uint32_t bits[4]; // VEC: bit c of bits[k] = logit 4k+c allowed; scalar: bit j of bits[0] = logit j allowed
+};
+
+template <bool VEC>
+__device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi, RawSlice<VEC>& r)
 {
     const uint32_t tid = threadIdx.x;
     const float* lrow = d.logits + (int64_t)row * d.logits_stride;
     const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
     const float nan = __uint_as_float(0x7fc00000u);
     if (VEC) {
-        float4 v[4];
-        uint32_t bits[4];
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k) {
             const uint32_t i = lo + k * 4096u + tid * 4u;
-            bits[k] = 0xfu;
+            r.bits[k] = 0xfu;
             if (i < hi) { // hi - lo is a multiple of 4 in this mode
-                v[k] = *reinterpret_cast<const float4*>(lrow + i);
+                r.v[k] = *reinterpret_cast<const float4*>(lrow + i);
                 if (mrow)
-                    bits[k] = mrow[i >> 5] >> (i & 31u);
+                    r.bits[k] = mrow[i >> 5] >> (i & 31u);
             } else {
-                v[k] = make_float4(nan, nan, nan, nan);
+                r.v[k] = make_float4(nan, nan, nan, nan);
             }
         }
+    } else {
+        float* f = reinterpret_cast<float*>(r.v);
+        uint32_t allowed = 0xffffu;
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) {
+            const uint32_t i = lo + j * (uint32_t)kThreads + tid;
+            f[j] = nan;
+            if (i < hi) {
+                f[j] = lrow[i];
+                if (mrow && !((mrow[i >> 5] >> (i & 31u)) & 1u))
+                    allowed &= ~(1u << j);
+            }
+        }
+        r.bits[0] = allowed;
+    }
+}
+
+// Mask and penalties (src/gen/sampler.cpp:22-28) applied to the raw logits; slots past the end of the
+// slice hold NaN, which never wins a comparison and never becomes a candidate.
+template <bool VEC>
+__device__ __forceinline__ void finish_slice(const RawSlice<VEC>& r, uint32_t lo, uint32_t hi, const mako_sampling_params& P,
+                                             bool pen, const uint32_t* s_cnt, float (&wv)[16])
+{
+    const uint32_t tid = threadIdx.x;
+    if (VEC) {
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k) {
-            wv[4 * k + 0] = (bits[k] & 1u) ? v[k].x : -INFINITY;
-            wv[4 * k + 1] = (bits[k] & 2u) ? v[k].y : -INFINITY;
-            wv[4 * k + 2] = (bits[k] & 4u) ? v[k].z : -INFINITY;
-            wv[4 * k + 3] = (bits[k] & 8u) ? v[k].w : -INFINITY;
+            wv[4 * k + 0] = (r.bits[k] & 1u) ? r.v[k].x : -INFINITY;
+            wv[4 * k + 1] = (r.bits[k] & 2u) ? r.v[k].y : -INFINITY;
+            wv[4 * k + 2] = (r.bits[k] & 4u) ? r.v[k].z : -INFINITY;
+            wv[4 * k + 3] = (r.bits[k] & 8u) ? r.v[k].w : -INFINITY;
+        }
+    } else {
+        const float* f = reinterpret_cast<const float*>(r.v);
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j)
+            wv[j] = ((r.bits[0] >> j) & 1u) ? f[j] : -INFINITY;
+    }
+    if (pen) {
+        if (VEC) {
+#pragma unroll
+            for (uint32_t k = 0; k < 4; ++k) {
+                const uint32_t i = lo + k * 4096u + tid * 4u;
+                if (i < hi) {
+                    const uint4 n = *reinterpret_cast<const uint4*>(s_cnt + (i - lo));
+                    if (n.x | n.y | n.z | n.w) {
+                        if (n.x)
+                            wv[4 * k + 0] = penalize(wv[4 * k + 0], n.x, P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+                        if (n.y)
+                            wv[4 * k + 1] = penalize(wv[4 * k + 1], n.y, P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+                        if (n.z)
+                            wv[4 * k + 2] = penalize(wv[4 * k + 2], n.z, P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+                        if (n.w)
+                            wv[4 * k + 3] = penalize(wv[4 * k + 3], n.w, P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j) {
+                const uint32_t i = lo + j * (uint32_t)kThreads + tid;
+                if (i < hi) {
+                    const uint32_t n = s_cnt[i - lo];
+                    if (n)
+                        wv[j] = penalize(wv[j], n, P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+                }
+            }
+        }
+    }
+}
+
+// Logits that moved out of their owner's registers: the thread that handles history entry h keeps the
+// penalised logit of that token (if it is the token's first entry) as an extra element of its own.
+template <int KH>
+struct Extras {
+    float v[KH > 0 ? KH : 1];
+    uint32_t i[KH > 0 ? KH : 1];
+};
+
+// The thread's logits after the mask and the penalties (src/gen/sampler.cpp:22-28): wv[16] in the slice
+// layout plus up to KH extras.
+//
+// KH > 0 (histories of at most KH * 1024 entries): thread t handles history entries t, t + 1024, ...  The
+// per-token counts are accumulated in LDS; for every distinct token of the slice the thread holding its first
+// entry computes the penalised logit once (one IEEE division per history entry instead of one per logit
+// slot) and keeps it as an extra, and the logit's owner drops it (NaN).  The election of the first entry
+// makes the arrangement, and with it every later summation order, deterministic.
+// KH == 0: any history length; counts in LDS, every owner penalises its own logits.
+template <bool VEC, int KH>
+__device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi,
+                                               uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, bool pen,
+                                               uint32_t* s_cnt, float (&wv)[16], Extras<KH>& ex)
+{
+    const uint32_t tid = threadIdx.x;
+    const float nan = __uint_as_float(0x7fc00000u);
+    RawSlice<VEC> raw;
+    load_raw<VEC>(d, row, lo, hi, raw);
+#pragma unroll
+    for (int k = 0; k < (KH > 0 ? KH : 1); ++k) {
+        ex.v[k] = nan;
+        ex.i[k] = kNone;
+    }
+    if (!pen) {
+        finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv);
+        return;
+    }
+    if (KH == 0) {
+        build_counts(d, row, hl, lo, hi, slice_len, s_cnt);
+        finish_slice<VEC>(raw, lo, hi, P, true, s_cnt, wv);
+        return;
+    }
+    // my history entries, and the masked raw logits of those that fall into this slice
+    const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
+    const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
+    const float* lrow = d.logits + (int64_t)row * d.logits_stride;
+    const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
+    uint32_t tok[KH > 0 ? KH : 1], cnt[KH > 0 ? KH : 1];
+    float rawv[KH > 0 ? KH : 1];
+#pragma unroll
+    for (int k = 0; k < KH; ++k) {
+        const uint32_t h = tid + (uint32_t)k * kThreads;
+        tok[k] = kNone;
+        cnt[k] = 1;
+        if (h < hl) {
+            tok[k] = (uint32_t)ht[h];
+            if (hc)
+                cnt[k] = hc[h];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < KH; ++k) {
+        rawv[k] = nan;
+        if (tok[k] >= lo && tok[k] < hi) {
+            rawv[k] = lrow[tok[k]];
+            if (mrow && !((mrow[tok[k] >> 5] >> (tok[k] & 31u)) & 1u))
+                rawv[k] = -INFINITY;
+        } else {
+            tok[k] = kNone;
+        }
+    }
+    uint4* z = reinterpret_cast<uint4*>(s_cnt); // slice_len is a multiple of 4
+    for (uint32_t i = tid; i < slice_len / 4; i += kThreads)
+        z[i] = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < KH; ++k)
+        if (tok[k] != kNone)
+            atomicAdd(&s_cnt[tok[k] - lo], cnt[k]);
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < KH; ++k)
+        if (tok[k] != kNone)
+            cnt[k] = s_cnt[tok[k] - lo]; // occurrences of the token in the whole history
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < KH; ++k)
+        if (tok[k] != kNone)
+            s_cnt[tok[k] - lo] = 0xffffffffu;
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < KH; ++k)
+        if (tok[k] != kNone)
+            atomicMin(&s_cnt[tok[k] - lo], tid + (uint32_t)k * kThreads + 1u);
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < KH; ++k)
+        if (tok[k] != kNone && s_cnt[tok[k] - lo] == tid + (uint32_t)k * kThreads + 1u) {
+            ex.v[k] = penalize(rawv[k], cnt[k], P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+            ex.i[k] = tok[k];
+        }
+    finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv);
+    // owners drop the logits that now live in an extra
+    if (VEC) {
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            const uint32_t i = lo + k * 4096u + tid * 4u;
+            if (i < hi) {
+                const uint4 n = *reinterpret_cast<const uint4*>(s_cnt + (i - lo));
+                wv[4 * k + 0] = n.x ? nan : wv[4 * k + 0];
+                wv[4 * k + 1] = n.y ? nan : wv[4 * k + 1];
+                wv[4 * k + 2] = n.z ? nan : wv[4 * k + 2];
+                wv[4 * k + 3] = n.w ? nan : wv[4 * k + 3];
+            }
         }
     } else {
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j) {
             const uint32_t i = lo + j * (uint32_t)kThreads + tid;
-            float v = nan;
-            if (i < hi) {
-                v = lrow[i];
-                if (mrow && !((mrow[i >> 5] >> (i & 31u)) & 1u))
-                    v = -INFINITY;
-            }
-            wv[j] = v;
-        }
-    }
-    if (pen) {
-#pragma unroll
-        for (uint32_t j = 0; j < 16; ++j) {
-            const uint32_t i = elem_index<VEC>(lo, tid, j);
-            if (i < hi) {
-                const uint32_t n = s_cnt[i - lo];
-                if (n)
-                    wv[j] = penalize(wv[j], n, P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
-            }
+            if (i < hi && s_cnt[i - lo])
+                wv[j] = nan;
         }
     }
 }
@@ -185,59 +351,31 @@ __device__ __forceinline__ void load_slice(const mako_sample_desc& d, uint32_t r
 // ---------------------------------------------------------------------------------------------
 
 struct ScanShared {
-    BlockScratch bs;
-    uint32_t sel[2][kWaves][16];
+    uint32_t wave_max[kWaves]; // order keys
+    uint32_t wave_kth[kWaves];
+    uint32_t argidx;
     uint32_t emit_n;
+    uint32_t emit_flags;
     float cw[kCap];
     uint32_t ci[kCap];
 };
 
-// A key `tau` such that at least K of the workgroup's 1024 keys are >= tau, found by a most-significant-
-// digit-first radix select with 4-bit digits: per round every wavefront counts its keys per digit value
-// with ballots, the counts meet in LDS, and the digit holding the K-th largest key is fixed.  The search
-// stops early once at most 8 surplus keys share the bucket; the bucket's lower edge is returned.
-__device__ __forceinline__ uint32_t select_kth_key(uint32_t key, uint32_t K, ScanShared& sm)
+// The j-th largest of the wavefront's 64 keys (j >= 1): the largest v with at least j keys >= v, built
+// bit by bit from the top.  One vector compare per bit; the rest is scalar.
+__device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 {
-    const int lane = lane_id(), wave = wave_id();
-    uint32_t prefix = 0, need = K;
-    for (int round = 0; round < 8; ++round) {
-        const int shift = 28 - 4 * round;
-        const bool active = round == 0 || (key >> (shift + 4)) == (prefix >> (shift + 4));
-        const uint32_t dg = (key >> shift) & 15u;
-        uint32_t mine = 0;
+    uint32_t prefix = 0;
 #pragma unroll
-        for (uint32_t dv = 0; dv < 16; ++dv) {
-            const uint32_t c = (uint32_t)__popcll(__ballot(active && dg == dv));
-            if ((uint32_t)lane == dv)
-                mine = c;
-        }
-        if (lane < 16)
-            sm.sel[round & 1][wave][lane] = mine;
-        __syncthreads();
-        uint32_t col = 0;
-        if (lane < 16)
-            for (int w = 0; w < kWaves; ++w)
-                col += sm.sel[round & 1][w][lane];
-        uint32_t suf = col; // keys of this bucket with digit >= lane
-        for (int o = 1; o < 16; o <<= 1) {
-            const uint32_t t = __shfl_down(suf, o);
-            if (lane + o < 16)
-                suf += t;
-        }
-        const unsigned long long bal = __ballot(lane < 16 && suf >= need) & 0xffffull;
-        const int D = 63 - __clzll(bal); // bal != 0: the bucket holds at least `need` keys
-        const uint32_t above = D < 15 ? (uint32_t)__shfl(suf, D + 1) : 0u;
-        const uint32_t in_d = (uint32_t)__shfl(col, D);
-        need -= above;
-        prefix |= (uint32_t)D << shift;
-        if (in_d - need <= 8u)
-            break;
+    for (int b = 31; b >= 0; --b) {
+        const uint32_t cand = prefix | (1u << b);
+        const uint32_t c = (uint32_t)__popcll(__ballot(key >= cand));
+        prefix = c >= j ? cand : prefix;
     }
     return prefix;
 }
 
 // grid = (slices, rows).
-template <bool VEC>
+template <bool VEC, int KH>
 __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scratch sc, uint32_t slice_len)
 {
     extern __shared__ uint32_t s_dyn[]; // [slice_len] token counts when the row has penalties
@@ -248,55 +386,89 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
     const mako_sampling_params P = d.params[row];
     const RowClass cls = classify(P);
-
     // Greedy rows ignore the penalties (src/gen/sampler.cpp:77-78).
-    const uint32_t hl = (d.hist_tokens && cls != kGreedy) ? d.hist_len[row] : 0u;
+    const uint32_t hl = (d.hist_tokens && cls != kGreedy) ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
     const bool pen = hl > 0 && !penalties_neutral(P);
-    if (pen)
-        build_counts(d, row, hl, lo, hi, slice_len, s_dyn);
-
+    if (tid == 0) {
+        sm.argidx = kNone;
+        sm.emit_n = 0;
+        sm.emit_flags = 0;
+    }
     float wv[16];
-    load_slice<VEC>(d, row, lo, hi, P, pen, s_dyn, wv);
+    Extras<KH> ex;
+    load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv, ex);
 
-    // first maximum of the thread's logits; its index order is increasing in j
+    // maximum of the thread's logits (NaNs ignored), then of the wave, then of the slice
     float best = -INFINITY;
-    uint32_t bidx = kNone;
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j)
-        if (wv[j] > best) {
-            best = wv[j];
-            bidx = elem_index<VEC>(lo, tid, j);
-        }
+        best = fmaxf(best, wv[j]);
+#pragma unroll
+    for (int k = 0; k < KH; ++k)
+        best = fmaxf(best, ex.v[k]);
     const uint32_t bkey = order_key(best);
-    const unsigned long long top = block_max_u64(((unsigned long long)bkey << 32) | (unsigned long long)(kNone - bidx), sm.bs);
+    const bool emits = cls == kTopK || cls == kNucleus;
+    const uint32_t wmax = __ockl_wfred_max_u32(bkey);
+    uint32_t wkth = 0;
+    if (emits) {
+        // Every logit that can be among the row's K largest is among this slice's K largest.  Each wave
+        // takes the ceil(K/16)-th largest of its per-thread maxima; at least K logits of the slice are >= the
+        // smallest of those 16 values, which becomes the emission threshold.
+        const uint32_t K = cls == kTopK ? P.top_k : kTopKFast;
+        wkth = wave_kth_largest(bkey, (K + kWaves - 1) / kWaves);
+    }
+    if (lane_id() == 0) {
+        sm.wave_max[wave_id()] = wmax;
+        sm.wave_kth[wave_id()] = wkth;
+    }
+    __syncthreads();
+    uint32_t mkey = 0, tau_key = 0xffffffffu;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        mkey = max(mkey, sm.wave_max[w]);
+        tau_key = min(tau_key, sm.wave_kth[w]);
+    }
+    // first index holding the maximum
+    if (bkey == mkey) {
+        const float M = order_unkey(mkey);
+        uint32_t first = kNone;
+#pragma unroll
+        for (int j = 15; j >= 0; --j)
+            if (wv[j] == M)
+                first = elem_index<VEC>(lo, tid, (uint32_t)j);
+#pragma unroll
+        for (int k = 0; k < KH; ++k)
+            if (ex.v[k] == M)
+                first = min(first, ex.i[k]);
+        if (first != kNone)
+            atomicMin(&sm.argidx, first);
+    }
 
     SliceStat st;
-    st.wmax = order_unkey((uint32_t)(top >> 32));
-    st.argidx = kNone - (uint32_t)top;
+    st.wmax = order_unkey(mkey);
     st.flags = 0;
     st.n_emit = 0;
     st.tau_key = 0;
     st.pad[0] = st.pad[1] = st.pad[2] = 0;
-    if (slice == 0 && tid == 0 && wv[0] != wv[0]) // only thread 0 publishes the record
-        st.flags |= kFlagFirstNan;
+    // element 0 of the row is NaN (it may have moved to an extra): only its holder raises the flag
+    bool first_nan = slice == 0 && tid == 0 && wv[0] != wv[0] && !(pen && KH > 0 && s_dyn[0]);
+#pragma unroll
+    for (int k = 0; k < KH; ++k)
+        first_nan = first_nan || (ex.i[k] == 0 && ex.v[k] != ex.v[k]);
+    if (first_nan)
+        atomicOr(&sm.emit_flags, kFlagFirstNan);
 
-    if (cls == kTopK || cls == kNucleus) {
-        // Every logit that can be among the row's K largest is among this slice's K largest, and those are
-        // all >= the K-th largest per-thread maximum.
-        const uint32_t K = cls == kTopK ? P.top_k : kTopKFast;
-        uint32_t tau_key = select_kth_key(bkey, K, sm);
+    if (emits) {
         if (tau_key <= kKeyNegInf) {
             tau_key = kKeyNegInf;
             st.flags |= kFlagComplete;
         }
-        const float tau = order_unkey(tau_key);
-        if (tid == 0)
-            sm.emit_n = 0;
-        __syncthreads();
+        // w >= tau and w > -inf in one compare: -inf itself is below the most negative finite float
+        const float tau = fmaxf(order_unkey(tau_key), -3.402823466e38f);
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j) {
             const float w = wv[j];
-            if (w >= tau && w > -INFINITY) {
+            if (w >= tau) {
                 const uint32_t pos = atomicAdd(&sm.emit_n, 1u);
                 if (pos < kCap) {
                     sm.cw[pos] = w;
@@ -304,7 +476,18 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
                 }
             }
         }
-        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < KH; ++k)
+            if (ex.v[k] >= tau) {
+                const uint32_t pos = atomicAdd(&sm.emit_n, 1u);
+                if (pos < kCap) {
+                    sm.cw[pos] = ex.v[k];
+                    sm.ci[pos] = ex.i[k];
+                }
+            }
+    }
+    __syncthreads();
+    if (emits) {
         const uint32_t n = sm.emit_n;
         if (n > kCap)
             st.flags |= kFlagOverflow;
@@ -316,8 +499,11 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
             sc.cand_i[base + tid] = sm.ci[tid];
         }
     }
-    if (tid == 0)
+    if (tid == 0) {
+        st.argidx = sm.argidx;
+        st.flags |= sm.emit_flags;
         sc.stats[(size_t)row * kMaxSlices + slice] = st;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -789,19 +975,18 @@ __device__ void bitonic_sort_desc(unsigned long long* a, uint32_t n)
 
 // Exact fp64 sum of q over one slice, and the number of candidates in it (q > 0 and q >= min_p).
 // The summation order is fixed: each thread adds its logits in index order, then lanes, then waves.
-template <bool VEC>
+template <bool VEC, int KH>
 __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slice,
                               uint32_t slice_len, const mako_sampling_params& P, float m, const FinishLds& L)
 {
     FinishShared& sm = *L.sm;
     const uint32_t lo = slice * slice_len;
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
-    const uint32_t hl = d.hist_tokens ? d.hist_len[row] : 0u;
+    const uint32_t hl = d.hist_tokens ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
     const bool pen = hl > 0 && !penalties_neutral(P);
-    if (pen)
-        build_counts(d, row, hl, lo, hi, slice_len, L.cnt);
     float wv[16];
-    load_slice<VEC>(d, row, lo, hi, P, pen, L.cnt, wv);
+    Extras<KH> ex;
+    load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, ex);
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
     double sum = 0;
@@ -809,6 +994,14 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j) {
         const float q = weight_of(wv[j], m, inv_t, sm.tab);
+        if (q >= floor_q && q > 0.0f) {
+            sum += (double)q;
+            ++n;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < KH; ++k) {
+        const float q = weight_of(ex.v[k], m, inv_t, sm.tab);
         if (q >= floor_q && q > 0.0f) {
             sum += (double)q;
             ++n;
@@ -823,7 +1016,7 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
 }
 
 // grid = (slices, rows).  Only top_k == 0 rows use more than their first workgroup.
-template <bool VEC>
+template <bool VEC, int KH>
 __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Scratch sc, uint32_t slices, uint32_t slice_len)
 {
     extern __shared__ unsigned long long s_dyn64[];
@@ -878,7 +1071,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Sc
 
     if (cls == kNucleus) {
         // second pass: all slices of the row in parallel; the last one to arrive finishes the row
-        slice_partial<VEC>(d, sc, row, slice, slice_len, P, m, L);
+        slice_partial<VEC, KH>(d, sc, row, slice, slice_len, P, m, L);
         if (tid == 0) {
             __threadfence();
             sm.ticket = atomicAdd(&sc.tickets[row], 1u);

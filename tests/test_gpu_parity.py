@@ -155,6 +155,18 @@ def test_special_values(gpu_ctx):
     assert_parity(gpu_ctx, w)
 
 
+@pytest.mark.parametrize("hist_len", [1500, 3000, 9000])
+def test_history_lengths(gpu_ctx, hist_len):
+    """Histories of up to 2 and up to 8 entries per thread stay in registers, longer ones take the generic route:
+    all three against the oracle, with heavy repetition (Zipf) and tokens that hit the row maximum."""
+    w = workloads.config3(rows=12, vocab=50000, hist_len=hist_len, seed=600 + hist_len)
+    top = w["logits"].argmax(axis=1)
+    w["hist"][:, 0] = top          # the most likely token is penalised
+    w["hist"][:6, 1] = 0           # and token 0
+    w["logits"][3, 0] = np.nan     # NaN at index 0 of a penalised token
+    assert_parity(gpu_ctx, w, cap=512)
+
+
 def test_history_forms_agree(gpu_ctx):
     """Raw accept() token lists and pre-aggregated (id, count) pairs give identical results."""
     w = workloads.config3(rows=8, vocab=30000, hist_len=300)
