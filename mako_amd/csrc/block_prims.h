@@ -22,6 +22,13 @@ __device__ __forceinline__ int wave_id()
     return threadIdx.x >> 6;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global load, which would serialise LDS set-up work behind the logits stream it is meant to overlap.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // Scratch shared by the primitives; one instance per kernel.
 struct BlockScratch {
     unsigned long long u64[kWaves];

@@ -96,8 +96,12 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap));
     MAKO_HIP(ctx, dev_alloc(&sc.part_sum, (size_t)max_rows * mako::kMaxSlices));
     MAKO_HIP(ctx, dev_alloc(&sc.part_n, (size_t)max_rows * mako::kMaxSlices));
-    MAKO_HIP(ctx, dev_alloc(&sc.tickets, (size_t)max_rows));
-    MAKO_HIP(ctx, hipMemset(sc.tickets, 0, (size_t)max_rows * sizeof(uint32_t)));
+    MAKO_HIP(ctx, dev_alloc(&sc.tickets, (size_t)max_rows * 32));
+    MAKO_HIP(ctx, hipMemset(sc.tickets, 0, (size_t)max_rows * 32 * sizeof(uint32_t)));
+    MAKO_HIP(ctx, dev_alloc(&sc.binc, (size_t)max_rows * mako::kBins));
+    MAKO_HIP(ctx, hipMemset(sc.binc, 0, (size_t)max_rows * mako::kBins * sizeof(uint32_t)));
+    MAKO_HIP(ctx, dev_alloc(&sc.bins, (size_t)max_rows * mako::kBins));
+    MAKO_HIP(ctx, hipMemset(sc.bins, 0, (size_t)max_rows * mako::kBins * sizeof(unsigned long long)));
     MAKO_HIP(ctx, dev_alloc(&sc.wbuf, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.cnt, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.key[0], rv));
@@ -124,7 +128,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.tickets,
+    void* ptrs[] = {sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.tickets, sc.binc, sc.bins,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
                     ctx->st_hist,  ctx->st_hcnt, ctx->st_hlen,  ctx->st_draft, ctx->st_tokens, ctx->st_acc};

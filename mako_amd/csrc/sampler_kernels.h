@@ -31,6 +31,7 @@ constexpr uint32_t kCap = 512;       // candidates kept per slice
 constexpr uint32_t kTopKFast = 128;  // largest top_k resolved from the per-slice candidates
 constexpr uint32_t kSortMax = 4096;  // candidates the finisher sorts in LDS
 constexpr uint32_t kDynLds = 65536;  // dynamic LDS of both kernels
+constexpr uint32_t kBins = 2048;     // weight histogram of top_k == 0 rows: bin = bits(q) >> 19 (16 bins per binade)
 
 constexpr uint32_t kFlagFirstNan = 1u; // element 0 of the row is NaN (slice 0 only)
 constexpr uint32_t kFlagOverflow = 2u; // more than kCap logits reached the slice's threshold
@@ -51,8 +52,12 @@ struct Scratch {
     uint32_t* cand_i;  // [max_rows][slices_cap][kCap] their token ids
     double* part_sum;  // [max_rows][kMaxSlices] exact fp64 sum of q over the slice (top_k == 0 rows)
     uint32_t* part_n;  // [max_rows][kMaxSlices] candidates (q > 0, q >= min_p) in the slice
-    uint32_t* tickets; // [max_rows] arrival counter of the row's slices; all zero between calls
-    float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path
+    uint32_t* tickets; // [max_rows][32] arrival counter of the row's slices (one per 128-byte line); zero between calls
+    uint32_t* binc;    // [max_rows][kBins] candidates per weight bin (top_k == 0 rows); all zero between calls
+    unsigned long long* bins; // [max_rows][kBins] sum of their 24-bit significands: the bin's exact mass is
+                              // bins * 2^(e - 150), e being the bin's exponent; all zero between calls
+    float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path; top_k == 0 rows keep
+                       // bits(q) of every logit here instead (0 where q is not a candidate)
     uint32_t* cnt;     // [max_rows][vpad] token counts; all zero between calls
     uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong
     uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, ping-pong
@@ -540,68 +545,83 @@ __device__ __forceinline__ unsigned long long match_digit(uint32_t digit, bool v
     return m;
 }
 
-// One stable counting-sort pass on bits [shift, shift + 8) of the keys, ascending.
+// One stable counting-sort pass on bits [shift, shift + 8) of the keys, ascending, by one workgroup.
+// Wave w owns the contiguous chunk [w * C, (w + 1) * C) of the input and walks it 64 pairs at a time: lanes
+// with equal digits find each other with ballots (match_digit), so ranks inside a group need no atomics, and
+// the wave's running output offsets per digit live in its private row of LDS.  Three barriers per pass.
 // Returns false (and moves nothing) when every key has the same digit.
 __device__ bool radix_pass(const uint32_t* ksrc, const uint32_t* isrc, uint32_t* kdst, uint32_t* idst, uint32_t n,
                            uint32_t shift, const FinishLds& L)
 {
     FinishShared& sm = *L.sm;
-    const uint32_t tid = threadIdx.x;
-    if (tid < 256)
-        sm.hist[tid] = 0;
+    const uint32_t tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+    const uint32_t chunk = ((n + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
+    const uint32_t beg = min(n, wave * chunk), end = min(n, beg + chunk);
+    uint32_t* woff = L.wcount + wave * 256u;
+    for (uint32_t j = lane; j < 256u; j += kWave)
+        woff[j] = 0;
     if (tid == 0)
         sm.flag = 0;
-    __syncthreads();
-    for (uint32_t base = 0; base < n; base += kThreads) {
-        const uint32_t i = base + tid;
-        const bool valid = i < n;
-        const uint32_t dg = valid ? ((ksrc[i] >> shift) & 255u) : 0u;
-        const unsigned long long mm = match_digit(dg, valid);
-        const unsigned long long below = mm & ((1ull << lane_id()) - 1ull);
-        if (valid && below == 0)
-            atomicAdd(&sm.hist[dg], (uint32_t)__popcll(mm));
+    const unsigned long long lower = (1ull << lane) - 1ull;
+    // per-wave digit counts (the row is private to the wave: in-order LDS, no barrier needed).  Four groups
+    // are fetched per trip, from clamped positions, so that their latencies overlap.
+    for (uint32_t base = beg; base < end; base += 4u * kWave) {
+        uint32_t key[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+            key[u] = ksrc[min(base + u * kWave + lane, end - 1u)];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const bool valid = base + u * kWave + lane < end;
+            const uint32_t dg = valid ? ((key[u] >> shift) & 255u) : 0u;
+            const unsigned long long mm = match_digit(dg, valid);
+            if (valid && (mm & lower) == 0)
+                woff[dg] += (uint32_t)__popcll(mm);
+        }
     }
     __syncthreads();
-    const uint32_t mine = tid < 256 ? sm.hist[tid] : 0u;
-    if (mine == n)
+    // digit totals -> global offsets; wave rows become each wave's first output position per digit
+    uint32_t mine = 0;
+    if (tid < 256)
+        for (int w = 0; w < kWaves; ++w)
+            mine += L.wcount[w * 256 + tid];
+    if (tid < 256 && mine == n)
         sm.flag = 1;
     uint32_t tot;
-    const uint32_t excl = block_excl_scan_u32(mine, tot, sm.bs); // its barriers publish sm.flag
+    uint32_t acc = block_excl_scan_u32(mine, tot, sm.bs); // its barriers publish sm.flag
     if (sm.flag)
         return false;
     if (tid < 256)
-        sm.run[tid] = excl;
+        for (int w = 0; w < kWaves; ++w) {
+            const uint32_t t = L.wcount[w * 256 + tid];
+            L.wcount[w * 256 + tid] = acc;
+            acc += t;
+        }
     __syncthreads();
-    for (uint32_t base = 0; base < n; base += kThreads) {
-        for (uint32_t j = tid; j < kWaves * 256; j += kThreads)
-            L.wcount[j] = 0;
-        __syncthreads();
-        const uint32_t i = base + tid;
-        const bool valid = i < n;
-        const uint32_t key = valid ? ksrc[i] : 0u;
-        const uint32_t dg = (key >> shift) & 255u;
-        const unsigned long long mm = match_digit(dg, valid);
-        const uint32_t rank = (uint32_t)__popcll(mm & ((1ull << lane_id()) - 1ull));
-        if (valid && rank == 0)
-            L.wcount[wave_id() * 256 + dg] = (uint32_t)__popcll(mm);
-        __syncthreads();
-        if (tid < 256) {
-            uint32_t acc = sm.run[tid];
-            for (int w = 0; w < kWaves; ++w) {
-                const uint32_t t = L.wcount[w * 256 + tid];
-                L.wcount[w * 256 + tid] = acc;
-                acc += t;
+    for (uint32_t base = beg; base < end; base += 4u * kWave) {
+        uint32_t key[4], id[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t i = min(base + u * kWave + lane, end - 1u);
+            key[u] = ksrc[i];
+            id[u] = isrc[i];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const bool valid = base + u * kWave + lane < end;
+            const uint32_t dg = valid ? ((key[u] >> shift) & 255u) : 0u;
+            const unsigned long long mm = match_digit(dg, valid);
+            const uint32_t off = woff[dg];
+            if (valid) {
+                const uint32_t pos = off + (uint32_t)__popcll(mm & lower);
+                kdst[pos] = key[u];
+                idst[pos] = id[u];
+                if ((mm & lower) == 0)
+                    woff[dg] = off + (uint32_t)__popcll(mm);
             }
-            sm.run[tid] = acc;
         }
-        __syncthreads();
-        if (valid) {
-            const uint32_t pos = L.wcount[wave_id() * 256 + dg] + rank;
-            kdst[pos] = key;
-            idst[pos] = isrc[i];
-        }
-        __syncthreads();
     }
+    __syncthreads();
     return true;
 }
 
@@ -818,6 +838,555 @@ __device__ void draw_from_list(const mako_sample_desc& d, uint32_t row, QAt qat,
         write_row(d, row, o);
 }
 
+// ---------------------------------------------------------------------------------------------
+// sorted lists: top-p cut, exact fp32 total and walk, in groups of 256 (see seqfp.h, "groups")
+// ---------------------------------------------------------------------------------------------
+
+constexpr uint32_t kGroup = 256;      // one wave, four consecutive entries per lane
+constexpr uint32_t kMaxGroups = 1024; // lists of up to 262144 entries
+
+struct GroupLds { // carved from the dynamic LDS block once sorting is over
+    double* pg;     // [kMaxGroups + 1] fp64 sum of the entries before each group
+    uint32_t* d0;   // [kMaxGroups] the group's map for the guessed epoch
+    uint32_t* d1;
+    uint32_t* cmax;
+    uint32_t* misc; // [4]
+};
+
+__device__ __forceinline__ int exponent_of(float x)
+{
+    uint32_t M;
+    int e;
+    seqfp::split(x, M, e);
+    return e;
+}
+
+// The four weights a lane owns in group g of a list of `len` entries (0 past the end).
+__device__ __forceinline__ void load_group(const uint32_t* kf, uint32_t g, uint32_t len, float (&q)[4])
+{
+    const uint32_t i = g * kGroup + lane_id() * 4u;
+    uint32_t k[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu}; // ~bits(0.0f)
+    if (i + 3 < len) {
+        const uint4 x = *reinterpret_cast<const uint4*>(kf + i);
+        k[0] = x.x;
+        k[1] = x.y;
+        k[2] = x.z;
+        k[3] = x.w;
+    } else {
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (i + j < len)
+                k[j] = kf[i + j];
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j)
+        q[j] = __uint_as_float(~k[j]);
+}
+
+__device__ __forceinline__ seqfp::Step32 wave_incl_scan_step32(seqfp::Step32 v)
+{
+    for (int o = 1; o < kWave; o <<= 1) {
+        seqfp::Step32 t;
+        t.d0 = __shfl_up(v.d0, o);
+        t.d1 = __shfl_up(v.d1, o);
+        t.cmax = __shfl_up(v.cmax, o);
+        if (lane_id() >= o)
+            v = seqfp::compose32(t, v);
+    }
+    return v;
+}
+
+// Group maps of entries [0, n) for epochs guessed from pg: sum (walk == false) or walk from r0.
+__device__ void build_group_maps(const uint32_t* kf, uint32_t n, bool walk, double r0, const GroupLds& G)
+{
+    using namespace seqfp;
+    const uint32_t groups = (n + kGroup - 1) / kGroup;
+    for (uint32_t g = wave_id(); g < groups; g += kWaves) {
+        const double guess = walk ? r0 - G.pg[g] : G.pg[g];
+        const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+        Step32 st = Step32{kSat, kSat, kSat};
+        if (eg > 0) { // uniform per wave
+            float q[4];
+            load_group(kf, g, n, q);
+            st = identity32();
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (g * kGroup + lane_id() * 4u + j < n)
+                    st = compose32(st, step32(q[j], eg));
+            st = wave_incl_scan_step32(st);
+        }
+        if (lane_id() == kWave - 1) {
+            G.d0[g] = st.d0;
+            G.d1[g] = st.d1;
+            G.cmax[g] = st.cmax;
+        }
+    }
+}
+
+// Entries [beg, end) of one group added to S one by one (exactly), by one wave.
+__device__ float exact_group_sum(const uint32_t* kf, uint32_t g, uint32_t n, float S)
+{
+    using namespace seqfp;
+    const uint32_t beg = g * kGroup, end = min(n, beg + kGroup), lane = lane_id();
+    float q[4];
+    load_group(kf, g, n, q);
+    uint32_t start = beg;
+    for (;;) {
+        uint32_t M;
+        int e;
+        split(S, M, e);
+        Step32 st = identity32();
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t i = beg + lane * 4u + j;
+            if (i >= start && i < end)
+                st = compose32(st, step32(q[j], e));
+        }
+        const Step32 incl = wave_incl_scan_step32(st);
+        Step32 excl;
+        excl.d0 = __shfl_up(incl.d0, 1);
+        excl.d1 = __shfl_up(incl.d1, 1);
+        if (lane == 0)
+            excl.d0 = excl.d1 = 0;
+        long long mm = (long long)M + (long long)((M & 1u) ? excl.d1 : excl.d0);
+        uint32_t hit = kNone;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t i = beg + lane * 4u + j;
+            if (hit == kNone && i >= start && i < end) {
+                if (add_event(mm, q[j], e))
+                    hit = i;
+                else
+                    mm = add_apply(mm, q[j], e);
+            }
+        }
+        const unsigned long long bal = __ballot(hit != kNone);
+        if (bal == 0) {
+            const uint32_t dt = (M & 1u) ? __shfl(incl.d1, kWave - 1) : __shfl(incl.d0, kWave - 1);
+            return join(M + dt, e);
+        }
+        const int first = __ffsll((long long)bal) - 1;
+        const uint32_t iev = __shfl(hit, first);
+        const uint32_t mev = (uint32_t)__shfl((int)(uint32_t)mm, first);
+        const float qev = __uint_as_float(~kf[iev]);
+        S = join(mev, e) + qev;
+        start = iev + 1;
+        if (start >= end)
+            return S;
+    }
+}
+
+// Entries of one group subtracted from r one by one (exactly), by one wave.  Returns true and the
+// entry's position when the walk stops inside the group, else false and the new r.
+__device__ bool exact_group_walk(const uint32_t* kf, uint32_t g, uint32_t n, float& r, uint32_t& pos)
+{
+    using namespace seqfp;
+    const uint32_t beg = g * kGroup, end = min(n, beg + kGroup), lane = lane_id();
+    float q[4];
+    load_group(kf, g, n, q);
+    uint32_t start = beg;
+    for (;;) {
+        uint32_t M;
+        int e;
+        split(r, M, e);
+        Step32 st = identity32();
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t i = beg + lane * 4u + j;
+            if (i >= start && i < end)
+                st = compose32(st, step32(q[j], e));
+        }
+        const Step32 incl = wave_incl_scan_step32(st);
+        Step32 excl;
+        excl.d0 = __shfl_up(incl.d0, 1);
+        excl.d1 = __shfl_up(incl.d1, 1);
+        if (lane == 0)
+            excl.d0 = excl.d1 = 0;
+        long long mm = (long long)M - (long long)((M & 1u) ? excl.d1 : excl.d0);
+        uint32_t hit = kNone;
+        bool stop = false;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t i = beg + lane * 4u + j;
+            if (hit == kNone && i >= start && i < end) {
+                if (walk_stop(mm, q[j], e)) {
+                    hit = i;
+                    stop = true;
+                } else if (sub_event(mm, q[j], e)) {
+                    hit = i;
+                } else {
+                    mm = sub_apply(mm, q[j], e);
+                }
+            }
+        }
+        const unsigned long long bal = __ballot(hit != kNone);
+        if (bal == 0) {
+            const uint32_t dt = (M & 1u) ? __shfl(incl.d1, kWave - 1) : __shfl(incl.d0, kWave - 1);
+            r = join(M - dt, e);
+            return false;
+        }
+        const int first = __ffsll((long long)bal) - 1;
+        const uint32_t iev = __shfl(hit, first);
+        if (__shfl((int)stop, first)) {
+            pos = iev;
+            return true;
+        }
+        const uint32_t mev = (uint32_t)__shfl((int)(uint32_t)mm, first);
+        r = join(mev, e) - __uint_as_float(~kf[iev]);
+        start = iev + 1;
+        if (start >= end)
+            return false;
+    }
+}
+
+// Tail of every path that ends with a list sorted by (q desc, idx asc) in global memory: kf[i] = ~bits(q_i),
+// jf[i] = token id, n1 entries (already cut to top_k).  Applies top-p (src/gen/sampler.cpp:44-61) against
+// total64 (the fp64 sum over the row's candidates; summed from the list when !have_total), then the exact
+// fp32 total (:80-82) and walk (:64-73).  All 1024 threads must call it.
+__device__ void sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf,
+                            const uint32_t* jf, uint32_t n1, bool have_total, double total64, uint32_t path,
+                            const FinishLds& L)
+{
+    using namespace seqfp;
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    auto qat = [=](uint32_t i) { return __uint_as_float(~kf[i]); };
+    auto idat = [=](uint32_t i) { return jf[i]; };
+    GroupLds G;
+    G.pg = reinterpret_cast<double*>(L.sortk);
+    G.d0 = reinterpret_cast<uint32_t*>(G.pg + kMaxGroups + 2);
+    G.d1 = G.d0 + kMaxGroups;
+    G.cmax = G.d1 + kMaxGroups;
+    G.misc = G.cmax + kMaxGroups;
+    const bool topp_active = P.top_p < 1.0f;
+    if (d.draft || n1 > kGroup * kMaxGroups) {
+        // verification and oversized lists take the generic windowed replay
+        uint32_t n = n1;
+        if (topp_active) {
+            if (!have_total) {
+                double part = 0;
+                for (uint32_t i = tid; i < n; i += kThreads)
+                    part += (double)qat(i);
+                total64 = block_sum_f64(part, sm.bs);
+            }
+            const double want = (double)P.top_p * total64;
+            double carry = 0;
+            uint32_t keep = n;
+            for (uint32_t base = 0; base < n; base += kThreads) {
+                const uint32_t i = base + tid;
+                const double q = i < n ? (double)qat(i) : 0.0;
+                double tile;
+                const double incl = carry + block_incl_scan_f64(q, tile, sm.bs);
+                const uint32_t hit = (i < n && incl >= want) ? i : kNone;
+                const uint32_t first = block_min_u32(hit, sm.bs);
+                if (first != kNone) {
+                    keep = first + 1;
+                    break;
+                }
+                carry += tile;
+            }
+            n = keep;
+        }
+        draw_from_list(d, row, qat, idat, n, path, sm);
+        return;
+    }
+
+    // fp64 group sums and their prefix
+    const uint32_t groups1 = (n1 + kGroup - 1) / kGroup;
+    __syncthreads();
+    for (uint32_t g = wave_id(); g < groups1; g += kWaves) {
+        float q[4];
+        load_group(kf, g, n1, q);
+        double s = (((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3];
+        for (int o = 32; o > 0; o >>= 1)
+            s += __shfl_xor(s, o);
+        if (lane_id() == 0)
+            G.pg[g + 1] = s;
+    }
+    __syncthreads();
+    {
+        const double v = tid < groups1 ? G.pg[tid + 1] : 0.0;
+        double all;
+        const double incl = block_incl_scan_f64(v, all, sm.bs);
+        if (tid < groups1)
+            G.pg[tid + 1] = incl;
+        if (tid == 0)
+            G.pg[0] = 0.0;
+        if (!have_total)
+            total64 = all;
+    }
+    __syncthreads();
+
+    // top-p: first entry at which the running fp64 sum reaches top_p * total
+    uint32_t n = n1;
+    if (topp_active) {
+        const double want = (double)P.top_p * total64;
+        const uint32_t hitg = (tid < groups1 && G.pg[tid + 1] >= want) ? tid : kNone;
+        const uint32_t gs = block_min_u32(hitg, sm.bs);
+        if (gs != kNone) {
+            if (wave_id() == 0) {
+                float q[4];
+                load_group(kf, gs, n1, q);
+                double p[4];
+                p[0] = (double)q[0];
+                p[1] = p[0] + (double)q[1];
+                p[2] = p[1] + (double)q[2];
+                p[3] = p[2] + (double)q[3];
+                double incl = p[3];
+                for (int o = 1; o < kWave; o <<= 1) {
+                    const double t = __shfl_up(incl, o);
+                    if (lane_id() >= o)
+                        incl += t;
+                }
+                const double base = G.pg[gs] + (incl - p[3]);
+                uint32_t hit = kNone;
+#pragma unroll
+                for (int j = 3; j >= 0; --j)
+                    if (base + p[j] >= want)
+                        hit = gs * kGroup + lane_id() * 4u + (uint32_t)j;
+                const unsigned long long bal = __ballot(hit != kNone && hit < n1);
+                uint32_t keep = min(n1, (gs + 1u) * kGroup);
+                if (bal)
+                    keep = (uint32_t)__shfl((int)hit, __ffsll((long long)bal) - 1) + 1u;
+                if (lane_id() == 0)
+                    G.misc[0] = keep;
+            }
+            __syncthreads();
+            n = G.misc[0];
+        }
+    }
+    if (n < 1)
+        n = 1;
+    __syncthreads();
+
+    // exact fp32 total: group maps in parallel, then one wave chains them
+    build_group_maps(kf, n, false, 0.0, G);
+    __syncthreads();
+    const uint32_t groups = (n + kGroup - 1) / kGroup;
+    if (wave_id() == 0) {
+        float S = 0.0f;
+        for (uint32_t g = 0; g < groups; ++g) {
+            uint32_t M;
+            int e;
+            split(S, M, e);
+            const int eg = G.pg[g] > 0 ? exponent_of((float)G.pg[g]) : 0;
+            const Step32 st = Step32{G.d0[g], G.d1[g], G.cmax[g]};
+            if (e == eg && group_add_ok((long long)M, st))
+                S = join(M + ((M & 1u) ? st.d1 : st.d0), e);
+            else
+                S = exact_group_sum(kf, g, n, S);
+        }
+        if (lane_id() == 0)
+            G.misc[1] = __float_as_uint(S);
+    }
+    __syncthreads();
+    const float total = __uint_as_float(G.misc[1]);
+    const float span = total - 0.0f;
+    const float prod = d.u[row] * span;
+    const float r0 = prod + 0.0f;
+    __syncthreads();
+
+    // exact walk
+    uint32_t pos = n - 1;
+    if (r0 < 0.0f) {
+        pos = 0;
+    } else if (r0 == r0 && r0 != INFINITY) {
+        build_group_maps(kf, n, true, (double)r0, G);
+        __syncthreads();
+        if (wave_id() == 0) {
+            float r = r0;
+            uint32_t at = n - 1;
+            for (uint32_t g = 0; g < groups; ++g) {
+                uint32_t M;
+                int e;
+                split(r, M, e);
+                const double guess = (double)r0 - G.pg[g];
+                const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+                const Step32 st = Step32{G.d0[g], G.d1[g], G.cmax[g]};
+                if (e == eg && group_sub_ok((long long)M, e, st, qat(g * kGroup))) {
+                    r = join(M - ((M & 1u) ? st.d1 : st.d0), e);
+                } else if (exact_group_walk(kf, g, n, r, at)) {
+                    break;
+                }
+            }
+            if (lane_id() == 0)
+                G.misc[2] = at;
+        }
+        __syncthreads();
+        pos = G.misc[2];
+    }
+
+    if (d.out_cand_idx && d.out_cand_q)
+        for (uint32_t j = tid; j < n && j < d.cand_cap; j += kThreads) {
+            d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
+            d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
+        }
+    if (tid == 0) {
+        RowOut o;
+        o.token = (int32_t)idat(pos);
+        o.n_cand = n;
+        o.total = total;
+        o.q = qat(pos);
+        o.path = path;
+        o.accepted = 0;
+        write_row(d, row, o);
+    }
+}
+
+// Common tail of the whole-row paths.  key[0]/idx[0] of the row hold n0 candidates (~bits(q), token id) in index
+// order.  Sorts them by (q desc, idx asc) when top-k or top-p is active, truncates (src/gen/sampler.cpp:39-61)
+// and draws.  `total64` (when have_total) is the fp64 sum of q over all candidates of the row, of which the list
+// may be only the heaviest part; otherwise it is summed from the list.
+__device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
+                                   uint32_t n0, bool have_total, double total64, uint32_t path, const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
+    uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
+    uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
+    uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
+
+    // order by (q desc, idx asc): stable LSD radix sort of ~bits(q), ascending
+    const bool topk_active = P.top_k > 0 && P.top_k < n0;
+    const bool topp_active = P.top_p < 1.0f;
+    uint32_t *ks = key0, *is = idx0, *kd = key1, *id = idx1;
+    if (topk_active || topp_active) {
+        for (uint32_t shift = 0; shift < 32; shift += 8) {
+            if (radix_pass(ks, is, kd, id, n0, shift, L)) {
+                uint32_t* t = ks;
+                ks = kd;
+                kd = t;
+                t = is;
+                is = id;
+                id = t;
+            }
+            __syncthreads();
+        }
+    }
+    const uint32_t n1 = topk_active ? P.top_k : n0; // sampler.cpp:40-43
+    if (topk_active || topp_active) {
+        sorted_tail(d, row, P, ks, is, n1, have_total, total64, path, L);
+        return;
+    }
+    // neither top-k nor top-p: the candidates stay in index order
+    const uint32_t* kf = ks;
+    const uint32_t* jf = is;
+    draw_from_list(
+        d, row, [=](uint32_t i) { return __uint_as_float(~kf[i]); }, [=](uint32_t i) { return jf[i]; }, n1, path, sm);
+}
+
+// A top_k == 0 row whose nucleus is wider than the per-slice candidate lists.  The second pass left bits(q) of
+// every logit in scratch and a histogram of them (16 bins per binade).  Walking the bins from the heaviest down
+// with each bin priced at its LOWEST weight finds a bin by which the nucleus must have ended; only the logits of
+// the bins above are gathered (in index order), sorted and drawn from.  `total64` is the row's exact fp64 total.
+__device__ void nucleus_big_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
+                                double total64, uint32_t c0, uint32_t c1, unsigned long long s0, unsigned long long s1,
+                                const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t V = d.n_vocab;
+    const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
+    uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
+    uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
+
+    // bins from the top: thread t prices bins kBins-1-2t and kBins-2-2t, whose counts are c0 and c1
+    const uint32_t b0 = kBins - 1u - 2u * tid, b1 = b0 - 1u;
+    // exact mass of a bin: sum of significands times the bin's power of two (bins never straddle a binade)
+    auto scale = [](uint32_t b) {
+        const uint32_t e = max(b >> 4, 1u); // biased exponent of the bin's weights (0 -> subnormal scale)
+        return __longlong_as_double((long long)(1023ull + e - 150ull) << 52);
+    };
+    const double m0 = (double)s0 * scale(b0), m1 = (double)s1 * scale(b1);
+    const double want = (double)P.top_p * total64;
+    double all;
+    const double incl = block_incl_scan_f64(m0 + m1, all, sm.bs);
+    // The nucleus ends in the first bin (from the top) at which the running mass reaches `want`.  These sums
+    // associate differently from the sorted prefix sums that make the final decision, so one more non-empty
+    // bin is taken along: the gather stops at the SECOND bin that satisfies the test.
+    const bool r0 = c0 && incl - m1 >= want, r1 = c1 && incl >= want;
+    uint32_t reached_total;
+    const uint32_t before = block_excl_scan_u32((uint32_t)r0 + (uint32_t)r1, reached_total, sm.bs);
+    uint32_t hit = kNone;
+    if (r0 && before + 1 == 2)
+        hit = b0;
+    else if (r1 && before + (uint32_t)r0 + 1 == 2)
+        hit = b1;
+    const uint32_t rev = block_min_u32(hit == kNone ? kNone : kBins - 1u - hit, sm.bs);
+    const uint32_t b_lo = rev == kNone ? 0u : kBins - 1u - rev; // not reached twice: keep every candidate
+    const uint32_t key_lo = b_lo << 19;
+
+    // gather the logits with bits(q) >= key_lo, in index order.  Wave w owns a contiguous chunk of the row:
+    // a counting sweep, one exchange of the 16 wave totals, then a writing sweep in which ranks come from
+    // ballots.  Lane l holds entries 4l..4l+3 of each 256-entry group.
+    const uint32_t lane = lane_id(), wave = wave_id();
+    const uint32_t chunk = ((V + kThreads * 4u - 1u) / (kThreads * 4u)) * kGroup; // per wave, a multiple of 256
+    const uint32_t beg = min(V, wave * chunk), end = min(V, beg + chunk);
+    auto fetch = [&](uint32_t i, uint32_t (&k)[4]) {
+        if (i + 3 < end) {
+            const uint4 x = *reinterpret_cast<const uint4*>(qk + i);
+            k[0] = x.x;
+            k[1] = x.y;
+            k[2] = x.z;
+            k[3] = x.w;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                k[j] = i + j < end ? qk[i + j] : 0u;
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (k[j] < key_lo)
+                k[j] = 0;
+    };
+    uint32_t mine = 0;
+    for (uint32_t base = beg; base < end; base += 2u * kGroup) {
+        uint32_t ka[4], kb[4];
+        fetch(base + lane * 4u, ka);
+        fetch(base + kGroup + lane * 4u, kb);
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            mine += (ka[j] != 0) + (kb[j] != 0);
+    }
+    for (int o = 32; o > 0; o >>= 1)
+        mine += __shfl_xor(mine, o);
+    if (lane == 0)
+        sm.bs.u64[wave] = mine;
+    __syncthreads();
+    uint32_t out = 0, n0 = 0;
+    for (int w = 0; w < kWaves; ++w) {
+        const uint32_t x = (uint32_t)sm.bs.u64[w];
+        if (w < (int)wave)
+            out += x;
+        n0 += x;
+    }
+    const unsigned long long lower = (1ull << lane) - 1ull;
+    for (uint32_t base = beg; base < end; base += kGroup) {
+        uint32_t k[4];
+        fetch(base + lane * 4u, k);
+        unsigned long long bal[4];
+        uint32_t before = 0, total = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            bal[j] = __ballot(k[j] != 0);
+            before += (uint32_t)__popcll(bal[j] & lower);
+            total += (uint32_t)__popcll(bal[j]);
+        }
+        uint32_t pos = out + before;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (k[j]) {
+                key0[pos] = ~k[j];
+                idx0[pos] = base + lane * 4u + j;
+                ++pos;
+            }
+        out += total;
+    }
+    __syncthreads();
+    sort_truncate_draw(d, sc, row, P, n0, true, total64, MAKO_PATH_GENERAL, L);
+}
+
 // Whole-row path: exact for every parameter combination.  One workgroup rebuilds the penalised
 // row in scratch, keeps the candidates, sorts them by (q desc, idx asc) when top-k or top-p is
 // active, truncates, and draws.  src/gen/sampler.cpp:20-62.
@@ -901,56 +1470,7 @@ __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32
         fallback_row(d, row, argidx);
         return;
     }
-
-    // 3. order by (q desc, idx asc): stable LSD radix sort of ~bits(q), ascending
-    const bool topk_active = P.top_k > 0 && P.top_k < n0;
-    const bool topp_active = P.top_p < 1.0f;
-    uint32_t *ks = key0, *is = idx0, *kd = key1, *id = idx1;
-    if (topk_active || topp_active) {
-        for (uint32_t shift = 0; shift < 32; shift += 8) {
-            if (radix_pass(ks, is, kd, id, n0, shift, L)) {
-                uint32_t* t = ks;
-                ks = kd;
-                kd = t;
-                t = is;
-                is = id;
-                id = t;
-            }
-            __syncthreads();
-        }
-    }
-    uint32_t n = topk_active ? P.top_k : n0; // sampler.cpp:40-43
-
-    // 4. top-p: shortest sorted prefix whose fp64 running sum reaches top_p * total (sampler.cpp:44-61)
-    if (topp_active) {
-        double part = 0;
-        for (uint32_t i = tid; i < n; i += kThreads)
-            part += (double)__uint_as_float(~ks[i]);
-        const double total64 = block_sum_f64(part, sm.bs);
-        const double want = (double)P.top_p * total64;
-        double carry = 0;
-        uint32_t keep = n;
-        for (uint32_t base = 0; base < n; base += kThreads) {
-            const uint32_t i = base + tid;
-            const double q = i < n ? (double)__uint_as_float(~ks[i]) : 0.0;
-            double tile;
-            const double incl = carry + block_incl_scan_f64(q, tile, sm.bs);
-            const uint32_t hit = (i < n && incl >= want) ? i : kNone;
-            const uint32_t first = block_min_u32(hit, sm.bs);
-            if (first != kNone) {
-                keep = first + 1;
-                break;
-            }
-            carry += tile;
-        }
-        n = keep;
-    }
-
-    const uint32_t* kf = ks;
-    const uint32_t* jf = is;
-    draw_from_list(
-        d, row, [=](uint32_t i) { return __uint_as_float(~kf[i]); }, [=](uint32_t i) { return jf[i]; }, n,
-        MAKO_PATH_GENERAL, sm);
+    sort_truncate_draw(d, sc, row, P, n0, false, 0.0, MAKO_PATH_GENERAL, L);
 }
 
 // Bitonic sort of a[0..n), n a power of two, descending.
@@ -991,10 +1511,12 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
     double sum = 0;
     uint32_t n = 0;
+    uint32_t qb[16], qe[KH > 0 ? KH : 1]; // bits(q), 0 where q is not a candidate
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j) {
         const float q = weight_of(wv[j], m, inv_t, sm.tab);
-        if (q >= floor_q && q > 0.0f) {
+        qb[j] = (q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
+        if (qb[j]) {
             sum += (double)q;
             ++n;
         }
@@ -1002,17 +1524,68 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
 #pragma unroll
     for (int k = 0; k < KH; ++k) {
         const float q = weight_of(ex.v[k], m, inv_t, sm.tab);
-        if (q >= floor_q && q > 0.0f) {
+        qe[k] = (q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
+        if (qe[k]) {
             sum += (double)q;
             ++n;
         }
     }
-    const double total = block_sum_f64(sum, sm.bs);
+    const double total = block_sum_f64(sum, sm.bs); // (its barriers also retire every use of L.cnt above)
     const uint32_t count = block_sum_u32(n, sm.bs);
     if (threadIdx.x == 0) {
         sc.part_sum[(size_t)row * kMaxSlices + slice] = total;
         sc.part_n[(size_t)row * kMaxSlices + slice] = count;
     }
+    // bits(q) of every logit of the slice (0 = not a candidate) and their histogram, for nucleus_big_row()
+    uint32_t* qk = reinterpret_cast<uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
+    uint32_t* hist = L.cnt;
+    unsigned long long* hsum = reinterpret_cast<unsigned long long*>(L.cnt + kBins);
+    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads) {
+        hist[b] = 0;
+        hsum[b] = 0;
+    }
+    __syncthreads();
+    // significand of a positive float (subnormals: no hidden bit), as seqfp::split
+    auto signif = [](uint32_t b) { return (unsigned long long)((b & 0x7fffffu) | ((b >> 23) ? 0x800000u : 0u)); };
+#pragma unroll
+    for (uint32_t j = 0; j < 16; ++j)
+        if (qb[j]) {
+            atomicAdd(&hist[qb[j] >> 19], 1u);
+            atomicAdd(&hsum[qb[j] >> 19], signif(qb[j]));
+        }
+    if (VEC) {
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            const uint32_t i = lo + k * 4096u + threadIdx.x * 4u;
+            if (i < hi)
+                *reinterpret_cast<uint4*>(qk + i) = make_uint4(qb[4 * k], qb[4 * k + 1], qb[4 * k + 2], qb[4 * k + 3]);
+        }
+    } else {
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) {
+            const uint32_t i = lo + j * (uint32_t)kThreads + threadIdx.x;
+            if (i < hi)
+                qk[i] = qb[j];
+        }
+    }
+    __syncthreads(); // the owners' stores land before the holders of moved logits overwrite theirs
+#pragma unroll
+    for (int k = 0; k < KH; ++k)
+        if (ex.i[k] != kNone) {
+            qk[ex.i[k]] = qe[k];
+            if (qe[k]) {
+                atomicAdd(&hist[qe[k] >> 19], 1u);
+                atomicAdd(&hsum[qe[k] >> 19], signif(qe[k]));
+            }
+        }
+    __syncthreads();
+    uint32_t* binc = sc.binc + (size_t)row * kBins;
+    unsigned long long* bins = sc.bins + (size_t)row * kBins;
+    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads)
+        if (hist[b]) {
+            atomicAdd(&binc[b], hist[b]);
+            atomicAdd(&bins[b], hsum[b]);
+        }
 }
 
 // grid = (slices, rows).  Only top_k == 0 rows use more than their first workgroup.
@@ -1072,20 +1645,49 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Sc
     if (cls == kNucleus) {
         // second pass: all slices of the row in parallel; the last one to arrive finishes the row
         slice_partial<VEC, KH>(d, sc, row, slice, slice_len, P, m, L);
+        __syncthreads(); // every thread's stores and atomics are acknowledged before the ticket is taken
         if (tid == 0) {
             __threadfence();
-            sm.ticket = atomicAdd(&sc.tickets[row], 1u);
+            sm.ticket = atomicAdd(&sc.tickets[(size_t)row * 32], 1u);
         }
         __syncthreads();
         if (sm.ticket != slices - 1)
             return;
         __threadfence();
         if (tid == 0)
-            sc.tickets[row] = 0;
+            sc.tickets[(size_t)row * 32] = 0;
     }
 
+    // top_k == 0: the row's exact total and candidate count from the second pass, and this thread's two bins of
+    // the weight histogram (read and cleared here so that the histogram is all zero again for the next call)
+    double row_total = 0;
+    uint32_t row_n0 = 0, bin_c0 = 0, bin_c1 = 0;
+    unsigned long long bin_s0 = 0, bin_s1 = 0;
+    if (cls == kNucleus) {
+        for (uint32_t s = 0; s < slices; ++s) {
+            row_total += sc.part_sum[(size_t)row * kMaxSlices + s];
+            row_n0 += sc.part_n[(size_t)row * kMaxSlices + s];
+        }
+        uint32_t* binc = sc.binc + (size_t)row * kBins;
+        bin_c0 = binc[kBins - 1u - 2u * tid];
+        bin_c1 = binc[kBins - 2u - 2u * tid];
+        binc[kBins - 1u - 2u * tid] = 0;
+        binc[kBins - 2u - 2u * tid] = 0;
+        unsigned long long* bins = sc.bins + (size_t)row * kBins;
+        bin_s0 = bins[kBins - 1u - 2u * tid];
+        bin_s1 = bins[kBins - 2u - 2u * tid];
+        bins[kBins - 1u - 2u * tid] = 0;
+        bins[kBins - 2u - 2u * tid] = 0;
+        if (row_n0 == 0) {
+            fallback_row(d, row, argidx);
+            return;
+        }
+    }
     if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
-        general_row(d, sc, row, P, m, argidx, L);
+        if (cls == kNucleus)
+            nucleus_big_row(d, sc, row, P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, L);
+        else
+            general_row(d, sc, row, P, m, argidx, L);
         return;
     }
 
@@ -1150,16 +1752,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Sc
             part += (double)qat(i);
         total64 = block_sum_f64(part, sm.bs);
     } else {
-        uint32_t n0 = 0;
-        total64 = 0;
-        for (uint32_t s = 0; s < slices; ++s) {
-            total64 += sc.part_sum[(size_t)row * kMaxSlices + s];
-            n0 += sc.part_n[(size_t)row * kMaxSlices + s];
-        }
-        if (n0 == 0) {
-            fallback_row(d, row, argidx);
-            return;
-        }
+        total64 = row_total;
         n1 = n_valid;
     }
 
@@ -1186,7 +1779,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Sc
     } else {
         // the nucleus must end inside the candidates, strictly above everything left behind
         if (keep == kNone || !(q_bound < qat(keep - 1))) {
-            general_row(d, sc, row, P, m, argidx, L);
+            nucleus_big_row(d, sc, row, P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, L);
             return;
         }
         n = keep;

@@ -197,4 +197,76 @@ SEQFP_HD long long sub_apply(long long m, float q, int e)
     return m - ((m & 1) ? s.d1 : s.d0);
 }
 
+// ---- groups ----------------------------------------------------------------
+//
+// A long sorted list is cut into groups.  The map of a whole group under a GUESSED epoch (taken from an
+// approximate fp64 prefix sum) can be built by any number of threads in parallel; a serial chain then walks
+// the groups with the exact state and uses a group's map only if the guess was right and nothing inside the
+// group can leave the binade (or, for the walk, stop).  A group that fails the test is replayed element by
+// element.  Results never depend on the guess, only the speed does.
+
+constexpr uint32_t kSat = 1u << 28; // "left the binade": larger than any state, small enough to add twice
+
+// 32-bit form of Step with saturation; once saturated the parities are meaningless and the user must
+// reject the map (d >= 2^24 can never pass the tests below).
+struct Step32 {
+    uint32_t d0, d1, cmax; // cmax: largest single increment seen
+};
+
+SEQFP_HD Step32 identity32()
+{
+    return Step32{0, 0, 0};
+}
+
+SEQFP_HD uint32_t sat_add(uint32_t a, uint32_t b)
+{
+    const uint32_t s = a + b;
+    return s > kSat ? kSat : s;
+}
+
+SEQFP_HD Step32 compose32(const Step32& first, const Step32& second)
+{
+    Step32 r;
+    r.d0 = sat_add(first.d0, (first.d0 & 1u) ? second.d1 : second.d0);
+    r.d1 = sat_add(first.d1, ((first.d1 + 1u) & 1u) ? second.d1 : second.d0);
+    r.cmax = first.cmax > second.cmax ? first.cmax : second.cmax;
+    return r;
+}
+
+// Map of one element (for additions and subtractions alike) in the epoch with exponent e.
+SEQFP_HD Step32 step32(float q, int e)
+{
+    uint32_t Mq, a, ce, co;
+    int eq;
+    split(q, Mq, eq);
+    if (eq > e)
+        return Step32{kSat, kSat, kSat};
+    unit_step(Mq, eq, e, a, ce, co);
+    return Step32{ce, co, ce > co ? ce : co};
+}
+
+// May a group's map g (built for exponent e) be applied to the running sum m * ulp(e)?  Sufficient: the state
+// after the group, plus one more of its largest increments, still lies inside the binade.
+SEQFP_HD bool group_add_ok(long long m, const Step32& g)
+{
+    const uint32_t d = (m & 1) ? g.d1 : g.d0;
+    return d < (1u << 24) && m + (long long)d + (long long)g.cmax + 1 < (1ll << 24);
+}
+
+// Same for the walk state r = m * ulp(e), for a group of a DESCENDING list whose first (largest) weight is
+// q_first: the state after the group must stay in the binade with room for one more decrement, and must
+// still be at least q_first, so no element of the group can have stopped the walk.
+SEQFP_HD bool group_sub_ok(long long m, int e, const Step32& g, float q_first)
+{
+    const uint32_t d = (m & 1) ? g.d1 : g.d0;
+    if (d >= (1u << 24))
+        return false;
+    const long long m_end = m - (long long)d;
+    if (e > 1 && m_end - (long long)g.cmax - 1 < (1ll << 23))
+        return false;
+    if (m_end <= 0)
+        return false;
+    return !walk_stop(m_end, q_first, e);
+}
+
 } // namespace seqfp

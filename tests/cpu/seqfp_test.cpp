@@ -142,6 +142,85 @@ static size_t emu_walk(const std::vector<float>& q, float r, int NT, int LMAX)
     }
 }
 
+// The grouped scheme of the kernels on a sorted list: group maps under epochs guessed from fp64 prefix
+// sums, a serial chain that accepts a map only when group_add_ok / group_sub_ok hold and otherwise replays the
+// group with real fp32 arithmetic.
+static int exponent_of(float x)
+{
+    uint32_t M;
+    int e;
+    split(x, M, e);
+    return e;
+}
+
+static float grouped_sum(const std::vector<float>& q, size_t GS, long* accepted, long* groups)
+{
+    const size_t n = q.size(), G = (n + GS - 1) / GS;
+    std::vector<double> pg(G + 1, 0.0);
+    for (size_t g = 0; g < G; ++g) {
+        double s = 0;
+        for (size_t i = g * GS; i < std::min(n, (g + 1) * GS); ++i)
+            s += q[i];
+        pg[g + 1] = pg[g] + s;
+    }
+    float S = 0.0f;
+    for (size_t g = 0; g < G; ++g) {
+        ++*groups;
+        const int eg = pg[g] > 0 ? exponent_of(float(pg[g])) : 0;
+        Step32 st = identity32();
+        for (size_t i = g * GS; i < std::min(n, (g + 1) * GS); ++i)
+            st = compose32(st, step32(q[i], eg));
+        uint32_t M;
+        int e;
+        split(S, M, e);
+        if (e == eg && group_add_ok(M, st)) {
+            ++*accepted;
+            S = join(uint32_t(M + ((M & 1) ? st.d1 : st.d0)), e);
+        } else {
+            for (size_t i = g * GS; i < std::min(n, (g + 1) * GS); ++i)
+                S += q[i];
+        }
+    }
+    return S;
+}
+
+static size_t grouped_walk(const std::vector<float>& q, float r, size_t GS, long* accepted, long* groups)
+{
+    const size_t n = q.size(), G = (n + GS - 1) / GS;
+    if (r < 0)
+        return 0;
+    std::vector<double> pg(G + 1, 0.0);
+    for (size_t g = 0; g < G; ++g) {
+        double s = 0;
+        for (size_t i = g * GS; i < std::min(n, (g + 1) * GS); ++i)
+            s += q[i];
+        pg[g + 1] = pg[g] + s;
+    }
+    const double r0 = r;
+    for (size_t g = 0; g < G; ++g) {
+        ++*groups;
+        const double guess = r0 - pg[g];
+        const int eg = guess > 0 ? exponent_of(float(guess)) : 0;
+        Step32 st = identity32();
+        for (size_t i = g * GS; i < std::min(n, (g + 1) * GS); ++i)
+            st = compose32(st, step32(q[i], eg));
+        uint32_t M;
+        int e;
+        split(r, M, e);
+        if (e == eg && group_sub_ok(M, e, st, q[g * GS])) {
+            ++*accepted;
+            r = join(uint32_t(M - ((M & 1) ? st.d1 : st.d0)), e);
+        } else {
+            for (size_t i = g * GS; i < std::min(n, (g + 1) * GS); ++i) {
+                if (r < q[i])
+                    return i;
+                r -= q[i];
+            }
+        }
+    }
+    return n - 1;
+}
+
 int main()
 {
     std::mt19937_64 rng(12345);
@@ -195,6 +274,49 @@ int main()
             }
         }
     }
+    // grouped scheme on sorted lists
+    long acc = 0, grp = 0;
+    for (int it = 0; it < 1500; ++it) {
+        const int kind = it % 5;
+        size_t n = 1 + rng() % (it % 25 == 0 ? 300000 : 20000);
+        std::vector<float> q(n);
+        for (auto& v : q) {
+            switch (kind) {
+            case 0: v = std::exp(2.5f * N(rng)); break;
+            case 1: v = std::exp(0.1f * N(rng)); break;
+            case 2: v = std::exp(6.0f * N(rng) - 6.0f); break;
+            case 3: v = float(1 + rng() % 16) * 0.0625f; break;
+            default: v = U(rng); break;
+            }
+            if (!(v > 0))
+                v = 1.0f;
+        }
+        const float mx = *std::max_element(q.begin(), q.end());
+        for (auto& v : q)
+            v = std::min(v / mx, 1.0f);
+        std::sort(q.begin(), q.end(), std::greater<float>());
+        const size_t GS = (it % 2) ? 256 : 64;
+        const float total = seq_sum(q);
+        const float got = grouped_sum(q, GS, &acc, &grp);
+        ++cases;
+        if (f2u(total) != f2u(got)) {
+            ++fails;
+            std::printf("GROUP SUM mismatch it=%d n=%zu kind=%d want=%a got=%a\n", it, n, kind, total, got);
+        }
+        for (int dd = 0; dd < 5; ++dd) {
+            float u = U(rng);
+            if (dd == 3) u = 0.0f;
+            if (dd == 4) u = std::nextafter(1.0f, 0.0f);
+            const float r = u * total;
+            const size_t a = seq_walk(q, r), b = grouped_walk(q, r, GS, &acc, &grp);
+            ++cases;
+            if (a != b) {
+                ++fails;
+                std::printf("GROUP WALK mismatch it=%d n=%zu kind=%d u=%a want=%zu got=%zu\n", it, n, kind, u, a, b);
+            }
+        }
+    }
+    std::printf("grouped: %ld of %ld groups took the fast map\n", acc, grp);
     std::printf("%ld cases, %ld failures, %ld sum rounds\n", cases, fails, rounds);
     return fails ? 1 : 0;
 }
