@@ -98,10 +98,10 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.part_n, (size_t)max_rows * mako::kMaxSlices));
     MAKO_HIP(ctx, dev_alloc(&sc.tickets, (size_t)max_rows * 32));
     MAKO_HIP(ctx, hipMemset(sc.tickets, 0, (size_t)max_rows * 32 * sizeof(uint32_t)));
-    MAKO_HIP(ctx, dev_alloc(&sc.binc, (size_t)max_rows * mako::kBins));
-    MAKO_HIP(ctx, hipMemset(sc.binc, 0, (size_t)max_rows * mako::kBins * sizeof(uint32_t)));
-    MAKO_HIP(ctx, dev_alloc(&sc.bins, (size_t)max_rows * mako::kBins));
-    MAKO_HIP(ctx, hipMemset(sc.bins, 0, (size_t)max_rows * mako::kBins * sizeof(unsigned long long)));
+    MAKO_HIP(ctx, dev_alloc(&sc.binc, (size_t)max_rows * sc.slices_cap * mako::kBins));
+    MAKO_HIP(ctx, dev_alloc(&sc.plan, (size_t)max_rows));
+    MAKO_HIP(ctx, hipMemset(sc.plan, 0, (size_t)max_rows * sizeof(mako::BigPlan)));
+    MAKO_HIP(ctx, dev_alloc(&sc.bins, (size_t)max_rows * sc.slices_cap * mako::kBins));
     MAKO_HIP(ctx, dev_alloc(&sc.wbuf, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.cnt, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.key[0], rv));
@@ -116,7 +116,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
                              (const void*)mako::scan_kernel<true, 8>,    (const void*)mako::scan_kernel<false, 8>,
                              (const void*)mako::finish_kernel<true, 0>,  (const void*)mako::finish_kernel<false, 0>,
                              (const void*)mako::finish_kernel<true, 2>,  (const void*)mako::finish_kernel<false, 2>,
-                             (const void*)mako::finish_kernel<true, 8>,  (const void*)mako::finish_kernel<false, 8>};
+                             (const void*)mako::finish_kernel<true, 8>,  (const void*)mako::finish_kernel<false, 8>,
+                             (const void*)mako::sort_kernel};
     for (const void* k : kernels)
         MAKO_HIP(ctx, hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)mako::kDynLds));
     return MAKO_OK;
@@ -128,7 +129,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.tickets, sc.binc, sc.bins,
+    void* ptrs[] = {sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.tickets, sc.binc, sc.bins, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
                     ctx->st_hist,  ctx->st_hcnt, ctx->st_hlen,  ctx->st_draft, ctx->st_tokens, ctx->st_acc};
@@ -194,6 +195,8 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     else
         MAKO_LAUNCH(false, 0);
 #undef MAKO_LAUNCH
+    // rows whose nucleus is too wide for the candidate lists left a work order; the others cost one load each
+    hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc);
     MAKO_HIP(ctx, hipGetLastError());
     return MAKO_OK;
 }
@@ -283,6 +286,15 @@ int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t
         MAKO_HIP(ctx, hipMemcpy(out_accepted, ctx->st_acc, n_rows, hipMemcpyDeviceToHost));
     return MAKO_OK;
 }
+
+#ifdef MAKO_TIMING
+// tuning builds only: copies the stage timestamps of row 0 (100 MHz wall clock) to the host
+int mako_sampler_debug_stamps(unsigned long long* out32)
+{
+    return hipMemcpyFromSymbol(out32, HIP_SYMBOL(mako::g_mako_stamp), 32 * sizeof(unsigned long long)) == hipSuccess
+               ? MAKO_OK : MAKO_ERR_HIP;
+}
+#endif
 
 int mako_sampler_debug_expf(const float* x_dev, float* y_dev, uint32_t n, void* stream)
 {

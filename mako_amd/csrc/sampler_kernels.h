@@ -25,6 +25,19 @@
 namespace mako {
 
 constexpr uint32_t kNone = 0xffffffffu;
+
+// Optional stage timestamps of row 0 (thread 0), for tuning builds only.
+#ifdef MAKO_TIMING
+__device__ unsigned long long g_mako_stamp[32];
+#define MAKO_STAMP(i)                                                                                                \
+    do {                                                                                                             \
+        if (threadIdx.x == 0 && blockIdx.y == 0)                                                                     \
+            g_mako_stamp[i] = wall_clock64();                                                                        \
+    } while (0)
+#else
+#define MAKO_STAMP(i) ((void)0)
+#endif
+
 constexpr uint32_t kSliceMax = 16384; // elements per slice: 16 per thread
 constexpr uint32_t kMaxSlices = 64;
 constexpr uint32_t kCap = 512;       // candidates kept per slice
@@ -46,6 +59,22 @@ struct SliceStat {
     uint32_t pad[3];
 };
 
+constexpr uint32_t kWorkers = 16; // workgroups that share the sort of one wide-nucleus row
+
+// Work order for a top_k == 0 row whose nucleus is too wide for the per-slice candidate lists: the weights
+// with bits(q) >= key_lo (n0 of them) are split by value into kWorkers contiguous ranges of about equal size.
+struct BigPlan {
+    uint32_t flag;   // 1: the row waits for sort_kernel's workers; 2: for its whole-row path (worker 0 alone)
+    uint32_t n0;     // entries to sort
+    uint32_t ticket; // workers that have finished
+    uint32_t pad;
+    double total64;  // exact fp64 sum of q over the row's candidates
+    uint32_t key_lo[kWorkers]; // worker w takes bits(q) in [key_lo[w], key_hi[w])
+    uint32_t key_hi[kWorkers];
+    uint32_t off[kWorkers];    // and writes them from position off[w] of the sorted list
+    uint32_t cnt[kWorkers];
+};
+
 struct Scratch {
     SliceStat* stats;  // [max_rows][kMaxSlices]
     float* cand_w;     // [max_rows][slices_cap][kCap] penalised logits of the slice's candidates
@@ -53,9 +82,10 @@ struct Scratch {
     double* part_sum;  // [max_rows][kMaxSlices] exact fp64 sum of q over the slice (top_k == 0 rows)
     uint32_t* part_n;  // [max_rows][kMaxSlices] candidates (q > 0, q >= min_p) in the slice
     uint32_t* tickets; // [max_rows][32] arrival counter of the row's slices (one per 128-byte line); zero between calls
-    uint32_t* binc;    // [max_rows][kBins] candidates per weight bin (top_k == 0 rows); all zero between calls
-    unsigned long long* bins; // [max_rows][kBins] sum of their 24-bit significands: the bin's exact mass is
-                              // bins * 2^(e - 150), e being the bin's exponent; all zero between calls
+    uint32_t* binc;    // [max_rows][slices_cap][kBins] candidates per weight bin of each slice (top_k == 0 rows)
+    BigPlan* plan;     // [max_rows]; flag and ticket zero between calls
+    unsigned long long* bins; // [max_rows][slices_cap][kBins] sum of their 24-bit significands: a bin's exact
+                              // mass is bins * 2^(e - 150), e being the bin's exponent
     float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path; top_k == 0 rows keep
                        // bits(q) of every logit here instead (0 where q is not a candidate)
     uint32_t* cnt;     // [max_rows][vpad] token counts; all zero between calls
@@ -522,6 +552,7 @@ struct FinishShared {
     uint32_t run[256];
     uint32_t flag;
     uint32_t ticket;
+    uint32_t soff[kMaxSlices + 1]; // first candidate of each slice in the row's flattened candidate list
 };
 
 // Views into the 64 KB dynamic LDS block; `cnt` (first pass) overlaps the two others (second pass).
@@ -901,151 +932,86 @@ __device__ void build_group_maps(const uint32_t* kf, uint32_t n, bool walk, doub
 {
     using namespace seqfp;
     const uint32_t groups = (n + kGroup - 1) / kGroup;
-    for (uint32_t g = wave_id(); g < groups; g += kWaves) {
-        const double guess = walk ? r0 - G.pg[g] : G.pg[g];
-        const int eg = guess > 0 ? exponent_of((float)guess) : 0;
-        Step32 st = Step32{kSat, kSat, kSat};
-        if (eg > 0) { // uniform per wave
-            float q[4];
-            load_group(kf, g, n, q);
-            st = identity32();
+    // four groups per trip and wave, their loads issued together
+    for (uint32_t g0 = wave_id() * 4u; g0 < groups; g0 += kWaves * 4u) {
+        float q[4][4];
 #pragma unroll
-            for (uint32_t j = 0; j < 4; ++j)
-                if (g * kGroup + lane_id() * 4u + j < n)
-                    st = compose32(st, step32(q[j], eg));
-            st = wave_incl_scan_step32(st);
-        }
-        if (lane_id() == kWave - 1) {
-            G.d0[g] = st.d0;
-            G.d1[g] = st.d1;
-            G.cmax[g] = st.cmax;
-        }
-    }
-}
-
-// Entries [beg, end) of one group added to S one by one (exactly), by one wave.
-__device__ float exact_group_sum(const uint32_t* kf, uint32_t g, uint32_t n, float S)
-{
-    using namespace seqfp;
-    const uint32_t beg = g * kGroup, end = min(n, beg + kGroup), lane = lane_id();
-    float q[4];
-    load_group(kf, g, n, q);
-    uint32_t start = beg;
-    for (;;) {
-        uint32_t M;
-        int e;
-        split(S, M, e);
-        Step32 st = identity32();
+        for (uint32_t u = 0; u < 4; ++u)
+            load_group(kf, min(g0 + u, groups - 1u), n, q[u]);
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            const uint32_t i = beg + lane * 4u + j;
-            if (i >= start && i < end)
-                st = compose32(st, step32(q[j], e));
-        }
-        const Step32 incl = wave_incl_scan_step32(st);
-        Step32 excl;
-        excl.d0 = __shfl_up(incl.d0, 1);
-        excl.d1 = __shfl_up(incl.d1, 1);
-        if (lane == 0)
-            excl.d0 = excl.d1 = 0;
-        long long mm = (long long)M + (long long)((M & 1u) ? excl.d1 : excl.d0);
-        uint32_t hit = kNone;
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t g = g0 + u;
+            const double guess = g < groups ? (walk ? r0 - G.pg[g] : G.pg[g]) : 0.0;
+            const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+            Step32 st = Step32{kSat, kSat, kSat};
+            if (eg > 0) { // uniform per wave
+                st = identity32();
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            const uint32_t i = beg + lane * 4u + j;
-            if (hit == kNone && i >= start && i < end) {
-                if (add_event(mm, q[j], e))
-                    hit = i;
-                else
-                    mm = add_apply(mm, q[j], e);
+                for (uint32_t j = 0; j < 4; ++j)
+                    if (g * kGroup + lane_id() * 4u + j < n)
+                        st = compose32(st, step32(q[u][j], eg));
+                st = wave_incl_scan_step32(st);
+            }
+            if (lane_id() == kWave - 1 && g < groups) {
+                G.d0[g] = st.d0;
+                G.d1[g] = st.d1;
+                G.cmax[g] = st.cmax;
             }
         }
-        const unsigned long long bal = __ballot(hit != kNone);
-        if (bal == 0) {
-            const uint32_t dt = (M & 1u) ? __shfl(incl.d1, kWave - 1) : __shfl(incl.d0, kWave - 1);
-            return join(M + dt, e);
-        }
-        const int first = __ffsll((long long)bal) - 1;
-        const uint32_t iev = __shfl(hit, first);
-        const uint32_t mev = (uint32_t)__shfl((int)(uint32_t)mm, first);
-        const float qev = __uint_as_float(~kf[iev]);
-        S = join(mev, e) + qev;
-        start = iev + 1;
-        if (start >= end)
-            return S;
     }
 }
 
-// Entries of one group subtracted from r one by one (exactly), by one wave.  Returns true and the
+// The entries of one group added to S one by one with real fp32 additions.  Each lane fetches its four
+// entries once; the wave then replays them in list order, reading them back by lane index, so the chain is
+// 256 dependent adds on uniform values and nothing else.
+__device__ float exact_group_sum(const uint32_t* kf, uint32_t g, uint32_t n, float S)
+{
+    float q[4];
+    load_group(kf, g, n, q); // entries past the end read as 0.0f: adding them changes nothing
+    const uint32_t cnt = min(n - g * kGroup, kGroup);
+    const uint32_t lanes = (cnt + 3u) / 4u;
+    for (uint32_t l = 0; l < lanes; ++l) {
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            S += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), l));
+    }
+    return S;
+}
+
+// The entries of one group subtracted from r one by one (src/gen/sampler.cpp:67-71).  Returns true and the
 // entry's position when the walk stops inside the group, else false and the new r.
 __device__ bool exact_group_walk(const uint32_t* kf, uint32_t g, uint32_t n, float& r, uint32_t& pos)
 {
-    using namespace seqfp;
-    const uint32_t beg = g * kGroup, end = min(n, beg + kGroup), lane = lane_id();
     float q[4];
     load_group(kf, g, n, q);
-    uint32_t start = beg;
-    for (;;) {
-        uint32_t M;
-        int e;
-        split(r, M, e);
-        Step32 st = identity32();
+    const uint32_t beg = g * kGroup, cnt = min(n - beg, kGroup);
+    for (uint32_t l = 0; l * 4u < cnt; ++l) {
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            const uint32_t i = beg + lane * 4u + j;
-            if (i >= start && i < end)
-                st = compose32(st, step32(q[j], e));
-        }
-        const Step32 incl = wave_incl_scan_step32(st);
-        Step32 excl;
-        excl.d0 = __shfl_up(incl.d0, 1);
-        excl.d1 = __shfl_up(incl.d1, 1);
-        if (lane == 0)
-            excl.d0 = excl.d1 = 0;
-        long long mm = (long long)M - (long long)((M & 1u) ? excl.d1 : excl.d0);
-        uint32_t hit = kNone;
-        bool stop = false;
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            const uint32_t i = beg + lane * 4u + j;
-            if (hit == kNone && i >= start && i < end) {
-                if (walk_stop(mm, q[j], e)) {
-                    hit = i;
-                    stop = true;
-                } else if (sub_event(mm, q[j], e)) {
-                    hit = i;
-                } else {
-                    mm = sub_apply(mm, q[j], e);
+            if (l * 4u + j < cnt) {
+                const float x = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), l));
+                if (r < x) {
+                    pos = beg + l * 4u + j;
+                    return true;
                 }
+                r -= x;
             }
         }
-        const unsigned long long bal = __ballot(hit != kNone);
-        if (bal == 0) {
-            const uint32_t dt = (M & 1u) ? __shfl(incl.d1, kWave - 1) : __shfl(incl.d0, kWave - 1);
-            r = join(M - dt, e);
-            return false;
-        }
-        const int first = __ffsll((long long)bal) - 1;
-        const uint32_t iev = __shfl(hit, first);
-        if (__shfl((int)stop, first)) {
-            pos = iev;
-            return true;
-        }
-        const uint32_t mev = (uint32_t)__shfl((int)(uint32_t)mm, first);
-        r = join(mev, e) - __uint_as_float(~kf[iev]);
-        start = iev + 1;
-        if (start >= end)
-            return false;
     }
+    return false;
 }
 
 // Tail of every path that ends with a list sorted by (q desc, idx asc) in global memory: kf[i] = ~bits(q_i),
 // jf[i] = token id, n1 entries (already cut to top_k).  Applies top-p (src/gen/sampler.cpp:44-61) against
 // total64 (the fp64 sum over the row's candidates; summed from the list when !have_total), then the exact
 // fp32 total (:80-82) and walk (:64-73).  All 1024 threads must call it.
-__device__ void sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf,
+//
+// When `need_cut` the list is only the heaviest part of the row's candidates and every candidate missing from
+// it weighs at most q_bound: the nucleus must then end inside the list, at an entry strictly heavier than
+// q_bound.  If it does not, nothing is written and false is returned (the caller widens the list).
+__device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf,
                             const uint32_t* jf, uint32_t n1, bool have_total, double total64, uint32_t path,
-                            const FinishLds& L)
+                            const FinishLds& L, bool need_cut = false, float q_bound = 0.0f)
 {
     using namespace seqfp;
     FinishShared& sm = *L.sm;
@@ -1071,7 +1037,7 @@ __device__ void sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             }
             const double want = (double)P.top_p * total64;
             double carry = 0;
-            uint32_t keep = n;
+            uint32_t keep = kNone;
             for (uint32_t base = 0; base < n; base += kThreads) {
                 const uint32_t i = base + tid;
                 const double q = i < n ? (double)qat(i) : 0.0;
@@ -1085,23 +1051,33 @@ __device__ void sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 }
                 carry += tile;
             }
-            n = keep;
+            if (need_cut && keep == kNone)
+                return false;
+            n = keep == kNone ? n : keep;
         }
+        if (need_cut && !(q_bound < qat(n - 1)))
+            return false;
         draw_from_list(d, row, qat, idat, n, path, sm);
-        return;
+        return true;
     }
 
     // fp64 group sums and their prefix
+    MAKO_STAMP(5);
     const uint32_t groups1 = (n1 + kGroup - 1) / kGroup;
     __syncthreads();
-    for (uint32_t g = wave_id(); g < groups1; g += kWaves) {
-        float q[4];
-        load_group(kf, g, n1, q);
-        double s = (((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3];
-        for (int o = 32; o > 0; o >>= 1)
-            s += __shfl_xor(s, o);
-        if (lane_id() == 0)
-            G.pg[g + 1] = s;
+    for (uint32_t g0 = wave_id() * 4u; g0 < groups1; g0 += kWaves * 4u) {
+        float q[4][4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+            load_group(kf, min(g0 + u, groups1 - 1u), n1, q[u]);
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            double s = (((double)q[u][0] + (double)q[u][1]) + (double)q[u][2]) + (double)q[u][3];
+            for (int o = 32; o > 0; o >>= 1)
+                s += __shfl_xor(s, o);
+            if (lane_id() == 0 && g0 + u < groups1)
+                G.pg[g0 + u + 1] = s;
+        }
     }
     __syncthreads();
     {
@@ -1118,11 +1094,14 @@ __device__ void sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     __syncthreads();
 
     // top-p: first entry at which the running fp64 sum reaches top_p * total
+    MAKO_STAMP(6);
     uint32_t n = n1;
     if (topp_active) {
         const double want = (double)P.top_p * total64;
         const uint32_t hitg = (tid < groups1 && G.pg[tid + 1] >= want) ? tid : kNone;
         const uint32_t gs = block_min_u32(hitg, sm.bs);
+        if (need_cut && gs == kNone)
+            return false;
         if (gs != kNone) {
             if (wave_id() == 0) {
                 float q[4];
@@ -1157,29 +1136,42 @@ __device__ void sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     }
     if (n < 1)
         n = 1;
+    if (need_cut && !(q_bound < qat(n - 1)))
+        return false;
     __syncthreads();
 
     // exact fp32 total: group maps in parallel, then one wave chains them
+    MAKO_STAMP(7);
     build_group_maps(kf, n, false, 0.0, G);
     __syncthreads();
     const uint32_t groups = (n + kGroup - 1) / kGroup;
     if (wave_id() == 0) {
+        // 64 groups at a time: lane l fetches group base + l's guess and map, the chain reads them by lane index
         float S = 0.0f;
-        for (uint32_t g = 0; g < groups; ++g) {
-            uint32_t M;
-            int e;
-            split(S, M, e);
-            const int eg = G.pg[g] > 0 ? exponent_of((float)G.pg[g]) : 0;
-            const Step32 st = Step32{G.d0[g], G.d1[g], G.cmax[g]};
-            if (e == eg && group_add_ok((long long)M, st))
-                S = join(M + ((M & 1u) ? st.d1 : st.d0), e);
-            else
-                S = exact_group_sum(kf, g, n, S);
+        for (uint32_t base = 0; base < groups; base += kWave) {
+            const uint32_t gl = min(base + lane_id(), groups - 1u);
+            const int eg_l = G.pg[gl] > 0 ? exponent_of((float)G.pg[gl]) : 0;
+            const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], cm_l = G.cmax[gl];
+            const uint32_t cnt = min((uint32_t)kWave, groups - base);
+            for (uint32_t k = 0; k < cnt; ++k) {
+                uint32_t M;
+                int e;
+                split(S, M, e);
+                const int eg = __builtin_amdgcn_readlane(eg_l, k);
+                const Step32 st = Step32{(uint32_t)__builtin_amdgcn_readlane((int)d0_l, k),
+                                         (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k),
+                                         (uint32_t)__builtin_amdgcn_readlane((int)cm_l, k)};
+                if (e == eg && group_add_ok((long long)M, st))
+                    S = join(M + ((M & 1u) ? st.d1 : st.d0), e);
+                else
+                    S = exact_group_sum(kf, base + k, n, S);
+            }
         }
         if (lane_id() == 0)
             G.misc[1] = __float_as_uint(S);
     }
     __syncthreads();
+    MAKO_STAMP(8);
     const float total = __uint_as_float(G.misc[1]);
     const float span = total - 0.0f;
     const float prod = d.u[row] * span;
@@ -1196,17 +1188,29 @@ __device__ void sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         if (wave_id() == 0) {
             float r = r0;
             uint32_t at = n - 1;
-            for (uint32_t g = 0; g < groups; ++g) {
-                uint32_t M;
-                int e;
-                split(r, M, e);
-                const double guess = (double)r0 - G.pg[g];
-                const int eg = guess > 0 ? exponent_of((float)guess) : 0;
-                const Step32 st = Step32{G.d0[g], G.d1[g], G.cmax[g]};
-                if (e == eg && group_sub_ok((long long)M, e, st, qat(g * kGroup))) {
-                    r = join(M - ((M & 1u) ? st.d1 : st.d0), e);
-                } else if (exact_group_walk(kf, g, n, r, at)) {
-                    break;
+            bool stopped = false;
+            for (uint32_t base = 0; base < groups && !stopped; base += kWave) {
+                const uint32_t gl = min(base + lane_id(), groups - 1u);
+                const double guess_l = (double)r0 - G.pg[gl];
+                const int eg_l = guess_l > 0 ? exponent_of((float)guess_l) : 0;
+                const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], cm_l = G.cmax[gl];
+                const float qf_l = qat(gl * kGroup);
+                const uint32_t cnt = min((uint32_t)kWave, groups - base);
+                for (uint32_t k = 0; k < cnt; ++k) {
+                    uint32_t M;
+                    int e;
+                    split(r, M, e);
+                    const int eg = __builtin_amdgcn_readlane(eg_l, k);
+                    const Step32 st = Step32{(uint32_t)__builtin_amdgcn_readlane((int)d0_l, k),
+                                             (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k),
+                                             (uint32_t)__builtin_amdgcn_readlane((int)cm_l, k)};
+                    const float q_first = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(qf_l), k));
+                    if (e == eg && group_sub_ok((long long)M, e, st, q_first)) {
+                        r = join(M - ((M & 1u) ? st.d1 : st.d0), e);
+                    } else if (exact_group_walk(kf, base + k, n, r, at)) {
+                        stopped = true;
+                        break;
+                    }
                 }
             }
             if (lane_id() == 0)
@@ -1216,6 +1220,7 @@ __device__ void sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         pos = G.misc[2];
     }
 
+    MAKO_STAMP(9);
     if (d.out_cand_idx && d.out_cand_q)
         for (uint32_t j = tid; j < n && j < d.cand_cap; j += kThreads) {
             d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
@@ -1231,7 +1236,10 @@ __device__ void sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         o.accepted = 0;
         write_row(d, row, o);
     }
+    return true;
 }
+
+__device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t* i1, uint32_t n, const FinishLds& L);
 
 // Common tail of the whole-row paths.  key[0]/idx[0] of the row hold n0 candidates (~bits(q), token id) in index
 // order.  Sorts them by (q desc, idx asc) when top-k or top-p is active, truncates (src/gen/sampler.cpp:39-61)
@@ -1250,20 +1258,10 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
     // order by (q desc, idx asc): stable LSD radix sort of ~bits(q), ascending
     const bool topk_active = P.top_k > 0 && P.top_k < n0;
     const bool topp_active = P.top_p < 1.0f;
-    uint32_t *ks = key0, *is = idx0, *kd = key1, *id = idx1;
-    if (topk_active || topp_active) {
-        for (uint32_t shift = 0; shift < 32; shift += 8) {
-            if (radix_pass(ks, is, kd, id, n0, shift, L)) {
-                uint32_t* t = ks;
-                ks = kd;
-                kd = t;
-                t = is;
-                is = id;
-                id = t;
-            }
-            __syncthreads();
-        }
-    }
+    if (topk_active || topp_active)
+        sort_segment(key0, idx0, key1, idx1, n0, L);
+    const uint32_t *ks = key0, *is = idx0;
+    MAKO_STAMP(12);
     const uint32_t n1 = topk_active ? P.top_k : n0; // sampler.cpp:40-43
     if (topk_active || topp_active) {
         sorted_tail(d, row, P, ks, is, n1, have_total, total64, path, L);
@@ -1276,22 +1274,15 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
         d, row, [=](uint32_t i) { return __uint_as_float(~kf[i]); }, [=](uint32_t i) { return jf[i]; }, n1, path, sm);
 }
 
-// A top_k == 0 row whose nucleus is wider than the per-slice candidate lists.  The second pass left bits(q) of
-// every logit in scratch and a histogram of them (16 bins per binade).  Walking the bins from the heaviest down
-// with each bin priced at its LOWEST weight finds a bin by which the nucleus must have ended; only the logits of
-// the bins above are gathered (in index order), sorted and drawn from.  `total64` is the row's exact fp64 total.
-__device__ void nucleus_big_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
-                                double total64, uint32_t c0, uint32_t c1, unsigned long long s0, unsigned long long s1,
-                                const FinishLds& L)
+// Plans a top_k == 0 row from the histogram of its weights (16 bins per binade, exact masses): finds the bin by
+// which the nucleus must have ended and splits the weights above it over kWorkers workers by value.
+// Thread t brings the counts (c0, c1) and significand sums (s0, s1) of bins kBins-1-2t and kBins-2-2t.
+// Returns n0, the number of weights to sort; the plan is written to `plan` (flag left untouched).
+__device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, uint32_t c0, uint32_t c1,
+                                 unsigned long long s0, unsigned long long s1, BigPlan* plan, const FinishLds& L)
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
-    const uint32_t V = d.n_vocab;
-    const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
-    uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
-    uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
-
-    // bins from the top: thread t prices bins kBins-1-2t and kBins-2-2t, whose counts are c0 and c1
     const uint32_t b0 = kBins - 1u - 2u * tid, b1 = b0 - 1u;
     // exact mass of a bin: sum of significands times the bin's power of two (bins never straddle a binade)
     auto scale = [](uint32_t b) {
@@ -1304,7 +1295,7 @@ __device__ void nucleus_big_row(const mako_sample_desc& d, const Scratch& sc, ui
     const double incl = block_incl_scan_f64(m0 + m1, all, sm.bs);
     // The nucleus ends in the first bin (from the top) at which the running mass reaches `want`.  These sums
     // associate differently from the sorted prefix sums that make the final decision, so one more non-empty
-    // bin is taken along: the gather stops at the SECOND bin that satisfies the test.
+    // bin is taken along: the list stops at the SECOND bin that satisfies the test.
     const bool r0 = c0 && incl - m1 >= want, r1 = c1 && incl >= want;
     uint32_t reached_total;
     const uint32_t before = block_excl_scan_u32((uint32_t)r0 + (uint32_t)r1, reached_total, sm.bs);
@@ -1315,11 +1306,59 @@ __device__ void nucleus_big_row(const mako_sample_desc& d, const Scratch& sc, ui
         hit = b1;
     const uint32_t rev = block_min_u32(hit == kNone ? kNone : kBins - 1u - hit, sm.bs);
     const uint32_t b_lo = rev == kNone ? 0u : kBins - 1u - rev; // not reached twice: keep every candidate
-    const uint32_t key_lo = b_lo << 19;
 
-    // gather the logits with bits(q) >= key_lo, in index order.  Wave w owns a contiguous chunk of the row:
-    // a counting sweep, one exchange of the 16 wave totals, then a writing sweep in which ranks come from
-    // ballots.  Lane l holds entries 4l..4l+3 of each 256-entry group.
+    // candidates above each bin, and the workers' shares
+    uint32_t count_all;
+    const uint32_t above0 = block_excl_scan_u32(c0 + c1, count_all, sm.bs), above1 = above0 + c0;
+    uint32_t* w_hi = L.wcount;            // highest bin of each worker
+    uint32_t* w_lo = L.wcount + kWorkers; // lowest bin
+    uint32_t* w_off = L.wcount + 2 * kWorkers;
+    uint32_t* w_cnt = L.wcount + 3 * kWorkers;
+    if (tid < kWorkers) {
+        w_hi[tid] = 0;
+        w_lo[tid] = kNone;
+        w_off[tid] = kNone;
+        w_cnt[tid] = 0;
+    }
+    if (b0 == b_lo)
+        sm.flag = above0 + c0;
+    if (b1 == b_lo)
+        sm.flag = above1 + c1;
+    __syncthreads();
+    const uint32_t n0 = sm.flag;
+    auto assign = [&](uint32_t b, uint32_t c, uint32_t above) {
+        if (c == 0 || b < b_lo)
+            return;
+        const uint32_t w = min(kWorkers - 1u, (uint32_t)(((unsigned long long)above * kWorkers) / n0));
+        atomicMax(&w_hi[w], b);
+        atomicMin(&w_lo[w], b);
+        atomicMin(&w_off[w], above);
+        atomicAdd(&w_cnt[w], c);
+    };
+    assign(b0, c0, above0);
+    assign(b1, c1, above1);
+    __syncthreads();
+    if (tid < kWorkers) {
+        plan->key_lo[tid] = w_lo[tid] << 19;
+        plan->key_hi[tid] = (w_hi[tid] + 1u) << 19;
+        plan->off[tid] = w_cnt[tid] ? w_off[tid] : 0u;
+        plan->cnt[tid] = w_cnt[tid];
+    }
+    if (tid == 0) {
+        plan->n0 = n0;
+        plan->total64 = total64;
+    }
+    __syncthreads();
+    return n0;
+}
+
+// Copies the weights of the row with key_lo <= bits(q) < key_hi, in index order, to kout / iout (as ~bits(q) and
+// token id).  Wave w owns a contiguous chunk of the row: a counting sweep, one exchange of the 16 wave totals,
+// then a writing sweep in which ranks come from ballots.  Lane l holds entries 4l..4l+3 of each 256-entry group.
+// Returns the number of entries written.
+__device__ uint32_t gather_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, uint32_t key_hi, uint32_t* kout,
+                                 uint32_t* iout, FinishShared& sm)
+{
     const uint32_t lane = lane_id(), wave = wave_id();
     const uint32_t chunk = ((V + kThreads * 4u - 1u) / (kThreads * 4u)) * kGroup; // per wave, a multiple of 256
     const uint32_t beg = min(V, wave * chunk), end = min(V, beg + chunk);
@@ -1337,20 +1376,24 @@ __device__ void nucleus_big_row(const mako_sample_desc& d, const Scratch& sc, ui
         }
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
-            if (k[j] < key_lo)
+            if (k[j] < key_lo || k[j] >= key_hi)
                 k[j] = 0;
     };
     uint32_t mine = 0;
-    for (uint32_t base = beg; base < end; base += 2u * kGroup) {
-        uint32_t ka[4], kb[4];
-        fetch(base + lane * 4u, ka);
-        fetch(base + kGroup + lane * 4u, kb);
+    for (uint32_t base = beg; base < end; base += 4u * kGroup) {
+        uint32_t k[4][4];
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            mine += (ka[j] != 0) + (kb[j] != 0);
+        for (uint32_t u = 0; u < 4; ++u)
+            fetch(base + u * kGroup + lane * 4u, k[u]);
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                mine += k[u][j] != 0;
     }
     for (int o = 32; o > 0; o >>= 1)
         mine += __shfl_xor(mine, o);
+    __syncthreads();
     if (lane == 0)
         sm.bs.u64[wave] = mine;
     __syncthreads();
@@ -1362,29 +1405,59 @@ __device__ void nucleus_big_row(const mako_sample_desc& d, const Scratch& sc, ui
         n0 += x;
     }
     const unsigned long long lower = (1ull << lane) - 1ull;
-    for (uint32_t base = beg; base < end; base += kGroup) {
-        uint32_t k[4];
-        fetch(base + lane * 4u, k);
-        unsigned long long bal[4];
-        uint32_t before = 0, total = 0;
+    for (uint32_t base = beg; base < end; base += 2u * kGroup) {
+        uint32_t k[2][4];
+        fetch(base + lane * 4u, k[0]);
+        fetch(base + kGroup + lane * 4u, k[1]);
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            bal[j] = __ballot(k[j] != 0);
-            before += (uint32_t)__popcll(bal[j] & lower);
-            total += (uint32_t)__popcll(bal[j]);
-        }
-        uint32_t pos = out + before;
+        for (uint32_t u = 0; u < 2; ++u) {
+            uint32_t before = 0, total = 0;
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            if (k[j]) {
-                key0[pos] = ~k[j];
-                idx0[pos] = base + lane * 4u + j;
-                ++pos;
+            for (uint32_t j = 0; j < 4; ++j) {
+                const unsigned long long bal = __ballot(k[u][j] != 0);
+                before += (uint32_t)__popcll(bal & lower);
+                total += (uint32_t)__popcll(bal);
             }
-        out += total;
+            uint32_t pos = out + before;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (k[u][j]) {
+                    kout[pos] = ~k[u][j];
+                    iout[pos] = base + u * kGroup + lane * 4u + j;
+                    ++pos;
+                }
+            out += total;
+        }
     }
     __syncthreads();
-    sort_truncate_draw(d, sc, row, P, n0, true, total64, MAKO_PATH_GENERAL, L);
+    return n0;
+}
+
+// Sorts n (key, id) pairs at (k0, i0) by key ascending, stably, with (k1, i1) as the second buffer; the result
+// ends in (k0, i0).
+__device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t* i1, uint32_t n, const FinishLds& L)
+{
+    if (n < 2)
+        return;
+    uint32_t *ks = k0, *is = i0, *kd = k1, *id = i1;
+    for (uint32_t shift = 0; shift < 32; shift += 8) {
+        if (radix_pass(ks, is, kd, id, n, shift, L)) {
+            uint32_t* t = ks;
+            ks = kd;
+            kd = t;
+            t = is;
+            is = id;
+            id = t;
+        }
+        __syncthreads();
+    }
+    if (ks != k0) {
+        for (uint32_t i = threadIdx.x; i < n; i += kThreads) {
+            k0[i] = ks[i];
+            i0[i] = is[i];
+        }
+        __syncthreads();
+    }
 }
 
 // Whole-row path: exact for every parameter combination.  One workgroup rebuilds the penalised
@@ -1473,24 +1546,86 @@ __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32
     sort_truncate_draw(d, sc, row, P, n0, false, 0.0, MAKO_PATH_GENERAL, L);
 }
 
-// Bitonic sort of a[0..n), n a power of two, descending.
-__device__ void bitonic_sort_desc(unsigned long long* a, uint32_t n)
+// Bitonic sort, descending, of 1024 * ITEMS keys held ITEMS per thread: key[t] is element t * 1024 + tid.
+// Partners 1024 or more apart are other registers of the same thread, partners less than 64 apart are lanes
+// of the same wave (shuffles); only the strides in between go through LDS (two barriers each).
+template <int ITEMS>
+__device__ void bitonic_sort_regs(unsigned long long (&key)[ITEMS], unsigned long long* lds)
 {
     const uint32_t tid = threadIdx.x;
-    for (uint32_t k = 2; k <= n; k <<= 1)
+    for (uint32_t k = 2; k <= 1024u * ITEMS; k <<= 1)
         for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-            for (uint32_t t = tid; t < n / 2; t += kThreads) {
-                const uint32_t i = ((t & ~(j - 1u)) << 1) | (t & (j - 1u));
-                const uint32_t p = i | j;
-                const unsigned long long x = a[i], y = a[p];
-                const bool desc = (i & k) == 0;
-                if ((x < y) == desc) {
-                    a[i] = y;
-                    a[p] = x;
+            if (j >= 1024u) {
+                // register-to-register stage; every index below is a compile-time constant so that key[]
+                // stays in registers
+#pragma unroll
+                for (uint32_t dj = 1; dj < (uint32_t)ITEMS; dj <<= 1)
+                    if (j == dj * 1024u) {
+#pragma unroll
+                        for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t)
+                            if ((t & dj) == 0) {
+                                const bool desc = ((t * 1024u + tid) & k) == 0;
+                                const unsigned long long a = key[t], b = key[t | dj];
+                                const bool swap = (a < b) == desc;
+                                key[t] = swap ? b : a;
+                                key[t | dj] = swap ? a : b;
+                            }
+                    }
+            } else if (j >= (uint32_t)kWave) {
+#pragma unroll
+                for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t)
+                    lds[t * 1024u + tid] = key[t];
+                __syncthreads();
+#pragma unroll
+                for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t) {
+                    const unsigned long long other = lds[t * 1024u + (tid ^ j)];
+                    const bool keep_max = ((tid & j) == 0) == (((t * 1024u + tid) & k) == 0);
+                    key[t] = keep_max ? (key[t] > other ? key[t] : other) : (key[t] < other ? key[t] : other);
+                }
+                __syncthreads();
+            } else {
+#pragma unroll
+                for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t) {
+                    const unsigned long long other = __shfl_xor(key[t], (int)j);
+                    const bool keep_max = ((tid & j) == 0) == (((t * 1024u + tid) & k) == 0);
+                    key[t] = keep_max ? (key[t] > other ? key[t] : other) : (key[t] < other ? key[t] : other);
                 }
             }
-            __syncthreads();
         }
+}
+
+// The row's candidates (all slices) weighted, sorted by (q desc, idx asc) and left in LDS as kf[i] = ~bits(q_i),
+// jf[i] = token id, invalid ones (q not a candidate) last.  Returns the number of valid candidates.
+template <int ITEMS>
+__device__ uint32_t sort_candidates(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_cands, float m, float inv_t,
+                                    float floor_q, uint32_t* kf, uint32_t* jf, const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    unsigned long long key[ITEMS];
+#pragma unroll
+    for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t) {
+        const uint32_t c = t * 1024u + tid;
+        key[t] = 0;
+        if (c < n_cands) {
+            uint32_t s = 0;
+            while (s + 1 < slices && c >= sm.soff[s + 1]) // slice holding candidate c
+                ++s;
+            const size_t at = ((size_t)row * sc.slices_cap + s) * kCap + (c - sm.soff[s]);
+            const float q = weight_of(sc.cand_w[at], m, inv_t, sm.tab);
+            if (q >= floor_q && q > 0.0f)
+                key[t] = ((unsigned long long)__float_as_uint(q) << 32) | (unsigned long long)(kNone - sc.cand_i[at]);
+        }
+    }
+    bitonic_sort_regs<ITEMS>(key, L.sortk);
+    uint32_t nv = 0;
+#pragma unroll
+    for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t) {
+        kf[t * 1024u + tid] = ~(uint32_t)(key[t] >> 32);
+        jf[t * 1024u + tid] = kNone - (uint32_t)key[t];
+        nv += key[t] != 0;
+    }
+    return block_sum_u32(nv, sm.bs); // (its barriers publish kf / jf)
 }
 
 // Exact fp64 sum of q over one slice, and the number of candidates in it (q > 0 and q >= min_p).
@@ -1579,31 +1714,66 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
             }
         }
     __syncthreads();
-    uint32_t* binc = sc.binc + (size_t)row * kBins;
-    unsigned long long* bins = sc.bins + (size_t)row * kBins;
-    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads)
-        if (hist[b]) {
-            atomicAdd(&binc[b], hist[b]);
-            atomicAdd(&bins[b], hsum[b]);
-        }
+    // the slice's histogram goes to its own place: no atomics, nothing to clear afterwards
+    uint32_t* binc = sc.binc + ((size_t)row * sc.slices_cap + slice) * kBins;
+    unsigned long long* bins = sc.bins + ((size_t)row * sc.slices_cap + slice) * kBins;
+    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads) {
+        binc[b] = hist[b];
+        bins[b] = hsum[b];
+    }
+}
+
+// Kernel arguments that are handed on by reference to out-of-line device functions would be spilled to scratch
+// memory (a microsecond per access); the two finishing kernels keep their copies in LDS instead.
+struct ArgsLds {
+    mako_sample_desc d;
+    Scratch sc;
+    mako_sampling_params P; // the row's parameters
+};
+
+__device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const Scratch& sc_arg, ArgsLds& a)
+{
+    static_assert(sizeof(mako_sample_desc) % 4 == 0 && sizeof(Scratch) % 4 == 0, "word copies");
+    const uint32_t* src_d = reinterpret_cast<const uint32_t*>(&d_arg);
+    const uint32_t* src_s = reinterpret_cast<const uint32_t*>(&sc_arg);
+    uint32_t* dst_d = reinterpret_cast<uint32_t*>(&a.d);
+    uint32_t* dst_s = reinterpret_cast<uint32_t*>(&a.sc);
+    for (uint32_t i = threadIdx.x; i < sizeof(mako_sample_desc) / 4; i += kThreads)
+        dst_d[i] = src_d[i];
+    for (uint32_t i = threadIdx.x; i < sizeof(Scratch) / 4; i += kThreads)
+        dst_s[i] = src_s[i];
+    const uint32_t* src_p = reinterpret_cast<const uint32_t*>(d_arg.params + blockIdx.y);
+    uint32_t* dst_p = reinterpret_cast<uint32_t*>(&a.P);
+    if (threadIdx.x < sizeof(mako_sampling_params) / 4)
+        dst_p[threadIdx.x] = src_p[threadIdx.x];
+    __syncthreads();
 }
 
 // grid = (slices, rows).  Only top_k == 0 rows use more than their first workgroup.
 template <bool VEC, int KH>
-__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Scratch sc, uint32_t slices, uint32_t slice_len)
+__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices,
+                                                          uint32_t slice_len)
 {
     extern __shared__ unsigned long long s_dyn64[];
     __shared__ FinishShared sm;
+    __shared__ ArgsLds s_args;
+    {
+        const mako_sampling_params P0 = d_arg.params[blockIdx.y];
+        if (classify(P0) != kNucleus && blockIdx.x != 0)
+            return;
+    }
+    stage_args(d_arg, sc_arg, s_args);
+    const mako_sample_desc& d = s_args.d;
+    const Scratch& sc = s_args.sc;
     FinishLds L;
     L.sm = &sm;
     L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
     L.sortk = s_dyn64;                                             // 32 KB
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);    // next 16 KB
     const uint32_t row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
-    const mako_sampling_params P = d.params[row];
+    const mako_sampling_params& P = s_args.P;
     const RowClass cls = classify(P);
-    if (cls != kNucleus && slice != 0)
-        return;
+    MAKO_STAMP(0);
     if (tid < 32)
         sm.tab[tid] = k_exp2_tab[tid];
     __syncthreads();
@@ -1628,6 +1798,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Sc
         argidx = 0;
     }
 
+    MAKO_STAMP(1);
     if (cls == kGreedy) { // sampler.cpp:77-78, 88-92
         if (tid == 0) {
             RowOut o;
@@ -1658,8 +1829,9 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Sc
             sc.tickets[(size_t)row * 32] = 0;
     }
 
+    MAKO_STAMP(2);
     // top_k == 0: the row's exact total and candidate count from the second pass, and this thread's two bins of
-    // the weight histogram (read and cleared here so that the histogram is all zero again for the next call)
+    // the weight histogram (summed over the slices)
     double row_total = 0;
     uint32_t row_n0 = 0, bin_c0 = 0, bin_c1 = 0;
     unsigned long long bin_s0 = 0, bin_s1 = 0;
@@ -1668,124 +1840,154 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d, Sc
             row_total += sc.part_sum[(size_t)row * kMaxSlices + s];
             row_n0 += sc.part_n[(size_t)row * kMaxSlices + s];
         }
-        uint32_t* binc = sc.binc + (size_t)row * kBins;
-        bin_c0 = binc[kBins - 1u - 2u * tid];
-        bin_c1 = binc[kBins - 2u - 2u * tid];
-        binc[kBins - 1u - 2u * tid] = 0;
-        binc[kBins - 2u - 2u * tid] = 0;
-        unsigned long long* bins = sc.bins + (size_t)row * kBins;
-        bin_s0 = bins[kBins - 1u - 2u * tid];
-        bin_s1 = bins[kBins - 2u - 2u * tid];
-        bins[kBins - 1u - 2u * tid] = 0;
-        bins[kBins - 2u - 2u * tid] = 0;
+        for (uint32_t s = 0; s < slices; ++s) {
+            const uint32_t* binc = sc.binc + ((size_t)row * sc.slices_cap + s) * kBins;
+            const unsigned long long* bins = sc.bins + ((size_t)row * sc.slices_cap + s) * kBins;
+            bin_c0 += binc[kBins - 1u - 2u * tid];
+            bin_c1 += binc[kBins - 2u - 2u * tid];
+            bin_s0 += bins[kBins - 1u - 2u * tid];
+            bin_s1 += bins[kBins - 2u - 2u * tid];
+        }
         if (row_n0 == 0) {
             fallback_row(d, row, argidx);
             return;
         }
     }
-    if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
-        if (cls == kNucleus)
-            nucleus_big_row(d, sc, row, P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, L);
-        else
-            general_row(d, sc, row, P, m, argidx, L);
+    // a top_k == 0 row is planned from its histogram first: only a narrow nucleus can end inside the candidates
+    bool try_candidates = true;
+    if (cls == kNucleus) {
+        const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, L);
+        try_candidates = n0 <= 1024u && !any_overflow && n_cands <= kSortMax;
+        if (!try_candidates) {
+            if (tid == 0)
+                sc.plan[row].flag = 1; // sort_kernel takes the row
+            return;
+        }
+    } else if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
+        if (tid == 0) {
+            sc.plan[row].total64 = (double)m; // carries the row maximum and its first index to the whole-row path
+            sc.plan[row].n0 = argidx;
+            sc.plan[row].flag = 2;
+        }
         return;
     }
 
     // ---- candidate path: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
-    uint32_t npad = 64;
-    while (npad < n_cands)
-        npad <<= 1;
-    // the largest weight a logit that was NOT emitted can have, over all slices (0 if none can be a candidate)
-    float q_bound = 0.0f;
-    {
-        uint32_t off = 0;
-        for (uint32_t s = 0; s < slices; ++s) {
-            const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
-            const size_t base = ((size_t)row * sc.slices_cap + s) * kCap;
-            for (uint32_t c = tid; c < st.n_emit; c += kThreads) {
-                const float q = weight_of(sc.cand_w[base + c], m, inv_t, sm.tab);
-                const uint32_t id = sc.cand_i[base + c];
-                unsigned long long k64 = 0;
-                if (q >= floor_q && q > 0.0f)
-                    k64 = ((unsigned long long)__float_as_uint(q) << 32) | (unsigned long long)(kNone - id);
-                L.sortk[off + c] = k64;
-            }
-            off += st.n_emit;
-            if (!(st.flags & kFlagComplete)) {
-                // everything left behind has an order key below tau_key
-                const float qb = weight_of(order_unkey(st.tau_key - 1u), m, inv_t, sm.tab);
-                if (qb >= floor_q && qb > 0.0f && qb > q_bound)
-                    q_bound = qb;
-            }
+    // where each slice's candidates start, and the largest weight a logit that was NOT emitted can have over
+    // all slices (0 if none can be a candidate): everything left behind has an order key below tau_key
+    if (tid == 0)
+        sm.flag = 0;
+    __syncthreads();
+    if (tid < slices) {
+        const SliceStat st = sc.stats[(size_t)row * kMaxSlices + tid];
+        sm.soff[tid + 1] = st.n_emit;
+        if (!(st.flags & kFlagComplete)) {
+            const float qb = weight_of(order_unkey(st.tau_key - 1u), m, inv_t, sm.tab);
+            if (qb >= floor_q && qb > 0.0f)
+                atomicMax(&sm.flag, __float_as_uint(qb)); // positive floats order like their bits
         }
-        for (uint32_t c = n_cands + tid; c < npad; c += kThreads)
-            L.sortk[c] = 0;
     }
     __syncthreads();
-    bitonic_sort_desc(L.sortk, npad);
-    uint32_t nv = 0;
-    for (uint32_t c = tid; c < npad; c += kThreads)
-        nv += L.sortk[c] != 0;
-    const uint32_t n_valid = block_sum_u32(nv, sm.bs);
-
-    auto qat = [&](uint32_t i) { return __uint_as_float((uint32_t)(L.sortk[i] >> 32)); };
-    auto idat = [&](uint32_t i) { return kNone - (uint32_t)L.sortk[i]; };
-
-    uint32_t n1;
-    double total64;
+    if (tid == 0) {
+        sm.soff[0] = 0;
+        for (uint32_t s = 0; s < slices; ++s)
+            sm.soff[s + 1] += sm.soff[s];
+    }
+    __syncthreads();
+    const float q_bound = __uint_as_float(sm.flag);
+    MAKO_STAMP(3);
+    uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax); // upper half of the dynamic block
+    uint32_t* jf = kf + kSortMax;
+    const uint32_t n_valid = n_cands <= 1024u ? sort_candidates<1>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L)
+                                              : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
+    MAKO_STAMP(4);
     if (cls == kTopK) {
         // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
-        const bool ok = n_valid >= P.top_k ? q_bound < qat(P.top_k - 1) : q_bound == 0.0f;
+        const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
         if (!ok) {
-            general_row(d, sc, row, P, m, argidx, L);
+            if (tid == 0) {
+                sc.plan[row].total64 = (double)m;
+                sc.plan[row].n0 = argidx;
+                sc.plan[row].flag = 2;
+            }
             return;
         }
         if (n_valid == 0) {
             fallback_row(d, row, argidx);
             return;
         }
-        n1 = min(P.top_k, n_valid); // sampler.cpp:40-43
-        double part = 0;
-        for (uint32_t i = tid; i < n1; i += kThreads)
-            part += (double)qat(i);
-        total64 = block_sum_f64(part, sm.bs);
-    } else {
-        total64 = row_total;
-        n1 = n_valid;
+        sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L); // sampler.cpp:40-43
+        return;
     }
-
-    // top-p over the sorted candidates (sampler.cpp:44-61)
-    const double want = (double)P.top_p * total64;
-    double carry = 0;
-    uint32_t keep = kNone;
-    for (uint32_t base = 0; base < n1; base += kThreads) {
-        const uint32_t i = base + tid;
-        const double q = i < n1 ? (double)qat(i) : 0.0;
-        double tile;
-        const double incl = carry + block_incl_scan_f64(q, tile, sm.bs);
-        const uint32_t hit = (i < n1 && incl >= want) ? i : kNone;
-        const uint32_t first = block_min_u32(hit, sm.bs);
-        if (first != kNone) {
-            keep = first + 1;
-            break;
-        }
-        carry += tile;
-    }
-    uint32_t n;
-    if (cls == kTopK) {
-        n = keep == kNone ? n1 : keep;
-    } else {
-        // the nucleus must end inside the candidates, strictly above everything left behind
-        if (keep == kNone || !(q_bound < qat(keep - 1))) {
-            nucleus_big_row(d, sc, row, P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, L);
-            return;
-        }
-        n = keep;
-    }
-    draw_from_list(d, row, qat, idat, n, cls == kTopK ? MAKO_PATH_TOPK : MAKO_PATH_NUCLEUS, sm);
+    // top_k == 0: the nucleus must end inside the candidates, strictly above everything left behind
+    if (n_valid == 0 || !sorted_tail(d, row, P, kf, jf, n_valid, true, row_total, MAKO_PATH_NUCLEUS, L, true, q_bound))
+        if (tid == 0)
+            sc.plan[row].flag = 1; // sort_kernel takes the row
 }
+
+// grid = (kWorkers, rows).  Rows without a work order cost one load.  Worker w gathers its range of weights from
+// the row's bits(q) array, sorts it and stores it at its place in the row's sorted list; the last worker to
+// finish cuts the nucleus and draws.
+__global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_arg)
+{
+    extern __shared__ unsigned long long s_dyn64[];
+    __shared__ FinishShared sm;
+    __shared__ ArgsLds s_args;
+    const uint32_t row = blockIdx.y, w = blockIdx.x, tid = threadIdx.x;
+    const uint32_t flag = sc_arg.plan[row].flag;
+    if (flag == 0 || (flag == 2 && w != 0))
+        return;
+    stage_args(d_arg, sc_arg, s_args);
+    const mako_sample_desc& d = s_args.d;
+    const Scratch& sc = s_args.sc;
+    BigPlan* plan = sc.plan + row;
+    FinishLds L;
+    L.sm = &sm;
+    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
+    L.sortk = s_dyn64;
+    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
+    if (tid < 32)
+        sm.tab[tid] = k_exp2_tab[tid];
+    if (flag == 2) {
+        // top_k > 128, no top-p, or a candidate list that could not be certified: the whole-row path
+        const float m = (float)plan->total64;
+        const uint32_t argidx = plan->n0;
+        __syncthreads();
+        if (tid == 0)
+            plan->flag = 0;
+        general_row(d, sc, row, s_args.P, m, argidx, L);
+        return;
+    }
+    const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
+    uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
+    uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
+    uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
+    uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
+    const uint32_t cnt = plan->cnt[w], off = plan->off[w];
+    const uint32_t n0 = plan->n0;
+    const double total64 = plan->total64;
+    if (cnt) {
+        gather_range(qk, d.n_vocab, plan->key_lo[w], plan->key_hi[w], key0 + off, idx0 + off, sm);
+        sort_segment(key0 + off, idx0 + off, key1 + off, idx1 + off, cnt, L);
+    }
+    __syncthreads(); // every thread's stores are acknowledged before the ticket is taken
+    if (tid == 0) {
+        __threadfence();
+        sm.ticket = atomicAdd(&plan->ticket, 1u);
+    }
+    __syncthreads();
+    if (sm.ticket != kWorkers - 1)
+        return;
+    __threadfence();
+    if (tid == 0) {
+        plan->ticket = 0;
+        plan->flag = 0;
+    }
+    sorted_tail(d, row, s_args.P, key0, idx0, n0, true, total64, MAKO_PATH_GENERAL, L);
+}
+
 
 __global__ void debug_expf_kernel(const float* x, float* y, uint32_t n)
 {
