@@ -884,6 +884,17 @@ struct GroupLds { // carved from the dynamic LDS block once sorting is over
     uint32_t* misc; // [4]
 };
 
+// Values every lane of the wave holds alike, moved to scalar registers so that loops and branches on them
+// compile to scalar control flow.
+__device__ __forceinline__ uint32_t uniform_u32(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
+}
+__device__ __forceinline__ bool uniform_bool(bool b)
+{
+    return __builtin_amdgcn_readfirstlane((int)b) != 0;
+}
+
 __device__ __forceinline__ int exponent_of(float x)
 {
     uint32_t M;
@@ -968,7 +979,7 @@ __device__ float exact_group_sum(const uint32_t* kf, uint32_t g, uint32_t n, flo
 {
     float q[4];
     load_group(kf, g, n, q); // entries past the end read as 0.0f: adding them changes nothing
-    const uint32_t cnt = min(n - g * kGroup, kGroup);
+    const uint32_t cnt = uniform_u32(min(n - g * kGroup, kGroup));
     const uint32_t lanes = (cnt + 3u) / 4u;
     for (uint32_t l = 0; l < lanes; ++l) {
 #pragma unroll
@@ -983,21 +994,26 @@ __device__ float exact_group_sum(const uint32_t* kf, uint32_t g, uint32_t n, flo
 __device__ bool exact_group_walk(const uint32_t* kf, uint32_t g, uint32_t n, float& r, uint32_t& pos)
 {
     float q[4];
-    load_group(kf, g, n, q);
-    const uint32_t beg = g * kGroup, cnt = min(n - beg, kGroup);
-    for (uint32_t l = 0; l * 4u < cnt; ++l) {
+    load_group(kf, g, n, q); // entries past the end read as 0.0f: r >= 0 never stops at them, r - 0 is r
+    const uint32_t beg = uniform_u32(g * kGroup), cnt = uniform_u32(min(n - g * kGroup, kGroup));
+    const uint32_t lanes = (cnt + 3u) / 4u;
+    const float nan = __uint_as_float(0x7fc00000u);
+    float rr = r; // NaN once the walk has stopped: no later comparison succeeds
+    uint32_t at = kNone;
+    for (uint32_t l = 0; l < lanes; ++l) {
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            if (l * 4u + j < cnt) {
-                const float x = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), l));
-                if (r < x) {
-                    pos = beg + l * 4u + j;
-                    return true;
-                }
-                r -= x;
-            }
+            const float x = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), l));
+            const bool stop = rr < x;
+            at = stop ? beg + l * 4u + j : at;
+            rr = stop ? nan : rr - x;
+        }
+        if (uniform_u32(at) != kNone) {
+            pos = uniform_u32(at);
+            return true;
         }
     }
+    r = rr;
     return false;
 }
 
@@ -1010,10 +1026,11 @@ __device__ bool exact_group_walk(const uint32_t* kf, uint32_t g, uint32_t n, flo
 // it weighs at most q_bound: the nucleus must then end inside the list, at an entry strictly heavier than
 // q_bound.  If it does not, nothing is written and false is returned (the caller widens the list).
 __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf,
-                            const uint32_t* jf, uint32_t n1, bool have_total, double total64, uint32_t path,
+                            const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
                             const FinishLds& L, bool need_cut = false, float q_bound = 0.0f)
 {
     using namespace seqfp;
+    const uint32_t n1 = uniform_u32(n1_arg);
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
     auto qat = [=](uint32_t i) { return __uint_as_float(~kf[i]); };
@@ -1059,6 +1076,78 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             return false;
         draw_from_list(d, row, qat, idat, n, path, sm);
         return true;
+    }
+
+    if (n1 <= kGroup) {
+        // short list: one wave does everything, the chain of fp32 roundings replayed with real additions
+        MAKO_STAMP(5);
+        __syncthreads(); // the list is published; sm.flag is free
+        if (wave_id() == 0) {
+            float q[4];
+            load_group(kf, 0, n1, q);
+            double p[4];
+            p[0] = (double)q[0];
+            p[1] = p[0] + (double)q[1];
+            p[2] = p[1] + (double)q[2];
+            p[3] = p[2] + (double)q[3];
+            double incl = p[3];
+            for (int o = 1; o < kWave; o <<= 1) {
+                const double t = __shfl_up(incl, o);
+                if (lane_id() >= o)
+                    incl += t;
+            }
+            if (!have_total)
+                total64 = __shfl(incl, kWave - 1);
+            uint32_t n = n1;
+            bool ok = true;
+            if (topp_active) {
+                const double want = (double)P.top_p * total64;
+                const double base = incl - p[3];
+                uint32_t hit = kNone;
+#pragma unroll
+                for (int j = 3; j >= 0; --j)
+                    if (base + p[j] >= want)
+                        hit = lane_id() * 4u + (uint32_t)j;
+                const unsigned long long bal = __ballot(hit != kNone && hit < n1);
+                if (bal)
+                    n = (uint32_t)__shfl((int)hit, __ffsll((long long)bal) - 1) + 1u;
+                else
+                    ok = !need_cut;
+            }
+            if (ok && need_cut && !(q_bound < qat(n - 1)))
+                ok = false;
+            if (ok) {
+                const float total = exact_group_sum(kf, 0, n, 0.0f);
+                const float span = total - 0.0f;
+                const float prod = d.u[row] * span;
+                float r = prod + 0.0f;
+                uint32_t pos = n - 1;
+                if (r < 0.0f)
+                    pos = 0;
+                else if (r == r && r != INFINITY)
+                    exact_group_walk(kf, 0, n, r, pos);
+                if (d.out_cand_idx && d.out_cand_q)
+                    for (uint32_t j = lane_id(); j < n && j < d.cand_cap; j += kWave) {
+                        d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
+                        d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
+                    }
+                if (lane_id() == 0) {
+                    RowOut o;
+                    o.token = (int32_t)idat(pos);
+                    o.n_cand = n;
+                    o.total = total;
+                    o.q = qat(pos);
+                    o.path = path;
+                    o.accepted = 0;
+                    write_row(d, row, o);
+                }
+            }
+            if (lane_id() == 0)
+                sm.flag = ok;
+        }
+        __syncthreads();
+        MAKO_STAMP(9);
+        return sm.flag != 0;
     }
 
     // fp64 group sums and their prefix
@@ -1131,7 +1220,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     G.misc[0] = keep;
             }
             __syncthreads();
-            n = G.misc[0];
+            n = uniform_u32(G.misc[0]);
         }
     }
     if (n < 1)
@@ -1144,31 +1233,40 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     MAKO_STAMP(7);
     build_group_maps(kf, n, false, 0.0, G);
     __syncthreads();
+    MAKO_STAMP(13);
     const uint32_t groups = (n + kGroup - 1) / kGroup;
     if (wave_id() == 0) {
-        // 64 groups at a time: lane l fetches group base + l's guess and map, the chain reads them by lane index
-        float S = 0.0f;
+        // 64 groups at a time: lane l fetches group base + l's guess and map; the chain reads them by lane index
+        // and keeps its state (significand M, exponent e) in scalar registers
+        uint32_t M = 0;
+        int e = 1; // 0.0f
         for (uint32_t base = 0; base < groups; base += kWave) {
             const uint32_t gl = min(base + lane_id(), groups - 1u);
             const int eg_l = G.pg[gl] > 0 ? exponent_of((float)G.pg[gl]) : 0;
             const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], cm_l = G.cmax[gl];
+            // group_add_ok: M + d + cmax + 1 < 2^24
+            const uint32_t lim_l = cm_l >= (1u << 24) - 1u ? 0u : (1u << 24) - 1u - cm_l;
             const uint32_t cnt = min((uint32_t)kWave, groups - base);
             for (uint32_t k = 0; k < cnt; ++k) {
-                uint32_t M;
-                int e;
-                split(S, M, e);
                 const int eg = __builtin_amdgcn_readlane(eg_l, k);
-                const Step32 st = Step32{(uint32_t)__builtin_amdgcn_readlane((int)d0_l, k),
-                                         (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k),
-                                         (uint32_t)__builtin_amdgcn_readlane((int)cm_l, k)};
-                if (e == eg && group_add_ok((long long)M, st))
-                    S = join(M + ((M & 1u) ? st.d1 : st.d0), e);
-                else
-                    S = exact_group_sum(kf, base + k, n, S);
+                const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, k);
+                const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k);
+                const uint32_t lim = (uint32_t)__builtin_amdgcn_readlane((int)lim_l, k);
+                const uint32_t dd = (M & 1u) ? d1 : d0;
+                if (e == eg && M + dd < lim) {
+                    M += dd;
+                } else {
+                    const float S = exact_group_sum(kf, base + k, n, join(M, e));
+                    uint32_t Mv;
+                    int ev;
+                    split(S, Mv, ev);
+                    M = uniform_u32(Mv);
+                    e = (int)uniform_u32((uint32_t)ev);
+                }
             }
         }
         if (lane_id() == 0)
-            G.misc[1] = __float_as_uint(S);
+            G.misc[1] = __float_as_uint(join(M, e));
     }
     __syncthreads();
     MAKO_STAMP(8);
@@ -1185,8 +1283,17 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     } else if (r0 == r0 && r0 != INFINITY) {
         build_group_maps(kf, n, true, (double)r0, G);
         __syncthreads();
+        MAKO_STAMP(14);
         if (wave_id() == 0) {
-            float r = r0;
+            uint32_t M;
+            int e;
+            {
+                uint32_t Mv;
+                int ev;
+                split(r0, Mv, ev);
+                M = uniform_u32(Mv);
+                e = (int)uniform_u32((uint32_t)ev);
+            }
             uint32_t at = n - 1;
             bool stopped = false;
             for (uint32_t base = 0; base < groups && !stopped; base += kWave) {
@@ -1194,22 +1301,41 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 const double guess_l = (double)r0 - G.pg[gl];
                 const int eg_l = guess_l > 0 ? exponent_of((float)guess_l) : 0;
                 const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], cm_l = G.cmax[gl];
-                const float qf_l = qat(gl * kGroup);
+                // group_sub_ok as one bound: the state after the group must be at least need_l, which keeps it
+                // inside the binade with room for one more decrement and at or above the group's first weight
+                uint32_t need_l = 1u;
+                {
+                    uint32_t Mq;
+                    int eq;
+                    split(qat(gl * kGroup), Mq, eq);
+                    const int dl = eg_l - eq;
+                    if (dl < 0)
+                        need_l = 1u << 31;
+                    else if (dl <= 25)
+                        need_l = max(1u, (uint32_t)(((unsigned long long)Mq + (1ull << dl) - 1ull) >> dl));
+                    if (eg_l > 1)
+                        need_l = max(need_l, min(cm_l, 1u << 30) + (1u << 23) + 1u);
+                }
                 const uint32_t cnt = min((uint32_t)kWave, groups - base);
                 for (uint32_t k = 0; k < cnt; ++k) {
-                    uint32_t M;
-                    int e;
-                    split(r, M, e);
                     const int eg = __builtin_amdgcn_readlane(eg_l, k);
-                    const Step32 st = Step32{(uint32_t)__builtin_amdgcn_readlane((int)d0_l, k),
-                                             (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k),
-                                             (uint32_t)__builtin_amdgcn_readlane((int)cm_l, k)};
-                    const float q_first = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(qf_l), k));
-                    if (e == eg && group_sub_ok((long long)M, e, st, q_first)) {
-                        r = join(M - ((M & 1u) ? st.d1 : st.d0), e);
-                    } else if (exact_group_walk(kf, base + k, n, r, at)) {
-                        stopped = true;
-                        break;
+                    const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, k);
+                    const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k);
+                    const uint32_t need = (uint32_t)__builtin_amdgcn_readlane((int)need_l, k);
+                    const uint32_t dd = (M & 1u) ? d1 : d0;
+                    if (e == eg && M >= dd + need) {
+                        M -= dd;
+                    } else {
+                        float r = join(M, e);
+                        if (exact_group_walk(kf, base + k, n, r, at)) {
+                            stopped = true;
+                            break;
+                        }
+                        uint32_t Mv;
+                        int ev;
+                        split(r, Mv, ev);
+                        M = uniform_u32(Mv);
+                        e = (int)uniform_u32((uint32_t)ev);
                     }
                 }
             }
@@ -1279,7 +1405,8 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
 // Thread t brings the counts (c0, c1) and significand sums (s0, s1) of bins kBins-1-2t and kBins-2-2t.
 // Returns n0, the number of weights to sort; the plan is written to `plan` (flag left untouched).
 __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, uint32_t c0, uint32_t c1,
-                                 unsigned long long s0, unsigned long long s1, BigPlan* plan, const FinishLds& L)
+                                 unsigned long long s0, unsigned long long s1, BigPlan* plan, const FinishLds& L,
+                                 uint32_t& thr_bits)
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
@@ -1306,6 +1433,7 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         hit = b1;
     const uint32_t rev = block_min_u32(hit == kNone ? kNone : kBins - 1u - hit, sm.bs);
     const uint32_t b_lo = rev == kNone ? 0u : kBins - 1u - rev; // not reached twice: keep every candidate
+    thr_bits = b_lo << 19;
 
     // candidates above each bin, and the workers' shares
     uint32_t count_all;
@@ -1628,6 +1756,120 @@ __device__ uint32_t sort_candidates(const Scratch& sc, uint32_t row, uint32_t sl
     return block_sum_u32(nv, sm.bs); // (its barriers publish kf / jf)
 }
 
+constexpr uint32_t kSmall = 256; // lists of up to this many entries are ordered by counting ranks
+
+// Fast route for rows that need only a few of their candidates.  Every thread weights up to four candidates;
+// those at or above a weight threshold (at most kSmall of them) are ordered by (q desc, idx asc) by counting, for
+// each, the entries that precede it, and left in LDS as kf[i] = ~bits(q_i), jf[i] = token id.
+//   top_k > 0:  the threshold is the lower edge of the quarter-binade bin that holds the top_k-th largest weight
+//               (one histogram over bits(q) >> 21), so the list is a superset of the row's top_k candidates.
+//   top_k == 0: the threshold is thr_bits, below which the nucleus cannot reach (from the row's histogram).
+// Returns the number of entries in the list, or kNone when they exceed kSmall (nothing is written then);
+// n_valid receives the number of candidates that have a weight at all.
+__device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_cands, float m, float inv_t,
+                                     float floor_q, uint32_t top_k, uint32_t thr_bits, uint32_t* kf, uint32_t* jf,
+                                     uint32_t& n_valid, const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    uint32_t* hist = reinterpret_cast<uint32_t*>(L.sortk);             // [512]
+    unsigned long long* sel = L.sortk + 256;                           // [kSmall]
+    uint32_t* rank = reinterpret_cast<uint32_t*>(L.sortk + 256 + kSmall); // [kSmall]
+    uint32_t* counter = rank + kSmall;
+    unsigned long long key[4];
+#pragma unroll
+    for (uint32_t t = 0; t < 4; ++t) {
+        const uint32_t c = t * 1024u + tid;
+        key[t] = 0;
+        if (c < n_cands) {
+            uint32_t s = 0;
+            while (s + 1 < slices && c >= sm.soff[s + 1]) // slice holding candidate c
+                ++s;
+            const size_t at = ((size_t)row * sc.slices_cap + s) * kCap + (c - sm.soff[s]);
+            const float q = weight_of(sc.cand_w[at], m, inv_t, sm.tab);
+            if (q >= floor_q && q > 0.0f)
+                key[t] = ((unsigned long long)__float_as_uint(q) << 32) | (unsigned long long)(kNone - sc.cand_i[at]);
+        }
+    }
+    if (tid < 512)
+        hist[tid] = 0;
+    if (tid < kSmall)
+        rank[tid] = 0;
+    if (tid == 0)
+        *counter = 0;
+    __syncthreads();
+    uint32_t n_list;
+    if (top_k > 0) {
+#pragma unroll
+        for (uint32_t t = 0; t < 4; ++t)
+            if (key[t])
+                atomicAdd(&hist[min((uint32_t)(key[t] >> 53), 511u)], 1u);
+        if (tid == 0) {
+            sm.flag = 0;
+            sm.ticket = 0;
+        }
+        __syncthreads();
+        const uint32_t c = tid < 512 ? hist[511u - tid] : 0u;
+        uint32_t total;
+        const uint32_t above = block_excl_scan_u32(c, total, sm.bs);
+        if (tid < 512 && above < top_k && top_k <= above + c) {
+            sm.flag = (511u - tid) << 21;
+            sm.ticket = above + c;
+        }
+        __syncthreads();
+        n_valid = total;
+        thr_bits = sm.flag;                              // 0 when the row has fewer than top_k candidates
+        n_list = total < top_k ? total : sm.ticket;
+        __syncthreads();
+    } else {
+        uint32_t mine = 0, ge = 0;
+#pragma unroll
+        for (uint32_t t = 0; t < 4; ++t) {
+            mine += key[t] != 0;
+            ge += key[t] != 0 && (uint32_t)(key[t] >> 32) >= thr_bits;
+        }
+        const uint32_t both = block_sum_u32((mine << 16) | ge, sm.bs); // each below 65536
+        n_valid = both >> 16;
+        n_list = both & 0xffffu;
+    }
+    if (n_list > kSmall)
+        return kNone;
+    // compaction in any order: the keys are distinct, the ranks below put them in place
+    const unsigned long long lower = (1ull << lane_id()) - 1ull;
+#pragma unroll
+    for (uint32_t t = 0; t < 4; ++t) {
+        const bool keep = key[t] != 0 && (uint32_t)(key[t] >> 32) >= thr_bits;
+        const unsigned long long bal = __ballot(keep);
+        if (bal) {
+            uint32_t base = 0;
+            if (lane_id() == (uint32_t)__ffsll((long long)bal) - 1u)
+                base = atomicAdd(counter, (uint32_t)__popcll(bal));
+            base = (uint32_t)__shfl((int)base, __ffsll((long long)bal) - 1);
+            if (keep)
+                sel[base + (uint32_t)__popcll(bal & lower)] = key[t];
+        }
+    }
+    __syncthreads();
+    {
+        const uint32_t e = tid & (kSmall - 1u), part = tid / kSmall; // four threads share the comparisons of an entry
+        const unsigned long long my = e < n_list ? sel[e] : ~0ull;
+        const uint32_t jb = min(n_list, part * (kSmall / 4u)), je = min(n_list, jb + kSmall / 4u);
+        uint32_t r = 0;
+        for (uint32_t j = jb; j < je; ++j)
+            r += sel[j] > my;
+        if (r)
+            atomicAdd(&rank[e], r);
+        __syncthreads();
+        if (tid < n_list) {
+            const uint32_t at = rank[tid];
+            kf[at] = ~(uint32_t)(my >> 32);
+            jf[at] = kNone - (uint32_t)my;
+        }
+    }
+    __syncthreads();
+    return n_list;
+}
+
 // Exact fp64 sum of q over one slice, and the number of candidates in it (q > 0 and q >= min_p).
 // The summation order is fixed: each thread adds its logits in index order, then lanes, then waves.
 template <bool VEC, int KH>
@@ -1855,8 +2097,9 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     }
     // a top_k == 0 row is planned from its histogram first: only a narrow nucleus can end inside the candidates
     bool try_candidates = true;
+    uint32_t thr_bits = 0;
     if (cls == kNucleus) {
-        const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, L);
+        const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, L, thr_bits);
         try_candidates = n0 <= 1024u && !any_overflow && n_cands <= kSortMax;
         if (!try_candidates) {
             if (tid == 0)
@@ -1900,6 +2143,32 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     MAKO_STAMP(3);
     uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax); // upper half of the dynamic block
     uint32_t* jf = kf + kSortMax;
+    if (!d.draft) {
+        // short lists: the top_k-th weight's neighbourhood, or the part of the candidates the nucleus can reach
+        uint32_t n_valid = 0;
+        const uint32_t n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, cls == kTopK ? P.top_k : 0u,
+                                                 thr_bits, kf, jf, n_valid, L);
+        MAKO_STAMP(4);
+        if (n_list != kNone) {
+            if (cls == kTopK) {
+                const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
+                if (ok && n_valid == 0) {
+                    fallback_row(d, row, argidx);
+                } else if (ok) {
+                    sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L);
+                } else if (tid == 0) {
+                    sc.plan[row].total64 = (double)m;
+                    sc.plan[row].n0 = argidx;
+                    sc.plan[row].flag = 2;
+                }
+                return;
+            }
+            if (n_list == 0 || !sorted_tail(d, row, P, kf, jf, n_list, true, row_total, MAKO_PATH_NUCLEUS, L, true, q_bound))
+                if (tid == 0)
+                    sc.plan[row].flag = 1;
+            return;
+        }
+    }
     const uint32_t n_valid = n_cands <= 1024u ? sort_candidates<1>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L)
                                               : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
     MAKO_STAMP(4);
