@@ -109,6 +109,14 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.idx[0], rv));
     MAKO_HIP(ctx, dev_alloc(&sc.idx[1], rv));
     MAKO_HIP(ctx, hipMemset(sc.cnt, 0, rv * sizeof(uint32_t)));
+    sc.g_cap = (uint32_t)(sc.vpad / mako::kGroup) + mako::kWorkers;
+    const size_t rg = (size_t)max_rows * sc.g_cap;
+    MAKO_HIP(ctx, dev_alloc(&sc.gt.sum, rg));
+    MAKO_HIP(ctx, dev_alloc(&sc.gt.d0, rg));
+    MAKO_HIP(ctx, dev_alloc(&sc.gt.d1, rg));
+    MAKO_HIP(ctx, dev_alloc(&sc.gt.cmax, rg));
+    MAKO_HIP(ctx, dev_alloc(&sc.gt.start, rg));
+    MAKO_HIP(ctx, dev_alloc(&sc.gt.pack, rg));
     MAKO_HIP(ctx, hipDeviceSynchronize());
     // both kernels overlay up to 64 KB of dynamic LDS on a few KB of static LDS
     const void* kernels[] = {(const void*)mako::scan_kernel<true, 0>,    (const void*)mako::scan_kernel<false, 0>,
@@ -118,8 +126,10 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
                              (const void*)mako::finish_kernel<true, 2>,  (const void*)mako::finish_kernel<false, 2>,
                              (const void*)mako::finish_kernel<true, 8>,  (const void*)mako::finish_kernel<false, 8>,
                              (const void*)mako::sort_kernel};
+    static_assert(mako::kSortLds >= mako::kDynLds, "sort_kernel's tail uses the finishing kernel's LDS layout");
     for (const void* k : kernels)
-        MAKO_HIP(ctx, hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)mako::kDynLds));
+        MAKO_HIP(ctx, hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          k == (const void*)mako::sort_kernel ? (int)mako::kSortLds : (int)mako::kDynLds));
     return MAKO_OK;
 }
 
@@ -129,7 +139,8 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.tickets, sc.binc, sc.bins, sc.plan,
+    void* ptrs[] = {sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack,
+                    sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.tickets, sc.binc, sc.bins, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
                     ctx->st_hist,  ctx->st_hcnt, ctx->st_hlen,  ctx->st_draft, ctx->st_tokens, ctx->st_acc};
@@ -179,7 +190,7 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
 #define MAKO_LAUNCH(V, K)                                                                                          \
     do {                                                                                                           \
         hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc, slice_len); \
-        hipLaunchKernelGGL((mako::finish_kernel<V, K>), grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc, \
+        hipLaunchKernelGGL((mako::finish_kernel<V, K>), dim3(d.n_rows, slices), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc, \
                            slices, slice_len);                                                                     \
     } while (0)
     if (vec && kh == 2)
@@ -196,7 +207,7 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
         MAKO_LAUNCH(false, 0);
 #undef MAKO_LAUNCH
     // rows whose nucleus is too wide for the candidate lists left a work order; the others cost one load each
-    hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc);
+    hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d, ctx->sc);
     MAKO_HIP(ctx, hipGetLastError());
     return MAKO_OK;
 }

@@ -31,7 +31,7 @@ constexpr uint32_t kNone = 0xffffffffu;
 __device__ unsigned long long g_mako_stamp[32];
 #define MAKO_STAMP(i)                                                                                                \
     do {                                                                                                             \
-        if (threadIdx.x == 0 && blockIdx.y == 0)                                                                     \
+        if (threadIdx.x == 0 && (gridDim.x == kWorkers ? blockIdx.y == 0 : blockIdx.x == 0))                         \
             g_mako_stamp[i] = wall_clock64();                                                                        \
     } while (0)
 #else
@@ -59,7 +59,12 @@ struct SliceStat {
     uint32_t pad[3];
 };
 
-constexpr uint32_t kWorkers = 16; // workgroups that share the sort of one wide-nucleus row
+constexpr uint32_t kWorkers = 32;  // workgroups that share the sort of one wide-nucleus row
+constexpr uint32_t kGroup = 256;      // a sorted list is processed in groups of one wave x four entries per lane
+constexpr uint32_t kMaxGroups = 1024; // groups per list
+constexpr uint32_t kSegCap = 6144;    // entries a worker sorts in LDS
+constexpr uint32_t kFine = 2048;      // value buckets of that sort
+constexpr uint32_t kSortLds = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u; // dynamic LDS of sort_kernel
 
 // Work order for a top_k == 0 row whose nucleus is too wide for the per-slice candidate lists: the weights
 // with bits(q) >= key_lo (n0 of them) are split by value into kWorkers contiguous ranges of about equal size.
@@ -67,12 +72,24 @@ struct BigPlan {
     uint32_t flag;   // 1: the row waits for sort_kernel's workers; 2: for its whole-row path (worker 0 alone)
     uint32_t n0;     // entries to sort
     uint32_t ticket; // workers that have finished
-    uint32_t pad;
+    uint32_t groups; // groups of the whole list: each worker's range is cut into groups of kGroup on its own
     double total64;  // exact fp64 sum of q over the row's candidates
     uint32_t key_lo[kWorkers]; // worker w takes bits(q) in [key_lo[w], key_hi[w])
     uint32_t key_hi[kWorkers];
     uint32_t off[kWorkers];    // and writes them from position off[w] of the sorted list
     uint32_t cnt[kWorkers];
+    uint32_t gbase[kWorkers];  // first group of worker w
+    double mass[kWorkers];     // sum of the weights above worker w's range
+};
+
+// Per-group records of a planned row's sorted list, written by the workers and read by the last of them.
+struct GroupTable {
+    double* sum;     // fp64 sum of the group's weights
+    uint32_t* d0;    // the group's map for the running fp32 sum in the epoch guessed from the mass before it
+    uint32_t* d1;
+    uint32_t* cmax;
+    uint32_t* start; // first entry of the group in the sorted list
+    uint32_t* pack;  // entries | guessed exponent << 16
 };
 
 struct Scratch {
@@ -91,8 +108,10 @@ struct Scratch {
     uint32_t* cnt;     // [max_rows][vpad] token counts; all zero between calls
     uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong
     uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, ping-pong
+    GroupTable gt;     // [max_rows][g_cap] each
     uint64_t vpad;
     uint32_t slices_cap;
+    uint32_t g_cap;    // vpad / kGroup + kWorkers
 };
 
 // Total order on floats as unsigned keys: -inf < ... < -0 = +0 < ... < +inf.  Never called on NaN.
@@ -873,26 +892,35 @@ __device__ void draw_from_list(const mako_sample_desc& d, uint32_t row, QAt qat,
 // sorted lists: top-p cut, exact fp32 total and walk, in groups of 256 (see seqfp.h, "groups")
 // ---------------------------------------------------------------------------------------------
 
-constexpr uint32_t kGroup = 256;      // one wave, four consecutive entries per lane
-constexpr uint32_t kMaxGroups = 1024; // lists of up to 262144 entries
-
-struct GroupLds { // carved from the dynamic LDS block once sorting is over
-    double* pg;     // [kMaxGroups + 1] fp64 sum of the entries before each group
-    uint32_t* d0;   // [kMaxGroups] the group's map for the guessed epoch
+struct GroupLds { // carved from the lower half of the dynamic LDS block once sorting is over
+    double* pg;      // [kMaxGroups + 2] fp64 sum of the entries before each group
+    uint32_t* d0;    // [kMaxGroups] the group's map for the guessed epoch
     uint32_t* d1;
     uint32_t* cmax;
-    uint32_t* misc; // [4]
+    uint32_t* start; // first entry of the group
+    uint32_t* pack;  // entries | guessed exponent << 16
+    uint32_t* misc;  // [4]
 };
+
+__device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
+{
+    GroupLds G;
+    G.pg = reinterpret_cast<double*>(L.sortk);
+    G.d0 = reinterpret_cast<uint32_t*>(G.pg + kMaxGroups + 2);
+    G.d1 = G.d0 + kMaxGroups;
+    G.cmax = G.d1 + kMaxGroups;
+    G.start = G.cmax + kMaxGroups;
+    G.pack = G.start + kMaxGroups;
+    G.misc = G.pack + kMaxGroups;
+    static_assert((kMaxGroups + 2) * 8 + 5 * kMaxGroups * 4 + 16 <= kSortMax * 8, "group records fit below the LDS lists");
+    return G;
+}
 
 // Values every lane of the wave holds alike, moved to scalar registers so that loops and branches on them
 // compile to scalar control flow.
 __device__ __forceinline__ uint32_t uniform_u32(uint32_t v)
 {
     return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
-}
-__device__ __forceinline__ bool uniform_bool(bool b)
-{
-    return __builtin_amdgcn_readfirstlane((int)b) != 0;
 }
 
 __device__ __forceinline__ int exponent_of(float x)
@@ -903,13 +931,14 @@ __device__ __forceinline__ int exponent_of(float x)
     return e;
 }
 
-// The four weights a lane owns in group g of a list of `len` entries (0 past the end).
-__device__ __forceinline__ void load_group(const uint32_t* kf, uint32_t g, uint32_t len, float (&q)[4])
+// The four weights a lane owns in the span of `len` (<= kGroup) entries that starts at kf[start]: entries
+// 4 * lane .. 4 * lane + 3, 0.0f past the end.  kf itself is 16-byte aligned.
+__device__ __forceinline__ void load_span(const uint32_t* kf, uint32_t start, uint32_t len, float (&q)[4])
 {
-    const uint32_t i = g * kGroup + lane_id() * 4u;
+    const uint32_t i = lane_id() * 4u;
     uint32_t k[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu}; // ~bits(0.0f)
-    if (i + 3 < len) {
-        const uint4 x = *reinterpret_cast<const uint4*>(kf + i);
+    if ((start & 3u) == 0 && i + 3 < len) {
+        const uint4 x = *reinterpret_cast<const uint4*>(kf + start + i);
         k[0] = x.x;
         k[1] = x.y;
         k[2] = x.z;
@@ -918,69 +947,81 @@ __device__ __forceinline__ void load_group(const uint32_t* kf, uint32_t g, uint3
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
             if (i + j < len)
-                k[j] = kf[i + j];
+                k[j] = kf[start + i + j];
     }
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j)
         q[j] = __uint_as_float(~k[j]);
 }
 
-__device__ __forceinline__ seqfp::Step32 wave_incl_scan_step32(seqfp::Step32 v)
+// Composition of the 64 lanes' maps in lane order; every lane receives the result.
+__device__ __forceinline__ seqfp::Step32 wave_compose_step32(seqfp::Step32 v)
 {
     for (int o = 1; o < kWave; o <<= 1) {
         seqfp::Step32 t;
-        t.d0 = __shfl_up(v.d0, o);
-        t.d1 = __shfl_up(v.d1, o);
-        t.cmax = __shfl_up(v.cmax, o);
-        if (lane_id() >= o)
-            v = seqfp::compose32(t, v);
+        t.d0 = __shfl_xor(v.d0, o);
+        t.d1 = __shfl_xor(v.d1, o);
+        t.cmax = __shfl_xor(v.cmax, o);
+        // the lane whose bit o is clear holds the earlier run
+        v = (lane_id() & o) ? seqfp::compose32(t, v) : seqfp::compose32(v, t);
     }
     return v;
 }
 
-// Group maps of entries [0, n) for epochs guessed from pg: sum (walk == false) or walk from r0.
-__device__ void build_group_maps(const uint32_t* kf, uint32_t n, bool walk, double r0, const GroupLds& G)
+// The map of one span for the epoch with exponent eg (eg == 0: no usable guess, the map is marked unusable).
+__device__ __forceinline__ seqfp::Step32 span_map(const float (&q)[4], uint32_t len, int eg)
 {
     using namespace seqfp;
-    const uint32_t groups = (n + kGroup - 1) / kGroup;
+    Step32 st = Step32{kSat, kSat, kSat};
+    if (eg > 0) { // uniform per wave
+        st = identity32();
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (lane_id() * 4u + j < len)
+                st = compose32(st, step32(q[j], eg));
+        st = wave_compose_step32(st);
+    }
+    return st;
+}
+
+// Group maps of groups [0, groups) for epochs guessed from pg: sum (walk == false) or walk from r0.
+__device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk, double r0, const GroupLds& G)
+{
+    using namespace seqfp;
     // four groups per trip and wave, their loads issued together
     for (uint32_t g0 = wave_id() * 4u; g0 < groups; g0 += kWaves * 4u) {
         float q[4][4];
+        uint32_t len[4];
 #pragma unroll
-        for (uint32_t u = 0; u < 4; ++u)
-            load_group(kf, min(g0 + u, groups - 1u), n, q[u]);
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t g = min(g0 + u, groups - 1u);
+            len[u] = uniform_u32(G.pack[g] & 0xffffu);
+            load_span(kf, uniform_u32(G.start[g]), len[u], q[u]);
+        }
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
             const uint32_t g = g0 + u;
             const double guess = g < groups ? (walk ? r0 - G.pg[g] : G.pg[g]) : 0.0;
             const int eg = guess > 0 ? exponent_of((float)guess) : 0;
-            Step32 st = Step32{kSat, kSat, kSat};
-            if (eg > 0) { // uniform per wave
-                st = identity32();
-#pragma unroll
-                for (uint32_t j = 0; j < 4; ++j)
-                    if (g * kGroup + lane_id() * 4u + j < n)
-                        st = compose32(st, step32(q[u][j], eg));
-                st = wave_incl_scan_step32(st);
-            }
-            if (lane_id() == kWave - 1 && g < groups) {
+            const Step32 st = span_map(q[u], len[u], eg);
+            if (lane_id() == 0 && g < groups) {
                 G.d0[g] = st.d0;
                 G.d1[g] = st.d1;
                 G.cmax[g] = st.cmax;
+                G.pack[g] = len[u] | ((uint32_t)eg << 16);
             }
         }
     }
 }
 
-// The entries of one group added to S one by one with real fp32 additions.  Each lane fetches its four
+// The entries of one span added to S one by one with real fp32 additions.  Each lane fetches its four
 // entries once; the wave then replays them in list order, reading them back by lane index, so the chain is
-// 256 dependent adds on uniform values and nothing else.
-__device__ float exact_group_sum(const uint32_t* kf, uint32_t g, uint32_t n, float S)
+// `len` dependent adds on uniform values and nothing else.
+__device__ float exact_span_sum(const uint32_t* kf, uint32_t start, uint32_t len, float S)
 {
     float q[4];
-    load_group(kf, g, n, q); // entries past the end read as 0.0f: adding them changes nothing
-    const uint32_t cnt = uniform_u32(min(n - g * kGroup, kGroup));
-    const uint32_t lanes = (cnt + 3u) / 4u;
+    load_span(kf, start, len, q); // entries past the end read as 0.0f: adding them changes nothing
+    const uint32_t lanes = (uniform_u32(len) + 3u) / 4u;
     for (uint32_t l = 0; l < lanes; ++l) {
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
@@ -989,14 +1030,14 @@ __device__ float exact_group_sum(const uint32_t* kf, uint32_t g, uint32_t n, flo
     return S;
 }
 
-// The entries of one group subtracted from r one by one (src/gen/sampler.cpp:67-71).  Returns true and the
-// entry's position when the walk stops inside the group, else false and the new r.
-__device__ bool exact_group_walk(const uint32_t* kf, uint32_t g, uint32_t n, float& r, uint32_t& pos)
+// The entries of one span subtracted from r one by one (src/gen/sampler.cpp:67-71).  Returns true and the
+// entry's position in the list when the walk stops inside the span, else false and the new r.
+__device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len, float& r, uint32_t& pos)
 {
     float q[4];
-    load_group(kf, g, n, q); // entries past the end read as 0.0f: r >= 0 never stops at them, r - 0 is r
-    const uint32_t beg = uniform_u32(g * kGroup), cnt = uniform_u32(min(n - g * kGroup, kGroup));
-    const uint32_t lanes = (cnt + 3u) / 4u;
+    load_span(kf, start, len, q); // entries past the end read as 0.0f: r >= 0 never stops at them, r - 0 is r
+    const uint32_t beg = uniform_u32(start);
+    const uint32_t lanes = (uniform_u32(len) + 3u) / 4u;
     const float nan = __uint_as_float(0x7fc00000u);
     float rr = r; // NaN once the walk has stopped: no later comparison succeeds
     uint32_t at = kNone;
@@ -1017,17 +1058,21 @@ __device__ bool exact_group_walk(const uint32_t* kf, uint32_t g, uint32_t n, flo
     return false;
 }
 
-// Tail of every path that ends with a list sorted by (q desc, idx asc) in global memory: kf[i] = ~bits(q_i),
-// jf[i] = token id, n1 entries (already cut to top_k).  Applies top-p (src/gen/sampler.cpp:44-61) against
-// total64 (the fp64 sum over the row's candidates; summed from the list when !have_total), then the exact
-// fp32 total (:80-82) and walk (:64-73).  All 1024 threads must call it.
+// Tail of every path that ends with a list sorted by (q desc, idx asc): kf[i] = ~bits(q_i), jf[i] = token id,
+// n1 entries (already cut to top_k).  Applies top-p (src/gen/sampler.cpp:44-61) against total64 (the fp64 sum over
+// the row's candidates; summed from the list when !have_total), then the exact fp32 total (:80-82) and walk
+// (:64-73).  All 1024 threads must call it.
 //
 // When `need_cut` the list is only the heaviest part of the row's candidates and every candidate missing from
 // it weighs at most q_bound: the nucleus must then end inside the list, at an entry strictly heavier than
 // q_bound.  If it does not, nothing is written and false is returned (the caller widens the list).
+//
+// `T` (with `t_groups` records at `t_base`) describes a list whose groups were prepared by sort_kernel's workers;
+// without it the list is cut into groups of kGroup here.
 __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf,
                             const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
-                            const FinishLds& L, bool need_cut = false, float q_bound = 0.0f)
+                            const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, const GroupTable* T = nullptr,
+                            size_t t_base = 0, uint32_t t_groups = 0)
 {
     using namespace seqfp;
     const uint32_t n1 = uniform_u32(n1_arg);
@@ -1035,14 +1080,9 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     const uint32_t tid = threadIdx.x;
     auto qat = [=](uint32_t i) { return __uint_as_float(~kf[i]); };
     auto idat = [=](uint32_t i) { return jf[i]; };
-    GroupLds G;
-    G.pg = reinterpret_cast<double*>(L.sortk);
-    G.d0 = reinterpret_cast<uint32_t*>(G.pg + kMaxGroups + 2);
-    G.d1 = G.d0 + kMaxGroups;
-    G.cmax = G.d1 + kMaxGroups;
-    G.misc = G.cmax + kMaxGroups;
+    const GroupLds G = group_lds(L);
     const bool topp_active = P.top_p < 1.0f;
-    if (d.draft || n1 > kGroup * kMaxGroups) {
+    if (d.draft || (!T && n1 > kGroup * kMaxGroups)) {
         // verification and oversized lists take the generic windowed replay
         uint32_t n = n1;
         if (topp_active) {
@@ -1078,13 +1118,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         return true;
     }
 
-    if (n1 <= kGroup) {
+    if (!T && n1 <= kGroup) {
         // short list: one wave does everything, the chain of fp32 roundings replayed with real additions
         MAKO_STAMP(5);
         __syncthreads(); // the list is published; sm.flag is free
         if (wave_id() == 0) {
             float q[4];
-            load_group(kf, 0, n1, q);
+            load_span(kf, 0, n1, q);
             double p[4];
             p[0] = (double)q[0];
             p[1] = p[0] + (double)q[1];
@@ -1117,7 +1157,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             if (ok && need_cut && !(q_bound < qat(n - 1)))
                 ok = false;
             if (ok) {
-                const float total = exact_group_sum(kf, 0, n, 0.0f);
+                const float total = exact_span_sum(kf, 0, n, 0.0f);
                 const float span = total - 0.0f;
                 const float prod = d.u[row] * span;
                 float r = prod + 0.0f;
@@ -1125,7 +1165,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 if (r < 0.0f)
                     pos = 0;
                 else if (r == r && r != INFINITY)
-                    exact_group_walk(kf, 0, n, r, pos);
+                    exact_span_walk(kf, 0, n, r, pos);
                 if (d.out_cand_idx && d.out_cand_q)
                     for (uint32_t j = lane_id(); j < n && j < d.cand_cap; j += kWave) {
                         d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
@@ -1150,22 +1190,39 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         return sm.flag != 0;
     }
 
-    // fp64 group sums and their prefix
+    // group records: fp64 sums (and, from the workers, the maps of the running sum)
     MAKO_STAMP(5);
-    const uint32_t groups1 = (n1 + kGroup - 1) / kGroup;
+    const uint32_t groups1 = T ? t_groups : (n1 + kGroup - 1) / kGroup;
     __syncthreads();
-    for (uint32_t g0 = wave_id() * 4u; g0 < groups1; g0 += kWaves * 4u) {
-        float q[4][4];
+    if (T) {
+        if (tid < groups1) {
+            G.pg[tid + 1] = T->sum[t_base + tid];
+            G.d0[tid] = T->d0[t_base + tid];
+            G.d1[tid] = T->d1[t_base + tid];
+            G.cmax[tid] = T->cmax[t_base + tid];
+            G.start[tid] = T->start[t_base + tid];
+            G.pack[tid] = T->pack[t_base + tid];
+        }
+    } else {
+        if (tid < groups1) {
+            G.start[tid] = tid * kGroup;
+            G.pack[tid] = min(kGroup, n1 - tid * kGroup);
+        }
+        for (uint32_t g0 = wave_id() * 4u; g0 < groups1; g0 += kWaves * 4u) {
+            float q[4][4];
 #pragma unroll
-        for (uint32_t u = 0; u < 4; ++u)
-            load_group(kf, min(g0 + u, groups1 - 1u), n1, q[u]);
+            for (uint32_t u = 0; u < 4; ++u) {
+                const uint32_t g = min(g0 + u, groups1 - 1u);
+                load_span(kf, g * kGroup, min(kGroup, n1 - g * kGroup), q[u]);
+            }
 #pragma unroll
-        for (uint32_t u = 0; u < 4; ++u) {
-            double s = (((double)q[u][0] + (double)q[u][1]) + (double)q[u][2]) + (double)q[u][3];
-            for (int o = 32; o > 0; o >>= 1)
-                s += __shfl_xor(s, o);
-            if (lane_id() == 0 && g0 + u < groups1)
-                G.pg[g0 + u + 1] = s;
+            for (uint32_t u = 0; u < 4; ++u) {
+                double s = (((double)q[u][0] + (double)q[u][1]) + (double)q[u][2]) + (double)q[u][3];
+                for (int o = 32; o > 0; o >>= 1)
+                    s += __shfl_xor(s, o);
+                if (lane_id() == 0 && g0 + u < groups1)
+                    G.pg[g0 + u + 1] = s;
+            }
         }
     }
     __syncthreads();
@@ -1184,7 +1241,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 
     // top-p: first entry at which the running fp64 sum reaches top_p * total
     MAKO_STAMP(6);
-    uint32_t n = n1;
+    uint32_t n = n1, groups = groups1;
     if (topp_active) {
         const double want = (double)P.top_p * total64;
         const uint32_t hitg = (tid < groups1 && G.pg[tid + 1] >= want) ? tid : kNone;
@@ -1193,8 +1250,9 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             return false;
         if (gs != kNone) {
             if (wave_id() == 0) {
+                const uint32_t st = G.start[gs], len = G.pack[gs] & 0xffffu;
                 float q[4];
-                load_group(kf, gs, n1, q);
+                load_span(kf, st, len, q);
                 double p[4];
                 p[0] = (double)q[0];
                 p[1] = p[0] + (double)q[1];
@@ -1211,16 +1269,20 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 #pragma unroll
                 for (int j = 3; j >= 0; --j)
                     if (base + p[j] >= want)
-                        hit = gs * kGroup + lane_id() * 4u + (uint32_t)j;
-                const unsigned long long bal = __ballot(hit != kNone && hit < n1);
-                uint32_t keep = min(n1, (gs + 1u) * kGroup);
+                        hit = lane_id() * 4u + (uint32_t)j;
+                const unsigned long long bal = __ballot(hit != kNone && hit < len);
+                uint32_t keep = len;
                 if (bal)
                     keep = (uint32_t)__shfl((int)hit, __ffsll((long long)bal) - 1) + 1u;
-                if (lane_id() == 0)
-                    G.misc[0] = keep;
+                if (lane_id() == 0) {
+                    G.misc[0] = st + keep;
+                    if (keep != len)
+                        G.pack[gs] = keep; // shortened: the prepared map no longer applies (exponent 0)
+                }
             }
             __syncthreads();
             n = uniform_u32(G.misc[0]);
+            groups = gs + 1u;
         }
     }
     if (n < 1)
@@ -1229,12 +1291,12 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         return false;
     __syncthreads();
 
-    // exact fp32 total: group maps in parallel, then one wave chains them
+    // exact fp32 total: group maps in parallel (here, or already by the workers), then one wave chains them
     MAKO_STAMP(7);
-    build_group_maps(kf, n, false, 0.0, G);
+    if (!T)
+        build_group_maps(kf, groups, false, 0.0, G);
     __syncthreads();
     MAKO_STAMP(13);
-    const uint32_t groups = (n + kGroup - 1) / kGroup;
     if (wave_id() == 0) {
         // 64 groups at a time: lane l fetches group base + l's guess and map; the chain reads them by lane index
         // and keeps its state (significand M, exponent e) in scalar registers
@@ -1242,21 +1304,22 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         int e = 1; // 0.0f
         for (uint32_t base = 0; base < groups; base += kWave) {
             const uint32_t gl = min(base + lane_id(), groups - 1u);
-            const int eg_l = G.pg[gl] > 0 ? exponent_of((float)G.pg[gl]) : 0;
+            const uint32_t pk_l = G.pack[gl], st_l = G.start[gl];
             const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], cm_l = G.cmax[gl];
             // group_add_ok: M + d + cmax + 1 < 2^24
             const uint32_t lim_l = cm_l >= (1u << 24) - 1u ? 0u : (1u << 24) - 1u - cm_l;
             const uint32_t cnt = min((uint32_t)kWave, groups - base);
             for (uint32_t k = 0; k < cnt; ++k) {
-                const int eg = __builtin_amdgcn_readlane(eg_l, k);
+                const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, k);
                 const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, k);
                 const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k);
                 const uint32_t lim = (uint32_t)__builtin_amdgcn_readlane((int)lim_l, k);
                 const uint32_t dd = (M & 1u) ? d1 : d0;
-                if (e == eg && M + dd < lim) {
+                if ((uint32_t)e == (pk >> 16) && M + dd < lim) {
                     M += dd;
                 } else {
-                    const float S = exact_group_sum(kf, base + k, n, join(M, e));
+                    const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, k);
+                    const float S = exact_span_sum(kf, st, pk & 0xffffu, join(M, e));
                     uint32_t Mv;
                     int ev;
                     split(S, Mv, ev);
@@ -1281,7 +1344,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     if (r0 < 0.0f) {
         pos = 0;
     } else if (r0 == r0 && r0 != INFINITY) {
-        build_group_maps(kf, n, true, (double)r0, G);
+        build_group_maps(kf, groups, true, (double)r0, G);
         __syncthreads();
         MAKO_STAMP(14);
         if (wave_id() == 0) {
@@ -1298,8 +1361,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             bool stopped = false;
             for (uint32_t base = 0; base < groups && !stopped; base += kWave) {
                 const uint32_t gl = min(base + lane_id(), groups - 1u);
-                const double guess_l = (double)r0 - G.pg[gl];
-                const int eg_l = guess_l > 0 ? exponent_of((float)guess_l) : 0;
+                const uint32_t pk_l = G.pack[gl], st_l = G.start[gl];
+                const int eg_l = (int)(pk_l >> 16);
                 const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], cm_l = G.cmax[gl];
                 // group_sub_ok as one bound: the state after the group must be at least need_l, which keeps it
                 // inside the binade with room for one more decrement and at or above the group's first weight
@@ -1307,7 +1370,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 {
                     uint32_t Mq;
                     int eq;
-                    split(qat(gl * kGroup), Mq, eq);
+                    split(qat(st_l), Mq, eq);
                     const int dl = eg_l - eq;
                     if (dl < 0)
                         need_l = 1u << 31;
@@ -1318,16 +1381,17 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 }
                 const uint32_t cnt = min((uint32_t)kWave, groups - base);
                 for (uint32_t k = 0; k < cnt; ++k) {
-                    const int eg = __builtin_amdgcn_readlane(eg_l, k);
+                    const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, k);
                     const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, k);
                     const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k);
                     const uint32_t need = (uint32_t)__builtin_amdgcn_readlane((int)need_l, k);
                     const uint32_t dd = (M & 1u) ? d1 : d0;
-                    if (e == eg && M >= dd + need) {
+                    if ((uint32_t)e == (pk >> 16) && M >= dd + need) {
                         M -= dd;
                     } else {
+                        const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, k);
                         float r = join(M, e);
-                        if (exact_group_walk(kf, base + k, n, r, at)) {
+                        if (exact_span_walk(kf, st, pk & 0xffffu, r, at)) {
                             stopped = true;
                             break;
                         }
@@ -1454,18 +1518,28 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         sm.flag = above1 + c1;
     __syncthreads();
     const uint32_t n0 = sm.flag;
-    auto assign = [&](uint32_t b, uint32_t c, uint32_t above) {
-        if (c == 0 || b < b_lo)
-            return;
-        const uint32_t w = min(kWorkers - 1u, (uint32_t)(((unsigned long long)above * kWorkers) / n0));
-        atomicMax(&w_hi[w], b);
-        atomicMin(&w_lo[w], b);
-        atomicMin(&w_off[w], above);
-        atomicAdd(&w_cnt[w], c);
+    auto worker_of = [&](uint32_t b, uint32_t c, uint32_t above) {
+        return (c == 0 || b < b_lo) ? kNone : min(kWorkers - 1u, (uint32_t)(((unsigned long long)above * kWorkers) / n0));
     };
-    assign(b0, c0, above0);
-    assign(b1, c1, above1);
+    const uint32_t wk0 = worker_of(b0, c0, above0), wk1 = worker_of(b1, c1, above1);
+    if (wk0 != kNone) {
+        atomicMax(&w_hi[wk0], b0);
+        atomicMin(&w_lo[wk0], b0);
+        atomicMin(&w_off[wk0], above0);
+        atomicAdd(&w_cnt[wk0], c0);
+    }
+    if (wk1 != kNone) {
+        atomicMax(&w_hi[wk1], b1);
+        atomicMin(&w_lo[wk1], b1);
+        atomicMin(&w_off[wk1], above1);
+        atomicAdd(&w_cnt[wk1], c1);
+    }
     __syncthreads();
+    // the mass above a worker's range, known to the thread that holds the range's highest bin
+    if (wk0 != kNone && w_hi[wk0] == b0)
+        plan->mass[wk0] = incl - m0 - m1;
+    if (wk1 != kNone && w_hi[wk1] == b1)
+        plan->mass[wk1] = incl - m1;
     if (tid < kWorkers) {
         plan->key_lo[tid] = w_lo[tid] << 19;
         plan->key_hi[tid] = (w_hi[tid] + 1u) << 19;
@@ -1473,6 +1547,12 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         plan->cnt[tid] = w_cnt[tid];
     }
     if (tid == 0) {
+        uint32_t g = 0;
+        for (uint32_t w = 0; w < kWorkers; ++w) {
+            plan->gbase[w] = g;
+            g += (w_cnt[w] + kGroup - 1u) / kGroup;
+        }
+        plan->groups = g;
         plan->n0 = n0;
         plan->total64 = total64;
     }
@@ -1588,6 +1668,187 @@ __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t*
     }
 }
 
+// Worker's sort, LDS-resident: the weights of the row with key_lo <= bits(q) < key_hi (at most kSegCap of them)
+// are collected from the row's bits(q) array in one sweep, dropped into kFine value buckets (descending), and
+// every entry then finds its place by counting the entries of its own bucket that precede it under
+// (q desc, idx asc).  The sorted range is written to kout / iout as ~bits(q) and token id.  Returns false, having
+// written nothing, when the range does not fit or a bucket is too crowded to be ranked by counting.
+__device__ bool lds_sort_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, uint32_t key_hi, uint32_t cnt, uint32_t* kout,
+                               uint32_t* iout, unsigned long long* dyn, FinishShared& sm)
+{
+    uint2* A = reinterpret_cast<uint2*>(dyn);                       // [kSegCap] (bits(q), idx), any order
+    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);         // [kSegCap] entry of A at each bucket-ordered slot
+    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap);      // [kFine + 1] bucket counts, then bucket starts
+    const uint32_t tid = threadIdx.x, lane = lane_id();
+    if (cnt > kSegCap)
+        return false;
+    for (uint32_t b = tid; b <= kFine; b += kThreads)
+        hist[b] = 0;
+    if (tid == 0) {
+        sm.ticket = 0;
+        sm.flag = 0;
+    }
+    __syncthreads();
+    // 1. collect: a slot range per wave and trip from one LDS atomic
+    for (uint32_t base = 0; base < V; base += 4u * kThreads * 4u) {
+        uint32_t k[4][4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t i = base + u * kThreads * 4u + tid * 4u;
+            if (i + 3 < V) {
+                const uint4 x = *reinterpret_cast<const uint4*>(qk + i);
+                k[u][0] = x.x;
+                k[u][1] = x.y;
+                k[u][2] = x.z;
+                k[u][3] = x.w;
+            } else {
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j)
+                    k[u][j] = i + j < V ? qk[i + j] : 0u;
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            uint32_t mine = 0;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                if (k[u][j] < key_lo || k[u][j] >= key_hi)
+                    k[u][j] = 0; // 0 is never a candidate's weight
+                mine += k[u][j] != 0;
+            }
+            // exclusive prefix of `mine` over the wave
+            uint32_t incl = mine;
+            for (int o = 1; o < kWave; o <<= 1) {
+                const uint32_t t = __shfl_up(incl, o);
+                if (lane >= (uint32_t)o)
+                    incl += t;
+            }
+            const uint32_t wave_total = (uint32_t)__shfl((int)incl, kWave - 1);
+            if (wave_total) { // uniform
+                uint32_t slot = 0;
+                if (lane == 0)
+                    slot = atomicAdd(&sm.ticket, wave_total);
+                slot = (uint32_t)__shfl((int)slot, 0) + incl - mine;
+                const uint32_t i = base + u * kThreads * 4u + tid * 4u;
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j)
+                    if (k[u][j]) {
+                        if (slot < kSegCap)
+                            A[slot] = make_uint2(k[u][j], i + j);
+                        ++slot;
+                    }
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t n = sm.ticket;
+    if (n != cnt) // (cannot happen: the plan counted the same array)
+        return false;
+    // 2. buckets by value, heaviest first
+    const uint32_t range = key_hi - key_lo; // > 0
+    const uint32_t shift = range > kFine ? 32u - (uint32_t)__clz((range - 1u) >> 11) : 0u; // (range - 1) >> shift < kFine
+    constexpr uint32_t kPer = kSegCap / kThreads;
+    uint32_t bucket[kPer], pib[kPer];
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t) {
+        const uint32_t e = t * kThreads + tid;
+        bucket[t] = kNone;
+        pib[t] = 0;
+        if (e < n) {
+            bucket[t] = (key_hi - 1u - A[e].x) >> shift;
+            pib[t] = atomicAdd(&hist[bucket[t]], 1u);
+        }
+    }
+    __syncthreads();
+    {
+        const uint32_t c0 = hist[2u * tid], c1 = hist[2u * tid + 1u];
+        if (max(c0, c1) > 64u)
+            sm.flag = 1;
+        uint32_t total;
+        const uint32_t ex = block_excl_scan_u32(c0 + c1, total, sm.bs); // (barriers: all counts are read before)
+        hist[2u * tid] = ex;
+        hist[2u * tid + 1u] = ex + c0;
+        if (tid == 0)
+            hist[kFine] = total;
+    }
+    __syncthreads();
+    if (sm.flag)
+        return false;
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t)
+        if (bucket[t] != kNone)
+            B[hist[bucket[t]] + pib[t]] = (uint16_t)(t * kThreads + tid);
+    __syncthreads();
+    // 3. rank inside the bucket, and out
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t) {
+        const uint32_t s = t * kThreads + tid;
+        if (s < n) {
+            const uint2 me = A[B[s]];
+            const uint32_t b = (key_hi - 1u - me.x) >> shift;
+            const uint32_t lo = hist[b], hi = hist[b + 1u];
+            uint32_t r = 0;
+            for (uint32_t x = lo; x < hi; ++x) {
+                const uint2 o = A[B[x]];
+                r += (o.x > me.x) || (o.x == me.x && o.y < me.y);
+            }
+            kout[lo + r] = ~me.x;
+            iout[lo + r] = me.y;
+        }
+    }
+    __syncthreads();
+    return true;
+}
+
+// Group records of a worker's sorted range (cnt entries from position off of the list kf): fp64 sums, and the
+// maps of the running fp32 sum for the epoch guessed from the mass above the range plus the sums before the group.
+__device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, size_t t_at, double mass, const GroupTable& T,
+                              const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    double* gs = reinterpret_cast<double*>(L.sortk); // [groups]
+    const uint32_t groups = (cnt + kGroup - 1u) / kGroup;
+    __syncthreads();
+    for (uint32_t g = wave_id(); g < groups; g += kWaves) {
+        float q[4];
+        load_span(kf, off + g * kGroup, min(kGroup, cnt - g * kGroup), q);
+        double s = (((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3];
+        for (int o = 32; o > 0; o >>= 1)
+            s += __shfl_xor(s, o);
+        if (lane_id() == 0)
+            gs[g] = s;
+    }
+    __syncthreads();
+    for (uint32_t g0 = 0; g0 < groups; g0 += kThreads) { // (one trip unless the range is the fallback's)
+        const uint32_t g = g0 + tid;
+        const double v = g < groups ? gs[g] : 0.0;
+        double all;
+        const double incl = block_incl_scan_f64(v, all, sm.bs);
+        if (g < groups) {
+            T.sum[t_at + g] = v;
+            gs[g] = mass + (incl - v);
+        }
+        mass += all;
+    }
+    __syncthreads();
+    for (uint32_t g = wave_id(); g < groups; g += kWaves) {
+        const uint32_t len = min(kGroup, cnt - g * kGroup);
+        float q[4];
+        load_span(kf, off + g * kGroup, len, q);
+        const double guess = gs[g];
+        const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+        const seqfp::Step32 st = span_map(q, len, eg);
+        if (lane_id() == 0) {
+            T.d0[t_at + g] = st.d0;
+            T.d1[t_at + g] = st.d1;
+            T.cmax[t_at + g] = st.cmax;
+            T.start[t_at + g] = off + g * kGroup;
+            T.pack[t_at + g] = len | ((uint32_t)eg << 16);
+        }
+    }
+}
+
 // Whole-row path: exact for every parameter combination.  One workgroup rebuilds the penalised
 // row in scratch, keeps the candidates, sorts them by (q desc, idx asc) when top-k or top-p is
 // active, truncates, and draws.  src/gen/sampler.cpp:20-62.
@@ -1600,9 +1861,7 @@ __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32
     float* wbuf = sc.wbuf + (size_t)row * sc.vpad;
     uint32_t* cnt = sc.cnt + (size_t)row * sc.vpad;
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
-    uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
-    uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
     const float* lrow = d.logits + (int64_t)row * d.logits_stride;
     const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
 
@@ -1973,7 +2232,7 @@ struct ArgsLds {
     mako_sampling_params P; // the row's parameters
 };
 
-__device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const Scratch& sc_arg, ArgsLds& a)
+__device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const Scratch& sc_arg, uint32_t row, ArgsLds& a)
 {
     static_assert(sizeof(mako_sample_desc) % 4 == 0 && sizeof(Scratch) % 4 == 0, "word copies");
     const uint32_t* src_d = reinterpret_cast<const uint32_t*>(&d_arg);
@@ -1984,14 +2243,15 @@ __device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const 
         dst_d[i] = src_d[i];
     for (uint32_t i = threadIdx.x; i < sizeof(Scratch) / 4; i += kThreads)
         dst_s[i] = src_s[i];
-    const uint32_t* src_p = reinterpret_cast<const uint32_t*>(d_arg.params + blockIdx.y);
+    const uint32_t* src_p = reinterpret_cast<const uint32_t*>(d_arg.params + row);
     uint32_t* dst_p = reinterpret_cast<uint32_t*>(&a.P);
     if (threadIdx.x < sizeof(mako_sampling_params) / 4)
         dst_p[threadIdx.x] = src_p[threadIdx.x];
     __syncthreads();
 }
 
-// grid = (slices, rows).  Only top_k == 0 rows use more than their first workgroup.
+// grid = (rows, slices): consecutive workgroups go to different XCDs, so the rows' first workgroups, which do all
+// the work of a top-k row, spread over the whole chip.  Only top_k == 0 rows use more than their first workgroup.
 template <bool VEC, int KH>
 __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices,
                                                           uint32_t slice_len)
@@ -2000,11 +2260,11 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
     {
-        const mako_sampling_params P0 = d_arg.params[blockIdx.y];
-        if (classify(P0) != kNucleus && blockIdx.x != 0)
+        const mako_sampling_params P0 = d_arg.params[blockIdx.x];
+        if (classify(P0) != kNucleus && blockIdx.y != 0)
             return;
     }
-    stage_args(d_arg, sc_arg, s_args);
+    stage_args(d_arg, sc_arg, blockIdx.x, s_args);
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
     FinishLds L;
@@ -2012,7 +2272,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
     L.sortk = s_dyn64;                                             // 32 KB
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);    // next 16 KB
-    const uint32_t row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
+    const uint32_t row = blockIdx.x, slice = blockIdx.y, tid = threadIdx.x;
     const mako_sampling_params& P = s_args.P;
     const RowClass cls = classify(P);
     MAKO_STAMP(0);
@@ -2100,10 +2360,17 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     uint32_t thr_bits = 0;
     if (cls == kNucleus) {
         const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, L, thr_bits);
-        try_candidates = n0 <= 1024u && !any_overflow && n_cands <= kSortMax;
+        try_candidates = n0 <= (d.draft ? 1024u : kSmall) && !any_overflow && n_cands <= kSortMax;
         if (!try_candidates) {
-            if (tid == 0)
-                sc.plan[row].flag = 1; // sort_kernel takes the row
+            // (a list too long for the workers' group records goes to the whole-row path)
+            const bool fits = n0 <= kGroup * (kMaxGroups - kWorkers);
+            if (tid == 0) {
+                if (!fits) {
+                    sc.plan[row].total64 = (double)m;
+                    sc.plan[row].n0 = argidx;
+                }
+                sc.plan[row].flag = fits ? 1 : 2;
+            }
             return;
         }
     } else if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
@@ -2196,7 +2463,8 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
             sc.plan[row].flag = 1; // sort_kernel takes the row
 }
 
-// grid = (kWorkers, rows).  Rows without a work order cost one load.  Worker w gathers its range of weights from
+// grid = (kWorkers, rows); a row's workers spread over the XCDs, and worker 0 (which alone serves the whole-row
+// path) sits on a different XCD from row to row.  Rows without a work order cost one load.  Worker w gathers its range of weights from
 // the row's bits(q) array, sorts it and stores it at its place in the row's sorted list; the last worker to
 // finish cuts the nucleus and draws.
 __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_arg)
@@ -2204,11 +2472,11 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     extern __shared__ unsigned long long s_dyn64[];
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
-    const uint32_t row = blockIdx.y, w = blockIdx.x, tid = threadIdx.x;
+    const uint32_t row = blockIdx.y, w = (blockIdx.x + blockIdx.y) % kWorkers, tid = threadIdx.x;
     const uint32_t flag = sc_arg.plan[row].flag;
     if (flag == 0 || (flag == 2 && w != 0))
         return;
-    stage_args(d_arg, sc_arg, s_args);
+    stage_args(d_arg, sc_arg, row, s_args);
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
     BigPlan* plan = sc.plan + row;
@@ -2235,11 +2503,19 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
     uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
     const uint32_t cnt = plan->cnt[w], off = plan->off[w];
-    const uint32_t n0 = plan->n0;
+    const uint32_t n0 = plan->n0, groups = plan->groups;
     const double total64 = plan->total64;
+    const size_t t_row = (size_t)row * sc.g_cap;
     if (cnt) {
-        gather_range(qk, d.n_vocab, plan->key_lo[w], plan->key_hi[w], key0 + off, idx0 + off, sm);
-        sort_segment(key0 + off, idx0 + off, key1 + off, idx1 + off, cnt, L);
+        const uint32_t key_lo = plan->key_lo[w], key_hi = plan->key_hi[w];
+        MAKO_STAMP(10);
+        if (!lds_sort_range(qk, d.n_vocab, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm)) {
+            gather_range(qk, d.n_vocab, key_lo, key_hi, key0 + off, idx0 + off, sm);
+            sort_segment(key0 + off, idx0 + off, key1 + off, idx1 + off, cnt, L);
+        }
+        MAKO_STAMP(11);
+        worker_groups(key0, off, cnt, t_row + plan->gbase[w], plan->mass[w], sc.gt, L);
+        MAKO_STAMP(12);
     }
     __syncthreads(); // every thread's stores are acknowledged before the ticket is taken
     if (tid == 0) {
@@ -2254,7 +2530,7 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         plan->ticket = 0;
         plan->flag = 0;
     }
-    sorted_tail(d, row, s_args.P, key0, idx0, n0, true, total64, MAKO_PATH_GENERAL, L);
+    sorted_tail(d, row, s_args.P, key0, idx0, n0, true, total64, MAKO_PATH_GENERAL, L, false, 0.0f, &sc.gt, t_row, groups);
 }
 
 
