@@ -17,9 +17,11 @@ __device__ __forceinline__ int lane_id()
 {
     return threadIdx.x & (kWave - 1);
 }
+// (read through a scalar register: the compiler then knows the value is the same in all 64 lanes, and branches
+// and loops on it become scalar control flow)
 __device__ __forceinline__ int wave_id()
 {
-    return threadIdx.x >> 6;
+    return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding

@@ -34,8 +34,14 @@ __device__ unsigned long long g_mako_stamp[32];
         if (threadIdx.x == 0 && (gridDim.x == kWorkers ? blockIdx.y == 0 : blockIdx.x == 0))                         \
             g_mako_stamp[i] = wall_clock64();                                                                        \
     } while (0)
+#define MAKO_COUNT(i, v)                                                                                             \
+    do {                                                                                                             \
+        if (lane_id() == 0)                                                                                          \
+            g_mako_stamp[i] += (v);                                                                                  \
+    } while (0)
 #else
 #define MAKO_STAMP(i) ((void)0)
+#define MAKO_COUNT(i, v) ((void)0)
 #endif
 
 constexpr uint32_t kSliceMax = 16384; // elements per slice: 16 per thread
@@ -1241,7 +1247,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 
     // top-p: first entry at which the running fp64 sum reaches top_p * total
     MAKO_STAMP(6);
-    uint32_t n = n1, groups = groups1;
+    uint32_t n = n1, groups = uniform_u32(groups1);
     if (topp_active) {
         const double want = (double)P.top_p * total64;
         const uint32_t hitg = (tid < groups1 && G.pg[tid + 1] >= want) ? tid : kNone;
@@ -1282,11 +1288,14 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             }
             __syncthreads();
             n = uniform_u32(G.misc[0]);
-            groups = gs + 1u;
+            groups = uniform_u32(gs + 1u);
         }
     }
     if (n < 1)
         n = 1;
+    // (values merged over branches the compiler cannot see as uniform: back to scalar registers)
+    n = uniform_u32(n);
+    groups = uniform_u32(groups);
     if (need_cut && !(q_bound < qat(n - 1)))
         return false;
     __syncthreads();
@@ -1298,27 +1307,40 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     __syncthreads();
     MAKO_STAMP(13);
     if (wave_id() == 0) {
-        // 64 groups at a time: lane l fetches group base + l's guess and map; the chain reads them by lane index
-        // and keeps its state (significand M, exponent e) in scalar registers
+        // 64 groups at a time, one per lane.  A scan composes the lanes' maps; every lane then knows the state after
+        // its group, provided all groups so far share the running epoch and stay inside the binade.  The run up to the
+        // first group that cannot promise this is applied in one step, that group is replayed entry by entry, and
+        // the scan resumes behind it.  The state (significand M, exponent e) lives in scalar registers.
         uint32_t M = 0;
         int e = 1; // 0.0f
         for (uint32_t base = 0; base < groups; base += kWave) {
             const uint32_t gl = min(base + lane_id(), groups - 1u);
             const uint32_t pk_l = G.pack[gl], st_l = G.start[gl];
             const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], cm_l = G.cmax[gl];
-            // group_add_ok: M + d + cmax + 1 < 2^24
-            const uint32_t lim_l = cm_l >= (1u << 24) - 1u ? 0u : (1u << 24) - 1u - cm_l;
             const uint32_t cnt = min((uint32_t)kWave, groups - base);
-            for (uint32_t k = 0; k < cnt; ++k) {
-                const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, k);
-                const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, k);
-                const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k);
-                const uint32_t lim = (uint32_t)__builtin_amdgcn_readlane((int)lim_l, k);
-                const uint32_t dd = (M & 1u) ? d1 : d0;
-                if ((uint32_t)e == (pk >> 16) && M + dd < lim) {
-                    M += dd;
-                } else {
-                    const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, k);
+            uint32_t done = 0;
+            while (done < cnt) {
+                const bool live = lane_id() >= done && lane_id() < cnt;
+                const bool same = live && (pk_l >> 16) == (uint32_t)e;
+                Step32 v = lane_id() < done ? identity32() : (same ? Step32{d0_l, d1_l, 0u} : Step32{kSat, kSat, 0u});
+                for (int o = 1; o < kWave; o <<= 1) {
+                    Step32 t;
+                    t.d0 = __shfl_up(v.d0, o);
+                    t.d1 = __shfl_up(v.d1, o);
+                    t.cmax = 0;
+                    if (lane_id() >= (uint32_t)o)
+                        v = compose32(t, v);
+                }
+                const uint32_t after = M + ((M & 1u) ? v.d1 : v.d0); // < 2^29: no wrap
+                const bool ok = same && after + cm_l + 1u < (1u << 24); // group_add_ok for every group so far
+                const unsigned long long bad = __ballot(live && !ok);
+                const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : cnt;
+                if (f > done)
+                    M = uniform_u32((uint32_t)__shfl((int)after, (int)f - 1));
+                if (f < cnt) {
+                    const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
+                    const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
+                    MAKO_COUNT(20, 1);
                     const float S = exact_span_sum(kf, st, pk & 0xffffu, join(M, e));
                     uint32_t Mv;
                     int ev;
@@ -1326,6 +1348,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     M = uniform_u32(Mv);
                     e = (int)uniform_u32((uint32_t)ev);
                 }
+                done = f + 1u;
             }
         }
         if (lane_id() == 0)
@@ -1344,7 +1367,12 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     if (r0 < 0.0f) {
         pos = 0;
     } else if (r0 == r0 && r0 != INFINITY) {
-        build_group_maps(kf, groups, true, (double)r0, G);
+        // only the groups that start before the mass r0 has been used up can be reached; the others get no map
+        const uint32_t beyond = (tid < groups && !((double)r0 - G.pg[tid] > 0)) ? tid : kNone;
+        const uint32_t reach = min(groups, block_min_u32(beyond, sm.bs));
+        if (tid >= reach && tid < groups)
+            G.pack[tid] &= 0xffffu;
+        build_group_maps(kf, reach, true, (double)r0, G);
         __syncthreads();
         MAKO_STAMP(14);
         if (wave_id() == 0) {
@@ -1380,17 +1408,30 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         need_l = max(need_l, min(cm_l, 1u << 30) + (1u << 23) + 1u);
                 }
                 const uint32_t cnt = min((uint32_t)kWave, groups - base);
-                for (uint32_t k = 0; k < cnt; ++k) {
-                    const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, k);
-                    const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, k);
-                    const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d1_l, k);
-                    const uint32_t need = (uint32_t)__builtin_amdgcn_readlane((int)need_l, k);
-                    const uint32_t dd = (M & 1u) ? d1 : d0;
-                    if ((uint32_t)e == (pk >> 16) && M >= dd + need) {
-                        M -= dd;
-                    } else {
-                        const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, k);
+                uint32_t done = 0;
+                while (done < cnt) {
+                    const bool live = lane_id() >= done && lane_id() < cnt;
+                    const bool same = live && (pk_l >> 16) == (uint32_t)e;
+                    Step32 v = lane_id() < done ? identity32() : (same ? Step32{d0_l, d1_l, 0u} : Step32{kSat, kSat, 0u});
+                    for (int o = 1; o < kWave; o <<= 1) {
+                        Step32 t;
+                        t.d0 = __shfl_up(v.d0, o);
+                        t.d1 = __shfl_up(v.d1, o);
+                        t.cmax = 0;
+                        if (lane_id() >= (uint32_t)o)
+                            v = compose32(t, v);
+                    }
+                    const uint32_t dd = (M & 1u) ? v.d1 : v.d0;
+                    const bool ok = same && dd <= M && M - dd >= need_l; // group_sub_ok for every group so far
+                    const unsigned long long bad = __ballot(live && !ok);
+                    const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : cnt;
+                    if (f > done)
+                        M = uniform_u32((uint32_t)__shfl((int)(M - dd), (int)f - 1));
+                    if (f < cnt) {
+                        const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
+                        const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
                         float r = join(M, e);
+                        MAKO_COUNT(22, 1);
                         if (exact_span_walk(kf, st, pk & 0xffffu, r, at)) {
                             stopped = true;
                             break;
@@ -1401,6 +1442,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         M = uniform_u32(Mv);
                         e = (int)uniform_u32((uint32_t)ev);
                     }
+                    done = f + 1u;
                 }
             }
             if (lane_id() == 0)
