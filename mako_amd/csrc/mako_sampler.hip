@@ -190,7 +190,7 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
 #define MAKO_LAUNCH(V, K)                                                                                          \
     do {                                                                                                           \
         hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc, slice_len); \
-        hipLaunchKernelGGL((mako::finish_kernel<V, K>), dim3(d.n_rows, slices), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc, \
+        hipLaunchKernelGGL((mako::finish_kernel<V, K>), grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc,  \
                            slices, slice_len);                                                                     \
     } while (0)
     if (vec && kh == 2)
@@ -207,7 +207,8 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
         MAKO_LAUNCH(false, 0);
 #undef MAKO_LAUNCH
     // rows whose nucleus is too wide for the candidate lists left a work order; the others cost one load each
-    hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d, ctx->sc);
+    hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d, ctx->sc,
+                       slices);
     MAKO_HIP(ctx, hipGetLastError());
     return MAKO_OK;
 }

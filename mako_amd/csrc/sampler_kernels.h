@@ -31,7 +31,7 @@ constexpr uint32_t kNone = 0xffffffffu;
 __device__ unsigned long long g_mako_stamp[32];
 #define MAKO_STAMP(i)                                                                                                \
     do {                                                                                                             \
-        if (threadIdx.x == 0 && (gridDim.x == kWorkers ? blockIdx.y == 0 : blockIdx.x == 0))                         \
+        if (threadIdx.x == 0 && blockIdx.y == 0)                                                                     \
             g_mako_stamp[i] = wall_clock64();                                                                        \
     } while (0)
 #define MAKO_COUNT(i, v)                                                                                             \
@@ -75,11 +75,14 @@ constexpr uint32_t kSortLds = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u; /
 // Work order for a top_k == 0 row whose nucleus is too wide for the per-slice candidate lists: the weights
 // with bits(q) >= key_lo (n0 of them) are split by value into kWorkers contiguous ranges of about equal size.
 struct BigPlan {
-    uint32_t flag;   // 1: the row waits for sort_kernel's workers; 2: for its whole-row path (worker 0 alone)
+    uint32_t flag;   // 1: the row waits for sort_kernel's workers; 2: for its whole-row path (worker 0 alone);
+                     // 3: a narrow nucleus, finished by worker 0 from the candidate lists
     uint32_t n0;     // entries to sort
     uint32_t ticket; // workers that have finished
     uint32_t groups; // groups of the whole list: each worker's range is cut into groups of kGroup on its own
     double total64;  // exact fp64 sum of q over the row's candidates
+    uint32_t thr;    // bits(q) below which the nucleus cannot reach
+    uint32_t pad;
     uint32_t key_lo[kWorkers]; // worker w takes bits(q) in [key_lo[w], key_hi[w])
     uint32_t key_hi[kWorkers];
     uint32_t off[kWorkers];    // and writes them from position off[w] of the sorted list
@@ -1206,8 +1209,10 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             G.d0[tid] = T->d0[t_base + tid];
             G.d1[tid] = T->d1[t_base + tid];
             G.cmax[tid] = T->cmax[t_base + tid];
-            G.start[tid] = T->start[t_base + tid];
-            G.pack[tid] = T->pack[t_base + tid];
+            // (clamped into the list: a record is only ever read, never trusted for addressing)
+            const uint32_t st = min(T->start[t_base + tid], n1), pk = T->pack[t_base + tid];
+            G.start[tid] = st;
+            G.pack[tid] = min(pk & 0xffffu, min(kGroup, n1 - st)) | (pk & 0xffff0000u);
         }
     } else {
         if (tid < groups1) {
@@ -1481,7 +1486,6 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
                                    uint32_t n0, bool have_total, double total64, uint32_t path, const FinishLds& L)
 {
     FinishShared& sm = *L.sm;
-    const uint32_t tid = threadIdx.x;
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
     uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
@@ -1607,7 +1611,7 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
 // then a writing sweep in which ranks come from ballots.  Lane l holds entries 4l..4l+3 of each 256-entry group.
 // Returns the number of entries written.
 __device__ uint32_t gather_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, uint32_t key_hi, uint32_t* kout,
-                                 uint32_t* iout, FinishShared& sm)
+                                 uint32_t* iout, uint32_t cap, FinishShared& sm)
 {
     const uint32_t lane = lane_id(), wave = wave_id();
     const uint32_t chunk = ((V + kThreads * 4u - 1u) / (kThreads * 4u)) * kGroup; // per wave, a multiple of 256
@@ -1672,8 +1676,10 @@ __device__ uint32_t gather_range(const uint32_t* qk, uint32_t V, uint32_t key_lo
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j)
                 if (k[u][j]) {
-                    kout[pos] = ~k[u][j];
-                    iout[pos] = base + u * kGroup + lane * 4u + j;
+                    if (pos < cap) { // (the caller's count of the range; never exceeded when the plan is sound)
+                        kout[pos] = ~k[u][j];
+                        iout[pos] = base + u * kGroup + lane * 4u + j;
+                    }
                     ++pos;
                 }
             out += total;
@@ -2185,6 +2191,7 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
     float wv[16];
     Extras<KH> ex;
     load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, ex);
+    MAKO_STAMP(24);
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
     double sum = 0;
@@ -2208,6 +2215,7 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
             ++n;
         }
     }
+    MAKO_STAMP(25);
     const double total = block_sum_f64(sum, sm.bs); // (its barriers also retire every use of L.cnt above)
     const uint32_t count = block_sum_u32(n, sm.bs);
     if (threadIdx.x == 0) {
@@ -2223,6 +2231,7 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
         hsum[b] = 0;
     }
     __syncthreads();
+    MAKO_STAMP(26);
     // significand of a positive float (subnormals: no hidden bit), as seqfp::split
     auto signif = [](uint32_t b) { return (unsigned long long)((b & 0x7fffffu) | ((b >> 23) ? 0x800000u : 0u)); };
 #pragma unroll
@@ -2257,6 +2266,7 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
             }
         }
     __syncthreads();
+    MAKO_STAMP(27);
     // the slice's histogram goes to its own place: no atomics, nothing to clear afterwards
     uint32_t* binc = sc.binc + ((size_t)row * sc.slices_cap + slice) * kBins;
     unsigned long long* bins = sc.bins + ((size_t)row * sc.slices_cap + slice) * kBins;
@@ -2292,39 +2302,14 @@ __device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const 
     __syncthreads();
 }
 
-// grid = (rows, slices): consecutive workgroups go to different XCDs, so the rows' first workgroups, which do all
-// the work of a top-k row, spread over the whole chip.  Only top_k == 0 rows use more than their first workgroup.
-template <bool VEC, int KH>
-__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices,
-                                                          uint32_t slice_len)
+// First maximum of the row (std::max_element semantics, NaNs never win unless at index 0) and the totals of the
+// slices' candidate lists, from the records scan_kernel left.
+__device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uint32_t slices, float& m, uint32_t& argidx,
+                                            uint32_t& n_cands, uint32_t& any_overflow)
 {
-    extern __shared__ unsigned long long s_dyn64[];
-    __shared__ FinishShared sm;
-    __shared__ ArgsLds s_args;
-    {
-        const mako_sampling_params P0 = d_arg.params[blockIdx.x];
-        if (classify(P0) != kNucleus && blockIdx.y != 0)
-            return;
-    }
-    stage_args(d_arg, sc_arg, blockIdx.x, s_args);
-    const mako_sample_desc& d = s_args.d;
-    const Scratch& sc = s_args.sc;
-    FinishLds L;
-    L.sm = &sm;
-    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
-    L.sortk = s_dyn64;                                             // 32 KB
-    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);    // next 16 KB
-    const uint32_t row = blockIdx.x, slice = blockIdx.y, tid = threadIdx.x;
-    const mako_sampling_params& P = s_args.P;
-    const RowClass cls = classify(P);
-    MAKO_STAMP(0);
-    if (tid < 32)
-        sm.tab[tid] = k_exp2_tab[tid];
-    __syncthreads();
-
-    // first maximum of the row (std::max_element semantics, NaNs never win unless at index 0)
     unsigned long long top = 0;
-    uint32_t n_cands = 0, any_overflow = 0;
+    n_cands = 0;
+    any_overflow = 0;
     for (uint32_t s = 0; s < slices; ++s) {
         const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
         const unsigned long long p = ((unsigned long long)order_key(st.wmax) << 32) | (unsigned long long)(kNone - st.argidx);
@@ -2333,14 +2318,81 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
         any_overflow |= st.flags & kFlagOverflow;
     }
     const bool first_nan = sc.stats[(size_t)row * kMaxSlices].flags & kFlagFirstNan;
-    float m = order_unkey((uint32_t)(top >> 32));
-    uint32_t argidx = kNone - (uint32_t)top;
+    m = order_unkey((uint32_t)(top >> 32));
+    argidx = kNone - (uint32_t)top;
     if (argidx == kNone)
         argidx = 0;
     if (first_nan) {
         m = __uint_as_float(0x7fc00000u);
         argidx = 0;
     }
+}
+
+// Where each slice's candidates start in the row's flattened candidate list (sm.soff), and the largest weight a
+// logit that was NOT emitted can have over all slices (0 if none can be a candidate): everything left behind
+// has an order key below its slice's tau_key.
+__device__ float candidate_bound(const Scratch& sc, uint32_t row, uint32_t slices, float m, float inv_t, float floor_q,
+                                 FinishShared& sm)
+{
+    const uint32_t tid = threadIdx.x;
+    if (tid == 0)
+        sm.flag = 0;
+    __syncthreads();
+    if (tid < slices) {
+        const SliceStat st = sc.stats[(size_t)row * kMaxSlices + tid];
+        sm.soff[tid + 1] = st.n_emit;
+        if (!(st.flags & kFlagComplete)) {
+            const float qb = weight_of(order_unkey(st.tau_key - 1u), m, inv_t, sm.tab);
+            if (qb >= floor_q && qb > 0.0f)
+                atomicMax(&sm.flag, __float_as_uint(qb)); // positive floats order like their bits
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        sm.soff[0] = 0;
+        for (uint32_t s = 0; s < slices; ++s)
+            sm.soff[s + 1] += sm.soff[s];
+    }
+    __syncthreads();
+    const float q_bound = __uint_as_float(sm.flag);
+    __syncthreads();
+    return q_bound;
+}
+
+// grid = (slices, rows), workgroup x of row r taking slice (x + r) % slices: consecutive workgroups go to different
+// XCDs, so this spreads both the slices of one row and the rows' slice-0 workgroups, which do all the work of a
+// top-k row, over the whole chip.  Only top_k == 0 rows use more than their slice-0 workgroup.
+template <bool VEC, int KH>
+__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices,
+                                                          uint32_t slice_len)
+{
+    extern __shared__ unsigned long long s_dyn64[];
+    __shared__ FinishShared sm;
+    __shared__ ArgsLds s_args;
+    {
+        const mako_sampling_params P0 = d_arg.params[blockIdx.y];
+        if (classify(P0) != kNucleus && (blockIdx.x + blockIdx.y) % slices != 0)
+            return;
+    }
+    stage_args(d_arg, sc_arg, blockIdx.y, s_args);
+    const mako_sample_desc& d = s_args.d;
+    const Scratch& sc = s_args.sc;
+    FinishLds L;
+    L.sm = &sm;
+    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
+    L.sortk = s_dyn64;                                             // 32 KB
+    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);    // next 16 KB
+    const uint32_t row = blockIdx.y, slice = (blockIdx.x + blockIdx.y) % slices, tid = threadIdx.x;
+    const mako_sampling_params& P = s_args.P;
+    const RowClass cls = classify(P);
+    MAKO_STAMP(0);
+    if (tid < 32)
+        sm.tab[tid] = k_exp2_tab[tid];
+    __syncthreads();
+
+    float m;
+    uint32_t argidx, n_cands, any_overflow;
+    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
 
     MAKO_STAMP(1);
     if (cls == kGreedy) { // sampler.cpp:77-78, 88-92
@@ -2392,30 +2444,32 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
             bin_s0 += bins[kBins - 1u - 2u * tid];
             bin_s1 += bins[kBins - 2u - 2u * tid];
         }
+        MAKO_STAMP(15);
         if (row_n0 == 0) {
             fallback_row(d, row, argidx);
             return;
         }
     }
-    // a top_k == 0 row is planned from its histogram first: only a narrow nucleus can end inside the candidates
-    bool try_candidates = true;
-    uint32_t thr_bits = 0;
+    // a top_k == 0 row is planned from its histogram and handed to sort_kernel: to its workers, or, when the
+    // nucleus is narrow enough to end inside the candidate lists, to worker 0 alone
     if (cls == kNucleus) {
+        uint32_t thr_bits = 0;
         const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, L, thr_bits);
-        try_candidates = n0 <= (d.draft ? 1024u : kSmall) && !any_overflow && n_cands <= kSortMax;
-        if (!try_candidates) {
-            // (a list too long for the workers' group records goes to the whole-row path)
-            const bool fits = n0 <= kGroup * (kMaxGroups - kWorkers);
-            if (tid == 0) {
-                if (!fits) {
-                    sc.plan[row].total64 = (double)m;
-                    sc.plan[row].n0 = argidx;
-                }
-                sc.plan[row].flag = fits ? 1 : 2;
+        MAKO_STAMP(16);
+        const bool narrow = !d.draft && n0 <= kSmall && !any_overflow && n_cands <= kSortMax;
+        // (a list too long for the workers' group records goes to the whole-row path)
+        const bool fits = n0 <= kGroup * (kMaxGroups - kWorkers);
+        if (tid == 0) {
+            if (!fits) {
+                sc.plan[row].total64 = (double)m;
+                sc.plan[row].n0 = argidx;
             }
-            return;
+            sc.plan[row].thr = thr_bits;
+            sc.plan[row].flag = !fits ? 2 : (narrow ? 3 : 1);
         }
-    } else if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
+        return;
+    }
+    if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
         if (tid == 0) {
             sc.plan[row].total64 = (double)m; // carries the row maximum and its first index to the whole-row path
             sc.plan[row].n0 = argidx;
@@ -2424,99 +2478,50 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
         return;
     }
 
-    // ---- candidate path: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
+    // ---- top-k rows: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
-    // where each slice's candidates start, and the largest weight a logit that was NOT emitted can have over
-    // all slices (0 if none can be a candidate): everything left behind has an order key below tau_key
-    if (tid == 0)
-        sm.flag = 0;
-    __syncthreads();
-    if (tid < slices) {
-        const SliceStat st = sc.stats[(size_t)row * kMaxSlices + tid];
-        sm.soff[tid + 1] = st.n_emit;
-        if (!(st.flags & kFlagComplete)) {
-            const float qb = weight_of(order_unkey(st.tau_key - 1u), m, inv_t, sm.tab);
-            if (qb >= floor_q && qb > 0.0f)
-                atomicMax(&sm.flag, __float_as_uint(qb)); // positive floats order like their bits
-        }
-    }
-    __syncthreads();
-    if (tid == 0) {
-        sm.soff[0] = 0;
-        for (uint32_t s = 0; s < slices; ++s)
-            sm.soff[s + 1] += sm.soff[s];
-    }
-    __syncthreads();
-    const float q_bound = __uint_as_float(sm.flag);
+    const float q_bound = candidate_bound(sc, row, slices, m, inv_t, floor_q, sm);
     MAKO_STAMP(3);
     uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax); // upper half of the dynamic block
     uint32_t* jf = kf + kSortMax;
-    if (!d.draft) {
-        // short lists: the top_k-th weight's neighbourhood, or the part of the candidates the nucleus can reach
-        uint32_t n_valid = 0;
-        const uint32_t n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, cls == kTopK ? P.top_k : 0u,
-                                                 thr_bits, kf, jf, n_valid, L);
-        MAKO_STAMP(4);
-        if (n_list != kNone) {
-            if (cls == kTopK) {
-                const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
-                if (ok && n_valid == 0) {
-                    fallback_row(d, row, argidx);
-                } else if (ok) {
-                    sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L);
-                } else if (tid == 0) {
-                    sc.plan[row].total64 = (double)m;
-                    sc.plan[row].n0 = argidx;
-                    sc.plan[row].flag = 2;
-                }
-                return;
-            }
-            if (n_list == 0 || !sorted_tail(d, row, P, kf, jf, n_list, true, row_total, MAKO_PATH_NUCLEUS, L, true, q_bound))
-                if (tid == 0)
-                    sc.plan[row].flag = 1;
-            return;
-        }
-    }
-    const uint32_t n_valid = n_cands <= 1024u ? sort_candidates<1>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L)
-                                              : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
+    uint32_t n_valid = 0;
+    uint32_t n_list = kNone;
+    if (!d.draft) // the top_k-th weight's neighbourhood only
+        n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, P.top_k, 0u, kf, jf, n_valid, L);
+    if (n_list == kNone)
+        n_valid = n_cands <= 1024u ? sort_candidates<1>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L)
+                                   : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
     MAKO_STAMP(4);
-    if (cls == kTopK) {
-        // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
-        const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
-        if (!ok) {
-            if (tid == 0) {
-                sc.plan[row].total64 = (double)m;
-                sc.plan[row].n0 = argidx;
-                sc.plan[row].flag = 2;
-            }
-            return;
+    // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
+    const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
+    if (!ok) {
+        if (tid == 0) {
+            sc.plan[row].total64 = (double)m;
+            sc.plan[row].n0 = argidx;
+            sc.plan[row].flag = 2;
         }
-        if (n_valid == 0) {
-            fallback_row(d, row, argidx);
-            return;
-        }
-        sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L); // sampler.cpp:40-43
         return;
     }
-    // top_k == 0: the nucleus must end inside the candidates, strictly above everything left behind
-    if (n_valid == 0 || !sorted_tail(d, row, P, kf, jf, n_valid, true, row_total, MAKO_PATH_NUCLEUS, L, true, q_bound))
-        if (tid == 0)
-            sc.plan[row].flag = 1; // sort_kernel takes the row
+    if (n_valid == 0) {
+        fallback_row(d, row, argidx);
+        return;
+    }
+    sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L); // sampler.cpp:40-43
 }
 
 // grid = (kWorkers, rows); a row's workers spread over the XCDs, and worker 0 (which alone serves the whole-row
 // path) sits on a different XCD from row to row.  Rows without a work order cost one load.  Worker w gathers its range of weights from
 // the row's bits(q) array, sorts it and stores it at its place in the row's sorted list; the last worker to
 // finish cuts the nucleus and draws.
-__global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_arg)
+__global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices)
 {
     extern __shared__ unsigned long long s_dyn64[];
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
     const uint32_t row = blockIdx.y, w = (blockIdx.x + blockIdx.y) % kWorkers, tid = threadIdx.x;
     const uint32_t flag = sc_arg.plan[row].flag;
-    if (flag == 0 || (flag == 2 && w != 0))
+    if (flag == 0 || (flag != 1 && w != 0))
         return;
     stage_args(d_arg, sc_arg, row, s_args);
     const mako_sample_desc& d = s_args.d;
@@ -2544,19 +2549,53 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
     uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
     uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
-    const uint32_t cnt = plan->cnt[w], off = plan->off[w];
-    const uint32_t n0 = plan->n0, groups = plan->groups;
+    const uint32_t n0 = min(plan->n0, d.n_vocab), groups = min(plan->groups, kMaxGroups);
     const double total64 = plan->total64;
+    if (flag == 3) {
+        // narrow nucleus: it should end inside the slices' candidate lists, strictly above everything they left out
+        const uint32_t thr_bits = plan->thr;
+        __syncthreads();
+        if (tid == 0)
+            plan->flag = 0;
+        const mako_sampling_params& P = s_args.P;
+        float m;
+        uint32_t argidx, n_cands, any_overflow;
+        row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
+        const float inv_t = 1.0f / P.temperature;
+        const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
+        const float q_bound = candidate_bound(sc, row, slices, m, inv_t, floor_q, sm);
+        MAKO_STAMP(3);
+        uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax);
+        uint32_t* jf = kf + kSortMax;
+        uint32_t n_valid = 0;
+        const uint32_t n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, 0u, thr_bits, kf, jf, n_valid, L);
+        MAKO_STAMP(4);
+        if (n_list != kNone && n_list > 0 &&
+            sorted_tail(d, row, P, kf, jf, n_list, true, total64, MAKO_PATH_NUCLEUS, L, true, q_bound))
+            return;
+        // not certifiable from the candidates: the row's weights at or above the threshold, from its bits(q) array
+        if (!lds_sort_range(qk, d.n_vocab, thr_bits, 0x7f800001u, n0, key0, idx0, s_dyn64, sm)) {
+            gather_range(qk, d.n_vocab, thr_bits, 0x7f800001u, key0, idx0, n0, sm);
+            sort_segment(key0, idx0, key1, idx1, n0, L);
+        }
+        sorted_tail(d, row, P, key0, idx0, n0, true, total64, MAKO_PATH_GENERAL, L);
+        return;
+    }
+    uint32_t cnt = plan->cnt[w];
+    const uint32_t off = plan->off[w], gbase = plan->gbase[w];
+    // (a sound plan never trips these; they keep every store of this worker inside the row's arrays)
+    if (off > n0 || cnt > n0 - off || gbase + (cnt + kGroup - 1u) / kGroup > min(groups, sc.g_cap))
+        cnt = 0;
     const size_t t_row = (size_t)row * sc.g_cap;
     if (cnt) {
         const uint32_t key_lo = plan->key_lo[w], key_hi = plan->key_hi[w];
         MAKO_STAMP(10);
         if (!lds_sort_range(qk, d.n_vocab, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm)) {
-            gather_range(qk, d.n_vocab, key_lo, key_hi, key0 + off, idx0 + off, sm);
+            gather_range(qk, d.n_vocab, key_lo, key_hi, key0 + off, idx0 + off, cnt, sm);
             sort_segment(key0 + off, idx0 + off, key1 + off, idx1 + off, cnt, L);
         }
         MAKO_STAMP(11);
-        worker_groups(key0, off, cnt, t_row + plan->gbase[w], plan->mass[w], sc.gt, L);
+        worker_groups(key0, off, cnt, t_row + gbase, plan->mass[w], sc.gt, L);
         MAKO_STAMP(12);
     }
     __syncthreads(); // every thread's stores are acknowledged before the ticket is taken
