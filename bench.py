@@ -127,6 +127,16 @@ def main():
     ms_per_step = ms / a.steps
     tokens = batch.o_tokens.download()
 
+    # per-kernel split of a batch: HIP events recorded by the library on the launch stream, a few extra steps
+    ctx.set_profile(True)
+    split = np.zeros(3)
+    n_split = min(a.steps, 50)
+    for i in range(n_split):
+        step(a.warmup + a.steps + i)
+        split += np.array(ctx.kernel_times_ms())
+    split /= n_split
+    ctx.set_profile(False)
+
     base, ref_tok = (None, None)
     if a.cpu_seconds > 0:
         base, ref_tok = cpu_baseline(w, a.cpu_seconds)
@@ -153,8 +163,11 @@ def main():
                    "host_wall_ms_per_step": wall * 1e3 / a.steps},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "bytes_per_launch": batch_bytes, "kernel": "scan_kernel + finish_kernel (one batch)",
-                     "launch_ms": ms_per_step},
+                     "bytes_per_launch": batch_bytes,
+                     "kernel": "scan_kernel + finish_kernel + sort_kernel (the three launches of one batch)",
+                     "launch_ms": ms_per_step,
+                     "kernel_ms": {"scan_kernel": split[0], "finish_kernel": split[1], "sort_kernel": split[2]},
+                     "scan_kernel_gbs": batch_bytes / (split[0] * 1e-3) / 1e9},
         "cpu_baseline": base,
         "parity": parity,
     }

@@ -110,6 +110,13 @@ int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t
 /* Text of the last failure on this context (never null). */
 const char* mako_sampler_last_error(const mako_sampler_ctx* ctx);
 
+/* Per-kernel timing for benchmarks (no counterpart in the reference).  While enabled, every
+ * mako_sampler_sample_batch records HIP events on its stream around its three kernels;
+ * mako_sampler_kernel_times waits for the last recorded batch and returns the milliseconds of
+ * scan_kernel, finish_kernel and sort_kernel in out_ms[0..2].  Off by default. */
+int mako_sampler_set_profile(mako_sampler_ctx* ctx, int enabled);
+int mako_sampler_kernel_times(mako_sampler_ctx* ctx, float* out_ms);
+
 /* Number of slices a row of n_vocab logits is split into by the scan kernel. */
 uint32_t mako_sampler_slices(uint32_t n_vocab);
 

@@ -81,6 +81,8 @@ EXPORTS = [
     "mako_sampler_sample_host",
     "mako_sampler_last_error",
     "mako_sampler_slices",
+    "mako_sampler_set_profile",
+    "mako_sampler_kernel_times",
     "mako_sampler_debug_expf",
     "mako_sampler_debug_div",
 ]
@@ -99,6 +101,8 @@ def load():
         lib.mako_sampler_sample_batch.argtypes = [C.c_void_p, C.POINTER(Desc), C.c_void_p]
         lib.mako_sampler_last_error.restype = C.c_char_p
         lib.mako_sampler_last_error.argtypes = [C.c_void_p]
+        lib.mako_sampler_set_profile.argtypes = [C.c_void_p, C.c_int]
+        lib.mako_sampler_kernel_times.argtypes = [C.c_void_p, C.POINTER(C.c_float)]
         lib.mako_sampler_slices.restype = C.c_uint32
         lib.mako_sampler_slices.argtypes = [C.c_uint32]
         lib.mako_sampler_debug_expf.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p]
@@ -141,6 +145,19 @@ class SamplerContext:
 
     def last_error(self):
         return self.lib.mako_sampler_last_error(self.ptr).decode()
+
+    def set_profile(self, enabled):
+        rc = self.lib.mako_sampler_set_profile(self.ptr, 1 if enabled else 0)
+        if rc != MAKO_OK:
+            raise MakoError("mako_sampler_set_profile: %d %s" % (rc, self.last_error()))
+
+    def kernel_times_ms(self):
+        """(scan, finish, sort) kernel milliseconds of the last batch sampled while profiling was on."""
+        out = (C.c_float * 3)()
+        rc = self.lib.mako_sampler_kernel_times(self.ptr, out)
+        if rc != MAKO_OK:
+            raise MakoError("mako_sampler_kernel_times: %d %s" % (rc, self.last_error()))
+        return [float(x) for x in out]
 
     def sample_batch(self, desc, stream=None):
         rc = self.lib.mako_sampler_sample_batch(self.ptr, C.byref(desc), stream.ptr if stream else None)

@@ -32,6 +32,8 @@ struct mako_sampler_ctx {
     int32_t* st_tokens = nullptr;
     uint8_t* st_acc = nullptr;
     std::string err = "";
+    bool profile = false, profiled = false;
+    hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
 };
 
 namespace {
@@ -147,7 +149,36 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
     for (void* p : ptrs)
         if (p)
             (void)hipFree(p);
+    for (hipEvent_t e : ctx->ev)
+        if (e)
+            (void)hipEventDestroy(e);
     delete ctx;
+}
+
+int mako_sampler_set_profile(mako_sampler_ctx* ctx, int enabled)
+{
+    if (!ctx)
+        return MAKO_ERR_INVALID_ARG;
+    MAKO_HIP(ctx, hipSetDevice(ctx->device));
+    if (enabled)
+        for (hipEvent_t& e : ctx->ev)
+            if (!e)
+                MAKO_HIP(ctx, hipEventCreate(&e));
+    ctx->profile = enabled != 0;
+    ctx->profiled = false;
+    return MAKO_OK;
+}
+
+int mako_sampler_kernel_times(mako_sampler_ctx* ctx, float* out_ms)
+{
+    if (!ctx || !out_ms)
+        return MAKO_ERR_INVALID_ARG;
+    if (!ctx->profiled)
+        return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: no profiled batch to report");
+    MAKO_HIP(ctx, hipEventSynchronize(ctx->ev[3]));
+    for (int i = 0; i < 3; ++i)
+        MAKO_HIP(ctx, hipEventElapsedTime(&out_ms[i], ctx->ev[i], ctx->ev[i + 1]));
+    return MAKO_OK;
 }
 
 const char* mako_sampler_last_error(const mako_sampler_ctx* ctx)
@@ -187,12 +218,21 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     const dim3 grid(slices, d.n_rows);
     // histories of up to 2 (8) entries per thread stay in registers; longer ones take the generic route
     const int kh = !d.hist_tokens ? 2 : (d.hist_stride <= 2 * mako::kThreads ? 2 : (d.hist_stride <= 8 * mako::kThreads ? 8 : 0));
+    const bool prof = ctx->profile;
+#define MAKO_MARK(i)                                                                                               \
+    do {                                                                                                           \
+        if (prof)                                                                                                  \
+            MAKO_HIP(ctx, hipEventRecord(ctx->ev[i], st));                                                         \
+    } while (0)
 #define MAKO_LAUNCH(V, K)                                                                                          \
     do {                                                                                                           \
         hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc, slice_len); \
+        MAKO_MARK(1);                                                                                              \
         hipLaunchKernelGGL((mako::finish_kernel<V, K>), grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc,  \
                            slices, slice_len);                                                                     \
+        MAKO_MARK(2);                                                                                              \
     } while (0)
+    MAKO_MARK(0);
     if (vec && kh == 2)
         MAKO_LAUNCH(true, 2);
     else if (vec && kh == 8)
@@ -209,6 +249,9 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     // rows whose nucleus is too wide for the candidate lists left a work order; the others cost one load each
     hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d, ctx->sc,
                        slices);
+    MAKO_MARK(3);
+#undef MAKO_MARK
+    ctx->profiled = prof;
     MAKO_HIP(ctx, hipGetLastError());
     return MAKO_OK;
 }
