@@ -1067,6 +1067,76 @@ __device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len
     return false;
 }
 
+// Same result as exact_span_walk for a span of a DESCENDING list, in far fewer dependent steps: the lanes' maps of
+// their four entries (for the binade r is in) are composed by a scan, the run of lanes that provably neither
+// stops the walk nor leaves the binade is applied at once, the first lane that cannot promise this is replayed
+// with real fp32 operations, and the scan resumes behind it in the binade r has reached.
+__device__ bool scan_span_walk(const uint32_t* kf, uint32_t start, uint32_t len, float& r, uint32_t& pos)
+{
+    using namespace seqfp;
+    float q[4];
+    load_span(kf, start, len, q); // entries past the end read as 0.0f
+    const uint32_t beg = uniform_u32(start);
+    const uint32_t lanes = (uniform_u32(len) + 3u) / 4u;
+    uint32_t Mq0;
+    int eq0;
+    split(q[0], Mq0, eq0); // the lane's largest entry
+    uint32_t done = 0;
+    while (done < lanes) {
+        uint32_t Mv;
+        int ev;
+        split(r, Mv, ev);
+        const uint32_t M = uniform_u32(Mv);
+        const int e = (int)uniform_u32((uint32_t)ev);
+        const bool live = lane_id() >= done && lane_id() < lanes;
+        Step32 v = identity32();
+        if (live) {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                v = compose32(v, step32(q[j], e));
+        }
+        // the state after this lane's entries must stay at or above its largest entry (no stop inside the lane)
+        // and inside the binade with room for one more decrement
+        uint32_t need = 1u;
+        {
+            const int dl = e - eq0;
+            if (dl < 0)
+                need = 1u << 31;
+            else if (dl <= 25)
+                need = max(1u, (uint32_t)(((unsigned long long)Mq0 + (1ull << dl) - 1ull) >> dl));
+            if (e > 1)
+                need = max(need, min(v.cmax, 1u << 30) + (1u << 23) + 1u);
+        }
+        for (int o = 1; o < kWave; o <<= 1) {
+            Step32 t;
+            t.d0 = __shfl_up(v.d0, o);
+            t.d1 = __shfl_up(v.d1, o);
+            t.cmax = 0;
+            if (lane_id() >= (uint32_t)o)
+                v = compose32(t, v);
+        }
+        const uint32_t dd = (M & 1u) ? v.d1 : v.d0;
+        const bool ok = dd <= M && M - dd >= need;
+        const unsigned long long bad = __ballot(live && !ok);
+        const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : lanes;
+        if (f > done)
+            r = join(uniform_u32((uint32_t)__shfl((int)(M - dd), (int)f - 1)), e);
+        if (f < lanes) {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                const float x = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), f));
+                if (__builtin_amdgcn_readfirstlane((int)(r < x))) {
+                    pos = beg + f * 4u + j;
+                    return true;
+                }
+                r -= x;
+            }
+        }
+        done = f + 1u;
+    }
+    return false;
+}
+
 // Tail of every path that ends with a list sorted by (q desc, idx asc): kf[i] = ~bits(q_i), jf[i] = token id,
 // n1 entries (already cut to top_k).  Applies top-p (src/gen/sampler.cpp:44-61) against total64 (the fp64 sum over
 // the row's candidates; summed from the list when !have_total), then the exact fp32 total (:80-82) and walk
@@ -1437,7 +1507,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
                         float r = join(M, e);
                         MAKO_COUNT(22, 1);
-                        if (exact_span_walk(kf, st, pk & 0xffffu, r, at)) {
+                        if (scan_span_walk(kf, st, pk & 0xffffu, r, at)) {
                             stopped = true;
                             break;
                         }
@@ -1757,26 +1827,22 @@ __device__ bool lds_sort_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, 
         }
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
-            uint32_t mine = 0;
+            // ranks inside the wave from ballots (any order will do), one LDS atomic per wave for the slots
+            uint32_t before = 0, wave_total = 0;
+            const unsigned long long lower = (1ull << lane) - 1ull;
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j) {
                 if (k[u][j] < key_lo || k[u][j] >= key_hi)
                     k[u][j] = 0; // 0 is never a candidate's weight
-                mine += k[u][j] != 0;
+                const unsigned long long bal = __ballot(k[u][j] != 0);
+                before += (uint32_t)__popcll(bal & lower);
+                wave_total += (uint32_t)__popcll(bal);
             }
-            // exclusive prefix of `mine` over the wave
-            uint32_t incl = mine;
-            for (int o = 1; o < kWave; o <<= 1) {
-                const uint32_t t = __shfl_up(incl, o);
-                if (lane >= (uint32_t)o)
-                    incl += t;
-            }
-            const uint32_t wave_total = (uint32_t)__shfl((int)incl, kWave - 1);
             if (wave_total) { // uniform
                 uint32_t slot = 0;
                 if (lane == 0)
                     slot = atomicAdd(&sm.ticket, wave_total);
-                slot = (uint32_t)__shfl((int)slot, 0) + incl - mine;
+                slot = uniform_u32(slot) + before;
                 const uint32_t i = base + u * kThreads * 4u + tid * 4u;
 #pragma unroll
                 for (uint32_t j = 0; j < 4; ++j)
@@ -2591,6 +2657,7 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         const uint32_t key_lo = plan->key_lo[w], key_hi = plan->key_hi[w];
         MAKO_STAMP(10);
         if (!lds_sort_range(qk, d.n_vocab, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm)) {
+            MAKO_COUNT(23, threadIdx.x == 0 ? 1 : 0);
             gather_range(qk, d.n_vocab, key_lo, key_hi, key0 + off, idx0 + off, cnt, sm);
             sort_segment(key0 + off, idx0 + off, key1 + off, idx1 + off, cnt, L);
         }
