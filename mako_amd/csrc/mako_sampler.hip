@@ -33,7 +33,7 @@ struct mako_sampler_ctx {
     uint8_t* st_acc = nullptr;
     std::string err = "";
     bool profile = false, profiled = false;
-    hipEvent_t ev[4] = {nullptr, nullptr, nullptr, nullptr};
+    hipEvent_t ev[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
 };
 
 namespace {
@@ -98,8 +98,6 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap));
     MAKO_HIP(ctx, dev_alloc(&sc.part_sum, (size_t)max_rows * mako::kMaxSlices));
     MAKO_HIP(ctx, dev_alloc(&sc.part_n, (size_t)max_rows * mako::kMaxSlices));
-    MAKO_HIP(ctx, dev_alloc(&sc.tickets, (size_t)max_rows * 32));
-    MAKO_HIP(ctx, hipMemset(sc.tickets, 0, (size_t)max_rows * 32 * sizeof(uint32_t)));
     MAKO_HIP(ctx, dev_alloc(&sc.binc, (size_t)max_rows * sc.slices_cap * mako::kBins));
     MAKO_HIP(ctx, dev_alloc(&sc.plan, (size_t)max_rows));
     MAKO_HIP(ctx, hipMemset(sc.plan, 0, (size_t)max_rows * sizeof(mako::BigPlan)));
@@ -127,7 +125,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
                              (const void*)mako::finish_kernel<true, 0>,  (const void*)mako::finish_kernel<false, 0>,
                              (const void*)mako::finish_kernel<true, 2>,  (const void*)mako::finish_kernel<false, 2>,
                              (const void*)mako::finish_kernel<true, 8>,  (const void*)mako::finish_kernel<false, 8>,
-                             (const void*)mako::sort_kernel};
+                             (const void*)mako::sort_kernel,             (const void*)mako::plan_kernel,
+                             (const void*)mako::tail_kernel};
     static_assert(mako::kSortLds >= mako::kDynLds, "sort_kernel's tail uses the finishing kernel's LDS layout");
     for (const void* k : kernels)
         MAKO_HIP(ctx, hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -142,7 +141,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
     void* ptrs[] = {sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack,
-                    sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.tickets, sc.binc, sc.bins, sc.plan,
+                    sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.binc, sc.bins, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
                     ctx->st_hist,  ctx->st_hcnt, ctx->st_hlen,  ctx->st_draft, ctx->st_tokens, ctx->st_acc};
@@ -175,8 +174,8 @@ int mako_sampler_kernel_times(mako_sampler_ctx* ctx, float* out_ms)
         return MAKO_ERR_INVALID_ARG;
     if (!ctx->profiled)
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: no profiled batch to report");
-    MAKO_HIP(ctx, hipEventSynchronize(ctx->ev[3]));
-    for (int i = 0; i < 3; ++i)
+    MAKO_HIP(ctx, hipEventSynchronize(ctx->ev[5]));
+    for (int i = 0; i < 5; ++i)
         MAKO_HIP(ctx, hipEventElapsedTime(&out_ms[i], ctx->ev[i], ctx->ev[i + 1]));
     return MAKO_OK;
 }
@@ -246,10 +245,15 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     else
         MAKO_LAUNCH(false, 0);
 #undef MAKO_LAUNCH
-    // rows whose nucleus is too wide for the candidate lists left a work order; the others cost one load each
+    // top_k == 0 rows: plan from the row's histogram, sort by the plan, cut and draw; the stages talk through
+    // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  Other rows cost a load.
+    hipLaunchKernelGGL(mako::plan_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc, slices);
+    MAKO_MARK(3);
     hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d, ctx->sc,
                        slices);
-    MAKO_MARK(3);
+    MAKO_MARK(4);
+    hipLaunchKernelGGL(mako::tail_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc);
+    MAKO_MARK(5);
 #undef MAKO_MARK
     ctx->profiled = prof;
     MAKO_HIP(ctx, hipGetLastError());

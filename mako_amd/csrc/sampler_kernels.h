@@ -78,7 +78,7 @@ struct BigPlan {
     uint32_t flag;   // 1: the row waits for sort_kernel's workers; 2: for its whole-row path (worker 0 alone);
                      // 3: a narrow nucleus, finished by worker 0 from the candidate lists
     uint32_t n0;     // entries to sort
-    uint32_t ticket; // workers that have finished
+    uint32_t pad0;
     uint32_t groups; // groups of the whole list: each worker's range is cut into groups of kGroup on its own
     double total64;  // exact fp64 sum of q over the row's candidates
     uint32_t thr;    // bits(q) below which the nucleus cannot reach
@@ -107,9 +107,8 @@ struct Scratch {
     uint32_t* cand_i;  // [max_rows][slices_cap][kCap] their token ids
     double* part_sum;  // [max_rows][kMaxSlices] exact fp64 sum of q over the slice (top_k == 0 rows)
     uint32_t* part_n;  // [max_rows][kMaxSlices] candidates (q > 0, q >= min_p) in the slice
-    uint32_t* tickets; // [max_rows][32] arrival counter of the row's slices (one per 128-byte line); zero between calls
     uint32_t* binc;    // [max_rows][slices_cap][kBins] candidates per weight bin of each slice (top_k == 0 rows)
-    BigPlan* plan;     // [max_rows]; flag and ticket zero between calls
+    BigPlan* plan;     // [max_rows]; flag zero between calls
     unsigned long long* bins; // [max_rows][slices_cap][kBins] sum of their 24-bit significands: a bin's exact
                               // mass is bins * 2^(e - 150), e being the bin's exponent
     float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path; top_k == 0 rows keep
@@ -2476,63 +2475,8 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     }
 
     if (cls == kNucleus) {
-        // second pass: all slices of the row in parallel; the last one to arrive finishes the row
+        // second pass, all slices of the row in parallel; plan_kernel continues once every slice is through
         slice_partial<VEC, KH>(d, sc, row, slice, slice_len, P, m, L);
-        __syncthreads(); // every thread's stores and atomics are acknowledged before the ticket is taken
-        if (tid == 0) {
-            __threadfence();
-            sm.ticket = atomicAdd(&sc.tickets[(size_t)row * 32], 1u);
-        }
-        __syncthreads();
-        if (sm.ticket != slices - 1)
-            return;
-        __threadfence();
-        if (tid == 0)
-            sc.tickets[(size_t)row * 32] = 0;
-    }
-
-    MAKO_STAMP(2);
-    // top_k == 0: the row's exact total and candidate count from the second pass, and this thread's two bins of
-    // the weight histogram (summed over the slices)
-    double row_total = 0;
-    uint32_t row_n0 = 0, bin_c0 = 0, bin_c1 = 0;
-    unsigned long long bin_s0 = 0, bin_s1 = 0;
-    if (cls == kNucleus) {
-        for (uint32_t s = 0; s < slices; ++s) {
-            row_total += sc.part_sum[(size_t)row * kMaxSlices + s];
-            row_n0 += sc.part_n[(size_t)row * kMaxSlices + s];
-        }
-        for (uint32_t s = 0; s < slices; ++s) {
-            const uint32_t* binc = sc.binc + ((size_t)row * sc.slices_cap + s) * kBins;
-            const unsigned long long* bins = sc.bins + ((size_t)row * sc.slices_cap + s) * kBins;
-            bin_c0 += binc[kBins - 1u - 2u * tid];
-            bin_c1 += binc[kBins - 2u - 2u * tid];
-            bin_s0 += bins[kBins - 1u - 2u * tid];
-            bin_s1 += bins[kBins - 2u - 2u * tid];
-        }
-        MAKO_STAMP(15);
-        if (row_n0 == 0) {
-            fallback_row(d, row, argidx);
-            return;
-        }
-    }
-    // a top_k == 0 row is planned from its histogram and handed to sort_kernel: to its workers, or, when the
-    // nucleus is narrow enough to end inside the candidate lists, to worker 0 alone
-    if (cls == kNucleus) {
-        uint32_t thr_bits = 0;
-        const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, L, thr_bits);
-        MAKO_STAMP(16);
-        const bool narrow = !d.draft && n0 <= kSmall && !any_overflow && n_cands <= kSortMax;
-        // (a list too long for the workers' group records goes to the whole-row path)
-        const bool fits = n0 <= kGroup * (kMaxGroups - kWorkers);
-        if (tid == 0) {
-            if (!fits) {
-                sc.plan[row].total64 = (double)m;
-                sc.plan[row].n0 = argidx;
-            }
-            sc.plan[row].thr = thr_bits;
-            sc.plan[row].flag = !fits ? 2 : (narrow ? 3 : 1);
-        }
         return;
     }
     if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
@@ -2574,6 +2518,85 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
         return;
     }
     sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L); // sampler.cpp:40-43
+}
+
+// grid = (1, rows).  top_k == 0 rows only: the row's exact total, candidate count and weight histogram are summed
+// over its slices and the row is planned: handed to sort_kernel's workers, or, when the nucleus is narrow enough to
+// end inside the candidate lists, to its worker 0 alone.
+__global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices)
+{
+    extern __shared__ unsigned long long s_dyn64[];
+    __shared__ FinishShared sm;
+    __shared__ ArgsLds s_args;
+    const uint32_t row = blockIdx.y, tid = threadIdx.x;
+    {
+        const mako_sampling_params P0 = d_arg.params[row];
+        if (classify(P0) != kNucleus)
+            return;
+    }
+    stage_args(d_arg, sc_arg, row, s_args);
+    const mako_sample_desc& d = s_args.d;
+    const Scratch& sc = s_args.sc;
+    const mako_sampling_params& P = s_args.P;
+    FinishLds L;
+    L.sm = &sm;
+    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
+    L.sortk = s_dyn64;
+    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
+    MAKO_STAMP(2);
+    // this thread's two bins of the histogram, every slice's loads in flight together
+    double row_total = 0;
+    uint32_t row_n0 = 0, bin_c0 = 0, bin_c1 = 0;
+    unsigned long long bin_s0 = 0, bin_s1 = 0;
+    for (uint32_t s0 = 0; s0 < slices; s0 += 8u) {
+        uint32_t c0[8], c1[8], pn[8];
+        unsigned long long h0[8], h1[8];
+        double ps[8];
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) {
+            const uint32_t sl = min(s0 + u, slices - 1u);
+            const uint32_t* binc = sc.binc + ((size_t)row * sc.slices_cap + sl) * kBins;
+            const unsigned long long* bins = sc.bins + ((size_t)row * sc.slices_cap + sl) * kBins;
+            c0[u] = binc[kBins - 1u - 2u * tid];
+            c1[u] = binc[kBins - 2u - 2u * tid];
+            h0[u] = bins[kBins - 1u - 2u * tid];
+            h1[u] = bins[kBins - 2u - 2u * tid];
+            ps[u] = sc.part_sum[(size_t)row * kMaxSlices + sl];
+            pn[u] = sc.part_n[(size_t)row * kMaxSlices + sl];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u)
+            if (s0 + u < slices) {
+                bin_c0 += c0[u];
+                bin_c1 += c1[u];
+                bin_s0 += h0[u];
+                bin_s1 += h1[u];
+                row_total += ps[u];
+                row_n0 += pn[u];
+            }
+    }
+    float m;
+    uint32_t argidx, n_cands, any_overflow;
+    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
+    MAKO_STAMP(15);
+    if (row_n0 == 0) {
+        fallback_row(d, row, argidx);
+        return;
+    }
+    uint32_t thr_bits = 0;
+    const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, L, thr_bits);
+    MAKO_STAMP(16);
+    const bool narrow = !d.draft && n0 <= kSmall && !any_overflow && n_cands <= kSortMax;
+    // (a list too long for the workers' group records goes to the whole-row path)
+    const bool fits = n0 <= kGroup * (kMaxGroups - kWorkers);
+    if (tid == 0) {
+        if (!fits) {
+            sc.plan[row].total64 = (double)m;
+            sc.plan[row].n0 = argidx;
+        }
+        sc.plan[row].thr = thr_bits;
+        sc.plan[row].flag = !fits ? 2 : (narrow ? 3 : 1);
+    }
 }
 
 // grid = (kWorkers, rows); a row's workers spread over the XCDs, and worker 0 (which alone serves the whole-row
@@ -2665,20 +2688,33 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         worker_groups(key0, off, cnt, t_row + gbase, plan->mass[w], sc.gt, L);
         MAKO_STAMP(12);
     }
-    __syncthreads(); // every thread's stores are acknowledged before the ticket is taken
-    if (tid == 0) {
-        __threadfence();
-        sm.ticket = atomicAdd(&plan->ticket, 1u);
-    }
-    __syncthreads();
-    if (sm.ticket != kWorkers - 1)
+}
+
+// grid = (1, rows).  Rows whose sorted list sort_kernel's workers have prepared: top-p cut, exact total, draw.
+__global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_arg)
+{
+    extern __shared__ unsigned long long s_dyn64[];
+    __shared__ FinishShared sm;
+    __shared__ ArgsLds s_args;
+    const uint32_t row = blockIdx.y, tid = threadIdx.x;
+    if (sc_arg.plan[row].flag != 1)
         return;
-    __threadfence();
-    if (tid == 0) {
-        plan->ticket = 0;
+    stage_args(d_arg, sc_arg, row, s_args);
+    const mako_sample_desc& d = s_args.d;
+    const Scratch& sc = s_args.sc;
+    BigPlan* plan = sc.plan + row;
+    FinishLds L;
+    L.sm = &sm;
+    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
+    L.sortk = s_dyn64;
+    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
+    const uint32_t n0 = min(plan->n0, d.n_vocab), groups = min(plan->groups, min(kMaxGroups, sc.g_cap));
+    const double total64 = plan->total64;
+    __syncthreads();
+    if (tid == 0)
         plan->flag = 0;
-    }
-    sorted_tail(d, row, s_args.P, key0, idx0, n0, true, total64, MAKO_PATH_GENERAL, L, false, 0.0f, &sc.gt, t_row, groups);
+    sorted_tail(d, row, s_args.P, sc.key[0] + (size_t)row * sc.vpad, sc.idx[0] + (size_t)row * sc.vpad, n0, true, total64,
+                MAKO_PATH_GENERAL, L, false, 0.0f, &sc.gt, (size_t)row * sc.g_cap, groups);
 }
 
 
