@@ -931,6 +931,34 @@ __device__ __forceinline__ uint32_t uniform_u32(uint32_t v)
     return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
 }
 
+// Cross-lane moves on the VALU data path (DPP) instead of through the LDS crossbar: a dependent chain of six
+// of them costs tens of cycles, not hundreds.  Lanes without a source lane receive 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_zero(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+
+// Inclusive scan, in lane order, of the 64 lanes' maps under composition (cmax is not touched).
+__device__ __forceinline__ void wave_scan_maps(uint32_t& d0, uint32_t& d1)
+{
+    using seqfp::Step32;
+#define MAKO_SCAN_STEP(CTRL, ROW_MASK)                                                                               \
+    {                                                                                                                \
+        const Step32 t = Step32{dpp_or_zero<CTRL, ROW_MASK>(d0), dpp_or_zero<CTRL, ROW_MASK>(d1), 0u};               \
+        const Step32 r = seqfp::compose32(t, Step32{d0, d1, 0u}); /* earlier lanes first; {0, 0} is the identity */  \
+        d0 = r.d0;                                                                                                   \
+        d1 = r.d1;                                                                                                   \
+    }
+    MAKO_SCAN_STEP(0x111, 0xf) // row_shr:1
+    MAKO_SCAN_STEP(0x112, 0xf) // row_shr:2
+    MAKO_SCAN_STEP(0x114, 0xf) // row_shr:4
+    MAKO_SCAN_STEP(0x118, 0xf) // row_shr:8
+    MAKO_SCAN_STEP(0x142, 0xa) // row_bcast:15 into rows 1 and 3
+    MAKO_SCAN_STEP(0x143, 0xc) // row_bcast:31 into rows 2 and 3
+#undef MAKO_SCAN_STEP
+}
+
 __device__ __forceinline__ int exponent_of(float x)
 {
     uint32_t M;
@@ -965,15 +993,12 @@ __device__ __forceinline__ void load_span(const uint32_t* kf, uint32_t start, ui
 // Composition of the 64 lanes' maps in lane order; every lane receives the result.
 __device__ __forceinline__ seqfp::Step32 wave_compose_step32(seqfp::Step32 v)
 {
-    for (int o = 1; o < kWave; o <<= 1) {
-        seqfp::Step32 t;
-        t.d0 = __shfl_xor(v.d0, o);
-        t.d1 = __shfl_xor(v.d1, o);
-        t.cmax = __shfl_xor(v.cmax, o);
-        // the lane whose bit o is clear holds the earlier run
-        v = (lane_id() & o) ? seqfp::compose32(t, v) : seqfp::compose32(v, t);
-    }
-    return v;
+    wave_scan_maps(v.d0, v.d1);
+    seqfp::Step32 r;
+    r.d0 = (uint32_t)__builtin_amdgcn_readlane((int)v.d0, kWave - 1);
+    r.d1 = (uint32_t)__builtin_amdgcn_readlane((int)v.d1, kWave - 1);
+    r.cmax = __ockl_wfred_max_u32(v.cmax);
+    return r;
 }
 
 // The map of one span for the epoch with exponent eg (eg == 0: no usable guess, the map is marked unusable).
@@ -1013,9 +1038,26 @@ __device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk,
             const int eg = guess > 0 ? exponent_of((float)guess) : 0;
             const Step32 st = span_map(q[u], len[u], eg);
             if (lane_id() == 0 && g < groups) {
+                uint32_t third = st.cmax;
+                if (walk) {
+                    // group_sub_ok as one bound (lane 0 holds the group's first, largest weight): the state after
+                    // the group must be at least `third`, which keeps it inside the binade with room for one
+                    // more decrement and at or above that weight, so that nothing in the group stopped the walk
+                    uint32_t Mq;
+                    int eq;
+                    split(q[u][0], Mq, eq);
+                    const int dl = eg - eq;
+                    third = 1u;
+                    if (dl < 0)
+                        third = 1u << 31;
+                    else if (dl <= 25)
+                        third = max(1u, (uint32_t)(((unsigned long long)Mq + (1ull << dl) - 1ull) >> dl));
+                    if (eg > 1)
+                        third = max(third, min(st.cmax, 1u << 30) + (1u << 23) + 1u);
+                }
                 G.d0[g] = st.d0;
                 G.d1[g] = st.d1;
-                G.cmax[g] = st.cmax;
+                G.cmax[g] = third;
                 G.pack[g] = len[u] | ((uint32_t)eg << 16);
             }
         }
@@ -1088,6 +1130,7 @@ __device__ bool scan_span_walk(const uint32_t* kf, uint32_t start, uint32_t len,
         const uint32_t M = uniform_u32(Mv);
         const int e = (int)uniform_u32((uint32_t)ev);
         const bool live = lane_id() >= done && lane_id() < lanes;
+        MAKO_COUNT(28, 1);
         Step32 v = identity32();
         if (live) {
 #pragma unroll
@@ -1106,20 +1149,36 @@ __device__ bool scan_span_walk(const uint32_t* kf, uint32_t start, uint32_t len,
             if (e > 1)
                 need = max(need, min(v.cmax, 1u << 30) + (1u << 23) + 1u);
         }
-        for (int o = 1; o < kWave; o <<= 1) {
-            Step32 t;
-            t.d0 = __shfl_up(v.d0, o);
-            t.d1 = __shfl_up(v.d1, o);
-            t.cmax = 0;
-            if (lane_id() >= (uint32_t)o)
-                v = compose32(t, v);
-        }
+        wave_scan_maps(v.d0, v.d1);
         const uint32_t dd = (M & 1u) ? v.d1 : v.d0;
         const bool ok = dd <= M && M - dd >= need;
         const unsigned long long bad = __ballot(live && !ok);
         const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : lanes;
         if (f > done)
             r = join(uniform_u32((uint32_t)__shfl((int)(M - dd), (int)f - 1)), e);
+        if (f < lanes && f - done < 8u) {
+            // little progress: r is down among the weights themselves, where it changes binade every few entries;
+            // the rest of the span is cheaper entry by entry
+            const float nan = __uint_as_float(0x7fc00000u);
+            float rr = r; // NaN once the walk has stopped: no later comparison succeeds
+            uint32_t at = kNone;
+            MAKO_COUNT(29, lanes - f);
+            for (uint32_t l = f; l < lanes; ++l) {
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) {
+                    const float x = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), l));
+                    const bool stop = rr < x;
+                    at = stop ? beg + l * 4u + j : at;
+                    rr = stop ? nan : rr - x;
+                }
+                if (uniform_u32(at) != kNone) {
+                    pos = uniform_u32(at);
+                    return true;
+                }
+            }
+            r = rr;
+            return false;
+        }
         if (f < lanes) {
 #pragma unroll
             for (uint32_t j = 0; j < 4; ++j) {
@@ -1397,14 +1456,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 const bool live = lane_id() >= done && lane_id() < cnt;
                 const bool same = live && (pk_l >> 16) == (uint32_t)e;
                 Step32 v = lane_id() < done ? identity32() : (same ? Step32{d0_l, d1_l, 0u} : Step32{kSat, kSat, 0u});
-                for (int o = 1; o < kWave; o <<= 1) {
-                    Step32 t;
-                    t.d0 = __shfl_up(v.d0, o);
-                    t.d1 = __shfl_up(v.d1, o);
-                    t.cmax = 0;
-                    if (lane_id() >= (uint32_t)o)
-                        v = compose32(t, v);
-                }
+                wave_scan_maps(v.d0, v.d1);
                 const uint32_t after = M + ((M & 1u) ? v.d1 : v.d0); // < 2^29: no wrap
                 const bool ok = same && after + cm_l + 1u < (1u << 24); // group_add_ok for every group so far
                 const unsigned long long bad = __ballot(live && !ok);
@@ -1464,37 +1516,15 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             for (uint32_t base = 0; base < groups && !stopped; base += kWave) {
                 const uint32_t gl = min(base + lane_id(), groups - 1u);
                 const uint32_t pk_l = G.pack[gl], st_l = G.start[gl];
-                const int eg_l = (int)(pk_l >> 16);
-                const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], cm_l = G.cmax[gl];
-                // group_sub_ok as one bound: the state after the group must be at least need_l, which keeps it
-                // inside the binade with room for one more decrement and at or above the group's first weight
-                uint32_t need_l = 1u;
-                {
-                    uint32_t Mq;
-                    int eq;
-                    split(qat(st_l), Mq, eq);
-                    const int dl = eg_l - eq;
-                    if (dl < 0)
-                        need_l = 1u << 31;
-                    else if (dl <= 25)
-                        need_l = max(1u, (uint32_t)(((unsigned long long)Mq + (1ull << dl) - 1ull) >> dl));
-                    if (eg_l > 1)
-                        need_l = max(need_l, min(cm_l, 1u << 30) + (1u << 23) + 1u);
-                }
+                const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], need_l = G.cmax[gl]; // (the bound, see build_group_maps)
                 const uint32_t cnt = min((uint32_t)kWave, groups - base);
                 uint32_t done = 0;
                 while (done < cnt) {
+                    MAKO_COUNT(30, 1);
                     const bool live = lane_id() >= done && lane_id() < cnt;
                     const bool same = live && (pk_l >> 16) == (uint32_t)e;
                     Step32 v = lane_id() < done ? identity32() : (same ? Step32{d0_l, d1_l, 0u} : Step32{kSat, kSat, 0u});
-                    for (int o = 1; o < kWave; o <<= 1) {
-                        Step32 t;
-                        t.d0 = __shfl_up(v.d0, o);
-                        t.d1 = __shfl_up(v.d1, o);
-                        t.cmax = 0;
-                        if (lane_id() >= (uint32_t)o)
-                            v = compose32(t, v);
-                    }
+                    wave_scan_maps(v.d0, v.d1);
                     const uint32_t dd = (M & 1u) ? v.d1 : v.d0;
                     const bool ok = same && dd <= M && M - dd >= need_l; // group_sub_ok for every group so far
                     const unsigned long long bad = __ballot(live && !ok);
