@@ -20,6 +20,9 @@ FLAGS = [
     "-fno-gpu-flush-denormals-to-zero",
     "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # every device function inlined into its kernel: no call stack, so the finishing kernels need no
+    # scratch memory (kernels that use scratch run far fewer workgroups at a time on this chip)
+    "-mllvm", "-amdgpu-function-calls=false",
     "-Wall",
     "-Wno-unused-command-line-argument",
 ]

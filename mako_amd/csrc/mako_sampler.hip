@@ -347,6 +347,11 @@ int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t
 }
 
 #ifdef MAKO_TIMING
+int mako_sampler_debug_wg(unsigned long long* out8192)
+{
+    return hipMemcpyFromSymbol(out8192, HIP_SYMBOL(mako::g_mako_wg), 8192 * sizeof(unsigned long long)) == hipSuccess
+               ? MAKO_OK : MAKO_ERR_HIP;
+}
 // tuning builds only: copies the stage timestamps of row 0 (100 MHz wall clock) to the host
 int mako_sampler_debug_stamps(unsigned long long* out32)
 {

@@ -34,6 +34,20 @@ __device__ unsigned long long g_mako_stamp[32];
         if (threadIdx.x == 0 && blockIdx.y == 0)                                                                     \
             g_mako_stamp[i] = wall_clock64();                                                                        \
     } while (0)
+__device__ unsigned long long g_mako_wg[2][4096];
+struct WgTimer {
+    __device__ WgTimer()
+    {
+        if (threadIdx.x == 0)
+            g_mako_wg[0][(blockIdx.y * gridDim.x + blockIdx.x) & 4095] = wall_clock64();
+    }
+    __device__ ~WgTimer()
+    {
+        if (threadIdx.x == 0)
+            g_mako_wg[1][(blockIdx.y * gridDim.x + blockIdx.x) & 4095] = wall_clock64();
+    }
+};
+#define MAKO_WG_TIMER WgTimer wg_timer_
 #define MAKO_COUNT(i, v)                                                                                             \
     do {                                                                                                             \
         if (lane_id() == 0)                                                                                          \
@@ -42,6 +56,7 @@ __device__ unsigned long long g_mako_stamp[32];
 #else
 #define MAKO_STAMP(i) ((void)0)
 #define MAKO_COUNT(i, v) ((void)0)
+#define MAKO_WG_TIMER ((void)0)
 #endif
 
 constexpr uint32_t kSliceMax = 16384; // elements per slice: 16 per thread
@@ -2464,6 +2479,9 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     extern __shared__ unsigned long long s_dyn64[];
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
+#ifdef MAKO_TIMING_FINISH
+    MAKO_WG_TIMER;
+#endif
     {
         const mako_sampling_params P0 = d_arg.params[blockIdx.y];
         if (classify(P0) != kNucleus && (blockIdx.x + blockIdx.y) % slices != 0)
