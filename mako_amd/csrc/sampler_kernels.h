@@ -29,9 +29,15 @@ constexpr uint32_t kNone = 0xffffffffu;
 // Optional stage timestamps of row 0 (thread 0), for tuning builds only.
 #ifdef MAKO_TIMING
 __device__ unsigned long long g_mako_stamp[32];
+__shared__ uint32_t s_mako_row; // the row this workgroup serves (set by MAKO_ROW at kernel entry)
+#define MAKO_ROW(r)                                                                                                  \
+    do {                                                                                                             \
+        if (threadIdx.x == 0)                                                                                        \
+            s_mako_row = (r);                                                                                        \
+    } while (0)
 #define MAKO_STAMP(i)                                                                                                \
     do {                                                                                                             \
-        if (threadIdx.x == 0 && blockIdx.y == 0)                                                                     \
+        if (threadIdx.x == 0 && s_mako_row == 0)                                                                     \
             g_mako_stamp[i] = wall_clock64();                                                                        \
     } while (0)
 __device__ unsigned long long g_mako_wg[2][4096];
@@ -55,6 +61,7 @@ struct WgTimer {
     } while (0)
 #else
 #define MAKO_STAMP(i) ((void)0)
+#define MAKO_ROW(r) ((void)0)
 #define MAKO_COUNT(i, v) ((void)0)
 #define MAKO_WG_TIMER ((void)0)
 #endif
@@ -132,6 +139,13 @@ struct Scratch {
     uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong
     uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, ping-pong
     GroupTable gt;     // [max_rows][g_cap] each
+    // Work lists.  sort_kernel and tail_kernel are launched with one workgroup per POSSIBLE piece of work, but
+    // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
+    // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
+    // (finish_kernel and plan_kernel get the same effect from find_piece().)
+    uint32_t* work_n;      // [2] entries in work_sort, work_tail; zeroed by scan_kernel
+    uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel and plan_kernel
+    uint32_t* work_tail;   // [max_rows] row; appended by plan_kernel
     uint64_t vpad;
     uint32_t slices_cap;
     uint32_t g_cap;    // vpad / kGroup + kWorkers
@@ -317,15 +331,22 @@ struct Extras {
 // slot) and keeps it as an extra, and the logit's owner drops it (NaN).  The election of the first entry
 // makes the arrangement, and with it every later summation order, deterministic.
 // KH == 0: any history length; counts in LDS, every owner penalises its own logits.
-template <bool VEC, int KH>
+struct NoOverlap {
+    __device__ __forceinline__ void operator()() const {}
+};
+
+// `overlap` runs right after the slice's loads have been issued: work that does not depend on them hides
+// behind their latency.  It must be reached by the whole workgroup or by none of it.
+template <bool VEC, int KH, typename Overlap = NoOverlap>
 __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi,
                                                uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, bool pen,
-                                               uint32_t* s_cnt, float (&wv)[16], Extras<KH>& ex)
+                                               uint32_t* s_cnt, float (&wv)[16], Extras<KH>& ex, Overlap overlap = Overlap())
 {
     const uint32_t tid = threadIdx.x;
     const float nan = __uint_as_float(0x7fc00000u);
     RawSlice<VEC> raw;
     load_raw<VEC>(d, row, lo, hi, raw);
+    overlap();
 #pragma unroll
     for (int k = 0; k < (KH > 0 ? KH : 1); ++k) {
         ex.v[k] = nan;
@@ -437,6 +458,37 @@ struct ScanShared {
     uint32_t ci[kCap];
 };
 
+// Which piece of work does workgroup `piece` of finish_kernel (per_nucleus = slices, per_other = 1) or of plan_kernel
+// (1, 0) serve?  Rows are taken in order, each contributing per_nucleus pieces if it is a top_k == 0 row and
+// per_other otherwise.  Every workgroup works this out for itself from the rows' parameters (a few loads and one
+// scan).  Returns false when there is no such piece; all threads receive the same answer.
+__device__ bool find_piece(const mako_sample_desc& d, uint32_t piece, uint32_t per_nucleus, uint32_t per_other,
+                           uint32_t& row, uint32_t& sub, BlockScratch& bs)
+{
+    const uint32_t tid = threadIdx.x;
+    uint32_t before = 0;
+    for (uint32_t base = 0; base < d.n_rows; base += kThreads) {
+        const uint32_t r = base + tid;
+        uint32_t pieces = 0;
+        if (r < d.n_rows)
+            pieces = classify(d.params[r]) == kNucleus ? per_nucleus : per_other;
+        uint32_t tot;
+        const uint32_t at = before + block_excl_scan_u32(pieces, tot, bs);
+        if (piece >= at && piece < at + pieces)
+            bs.bcast = ((unsigned long long)r << 32) | (unsigned long long)(piece - at);
+        before += tot;
+        if (piece < before) { // uniform
+            __syncthreads();
+            const unsigned long long v = bs.bcast;
+            __syncthreads();
+            row = (uint32_t)(v >> 32);
+            sub = (uint32_t)v;
+            return true;
+        }
+    }
+    return false;
+}
+
 // The j-th largest of the wavefront's 64 keys (j >= 1): the largest v with at least j keys >= v, built
 // bit by bit from the top.  One vector compare per bit; the rest is scalar.
 __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
@@ -455,6 +507,7 @@ __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 template <bool VEC, int KH>
 __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scratch sc, uint32_t slice_len)
 {
+    MAKO_ROW(blockIdx.y);
     extern __shared__ uint32_t s_dyn[]; // [slice_len] token counts when the row has penalties
     __shared__ ScanShared sm;
 
@@ -470,6 +523,10 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
         sm.argidx = kNone;
         sm.emit_n = 0;
         sm.emit_flags = 0;
+        if (row == 0 && slice == 0) { // the lists finish_kernel and plan_kernel append to start empty
+            sc.work_n[0] = 0;
+            sc.work_n[1] = 0;
+        }
     }
     float wv[16];
     Extras<KH> ex;
@@ -2469,9 +2526,9 @@ __device__ float candidate_bound(const Scratch& sc, uint32_t row, uint32_t slice
     return q_bound;
 }
 
-// grid = (slices, rows), workgroup x of row r taking slice (x + r) % slices: consecutive workgroups go to different
-// XCDs, so this spreads both the slices of one row and the rows' slice-0 workgroups, which do all the work of a
-// top-k row, over the whole chip.  Only top_k == 0 rows use more than their slice-0 workgroup.
+// grid = (slices, rows) workgroups, of which workgroup i serves the i-th piece of work in row order: one piece per
+// row, and one per slice for top_k == 0 rows (find_piece).  The busy workgroups are then the first ones dispatched
+// and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
 template <bool VEC, int KH>
 __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices,
                                                           uint32_t slice_len)
@@ -2482,12 +2539,12 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
 #ifdef MAKO_TIMING_FINISH
     MAKO_WG_TIMER;
 #endif
-    {
-        const mako_sampling_params P0 = d_arg.params[blockIdx.y];
-        if (classify(P0) != kNucleus && (blockIdx.x + blockIdx.y) % slices != 0)
-            return;
-    }
-    stage_args(d_arg, sc_arg, blockIdx.y, s_args);
+    uint32_t row, slice;
+    if (!find_piece(d_arg, blockIdx.y * gridDim.x + blockIdx.x, slices, 1u, row, slice, sm.bs))
+        return;
+    const uint32_t tid = threadIdx.x;
+    MAKO_ROW(row);
+    stage_args(d_arg, sc_arg, row, s_args);
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
     FinishLds L;
@@ -2495,7 +2552,6 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
     L.sortk = s_dyn64;                                             // 32 KB
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);    // next 16 KB
-    const uint32_t row = blockIdx.y, slice = (blockIdx.x + blockIdx.y) % slices, tid = threadIdx.x;
     const mako_sampling_params& P = s_args.P;
     const RowClass cls = classify(P);
     MAKO_STAMP(0);
@@ -2532,6 +2588,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
             sc.plan[row].total64 = (double)m; // carries the row maximum and its first index to the whole-row path
             sc.plan[row].n0 = argidx;
             sc.plan[row].flag = 2;
+            sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
         }
         return;
     }
@@ -2558,6 +2615,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
             sc.plan[row].total64 = (double)m;
             sc.plan[row].n0 = argidx;
             sc.plan[row].flag = 2;
+            sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
         }
         return;
     }
@@ -2568,7 +2626,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L); // sampler.cpp:40-43
 }
 
-// grid = (1, rows).  top_k == 0 rows only: the row's exact total, candidate count and weight histogram are summed
+// grid = (1, rows), workgroup i serving the i-th top_k == 0 row (find_piece): the row's exact total, candidate count and weight histogram are summed
 // over its slices and the row is planned: handed to sort_kernel's workers, or, when the nucleus is narrow enough to
 // end inside the candidate lists, to its worker 0 alone.
 __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices)
@@ -2576,12 +2634,11 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     extern __shared__ unsigned long long s_dyn64[];
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
-    const uint32_t row = blockIdx.y, tid = threadIdx.x;
-    {
-        const mako_sampling_params P0 = d_arg.params[row];
-        if (classify(P0) != kNucleus)
-            return;
-    }
+    uint32_t row, sub;
+    if (!find_piece(d_arg, blockIdx.y, 1u, 0u, row, sub, sm.bs))
+        return;
+    const uint32_t tid = threadIdx.x;
+    MAKO_ROW(row);
     stage_args(d_arg, sc_arg, row, s_args);
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
@@ -2645,10 +2702,18 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         sc.plan[row].thr = thr_bits;
         sc.plan[row].flag = !fits ? 2 : (narrow ? 3 : 1);
     }
+    // the row's pieces of work for sort_kernel (all workers, or worker 0 alone) and tail_kernel
+    const uint32_t pieces = (fits && !narrow) ? kWorkers : 1u;
+    if (tid == 0)
+        sm.flag = atomicAdd(&sc.work_n[0], pieces);
+    __syncthreads();
+    if (tid < pieces)
+        sc.work_sort[sm.flag + tid] = (row << 8) | tid;
+    if (tid == 0 && fits && !narrow)
+        sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
 }
 
-// grid = (kWorkers, rows); a row's workers spread over the XCDs, and worker 0 (which alone serves the whole-row
-// path) sits on a different XCD from row to row.  Rows without a work order cost one load.  Worker w gathers its range of weights from
+// grid = (kWorkers, rows) workgroups, of which workgroup i serves entry i of the work list.  Worker w gathers its range of weights from
 // the row's bits(q) array, sorts it and stores it at its place in the row's sorted list; the last worker to
 // finish cuts the nucleus and draws.
 __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices)
@@ -2656,9 +2721,14 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     extern __shared__ unsigned long long s_dyn64[];
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
-    const uint32_t row = blockIdx.y, w = (blockIdx.x + blockIdx.y) % kWorkers, tid = threadIdx.x;
+    const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
+    if (piece >= sc_arg.work_n[0])
+        return;
+    const uint32_t item = sc_arg.work_sort[piece];
+    const uint32_t row = item >> 8, w = item & 255u, tid = threadIdx.x;
+    MAKO_ROW(row);
     const uint32_t flag = sc_arg.plan[row].flag;
-    if (flag == 0 || (flag != 1 && w != 0))
+    if (flag == 0 || (flag != 1 && w != 0)) // (never: the list holds exactly the flagged rows' pieces)
         return;
     stage_args(d_arg, sc_arg, row, s_args);
     const mako_sample_desc& d = s_args.d;
@@ -2744,7 +2814,10 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     extern __shared__ unsigned long long s_dyn64[];
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
-    const uint32_t row = blockIdx.y, tid = threadIdx.x;
+    if (blockIdx.y >= sc_arg.work_n[1])
+        return;
+    const uint32_t row = sc_arg.work_tail[blockIdx.y], tid = threadIdx.x;
+    MAKO_ROW(row);
     if (sc_arg.plan[row].flag != 1)
         return;
     stage_args(d_arg, sc_arg, row, s_args);
