@@ -226,6 +226,69 @@ def test_config5_masks(gpu_ctx):
         assert_parity(gpu_ctx, workloads.config5(rows=32, density=density))
 
 
+def test_wide_nucleus_walk_depths(gpu_ctx):
+    """top_k = 0 rows whose nuclei hold tens of thousands of tokens, drawn at u from 0 to 1 - 2^-24: the walk
+    ends anywhere between the first candidate and the last, crossing many binades of r on the way."""
+    rng = np.random.default_rng(4242)
+    us = np.array([0.0, 1e-7, 0.03, 0.5, 0.9, 0.999, 0.99999, 1.0 - 2.0**-24], np.float32)
+    b = 2 * len(us)
+    logits = (rng.standard_normal((b, 129280)) * 3).astype(np.float32)
+    p = api.make_params(b, 1.0, 0, 0.95)
+    p["temperature"] = np.repeat(np.array([1.0, 1.2], np.float32), len(us))
+    p["top_p"] = rng.choice(np.array([0.9, 0.99, 0.9999], np.float32), b)
+    w = dict(name="walk_depths", logits=logits, params=p, u=np.tile(us, 2))
+    g = assert_parity(gpu_ctx, w, cap=1024)
+    _say("walk depths: nuclei %s" % g["n_cand"].tolist())
+    assert g["n_cand"].min() > 5000
+
+
+def test_tied_wide_nucleus(gpu_ctx):
+    """Logits on a grid of 1/8: every weight is shared by hundreds of tokens, so candidates tie in q and the order
+    inside a tie is by token id.  The workers' counting sort gives such rows to the stable radix sort."""
+    rng = np.random.default_rng(4343)
+    b = 6
+    logits = (np.round(rng.standard_normal((b, 129280)) * 3 * 8) / 8).astype(np.float32)
+    p = api.make_params(b, 1.0, 0, 0.95)
+    p["top_p"] = np.array([0.5, 0.9, 0.95, 0.99, 0.999, 0.95], np.float32)
+    p["temperature"][5] = 0.4
+    w = dict(name="tied_wide", logits=logits, params=p, u=rng.random(b).astype(np.float32))
+    assert_parity(gpu_ctx, w, cap=2048)
+
+
+def test_narrow_nucleus_inside_one_slice(gpu_ctx):
+    """A nucleus of ~200 tokens that all live in one 16K-token slice, 14 to each wavefront of the scan: the slice
+    keeps only those at or above the smallest of the wavefronts' 8th largest, the certificate of the candidate
+    list fails, and the row is rebuilt from its weight array."""
+    rng = np.random.default_rng(4444)
+    b, v = 4, 129280
+    slice_len = 16160  # ceil(129280 / 8)
+    logits = (rng.standard_normal((b, v)) * 0.5).astype(np.float32)
+    for r in range(b):
+        for wave in range(16):
+            lanes = rng.choice(64, 14, replace=False)
+            hot = slice_len + 4 * (64 * wave + lanes)  # element 0 of 14 threads of this wave, slice 1
+            logits[r, hot] += np.float32(12.0) + rng.random(14).astype(np.float32)
+    p = api.make_params(b, 1.0, 0, 0.9)
+    p["top_p"] = np.array([0.5, 0.9, 0.97, 0.99], np.float32)
+    w = dict(name="one_slice", logits=logits, params=p, u=rng.random(b).astype(np.float32))
+    g = assert_parity(gpu_ctx, w, cap=512)
+    _say("one-slice nuclei: %s paths %s" % (g["n_cand"].tolist(), g["path"].tolist()))
+    assert (g["path"] == api.PATH_GENERAL).any() and (g["path"] == api.PATH_NUCLEUS).any()
+
+
+def test_more_rows_than_threads():
+    """1100 rows in one batch: the per-workgroup search for its piece of work loops over the rows."""
+    ctx = api.SamplerContext(max_rows=1100, max_vocab=320, max_hist=0)
+    try:
+        rng = np.random.default_rng(4545)
+        w = _random_case(rng, 320, 1100)
+        w.pop("hist", None)
+        w.pop("hist_len", None)
+        assert_parity(ctx, w, cap=64)
+    finally:
+        ctx.close()
+
+
 def test_full_size_properties(gpu_ctx):
     """Size-independent properties at the full benchmark sizes (B=256, V=151552), no oracle:
     ids inside the allowed set, greedy rows equal numpy's first argmax, u=0 returns the most likely candidate,
