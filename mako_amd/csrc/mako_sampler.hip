@@ -98,10 +98,12 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap));
     MAKO_HIP(ctx, dev_alloc(&sc.part_sum, (size_t)max_rows * mako::kMaxSlices));
     MAKO_HIP(ctx, dev_alloc(&sc.part_n, (size_t)max_rows * mako::kMaxSlices));
-    MAKO_HIP(ctx, dev_alloc(&sc.binc, (size_t)max_rows * sc.slices_cap * mako::kBins));
+    MAKO_HIP(ctx, dev_alloc(&sc.binc, (size_t)max_rows * mako::kBins));
+    MAKO_HIP(ctx, hipMemset(sc.binc, 0, (size_t)max_rows * mako::kBins * sizeof(uint32_t)));
     MAKO_HIP(ctx, dev_alloc(&sc.plan, (size_t)max_rows));
     MAKO_HIP(ctx, hipMemset(sc.plan, 0, (size_t)max_rows * sizeof(mako::BigPlan)));
-    MAKO_HIP(ctx, dev_alloc(&sc.bins, (size_t)max_rows * sc.slices_cap * mako::kBins));
+    MAKO_HIP(ctx, dev_alloc(&sc.bins, (size_t)max_rows * mako::kBins));
+    MAKO_HIP(ctx, hipMemset(sc.bins, 0, (size_t)max_rows * mako::kBins * sizeof(unsigned long long)));
     MAKO_HIP(ctx, dev_alloc(&sc.wbuf, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.cnt, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.key[0], rv));

@@ -129,9 +129,10 @@ struct Scratch {
     uint32_t* cand_i;  // [max_rows][slices_cap][kCap] their token ids
     double* part_sum;  // [max_rows][kMaxSlices] exact fp64 sum of q over the slice (top_k == 0 rows)
     uint32_t* part_n;  // [max_rows][kMaxSlices] candidates (q > 0, q >= min_p) in the slice
-    uint32_t* binc;    // [max_rows][slices_cap][kBins] candidates per weight bin of each slice (top_k == 0 rows)
+    uint32_t* binc;    // [max_rows][kBins] candidates per weight bin (top_k == 0 rows); the slices add their
+                       // counts with atomics, plan_kernel reads the row's bins and leaves them zero
     BigPlan* plan;     // [max_rows]; flag zero between calls
-    unsigned long long* bins; // [max_rows][slices_cap][kBins] sum of their 24-bit significands: a bin's exact
+    unsigned long long* bins; // [max_rows][kBins] sum of the bin's 24-bit significands, likewise: a bin's exact
                               // mass is bins * 2^(e - 150), e being the bin's exponent
     float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path; top_k == 0 rows keep
                        // bits(q) of every logit here instead (0 where q is not a candidate)
@@ -2434,13 +2435,14 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
         }
     __syncthreads();
     MAKO_STAMP(27);
-    // the slice's histogram goes to its own place: no atomics, nothing to clear afterwards
-    uint32_t* binc = sc.binc + ((size_t)row * sc.slices_cap + slice) * kBins;
-    unsigned long long* bins = sc.bins + ((size_t)row * sc.slices_cap + slice) * kBins;
-    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads) {
-        binc[b] = hist[b];
-        bins[b] = hsum[b];
-    }
+    // the slice's non-empty bins are added to the row's histogram (a few hundred atomics per slice, none waited for)
+    uint32_t* binc = sc.binc + (size_t)row * kBins;
+    unsigned long long* bins = sc.bins + (size_t)row * kBins;
+    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads)
+        if (hist[b]) {
+            atomicAdd(&binc[b], hist[b]);
+            atomicAdd(&bins[b], hsum[b]);
+        }
 }
 
 // Kernel arguments that are handed on by reference to out-of-line device functions would be spilled to scratch
@@ -2649,36 +2651,36 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     L.sortk = s_dyn64;
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
     MAKO_STAMP(2);
-    // this thread's two bins of the histogram, every slice's loads in flight together
+    // this thread's two bins of the row's histogram (left zero for the next batch), the slices' exact sums in order
+    uint32_t* binc = sc.binc + (size_t)row * kBins;
+    unsigned long long* bins = sc.bins + (size_t)row * kBins;
+    const uint32_t bin_c0 = binc[kBins - 1u - 2u * tid], bin_c1 = binc[kBins - 2u - 2u * tid];
+    const unsigned long long bin_s0 = bins[kBins - 1u - 2u * tid], bin_s1 = bins[kBins - 2u - 2u * tid];
     double row_total = 0;
-    uint32_t row_n0 = 0, bin_c0 = 0, bin_c1 = 0;
-    unsigned long long bin_s0 = 0, bin_s1 = 0;
+    uint32_t row_n0 = 0;
     for (uint32_t s0 = 0; s0 < slices; s0 += 8u) {
-        uint32_t c0[8], c1[8], pn[8];
-        unsigned long long h0[8], h1[8];
+        uint32_t pn[8];
         double ps[8];
 #pragma unroll
         for (uint32_t u = 0; u < 8; ++u) {
             const uint32_t sl = min(s0 + u, slices - 1u);
-            const uint32_t* binc = sc.binc + ((size_t)row * sc.slices_cap + sl) * kBins;
-            const unsigned long long* bins = sc.bins + ((size_t)row * sc.slices_cap + sl) * kBins;
-            c0[u] = binc[kBins - 1u - 2u * tid];
-            c1[u] = binc[kBins - 2u - 2u * tid];
-            h0[u] = bins[kBins - 1u - 2u * tid];
-            h1[u] = bins[kBins - 2u - 2u * tid];
             ps[u] = sc.part_sum[(size_t)row * kMaxSlices + sl];
             pn[u] = sc.part_n[(size_t)row * kMaxSlices + sl];
         }
 #pragma unroll
         for (uint32_t u = 0; u < 8; ++u)
             if (s0 + u < slices) {
-                bin_c0 += c0[u];
-                bin_c1 += c1[u];
-                bin_s0 += h0[u];
-                bin_s1 += h1[u];
                 row_total += ps[u];
                 row_n0 += pn[u];
             }
+    }
+    if (bin_c0) {
+        binc[kBins - 1u - 2u * tid] = 0;
+        bins[kBins - 1u - 2u * tid] = 0;
+    }
+    if (bin_c1) {
+        binc[kBins - 2u - 2u * tid] = 0;
+        bins[kBins - 2u - 2u * tid] = 0;
     }
     float m;
     uint32_t argidx, n_cands, any_overflow;
