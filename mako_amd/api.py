@@ -152,8 +152,8 @@ class SamplerContext:
             raise MakoError("mako_sampler_set_profile: %d %s" % (rc, self.last_error()))
 
     def kernel_times_ms(self):
-        """(scan, finish, plan, sort, tail) kernel milliseconds of the last batch sampled while profiling was on."""
-        out = (C.c_float * 5)()
+        """(scan, finish, plan, partition, sort, tail) kernel milliseconds of the last batch sampled while profiling was on."""
+        out = (C.c_float * 6)()
         rc = self.lib.mako_sampler_kernel_times(self.ptr, out)
         if rc != MAKO_OK:
             raise MakoError("mako_sampler_kernel_times: %d %s" % (rc, self.last_error()))

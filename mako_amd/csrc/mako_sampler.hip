@@ -33,7 +33,7 @@ struct mako_sampler_ctx {
     uint8_t* st_acc = nullptr;
     std::string err = "";
     bool profile = false, profiled = false;
-    hipEvent_t ev[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    hipEvent_t ev[MAKO_SAMPLER_KERNELS + 1] = {};
 };
 
 namespace {
@@ -119,6 +119,7 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.gt.cmax, rg));
     MAKO_HIP(ctx, dev_alloc(&sc.gt.start, rg));
     MAKO_HIP(ctx, dev_alloc(&sc.gt.pack, rg));
+    MAKO_HIP(ctx, dev_alloc(&sc.bin_worker, (size_t)max_rows * mako::kBins));
     MAKO_HIP(ctx, dev_alloc(&sc.work_n, 2));
     MAKO_HIP(ctx, hipMemset(sc.work_n, 0, 2 * sizeof(uint32_t)));
     MAKO_HIP(ctx, dev_alloc(&sc.work_sort, (size_t)max_rows * mako::kWorkers));
@@ -146,7 +147,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack,
+    void* ptrs[] = {sc.bin_worker, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack,
                     sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.binc, sc.bins, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
@@ -180,8 +181,8 @@ int mako_sampler_kernel_times(mako_sampler_ctx* ctx, float* out_ms)
         return MAKO_ERR_INVALID_ARG;
     if (!ctx->profiled)
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: no profiled batch to report");
-    MAKO_HIP(ctx, hipEventSynchronize(ctx->ev[5]));
-    for (int i = 0; i < 5; ++i)
+    MAKO_HIP(ctx, hipEventSynchronize(ctx->ev[MAKO_SAMPLER_KERNELS]));
+    for (int i = 0; i < MAKO_SAMPLER_KERNELS; ++i)
         MAKO_HIP(ctx, hipEventElapsedTime(&out_ms[i], ctx->ev[i], ctx->ev[i + 1]));
     return MAKO_OK;
 }
@@ -255,11 +256,13 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  Other rows cost a load.
     hipLaunchKernelGGL(mako::plan_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc, slices);
     MAKO_MARK(3);
+    hipLaunchKernelGGL(mako::partition_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), 0, st, d, ctx->sc);
+    MAKO_MARK(4);
     hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d, ctx->sc,
                        slices);
-    MAKO_MARK(4);
-    hipLaunchKernelGGL(mako::tail_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc);
     MAKO_MARK(5);
+    hipLaunchKernelGGL(mako::tail_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc);
+    MAKO_MARK(6);
 #undef MAKO_MARK
     ctx->profiled = prof;
     MAKO_HIP(ctx, hipGetLastError());

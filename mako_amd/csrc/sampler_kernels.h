@@ -110,6 +110,7 @@ struct BigPlan {
     uint32_t off[kWorkers];    // and writes them from position off[w] of the sorted list
     uint32_t cnt[kWorkers];
     uint32_t gbase[kWorkers];  // first group of worker w
+    uint32_t cursor[kWorkers]; // entries partition_kernel has handed to worker w so far
     double mass[kWorkers];     // sum of the weights above worker w's range
 };
 
@@ -137,8 +138,10 @@ struct Scratch {
     float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path; top_k == 0 rows keep
                        // bits(q) of every logit here instead (0 where q is not a candidate)
     uint32_t* cnt;     // [max_rows][vpad] token counts; all zero between calls
-    uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong
-    uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, ping-pong
+    uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong; [1] also takes the workers' unsorted
+                       // shares (bits(q)) from partition_kernel
+    uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, likewise
+    uint8_t* bin_worker; // [max_rows][kBins] the worker that takes the weights of each histogram bin (0xff: none)
     GroupTable gt;     // [max_rows][g_cap] each
     // Work lists.  sort_kernel and tail_kernel are launched with one workgroup per POSSIBLE piece of work, but
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
@@ -1687,8 +1690,8 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
 // Thread t brings the counts (c0, c1) and significand sums (s0, s1) of bins kBins-1-2t and kBins-2-2t.
 // Returns n0, the number of weights to sort; the plan is written to `plan` (flag left untouched).
 __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, uint32_t c0, uint32_t c1,
-                                 unsigned long long s0, unsigned long long s1, BigPlan* plan, const FinishLds& L,
-                                 uint32_t& thr_bits)
+                                 unsigned long long s0, unsigned long long s1, BigPlan* plan, uint8_t* bin_worker,
+                                 const FinishLds& L, uint32_t& thr_bits)
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
@@ -1758,7 +1761,10 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         plan->mass[wk0] = incl - m0 - m1;
     if (wk1 != kNone && w_hi[wk1] == b1)
         plan->mass[wk1] = incl - m1;
+    bin_worker[b0] = (uint8_t)wk0; // (kNone -> 0xff)
+    bin_worker[b1] = (uint8_t)wk1;
     if (tid < kWorkers) {
+        plan->cursor[tid] = 0;
         plan->key_lo[tid] = w_lo[tid] << 19;
         plan->key_hi[tid] = (w_hi[tid] + 1u) << 19;
         plan->off[tid] = w_cnt[tid] ? w_off[tid] : 0u;
@@ -1888,6 +1894,9 @@ __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t*
     }
 }
 
+__device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, uint32_t* kout, uint32_t* iout,
+                                unsigned long long* dyn, FinishShared& sm);
+
 // Worker's sort, LDS-resident: the weights of the row with key_lo <= bits(q) < key_hi (at most kSegCap of them)
 // are collected from the row's bits(q) array in one sweep, dropped into kFine value buckets (descending), and
 // every entry then finds its place by counting the entries of its own bucket that precede it under
@@ -1957,9 +1966,20 @@ __device__ bool lds_sort_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, 
         }
     }
     __syncthreads();
-    const uint32_t n = sm.ticket;
-    if (n != cnt) // (cannot happen: the plan counted the same array)
+    if (sm.ticket != cnt) // (cannot happen: the plan counted the same array)
         return false;
+    return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm);
+}
+
+// Second half of the workers' sort: the n entries (bits(q), idx) in LDS at A, all with key_lo <= bits(q) < key_hi,
+// go to kout / iout ordered by (q desc, idx asc).  hist must be zero and sm.flag 0 on entry.
+__device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, uint32_t* kout, uint32_t* iout,
+                                unsigned long long* dyn, FinishShared& sm)
+{
+    uint2* A = reinterpret_cast<uint2*>(dyn);
+    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap);
+    const uint32_t tid = threadIdx.x;
     // 2. buckets by value, heaviest first
     const uint32_t range = key_hi - key_lo; // > 0
     const uint32_t shift = range > kFine ? 32u - (uint32_t)__clz((range - 1u) >> 11) : 0u; // (range - 1) >> shift < kFine
@@ -2014,6 +2034,37 @@ __device__ bool lds_sort_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, 
     }
     __syncthreads();
     return true;
+}
+
+// The worker's share as partition_kernel left it (cnt <= kSegCap entries, bits(q) in ks and token ids in is, any
+// order), sorted into kout / iout.
+__device__ bool lds_sort_staged(const uint32_t* ks, const uint32_t* is, uint32_t key_lo, uint32_t key_hi, uint32_t cnt,
+                                uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm)
+{
+    uint2* A = reinterpret_cast<uint2*>(dyn);
+    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap);
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t b = tid; b <= kFine; b += kThreads)
+        hist[b] = 0;
+    if (tid == 0)
+        sm.flag = 0;
+    constexpr uint32_t kPer = kSegCap / kThreads;
+    uint32_t k[kPer], id[kPer];
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t) { // (all loads first, from clamped positions)
+        const uint32_t e = min(t * kThreads + tid, cnt - 1u);
+        k[t] = ks[e];
+        id[t] = is[e];
+    }
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t) {
+        const uint32_t e = t * kThreads + tid;
+        if (e < cnt)
+            A[e] = make_uint2(min(max(k[t], key_lo), key_hi - 1u), id[t]); // (clamped: a bucket index is always valid)
+    }
+    __syncthreads();
+    return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm);
 }
 
 // Group records of a worker's sorted range (cnt entries from position off of the list kf): fp64 sums, and the
@@ -2691,7 +2742,7 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         return;
     }
     uint32_t thr_bits = 0;
-    const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, L, thr_bits);
+    const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, sc.bin_worker + (size_t)row * kBins, L, thr_bits);
     MAKO_STAMP(16);
     const bool narrow = !d.draft && n0 <= kSmall && !any_overflow && n_cands <= kSortMax;
     // (a list too long for the workers' group records goes to the whole-row path)
@@ -2713,6 +2764,81 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         sc.work_sort[sm.flag + tid] = (row << 8) | tid;
     if (tid == 0 && fits && !narrow)
         sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
+}
+
+// grid = (kWorkers, rows) workgroups over the same work list as sort_kernel; only planned wide rows do anything.
+// Piece c of a row reads the c-th part of the row's bits(q) array once and hands every weight the plan wants to
+// the worker that will sort it: positions inside the workgroup from LDS counters, one global atomic per worker to
+// reserve the workgroup's run in that worker's share.  (Without this step each of the 32 workers would sweep the
+// whole row to find its own weights.)
+__global__ __launch_bounds__(kThreads) void partition_kernel(mako_sample_desc d, Scratch sc)
+{
+    __shared__ uint32_t s_count[kWorkers], s_base[kWorkers], s_off[kWorkers], s_cnt[kWorkers];
+    __shared__ uint32_t s_table[kBins / 4];
+    const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
+    if (piece >= sc.work_n[0])
+        return;
+    const uint32_t item = sc.work_sort[piece];
+    const uint32_t row = item >> 8, c = item & 255u, tid = threadIdx.x;
+    MAKO_ROW(row);
+    BigPlan* plan = sc.plan + row;
+    if (plan->flag != 1)
+        return;
+    const uint32_t V = d.n_vocab;
+    const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
+    uint32_t* kstage = sc.key[1] + (size_t)row * sc.vpad;
+    uint32_t* istage = sc.idx[1] + (size_t)row * sc.vpad;
+    const uint32_t part = (((V + kWorkers - 1u) / kWorkers) + 3u) & ~3u; // entries per piece, a multiple of 4
+    const uint32_t lo = min(V, c * part), hi = min(V, lo + part);
+    // the first loads go out before anything else
+    uint4 x = make_uint4(0, 0, 0, 0);
+    {
+        const uint32_t i = lo + tid * 4u;
+        if (i < hi)
+            x = *reinterpret_cast<const uint4*>(qk + i); // (the array is padded to a multiple of 1024 entries past V)
+    }
+    if (tid < kBins / 4)
+        s_table[tid] = reinterpret_cast<const uint32_t*>(sc.bin_worker + (size_t)row * kBins)[tid];
+    if (tid < kWorkers) {
+        s_count[tid] = 0;
+        s_off[tid] = plan->off[tid];
+        s_cnt[tid] = plan->cnt[tid];
+    }
+    __syncthreads();
+    const uint8_t* table = reinterpret_cast<const uint8_t*>(s_table);
+    for (uint32_t base = lo; base < hi; base += kThreads * 4u) {
+        const uint32_t i = base + tid * 4u;
+        if (base != lo) {
+            x = make_uint4(0, 0, 0, 0);
+            if (i < hi)
+                x = *reinterpret_cast<const uint4*>(qk + i);
+        }
+        const uint32_t k[4] = {x.x, x.y, x.z, x.w};
+        uint32_t dest[4], lpos[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            dest[j] = (i + j < hi && k[j] != 0) ? table[min(k[j] >> 19, kBins - 1u)] : 0xffu;
+            lpos[j] = 0;
+            if (dest[j] < kWorkers)
+                lpos[j] = atomicAdd(&s_count[dest[j]], 1u);
+        }
+        __syncthreads();
+        if (tid < kWorkers) {
+            s_base[tid] = s_count[tid] ? atomicAdd(&plan->cursor[tid], s_count[tid]) : 0u;
+            s_count[tid] = 0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (dest[j] < kWorkers) {
+                const uint32_t at = s_base[dest[j]] + lpos[j];
+                if (at < s_cnt[dest[j]] && s_off[dest[j]] + at < V) { // (always, when the plan is sound)
+                    kstage[s_off[dest[j]] + at] = k[j];
+                    istage[s_off[dest[j]] + at] = i + j;
+                }
+            }
+        __syncthreads();
+    }
 }
 
 // grid = (kWorkers, rows) workgroups, of which workgroup i serves entry i of the work list.  Worker w gathers its range of weights from
@@ -2799,7 +2925,7 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     if (cnt) {
         const uint32_t key_lo = plan->key_lo[w], key_hi = plan->key_hi[w];
         MAKO_STAMP(10);
-        if (!lds_sort_range(qk, d.n_vocab, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm)) {
+        if (cnt > kSegCap || !lds_sort_staged(key1 + off, idx1 + off, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm)) {
             MAKO_COUNT(23, threadIdx.x == 0 ? 1 : 0);
             gather_range(qk, d.n_vocab, key_lo, key_hi, key0 + off, idx0 + off, cnt, sm);
             sort_segment(key0 + off, idx0 + off, key1 + off, idx1 + off, cnt, L);
