@@ -119,6 +119,7 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.gt.cmax, rg));
     MAKO_HIP(ctx, dev_alloc(&sc.gt.start, rg));
     MAKO_HIP(ctx, dev_alloc(&sc.gt.pack, rg));
+    MAKO_HIP(ctx, dev_alloc(&sc.gt.quarters, rg * 4));
     MAKO_HIP(ctx, dev_alloc(&sc.bin_worker, (size_t)max_rows * mako::kBins));
     MAKO_HIP(ctx, dev_alloc(&sc.work_n, 2));
     MAKO_HIP(ctx, hipMemset(sc.work_n, 0, 2 * sizeof(uint32_t)));
@@ -147,7 +148,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {sc.bin_worker, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack,
+    void* ptrs[] = {sc.bin_worker, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
                     sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.binc, sc.bins, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,

@@ -121,7 +121,8 @@ struct GroupTable {
     uint32_t* d1;
     uint32_t* cmax;
     uint32_t* start; // first entry of the group in the sorted list
-    uint32_t* pack;  // entries | guessed exponent << 16
+    uint32_t* pack;  // entries | guessed exponent << 16 | kHasQuarters if `quarters` holds records for the group
+    uint4* quarters; // [4] per group: the maps of the group's four quarters (see build_quarters)
 };
 
 struct Scratch {
@@ -235,18 +236,27 @@ __device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row
     const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
     const float nan = __uint_as_float(0x7fc00000u);
     if (VEC) {
+        // all four loads go out back to back, from clamped addresses and without a branch between them (a branch
+        // would make the compiler wait for each load before the next); what lies past the slice is dropped after
+        uint32_t at[4];
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k) {
             const uint32_t i = lo + k * 4096u + tid * 4u;
-            r.bits[k] = 0xfu;
-            if (i < hi) { // hi - lo is a multiple of 4 in this mode
-                r.v[k] = *reinterpret_cast<const float4*>(lrow + i);
-                if (mrow)
-                    r.bits[k] = mrow[i >> 5] >> (i & 31u);
-            } else {
-                r.v[k] = make_float4(nan, nan, nan, nan);
-            }
+            at[k] = i < hi ? i : hi - 4u; // hi - lo is a positive multiple of 4 in this mode
+            r.v[k] = *reinterpret_cast<const float4*>(lrow + at[k]);
         }
+        if (mrow) {
+#pragma unroll
+            for (uint32_t k = 0; k < 4; ++k)
+                r.bits[k] = mrow[at[k] >> 5] >> (at[k] & 31u);
+        }
+        if (!mrow) {
+#pragma unroll
+            for (uint32_t k = 0; k < 4; ++k)
+                r.bits[k] = 0xfu;
+        }
+        // (finish_slice() replaces what was read past the slice: nothing here touches the loaded values, so the
+        // loads stay in flight while the caller goes on)
     } else {
         float* f = reinterpret_cast<float*>(r.v);
         uint32_t allowed = 0xffffu;
@@ -272,12 +282,14 @@ __device__ __forceinline__ void finish_slice(const RawSlice<VEC>& r, uint32_t lo
 {
     const uint32_t tid = threadIdx.x;
     if (VEC) {
+        const float nan = __uint_as_float(0x7fc00000u);
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k) {
-            wv[4 * k + 0] = (r.bits[k] & 1u) ? r.v[k].x : -INFINITY;
-            wv[4 * k + 1] = (r.bits[k] & 2u) ? r.v[k].y : -INFINITY;
-            wv[4 * k + 2] = (r.bits[k] & 4u) ? r.v[k].z : -INFINITY;
-            wv[4 * k + 3] = (r.bits[k] & 8u) ? r.v[k].w : -INFINITY;
+            const bool inside = lo + k * 4096u + tid * 4u < hi;
+            wv[4 * k + 0] = !inside ? nan : ((r.bits[k] & 1u) ? r.v[k].x : -INFINITY);
+            wv[4 * k + 1] = !inside ? nan : ((r.bits[k] & 2u) ? r.v[k].y : -INFINITY);
+            wv[4 * k + 2] = !inside ? nan : ((r.bits[k] & 4u) ? r.v[k].z : -INFINITY);
+            wv[4 * k + 3] = !inside ? nan : ((r.bits[k] & 8u) ? r.v[k].w : -INFINITY);
         }
     } else {
         const float* f = reinterpret_cast<const float*>(r.v);
@@ -372,26 +384,41 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
     uint32_t tok[KH > 0 ? KH : 1], cnt[KH > 0 ? KH : 1];
     float rawv[KH > 0 ? KH : 1];
+    // (loads from clamped positions, issued in two groups without branches between them; what was not wanted is
+    // dropped afterwards: a branch around each load would make every load wait for the one before)
+    bool have[KH > 0 ? KH : 1];
 #pragma unroll
     for (int k = 0; k < KH; ++k) {
         const uint32_t h = tid + (uint32_t)k * kThreads;
-        tok[k] = kNone;
-        cnt[k] = 1;
-        if (h < hl) {
-            tok[k] = (uint32_t)ht[h];
-            if (hc)
-                cnt[k] = hc[h];
-        }
+        have[k] = h < hl;
+        tok[k] = (uint32_t)ht[have[k] ? h : 0u]; // hl > 0 here
+    }
+    if (hc) {
+#pragma unroll
+        for (int k = 0; k < KH; ++k)
+            cnt[k] = hc[have[k] ? tid + (uint32_t)k * kThreads : 0u];
+    }
+    uint32_t mw[KH > 0 ? KH : 1];
+#pragma unroll
+    for (int k = 0; k < KH; ++k) {
+        have[k] = have[k] && tok[k] >= lo && tok[k] < hi;
+        rawv[k] = lrow[have[k] ? tok[k] : lo];
+    }
+    if (mrow) {
+#pragma unroll
+        for (int k = 0; k < KH; ++k)
+            mw[k] = mrow[(have[k] ? tok[k] : lo) >> 5];
     }
 #pragma unroll
     for (int k = 0; k < KH; ++k) {
-        rawv[k] = nan;
-        if (tok[k] >= lo && tok[k] < hi) {
-            rawv[k] = lrow[tok[k]];
-            if (mrow && !((mrow[tok[k] >> 5] >> (tok[k] & 31u)) & 1u))
-                rawv[k] = -INFINITY;
-        } else {
+        if (!hc)
+            cnt[k] = 1;
+        if (mrow && !((mw[k] >> (tok[k] & 31u)) & 1u))
+            rawv[k] = -INFINITY;
+        if (!have[k]) {
+            rawv[k] = nan;
             tok[k] = kNone;
+            cnt[k] = 1;
         }
     }
     uint4* z = reinterpret_cast<uint4*>(s_cnt); // slice_len is a multiple of 4
@@ -976,28 +1003,28 @@ __device__ void draw_from_list(const mako_sample_desc& d, uint32_t row, QAt qat,
 // sorted lists: top-p cut, exact fp32 total and walk, in groups of 256 (see seqfp.h, "groups")
 // ---------------------------------------------------------------------------------------------
 
-struct GroupLds { // carved from the lower half of the dynamic LDS block once sorting is over
-    double* pg;      // [kMaxGroups + 2] fp64 sum of the entries before each group
-    uint32_t* d0;    // [kMaxGroups] the group's map for the guessed epoch
-    uint32_t* d1;
-    uint32_t* cmax;
-    uint32_t* start; // first entry of the group
-    uint32_t* pack;  // entries | guessed exponent << 16
-    uint32_t* misc;  // [4]
+struct GroupLds { // carved from the dynamic LDS block once sorting is over; one pointer, the rest is offsets
+    unsigned long long* base;
+    __device__ __forceinline__ double* pg() const { return reinterpret_cast<double*>(base); } // [kMaxGroups + 2] fp64 sum of the entries before each group
+    __device__ __forceinline__ uint32_t* d0() const { return reinterpret_cast<uint32_t*>(base + kMaxGroups + 2); } // [kMaxGroups] the group's map for the guessed epoch
+    __device__ __forceinline__ uint32_t* d1() const { return d0() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* cmax() const { return d1() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* start() const { return cmax() + kMaxGroups; } // first entry of the group
+    // entries (bits 0-8) | quarter-record slot + 1 (bits 9-15) | guessed exponent << 16
+    __device__ __forceinline__ uint32_t* pack() const { return start() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* misc() const { return pack() + kMaxGroups; } // [4]; misc[3] counts the quarter-record slots in use
+    // [kQuarterSlots][4], in the upper half of the dynamic LDS block
+    __device__ __forceinline__ uint4* quarters() const { return reinterpret_cast<uint4*>(base + kSortMax); }
 };
+constexpr uint32_t kLenMask = 0x1ffu;
+constexpr uint32_t kHasQuarters = 1u << 31;
+constexpr uint32_t kQuarterSlots = 96;
+constexpr uint32_t kQuarter = kGroup / 4;
 
 __device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
 {
-    GroupLds G;
-    G.pg = reinterpret_cast<double*>(L.sortk);
-    G.d0 = reinterpret_cast<uint32_t*>(G.pg + kMaxGroups + 2);
-    G.d1 = G.d0 + kMaxGroups;
-    G.cmax = G.d1 + kMaxGroups;
-    G.start = G.cmax + kMaxGroups;
-    G.pack = G.start + kMaxGroups;
-    G.misc = G.pack + kMaxGroups;
     static_assert((kMaxGroups + 2) * 8 + 5 * kMaxGroups * 4 + 16 <= kSortMax * 8, "group records fit below the LDS lists");
-    return G;
+    return GroupLds{L.sortk};
 }
 
 // Values every lane of the wave holds alike, moved to scalar registers so that loops and branches on them
@@ -1093,8 +1120,52 @@ __device__ __forceinline__ seqfp::Step32 span_map(const float (&q)[4], uint32_t 
     return st;
 }
 
+// A group inside which the running sum is expected to change binade cannot be applied as one map.  Its four
+// quarters (64 entries = the 16 lanes of one DPP row each) get maps of their own, each for the binade guessed from
+// the fp64 sum up to ITS first entry: the chain then replays only the quarter in which the change happens.
+// `at_start` is the estimate of the sum at the group's first entry.  One wave; the four records (d0, d1, cmax,
+// exponent) go to out[0..3].
+__device__ void build_quarters(const float (&q)[4], uint32_t len, double at_start, uint4* out)
+{
+    using namespace seqfp;
+    const uint32_t lane = lane_id(), quarter = lane >> 4;
+    double rs = (((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3];
+    for (int o = 1; o < 16; o <<= 1)
+        rs += __shfl_xor(rs, o);
+    const double s0 = __shfl(rs, 0), s1 = __shfl(rs, 16), s2 = __shfl(rs, 32);
+    const double before = quarter == 0 ? 0.0 : (quarter == 1 ? s0 : (quarter == 2 ? s0 + s1 : (s0 + s1) + s2));
+    const double guess = at_start + before;
+    const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+    Step32 v = Step32{kSat, kSat, kSat};
+    if (eg > 0) {
+        v = identity32();
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (lane * 4u + j < len)
+                v = compose32(v, step32(q[j], eg));
+    }
+    uint32_t cm = v.cmax;
+    for (int o = 1; o < 16; o <<= 1)
+        cm = max(cm, (uint32_t)__shfl_xor((int)cm, o));
+    // inclusive scan inside the row of 16 lanes
+#define MAKO_ROW_STEP(CTRL)                                                                                          \
+    {                                                                                                                \
+        const Step32 t = Step32{dpp_or_zero<CTRL, 0xf>(v.d0), dpp_or_zero<CTRL, 0xf>(v.d1), 0u};                     \
+        const Step32 r = compose32(t, Step32{v.d0, v.d1, 0u});                                                       \
+        v.d0 = r.d0;                                                                                                 \
+        v.d1 = r.d1;                                                                                                 \
+    }
+    MAKO_ROW_STEP(0x111)
+    MAKO_ROW_STEP(0x112)
+    MAKO_ROW_STEP(0x114)
+    MAKO_ROW_STEP(0x118)
+#undef MAKO_ROW_STEP
+    if ((lane & 15u) == 15u)
+        out[quarter] = make_uint4(v.d0, v.d1, cm, (uint32_t)eg);
+}
+
 // Group maps of groups [0, groups) for epochs guessed from pg: sum (walk == false) or walk from r0.
-__device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk, double r0, const GroupLds& G)
+__device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk, double r0, const GroupLds G)
 {
     using namespace seqfp;
     // four groups per trip and wave, their loads issued together
@@ -1104,15 +1175,31 @@ __device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk,
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
             const uint32_t g = min(g0 + u, groups - 1u);
-            len[u] = uniform_u32(G.pack[g] & 0xffffu);
-            load_span(kf, uniform_u32(G.start[g]), len[u], q[u]);
+            len[u] = uniform_u32(G.pack()[g] & kLenMask);
+            load_span(kf, uniform_u32(G.start()[g]), len[u], q[u]);
         }
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
             const uint32_t g = g0 + u;
-            const double guess = g < groups ? (walk ? r0 - G.pg[g] : G.pg[g]) : 0.0;
+            const double guess = g < groups ? (walk ? r0 - G.pg()[g] : G.pg()[g]) : 0.0;
             const int eg = guess > 0 ? exponent_of((float)guess) : 0;
             const Step32 st = span_map(q[u], len[u], eg);
+            // a group in which the running sum is expected to change binade (or starts from zero) gets quarter
+            // records; the walk replays such groups with scan_span_walk instead
+            uint32_t slot = 0;
+            if (!walk && g < groups) { // uniform
+                const double at_end = G.pg()[g + 1];
+                const int e_end = at_end > 0 ? exponent_of((float)at_end) : 0;
+                if (uniform_u32((uint32_t)(e_end != eg)) || g == 0) {
+                    if (lane_id() == 0)
+                        slot = atomicAdd(&G.misc()[3], 1u) + 1u;
+                    slot = uniform_u32(slot);
+                    if (slot > kQuarterSlots)
+                        slot = 0;
+                    else
+                        build_quarters(q[u], len[u], G.pg()[g], G.quarters() + (slot - 1u) * 4u);
+                }
+            }
             if (lane_id() == 0 && g < groups) {
                 uint32_t third = st.cmax;
                 if (walk) {
@@ -1131,13 +1218,51 @@ __device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk,
                     if (eg > 1)
                         third = max(third, min(st.cmax, 1u << 30) + (1u << 23) + 1u);
                 }
-                G.d0[g] = st.d0;
-                G.d1[g] = st.d1;
-                G.cmax[g] = third;
-                G.pack[g] = len[u] | ((uint32_t)eg << 16);
+                G.d0()[g] = st.d0;
+                G.d1()[g] = st.d1;
+                G.cmax()[g] = third;
+                G.pack()[g] = len[u] | (slot << 9) | ((uint32_t)eg << 16);
             }
         }
     }
+}
+
+__device__ float exact_span_sum(const uint32_t* kf, uint32_t start, uint32_t len, float S);
+__device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len, float& r, uint32_t& pos);
+
+// State of a chain between groups: significand and exponent of the running value, and where the walk stopped.
+struct ChainState {
+    uint32_t M;
+    int e;
+    uint32_t pos; // kNone while the walk goes on
+};
+
+// One group applied to the running sum quarter by quarter (records at `rec`), replaying only the quarters whose
+// map does not apply.  One wave.  (State by value: the chain keeps it in scalar registers.)
+__device__ __forceinline__ ChainState sum_by_quarters(const uint32_t* kf, uint32_t st, uint32_t len, const uint4* rec,
+                                                      ChainState c)
+{
+    using namespace seqfp;
+#pragma unroll 1
+    for (uint32_t k = 0; k < 4u; ++k) {
+        if (k * kQuarter < len) { // uniform
+            const uint4 r = rec[k];
+            const uint32_t d0 = uniform_u32(r.x), d1 = uniform_u32(r.y), cm = uniform_u32(r.z), eg = uniform_u32(r.w);
+            const uint32_t dd = (c.M & 1u) ? d1 : d0;
+            const uint32_t lim = cm >= (1u << 24) - 1u ? 0u : (1u << 24) - 1u - cm;
+            if ((uint32_t)c.e == eg && c.M + dd < lim) {
+                c.M += dd;
+            } else {
+                const float S = exact_span_sum(kf, st + k * kQuarter, min(kQuarter, len - k * kQuarter), join(c.M, c.e));
+                uint32_t Mv;
+                int ev;
+                split(S, Mv, ev);
+                c.M = uniform_u32(Mv);
+                c.e = (int)uniform_u32((uint32_t)ev);
+            }
+        }
+    }
+    return c;
 }
 
 // The entries of one span added to S one by one with real fp32 additions.  Each lane fetches its four
@@ -1282,9 +1407,10 @@ __device__ bool scan_span_walk(const uint32_t* kf, uint32_t start, uint32_t len,
 //
 // `T` (with `t_groups` records at `t_base`) describes a list whose groups were prepared by sort_kernel's workers;
 // without it the list is cut into groups of kGroup here.
+template <bool PLANNED = false>
 __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf,
                             const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
-                            const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, const GroupTable* T = nullptr,
+                            const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, GroupTable T = GroupTable{},
                             size_t t_base = 0, uint32_t t_groups = 0)
 {
     using namespace seqfp;
@@ -1295,7 +1421,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     auto idat = [=](uint32_t i) { return jf[i]; };
     const GroupLds G = group_lds(L);
     const bool topp_active = P.top_p < 1.0f;
-    if (d.draft || (!T && n1 > kGroup * kMaxGroups)) {
+    if (d.draft || (!PLANNED && n1 > kGroup * kMaxGroups)) {
         // verification and oversized lists take the generic windowed replay
         uint32_t n = n1;
         if (topp_active) {
@@ -1331,7 +1457,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         return true;
     }
 
-    if (!T && n1 <= kGroup) {
+    if (!PLANNED && n1 <= kGroup) {
         // short list: one wave does everything, the chain of fp32 roundings replayed with real additions
         MAKO_STAMP(5);
         __syncthreads(); // the list is published; sm.flag is free
@@ -1405,23 +1531,34 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 
     // group records: fp64 sums (and, from the workers, the maps of the running sum)
     MAKO_STAMP(5);
-    const uint32_t groups1 = T ? t_groups : (n1 + kGroup - 1) / kGroup;
+    const uint32_t groups1 = PLANNED ? t_groups : (n1 + kGroup - 1) / kGroup;
+    if (tid == 0)
+        G.misc()[3] = 0;
     __syncthreads();
-    if (T) {
+    if constexpr (PLANNED) {
         if (tid < groups1) {
-            G.pg[tid + 1] = T->sum[t_base + tid];
-            G.d0[tid] = T->d0[t_base + tid];
-            G.d1[tid] = T->d1[t_base + tid];
-            G.cmax[tid] = T->cmax[t_base + tid];
+            G.pg()[tid + 1] = T.sum[t_base + tid];
+            G.d0()[tid] = T.d0[t_base + tid];
+            G.d1()[tid] = T.d1[t_base + tid];
+            G.cmax()[tid] = T.cmax[t_base + tid];
             // (clamped into the list: a record is only ever read, never trusted for addressing)
-            const uint32_t st = min(T->start[t_base + tid], n1), pk = T->pack[t_base + tid];
-            G.start[tid] = st;
-            G.pack[tid] = min(pk & 0xffffu, min(kGroup, n1 - st)) | (pk & 0xffff0000u);
+            const uint32_t st = min(T.start[t_base + tid], n1), pk = T.pack[t_base + tid];
+            uint32_t slot = 0;
+            if (pk & kHasQuarters) {
+                slot = atomicAdd(&G.misc()[3], 1u) + 1u;
+                if (slot > kQuarterSlots)
+                    slot = 0;
+                else
+                    for (uint32_t k = 0; k < 4; ++k)
+                        G.quarters()[(slot - 1u) * 4u + k] = T.quarters[(t_base + tid) * 4u + k];
+            }
+            G.start()[tid] = st;
+            G.pack()[tid] = min(pk & kLenMask, min(kGroup, n1 - st)) | (slot << 9) | (pk & 0x00ff0000u);
         }
     } else {
         if (tid < groups1) {
-            G.start[tid] = tid * kGroup;
-            G.pack[tid] = min(kGroup, n1 - tid * kGroup);
+            G.start()[tid] = tid * kGroup;
+            G.pack()[tid] = min(kGroup, n1 - tid * kGroup);
         }
         for (uint32_t g0 = wave_id() * 4u; g0 < groups1; g0 += kWaves * 4u) {
             float q[4][4];
@@ -1436,19 +1573,19 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 for (int o = 32; o > 0; o >>= 1)
                     s += __shfl_xor(s, o);
                 if (lane_id() == 0 && g0 + u < groups1)
-                    G.pg[g0 + u + 1] = s;
+                    G.pg()[g0 + u + 1] = s;
             }
         }
     }
     __syncthreads();
     {
-        const double v = tid < groups1 ? G.pg[tid + 1] : 0.0;
+        const double v = tid < groups1 ? G.pg()[tid + 1] : 0.0;
         double all;
         const double incl = block_incl_scan_f64(v, all, sm.bs);
         if (tid < groups1)
-            G.pg[tid + 1] = incl;
+            G.pg()[tid + 1] = incl;
         if (tid == 0)
-            G.pg[0] = 0.0;
+            G.pg()[0] = 0.0;
         if (!have_total)
             total64 = all;
     }
@@ -1459,13 +1596,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     uint32_t n = n1, groups = uniform_u32(groups1);
     if (topp_active) {
         const double want = (double)P.top_p * total64;
-        const uint32_t hitg = (tid < groups1 && G.pg[tid + 1] >= want) ? tid : kNone;
+        const uint32_t hitg = (tid < groups1 && G.pg()[tid + 1] >= want) ? tid : kNone;
         const uint32_t gs = block_min_u32(hitg, sm.bs);
         if (need_cut && gs == kNone)
             return false;
         if (gs != kNone) {
             if (wave_id() == 0) {
-                const uint32_t st = G.start[gs], len = G.pack[gs] & 0xffffu;
+                const uint32_t st = G.start()[gs], len = G.pack()[gs] & kLenMask;
                 float q[4];
                 load_span(kf, st, len, q);
                 double p[4];
@@ -1479,7 +1616,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     if (lane_id() >= o)
                         incl += t;
                 }
-                const double base = G.pg[gs] + (incl - p[3]);
+                const double base = G.pg()[gs] + (incl - p[3]);
                 uint32_t hit = kNone;
 #pragma unroll
                 for (int j = 3; j >= 0; --j)
@@ -1490,13 +1627,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 if (bal)
                     keep = (uint32_t)__shfl((int)hit, __ffsll((long long)bal) - 1) + 1u;
                 if (lane_id() == 0) {
-                    G.misc[0] = st + keep;
+                    G.misc()[0] = st + keep;
                     if (keep != len)
-                        G.pack[gs] = keep; // shortened: the prepared map no longer applies (exponent 0)
+                        G.pack()[gs] = keep; // shortened: the prepared map no longer applies (exponent 0)
                 }
             }
             __syncthreads();
-            n = uniform_u32(G.misc[0]);
+            n = uniform_u32(G.misc()[0]);
             groups = uniform_u32(gs + 1u);
         }
     }
@@ -1511,7 +1648,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 
     // exact fp32 total: group maps in parallel (here, or already by the workers), then one wave chains them
     MAKO_STAMP(7);
-    if (!T)
+    if (!PLANNED)
         build_group_maps(kf, groups, false, 0.0, G);
     __syncthreads();
     MAKO_STAMP(13);
@@ -1524,8 +1661,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         int e = 1; // 0.0f
         for (uint32_t base = 0; base < groups; base += kWave) {
             const uint32_t gl = min(base + lane_id(), groups - 1u);
-            const uint32_t pk_l = G.pack[gl], st_l = G.start[gl];
-            const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], cm_l = G.cmax[gl];
+            const uint32_t pk_l = G.pack()[gl], st_l = G.start()[gl];
+            const uint32_t d0_l = G.d0()[gl], d1_l = G.d1()[gl], cm_l = G.cmax()[gl];
             const uint32_t cnt = min((uint32_t)kWave, groups - base);
             uint32_t done = 0;
             while (done < cnt) {
@@ -1543,22 +1680,30 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
                     const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
                     MAKO_COUNT(20, 1);
-                    const float S = exact_span_sum(kf, st, pk & 0xffffu, join(M, e));
-                    uint32_t Mv;
-                    int ev;
-                    split(S, Mv, ev);
-                    M = uniform_u32(Mv);
-                    e = (int)uniform_u32((uint32_t)ev);
+                    const uint32_t slot = (pk >> 9) & 0x7fu;
+                    if (slot) {
+                        const ChainState c = sum_by_quarters(kf, st, pk & kLenMask, G.quarters() + (slot - 1u) * 4u,
+                                                             ChainState{M, e, kNone});
+                        M = c.M;
+                        e = c.e;
+                    } else {
+                        const float S = exact_span_sum(kf, st, pk & kLenMask, join(M, e));
+                        uint32_t Mv;
+                        int ev;
+                        split(S, Mv, ev);
+                        M = uniform_u32(Mv);
+                        e = (int)uniform_u32((uint32_t)ev);
+                    }
                 }
                 done = f + 1u;
             }
         }
         if (lane_id() == 0)
-            G.misc[1] = __float_as_uint(join(M, e));
+            G.misc()[1] = __float_as_uint(join(M, e));
     }
     __syncthreads();
     MAKO_STAMP(8);
-    const float total = __uint_as_float(G.misc[1]);
+    const float total = __uint_as_float(G.misc()[1]);
     const float span = total - 0.0f;
     const float prod = d.u[row] * span;
     const float r0 = prod + 0.0f;
@@ -1570,10 +1715,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         pos = 0;
     } else if (r0 == r0 && r0 != INFINITY) {
         // only the groups that start before the mass r0 has been used up can be reached; the others get no map
-        const uint32_t beyond = (tid < groups && !((double)r0 - G.pg[tid] > 0)) ? tid : kNone;
+        const uint32_t beyond = (tid < groups && !((double)r0 - G.pg()[tid] > 0)) ? tid : kNone;
         const uint32_t reach = min(groups, block_min_u32(beyond, sm.bs));
         if (tid >= reach && tid < groups)
-            G.pack[tid] &= 0xffffu;
+            G.pack()[tid] &= kLenMask;
+        if (tid == 0)
+            G.misc()[3] = 0; // the running sum's quarter records are done with
+        __syncthreads();
         build_group_maps(kf, reach, true, (double)r0, G);
         __syncthreads();
         MAKO_STAMP(14);
@@ -1591,8 +1739,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             bool stopped = false;
             for (uint32_t base = 0; base < groups && !stopped; base += kWave) {
                 const uint32_t gl = min(base + lane_id(), groups - 1u);
-                const uint32_t pk_l = G.pack[gl], st_l = G.start[gl];
-                const uint32_t d0_l = G.d0[gl], d1_l = G.d1[gl], need_l = G.cmax[gl]; // (the bound, see build_group_maps)
+                const uint32_t pk_l = G.pack()[gl], st_l = G.start()[gl];
+                const uint32_t d0_l = G.d0()[gl], d1_l = G.d1()[gl], need_l = G.cmax()[gl]; // (the bound, see build_group_maps)
                 const uint32_t cnt = min((uint32_t)kWave, groups - base);
                 uint32_t done = 0;
                 while (done < cnt) {
@@ -1610,9 +1758,9 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     if (f < cnt) {
                         const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
                         const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
-                        float r = join(M, e);
                         MAKO_COUNT(22, 1);
-                        if (scan_span_walk(kf, st, pk & 0xffffu, r, at)) {
+                        float r = join(M, e);
+                        if (scan_span_walk(kf, st, pk & kLenMask, r, at)) {
                             stopped = true;
                             break;
                         }
@@ -1626,10 +1774,10 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 }
             }
             if (lane_id() == 0)
-                G.misc[2] = at;
+                G.misc()[2] = at;
         }
         __syncthreads();
-        pos = G.misc[2];
+        pos = G.misc()[2];
     }
 
     MAKO_STAMP(9);
@@ -2074,7 +2222,8 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
-    double* gs = reinterpret_cast<double*>(L.sortk); // [groups]
+    double* gs = reinterpret_cast<double*>(L.sortk); // [groups] estimate of the sum before each group
+    double* ge = gs + kMaxGroups;                    // [groups] and after it
     const uint32_t groups = (cnt + kGroup - 1u) / kGroup;
     __syncthreads();
     for (uint32_t g = wave_id(); g < groups; g += kWaves) {
@@ -2095,6 +2244,7 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
         if (g < groups) {
             T.sum[t_at + g] = v;
             gs[g] = mass + (incl - v);
+            ge[g] = mass + incl;
         }
         mass += all;
     }
@@ -2106,12 +2256,17 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
         const double guess = gs[g];
         const int eg = guess > 0 ? exponent_of((float)guess) : 0;
         const seqfp::Step32 st = span_map(q, len, eg);
+        // the sum is expected to change binade inside the group (or starts at zero): records for its quarters
+        const double at_end = ge[g];
+        const bool split4 = uniform_u32((uint32_t)(eg == 0 || exponent_of((float)at_end) != eg)) != 0;
+        if (split4)
+            build_quarters(q, len, guess, T.quarters + (t_at + g) * 4u);
         if (lane_id() == 0) {
             T.d0[t_at + g] = st.d0;
             T.d1[t_at + g] = st.d1;
             T.cmax[t_at + g] = st.cmax;
             T.start[t_at + g] = off + g * kGroup;
-            T.pack[t_at + g] = len | ((uint32_t)eg << 16);
+            T.pack[t_at + g] = len | ((uint32_t)eg << 16) | (split4 ? kHasQuarters : 0u);
         }
     }
 }
@@ -2398,15 +2553,15 @@ __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t s
 
 // Exact fp64 sum of q over one slice, and the number of candidates in it (q > 0 and q >= min_p).
 // The summation order is fixed: each thread adds its logits in index order, then lanes, then waves.
-template <bool VEC, int KH>
+// (PEN: the row has penalties to apply; a compile-time fact so that each case gets straight-line code of its own.)
+template <bool VEC, int KH, bool PEN>
 __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slice,
-                              uint32_t slice_len, const mako_sampling_params& P, float m, const FinishLds& L)
+                              uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, float m, const FinishLds& L)
 {
     FinishShared& sm = *L.sm;
     const uint32_t lo = slice * slice_len;
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
-    const uint32_t hl = d.hist_tokens ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
-    const bool pen = hl > 0 && !penalties_neutral(P);
+    constexpr bool pen = PEN;
     float wv[16];
     Extras<KH> ex;
     load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, ex);
@@ -2426,7 +2581,7 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
         }
     }
 #pragma unroll
-    for (int k = 0; k < KH; ++k) {
+    for (int k = 0; k < (PEN ? KH : 0); ++k) {
         const float q = weight_of(ex.v[k], m, inv_t, sm.tab);
         qe[k] = (q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
         if (qe[k]) {
@@ -2476,7 +2631,7 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
     }
     __syncthreads(); // the owners' stores land before the holders of moved logits overwrite theirs
 #pragma unroll
-    for (int k = 0; k < KH; ++k)
+    for (int k = 0; k < (PEN ? KH : 0); ++k)
         if (ex.i[k] != kNone) {
             qk[ex.i[k]] = qe[k];
             if (qe[k]) {
@@ -2633,7 +2788,11 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
 
     if (cls == kNucleus) {
         // second pass, all slices of the row in parallel; plan_kernel continues once every slice is through
-        slice_partial<VEC, KH>(d, sc, row, slice, slice_len, P, m, L);
+        const uint32_t hl = d.hist_tokens ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
+        if (hl > 0 && !penalties_neutral(P))
+            slice_partial<VEC, KH, true>(d, sc, row, slice, slice_len, P, hl, m, L);
+        else
+            slice_partial<VEC, KH, false>(d, sc, row, slice, slice_len, P, hl, m, L);
         return;
     }
     if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
@@ -2962,8 +3121,8 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     __syncthreads();
     if (tid == 0)
         plan->flag = 0;
-    sorted_tail(d, row, s_args.P, sc.key[0] + (size_t)row * sc.vpad, sc.idx[0] + (size_t)row * sc.vpad, n0, true, total64,
-                MAKO_PATH_GENERAL, L, false, 0.0f, &sc.gt, (size_t)row * sc.g_cap, groups);
+    sorted_tail<true>(d, row, s_args.P, sc.key[0] + (size_t)row * sc.vpad, sc.idx[0] + (size_t)row * sc.vpad, n0, true,
+                      total64, MAKO_PATH_GENERAL, L, false, 0.0f, sc.gt, (size_t)row * sc.g_cap, groups);
 }
 
 
