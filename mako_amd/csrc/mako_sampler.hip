@@ -19,6 +19,7 @@ struct mako_sampler_ctx {
     int device = 0;
     uint32_t max_rows = 0, max_vocab = 0, max_hist = 0;
     mako::Scratch sc{};
+    mako::Scratch* sc_dev = nullptr; // the same record in device memory: the kernels take a pointer to it
     // staging for the host-pointer call
     float* st_logits = nullptr;
     mako_sampling_params* st_params = nullptr;
@@ -125,6 +126,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, hipMemset(sc.work_n, 0, 2 * sizeof(uint32_t)));
     MAKO_HIP(ctx, dev_alloc(&sc.work_sort, (size_t)max_rows * mako::kWorkers));
     MAKO_HIP(ctx, dev_alloc(&sc.work_tail, (size_t)max_rows));
+    MAKO_HIP(ctx, dev_alloc(&ctx->sc_dev, 1));
+    MAKO_HIP(ctx, hipMemcpy(ctx->sc_dev, &sc, sizeof sc, hipMemcpyHostToDevice));
     MAKO_HIP(ctx, hipDeviceSynchronize());
     // both kernels overlay up to 64 KB of dynamic LDS on a few KB of static LDS
     const void* kernels[] = {(const void*)mako::scan_kernel<true, 0>,    (const void*)mako::scan_kernel<false, 0>,
@@ -148,7 +151,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {sc.bin_worker, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
+    void* ptrs[] = {ctx->sc_dev, sc.bin_worker, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
                     sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.binc, sc.bins, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
@@ -233,9 +236,9 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     } while (0)
 #define MAKO_LAUNCH(V, K)                                                                                          \
     do {                                                                                                           \
-        hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc, slice_len); \
+        hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc_dev, slice_len); \
         MAKO_MARK(1);                                                                                              \
-        hipLaunchKernelGGL((mako::finish_kernel<V, K>), grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc,  \
+        hipLaunchKernelGGL((mako::finish_kernel<V, K>), grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev,  \
                            slices, slice_len);                                                                     \
         MAKO_MARK(2);                                                                                              \
     } while (0)
@@ -255,14 +258,14 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
 #undef MAKO_LAUNCH
     // top_k == 0 rows: plan from the row's histogram, sort by the plan, cut and draw; the stages talk through
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  Other rows cost a load.
-    hipLaunchKernelGGL(mako::plan_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc, slices);
+    hipLaunchKernelGGL(mako::plan_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev, slices);
     MAKO_MARK(3);
-    hipLaunchKernelGGL(mako::partition_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), 0, st, d, ctx->sc);
+    hipLaunchKernelGGL(mako::partition_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), 0, st, d, ctx->sc_dev);
     MAKO_MARK(4);
-    hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d, ctx->sc,
+    hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d, ctx->sc_dev,
                        slices);
     MAKO_MARK(5);
-    hipLaunchKernelGGL(mako::tail_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc);
+    hipLaunchKernelGGL(mako::tail_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev);
     MAKO_MARK(6);
 #undef MAKO_MARK
     ctx->profiled = prof;

@@ -479,7 +479,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
 // scan_kernel
 // ---------------------------------------------------------------------------------------------
 
-struct ScanShared {
+struct alignas(16) ScanShared {
     uint32_t wave_max[kWaves]; // order keys
     uint32_t wave_kth[kWaves];
     uint32_t argidx;
@@ -536,10 +536,12 @@ __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 
 // grid = (slices, rows).
 template <bool VEC, int KH>
-__global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scratch sc, uint32_t slice_len)
+__global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, const Scratch* sc_dev, uint32_t slice_len)
 {
+    const Scratch& sc = *sc_dev;
     MAKO_ROW(blockIdx.y);
-    extern __shared__ uint32_t s_dyn[]; // [slice_len] token counts when the row has penalties
+    // (16-byte alignment: the table is cleared and read with 128-bit LDS operations, which crawl when misaligned)
+    extern __shared__ __align__(16) uint32_t s_dyn[]; // [slice_len] token counts when the row has penalties
     __shared__ ScanShared sm;
 
     const uint32_t row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
@@ -675,7 +677,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
 // finish_kernel
 // ---------------------------------------------------------------------------------------------
 
-struct FinishShared {
+struct alignas(16) FinishShared {
     BlockScratch bs;
     uint64_t tab[32];
     uint32_t hist[256];
@@ -2653,7 +2655,7 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
 
 // Kernel arguments that are handed on by reference to out-of-line device functions would be spilled to scratch
 // memory (a microsecond per access); the two finishing kernels keep their copies in LDS instead.
-struct ArgsLds {
+struct alignas(16) ArgsLds {
     mako_sample_desc d;
     Scratch sc;
     mako_sampling_params P; // the row's parameters
@@ -2738,10 +2740,11 @@ __device__ float candidate_bound(const Scratch& sc, uint32_t row, uint32_t slice
 // row, and one per slice for top_k == 0 rows (find_piece).  The busy workgroups are then the first ones dispatched
 // and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
 template <bool VEC, int KH>
-__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices,
+__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices,
                                                           uint32_t slice_len)
 {
-    extern __shared__ unsigned long long s_dyn64[];
+    const Scratch& sc_arg = *sc_dev;
+    extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
 #ifdef MAKO_TIMING_FINISH
@@ -2841,9 +2844,10 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
 // grid = (1, rows), workgroup i serving the i-th top_k == 0 row (find_piece): the row's exact total, candidate count and weight histogram are summed
 // over its slices and the row is planned: handed to sort_kernel's workers, or, when the nucleus is narrow enough to
 // end inside the candidate lists, to its worker 0 alone.
-__global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices)
+__global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
 {
-    extern __shared__ unsigned long long s_dyn64[];
+    const Scratch& sc_arg = *sc_dev;
+    extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
     uint32_t row, sub;
@@ -2930,8 +2934,9 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
 // the worker that will sort it: positions inside the workgroup from LDS counters, one global atomic per worker to
 // reserve the workgroup's run in that worker's share.  (Without this step each of the 32 workers would sweep the
 // whole row to find its own weights.)
-__global__ __launch_bounds__(kThreads) void partition_kernel(mako_sample_desc d, Scratch sc)
+__global__ __launch_bounds__(kThreads) void partition_kernel(mako_sample_desc d, const Scratch* sc_dev)
 {
+    const Scratch& sc = *sc_dev;
     __shared__ uint32_t s_count[kWorkers], s_base[kWorkers], s_off[kWorkers], s_cnt[kWorkers];
     __shared__ uint32_t s_table[kBins / 4];
     const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
@@ -3003,9 +3008,10 @@ __global__ __launch_bounds__(kThreads) void partition_kernel(mako_sample_desc d,
 // grid = (kWorkers, rows) workgroups, of which workgroup i serves entry i of the work list.  Worker w gathers its range of weights from
 // the row's bits(q) array, sorts it and stores it at its place in the row's sorted list; the last worker to
 // finish cuts the nucleus and draws.
-__global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_arg, uint32_t slices)
+__global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
 {
-    extern __shared__ unsigned long long s_dyn64[];
+    const Scratch& sc_arg = *sc_dev;
+    extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
     const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
@@ -3096,9 +3102,10 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
 }
 
 // grid = (1, rows).  Rows whose sorted list sort_kernel's workers have prepared: top-p cut, exact total, draw.
-__global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_arg)
+__global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, const Scratch* sc_dev)
 {
-    extern __shared__ unsigned long long s_dyn64[];
+    const Scratch& sc_arg = *sc_dev;
+    extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
     if (blockIdx.y >= sc_arg.work_n[1])
