@@ -72,7 +72,31 @@ constexpr uint32_t kCap = 512;       // candidates kept per slice
 constexpr uint32_t kTopKFast = 128;  // largest top_k resolved from the per-slice candidates
 constexpr uint32_t kSortMax = 4096;  // candidates the finisher sorts in LDS
 constexpr uint32_t kDynLds = 65536;  // dynamic LDS of both kernels
-constexpr uint32_t kBins = 2048;     // weight histogram of top_k == 0 rows: bin = bits(q) >> 19 (16 bins per binade)
+constexpr uint32_t kBins = 2048;     // weight histogram of top_k == 0 rows, see weight_bin()
+
+// Histogram bin of a weight q in (0, 1], by its bits: 128 bins per binade for the eight binades below 1.0 (bins
+// 1024..2047) and 8 per binade for everything smaller, subnormals included (bins 71..1023; bins below 71 stay
+// empty).  Bin edges include every binade boundary, so all weights of a bin share their exponent and the bin's
+// mass is exactly (sum of 24-bit significands) * 2^(exponent - 150).  The fine bins keep near-flat rows, whose
+// weights all lie within a factor of two, spread over all workers.
+constexpr uint32_t kFineFrom = 0x3b810000u; // bits(2^-8) + 0x10000: the top fine bin holds 1.0 alone
+constexpr uint32_t kCoarseShift = 20;       // 8 bins per binade
+constexpr uint32_t kCoarseBase = 1023u - ((kFineFrom - 1u) >> kCoarseShift); // 71
+__device__ __forceinline__ uint32_t weight_bin(uint32_t bits)
+{
+    return bits >= kFineFrom ? min(1024u + ((bits - kFineFrom) >> 16), kBins - 1u) : (bits >> kCoarseShift) + kCoarseBase;
+}
+// Smallest bits(q) of a bin, and one past the largest.
+__device__ __forceinline__ uint32_t bin_lo_key(uint32_t b)
+{
+    if (b >= 1024u)
+        return kFineFrom + ((b - 1024u) << 16);
+    return b > kCoarseBase ? (b - kCoarseBase) << kCoarseShift : 0u;
+}
+__device__ __forceinline__ uint32_t bin_hi_key(uint32_t b)
+{
+    return b + 1u < kBins ? bin_lo_key(b + 1u) : kFineFrom + (1024u << 16); // (just above bits(1.0f))
+}
 
 constexpr uint32_t kFlagFirstNan = 1u; // element 0 of the row is NaN (slice 0 only)
 constexpr uint32_t kFlagOverflow = 2u; // more than kCap logits reached the slice's threshold
@@ -1835,7 +1859,7 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
         d, row, [=](uint32_t i) { return __uint_as_float(~kf[i]); }, [=](uint32_t i) { return jf[i]; }, n1, path, sm);
 }
 
-// Plans a top_k == 0 row from the histogram of its weights (16 bins per binade, exact masses): finds the bin by
+// Plans a top_k == 0 row from the histogram of its weights (weight_bin(), exact masses): finds the bin by
 // which the nucleus must have ended and splits the weights above it over kWorkers workers by value.
 // Thread t brings the counts (c0, c1) and significand sums (s0, s1) of bins kBins-1-2t and kBins-2-2t.
 // Returns n0, the number of weights to sort; the plan is written to `plan` (flag left untouched).
@@ -1848,7 +1872,7 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
     const uint32_t b0 = kBins - 1u - 2u * tid, b1 = b0 - 1u;
     // exact mass of a bin: sum of significands times the bin's power of two (bins never straddle a binade)
     auto scale = [](uint32_t b) {
-        const uint32_t e = max(b >> 4, 1u); // biased exponent of the bin's weights (0 -> subnormal scale)
+        const uint32_t e = max(bin_lo_key(b) >> 23, 1u); // biased exponent of the bin's weights (subnormals: 1)
         return __longlong_as_double((long long)(1023ull + e - 150ull) << 52);
     };
     const double m0 = (double)s0 * scale(b0), m1 = (double)s1 * scale(b1);
@@ -1868,7 +1892,7 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         hit = b1;
     const uint32_t rev = block_min_u32(hit == kNone ? kNone : kBins - 1u - hit, sm.bs);
     const uint32_t b_lo = rev == kNone ? 0u : kBins - 1u - rev; // not reached twice: keep every candidate
-    thr_bits = b_lo << 19;
+    thr_bits = bin_lo_key(b_lo);
 
     // candidates above each bin, and the workers' shares
     uint32_t count_all;
@@ -1915,8 +1939,8 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
     bin_worker[b1] = (uint8_t)wk1;
     if (tid < kWorkers) {
         plan->cursor[tid] = 0;
-        plan->key_lo[tid] = w_lo[tid] << 19;
-        plan->key_hi[tid] = (w_hi[tid] + 1u) << 19;
+        plan->key_lo[tid] = bin_lo_key(min(w_lo[tid], kBins - 1u));
+        plan->key_hi[tid] = bin_hi_key(w_hi[tid]);
         plan->off[tid] = w_cnt[tid] ? w_off[tid] : 0u;
         plan->cnt[tid] = w_cnt[tid];
     }
@@ -2215,6 +2239,141 @@ __device__ bool lds_sort_staged(const uint32_t* ks, const uint32_t* is, uint32_t
     }
     __syncthreads();
     return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm);
+}
+
+// A share too large for one LDS sort is cut by value into runs that fit: one counting sweep over the share (the
+// same kFine buckets as the sort uses) finds run boundaries at bucket edges, then each run is collected from the
+// share and sorted on its own.  Returns false (the caller falls back to the radix sort through global memory)
+// when a single bucket holds more than fits.
+__device__ bool lds_sort_staged_runs(const uint32_t* ks, const uint32_t* is, uint32_t key_lo, uint32_t key_hi, uint32_t cnt,
+                                     uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm)
+{
+    uint2* A = reinterpret_cast<uint2*>(dyn);
+    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap); // [kFine + 1]
+    const uint32_t tid = threadIdx.x, lane = lane_id();
+    const uint32_t range = key_hi - key_lo;
+    const uint32_t shift = range > kFine ? 32u - (uint32_t)__clz((range - 1u) >> 11) : 0u;
+    for (uint32_t b = tid; b <= kFine; b += kThreads)
+        hist[b] = 0;
+    __syncthreads();
+    constexpr uint32_t kTrip = 8; // loads in flight per thread: the sweeps below are bound by memory latency
+    for (uint32_t base = 0; base < cnt; base += kTrip * kThreads) {
+        uint32_t k[kTrip];
+#pragma unroll
+        for (uint32_t u = 0; u < kTrip; ++u)
+            k[u] = ks[min(base + u * kThreads + tid, cnt - 1u)];
+#pragma unroll
+        for (uint32_t u = 0; u < kTrip; ++u)
+            if (base + u * kThreads + tid < cnt)
+                atomicAdd(&hist[(key_hi - 1u - min(max(k[u], key_lo), key_hi - 1u)) >> shift], 1u);
+    }
+    __syncthreads();
+    // bucket starts (exclusive scan), kept in sm.hist / sm.run as run boundaries below
+    uint32_t total;
+    const uint32_t c0 = hist[2u * tid], c1 = hist[2u * tid + 1u];
+    const uint32_t ex = block_excl_scan_u32(c0 + c1, total, sm.bs);
+    __syncthreads();
+    hist[2u * tid] = ex;
+    hist[2u * tid + 1u] = ex + c0;
+    if (tid == 0) {
+        hist[kFine] = total;
+        sm.flag = 0;
+    }
+    __syncthreads();
+    // runs: greedily as many whole buckets as fit (thread 0; a handful of runs).  Run r covers buckets
+    // [sm.hist[r], sm.hist[64 + r]) = entries [sm.run[r], sm.run[r] + sm.run[64 + r]) of the sorted share.
+    if (tid == 0) {
+        uint32_t runs = 0, b0 = 0;
+        while (b0 < kFine && runs < 64u) {
+            uint32_t b1 = b0 + 1u;
+            if (hist[b1] - hist[b0] > kSegCap) { // one bucket alone is too much
+                runs = 0xffffffffu;
+                break;
+            }
+            { // the last bucket edge within reach: the bucket starts never decrease, so bisect
+                uint32_t lo = b1, hi = kFine;
+                while (lo < hi) {
+                    const uint32_t mid = (lo + hi + 1u) / 2u;
+                    if (hist[mid] - hist[b0] <= kSegCap)
+                        lo = mid;
+                    else
+                        hi = mid - 1u;
+                }
+                b1 = lo;
+            }
+            if (hist[b1] != hist[b0]) {
+                sm.hist[runs] = b0;
+                sm.hist[64u + runs] = b1;
+                sm.run[runs] = hist[b0];
+                sm.run[64u + runs] = hist[b1] - hist[b0];
+                ++runs;
+            }
+            b0 = b1;
+        }
+        if (runs != 0xffffffffu && b0 < kFine)
+            runs = 0xffffffffu;
+        sm.ticket = runs;
+    }
+    __syncthreads();
+    const uint32_t runs = sm.ticket;
+    if (runs == 0xffffffffu)
+        return false;
+    for (uint32_t r = 0; r < runs; ++r) {
+        const uint32_t b0 = sm.hist[r], b1 = sm.hist[64u + r];
+        const uint32_t at = sm.run[r], n = sm.run[64u + r];
+        // keys of buckets [b0, b1): (key_hi - 1 - k) >> shift in [b0, b1)
+        const uint32_t hi_r = key_hi - (b0 << shift);
+        const uint32_t lo_r = ((unsigned long long)b1 << shift) >= range ? key_lo : key_hi - (b1 << shift);
+        __syncthreads();
+        for (uint32_t b = tid; b <= kFine; b += kThreads)
+            hist[b] = 0;
+        if (tid == 0) {
+            sm.ticket = 0;
+            sm.flag = 0;
+        }
+        __syncthreads();
+        const unsigned long long lower = (1ull << lane) - 1ull;
+        for (uint32_t base = 0; base < cnt; base += kTrip * kThreads) {
+            uint32_t k[kTrip], id[kTrip];
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u) {
+                const uint32_t e = min(base + u * kThreads + tid, cnt - 1u);
+                k[u] = ks[e];
+                id[u] = is[e];
+            }
+            // slots for the whole trip from one LDS atomic per wave
+            bool mine[kTrip];
+            uint32_t before = 0, wave_total = 0;
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u) {
+                k[u] = min(max(k[u], key_lo), key_hi - 1u);
+                mine[u] = base + u * kThreads + tid < cnt && k[u] >= lo_r && k[u] < hi_r;
+                const unsigned long long bal = __ballot(mine[u]);
+                before += (uint32_t)__popcll(bal & lower);
+                wave_total += (uint32_t)__popcll(bal);
+            }
+            if (wave_total) { // uniform
+                uint32_t slot = 0;
+                if (lane == 0)
+                    slot = atomicAdd(&sm.ticket, wave_total);
+                slot = uniform_u32(slot) + before;
+#pragma unroll
+                for (uint32_t u = 0; u < kTrip; ++u)
+                    if (mine[u]) {
+                        if (slot < kSegCap)
+                            A[slot] = make_uint2(k[u], id[u]);
+                        ++slot;
+                    }
+            }
+        }
+        __syncthreads();
+        if (sm.ticket != n) // (cannot happen: the same keys were counted above)
+            return false;
+        if (!lds_bucket_sort(n, lo_r, hi_r, kout + at, iout + at, dyn, sm))
+            return false; // (a crowded bucket: ties)
+    }
+    return true;
 }
 
 // Group records of a worker's sorted range (cnt entries from position off of the list kf): fp64 sums, and the
@@ -2613,8 +2772,8 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j)
         if (qb[j]) {
-            atomicAdd(&hist[qb[j] >> 19], 1u);
-            atomicAdd(&hsum[qb[j] >> 19], signif(qb[j]));
+            atomicAdd(&hist[weight_bin(qb[j])], 1u);
+            atomicAdd(&hsum[weight_bin(qb[j])], signif(qb[j]));
         }
     if (VEC) {
 #pragma unroll
@@ -2637,8 +2796,8 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
         if (ex.i[k] != kNone) {
             qk[ex.i[k]] = qe[k];
             if (qe[k]) {
-                atomicAdd(&hist[qe[k] >> 19], 1u);
-                atomicAdd(&hsum[qe[k] >> 19], signif(qe[k]));
+                atomicAdd(&hist[weight_bin(qe[k])], 1u);
+                atomicAdd(&hsum[weight_bin(qe[k])], signif(qe[k]));
             }
         }
     __syncthreads();
@@ -2981,7 +3140,7 @@ __global__ __launch_bounds__(kThreads) void partition_kernel(mako_sample_desc d,
         uint32_t dest[4], lpos[4];
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            dest[j] = (i + j < hi && k[j] != 0) ? table[min(k[j] >> 19, kBins - 1u)] : 0xffu;
+            dest[j] = (i + j < hi && k[j] != 0) ? table[weight_bin(k[j])] : 0xffu;
             lpos[j] = 0;
             if (dest[j] < kWorkers)
                 lpos[j] = atomicAdd(&s_count[dest[j]], 1u);
@@ -3090,7 +3249,15 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     if (cnt) {
         const uint32_t key_lo = plan->key_lo[w], key_hi = plan->key_hi[w];
         MAKO_STAMP(10);
-        if (cnt > kSegCap || !lds_sort_staged(key1 + off, idx1 + off, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm)) {
+        MAKO_COUNT(31, threadIdx.x == 0 && cnt > kSegCap ? 1 : 0);
+        MAKO_COUNT(21, threadIdx.x == 0 ? cnt : 0);
+        const bool sorted = cnt <= kSegCap
+                                ? lds_sort_staged(key1 + off, idx1 + off, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm)
+                                : lds_sort_staged_runs(key1 + off, idx1 + off, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm);
+        if (cnt > kSegCap)
+            MAKO_STAMP(18);
+        if (!sorted) {
+            MAKO_STAMP(17);
             MAKO_COUNT(23, threadIdx.x == 0 ? 1 : 0);
             gather_range(qk, d.n_vocab, key_lo, key_hi, key0 + off, idx0 + off, cnt, sm);
             sort_segment(key0 + off, idx0 + off, key1 + off, idx1 + off, cnt, L);
