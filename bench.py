@@ -22,6 +22,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per batch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
+# for a device-to-device copy of known size (see the traffic summary under profiles/)
+MEASURED_TRAFFIC_BYTES = {"config3": 77.4e6}
 
 
 def make_workload(name):
@@ -80,6 +83,9 @@ def main():
     ap.add_argument("--workload", default="config3")
     ap.add_argument("--pool-mb", type=int, default=640, help="rotate the logits through this many MB of copies")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--calibrate-copy-mb", type=int, default=0,
+                    help="also run one device-to-device copy of this many MB (a kernel of known traffic, to scale "
+                         "rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
     a = ap.parse_args()
     if a.gpus != 1:
         raise SystemExit("bench.py measures one GPU: rows are independent, a multi-GPU run is a plain batch split "
@@ -110,6 +116,11 @@ def main():
         batch.desc.logits = pool[i % n_copies].ptr
         ctx.sample_batch(batch.desc, stream)
 
+    if a.calibrate_copy_mb:
+        n = a.calibrate_copy_mb << 20
+        src, dst = hip.DeviceArray((n,), np.uint8), hip.DeviceArray((n,), np.uint8)
+        hip.check(hip.lib().hipMemcpy(dst.ptr, src.ptr, n, hip.hipMemcpyDeviceToDevice), "hipMemcpy D2D")
+        hip.synchronize()
     for i in range(a.warmup):
         step(i)
     stream.synchronize()
@@ -162,7 +173,7 @@ def main():
                    "rows": rows, "vocab": vocab, "logit_copies_rotated": n_copies,
                    "host_wall_ms_per_step": wall * 1e3 / a.steps},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
                      "bytes_per_launch": batch_bytes,
                      "kernel": "scan + finish + plan + partition + sort + tail kernels (the six launches of one batch)",
                      "launch_ms": ms_per_step,
