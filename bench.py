@@ -83,6 +83,8 @@ def main():
     ap.add_argument("--workload", default="config3")
     ap.add_argument("--pool-mb", type=int, default=640, help="rotate the logits through this many MB of copies")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--host-pointer-calls", type=int, default=5,
+                    help="also time this many calls of the host-pointer entry point (PCIe-inclusive rate; 0 = skip)")
     ap.add_argument("--calibrate-copy-mb", type=int, default=0,
                     help="also run one device-to-device copy of this many MB (a kernel of known traffic, to scale "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -148,6 +150,35 @@ def main():
     split /= n_split
     ctx.set_profile(False)
 
+    # the host-pointer entry point on the same batch (logits staged over PCIe inside the call): reported beside the
+    # headline value, never as it
+    host_rate = None
+    if a.host_pointer_calls > 0:
+        tok_h = np.zeros(rows, np.int32)
+        hist = np.ascontiguousarray(w["hist"], np.int32) if "hist" in w else None
+        hlen = np.ascontiguousarray(w["hist_len"], np.uint32) if "hist" in w else None
+        mask = np.ascontiguousarray(w["mask"], np.uint32) if "mask" in w else None
+        lg = np.ascontiguousarray(w["logits"], np.float32)
+        pr = np.ascontiguousarray(w["params"])
+        uu = np.ascontiguousarray(w["u"], np.float32)
+
+        def host_call():
+            rc = ctx.lib.mako_sampler_sample_host(
+                ctx.ptr, lg.ctypes.data, vocab, rows, vocab, pr.ctypes.data, uu.ctypes.data,
+                mask.ctypes.data if mask is not None else None, mask.shape[1] if mask is not None else 0,
+                hist.ctypes.data if hist is not None else None, None, hist.shape[1] if hist is not None else 0,
+                hlen.ctypes.data if hlen is not None else None, None, None, None, tok_h.ctypes.data)
+            if rc != 0:
+                raise SystemExit("mako_sampler_sample_host failed: %s" % ctx.last_error())
+
+        host_call()
+        t0 = time.perf_counter()
+        for _ in range(a.host_pointer_calls):
+            host_call()
+        host_rate = rows * a.host_pointer_calls / (time.perf_counter() - t0)
+        if not np.array_equal(tok_h, tokens):
+            raise SystemExit("host-pointer call disagrees with the device-pointer call")
+
     base, ref_tok = (None, None)
     if a.cpu_seconds > 0:
         base, ref_tok = cpu_baseline(w, a.cpu_seconds)
@@ -180,6 +211,7 @@ def main():
                      "kernel_ms": dict(zip(["scan_kernel", "finish_kernel", "plan_kernel", "partition_kernel", "sort_kernel", "tail_kernel"],
                                            [float(x) for x in split])),
                      "scan_kernel_gbs": batch_bytes / (split[0] * 1e-3) / 1e9},
+        "host_pointer_rows_per_s": host_rate,
         "cpu_baseline": base,
         "parity": parity,
     }
