@@ -54,16 +54,31 @@ struct WgTimer {
     }
 };
 #define MAKO_WG_TIMER WgTimer wg_timer_
+#define MAKO_TIC(k)                                                                                                  \
+    __builtin_amdgcn_s_waitcnt(0);                                                                                   \
+    const unsigned long long tic_##k = wall_clock64()
+#define MAKO_TOC(k, i)                                                                                               \
+    do {                                                                                                             \
+        __builtin_amdgcn_s_waitcnt(0);                                                                               \
+        if (lane_id() == 0)                                                                                          \
+            g_mako_stamp[i] += wall_clock64() - tic_##k;                                                             \
+    } while (0)
+#ifdef MAKO_TIMING_COUNTS // event counters: each costs a global round trip, so never together with timestamps
 #define MAKO_COUNT(i, v)                                                                                             \
     do {                                                                                                             \
         if (lane_id() == 0)                                                                                          \
             g_mako_stamp[i] += (v);                                                                                  \
     } while (0)
 #else
+#define MAKO_COUNT(i, v) ((void)0)
+#endif
+#else
 #define MAKO_STAMP(i) ((void)0)
 #define MAKO_ROW(r) ((void)0)
 #define MAKO_COUNT(i, v) ((void)0)
 #define MAKO_WG_TIMER ((void)0)
+#define MAKO_TIC(k) ((void)0)
+#define MAKO_TOC(k, i) ((void)0)
 #endif
 
 constexpr uint32_t kSliceMax = 16384; // elements per slice: 16 per thread
@@ -1211,7 +1226,7 @@ __device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk,
             const int eg = guess > 0 ? exponent_of((float)guess) : 0;
             const Step32 st = span_map(q[u], len[u], eg);
             // a group in which the running sum is expected to change binade (or starts from zero) gets quarter
-            // records; the walk replays such groups with scan_span_walk instead
+            // records; the walk replays such groups whole
             uint32_t slot = 0;
             if (!walk && g < groups) { // uniform
                 const double at_end = G.pg()[g + 1];
@@ -1291,134 +1306,108 @@ __device__ __forceinline__ ChainState sum_by_quarters(const uint32_t* kf, uint32
     return c;
 }
 
-// The entries of one span added to S one by one with real fp32 additions.  Each lane fetches its four
-// entries once; the wave then replays them in list order, reading them back by lane index, so the chain is
-// `len` dependent adds on uniform values and nothing else.
+// The entries of one span (at most 256), one per lane and register: x[j] of lane l is entry 64 * j + l, 0.0f past
+// the end.
+__device__ __forceinline__ void load_span_lanes(const uint32_t* kf, uint32_t start, uint32_t len, float (&x)[4])
+{
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        const uint32_t i = j * kWave + lane_id();
+        const uint32_t k = kf[start + min(i, len - 1u)]; // every lane loads, from inside the span
+        x[j] = i < len ? __uint_as_float(~k) : 0.0f;
+    }
+}
+
+// One step of a chain that travels across the lanes: every lane takes the value of the lane below it (lane 0:
+// of lane 63) and subtracts / adds its own entry.  Started from a uniform value, lane t holds after t + 1 steps
+// the value a sequential loop would hold after entries 0..t; the other lanes hold values nobody reads.  One
+// dependent instruction per entry, where a broadcast per entry costs three.
+__device__ __forceinline__ float ror_sub(float v, float x)
+{
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), 0x13C /* wave_ror:1 */,
+                                                                 0xf, 0xf, false)) - x;
+}
+__device__ __forceinline__ float ror_add(float v, float x)
+{
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), 0x13C /* wave_ror:1 */,
+                                                                 0xf, 0xf, false)) + x;
+}
+
+// S plus the entries of one span (len in 1..256), added one by one in fp32 (src/gen/sampler.cpp:80-82).  One wave.
 __device__ float exact_span_sum(const uint32_t* kf, uint32_t start, uint32_t len, float S)
 {
-    float q[4];
-    load_span(kf, start, len, q); // entries past the end read as 0.0f: adding them changes nothing
-    const uint32_t lanes = (uniform_u32(len) + 3u) / 4u;
-    for (uint32_t l = 0; l < lanes; ++l) {
+    float x[4];
+    const uint32_t n = uniform_u32(len);
+    if (n == 0)
+        return S;
+    load_span_lanes(kf, uniform_u32(start), n, x);
+    float v = S; // uniform
+    for (uint32_t base = 0; base < n; base += kWave) {
+        const float cur = x[0];
+        for (uint32_t b = 0; b < kWave && base + b < n; b += 16u) {
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            S += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), l));
+            for (uint32_t k = 0; k < 16; ++k)
+                v = ror_add(v, cur);
+        }
+        x[0] = x[1];
+        x[1] = x[2];
+        x[2] = x[3];
     }
-    return S;
+    // entries past the end added 0.0f: the lane of the last step holds the sum
+    const uint32_t steps = (n + 15u) & ~15u;
+    return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), (steps - 1u) & 63u));
 }
 
-// The entries of one span subtracted from r one by one (src/gen/sampler.cpp:67-71).  Returns true and the
-// entry's position in the list when the walk stops inside the span, else false and the new r.
+// The entries of one span (len in 1..256) subtracted from r one by one (src/gen/sampler.cpp:67-71).  Returns true
+// and the entry's position in the list when the walk stops inside the span, else false and the new r.  One wave.
+//
+// The walk stops at the first entry with r < x, which is the first entry whose subtraction turns r negative (x != r
+// gives a nonzero difference, denormals kept), and a negative r stays negative under every later subtraction of a
+// weight.  So sixteen entries are subtracted without looking, and only a block that ends negative is walked again
+// from its saved start to find the entry.
 __device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len, float& r, uint32_t& pos)
 {
-    float q[4];
-    load_span(kf, start, len, q); // entries past the end read as 0.0f: r >= 0 never stops at them, r - 0 is r
+    float x[4];
+    const uint32_t n = uniform_u32(len);
     const uint32_t beg = uniform_u32(start);
-    const uint32_t lanes = (uniform_u32(len) + 3u) / 4u;
-    const float nan = __uint_as_float(0x7fc00000u);
-    float rr = r; // NaN once the walk has stopped: no later comparison succeeds
-    uint32_t at = kNone;
-    for (uint32_t l = 0; l < lanes; ++l) {
+    if (n == 0)
+        return false;
+    MAKO_TIC(0);
+    load_span_lanes(kf, beg, n, x);
+    MAKO_TOC(0, 17);
+    MAKO_TIC(1);
+    float v = r;    // uniform
+    float r_in = r; // the walk's value in front of the current block
+    for (uint32_t base = 0; base < n; base += kWave) {
+        const float cur = x[0];
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            const float x = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), l));
-            const bool stop = rr < x;
-            at = stop ? beg + l * 4u + j : at;
-            rr = stop ? nan : rr - x;
-        }
-        if (uniform_u32(at) != kNone) {
-            pos = uniform_u32(at);
-            return true;
-        }
-    }
-    r = rr;
-    return false;
-}
-
-// Same result as exact_span_walk for a span of a DESCENDING list, in far fewer dependent steps: the lanes' maps of
-// their four entries (for the binade r is in) are composed by a scan, the run of lanes that provably neither
-// stops the walk nor leaves the binade is applied at once, the first lane that cannot promise this is replayed
-// with real fp32 operations, and the scan resumes behind it in the binade r has reached.
-__device__ bool scan_span_walk(const uint32_t* kf, uint32_t start, uint32_t len, float& r, uint32_t& pos)
-{
-    using namespace seqfp;
-    float q[4];
-    load_span(kf, start, len, q); // entries past the end read as 0.0f
-    const uint32_t beg = uniform_u32(start);
-    const uint32_t lanes = (uniform_u32(len) + 3u) / 4u;
-    uint32_t Mq0;
-    int eq0;
-    split(q[0], Mq0, eq0); // the lane's largest entry
-    uint32_t done = 0;
-    while (done < lanes) {
-        uint32_t Mv;
-        int ev;
-        split(r, Mv, ev);
-        const uint32_t M = uniform_u32(Mv);
-        const int e = (int)uniform_u32((uint32_t)ev);
-        const bool live = lane_id() >= done && lane_id() < lanes;
-        MAKO_COUNT(28, 1);
-        Step32 v = identity32();
-        if (live) {
+        for (uint32_t b = 0; b < kWave; b += 16u) {
+            if (base + b >= n)
+                break;
 #pragma unroll
-            for (uint32_t j = 0; j < 4; ++j)
-                v = compose32(v, step32(q[j], e));
-        }
-        // the state after this lane's entries must stay at or above its largest entry (no stop inside the lane)
-        // and inside the binade with room for one more decrement
-        uint32_t need = 1u;
-        {
-            const int dl = e - eq0;
-            if (dl < 0)
-                need = 1u << 31;
-            else if (dl <= 25)
-                need = max(1u, (uint32_t)(((unsigned long long)Mq0 + (1ull << dl) - 1ull) >> dl));
-            if (e > 1)
-                need = max(need, min(v.cmax, 1u << 30) + (1u << 23) + 1u);
-        }
-        wave_scan_maps(v.d0, v.d1);
-        const uint32_t dd = (M & 1u) ? v.d1 : v.d0;
-        const bool ok = dd <= M && M - dd >= need;
-        const unsigned long long bad = __ballot(live && !ok);
-        const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : lanes;
-        if (f > done)
-            r = join(uniform_u32((uint32_t)__shfl((int)(M - dd), (int)f - 1)), e);
-        if (f < lanes && f - done < 8u) {
-            // little progress: r is down among the weights themselves, where it changes binade every few entries;
-            // the rest of the span is cheaper entry by entry
-            const float nan = __uint_as_float(0x7fc00000u);
-            float rr = r; // NaN once the walk has stopped: no later comparison succeeds
-            uint32_t at = kNone;
-            MAKO_COUNT(29, lanes - f);
-            for (uint32_t l = f; l < lanes; ++l) {
-#pragma unroll
-                for (uint32_t j = 0; j < 4; ++j) {
-                    const float x = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), l));
-                    const bool stop = rr < x;
-                    at = stop ? beg + l * 4u + j : at;
-                    rr = stop ? nan : rr - x;
-                }
-                if (uniform_u32(at) != kNone) {
-                    pos = uniform_u32(at);
-                    return true;
+            for (uint32_t k = 0; k < 16; ++k)
+                v = ror_sub(v, cur);
+            const uint32_t out = (uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), (b + 15u) & 63u);
+            if (out >> 31) {
+                float rr = r_in;
+                for (uint32_t l = b; l < b + 16u; ++l) {
+                    const float xv = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(cur), l & 63u));
+                    if (__ballot(rr < xv) != 0ull) {
+                        pos = beg + base + l;
+                        MAKO_TOC(1, 18);
+                        return true;
+                    }
+                    rr -= xv;
                 }
             }
-            r = rr;
-            return false;
+            r_in = __uint_as_float(out);
         }
-        if (f < lanes) {
-#pragma unroll
-            for (uint32_t j = 0; j < 4; ++j) {
-                const float x = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(q[j]), f));
-                if (__builtin_amdgcn_readfirstlane((int)(r < x))) {
-                    pos = beg + f * 4u + j;
-                    return true;
-                }
-                r -= x;
-            }
-        }
-        done = f + 1u;
+        x[0] = x[1];
+        x[1] = x[2];
+        x[2] = x[3];
     }
+    r = r_in;
+    MAKO_TOC(1, 18);
     return false;
 }
 
@@ -1786,7 +1775,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
                         MAKO_COUNT(22, 1);
                         float r = join(M, e);
-                        if (scan_span_walk(kf, st, pk & kLenMask, r, at)) {
+                        const bool stop = exact_span_walk(kf, st, pk & kLenMask, r, at);
+                        if (stop) {
                             stopped = true;
                             break;
                         }
