@@ -79,7 +79,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
 {
     if (!out || max_rows == 0 || max_vocab == 0)
         return MAKO_ERR_INVALID_ARG;
-    if (mako_sampler_slices(max_vocab) > mako::kMaxSlices)
+    // (kMaxSlices slices of kSliceMax logits; one logit fewer so that a histogram bin's count fits its 20 bits)
+    if (mako_sampler_slices(max_vocab) > mako::kMaxSlices || max_vocab >= (1u << (64 - mako::kBinSumBits)))
         return MAKO_ERR_INVALID_ARG;
     mako_sampler_ctx* ctx = new (std::nothrow) mako_sampler_ctx;
     if (!ctx)
@@ -99,8 +100,6 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap));
     MAKO_HIP(ctx, dev_alloc(&sc.part_sum, (size_t)max_rows * mako::kMaxSlices));
     MAKO_HIP(ctx, dev_alloc(&sc.part_n, (size_t)max_rows * mako::kMaxSlices));
-    MAKO_HIP(ctx, dev_alloc(&sc.binc, (size_t)max_rows * mako::kBins));
-    MAKO_HIP(ctx, hipMemset(sc.binc, 0, (size_t)max_rows * mako::kBins * sizeof(uint32_t)));
     MAKO_HIP(ctx, dev_alloc(&sc.plan, (size_t)max_rows));
     MAKO_HIP(ctx, hipMemset(sc.plan, 0, (size_t)max_rows * sizeof(mako::BigPlan)));
     MAKO_HIP(ctx, dev_alloc(&sc.bins, (size_t)max_rows * mako::kBins));
@@ -152,7 +151,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
     void* ptrs[] = {ctx->sc_dev, sc.bin_worker, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
-                    sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.binc, sc.bins, sc.plan,
+                    sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.bins, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
                     ctx->st_hist,  ctx->st_hcnt, ctx->st_hlen,  ctx->st_draft, ctx->st_tokens, ctx->st_acc};

@@ -88,6 +88,7 @@ constexpr uint32_t kTopKFast = 128;  // largest top_k resolved from the per-slic
 constexpr uint32_t kSortMax = 4096;  // candidates the finisher sorts in LDS
 constexpr uint32_t kDynLds = 65536;  // dynamic LDS of both kernels
 constexpr uint32_t kBins = 2048;     // weight histogram of top_k == 0 rows, see weight_bin()
+constexpr uint32_t kBinSumBits = 44; // a bin's record: count << 44 | sum of 24-bit significands
 
 // Histogram bin of a weight q in (0, 1], by its bits: 128 bins per binade for the eight binades below 1.0 (bins
 // 1024..2047) and 8 per binade for everything smaller, subnormals included (bins 71..1023; bins below 71 stay
@@ -170,11 +171,12 @@ struct Scratch {
     uint32_t* cand_i;  // [max_rows][slices_cap][kCap] their token ids
     double* part_sum;  // [max_rows][kMaxSlices] exact fp64 sum of q over the slice (top_k == 0 rows)
     uint32_t* part_n;  // [max_rows][kMaxSlices] candidates (q > 0, q >= min_p) in the slice
-    uint32_t* binc;    // [max_rows][kBins] candidates per weight bin (top_k == 0 rows); the slices add their
-                       // counts with atomics, plan_kernel reads the row's bins and leaves them zero
     BigPlan* plan;     // [max_rows]; flag zero between calls
-    unsigned long long* bins; // [max_rows][kBins] sum of the bin's 24-bit significands, likewise: a bin's exact
-                              // mass is bins * 2^(e - 150), e being the bin's exponent
+    unsigned long long* bins; // [max_rows][kBins] weight histogram of top_k == 0 rows: candidates in the bin << 44 |
+                              // sum of their 24-bit significands (kBinSumBits: at most 2^20 - 1 logits per row).
+                              // A bin's exact mass is that sum * 2^(e - 150), e being the bin's exponent.  The
+                              // slices add with one atomic per non-empty bin; plan_kernel reads the row's bins
+                              // and leaves them zero
     float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path; top_k == 0 rows keep
                        // bits(q) of every logit here instead (0 where q is not a candidate)
     uint32_t* cnt;     // [max_rows][vpad] token counts; all zero between calls
@@ -2554,6 +2556,44 @@ __device__ void bitonic_sort_regs(unsigned long long (&key)[ITEMS], unsigned lon
         }
 }
 
+// Keys (bits(q) << 32 | ~token id, 0 = not a candidate) of candidates t * 1024 + tid of the row's flattened
+// candidate list (all slices; sm.soff holds the slices' offsets), t < ITEMS.  Positions first, then every load
+// from a clamped position with no branch in between (a branch around each load would make it wait for the one
+// before), then the weights of the candidates that exist.
+template <int ITEMS>
+__device__ __forceinline__ void candidate_keys(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_cands, float m,
+                                               float inv_t, float floor_q, const FinishShared& sm,
+                                               unsigned long long (&key)[ITEMS])
+{
+    const uint32_t tid = threadIdx.x;
+    size_t at[ITEMS];
+#pragma unroll
+    for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t) {
+        const uint32_t c = t * 1024u + tid < n_cands ? t * 1024u + tid : 0u; // (past the end: candidate 0, a short search)
+        uint32_t s = 0;
+        while (s + 1 < slices && c >= sm.soff[s + 1]) // slice holding candidate c
+            ++s;
+        at[t] = ((size_t)row * sc.slices_cap + s) * kCap + (c - sm.soff[s]);
+    }
+    float w[ITEMS];
+    uint32_t id[ITEMS];
+#pragma unroll
+    for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t)
+        w[t] = sc.cand_w[at[t]];
+#pragma unroll
+    for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t)
+        id[t] = sc.cand_i[at[t]];
+#pragma unroll
+    for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t) {
+        key[t] = 0;
+        if (t * 1024u < n_cands) { // uniform: whole trips past the end of the list are skipped
+            const float q = weight_of(w[t], m, inv_t, sm.tab);
+            if (t * 1024u + tid < n_cands && q >= floor_q && q > 0.0f)
+                key[t] = ((unsigned long long)__float_as_uint(q) << 32) | (unsigned long long)(kNone - id[t]);
+        }
+    }
+}
+
 // The row's candidates (all slices) weighted, sorted by (q desc, idx asc) and left in LDS as kf[i] = ~bits(q_i),
 // jf[i] = token id, invalid ones (q not a candidate) last.  Returns the number of valid candidates.
 template <int ITEMS>
@@ -2563,20 +2603,7 @@ __device__ uint32_t sort_candidates(const Scratch& sc, uint32_t row, uint32_t sl
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
     unsigned long long key[ITEMS];
-#pragma unroll
-    for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t) {
-        const uint32_t c = t * 1024u + tid;
-        key[t] = 0;
-        if (c < n_cands) {
-            uint32_t s = 0;
-            while (s + 1 < slices && c >= sm.soff[s + 1]) // slice holding candidate c
-                ++s;
-            const size_t at = ((size_t)row * sc.slices_cap + s) * kCap + (c - sm.soff[s]);
-            const float q = weight_of(sc.cand_w[at], m, inv_t, sm.tab);
-            if (q >= floor_q && q > 0.0f)
-                key[t] = ((unsigned long long)__float_as_uint(q) << 32) | (unsigned long long)(kNone - sc.cand_i[at]);
-        }
-    }
+    candidate_keys<ITEMS>(sc, row, slices, n_cands, m, inv_t, floor_q, sm, key);
     bitonic_sort_regs<ITEMS>(key, L.sortk);
     uint32_t nv = 0;
 #pragma unroll
@@ -2609,20 +2636,8 @@ __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t s
     uint32_t* rank = reinterpret_cast<uint32_t*>(L.sortk + 256 + kSmall); // [kSmall]
     uint32_t* counter = rank + kSmall;
     unsigned long long key[4];
-#pragma unroll
-    for (uint32_t t = 0; t < 4; ++t) {
-        const uint32_t c = t * 1024u + tid;
-        key[t] = 0;
-        if (c < n_cands) {
-            uint32_t s = 0;
-            while (s + 1 < slices && c >= sm.soff[s + 1]) // slice holding candidate c
-                ++s;
-            const size_t at = ((size_t)row * sc.slices_cap + s) * kCap + (c - sm.soff[s]);
-            const float q = weight_of(sc.cand_w[at], m, inv_t, sm.tab);
-            if (q >= floor_q && q > 0.0f)
-                key[t] = ((unsigned long long)__float_as_uint(q) << 32) | (unsigned long long)(kNone - sc.cand_i[at]);
-        }
-    }
+    candidate_keys<4>(sc, row, slices, n_cands, m, inv_t, floor_q, sm, key);
+    MAKO_STAMP(17);
     if (tid < 512)
         hist[tid] = 0;
     if (tid < kSmall)
@@ -2664,6 +2679,7 @@ __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t s
         n_valid = both >> 16;
         n_list = both & 0xffffu;
     }
+    MAKO_STAMP(18);
     if (n_list > kSmall)
         return kNone;
     // compaction in any order: the keys are distinct, the ranks below put them in place
@@ -2682,13 +2698,18 @@ __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t s
         }
     }
     __syncthreads();
+    MAKO_STAMP(19);
     {
         const uint32_t e = tid & (kSmall - 1u), part = tid / kSmall; // four threads share the comparisons of an entry
         const unsigned long long my = e < n_list ? sel[e] : ~0ull;
-        const uint32_t jb = min(n_list, part * (kSmall / 4u)), je = min(n_list, jb + kSmall / 4u);
+        // each of the four takes a quarter of the list; waves whose entries lie past its end have nothing to count
+        const uint32_t chunk = (n_list + 3u) / 4u, jb = part * chunk, je = min(n_list, jb + chunk);
         uint32_t r = 0;
-        for (uint32_t j = jb; j < je; ++j)
-            r += sel[j] > my;
+        if ((e & ~(kWave - 1u)) < n_list) {
+#pragma unroll 4
+            for (uint32_t j = jb; j < je; ++j)
+                r += sel[j] > my;
+        }
         if (r)
             atomicAdd(&rank[e], r);
         __syncthreads();
@@ -2749,22 +2770,19 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
     }
     // bits(q) of every logit of the slice (0 = not a candidate) and their histogram, for nucleus_big_row()
     uint32_t* qk = reinterpret_cast<uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
-    uint32_t* hist = L.cnt;
-    unsigned long long* hsum = reinterpret_cast<unsigned long long*>(L.cnt + kBins);
-    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads) {
+    unsigned long long* hist = reinterpret_cast<unsigned long long*>(L.cnt); // count << kBinSumBits | significands
+    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads)
         hist[b] = 0;
-        hsum[b] = 0;
-    }
     __syncthreads();
     MAKO_STAMP(26);
-    // significand of a positive float (subnormals: no hidden bit), as seqfp::split
-    auto signif = [](uint32_t b) { return (unsigned long long)((b & 0x7fffffu) | ((b >> 23) ? 0x800000u : 0u)); };
+    // one candidate and the significand of a positive float (subnormals: no hidden bit, as seqfp::split)
+    auto record = [](uint32_t b) {
+        return (1ull << kBinSumBits) | (unsigned long long)((b & 0x7fffffu) | ((b >> 23) ? 0x800000u : 0u));
+    };
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j)
-        if (qb[j]) {
-            atomicAdd(&hist[weight_bin(qb[j])], 1u);
-            atomicAdd(&hsum[weight_bin(qb[j])], signif(qb[j]));
-        }
+        if (qb[j])
+            atomicAdd(&hist[weight_bin(qb[j])], record(qb[j]));
     if (VEC) {
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k) {
@@ -2785,21 +2803,16 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
     for (int k = 0; k < (PEN ? KH : 0); ++k)
         if (ex.i[k] != kNone) {
             qk[ex.i[k]] = qe[k];
-            if (qe[k]) {
-                atomicAdd(&hist[weight_bin(qe[k])], 1u);
-                atomicAdd(&hsum[weight_bin(qe[k])], signif(qe[k]));
-            }
+            if (qe[k])
+                atomicAdd(&hist[weight_bin(qe[k])], record(qe[k]));
         }
     __syncthreads();
     MAKO_STAMP(27);
     // the slice's non-empty bins are added to the row's histogram (a few hundred atomics per slice, none waited for)
-    uint32_t* binc = sc.binc + (size_t)row * kBins;
     unsigned long long* bins = sc.bins + (size_t)row * kBins;
     for (uint32_t b = threadIdx.x; b < kBins; b += kThreads)
-        if (hist[b]) {
-            atomicAdd(&binc[b], hist[b]);
-            atomicAdd(&bins[b], hsum[b]);
-        }
+        if (hist[b])
+            atomicAdd(&bins[b], hist[b]);
 }
 
 // Kernel arguments that are handed on by reference to out-of-line device functions would be spilled to scratch
@@ -3015,10 +3028,10 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
     MAKO_STAMP(2);
     // this thread's two bins of the row's histogram (left zero for the next batch), the slices' exact sums in order
-    uint32_t* binc = sc.binc + (size_t)row * kBins;
     unsigned long long* bins = sc.bins + (size_t)row * kBins;
-    const uint32_t bin_c0 = binc[kBins - 1u - 2u * tid], bin_c1 = binc[kBins - 2u - 2u * tid];
-    const unsigned long long bin_s0 = bins[kBins - 1u - 2u * tid], bin_s1 = bins[kBins - 2u - 2u * tid];
+    const unsigned long long rec0 = bins[kBins - 1u - 2u * tid], rec1 = bins[kBins - 2u - 2u * tid];
+    const uint32_t bin_c0 = (uint32_t)(rec0 >> kBinSumBits), bin_c1 = (uint32_t)(rec1 >> kBinSumBits);
+    const unsigned long long bin_s0 = rec0 & ((1ull << kBinSumBits) - 1ull), bin_s1 = rec1 & ((1ull << kBinSumBits) - 1ull);
     double row_total = 0;
     uint32_t row_n0 = 0;
     for (uint32_t s0 = 0; s0 < slices; s0 += 8u) {
@@ -3037,14 +3050,10 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
                 row_n0 += pn[u];
             }
     }
-    if (bin_c0) {
-        binc[kBins - 1u - 2u * tid] = 0;
+    if (rec0)
         bins[kBins - 1u - 2u * tid] = 0;
-    }
-    if (bin_c1) {
-        binc[kBins - 2u - 2u * tid] = 0;
+    if (rec1)
         bins[kBins - 2u - 2u * tid] = 0;
-    }
     float m;
     uint32_t argidx, n_cands, any_overflow;
     row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
