@@ -7,6 +7,16 @@
 
 #include "seqfp.h"
 
+// Wavefront reductions and scans of the device library (DPP row shifts and broadcasts: a dozen instructions where
+// a shuffle-based butterfly pays six trips through the LDS crossbar).
+extern "C" __device__ uint32_t __ockl_wfred_add_u32(uint32_t);
+extern "C" __device__ uint32_t __ockl_wfred_min_u32(uint32_t);
+extern "C" __device__ uint32_t __ockl_wfred_max_u32(uint32_t);
+extern "C" __device__ unsigned long long __ockl_wfred_max_u64(unsigned long long);
+extern "C" __device__ double __ockl_wfred_add_f64(double);
+extern "C" __device__ uint32_t __ockl_wfscan_add_u32(uint32_t, bool inclusive);
+extern "C" __device__ double __ockl_wfscan_add_f64(double, bool inclusive);
+
 namespace mako {
 
 constexpr int kThreads = 1024;
@@ -41,8 +51,7 @@ struct BlockScratch {
 
 __device__ __forceinline__ uint32_t block_sum_u32(uint32_t v, BlockScratch& s)
 {
-    for (int o = 32; o > 0; o >>= 1)
-        v += __shfl_xor(v, o);
+    v = __ockl_wfred_add_u32(v);
     if (lane_id() == 0)
         s.u64[wave_id()] = v;
     __syncthreads();
@@ -55,8 +64,7 @@ __device__ __forceinline__ uint32_t block_sum_u32(uint32_t v, BlockScratch& s)
 
 __device__ __forceinline__ uint32_t block_min_u32(uint32_t v, BlockScratch& s)
 {
-    for (int o = 32; o > 0; o >>= 1)
-        v = min(v, (uint32_t)__shfl_xor(v, o));
+    v = __ockl_wfred_min_u32(v);
     if (lane_id() == 0)
         s.u64[wave_id()] = v;
     __syncthreads();
@@ -69,10 +77,7 @@ __device__ __forceinline__ uint32_t block_min_u32(uint32_t v, BlockScratch& s)
 
 __device__ __forceinline__ unsigned long long block_max_u64(unsigned long long v, BlockScratch& s)
 {
-    for (int o = 32; o > 0; o >>= 1) {
-        const unsigned long long t = __shfl_xor(v, o);
-        v = t > v ? t : v;
-    }
+    v = __ockl_wfred_max_u64(v);
     if (lane_id() == 0)
         s.u64[wave_id()] = v;
     __syncthreads();
@@ -86,12 +91,7 @@ __device__ __forceinline__ unsigned long long block_max_u64(unsigned long long v
 // Exclusive prefix sum in thread order; `total` receives the workgroup sum.
 __device__ __forceinline__ uint32_t block_excl_scan_u32(uint32_t v, uint32_t& total, BlockScratch& s)
 {
-    uint32_t incl = v;
-    for (int o = 1; o < kWave; o <<= 1) {
-        const uint32_t t = __shfl_up(incl, o);
-        if (lane_id() >= o)
-            incl += t;
-    }
+    const uint32_t incl = __ockl_wfscan_add_u32(v, true);
     if (lane_id() == kWave - 1)
         s.u64[wave_id()] = incl;
     __syncthreads();
@@ -107,12 +107,11 @@ __device__ __forceinline__ uint32_t block_excl_scan_u32(uint32_t v, uint32_t& to
     return pre + incl - v;
 }
 
-// Sum of doubles in a fixed order (lanes by butterfly, then waves in order):
+// Sum of doubles in a fixed order (the wavefront reduction's, then waves in order):
 // the same inputs always give the same bits.
 __device__ __forceinline__ double block_sum_f64(double v, BlockScratch& s)
 {
-    for (int o = 32; o > 0; o >>= 1)
-        v += __shfl_xor(v, o);
+    v = __ockl_wfred_add_f64(v);
     if (lane_id() == 0)
         s.f64[wave_id()] = v;
     __syncthreads();
@@ -126,11 +125,7 @@ __device__ __forceinline__ double block_sum_f64(double v, BlockScratch& s)
 // Inclusive prefix sum of doubles in thread order; fixed association.
 __device__ __forceinline__ double block_incl_scan_f64(double v, double& total, BlockScratch& s)
 {
-    for (int o = 1; o < kWave; o <<= 1) {
-        const double t = __shfl_up(v, o);
-        if (lane_id() >= o)
-            v += t;
-    }
+    v = __ockl_wfscan_add_f64(v, true);
     if (lane_id() == kWave - 1)
         s.f64[wave_id()] = v;
     __syncthreads();
