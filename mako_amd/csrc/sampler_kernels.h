@@ -1072,6 +1072,15 @@ __device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
 
 // Values every lane of the wave holds alike, moved to scalar registers so that loops and branches on them
 // compile to scalar control flow.
+// A double from a lane whose number is the same for the whole wave.
+__device__ __forceinline__ double readlane_f64(double v, uint32_t lane)
+{
+    const long long b = __double_as_longlong(v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, (int)lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), (int)lane);
+    return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
 __device__ __forceinline__ uint32_t uniform_u32(uint32_t v)
 {
     return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
@@ -1486,14 +1495,9 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             p[1] = p[0] + (double)q[1];
             p[2] = p[1] + (double)q[2];
             p[3] = p[2] + (double)q[3];
-            double incl = p[3];
-            for (int o = 1; o < kWave; o <<= 1) {
-                const double t = __shfl_up(incl, o);
-                if (lane_id() >= o)
-                    incl += t;
-            }
+            const double incl = __ockl_wfscan_add_f64(p[3], true);
             if (!have_total)
-                total64 = __shfl(incl, kWave - 1);
+                total64 = readlane_f64(incl, kWave - 1);
             uint32_t n = n1;
             bool ok = true;
             if (topp_active) {
@@ -1506,7 +1510,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         hit = lane_id() * 4u + (uint32_t)j;
                 const unsigned long long bal = __ballot(hit != kNone && hit < n1);
                 if (bal)
-                    n = (uint32_t)__shfl((int)hit, __ffsll((long long)bal) - 1) + 1u;
+                    n = (uint32_t)__builtin_amdgcn_readlane((int)hit, __ffsll((long long)bal) - 1) + 1u;
                 else
                     ok = !need_cut;
             }
@@ -1586,9 +1590,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             }
 #pragma unroll
             for (uint32_t u = 0; u < 4; ++u) {
-                double s = (((double)q[u][0] + (double)q[u][1]) + (double)q[u][2]) + (double)q[u][3];
-                for (int o = 32; o > 0; o >>= 1)
-                    s += __shfl_xor(s, o);
+                const double s = __ockl_wfred_add_f64((((double)q[u][0] + (double)q[u][1]) + (double)q[u][2]) + (double)q[u][3]);
                 if (lane_id() == 0 && g0 + u < groups1)
                     G.pg()[g0 + u + 1] = s;
             }
@@ -1627,12 +1629,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 p[1] = p[0] + (double)q[1];
                 p[2] = p[1] + (double)q[2];
                 p[3] = p[2] + (double)q[3];
-                double incl = p[3];
-                for (int o = 1; o < kWave; o <<= 1) {
-                    const double t = __shfl_up(incl, o);
-                    if (lane_id() >= o)
-                        incl += t;
-                }
+                const double incl = __ockl_wfscan_add_f64(p[3], true);
                 const double base = G.pg()[gs] + (incl - p[3]);
                 uint32_t hit = kNone;
 #pragma unroll
@@ -1642,7 +1639,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 const unsigned long long bal = __ballot(hit != kNone && hit < len);
                 uint32_t keep = len;
                 if (bal)
-                    keep = (uint32_t)__shfl((int)hit, __ffsll((long long)bal) - 1) + 1u;
+                    keep = (uint32_t)__builtin_amdgcn_readlane((int)hit, __ffsll((long long)bal) - 1) + 1u;
                 if (lane_id() == 0) {
                     G.misc()[0] = st + keep;
                     if (keep != len)
@@ -1692,7 +1689,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 const unsigned long long bad = __ballot(live && !ok);
                 const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : cnt;
                 if (f > done)
-                    M = uniform_u32((uint32_t)__shfl((int)after, (int)f - 1));
+                    M = (uint32_t)__builtin_amdgcn_readlane((int)after, (int)f - 1);
                 if (f < cnt) {
                     const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
                     const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
@@ -1771,7 +1768,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     const unsigned long long bad = __ballot(live && !ok);
                     const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : cnt;
                     if (f > done)
-                        M = uniform_u32((uint32_t)__shfl((int)(M - dd), (int)f - 1));
+                        M = (uint32_t)__builtin_amdgcn_readlane((int)(M - dd), (int)f - 1);
                     if (f < cnt) {
                         const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
                         const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
@@ -1989,8 +1986,7 @@ __device__ uint32_t gather_range(const uint32_t* qk, uint32_t V, uint32_t key_lo
             for (uint32_t j = 0; j < 4; ++j)
                 mine += k[u][j] != 0;
     }
-    for (int o = 32; o > 0; o >>= 1)
-        mine += __shfl_xor(mine, o);
+    mine = __ockl_wfred_add_u32(mine);
     __syncthreads();
     if (lane == 0)
         sm.bs.u64[wave] = mine;
@@ -2382,9 +2378,7 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
     for (uint32_t g = wave_id(); g < groups; g += kWaves) {
         float q[4];
         load_span(kf, off + g * kGroup, min(kGroup, cnt - g * kGroup), q);
-        double s = (((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3];
-        for (int o = 32; o > 0; o >>= 1)
-            s += __shfl_xor(s, o);
+        const double s = __ockl_wfred_add_f64((((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3]);
         if (lane_id() == 0)
             gs[g] = s;
     }
@@ -2692,7 +2686,7 @@ __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t s
             uint32_t base = 0;
             if (lane_id() == (uint32_t)__ffsll((long long)bal) - 1u)
                 base = atomicAdd(counter, (uint32_t)__popcll(bal));
-            base = (uint32_t)__shfl((int)base, __ffsll((long long)bal) - 1);
+            base = (uint32_t)__builtin_amdgcn_readlane((int)base, __ffsll((long long)bal) - 1);
             if (keep)
                 sel[base + (uint32_t)__popcll(bal & lower)] = key[t];
         }
