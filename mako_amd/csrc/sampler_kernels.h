@@ -1058,15 +1058,24 @@ struct GroupLds { // carved from the dynamic LDS block once sorting is over; one
     __device__ __forceinline__ uint32_t* misc() const { return pack() + kMaxGroups; } // [4]; misc[3] counts the quarter-record slots in use
     // [kQuarterSlots][4], in the upper half of the dynamic LDS block
     __device__ __forceinline__ uint4* quarters() const { return reinterpret_cast<uint4*>(base + kSortMax); }
+    // the walk's maps, bounds and packs ([kMaxGroups] each, behind the quarter records): built while the running
+    // sum is still being chained, so they cannot share the arrays above
+    __device__ __forceinline__ uint32_t* w_d0() const { return reinterpret_cast<uint32_t*>(base + kSortMax) + 1536; }
+    __device__ __forceinline__ uint32_t* w_d1() const { return w_d0() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* w_need() const { return w_d1() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* w_pack() const { return w_need() + kMaxGroups; }
 };
 constexpr uint32_t kLenMask = 0x1ffu;
 constexpr uint32_t kHasQuarters = 1u << 31;
 constexpr uint32_t kQuarterSlots = 96;
 constexpr uint32_t kQuarter = kGroup / 4;
+constexpr uint32_t kSeqMax = 1024; // sorted lists up to this long get their total and walk entry by entry
 
 __device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
 {
     static_assert((kMaxGroups + 2) * 8 + 5 * kMaxGroups * 4 + 16 <= kSortMax * 8, "group records fit below the LDS lists");
+    static_assert(kQuarterSlots * 16 == 1536 && kSortMax * 8 + 1536 * 4 + 4 * kMaxGroups * 4 <= kDynLds,
+                  "the walk's records sit behind the quarter records and fit the dynamic LDS block");
     return GroupLds{L.sortk};
 }
 
@@ -1134,11 +1143,15 @@ __device__ __forceinline__ void load_span(const uint32_t* kf, uint32_t start, ui
         k[1] = x.y;
         k[2] = x.z;
         k[3] = x.w;
-    } else {
+    } else if (len) {
+        // (every load from a position inside the span, none behind a branch of its own: they are in flight together)
+        uint32_t t[4];
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
-            if (i + j < len)
-                k[j] = kf[start + i + j];
+            t[j] = kf[start + min(i + j, len - 1u)];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            k[j] = i + j < len ? t[j] : k[j];
     }
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j)
@@ -1216,23 +1229,33 @@ __device__ void build_quarters(const float (&q)[4], uint32_t len, double at_star
         out[quarter] = make_uint4(v.d0, v.d1, cm, (uint32_t)eg);
 }
 
-// Group maps of groups [0, groups) for epochs guessed from pg: sum (walk == false) or walk from r0.
-__device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk, double r0, const GroupLds G)
+// Group maps of groups [0, groups) for epochs guessed from pg: of the running sum (walk == false, into G.d0 / d1 /
+// cmax / pack) or of the walk from r0 (into G.w_d0 / w_d1 / w_need / w_pack).  The calling wave is number `part` of
+// `parts` that share the work.
+__device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk, double r0, const GroupLds G,
+                                 uint32_t part = wave_id(), uint32_t parts = kWaves)
 {
     using namespace seqfp;
-    // four groups per trip and wave, their loads issued together
-    for (uint32_t g0 = wave_id() * 4u; g0 < groups; g0 += kWaves * 4u) {
+    uint32_t* const o_d0 = walk ? G.w_d0() : G.d0();
+    uint32_t* const o_d1 = walk ? G.w_d1() : G.d1();
+    uint32_t* const o_c = walk ? G.w_need() : G.cmax();
+    uint32_t* const o_pack = walk ? G.w_pack() : G.pack();
+    // Up to four groups per trip and wave, their loads issued together; a wave's groups lie `parts` apart, so that a
+    // short list is spread over all the waves (a map costs a wave about a microsecond).
+    for (uint32_t g0 = part; g0 < groups; g0 += parts * 4u) {
         float q[4][4];
         uint32_t len[4];
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
-            const uint32_t g = min(g0 + u, groups - 1u);
+            const uint32_t g = min(g0 + u * parts, groups - 1u);
             len[u] = uniform_u32(G.pack()[g] & kLenMask);
             load_span(kf, uniform_u32(G.start()[g]), len[u], q[u]);
         }
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
-            const uint32_t g = g0 + u;
+            const uint32_t g = g0 + u * parts;
+            if (g >= groups) // uniform
+                break;
             const double guess = g < groups ? (walk ? r0 - G.pg()[g] : G.pg()[g]) : 0.0;
             const int eg = guess > 0 ? exponent_of((float)guess) : 0;
             const Step32 st = span_map(q[u], len[u], eg);
@@ -1270,10 +1293,10 @@ __device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk,
                     if (eg > 1)
                         third = max(third, min(st.cmax, 1u << 30) + (1u << 23) + 1u);
                 }
-                G.d0()[g] = st.d0;
-                G.d1()[g] = st.d1;
-                G.cmax()[g] = third;
-                G.pack()[g] = len[u] | (slot << 9) | ((uint32_t)eg << 16);
+                o_d0[g] = st.d0;
+                o_d1[g] = st.d1;
+                o_c[g] = third;
+                o_pack[g] = len[u] | (slot << 9) | ((uint32_t)eg << 16);
             }
         }
     }
@@ -1369,13 +1392,60 @@ __device__ float exact_span_sum(const uint32_t* kf, uint32_t start, uint32_t len
     return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), (steps - 1u) & 63u));
 }
 
-// The entries of one span (len in 1..256) subtracted from r one by one (src/gen/sampler.cpp:67-71).  Returns true
-// and the entry's position in the list when the walk stops inside the span, else false and the new r.  One wave.
+// The entries of one span (n in 1..256, in registers as load_span_lanes() leaves them; the span starts at entry
+// `beg` of the list) subtracted from r one by one (src/gen/sampler.cpp:67-71).  Returns true and the entry's
+// position in the list when the walk stops inside the span, else false and the new r.  One wave.
 //
 // The walk stops at the first entry with r < x, which is the first entry whose subtraction turns r negative (x != r
 // gives a nonzero difference, denormals kept), and a negative r stays negative under every later subtraction of a
-// weight.  So sixteen entries are subtracted without looking, and only a block that ends negative is walked again
-// from its saved start to find the entry.
+// weight.  So 64 entries are subtracted without looking; only a block that ends negative is gone through again,
+// sixteen entries at a time, and the sixteen that turn r negative one by one.
+__device__ __forceinline__ bool walk_lanes(float (&x)[4], uint32_t n, uint32_t beg, float& r, uint32_t& pos)
+{
+    float v = r;    // uniform
+    float r_in = r; // the walk's value in front of the current block
+    for (uint32_t base = 0; base < n; base += kWave) {
+        const float cur = x[0];
+        const bool whole = n - base > 48u; // (a short rest goes sixteen at a time straight away)
+        uint32_t out = 0x80000000u;
+        if (whole) {
+#pragma unroll
+            for (uint32_t k = 0; k < kWave; ++k)
+                v = ror_sub(v, cur);
+            out = (uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), kWave - 1);
+        }
+        if (out >> 31) {
+            v = r_in;
+            for (uint32_t b = 0; b < kWave && base + b < n; b += 16u) {
+#pragma unroll
+                for (uint32_t k = 0; k < 16; ++k)
+                    v = ror_sub(v, cur);
+                const uint32_t o16 = (uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), (b + 15u) & 63u);
+                if (o16 >> 31) {
+                    float rr = r_in;
+                    for (uint32_t l = b; l < b + 16u; ++l) {
+                        const float xv =
+                            __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(cur), l & 63u));
+                        if (__ballot(rr < xv) != 0ull) {
+                            pos = beg + base + l;
+                            return true;
+                        }
+                        rr -= xv;
+                    }
+                }
+                r_in = __uint_as_float(o16);
+            }
+        }
+        if (whole)
+            r_in = __uint_as_float(out);
+        x[0] = x[1];
+        x[1] = x[2];
+        x[2] = x[3];
+    }
+    r = r_in;
+    return false;
+}
+
 __device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len, float& r, uint32_t& pos)
 {
     float x[4];
@@ -1383,43 +1453,8 @@ __device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len
     const uint32_t beg = uniform_u32(start);
     if (n == 0)
         return false;
-    MAKO_TIC(0);
     load_span_lanes(kf, beg, n, x);
-    MAKO_TOC(0, 17);
-    MAKO_TIC(1);
-    float v = r;    // uniform
-    float r_in = r; // the walk's value in front of the current block
-    for (uint32_t base = 0; base < n; base += kWave) {
-        const float cur = x[0];
-#pragma unroll
-        for (uint32_t b = 0; b < kWave; b += 16u) {
-            if (base + b >= n)
-                break;
-#pragma unroll
-            for (uint32_t k = 0; k < 16; ++k)
-                v = ror_sub(v, cur);
-            const uint32_t out = (uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), (b + 15u) & 63u);
-            if (out >> 31) {
-                float rr = r_in;
-                for (uint32_t l = b; l < b + 16u; ++l) {
-                    const float xv = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(cur), l & 63u));
-                    if (__ballot(rr < xv) != 0ull) {
-                        pos = beg + base + l;
-                        MAKO_TOC(1, 18);
-                        return true;
-                    }
-                    rr -= xv;
-                }
-            }
-            r_in = __uint_as_float(out);
-        }
-        x[0] = x[1];
-        x[1] = x[2];
-        x[2] = x[3];
-    }
-    r = r_in;
-    MAKO_TOC(1, 18);
-    return false;
+    return walk_lanes(x, n, beg, r, pos);
 }
 
 // Tail of every path that ends with a list sorted by (q desc, idx asc): kf[i] = ~bits(q_i), jf[i] = token id,
@@ -1660,12 +1695,90 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         return false;
     __syncthreads();
 
-    // exact fp32 total: group maps in parallel (here, or already by the workers), then one wave chains them
+    // candidates and the row's results, once total and position are known
+    auto emit = [&](float total, uint32_t pos) {
+        if (d.out_cand_idx && d.out_cand_q)
+            for (uint32_t j = tid; j < n && j < d.cand_cap; j += kThreads) {
+                d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
+                d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
+            }
+        if (tid == 0) {
+            RowOut o;
+            o.token = (int32_t)idat(pos);
+            o.n_cand = n;
+            o.total = total;
+            o.q = qat(pos);
+            o.path = path;
+            o.accepted = 0;
+            write_row(d, row, o);
+        }
+    };
+
     MAKO_STAMP(7);
+    if (n <= kSeqMax) {
+        // A nucleus this short is gone through entry by entry, once for the total and once for the walk (five
+        // nanoseconds an entry each way): the group maps below only pay on longer lists.
+        if (wave_id() == 0) {
+            float S = 0.0f;
+            for (uint32_t b = 0; b < n; b += kGroup)
+                S = exact_span_sum(kf, b, min(kGroup, n - b), S);
+            const float span = S - 0.0f;
+            const float prod = d.u[row] * span;
+            const float r0 = prod + 0.0f;
+            uint32_t at = n - 1;
+            if (r0 < 0.0f) {
+                at = 0;
+            } else if (r0 == r0 && r0 != INFINITY) {
+                float r = r0;
+                for (uint32_t b = 0; b < n; b += kGroup)
+                    if (exact_span_walk(kf, b, min(kGroup, n - b), r, at))
+                        break;
+            }
+            if (lane_id() == 0) {
+                G.misc()[1] = __float_as_uint(S);
+                G.misc()[2] = at;
+            }
+        }
+        __syncthreads();
+        MAKO_STAMP(9);
+        emit(__uint_as_float(G.misc()[1]), G.misc()[2]);
+        return true;
+    }
+
+    // exact fp32 total: group maps in parallel (here, or already by the workers), then one wave chains them
     if (!PLANNED)
         build_group_maps(kf, groups, false, 0.0, G);
     __syncthreads();
     MAKO_STAMP(13);
+    // While one wave chains the running sum, the others already prepare the walk: its maps only need the binade r is
+    // expected to be in at each group, and the fp64 sums give that (a wrong guess costs a replay, never the result).
+    // Groups that start after the mass r0 could have is used up get no map.
+    const double r0_guess = (double)d.u[row] * G.pg()[groups];
+    uint32_t reach;
+    {
+        const uint32_t beyond = (tid < groups && !(r0_guess * 1.001 - G.pg()[tid] > 0)) ? tid : kNone;
+        reach = min(groups, block_min_u32(beyond, sm.bs));
+        if (tid < groups)
+            G.w_pack()[tid] = G.pack()[tid] & kLenMask;
+        __syncthreads();
+    }
+#ifdef MAKO_TIMING
+    if (tid == 0 && s_mako_row == 0) {
+        g_mako_stamp[20] = groups;
+        g_mako_stamp[21] = reach;
+        g_mako_stamp[22] = n;
+    }
+    const unsigned long long tb0 = wall_clock64();
+#endif
+    if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess) {
+        // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
+        build_group_maps(kf, reach, true, r0_guess, G, (uint32_t)(wave_id() >> 2) * 3u + (uint32_t)(wave_id() & 3) - 1u,
+                         3u * kWaves / 4u);
+#ifdef MAKO_TIMING
+        if (tid == 64 && s_mako_row == 0)
+            g_mako_stamp[23] = wall_clock64() - tb0;
+#endif
+    }
     if (wave_id() == 0) {
         // 64 groups at a time, one per lane.  A scan composes the lanes' maps; every lane then knows the state after
         // its group, provided all groups so far share the running epoch and stay inside the binade.  The run up to the
@@ -1728,16 +1841,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     if (r0 < 0.0f) {
         pos = 0;
     } else if (r0 == r0 && r0 != INFINITY) {
-        // only the groups that start before the mass r0 has been used up can be reached; the others get no map
-        const uint32_t beyond = (tid < groups && !((double)r0 - G.pg()[tid] > 0)) ? tid : kNone;
-        const uint32_t reach = min(groups, block_min_u32(beyond, sm.bs));
-        if (tid >= reach && tid < groups)
-            G.pack()[tid] &= kLenMask;
-        if (tid == 0)
-            G.misc()[3] = 0; // the running sum's quarter records are done with
-        __syncthreads();
-        build_group_maps(kf, reach, true, (double)r0, G);
-        __syncthreads();
         MAKO_STAMP(14);
         if (wave_id() == 0) {
             uint32_t M;
@@ -1753,8 +1856,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             bool stopped = false;
             for (uint32_t base = 0; base < groups && !stopped; base += kWave) {
                 const uint32_t gl = min(base + lane_id(), groups - 1u);
-                const uint32_t pk_l = G.pack()[gl], st_l = G.start()[gl];
-                const uint32_t d0_l = G.d0()[gl], d1_l = G.d1()[gl], need_l = G.cmax()[gl]; // (the bound, see build_group_maps)
+                const uint32_t pk_l = G.w_pack()[gl], st_l = G.start()[gl];
+                const uint32_t d0_l = G.w_d0()[gl], d1_l = G.w_d1()[gl], need_l = G.w_need()[gl]; // (the bound, see build_group_maps)
                 const uint32_t cnt = min((uint32_t)kWave, groups - base);
                 uint32_t done = 0;
                 while (done < cnt) {
@@ -1769,23 +1872,65 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : cnt;
                     if (f > done)
                         M = (uint32_t)__builtin_amdgcn_readlane((int)(M - dd), (int)f - 1);
-                    if (f < cnt) {
-                        const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
-                        const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
-                        MAKO_COUNT(22, 1);
-                        float r = join(M, e);
-                        const bool stop = exact_span_walk(kf, st, pk & kLenMask, r, at);
-                        if (stop) {
-                            stopped = true;
-                            break;
-                        }
-                        uint32_t Mv;
-                        int ev;
-                        split(r, Mv, ev);
-                        M = uniform_u32(Mv);
-                        e = (int)uniform_u32((uint32_t)ev);
+                    if (f >= cnt)
+                        break;
+                    // Group f goes entry by entry.  Where one group does, its neighbours tend to follow (r is down
+                    // among the weights and changes binade every few entries), so the groups behind it are tried one
+                    // at a time with a few scalar operations each, the next one's entries already on their way,
+                    // and the scan takes over again once four in a row have gone through as maps.
+                    uint32_t g = f, passed = 0;
+                    float xa[4];
+                    {
+                        const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g);
+                        const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g);
+                        if (pk & kLenMask)
+                            load_span_lanes(kf, st, pk & kLenMask, xa);
                     }
-                    done = f + 1u;
+                    while (g < cnt && passed < 4u) {
+                        const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g);
+                        const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g);
+                        const uint32_t g1 = min(g + 1u, cnt - 1u);
+                        const uint32_t st1 = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g1);
+                        const uint32_t pk1 = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g1);
+                        float xb[4];
+                        if (pk1 & kLenMask)
+                            load_span_lanes(kf, st1, pk1 & kLenMask, xb); // (used only if group g + 1 is replayed)
+                        bool by_map = false;
+                        if (g != f && (pk >> 16) == (uint32_t)e) {
+                            const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, g);
+                            const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d1_l, g);
+                            const uint32_t need = (uint32_t)__builtin_amdgcn_readlane((int)need_l, g);
+                            const uint32_t d1g = (M & 1u) ? d1 : d0;
+                            if (d1g <= M && M - d1g >= need) { // group_sub_ok
+                                M -= d1g;
+                                by_map = true;
+                            }
+                        }
+                        if (by_map) {
+                            ++passed;
+                        } else {
+                            MAKO_COUNT(22, 1);
+                            passed = 0;
+                            float r = join(M, e);
+                            if ((pk & kLenMask) && walk_lanes(xa, pk & kLenMask, st, r, at)) {
+                                stopped = true;
+                                break;
+                            }
+                            uint32_t Mv;
+                            int ev;
+                            split(r, Mv, ev);
+                            M = uniform_u32(Mv);
+                            e = (int)uniform_u32((uint32_t)ev);
+                        }
+                        xa[0] = xb[0];
+                        xa[1] = xb[1];
+                        xa[2] = xb[2];
+                        xa[3] = xb[3];
+                        ++g;
+                    }
+                    if (stopped)
+                        break;
+                    done = g;
                 }
             }
             if (lane_id() == 0)
@@ -1796,21 +1941,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     }
 
     MAKO_STAMP(9);
-    if (d.out_cand_idx && d.out_cand_q)
-        for (uint32_t j = tid; j < n && j < d.cand_cap; j += kThreads) {
-            d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
-            d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
-        }
-    if (tid == 0) {
-        RowOut o;
-        o.token = (int32_t)idat(pos);
-        o.n_cand = n;
-        o.total = total;
-        o.q = qat(pos);
-        o.path = path;
-        o.accepted = 0;
-        write_row(d, row, o);
-    }
+    emit(total, pos);
     return true;
 }
 
