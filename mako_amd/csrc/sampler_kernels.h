@@ -17,6 +17,8 @@
 #include <math.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/mako_sampler.h"
 #include "block_prims.h"
 #include "device_math.h"
@@ -1070,6 +1072,7 @@ constexpr uint32_t kHasQuarters = 1u << 31;
 constexpr uint32_t kQuarterSlots = 96;
 constexpr uint32_t kQuarter = kGroup / 4;
 constexpr uint32_t kSeqMax = 1024; // sorted lists up to this long get their total and walk entry by entry
+constexpr uint32_t kWalkSeqGroups = 8; // a walk expected to end within this many groups gets no maps
 
 __device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
 {
@@ -1131,31 +1134,55 @@ __device__ __forceinline__ int exponent_of(float x)
     return e;
 }
 
+// A sorted list's keys, wherever they are (LDS or device memory: loads through a generic pointer, which the
+// hardware completes in no particular order, so that the code has to wait for all of them at once) ...
+struct AnyKeys {
+    const uint32_t* p;
+    __device__ __forceinline__ uint32_t operator[](uint32_t i) const { return p[i]; }
+    __device__ __forceinline__ uint4 vec(uint32_t i) const { return *reinterpret_cast<const uint4*>(p + i); }
+};
+// ... or known to be in device memory: plain global loads, which can be left in flight and waited for one by one.
+struct GlobalKeys {
+    const uint32_t* p;
+    __device__ __forceinline__ uint32_t operator[](uint32_t i) const
+    {
+        return ((const __attribute__((address_space(1))) uint32_t*)p)[i];
+    }
+    __device__ __forceinline__ uint4 vec(uint32_t i) const
+    {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 v = *((const __attribute__((address_space(1))) u32x4*)(p + i));
+        return make_uint4(v.x, v.y, v.z, v.w);
+    }
+};
+
 // The four weights a lane owns in the span of `len` (<= kGroup) entries that starts at kf[start]: entries
 // 4 * lane .. 4 * lane + 3, 0.0f past the end.  kf itself is 16-byte aligned.
-__device__ __forceinline__ void load_span(const uint32_t* kf, uint32_t start, uint32_t len, float (&q)[4])
+template <typename Keys>
+__device__ __forceinline__ void load_span(Keys kf, uint32_t start, uint32_t len, float (&q)[4])
 {
     const uint32_t i = lane_id() * 4u;
-    uint32_t k[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu}; // ~bits(0.0f)
+    uint32_t k[4] = {0u, 0u, 0u, 0u}; // bits(0.0f)
     if ((start & 3u) == 0 && i + 3 < len) {
-        const uint4 x = *reinterpret_cast<const uint4*>(kf + start + i);
-        k[0] = x.x;
-        k[1] = x.y;
-        k[2] = x.z;
-        k[3] = x.w;
+        const uint4 x = kf.vec(start + i);
+        k[0] = ~x.x;
+        k[1] = ~x.y;
+        k[2] = ~x.z;
+        k[3] = ~x.w;
     } else if (len) {
-        // (every load from a position inside the span, none behind a branch of its own: they are in flight together)
-        uint32_t t[4];
+        // (every load from a position inside the span, and what lies past the end masked with an AND: a select
+        // would be turned into a branch around each load, and each would wait for the one before)
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
-            t[j] = kf[start + min(i + j, len - 1u)];
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            k[j] = i + j < len ? t[j] : k[j];
+            k[j] = ~kf[start + min(i + j, len - 1u)] & (i + j < len ? 0xffffffffu : 0u);
     }
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j)
-        q[j] = __uint_as_float(~k[j]);
+        q[j] = __uint_as_float(k[j]);
+}
+__device__ __forceinline__ void load_span(const uint32_t* kf, uint32_t start, uint32_t len, float (&q)[4])
+{
+    load_span(AnyKeys{kf}, start, len, q);
 }
 
 // Composition of the 64 lanes' maps in lane order; every lane receives the result.
@@ -1232,7 +1259,8 @@ __device__ void build_quarters(const float (&q)[4], uint32_t len, double at_star
 // Group maps of groups [0, groups) for epochs guessed from pg: of the running sum (walk == false, into G.d0 / d1 /
 // cmax / pack) or of the walk from r0 (into G.w_d0 / w_d1 / w_need / w_pack).  The calling wave is number `part` of
 // `parts` that share the work.
-__device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk, double r0, const GroupLds G,
+template <typename Keys>
+__device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0, const GroupLds G,
                                  uint32_t part = wave_id(), uint32_t parts = kWaves)
 {
     using namespace seqfp;
@@ -1302,54 +1330,32 @@ __device__ void build_group_maps(const uint32_t* kf, uint32_t groups, bool walk,
     }
 }
 
-__device__ float exact_span_sum(const uint32_t* kf, uint32_t start, uint32_t len, float S);
-__device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len, float& r, uint32_t& pos);
-
-// State of a chain between groups: significand and exponent of the running value, and where the walk stopped.
-struct ChainState {
-    uint32_t M;
-    int e;
-    uint32_t pos; // kNone while the walk goes on
-};
-
-// One group applied to the running sum quarter by quarter (records at `rec`), replaying only the quarters whose
-// map does not apply.  One wave.  (State by value: the chain keeps it in scalar registers.)
-__device__ __forceinline__ ChainState sum_by_quarters(const uint32_t* kf, uint32_t st, uint32_t len, const uint4* rec,
-                                                      ChainState c)
-{
-    using namespace seqfp;
-#pragma unroll 1
-    for (uint32_t k = 0; k < 4u; ++k) {
-        if (k * kQuarter < len) { // uniform
-            const uint4 r = rec[k];
-            const uint32_t d0 = uniform_u32(r.x), d1 = uniform_u32(r.y), cm = uniform_u32(r.z), eg = uniform_u32(r.w);
-            const uint32_t dd = (c.M & 1u) ? d1 : d0;
-            const uint32_t lim = cm >= (1u << 24) - 1u ? 0u : (1u << 24) - 1u - cm;
-            if ((uint32_t)c.e == eg && c.M + dd < lim) {
-                c.M += dd;
-            } else {
-                const float S = exact_span_sum(kf, st + k * kQuarter, min(kQuarter, len - k * kQuarter), join(c.M, c.e));
-                uint32_t Mv;
-                int ev;
-                split(S, Mv, ev);
-                c.M = uniform_u32(Mv);
-                c.e = (int)uniform_u32((uint32_t)ev);
-            }
-        }
-    }
-    return c;
-}
-
 // The entries of one span (at most 256), one per lane and register: x[j] of lane l is entry 64 * j + l, 0.0f past
 // the end.
-__device__ __forceinline__ void load_span_lanes(const uint32_t* kf, uint32_t start, uint32_t len, float (&x)[4])
+template <typename Keys>
+__device__ __forceinline__ void load_span_lanes(Keys kf, uint32_t start, uint32_t len, float (&x)[4])
 {
 #pragma unroll
     for (uint32_t j = 0; j < 4; ++j) {
         const uint32_t i = j * kWave + lane_id();
-        const uint32_t k = kf[start + min(i, len - 1u)]; // every lane loads, from inside the span
-        x[j] = i < len ? __uint_as_float(~k) : 0.0f;
+        // (every lane loads, from inside the span; masked with an AND, as in load_span)
+        x[j] = __uint_as_float(~kf[start + min(i, len - 1u)] & (i < len ? 0xffffffffu : 0u));
     }
+}
+// The same in two steps, for loads that are to stay in flight while other work goes on: the words as loaded
+// (nothing touches them here), and their conversion once they are wanted.
+template <typename Keys>
+__device__ __forceinline__ void fetch_span_lanes(Keys kf, uint32_t start, uint32_t len, uint32_t (&raw)[4])
+{
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j)
+        raw[j] = kf[start + min(j * kWave + lane_id(), len - 1u)];
+}
+__device__ __forceinline__ void take_span_lanes(const uint32_t (&raw)[4], uint32_t len, float (&x)[4])
+{
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j)
+        x[j] = __uint_as_float(~raw[j] & (j * kWave + lane_id() < len ? 0xffffffffu : 0u));
 }
 
 // One step of a chain that travels across the lanes: every lane takes the value of the lane below it (lane 0:
@@ -1368,7 +1374,8 @@ __device__ __forceinline__ float ror_add(float v, float x)
 }
 
 // S plus the entries of one span (len in 1..256), added one by one in fp32 (src/gen/sampler.cpp:80-82).  One wave.
-__device__ float exact_span_sum(const uint32_t* kf, uint32_t start, uint32_t len, float S)
+template <typename Keys>
+__device__ float exact_span_sum(Keys kf, uint32_t start, uint32_t len, float S)
 {
     float x[4];
     const uint32_t n = uniform_u32(len);
@@ -1446,7 +1453,8 @@ __device__ __forceinline__ bool walk_lanes(float (&x)[4], uint32_t n, uint32_t b
     return false;
 }
 
-__device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len, float& r, uint32_t& pos)
+template <typename Keys>
+__device__ bool exact_span_walk(Keys kf, uint32_t start, uint32_t len, float& r, uint32_t& pos)
 {
     float x[4];
     const uint32_t n = uniform_u32(len);
@@ -1455,6 +1463,41 @@ __device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len
         return false;
     load_span_lanes(kf, beg, n, x);
     return walk_lanes(x, n, beg, r, pos);
+}
+
+// State of a chain between groups: significand and exponent of the running value, and where the walk stopped.
+struct ChainState {
+    uint32_t M;
+    int e;
+    uint32_t pos; // kNone while the walk goes on
+};
+
+// One group applied to the running sum quarter by quarter (records at `rec`), replaying only the quarters whose
+// map does not apply.  One wave.  (State by value: the chain keeps it in scalar registers.)
+template <typename Keys>
+__device__ __forceinline__ ChainState sum_by_quarters(Keys kf, uint32_t st, uint32_t len, const uint4* rec, ChainState c)
+{
+    using namespace seqfp;
+#pragma unroll 1
+    for (uint32_t k = 0; k < 4u; ++k) {
+        if (k * kQuarter < len) { // uniform
+            const uint4 r = rec[k];
+            const uint32_t d0 = uniform_u32(r.x), d1 = uniform_u32(r.y), cm = uniform_u32(r.z), eg = uniform_u32(r.w);
+            const uint32_t dd = (c.M & 1u) ? d1 : d0;
+            const uint32_t lim = cm >= (1u << 24) - 1u ? 0u : (1u << 24) - 1u - cm;
+            if ((uint32_t)c.e == eg && c.M + dd < lim) {
+                c.M += dd;
+            } else {
+                const float S = exact_span_sum(kf, st + k * kQuarter, min(kQuarter, len - k * kQuarter), join(c.M, c.e));
+                uint32_t Mv;
+                int ev;
+                split(S, Mv, ev);
+                c.M = uniform_u32(Mv);
+                c.e = (int)uniform_u32((uint32_t)ev);
+            }
+        }
+    }
+    return c;
 }
 
 // Tail of every path that ends with a list sorted by (q desc, idx asc): kf[i] = ~bits(q_i), jf[i] = token id,
@@ -1469,12 +1512,14 @@ __device__ bool exact_span_walk(const uint32_t* kf, uint32_t start, uint32_t len
 // `T` (with `t_groups` records at `t_base`) describes a list whose groups were prepared by sort_kernel's workers;
 // without it the list is cut into groups of kGroup here.
 template <bool PLANNED = false>
-__device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf,
+__device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf_ptr,
                             const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
                             const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, GroupTable T = GroupTable{},
                             size_t t_base = 0, uint32_t t_groups = 0)
 {
     using namespace seqfp;
+    // (a planned row's list is in device memory; the other callers may hand over a list in LDS)
+    const typename std::conditional<PLANNED, GlobalKeys, AnyKeys>::type kf{kf_ptr};
     const uint32_t n1 = uniform_u32(n1_arg);
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
@@ -1770,7 +1815,9 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     }
     const unsigned long long tb0 = wall_clock64();
 #endif
-    if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess) {
+    // (a walk that will end within a few groups goes through them entry by entry: about as fast as a group's map
+    // would be to build)
+    if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && reach > kWalkSeqGroups) {
         // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
         build_group_maps(kf, reach, true, r0_guess, G, (uint32_t)(wave_id() >> 2) * 3u + (uint32_t)(wave_id() & 3) - 1u,
                          3u * kWaves / 4u);
@@ -1879,22 +1926,24 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     // at a time with a few scalar operations each, the next one's entries already on their way,
                     // and the scan takes over again once four in a row have gone through as maps.
                     uint32_t g = f, passed = 0;
-                    float xa[4];
+                    uint32_t raw[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu}; // the entries of group g
                     {
                         const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g);
                         const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g);
                         if (pk & kLenMask)
-                            load_span_lanes(kf, st, pk & kLenMask, xa);
+                            fetch_span_lanes(kf, st, pk & kLenMask, raw);
                     }
                     while (g < cnt && passed < 4u) {
                         const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g);
                         const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g);
+                        float xa[4];
+                        take_span_lanes(raw, pk & kLenMask, xa);
+                        // (the next group's entries set out now; they are used only if that group is replayed too)
                         const uint32_t g1 = min(g + 1u, cnt - 1u);
                         const uint32_t st1 = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g1);
                         const uint32_t pk1 = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g1);
-                        float xb[4];
                         if (pk1 & kLenMask)
-                            load_span_lanes(kf, st1, pk1 & kLenMask, xb); // (used only if group g + 1 is replayed)
+                            fetch_span_lanes(kf, st1, pk1 & kLenMask, raw);
                         bool by_map = false;
                         if (g != f && (pk >> 16) == (uint32_t)e) {
                             const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, g);
@@ -1922,10 +1971,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                             M = uniform_u32(Mv);
                             e = (int)uniform_u32((uint32_t)ev);
                         }
-                        xa[0] = xb[0];
-                        xa[1] = xb[1];
-                        xa[2] = xb[2];
-                        xa[3] = xb[3];
                         ++g;
                     }
                     if (stopped)
