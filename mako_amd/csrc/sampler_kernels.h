@@ -1048,6 +1048,7 @@ __device__ void draw_from_list(const mako_sample_desc& d, uint32_t row, QAt qat,
 // sorted lists: top-p cut, exact fp32 total and walk, in groups of 256 (see seqfp.h, "groups")
 // ---------------------------------------------------------------------------------------------
 
+constexpr uint32_t kWalkSeqGroups = 8; // a walk expected to end within this many groups goes entry by entry from LDS
 struct GroupLds { // carved from the dynamic LDS block once sorting is over; one pointer, the rest is offsets
     unsigned long long* base;
     __device__ __forceinline__ double* pg() const { return reinterpret_cast<double*>(base); } // [kMaxGroups + 2] fp64 sum of the entries before each group
@@ -1066,18 +1067,20 @@ struct GroupLds { // carved from the dynamic LDS block once sorting is over; one
     __device__ __forceinline__ uint32_t* w_d1() const { return w_d0() + kMaxGroups; }
     __device__ __forceinline__ uint32_t* w_need() const { return w_d1() + kMaxGroups; }
     __device__ __forceinline__ uint32_t* w_pack() const { return w_need() + kMaxGroups; }
+    // [kWalkSeqGroups * kGroup + kWave] the head of the list as floats, for a walk that ends within it
+    __device__ __forceinline__ float* head() const { return reinterpret_cast<float*>(w_pack() + kMaxGroups); }
 };
 constexpr uint32_t kLenMask = 0x1ffu;
 constexpr uint32_t kHasQuarters = 1u << 31;
 constexpr uint32_t kQuarterSlots = 96;
 constexpr uint32_t kQuarter = kGroup / 4;
 constexpr uint32_t kSeqMax = 1024; // sorted lists up to this long get their total and walk entry by entry
-constexpr uint32_t kWalkSeqGroups = 8; // a walk expected to end within this many groups gets no maps
 
 __device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
 {
     static_assert((kMaxGroups + 2) * 8 + 5 * kMaxGroups * 4 + 16 <= kSortMax * 8, "group records fit below the LDS lists");
-    static_assert(kQuarterSlots * 16 == 1536 && kSortMax * 8 + 1536 * 4 + 4 * kMaxGroups * 4 <= kDynLds,
+    static_assert(kQuarterSlots * 16 == 1536 &&
+                      kSortMax * 8 + 1536 * 4 + 4 * kMaxGroups * 4 + (kWalkSeqGroups * kGroup + kWave) * 4 <= kDynLds,
                   "the walk's records sit behind the quarter records and fit the dynamic LDS block");
     return GroupLds{L.sortk};
 }
@@ -1465,6 +1468,54 @@ __device__ bool exact_span_walk(Keys kf, uint32_t start, uint32_t len, float& r,
     return walk_lanes(x, n, beg, r, pos);
 }
 
+// The walk over the first `n` entries of the list, staged in LDS as floats (16-byte aligned, zeros up to the next
+// multiple of 64): every lane of the wave reads the same four entries with one broadcast load and subtracts them
+// in turn, three nanoseconds an entry (the travelling chain of walk_lanes() takes five).  Blocks of 64 blind, then
+// of 16, then entry by entry, as there.  Returns true and the position when the walk stops, else false and the new r.
+__device__ __forceinline__ bool walk_lds(const float* sx, uint32_t n, float& r, uint32_t& pos)
+{
+    float v = r;
+    for (uint32_t base = 0; base < n; base += kWave) {
+        const float r_in = v;
+        const float4* p = reinterpret_cast<const float4*>(sx + base);
+#pragma unroll
+        for (uint32_t i = 0; i < kWave / 4u; ++i) {
+            const float4 x = p[i];
+            v -= x.x;
+            v -= x.y;
+            v -= x.z;
+            v -= x.w;
+        }
+        if (__ballot(v < 0.0f) != 0ull) {
+            float rr = r_in;
+            for (uint32_t b = 0; b < kWave; b += 16u) {
+                float r16 = rr;
+#pragma unroll
+                for (uint32_t i = 0; i < 4u; ++i) {
+                    const float4 x = p[b / 4u + i];
+                    r16 -= x.x;
+                    r16 -= x.y;
+                    r16 -= x.z;
+                    r16 -= x.w;
+                }
+                if (__ballot(r16 < 0.0f) != 0ull) {
+                    for (uint32_t l = b; l < b + 16u; ++l) {
+                        const float xv = sx[base + l];
+                        if (__ballot(rr < xv) != 0ull) {
+                            pos = base + l;
+                            return true;
+                        }
+                        rr -= xv;
+                    }
+                }
+                rr = r16;
+            }
+        }
+    }
+    r = v;
+    return false;
+}
+
 // State of a chain between groups: significand and exponent of the running value, and where the walk stopped.
 struct ChainState {
     uint32_t M;
@@ -1520,6 +1571,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     using namespace seqfp;
     // (a planned row's list is in device memory; the other callers may hand over a list in LDS)
     const typename std::conditional<PLANNED, GlobalKeys, AnyKeys>::type kf{kf_ptr};
+    const float u_row = d.u[row]; // (asked for here, wanted much later)
     const uint32_t n1 = uniform_u32(n1_arg);
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
@@ -1599,7 +1651,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             if (ok) {
                 const float total = exact_span_sum(kf, 0, n, 0.0f);
                 const float span = total - 0.0f;
-                const float prod = d.u[row] * span;
+                const float prod = u_row * span;
                 float r = prod + 0.0f;
                 uint32_t pos = n - 1;
                 if (r < 0.0f)
@@ -1768,7 +1820,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             for (uint32_t b = 0; b < n; b += kGroup)
                 S = exact_span_sum(kf, b, min(kGroup, n - b), S);
             const float span = S - 0.0f;
-            const float prod = d.u[row] * span;
+            const float prod = u_row * span;
             const float r0 = prod + 0.0f;
             uint32_t at = n - 1;
             if (r0 < 0.0f) {
@@ -1798,7 +1850,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     // While one wave chains the running sum, the others already prepare the walk: its maps only need the binade r is
     // expected to be in at each group, and the fp64 sums give that (a wrong guess costs a replay, never the result).
     // Groups that start after the mass r0 could have is used up get no map.
-    const double r0_guess = (double)d.u[row] * G.pg()[groups];
+    const double r0_guess = (double)u_row * G.pg()[groups];
     uint32_t reach;
     {
         const uint32_t beyond = (tid < groups && !(r0_guess * 1.001 - G.pg()[tid] > 0)) ? tid : kNone;
@@ -1815,9 +1867,16 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     }
     const unsigned long long tb0 = wall_clock64();
 #endif
-    // (a walk that will end within a few groups goes through them entry by entry: about as fast as a group's map
-    // would be to build)
-    if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && reach > kWalkSeqGroups) {
+    // A walk that will end within a few groups goes through them entry by entry, from a copy in LDS: faster than
+    // the groups' maps would be to build.
+    const bool head_walk = reach <= kWalkSeqGroups; // uniform
+    const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
+    if (wave_id() != 0 && head_walk) {
+        for (uint32_t i = (uint32_t)(wave_id() - 1) * kWave + lane_id(); i < ((head_n + kWave - 1u) & ~(kWave - 1u));
+             i += (kWaves - 1u) * kWave)
+            G.head()[i] = __uint_as_float(~kf[min(i, head_n - 1u)] & (i < head_n ? 0xffffffffu : 0u));
+    }
+    if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && !head_walk) {
         // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
         build_group_maps(kf, reach, true, r0_guess, G, (uint32_t)(wave_id() >> 2) * 3u + (uint32_t)(wave_id() & 3) - 1u,
                          3u * kWaves / 4u);
@@ -1879,7 +1938,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     MAKO_STAMP(8);
     const float total = __uint_as_float(G.misc()[1]);
     const float span = total - 0.0f;
-    const float prod = d.u[row] * span;
+    const float prod = u_row * span;
     const float r0 = prod + 0.0f;
     __syncthreads();
 
@@ -1901,12 +1960,23 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             }
             uint32_t at = n - 1;
             bool stopped = false;
+            uint32_t first = 0; // groups already walked
+            if (head_walk && head_n) {
+                float r = r0;
+                stopped = walk_lds(G.head(), head_n, r, at);
+                uint32_t Mv;
+                int ev;
+                split(r, Mv, ev);
+                M = uniform_u32(Mv);
+                e = (int)uniform_u32((uint32_t)ev);
+                first = reach;
+            }
             for (uint32_t base = 0; base < groups && !stopped; base += kWave) {
                 const uint32_t gl = min(base + lane_id(), groups - 1u);
                 const uint32_t pk_l = G.w_pack()[gl], st_l = G.start()[gl];
                 const uint32_t d0_l = G.w_d0()[gl], d1_l = G.w_d1()[gl], need_l = G.w_need()[gl]; // (the bound, see build_group_maps)
                 const uint32_t cnt = min((uint32_t)kWave, groups - base);
-                uint32_t done = 0;
+                uint32_t done = base == 0 ? first : 0u; // (first <= kWalkSeqGroups)
                 while (done < cnt) {
                     MAKO_COUNT(30, 1);
                     const bool live = lane_id() >= done && lane_id() < cnt;
