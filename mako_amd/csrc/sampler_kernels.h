@@ -1468,49 +1468,51 @@ __device__ bool exact_span_walk(Keys kf, uint32_t start, uint32_t len, float& r,
     return walk_lanes(x, n, beg, r, pos);
 }
 
-// The walk over the first `n` entries of the list, staged in LDS as floats (16-byte aligned, zeros up to the next
-// multiple of 64): every lane of the wave reads the same four entries with one broadcast load and subtracts them
-// in turn, three nanoseconds an entry (the travelling chain of walk_lanes() takes five).  Blocks of 64 blind, then
-// of 16, then entry by entry, as there.  Returns true and the position when the walk stops, else false and the new r.
+// The walk over the first `n` entries of the list, staged in LDS as floats (16-byte aligned): every lane of the
+// wave reads the same four entries with one broadcast load and subtracts them in turn, three nanoseconds an entry
+// (the travelling chain of walk_lanes() takes five).  Blocks of 64 blind, then of 16, then entry by entry, as there.
+// Returns true and the position when the walk stops, else false and the new r.
 __device__ __forceinline__ bool walk_lds(const float* sx, uint32_t n, float& r, uint32_t& pos)
 {
     float v = r;
-    for (uint32_t base = 0; base < n; base += kWave) {
-        const float r_in = v;
+    uint32_t base = 0;
+    for (; base + kWave <= n; base += kWave) {
         const float4* p = reinterpret_cast<const float4*>(sx + base);
+        float t = v;
 #pragma unroll
         for (uint32_t i = 0; i < kWave / 4u; ++i) {
             const float4 x = p[i];
-            v -= x.x;
-            v -= x.y;
-            v -= x.z;
-            v -= x.w;
+            t -= x.x;
+            t -= x.y;
+            t -= x.z;
+            t -= x.w;
         }
-        if (__ballot(v < 0.0f) != 0ull) {
-            float rr = r_in;
-            for (uint32_t b = 0; b < kWave; b += 16u) {
-                float r16 = rr;
+        if (__ballot(t < 0.0f) != 0ull)
+            break; // the walk stops in this block: found below
+        v = t;
+    }
+    for (; base + 16u <= n; base += 16u) {
+        const float4* p = reinterpret_cast<const float4*>(sx + base);
+        float t = v;
 #pragma unroll
-                for (uint32_t i = 0; i < 4u; ++i) {
-                    const float4 x = p[b / 4u + i];
-                    r16 -= x.x;
-                    r16 -= x.y;
-                    r16 -= x.z;
-                    r16 -= x.w;
-                }
-                if (__ballot(r16 < 0.0f) != 0ull) {
-                    for (uint32_t l = b; l < b + 16u; ++l) {
-                        const float xv = sx[base + l];
-                        if (__ballot(rr < xv) != 0ull) {
-                            pos = base + l;
-                            return true;
-                        }
-                        rr -= xv;
-                    }
-                }
-                rr = r16;
-            }
+        for (uint32_t i = 0; i < 4u; ++i) {
+            const float4 x = p[i];
+            t -= x.x;
+            t -= x.y;
+            t -= x.z;
+            t -= x.w;
         }
+        if (__ballot(t < 0.0f) != 0ull)
+            break;
+        v = t;
+    }
+    for (const uint32_t end = min(n, base + 16u); base < end; ++base) {
+        const float x = sx[base];
+        if (__ballot(v < x) != 0ull) {
+            pos = base;
+            return true;
+        }
+        v -= x;
     }
     r = v;
     return false;
@@ -1519,7 +1521,8 @@ __device__ __forceinline__ bool walk_lds(const float* sx, uint32_t n, float& r, 
 // S plus the first `n` entries of a list staged in LDS as for walk_lds(), added one by one in fp32.
 __device__ __forceinline__ float sum_lds(const float* sx, uint32_t n, float S)
 {
-    for (uint32_t base = 0; base < n; base += 16u) {
+    uint32_t base = 0;
+    for (; base + 16u <= n; base += 16u) {
         const float4* p = reinterpret_cast<const float4*>(sx + base);
 #pragma unroll
         for (uint32_t i = 0; i < 4u; ++i) {
@@ -1530,6 +1533,8 @@ __device__ __forceinline__ float sum_lds(const float* sx, uint32_t n, float S)
             S += x.w;
         }
     }
+    for (; base < n; ++base)
+        S += sx[base];
     return S;
 }
 
@@ -1704,6 +1709,20 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     const uint32_t groups1 = PLANNED ? t_groups : (n1 + kGroup - 1) / kGroup;
     if (tid == 0)
         G.misc()[3] = 0;
+    // The head of the list as floats in LDS (loads set out now, wanted after the cut): where the running sum and
+    // the walk change binade every few entries, both go through it entry by entry.
+    constexpr uint32_t kHead = kWalkSeqGroups * kGroup;
+    {
+        uint32_t raw[kHead / kThreads];
+#pragma unroll
+        for (uint32_t t = 0; t < kHead / kThreads; ++t)
+            raw[t] = kf[min(t * kThreads + tid, n1 - 1u)];
+#pragma unroll
+        for (uint32_t t = 0; t < kHead / kThreads; ++t)
+            G.head()[t * kThreads + tid] = __uint_as_float(~raw[t] & (t * kThreads + tid < n1 ? 0xffffffffu : 0u));
+        if (tid < kWave)
+            G.head()[kHead + tid] = 0.0f;
+    }
     __syncthreads();
     if constexpr (PLANNED) {
         if (tid < groups1) {
@@ -1832,9 +1851,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     if (n <= kSeqMax) {
         // A nucleus this short is copied to LDS and gone through entry by entry, once for the total and once for the
         // walk (three nanoseconds an entry each way): the group maps below only pay on longer lists.
-        for (uint32_t i = tid; i < ((n + kWave - 1u) & ~(kWave - 1u)); i += kThreads)
-            G.head()[i] = __uint_as_float(~kf[min(i, n - 1u)] & (i < n ? 0xffffffffu : 0u));
-        __syncthreads();
         if (wave_id() == 0) {
             const float S = sum_lds(G.head(), n, 0.0f);
             const float span = S - 0.0f;
@@ -1887,11 +1903,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     // the groups' maps would be to build.
     const bool head_walk = reach <= kWalkSeqGroups; // uniform
     const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
-    if (wave_id() != 0 && head_walk) {
-        for (uint32_t i = (uint32_t)(wave_id() - 1) * kWave + lane_id(); i < ((head_n + kWave - 1u) & ~(kWave - 1u));
-             i += (kWaves - 1u) * kWave)
-            G.head()[i] = __uint_as_float(~kf[min(i, head_n - 1u)] & (i < head_n ? 0xffffffffu : 0u));
-    }
     if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && !head_walk) {
         // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
         build_group_maps(kf, reach, true, r0_guess, G, (uint32_t)(wave_id() >> 2) * 3u + (uint32_t)(wave_id() & 3) - 1u,
@@ -1908,12 +1919,38 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         // the scan resumes behind it.  The state (significand M, exponent e) lives in scalar registers.
         uint32_t M = 0;
         int e = 1; // 0.0f
+        // The sum changes binade every few entries at first.  The leading groups, up to the last of the first few in
+        // which the fp64 sums expect a change, are added entry by entry from the copy in LDS.
+        uint32_t first = 0;
+        MAKO_TIC(0);
+        {
+            const uint32_t gq = min((uint32_t)lane_id(), groups - 1u);
+            const bool cross = (uint32_t)lane_id() < min(groups, kWalkSeqGroups) &&
+                               (lane_id() == 0 || exponent_of((float)G.pg()[gq]) != exponent_of((float)G.pg()[gq + 1u]));
+            const unsigned long long bal = __ballot(cross);
+            first = bal ? 64u - (uint32_t)__clzll((long long)bal) : 0u;
+            if (first) {
+                const uint32_t hs = first == groups ? n : uniform_u32(G.start()[min(first, groups - 1u)]);
+                const float S = sum_lds(G.head(), min(hs, kHead), 0.0f);
+                uint32_t Mv;
+                int ev;
+                split(S, Mv, ev);
+                M = uniform_u32(Mv);
+                e = (int)uniform_u32((uint32_t)ev);
+            }
+        }
+        MAKO_TOC(0, 17);
+#ifdef MAKO_TIMING
+        if (lane_id() == 0)
+            g_mako_stamp[19] = first;
+#endif
+        MAKO_TIC(1);
         for (uint32_t base = 0; base < groups; base += kWave) {
             const uint32_t gl = min(base + lane_id(), groups - 1u);
             const uint32_t pk_l = G.pack()[gl], st_l = G.start()[gl];
             const uint32_t d0_l = G.d0()[gl], d1_l = G.d1()[gl], cm_l = G.cmax()[gl];
             const uint32_t cnt = min((uint32_t)kWave, groups - base);
-            uint32_t done = 0;
+            uint32_t done = base == 0 ? first : 0u; // (first <= kWalkSeqGroups)
             while (done < cnt) {
                 const bool live = lane_id() >= done && lane_id() < cnt;
                 const bool same = live && (pk_l >> 16) == (uint32_t)e;
@@ -1928,7 +1965,10 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 if (f < cnt) {
                     const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
                     const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
-                    MAKO_COUNT(20, 1);
+#ifdef MAKO_TIMING
+                    if (lane_id() == 0)
+                        g_mako_stamp[21] += 1;
+#endif
                     const uint32_t slot = (pk >> 9) & 0x7fu;
                     if (slot) {
                         const ChainState c = sum_by_quarters(kf, st, pk & kLenMask, G.quarters() + (slot - 1u) * 4u,
@@ -1947,6 +1987,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 done = f + 1u;
             }
         }
+        MAKO_TOC(1, 18);
         if (lane_id() == 0)
             G.misc()[1] = __float_as_uint(join(M, e));
     }
