@@ -48,6 +48,12 @@ typedef struct mako_sampling_params {
 #define MAKO_PATH_TOPK 3u     /* resolved from the per-slice top-k candidates */
 #define MAKO_PATH_NUCLEUS 4u  /* top_k == 0: nucleus resolved from the per-slice candidates */
 #define MAKO_PATH_GENERAL 5u  /* whole-row sort path */
+#define MAKO_PATH_FORCED 6u   /* not sampled: force_token / close_token took the row */
+
+/* out_forced values */
+#define MAKO_FORCED_NONE 0u  /* the row was sampled (or verified) */
+#define MAKO_FORCED_TOKEN 1u /* force_token was taken */
+#define MAKO_FORCED_CLOSE 2u /* close_token was taken: fewer than close_max_above logits above its own */
 
 typedef struct mako_sample_desc {
     /* ---- inputs (device pointers) ---- */
@@ -80,6 +86,25 @@ typedef struct mako_sample_desc {
     int32_t* out_cand_idx;   /* [n_rows][cand_cap] first candidates, in candidate order */
     float* out_cand_q;       /* [n_rows][cand_cap] and their weights */
     uint32_t cand_cap;
+    /* ---- the decode loop's hooks around the sampler (optional; zero / null = the sampler alone) ----
+     * Session::run asks its `forced` callback before every sample() / verify() (src/gen/session.hpp:43-45,
+     * src/gen/session.cpp:441-443, 483-485, 524-525): a token >= 0 is taken instead of sampling (a draft is kept
+     * only if it equals it), no uniform is consumed, and the token goes through accept() like a sampled one. */
+    const int32_t* force_token; /* [n_rows]: >= 0: the callback's answer is already known to the caller */
+    /* ReasoningBudget::forced's last stretch (src/server/openai.cpp:589-604): close_token[r] in [0, n_vocab) is
+     * taken iff fewer than close_max_above logits of the row are strictly greater than logits[close_token[r]]
+     * (the reference stops counting at 3).  The test sees the logits the sampler is given: a token the mask
+     * clears counts as -inf, and a cleared close_token is never taken.  force_token[r] >= 0 wins over it. */
+    const int32_t* close_token; /* [n_rows], < 0: none */
+    uint32_t close_max_above;
+    uint8_t* out_forced;        /* [n_rows] MAKO_FORCED_*; required when force_token or close_token is given */
+    uint32_t* out_above;        /* optional [n_rows]: logits strictly above logits[close_token[r]] (all of them,
+                                   not capped); 0xffffffff where there is no close_token or the mask clears it */
+    /* Sampler::accept of the chosen token (src/gen/session.cpp:419-421) without a trip to the host: when nonzero,
+     * row r's token is written to hist_tokens[r][hist_len[r]] and hist_len[r] is incremented, provided
+     * hist_len[r] < hist_stride (else the history is left as it is).  hist_tokens and hist_len must then be
+     * writable device memory, hist_counts null, and draft null (the rows of a verify batch share one history). */
+    uint32_t append_history;
 } mako_sample_desc;
 
 typedef struct mako_sampler_ctx mako_sampler_ctx;

@@ -16,7 +16,8 @@ LIB_PATH = os.path.join(_HERE, "libmako_sampler.so")
 MAKO_OK = 0
 MAKO_ERR_INVALID_ARG = -1
 MAKO_ERR_HIP = -2
-PATH_GREEDY, PATH_FALLBACK, PATH_TOPK, PATH_NUCLEUS, PATH_GENERAL = 1, 2, 3, 4, 5
+PATH_GREEDY, PATH_FALLBACK, PATH_TOPK, PATH_NUCLEUS, PATH_GENERAL, PATH_FORCED = 1, 2, 3, 4, 5, 6
+FORCED_NONE, FORCED_TOKEN, FORCED_CLOSE = 0, 1, 2
 
 # mako_sampling_params / SamplingParams (src/gen/sampler.hpp:11-20)
 PARAMS_DTYPE = np.dtype(
@@ -71,6 +72,12 @@ class Desc(C.Structure):
         ("out_cand_idx", C.c_void_p),
         ("out_cand_q", C.c_void_p),
         ("cand_cap", C.c_uint32),
+        ("force_token", C.c_void_p),
+        ("close_token", C.c_void_p),
+        ("close_max_above", C.c_uint32),
+        ("out_forced", C.c_void_p),
+        ("out_above", C.c_void_p),
+        ("append_history", C.c_uint32),
     ]
 
 
@@ -169,7 +176,8 @@ class Batch:
     """Device-resident inputs and outputs of one batch, built from host arrays."""
 
     def __init__(self, logits, params, u, mask=None, hist=None, hist_len=None, hist_counts=None, draft=None, u2=None,
-                 cand_cap=0, diagnostics=True):
+                 cand_cap=0, diagnostics=True, force_token=None, close_token=None, close_max_above=3,
+                 append_history=False):
         logits = np.ascontiguousarray(logits, np.float32)
         self.n_rows, self.n_vocab = logits.shape
         b = self.n_rows
@@ -179,7 +187,8 @@ class Batch:
         d.logits, d.logits_stride = self.d_logits.ptr, self.n_vocab
         d.n_rows, d.n_vocab = b, self.n_vocab
         d.params = self._up(np.ascontiguousarray(params, PARAMS_DTYPE)).ptr
-        d.u = self._up(np.ascontiguousarray(u, np.float32)).ptr
+        self.d_u = self._up(np.ascontiguousarray(u, np.float32))
+        d.u = self.d_u.ptr
         if mask is not None:
             mask = np.ascontiguousarray(mask, np.uint32)
             d.mask, d.mask_stride = self._up(mask).ptr, mask.shape[1]
@@ -187,8 +196,10 @@ class Batch:
             hist = np.ascontiguousarray(hist, np.int32)
             if hist_len is None:
                 hist_len = np.full(b, hist.shape[1], np.uint32)
-            d.hist_tokens, d.hist_stride = self._up(hist).ptr, hist.shape[1]
-            d.hist_len = self._up(np.ascontiguousarray(hist_len, np.uint32)).ptr
+            self.d_hist = self._up(hist)
+            self.d_hist_len = self._up(np.ascontiguousarray(hist_len, np.uint32))
+            d.hist_tokens, d.hist_stride = self.d_hist.ptr, hist.shape[1]
+            d.hist_len = self.d_hist_len.ptr
             if hist_counts is not None:
                 d.hist_counts = self._up(np.ascontiguousarray(hist_counts, np.uint32)).ptr
         if draft is not None:
@@ -205,6 +216,19 @@ class Batch:
             self.o_q = self._new((b,), np.float32)
             self.o_path = self._new((b,), np.uint8)
             d.out_n_cand, d.out_total, d.out_q, d.out_path = self.o_n.ptr, self.o_total.ptr, self.o_q.ptr, self.o_path.ptr
+        self.hooks = force_token is not None or close_token is not None
+        if force_token is not None:
+            self.d_force = self._up(np.ascontiguousarray(force_token, np.int32))
+            d.force_token = self.d_force.ptr
+        if close_token is not None:
+            d.close_token = self._up(np.ascontiguousarray(close_token, np.int32)).ptr
+            d.close_max_above = close_max_above
+            self.o_above = self._new((b,), np.uint32)
+            d.out_above = self.o_above.ptr
+        if self.hooks:
+            self.o_forced = self._new((b,), np.uint8)
+            d.out_forced = self.o_forced.ptr
+        d.append_history = 1 if append_history else 0
         self.cand_cap = cand_cap
         if cand_cap:
             self.o_ci = self._new((b, cand_cap), np.int32)
@@ -233,7 +257,16 @@ class Batch:
             r.update(cand_idx=self.o_ci.download(), cand_q=self.o_cq.download())
         if hasattr(self, "o_acc"):
             r["accepted"] = self.o_acc.download()
+        if self.hooks:
+            r["forced"] = self.o_forced.download()
+        if hasattr(self, "o_above"):
+            r["above"] = self.o_above.download()
         return r
+
+    def history(self):
+        """(tokens, lengths) of the device-resident histories, as append_history leaves them."""
+        hip.synchronize()
+        return self.d_hist.download(), self.d_hist_len.download()
 
 
 def sample(ctx, logits, params, u, **kw):

@@ -132,6 +132,9 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     const void* kernels[] = {(const void*)mako::scan_kernel<true, 0>,    (const void*)mako::scan_kernel<false, 0>,
                              (const void*)mako::scan_kernel<true, 2>,    (const void*)mako::scan_kernel<false, 2>,
                              (const void*)mako::scan_kernel<true, 8>,    (const void*)mako::scan_kernel<false, 8>,
+                             (const void*)mako::scan_kernel<true, 0, true>, (const void*)mako::scan_kernel<false, 0, true>,
+                             (const void*)mako::scan_kernel<true, 2, true>, (const void*)mako::scan_kernel<false, 2, true>,
+                             (const void*)mako::scan_kernel<true, 8, true>, (const void*)mako::scan_kernel<false, 8, true>,
                              (const void*)mako::finish_kernel<true, 0>,  (const void*)mako::finish_kernel<false, 0>,
                              (const void*)mako::finish_kernel<true, 2>,  (const void*)mako::finish_kernel<false, 2>,
                              (const void*)mako::finish_kernel<true, 8>,  (const void*)mako::finish_kernel<false, 8>,
@@ -218,6 +221,13 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: draft, u2 and out_accepted go together");
     if ((d.out_cand_idx != nullptr) != (d.out_cand_q != nullptr))
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: out_cand_idx and out_cand_q go together");
+    if ((d.force_token || d.close_token) && !d.out_forced)
+        return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: force_token / close_token need out_forced");
+    if (d.out_above && !d.close_token)
+        return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: out_above needs close_token");
+    if (d.append_history && (!d.hist_tokens || !d.hist_len || d.hist_counts || d.draft))
+        return fail(ctx, MAKO_ERR_INVALID_ARG,
+                    "sampler: append_history needs hist_tokens and hist_len, and neither hist_counts nor draft");
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t slices = mako_sampler_slices(d.n_vocab);
@@ -235,7 +245,12 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     } while (0)
 #define MAKO_LAUNCH(V, K)                                                                                          \
     do {                                                                                                           \
-        hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc_dev, slice_len); \
+        if (d.close_token)                                                                                         \
+            hipLaunchKernelGGL((mako::scan_kernel<V, K, true>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc_dev,   \
+                               slice_len);                                                                         \
+        else                                                                                                       \
+            hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc_dev,        \
+                               slice_len);                                                                         \
         MAKO_MARK(1);                                                                                              \
         hipLaunchKernelGGL((mako::finish_kernel<V, K>), grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev,  \
                            slices, slice_len);                                                                     \

@@ -126,7 +126,8 @@ struct SliceStat {
     uint32_t flags;
     uint32_t n_emit;  // candidates written for this slice
     uint32_t tau_key; // order key of the emission threshold: every logit with key >= tau_key was emitted
-    uint32_t pad[3];
+    uint32_t above;   // logits of the slice strictly above the row's close_token logit (0 without one)
+    uint32_t pad[2];
 };
 
 constexpr uint32_t kWorkers = 32;  // workgroups that share the sort of one wide-nucleus row
@@ -317,6 +318,32 @@ __device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row
     }
 }
 
+// How many of the thread's logits (as the sampler is given them: a token the mask clears is -inf) are strictly
+// greater than v: the count of ReasoningBudget::forced, src/server/openai.cpp:599-602.
+template <bool VEC>
+__device__ __forceinline__ uint32_t count_above(const RawSlice<VEC>& r, uint32_t lo, uint32_t hi, float v)
+{
+    const uint32_t tid = threadIdx.x;
+    uint32_t c = 0;
+    if (VEC) {
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            if (lo + k * 4096u + tid * 4u < hi) {
+                c += ((r.bits[k] & 1u) && r.v[k].x > v) ? 1u : 0u;
+                c += ((r.bits[k] & 2u) && r.v[k].y > v) ? 1u : 0u;
+                c += ((r.bits[k] & 4u) && r.v[k].z > v) ? 1u : 0u;
+                c += ((r.bits[k] & 8u) && r.v[k].w > v) ? 1u : 0u;
+            }
+        }
+    } else {
+        const float* f = reinterpret_cast<const float*>(r.v);
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j)
+            c += (lo + j * (uint32_t)kThreads + tid < hi && ((r.bits[0] >> j) & 1u) && f[j] > v) ? 1u : 0u;
+    }
+    return c;
+}
+
 // Mask and penalties (src/gen/sampler.cpp:22-28) applied to the raw logits; slots past the end of the
 // slice hold NaN, which never wins a comparison and never becomes a candidate.
 template <bool VEC>
@@ -399,13 +426,16 @@ struct NoOverlap {
 template <bool VEC, int KH, typename Overlap = NoOverlap>
 __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi,
                                                uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, bool pen,
-                                               uint32_t* s_cnt, float (&wv)[16], Extras<KH>& ex, Overlap overlap = Overlap())
+                                               uint32_t* s_cnt, float (&wv)[16], Extras<KH>& ex, Overlap overlap = Overlap(),
+                                               bool want_above = false, float close_v = 0.0f, uint32_t* above = nullptr)
 {
     const uint32_t tid = threadIdx.x;
     const float nan = __uint_as_float(0x7fc00000u);
     RawSlice<VEC> raw;
     load_raw<VEC>(d, row, lo, hi, raw);
     overlap();
+    if (want_above) // uniform
+        *above = count_above<VEC>(raw, lo, hi, close_v);
 #pragma unroll
     for (int k = 0; k < (KH > 0 ? KH : 1); ++k) {
         ex.v[k] = nan;
@@ -525,6 +555,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
 struct alignas(16) ScanShared {
     uint32_t wave_max[kWaves]; // order keys
     uint32_t wave_kth[kWaves];
+    uint32_t wave_above[kWaves];
     uint32_t argidx;
     uint32_t emit_n;
     uint32_t emit_flags;
@@ -578,7 +609,9 @@ __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 }
 
 // grid = (slices, rows).
-template <bool VEC, int KH>
+// (ABOVE: the batch has close tokens, whose logits' ranks are counted on the way; a variant of its own because the
+// count's registers would cost every other batch half its occupancy)
+template <bool VEC, int KH, bool ABOVE = false>
 __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, const Scratch* sc_dev, uint32_t slice_len)
 {
     const Scratch& sc = *sc_dev;
@@ -604,9 +637,27 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
             sc.work_n[1] = 0;
         }
     }
+    // ReasoningBudget::forced's question (src/server/openai.cpp:598-602), answered in the same pass over the logits
+    bool want_above = false;
+    float close_v = 0.0f;
+    if (ABOVE && d.close_token) {
+        const int32_t ct = d.close_token[row];
+        if (ct >= 0 && (uint32_t)ct < d.n_vocab &&
+            (!d.mask || ((d.mask[(int64_t)row * d.mask_stride + ((uint32_t)ct >> 5)] >> ((uint32_t)ct & 31u)) & 1u))) {
+            want_above = true;
+            close_v = d.logits[(int64_t)row * d.logits_stride + ct];
+        }
+    }
+    uint32_t above = 0;
     float wv[16];
     Extras<KH> ex;
-    load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv, ex);
+    if (ABOVE) {
+        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv, ex, NoOverlap(), want_above, close_v, &above);
+        if (want_above) // uniform
+            above = __ockl_wfred_add_u32(above);
+    } else {
+        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv, ex);
+    }
 
     // maximum of the thread's logits (NaNs ignored), then of the wave, then of the slice
     float best = -INFINITY;
@@ -630,13 +681,17 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
     if (lane_id() == 0) {
         sm.wave_max[wave_id()] = wmax;
         sm.wave_kth[wave_id()] = wkth;
+        if (ABOVE)
+            sm.wave_above[wave_id()] = above;
     }
     __syncthreads();
-    uint32_t mkey = 0, tau_key = 0xffffffffu;
+    uint32_t mkey = 0, tau_key = 0xffffffffu, above_slice = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
         mkey = max(mkey, sm.wave_max[w]);
         tau_key = min(tau_key, sm.wave_kth[w]);
+        if (ABOVE)
+            above_slice += sm.wave_above[w];
     }
     // first index holding the maximum
     if (bkey == mkey) {
@@ -659,7 +714,8 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
     st.flags = 0;
     st.n_emit = 0;
     st.tau_key = 0;
-    st.pad[0] = st.pad[1] = st.pad[2] = 0;
+    st.above = above_slice;
+    st.pad[0] = st.pad[1] = 0;
     // element 0 of the row is NaN (it may have moved to an extra): only its holder raises the flag
     bool first_nan = slice == 0 && tid == 0 && wv[0] != wv[0] && !(pen && KH > 0 && s_dyn[0]);
 #pragma unroll
@@ -951,11 +1007,24 @@ struct RowOut {
     float q;
     uint32_t path;
     uint32_t accepted;
+    uint32_t forced = MAKO_FORCED_NONE;
 };
 
+// The row's results; with append_history also Sampler::accept of the token (src/gen/session.cpp:419-421).  Called
+// once per row, by one thread, after everything that reads the row's history in this batch.
 __device__ __forceinline__ void write_row(const mako_sample_desc& d, uint32_t row, const RowOut& o)
 {
     d.out_tokens[row] = o.token;
+    if (d.out_forced)
+        d.out_forced[row] = (uint8_t)o.forced;
+    if (d.append_history) {
+        uint32_t* hl = const_cast<uint32_t*>(d.hist_len);
+        const uint32_t len = hl[row];
+        if (len < (uint32_t)d.hist_stride) {
+            const_cast<int32_t*>(d.hist_tokens)[(int64_t)row * d.hist_stride + len] = o.token;
+            hl[row] = len + 1u;
+        }
+    }
     if (d.out_n_cand)
         d.out_n_cand[row] = o.n_cand;
     if (d.out_total)
@@ -3195,6 +3264,39 @@ __device__ float candidate_bound(const Scratch& sc, uint32_t row, uint32_t slice
     return q_bound;
 }
 
+// Is the row's token decided without sampling (Session's `forced` callback, src/gen/session.cpp:441-443)?  Returns
+// MAKO_FORCED_* and the token; `above` receives the logits strictly above the close_token's (kNone without one).
+// The same answer in every thread and in every workgroup that asks.
+__device__ __forceinline__ uint32_t row_forced(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slices,
+                                               int32_t& token, uint32_t& above)
+{
+    uint32_t kind = MAKO_FORCED_NONE;
+    above = kNone;
+    token = -1;
+    if (d.close_token) {
+        const int32_t ct = d.close_token[row];
+        if (ct >= 0 && (uint32_t)ct < d.n_vocab &&
+            (!d.mask || ((d.mask[(int64_t)row * d.mask_stride + ((uint32_t)ct >> 5)] >> ((uint32_t)ct & 31u)) & 1u))) {
+            uint32_t a = 0;
+            for (uint32_t s = 0; s < slices; ++s)
+                a += sc.stats[(size_t)row * kMaxSlices + s].above;
+            above = a;
+            if (a < d.close_max_above) { // src/server/openai.cpp:600-603
+                kind = MAKO_FORCED_CLOSE;
+                token = ct;
+            }
+        }
+    }
+    if (d.force_token) {
+        const int32_t ft = d.force_token[row];
+        if (ft >= 0) {
+            kind = MAKO_FORCED_TOKEN;
+            token = ft;
+        }
+    }
+    return kind;
+}
+
 // grid = (slices, rows) workgroups, of which workgroup i serves the i-th piece of work in row order: one piece per
 // row, and one per slice for top_k == 0 rows (find_piece).  The busy workgroups are then the first ones dispatched
 // and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
@@ -3225,6 +3327,28 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     const mako_sampling_params& P = s_args.P;
     const RowClass cls = classify(P);
     MAKO_STAMP(0);
+    if (d.force_token || d.close_token) { // uniform
+        int32_t ftok;
+        uint32_t above;
+        const uint32_t kind = row_forced(d, sc, row, slices, ftok, above);
+        if (slice == 0 && tid == 0 && d.out_above)
+            d.out_above[row] = above;
+        if (kind != MAKO_FORCED_NONE) {
+            // a token >= 0 is taken instead of sampling, and a draft is kept only if it matches (session.hpp:43-45)
+            if (slice == 0 && tid == 0) {
+                RowOut o;
+                o.token = ftok;
+                o.n_cand = 0;
+                o.total = 0.0f;
+                o.q = 0.0f;
+                o.path = MAKO_PATH_FORCED;
+                o.accepted = d.draft ? (d.draft[row] == ftok) : 0u;
+                o.forced = kind;
+                write_row(d, row, o);
+            }
+            return;
+        }
+    }
     if (tid < 32)
         sm.tab[tid] = k_exp2_tab[tid];
     __syncthreads();
@@ -3323,6 +3447,12 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
     L.sortk = s_dyn64;
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
+    if (d.force_token || d.close_token) { // finish_kernel gave a forced row its token
+        int32_t ftok;
+        uint32_t above;
+        if (row_forced(d, sc, row, slices, ftok, above) != MAKO_FORCED_NONE)
+            return;
+    }
     MAKO_STAMP(2);
     // this thread's two bins of the row's histogram (left zero for the next batch), the slices' exact sums in order
     unsigned long long* bins = sc.bins + (size_t)row * kBins;

@@ -462,3 +462,26 @@ int32_t or_verify(const float* logits, uint32_t n_vocab, const or_params* p, con
     free(d.cand);
     return token;
 }
+
+/* src/server/openai.cpp:589-604, the part that looks at the logits. */
+int32_t or_close_forced(const float* logits, uint32_t n_vocab, const uint32_t* mask, int32_t think_end,
+                        uint32_t max_above, uint32_t* above)
+{
+    if (above)
+        *above = 0xffffffffu;
+    if (think_end < 0 || (uint32_t)think_end >= n_vocab) /* :590, :594 */
+        return -1;
+    if (mask && !((mask[(uint32_t)think_end >> 5] >> ((uint32_t)think_end & 31u)) & 1u))
+        return -1;
+    const float v = logits[think_end]; /* :596 */
+    uint32_t n = 0;
+    for (uint32_t i = 0; i < n_vocab; ++i) { /* :598-600 */
+        const int allowed = !mask || ((mask[i >> 5] >> (i & 31u)) & 1u);
+        const float w = allowed ? logits[i] : -INFINITY;
+        if (w > v)
+            ++n;
+    }
+    if (above)
+        *above = n;
+    return n >= max_above ? -1 : think_end; /* :600, :602-603 */
+}

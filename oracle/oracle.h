@@ -75,6 +75,18 @@ int32_t or_verify(const float* logits, uint32_t n_vocab, const or_params* p,
                   int32_t draft, float u1, float u2, int order_mode,
                   int* accepted, or_trace* trace);
 
+/*
+ * The last-stretch test of ReasoningBudget::forced (src/server/openai.cpp:596-604):
+ * returns think_end when fewer than max_above (3 in the reference) logits are
+ * strictly greater than logits[think_end], else -1; -1 also when think_end is
+ * negative or not below n_vocab (:590, :594).  `mask` as in or_sample (a build
+ * extension: a cleared bit is -inf, and a cleared think_end is never returned).
+ * `above`, if given, receives the full count (the reference stops at 3).
+ * Pinned by the known answers of tests/server_test.cpp:142-152.
+ */
+int32_t or_close_forced(const float* logits, uint32_t n_vocab, const uint32_t* mask, int32_t think_end,
+                        uint32_t max_above, uint32_t* above);
+
 /* libstdc++ nth_element restated, exposed for its own pin test:
  * keys are (q, idx) pairs ordered by (q desc, idx asc). */
 void or_nth_element(float* q, int32_t* idx, uint32_t n, uint32_t nth);

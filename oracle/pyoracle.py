@@ -95,6 +95,18 @@ class _Oracle:
                                   C.POINTER(C.c_int), C.POINTER(Trace)]
         lib.or_nth_element.argtypes = [C.POINTER(C.c_float), C.POINTER(C.c_int32), C.c_uint32, C.c_uint32]
         lib.or_debug_heap_selects.restype = C.c_long
+        lib.or_close_forced.restype = C.c_int32
+        lib.or_close_forced.argtypes = [C.POINTER(C.c_float), C.c_uint32, C.POINTER(C.c_uint32), C.c_int32, C.c_uint32,
+                                        C.POINTER(C.c_uint32)]
+
+    def close_forced(self, logits, think_end, max_above=3, mask=None):
+        """(token or -1, logits strictly above logits[think_end]) -- ReasoningBudget::forced's last-stretch test."""
+        logits = np.ascontiguousarray(logits, np.float32)
+        m = np.ascontiguousarray(mask, np.uint32) if mask is not None else None
+        above = C.c_uint32()
+        t = self.lib.or_close_forced(_fp(logits), logits.shape[0], _up(m) if m is not None else None, int(think_end),
+                                     int(max_above), C.byref(above))
+        return int(t), int(above.value)
 
     def heap_selects(self):
         return self.lib.or_debug_heap_selects()

@@ -200,6 +200,118 @@ def test_verify_matches_oracle(gpu_ctx):
         assert g["tokens"][r] == t and bool(g["accepted"][r]) == tr["accepted"], (r, g["tokens"][r], t)
 
 
+def _choose(o, w, r, force, close, max_above):
+    """Session::run's `choose` (src/gen/session.cpp:441-443) with ReasoningBudget::forced's last-stretch test as the
+    callback (src/server/openai.cpp:589-604): (token, forced kind, logits above the close token)."""
+    above = 0xFFFFFFFF
+    kind, tok = api.FORCED_NONE, -1
+    mask = w["mask"][r] if "mask" in w else None
+    if close is not None and close[r] >= 0:
+        t, above = o.close_forced(w["logits"][r], int(close[r]), max_above, mask)
+        if t >= 0:
+            kind, tok = api.FORCED_CLOSE, t
+    if force is not None and force[r] >= 0:
+        kind, tok = api.FORCED_TOKEN, int(force[r])
+    if kind == api.FORCED_NONE:
+        p = pyoracle.params_from_record(w["params"][r])
+        hist = w["hist"][r, : w["hist_len"][r]] if "hist" in w else None
+        tok = o.sample(w["logits"][r], p, float(w["u"][r]), hist, mask)[0]
+    return tok, kind, above
+
+
+@pytest.mark.parametrize("v", [1000, 40000, 129280])
+def test_forced_and_close_tokens(gpu_ctx, v):
+    """The decode loop's `forced` hook: known tokens, and the close token taken iff fewer than three logits lie
+    strictly above its own (src/server/openai.cpp:596-603), counted in the sampler's own pass over the logits."""
+    rng = np.random.default_rng(4000 + v)
+    o = pyoracle.oracle()
+    b = 32
+    for it in range(3):
+        w = _random_case(rng, v, b)
+        close = rng.integers(0, v, b).astype(np.int32)
+        order = np.argsort(-w["logits"], axis=1, kind="stable")
+        for r in range(b):  # put the close token near the top in most rows: ranks 0..5, ties included
+            if r % 4 != 3:
+                close[r] = order[r, int(rng.integers(0, min(6, v)))]
+        close[::7] = -1
+        close[5] = v + 3  # out of range: ignored (:594)
+        force = np.full(b, -1, np.int32)
+        force[::5] = rng.integers(0, v, len(force[::5]))
+        max_above = int(rng.choice([3, 3, 1, 0, 5]))
+        _say("forced/close case v=%d it=%d max_above=%d" % (v, it, max_above))
+        g = api.sample(gpu_ctx, w["logits"], w["params"], w["u"], mask=w.get("mask"), hist=w.get("hist"),
+                       hist_len=w.get("hist_len"), force_token=force, close_token=close, close_max_above=max_above)
+        for r in range(b):
+            tok, kind, above = _choose(o, w, r, force, close, max_above)
+            assert (g["tokens"][r], g["forced"][r], g["above"][r]) == (tok, kind, above), \
+                (r, g["tokens"][r], g["forced"][r], g["above"][r], tok, kind, above)
+            if kind != api.FORCED_NONE:
+                assert g["path"][r] == api.PATH_FORCED
+
+
+def test_forced_token_meets_draft(gpu_ctx):
+    """With a draft, a forced token is returned and the draft is kept only if it equals it
+    (src/gen/session.cpp:483-485, 524-525)."""
+    rng = np.random.default_rng(91)
+    v, b = 5000, 16
+    w = _random_case(rng, v, b)
+    force = np.full(b, -1, np.int32)
+    force[::2] = rng.integers(0, v, b // 2)
+    draft = rng.integers(0, v, b).astype(np.int32)
+    draft[::4] = force[::4]
+    u2 = rng.random(b).astype(np.float32)
+    g = api.sample(gpu_ctx, w["logits"], w["params"], w["u"], mask=w.get("mask"), hist=w.get("hist"),
+                   hist_len=w.get("hist_len"), draft=draft, u2=u2, force_token=force)
+    ref = oracle_rows(w, draft=draft, u2=u2)
+    for r in range(b):
+        if force[r] >= 0:
+            assert g["tokens"][r] == force[r] and bool(g["accepted"][r]) == (force[r] == draft[r]) and g["forced"][r] == 1
+        else:
+            assert g["tokens"][r] == ref[r][0] and bool(g["accepted"][r]) == ref[r][1]["accepted"] and g["forced"][r] == 0
+
+
+def test_append_history_decode_loop(gpu_ctx):
+    """Sampler::accept on the device (src/gen/session.cpp:419-421): six decode steps whose histories never leave the
+    GPU give the tokens of a host loop that keeps the histories itself, forced tokens included; a full history
+    buffer is left as it is."""
+    rng = np.random.default_rng(12)
+    o = pyoracle.oracle()
+    v, b, stride, steps = 3000, 12, 16, 6
+    p = api.make_params(b, 0.8, 0, 0.95, presence_penalty=0.4, frequency_penalty=0.3, repetition_penalty=1.3)
+    p["top_k"][::3] = 20
+    p["temperature"][1] = 0.0
+    hist = rng.integers(0, v, (b, stride)).astype(np.int32)
+    hist_len = rng.integers(0, 12, b).astype(np.uint32)
+    hist_len[2] = stride - 2  # fills up on the way
+    host_hist = [list(hist[r, : hist_len[r]]) for r in range(b)]
+    logits0 = (rng.standard_normal((b, v)) * 2).astype(np.float32)
+    batch = api.Batch(logits0, p, np.zeros(b, np.float32), hist=hist, hist_len=hist_len, force_token=np.full(b, -1, np.int32),
+                      append_history=True)
+    for step in range(steps):
+        logits = (rng.standard_normal((b, v)) * 2).astype(np.float32)
+        logits[np.arange(b), [h[-1] if h else 0 for h in host_hist]] += 3.0  # the penalties matter
+        u = rng.random(b).astype(np.float32)
+        force = np.full(b, -1, np.int32)
+        force[step % b] = int(rng.integers(0, v))
+        batch.d_logits.upload(logits)
+        batch.d_u.upload(u)
+        batch.d_force.upload(force)
+        _say("append step %d" % step)
+        gpu_ctx.sample_batch(batch.desc)
+        g = batch.results()
+        for r in range(b):
+            if force[r] >= 0:
+                tok = int(force[r])
+            else:
+                tok = o.sample(logits[r], pyoracle.params_from_record(p[r]), float(u[r]), np.array(host_hist[r], np.int32))[0]
+            assert g["tokens"][r] == tok, (step, r, g["tokens"][r], tok)
+            if len(host_hist[r]) < stride:
+                host_hist[r].append(tok)
+    ht, hl = batch.history()
+    for r in range(b):
+        assert hl[r] == len(host_hist[r]) and list(ht[r, : hl[r]]) == host_hist[r], r
+
+
 def test_config1(gpu_ctx):
     assert_parity(gpu_ctx, workloads.config1(rows=4))
 

@@ -252,3 +252,39 @@ def test_oracle_equals_reference(oracle, reference):
         draft = int(rng.integers(0, v)) if it % 2 else t1
         got = oracle.verify(logits, p, draft, float(u1), float(u2), hist, mask, order_mode=0)
         assert got == reference.verify(logits, p, seed, draft, hist, mask), it
+
+
+def test_close_forced_known_answers(oracle):
+    """ReasoningBudget::forced's last-stretch test (src/server/openai.cpp:589-604) on the reference's own cases
+    (tests/server_test.cpp:138-152: all logits 0, </think> at 1.0; three logits at 2.0 -> not forced, two -> forced),
+    and against a brute-force count."""
+    nv, end = 300, 271
+    logits = np.zeros(nv, np.float32)
+    assert oracle.close_forced(logits, end) == (end, 0)  # nothing above: taken
+    logits[end] = 1.0
+    assert oracle.close_forced(logits, end) == (end, 0)
+    logits[:3] = 2.0  # three above </think>: the fourth is not closed early (:147-149)
+    assert oracle.close_forced(logits, end) == (-1, 3)
+    logits[2] = 0.0  # third closes early (:150-151)
+    assert oracle.close_forced(logits, end) == (end, 2)
+    assert oracle.close_forced(logits, -1)[0] == -1 and oracle.close_forced(logits, nv)[0] == -1  # :590, :594
+    # ties are not above (strict >), NaNs never are
+    logits[10:20] = 1.0
+    logits[30] = np.nan
+    assert oracle.close_forced(logits, end) == (end, 2)
+    logits[end] = np.nan
+    assert oracle.close_forced(logits, end) == (end, 0)
+    rng = np.random.default_rng(3)
+    for _ in range(200):
+        n = int(rng.integers(1, 400))
+        x = np.round(rng.standard_normal(n) * 2).astype(np.float32)
+        t = int(rng.integers(0, n))
+        k = int(rng.integers(0, 6))
+        mask = rng.integers(0, 2**32, (n + 31) // 32, dtype=np.uint64).astype(np.uint32) if rng.integers(0, 2) else None
+        allowed = np.ones(n, bool) if mask is None else ((mask[np.arange(n) >> 5] >> (np.arange(n) & 31)) & 1).astype(bool)
+        tok, above = oracle.close_forced(x, t, k, mask)
+        if not allowed[t]:
+            assert tok == -1 and above == 0xFFFFFFFF
+            continue
+        want = int(np.sum(np.where(allowed, x, -np.inf) > x[t]))
+        assert above == want and tok == (t if want < k else -1)
