@@ -2238,26 +2238,6 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
     };
     const double m0 = (double)s0 * scale(b0), m1 = (double)s1 * scale(b1);
     const double want = (double)P.top_p * total64;
-    double all;
-    const double incl = block_incl_scan_f64(m0 + m1, all, sm.bs);
-    // The nucleus ends in the first bin (from the top) at which the running mass reaches `want`.  These sums
-    // associate differently from the sorted prefix sums that make the final decision, so one more non-empty
-    // bin is taken along: the list stops at the SECOND bin that satisfies the test.
-    const bool r0 = c0 && incl - m1 >= want, r1 = c1 && incl >= want;
-    uint32_t reached_total;
-    const uint32_t before = block_excl_scan_u32((uint32_t)r0 + (uint32_t)r1, reached_total, sm.bs);
-    uint32_t hit = kNone;
-    if (r0 && before + 1 == 2)
-        hit = b0;
-    else if (r1 && before + (uint32_t)r0 + 1 == 2)
-        hit = b1;
-    const uint32_t rev = block_min_u32(hit == kNone ? kNone : kBins - 1u - hit, sm.bs);
-    const uint32_t b_lo = rev == kNone ? 0u : kBins - 1u - rev; // not reached twice: keep every candidate
-    thr_bits = bin_lo_key(b_lo);
-
-    // candidates above each bin, and the workers' shares
-    uint32_t count_all;
-    const uint32_t above0 = block_excl_scan_u32(c0 + c1, count_all, sm.bs), above1 = above0 + c0;
     uint32_t* w_hi = L.wcount;            // highest bin of each worker
     uint32_t* w_lo = L.wcount + kWorkers; // lowest bin
     uint32_t* w_off = L.wcount + 2 * kWorkers;
@@ -2268,11 +2248,54 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         w_off[tid] = kNone;
         w_cnt[tid] = 0;
     }
-    if (b0 == b_lo)
-        sm.flag = above0 + c0;
-    if (b1 == b_lo)
-        sm.flag = above1 + c1;
+    // running mass (inclusive) and candidates above each bin (exclusive), from the top bin down: wave scans, and
+    // one exchange of the sixteen waves' totals for both
+    const double mass_w = __ockl_wfscan_add_f64(m0 + m1, true);
+    const uint32_t cnt_w = __ockl_wfscan_add_u32(c0 + c1, true);
+    if (lane_id() == kWave - 1) {
+        sm.bs.f64[wave_id()] = mass_w;
+        sm.bs.u64[wave_id()] = cnt_w;
+    }
     __syncthreads();
+    double pre_m = 0;
+    uint32_t pre_c = 0, count_all = 0;
+    for (int w = 0; w < kWaves; ++w) {
+        const double x = sm.bs.f64[w];
+        const uint32_t y = (uint32_t)sm.bs.u64[w];
+        if (w < wave_id()) {
+            pre_m += x;
+            pre_c += y;
+        }
+        count_all += y;
+    }
+    const double incl = pre_m + mass_w;
+    const uint32_t above0 = pre_c + cnt_w - (c0 + c1), above1 = above0 + c0;
+    // The nucleus ends in the first bin (from the top) at which the running mass reaches `want`.  These sums
+    // associate differently from the sorted prefix sums that make the final decision, so one more non-empty
+    // bin is taken along: the list stops at the SECOND bin that satisfies the test.
+    const bool r0 = c0 && incl - m1 >= want, r1 = c1 && incl >= want;
+    const uint32_t reached = (uint32_t)r0 + (uint32_t)r1;
+    const uint32_t reached_w = __ockl_wfscan_add_u32(reached, true);
+    if (lane_id() == kWave - 1)
+        sm.hist[wave_id()] = reached_w;
+    if (tid == 0) {
+        sm.ticket = 0;        // the lowest bin taken; not reached twice: every candidate is kept
+        sm.flag = count_all;  // the number of weights to sort
+    }
+    __syncthreads();
+    uint32_t before = reached_w - reached;
+    for (int w = 0; w < kWaves; ++w)
+        before += w < wave_id() ? sm.hist[w] : 0u;
+    if (r0 && before + 1 == 2) {
+        sm.ticket = b0;
+        sm.flag = above0 + c0;
+    } else if (r1 && before + (uint32_t)r0 + 1 == 2) {
+        sm.ticket = b1;
+        sm.flag = above1 + c1;
+    }
+    __syncthreads();
+    const uint32_t b_lo = sm.ticket;
+    thr_bits = bin_lo_key(b_lo);
     const uint32_t n0 = sm.flag;
     auto worker_of = [&](uint32_t b, uint32_t c, uint32_t above) {
         return (c == 0 || b < b_lo) ? kNone : min(kWorkers - 1u, (uint32_t)(((unsigned long long)above * kWorkers) / n0));
@@ -2305,15 +2328,16 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         plan->off[tid] = w_cnt[tid] ? w_off[tid] : 0u;
         plan->cnt[tid] = w_cnt[tid];
     }
-    if (tid == 0) {
-        uint32_t g = 0;
-        for (uint32_t w = 0; w < kWorkers; ++w) {
-            plan->gbase[w] = g;
-            g += (w_cnt[w] + kGroup - 1u) / kGroup;
+    if (wave_id() == 0) { // the workers' first group records: a scan over their group counts
+        const uint32_t mine = lane_id() < (int)kWorkers ? (w_cnt[lane_id()] + kGroup - 1u) / kGroup : 0u;
+        const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
+        if (lane_id() < (int)kWorkers)
+            plan->gbase[lane_id()] = upto - mine;
+        if (lane_id() == kWave - 1) {
+            plan->groups = upto;
+            plan->n0 = n0;
+            plan->total64 = total64;
         }
-        plan->groups = g;
-        plan->n0 = n0;
-        plan->total64 = total64;
     }
     __syncthreads();
     return n0;
