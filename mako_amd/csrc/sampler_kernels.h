@@ -3236,17 +3236,16 @@ __device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const 
 __device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uint32_t slices, float& m, uint32_t& argidx,
                                             uint32_t& n_cands, uint32_t& any_overflow)
 {
-    unsigned long long top = 0;
-    n_cands = 0;
-    any_overflow = 0;
-    for (uint32_t s = 0; s < slices; ++s) {
-        const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
-        const unsigned long long p = ((unsigned long long)order_key(st.wmax) << 32) | (unsigned long long)(kNone - st.argidx);
-        top = p > top ? p : top;
-        n_cands += st.n_emit;
-        any_overflow |= st.flags & kFlagOverflow;
-    }
-    const bool first_nan = sc.stats[(size_t)row * kMaxSlices].flags & kFlagFirstNan;
+    // lane s of every wave takes slice s (at most kMaxSlices = 64 of them): one load each, then wave reductions
+    const uint32_t s = min((uint32_t)lane_id(), slices - 1u);
+    const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
+    const bool mine = (uint32_t)lane_id() < slices;
+    const unsigned long long p =
+        mine ? ((unsigned long long)order_key(st.wmax) << 32) | (unsigned long long)(kNone - st.argidx) : 0ull;
+    const unsigned long long top = __ockl_wfred_max_u64(p);
+    n_cands = __ockl_wfred_add_u32(mine ? st.n_emit : 0u);
+    any_overflow = __ballot(mine && (st.flags & kFlagOverflow)) != 0ull ? kFlagOverflow : 0u;
+    const bool first_nan = __ballot(lane_id() == 0 && (st.flags & kFlagFirstNan)) != 0ull;
     m = order_unkey((uint32_t)(top >> 32));
     argidx = kNone - (uint32_t)top;
     if (argidx == kNone)
