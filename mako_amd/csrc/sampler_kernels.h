@@ -571,6 +571,21 @@ __device__ bool find_piece(const mako_sample_desc& d, uint32_t piece, uint32_t p
                            uint32_t& row, uint32_t& sub, BlockScratch& bs)
 {
     const uint32_t tid = threadIdx.x;
+    if (d.n_rows <= (uint32_t)kWave) {
+        // up to 64 rows: every wave works it out for itself, one row per lane, without a barrier
+        const uint32_t r = lane_id();
+        uint32_t pieces = 0;
+        if (r < d.n_rows)
+            pieces = classify(d.params[r]) == kNucleus ? per_nucleus : per_other;
+        const uint32_t upto = __ockl_wfscan_add_u32(pieces, true);
+        const unsigned long long bal = __ballot(piece >= upto - pieces && piece < upto);
+        if (bal == 0ull)
+            return false;
+        const int owner = __ffsll((long long)bal) - 1;
+        row = (uint32_t)owner;
+        sub = piece - (uint32_t)__builtin_amdgcn_readlane((int)(upto - pieces), owner);
+        return true;
+    }
     uint32_t before = 0;
     for (uint32_t base = 0; base < d.n_rows; base += kThreads) {
         const uint32_t r = base + tid;
