@@ -34,6 +34,7 @@ struct mako_sampler_ctx {
     uint8_t* st_acc = nullptr;
     std::string err = "";
     bool profile = false, profiled = false;
+    uint32_t cus = 256; // compute units: workgroups of the finishing kernels that run at a time
     hipEvent_t ev[MAKO_SAMPLER_KERNELS + 1] = {};
 };
 
@@ -91,6 +92,12 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     ctx->max_vocab = max_vocab;
     ctx->max_hist = max_hist;
     MAKO_HIP(ctx, hipSetDevice(device));
+    {
+        int n = 0;
+        MAKO_HIP(ctx, hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device));
+        if (n > 0)
+            ctx->cus = (uint32_t)n;
+    }
     mako::Scratch& sc = ctx->sc;
     sc.vpad = ((uint64_t)max_vocab + 1023u) & ~1023ull;
     const size_t rv = (size_t)max_rows * sc.vpad;
@@ -121,8 +128,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.gt.pack, rg));
     MAKO_HIP(ctx, dev_alloc(&sc.gt.quarters, rg * 4));
     MAKO_HIP(ctx, dev_alloc(&sc.bin_worker, (size_t)max_rows * mako::kBins));
-    MAKO_HIP(ctx, dev_alloc(&sc.work_n, 2));
-    MAKO_HIP(ctx, hipMemset(sc.work_n, 0, 2 * sizeof(uint32_t)));
+    MAKO_HIP(ctx, dev_alloc(&sc.work_n, 8));
+    MAKO_HIP(ctx, hipMemset(sc.work_n, 0, 8 * sizeof(uint32_t)));
     MAKO_HIP(ctx, dev_alloc(&sc.work_sort, (size_t)max_rows * mako::kWorkers));
     MAKO_HIP(ctx, dev_alloc(&sc.work_tail, (size_t)max_rows));
     MAKO_HIP(ctx, dev_alloc(&ctx->sc_dev, 1));
@@ -235,6 +242,11 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     const bool vec = d.n_vocab % 4 == 0 && d.logits_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(d.logits) & 15u) == 0;
     const size_t lds = d.hist_tokens ? (size_t)slice_len * sizeof(uint32_t) : 0;
     const dim3 grid(slices, d.n_rows);
+    // The second pass cuts top_k == 0 rows into pieces of one to four blocks of 4096 logits (decided on the device:
+    // pieces finer than slices only while all of them fit one round of workgroups), so this many workgroups can
+    // have work; the others leave after a look at the rows' parameters.
+    const uint32_t pieces_max = std::min<uint32_t>(mako::kMaxSlices, std::max(slices, (d.n_vocab + 4095u) / 4096u));
+    const uint32_t finish_wgs = std::max(d.n_rows * slices, std::min(ctx->cus, d.n_rows * pieces_max));
     // histories of up to 2 (8) entries per thread stay in registers; longer ones take the generic route
     const int kh = !d.hist_tokens ? 2 : (d.hist_stride <= 2 * mako::kThreads ? 2 : (d.hist_stride <= 8 * mako::kThreads ? 8 : 0));
     const bool prof = ctx->profile;
@@ -247,13 +259,13 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     do {                                                                                                           \
         if (d.close_token)                                                                                         \
             hipLaunchKernelGGL((mako::scan_kernel<V, K, true>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc_dev,   \
-                               slice_len);                                                                         \
+                               slice_len, ctx->cus);                                                               \
         else                                                                                                       \
             hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc_dev,        \
-                               slice_len);                                                                         \
+                               slice_len, ctx->cus);                                                               \
         MAKO_MARK(1);                                                                                              \
-        hipLaunchKernelGGL((mako::finish_kernel<V, K>), grid, dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev,  \
-                           slices, slice_len);                                                                     \
+        hipLaunchKernelGGL((mako::finish_kernel<V, K>), dim3(1, finish_wgs), dim3(mako::kThreads),                 \
+                           mako::kDynLds, st, d, ctx->sc_dev, slices);                                             \
         MAKO_MARK(2);                                                                                              \
     } while (0)
     MAKO_MARK(0);

@@ -192,7 +192,9 @@ struct Scratch {
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
     // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
     // (finish_kernel and plan_kernel get the same effect from find_piece().)
-    uint32_t* work_n;      // [2] entries in work_sort, work_tail; zeroed by scan_kernel
+    uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); then, 16-byte aligned at [4],
+                           // the second pass's pieces per top_k == 0 row, their length and the number of workgroups
+                           // with work (scan_kernel's first workgroup decides, see second_pass_pieces())
     uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel and plan_kernel
     uint32_t* work_tail;   // [max_rows] row; appended by plan_kernel
     uint64_t vpad;
@@ -563,6 +565,34 @@ struct alignas(16) ScanShared {
     uint32_t ci[kCap];
 };
 
+// Into how many pieces finish_kernel cuts each top_k == 0 row, and how long a piece is.  A piece is one to four
+// blocks of 4096 logits (a slice is four): as few blocks as keep all the pieces of the batch within one round of
+// workgroups (`cus` of them run at a time, one per CU), since the pass is bound by instruction issue and more
+// workgroups with less work each finish sooner.  Worked out from the rows' parameters by one wave of scan_kernel's
+// first workgroup and left in Scratch::work_n; batches of more than 64 rows take whole slices.
+__device__ __forceinline__ uint32_t second_pass_pieces(const mako_sample_desc& d, uint32_t slices, uint32_t slice_len,
+                                                       uint32_t cus, uint32_t& piece_len, uint32_t& busy)
+{
+    piece_len = slice_len;
+    busy = d.n_rows * slices; // (no more than that)
+    if (d.n_rows > (uint32_t)kWave)
+        return slices;
+    const uint32_t r = lane_id();
+    const bool nucleus = r < d.n_rows && classify(d.params[r]) == kNucleus;
+    const uint32_t rows = (uint32_t)__popcll(__ballot(nucleus));
+    busy = rows * slices;
+    for (uint32_t blocks = 1; blocks < 4u; ++blocks) {
+        const uint32_t len = blocks * 4096u;
+        const uint32_t n = (d.n_vocab + len - 1u) / len;
+        if (len < slice_len && n <= kMaxSlices && rows * n <= cus) {
+            piece_len = len;
+            busy = rows * n;
+            return n;
+        }
+    }
+    return slices;
+}
+
 // Which piece of work does workgroup `piece` of finish_kernel (per_nucleus = slices, per_other = 1) or of plan_kernel
 // (1, 0) serve?  Rows are taken in order, each contributing per_nucleus pieces if it is a top_k == 0 row and
 // per_other otherwise.  Every workgroup works this out for itself from the rows' parameters (a few loads and one
@@ -627,15 +657,20 @@ __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 // (ABOVE: the batch has close tokens, whose logits' ranks are counted on the way; a variant of its own because the
 // count's registers would cost every other batch half its occupancy)
 template <bool VEC, int KH, bool ABOVE = false>
-__global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, const Scratch* sc_dev, uint32_t slice_len)
+__global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, const Scratch* sc_dev, uint32_t slice_len,
+                                                        uint32_t cus)
 {
     const Scratch& sc = *sc_dev;
     MAKO_ROW(blockIdx.y);
+#ifdef MAKO_TIMING_SCAN
+    MAKO_WG_TIMER;
+#endif
     // (16-byte alignment: the table is cleared and read with 128-bit LDS operations, which crawl when misaligned)
     extern __shared__ __align__(16) uint32_t s_dyn[]; // [slice_len] token counts when the row has penalties
     __shared__ ScanShared sm;
 
     const uint32_t row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
+    MAKO_STAMP(28);
     const uint32_t lo = slice * slice_len;
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
     const mako_sampling_params P = d.params[row];
@@ -651,6 +686,12 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
             sc.work_n[0] = 0;
             sc.work_n[1] = 0;
         }
+    }
+    if (row == 0 && slice == 0 && wave_id() == 1) { // how the second pass will be cut up
+        uint32_t piece_len, busy;
+        const uint32_t pieces = second_pass_pieces(d, gridDim.x, slice_len, cus, piece_len, busy);
+        if (lane_id() == 0)
+            *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(pieces, piece_len, busy, 0u);
     }
     // ReasoningBudget::forced's question (src/server/openai.cpp:598-602), answered in the same pass over the logits
     bool want_above = false;
@@ -674,6 +715,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
         load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv, ex);
     }
 
+    MAKO_STAMP(29);
     // maximum of the thread's logits (NaNs ignored), then of the wave, then of the slice
     float best = -INFINITY;
 #pragma unroll
@@ -700,6 +742,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
             sm.wave_above[wave_id()] = above;
     }
     __syncthreads();
+    MAKO_STAMP(30);
     uint32_t mkey = 0, tau_key = 0xffffffffu, above_slice = 0;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
@@ -768,6 +811,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
             }
     }
     __syncthreads();
+    MAKO_STAMP(31);
     if (emits) {
         const uint32_t n = sm.emit_n;
         if (n > kCap)
@@ -785,6 +829,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
         st.flags |= sm.emit_flags;
         sc.stats[(size_t)row * kMaxSlices + slice] = st;
     }
+    MAKO_STAMP(27);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -3148,13 +3193,18 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
     double sum = 0;
     uint32_t n = 0;
     uint32_t qb[16], qe[KH > 0 ? KH : 1]; // bits(q), 0 where q is not a candidate
+    // (a piece may be shorter than the sixteen logits per thread: whole blocks past its end are skipped; the test is
+    // the same for every thread)
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j) {
-        const float q = weight_of(wv[j], m, inv_t, sm.tab);
-        qb[j] = (q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
-        if (qb[j]) {
-            sum += (double)q;
-            ++n;
+        qb[j] = 0u;
+        if (lo + (VEC ? (j / 4u) * 4096u : j * (uint32_t)kThreads) < hi) {
+            const float q = weight_of(wv[j], m, inv_t, sm.tab);
+            qb[j] = (q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
+            if (qb[j]) {
+                sum += (double)q;
+                ++n;
+            }
         }
     }
 #pragma unroll
@@ -3335,12 +3385,12 @@ __device__ __forceinline__ uint32_t row_forced(const mako_sample_desc& d, const 
     return kind;
 }
 
-// grid = (slices, rows) workgroups, of which workgroup i serves the i-th piece of work in row order: one piece per
-// row, and one per slice for top_k == 0 rows (find_piece).  The busy workgroups are then the first ones dispatched
-// and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
+// Second pass over the top_k == 0 rows.  grid = (most pieces a row can have, rows) workgroups, of which workgroup i
+// serves the i-th piece of work in row order, second_pass_pieces() per top_k == 0 row (find_piece): the busy
+// workgroups are then the first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the
+// mix of rows.
 template <bool VEC, int KH>
-__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices,
-                                                          uint32_t slice_len)
+__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
 {
     const Scratch& sc_arg = *sc_dev;
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
@@ -3349,8 +3399,13 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
 #ifdef MAKO_TIMING_FINISH
     MAKO_WG_TIMER;
 #endif
-    uint32_t row, slice;
-    if (!find_piece(d_arg, blockIdx.y * gridDim.x + blockIdx.x, slices, 1u, row, slice, sm.bs))
+    // (pieces per row, their length, workgroups with work: the others leave at once)
+    const uint4 cut = *reinterpret_cast<const uint4*>(sc_arg.work_n + 4);
+    if (blockIdx.y * gridDim.x + blockIdx.x >= cut.z)
+        return;
+    const uint32_t pieces = cut.x, piece_len = cut.y;
+    uint32_t row, piece;
+    if (!find_piece(d_arg, blockIdx.y * gridDim.x + blockIdx.x, pieces, 0u, row, piece, sm.bs))
         return;
     const uint32_t tid = threadIdx.x;
     MAKO_ROW(row);
@@ -3363,17 +3418,59 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     L.sortk = s_dyn64;                                             // 32 KB
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);    // next 16 KB
     const mako_sampling_params& P = s_args.P;
-    const RowClass cls = classify(P);
     MAKO_STAMP(0);
+    if (d.force_token || d.close_token) { // a forced row needs no weights (plan_kernel writes its token)
+        int32_t ftok;
+        uint32_t above;
+        if (row_forced(d, sc, row, slices, ftok, above) != MAKO_FORCED_NONE)
+            return;
+    }
+    if (tid < 32)
+        sm.tab[tid] = k_exp2_tab[tid];
+    __syncthreads();
+    float m;
+    uint32_t argidx, n_cands, any_overflow;
+    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
+    MAKO_STAMP(1);
+    const uint32_t hl = d.hist_tokens ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
+    if (hl > 0 && !penalties_neutral(P))
+        slice_partial<VEC, KH, true>(d, sc, row, piece, piece_len, P, hl, m, L);
+    else
+        slice_partial<VEC, KH, false>(d, sc, row, piece, piece_len, P, hl, m, L);
+}
+
+// grid = (1, rows), one workgroup per row.  Rows whose token is forced, greedy rows and top-k rows are finished here
+// from the records scan_kernel left; a top_k == 0 row's exact total, candidate count and weight histogram (from
+// finish_kernel) are summed over its pieces and the row is planned: handed to sort_kernel's workers, or, when the
+// nucleus is narrow enough to end inside the candidate lists, to its worker 0 alone.
+__global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
+{
+    const Scratch& sc_arg = *sc_dev;
+    extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
+    __shared__ FinishShared sm;
+    __shared__ ArgsLds s_args;
+    const uint32_t row = blockIdx.y;
+    const uint32_t tid = threadIdx.x;
+    MAKO_ROW(row);
+    stage_args(d_arg, sc_arg, row, s_args);
+    const mako_sample_desc& d = s_args.d;
+    const Scratch& sc = s_args.sc;
+    const mako_sampling_params& P = s_args.P;
+    FinishLds L;
+    L.sm = &sm;
+    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
+    L.sortk = s_dyn64;
+    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
+    const RowClass cls = classify(P);
     if (d.force_token || d.close_token) { // uniform
         int32_t ftok;
         uint32_t above;
         const uint32_t kind = row_forced(d, sc, row, slices, ftok, above);
-        if (slice == 0 && tid == 0 && d.out_above)
+        if (tid == 0 && d.out_above)
             d.out_above[row] = above;
         if (kind != MAKO_FORCED_NONE) {
             // a token >= 0 is taken instead of sampling, and a draft is kept only if it matches (session.hpp:43-45)
-            if (slice == 0 && tid == 0) {
+            if (tid == 0) {
                 RowOut o;
                 o.token = ftok;
                 o.n_cand = 0;
@@ -3390,12 +3487,9 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     if (tid < 32)
         sm.tab[tid] = k_exp2_tab[tid];
     __syncthreads();
-
     float m;
     uint32_t argidx, n_cands, any_overflow;
     row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
-
-    MAKO_STAMP(1);
     if (cls == kGreedy) { // sampler.cpp:77-78, 88-92
         if (tid == 0) {
             RowOut o;
@@ -3410,118 +3504,69 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
         return;
     }
 
-    if (cls == kNucleus) {
-        // second pass, all slices of the row in parallel; plan_kernel continues once every slice is through
-        const uint32_t hl = d.hist_tokens ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
-        if (hl > 0 && !penalties_neutral(P))
-            slice_partial<VEC, KH, true>(d, sc, row, slice, slice_len, P, hl, m, L);
-        else
-            slice_partial<VEC, KH, false>(d, sc, row, slice, slice_len, P, hl, m, L);
-        return;
-    }
-    if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
-        if (tid == 0) {
-            sc.plan[row].total64 = (double)m; // carries the row maximum and its first index to the whole-row path
-            sc.plan[row].n0 = argidx;
-            sc.plan[row].flag = 2;
-            sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
-        }
-        return;
-    }
-
-    // ---- top-k rows: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
-    const float inv_t = 1.0f / P.temperature;
-    const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
-    const float q_bound = candidate_bound(sc, row, slices, m, inv_t, floor_q, sm);
-    MAKO_STAMP(3);
-    uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax); // upper half of the dynamic block
-    uint32_t* jf = kf + kSortMax;
-    uint32_t n_valid = 0;
-    uint32_t n_list = kNone;
-    if (!d.draft) // the top_k-th weight's neighbourhood only
-        n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, P.top_k, 0u, kf, jf, n_valid, L);
-    if (n_list == kNone)
-        n_valid = n_cands <= 1024u ? sort_candidates<1>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L)
-                                   : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
-    MAKO_STAMP(4);
-    // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
-    const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
-    if (!ok) {
-        if (tid == 0) {
-            sc.plan[row].total64 = (double)m;
-            sc.plan[row].n0 = argidx;
-            sc.plan[row].flag = 2;
-            sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
-        }
-        return;
-    }
-    if (n_valid == 0) {
-        fallback_row(d, row, argidx);
-        return;
-    }
-    sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L); // sampler.cpp:40-43
-}
-
-// grid = (1, rows), workgroup i serving the i-th top_k == 0 row (find_piece): the row's exact total, candidate count and weight histogram are summed
-// over its slices and the row is planned: handed to sort_kernel's workers, or, when the nucleus is narrow enough to
-// end inside the candidate lists, to its worker 0 alone.
-__global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
-{
-    const Scratch& sc_arg = *sc_dev;
-    extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
-    __shared__ FinishShared sm;
-    __shared__ ArgsLds s_args;
-    uint32_t row, sub;
-    if (!find_piece(d_arg, blockIdx.y, 1u, 0u, row, sub, sm.bs))
-        return;
-    const uint32_t tid = threadIdx.x;
-    MAKO_ROW(row);
-    stage_args(d_arg, sc_arg, row, s_args);
-    const mako_sample_desc& d = s_args.d;
-    const Scratch& sc = s_args.sc;
-    const mako_sampling_params& P = s_args.P;
-    FinishLds L;
-    L.sm = &sm;
-    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
-    L.sortk = s_dyn64;
-    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
-    if (d.force_token || d.close_token) { // finish_kernel gave a forced row its token
-        int32_t ftok;
-        uint32_t above;
-        if (row_forced(d, sc, row, slices, ftok, above) != MAKO_FORCED_NONE)
+    if (cls != kNucleus) {
+        if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
+            if (tid == 0) {
+                sc.plan[row].total64 = (double)m; // carries the row maximum and its first index to the whole-row path
+                sc.plan[row].n0 = argidx;
+                sc.plan[row].flag = 2;
+                sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
+            }
             return;
+        }
+
+        // ---- top-k rows: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
+        const float inv_t = 1.0f / P.temperature;
+        const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
+        const float q_bound = candidate_bound(sc, row, slices, m, inv_t, floor_q, sm);
+        MAKO_STAMP(3);
+        uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax); // upper half of the dynamic block
+        uint32_t* jf = kf + kSortMax;
+        uint32_t n_valid = 0;
+        uint32_t n_list = kNone;
+        if (!d.draft) // the top_k-th weight's neighbourhood only
+            n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, P.top_k, 0u, kf, jf, n_valid, L);
+        if (n_list == kNone)
+            n_valid = n_cands <= 1024u ? sort_candidates<1>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L)
+                                       : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
+        MAKO_STAMP(4);
+        // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
+        const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
+        if (!ok) {
+            if (tid == 0) {
+                sc.plan[row].total64 = (double)m;
+                sc.plan[row].n0 = argidx;
+                sc.plan[row].flag = 2;
+                sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
+            }
+            return;
+        }
+        if (n_valid == 0) {
+            fallback_row(d, row, argidx);
+            return;
+        }
+        sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L); // sampler.cpp:40-43
+
+        return;
     }
+
     MAKO_STAMP(2);
-    // this thread's two bins of the row's histogram (left zero for the next batch), the slices' exact sums in order
+    const uint32_t pieces = uniform_u32(sc.work_n[4]);
+    // this thread's two bins of the row's histogram (left zero for the next batch), the pieces' exact sums (one per
+    // lane, added up in the wave reduction's fixed order)
     unsigned long long* bins = sc.bins + (size_t)row * kBins;
     const unsigned long long rec0 = bins[kBins - 1u - 2u * tid], rec1 = bins[kBins - 2u - 2u * tid];
     const uint32_t bin_c0 = (uint32_t)(rec0 >> kBinSumBits), bin_c1 = (uint32_t)(rec1 >> kBinSumBits);
     const unsigned long long bin_s0 = rec0 & ((1ull << kBinSumBits) - 1ull), bin_s1 = rec1 & ((1ull << kBinSumBits) - 1ull);
-    double row_total = 0;
-    uint32_t row_n0 = 0;
-    for (uint32_t s0 = 0; s0 < slices; s0 += 8u) {
-        uint32_t pn[8];
-        double ps[8];
-#pragma unroll
-        for (uint32_t u = 0; u < 8; ++u) {
-            const uint32_t sl = min(s0 + u, slices - 1u);
-            ps[u] = sc.part_sum[(size_t)row * kMaxSlices + sl];
-            pn[u] = sc.part_n[(size_t)row * kMaxSlices + sl];
-        }
-#pragma unroll
-        for (uint32_t u = 0; u < 8; ++u)
-            if (s0 + u < slices) {
-                row_total += ps[u];
-                row_n0 += pn[u];
-            }
-    }
+    const uint32_t pc = min((uint32_t)lane_id(), pieces - 1u); // pieces <= kMaxSlices = 64
+    const double ps = sc.part_sum[(size_t)row * kMaxSlices + pc];
+    const uint32_t pn = sc.part_n[(size_t)row * kMaxSlices + pc];
+    const double row_total = __ockl_wfred_add_f64((uint32_t)lane_id() < pieces ? ps : 0.0);
+    const uint32_t row_n0 = __ockl_wfred_add_u32((uint32_t)lane_id() < pieces ? pn : 0u);
     if (rec0)
         bins[kBins - 1u - 2u * tid] = 0;
     if (rec1)
         bins[kBins - 2u - 2u * tid] = 0;
-    float m;
-    uint32_t argidx, n_cands, any_overflow;
-    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
     MAKO_STAMP(15);
     if (row_n0 == 0) {
         fallback_row(d, row, argidx);
@@ -3542,11 +3587,11 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         sc.plan[row].flag = !fits ? 2 : (narrow ? 3 : 1);
     }
     // the row's pieces of work for sort_kernel (all workers, or worker 0 alone) and tail_kernel
-    const uint32_t pieces = (fits && !narrow) ? kWorkers : 1u;
+    const uint32_t work = (fits && !narrow) ? kWorkers : 1u;
     if (tid == 0)
-        sm.flag = atomicAdd(&sc.work_n[0], pieces);
+        sm.flag = atomicAdd(&sc.work_n[0], work);
     __syncthreads();
-    if (tid < pieces)
+    if (tid < work)
         sc.work_sort[sm.flag + tid] = (row << 8) | tid;
     if (tid == 0 && fits && !narrow)
         sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
