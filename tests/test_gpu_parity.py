@@ -388,6 +388,22 @@ def test_narrow_nucleus_inside_one_slice(gpu_ctx):
     assert (g["path"] == api.PATH_GENERAL).any() and (g["path"] == api.PATH_NUCLEUS).any()
 
 
+@pytest.mark.parametrize("v", [40000, 129280])
+def test_second_pass_piece_sizes(gpu_ctx, v):
+    """The second pass over top_k == 0 rows is cut into pieces of one to four 4096-logit blocks depending on how many
+    such rows the batch has: every cut gives the same tokens, totals and candidate lists."""
+    rng = np.random.default_rng(600 + v)
+    b = 64
+    for n_nucleus in (1, 5, 8, 16, 21, 33, 64):
+        w = _random_case(rng, v, b)
+        w["params"]["temperature"] = np.float32(0.9)
+        w["params"]["top_p"] = np.float32(0.93)
+        w["params"]["top_k"] = np.uint32(40)
+        w["params"]["top_k"][rng.permutation(b)[:n_nucleus]] = 0
+        _say("piece sizes v=%d nucleus rows=%d" % (v, n_nucleus))
+        assert_parity(gpu_ctx, w, cap=256)
+
+
 def test_more_rows_than_threads():
     """1100 rows in one batch: the per-workgroup search for its piece of work loops over the rows."""
     ctx = api.SamplerContext(max_rows=1100, max_vocab=320, max_hist=0)
