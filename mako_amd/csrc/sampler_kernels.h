@@ -3217,18 +3217,23 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
         }
     }
     MAKO_STAMP(25);
-    const double total = block_sum_f64(sum, sm.bs); // (its barriers also retire every use of L.cnt above)
-    const uint32_t count = block_sum_u32(n, sm.bs);
-    if (threadIdx.x == 0) {
-        sc.part_sum[(size_t)row * kMaxSlices + slice] = total;
-        sc.part_n[(size_t)row * kMaxSlices + slice] = count;
+    // the piece's sum and count: wave reductions, one exchange of the sixteen waves' results for both (the barrier
+    // also retires every use of L.cnt above); they are stored at the very end, so that no barrier waits for the store
+    {
+        const double sw = __ockl_wfred_add_f64(sum);
+        const uint32_t nw = __ockl_wfred_add_u32(n);
+        if (lane_id() == 0) {
+            sm.bs.f64[wave_id()] = sw;
+            sm.bs.u64[wave_id()] = nw;
+        }
     }
+    lds_barrier();
     // bits(q) of every logit of the slice (0 = not a candidate) and their histogram, for nucleus_big_row()
     uint32_t* qk = reinterpret_cast<uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
     unsigned long long* hist = reinterpret_cast<unsigned long long*>(L.cnt); // count << kBinSumBits | significands
     for (uint32_t b = threadIdx.x; b < kBins; b += kThreads)
         hist[b] = 0;
-    __syncthreads();
+    lds_barrier();
     MAKO_STAMP(26);
     // one candidate and the significand of a positive float (subnormals: no hidden bit, as seqfp::split)
     auto record = [](uint32_t b) {
@@ -3261,13 +3266,23 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
             if (qe[k])
                 atomicAdd(&hist[weight_bin(qe[k])], record(qe[k]));
         }
-    __syncthreads();
+    lds_barrier(); // (the histogram is complete; nobody waits for the stores above)
     MAKO_STAMP(27);
     // the slice's non-empty bins are added to the row's histogram (a few hundred atomics per slice, none waited for)
     unsigned long long* bins = sc.bins + (size_t)row * kBins;
     for (uint32_t b = threadIdx.x; b < kBins; b += kThreads)
         if (hist[b])
             atomicAdd(&bins[b], hist[b]);
+    if (threadIdx.x == 0) {
+        double total = 0;
+        uint32_t count = 0;
+        for (int w = 0; w < kWaves; ++w) { // waves in order: the same inputs always give the same bits
+            total += sm.bs.f64[w];
+            count += (uint32_t)sm.bs.u64[w];
+        }
+        sc.part_sum[(size_t)row * kMaxSlices + slice] = total;
+        sc.part_n[(size_t)row * kMaxSlices + slice] = count;
+    }
 }
 
 // Kernel arguments that are handed on by reference to out-of-line device functions would be spilled to scratch
