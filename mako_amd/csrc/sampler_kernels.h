@@ -433,6 +433,28 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
 {
     const uint32_t tid = threadIdx.x;
     const float nan = __uint_as_float(0x7fc00000u);
+    // My history entries go first: loads return in the order they were issued, so whatever waits for these does not
+    // wait for the logits behind them, and the counting in LDS below runs while the logits are still on their way.
+    // (Loads from clamped positions, issued without branches between them; what was not wanted is dropped
+    // afterwards: a branch around each load would make every load wait for the one before.)
+    const bool extras = KH > 0 && pen; // uniform
+    const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
+    const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
+    uint32_t tok[KH > 0 ? KH : 1], cnt[KH > 0 ? KH : 1];
+    bool have[KH > 0 ? KH : 1];
+    if (extras) {
+#pragma unroll
+        for (int k = 0; k < KH; ++k) {
+            const uint32_t h = tid + (uint32_t)k * kThreads;
+            have[k] = h < hl;
+            tok[k] = (uint32_t)ht[have[k] ? h : 0u]; // hl > 0 here
+        }
+        if (hc) {
+#pragma unroll
+            for (int k = 0; k < KH; ++k)
+                cnt[k] = hc[have[k] ? tid + (uint32_t)k * kThreads : 0u];
+        }
+    }
     RawSlice<VEC> raw;
     load_raw<VEC>(d, row, lo, hi, raw);
     overlap();
@@ -452,27 +474,10 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         finish_slice<VEC>(raw, lo, hi, P, true, s_cnt, wv);
         return;
     }
-    // my history entries, and the masked raw logits of those that fall into this slice
-    const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
-    const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
+    // the masked raw logits of the entries that fall into this slice (asked for now, looked at after the counting)
     const float* lrow = d.logits + (int64_t)row * d.logits_stride;
     const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
-    uint32_t tok[KH > 0 ? KH : 1], cnt[KH > 0 ? KH : 1];
     float rawv[KH > 0 ? KH : 1];
-    // (loads from clamped positions, issued in two groups without branches between them; what was not wanted is
-    // dropped afterwards: a branch around each load would make every load wait for the one before)
-    bool have[KH > 0 ? KH : 1];
-#pragma unroll
-    for (int k = 0; k < KH; ++k) {
-        const uint32_t h = tid + (uint32_t)k * kThreads;
-        have[k] = h < hl;
-        tok[k] = (uint32_t)ht[have[k] ? h : 0u]; // hl > 0 here
-    }
-    if (hc) {
-#pragma unroll
-        for (int k = 0; k < KH; ++k)
-            cnt[k] = hc[have[k] ? tid + (uint32_t)k * kThreads : 0u];
-    }
     uint32_t mw[KH > 0 ? KH : 1];
 #pragma unroll
     for (int k = 0; k < KH; ++k) {
@@ -484,46 +489,49 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         for (int k = 0; k < KH; ++k)
             mw[k] = mrow[(have[k] ? tok[k] : lo) >> 5];
     }
+    uint32_t bit[KH > 0 ? KH : 1];
 #pragma unroll
     for (int k = 0; k < KH; ++k) {
         if (!hc)
             cnt[k] = 1;
-        if (mrow && !((mw[k] >> (tok[k] & 31u)) & 1u))
-            rawv[k] = -INFINITY;
+        bit[k] = tok[k] & 31u;
         if (!have[k]) {
-            rawv[k] = nan;
             tok[k] = kNone;
             cnt[k] = 1;
         }
     }
+    // (barriers that order LDS traffic only: the logits stay in flight)
     uint4* z = reinterpret_cast<uint4*>(s_cnt); // slice_len is a multiple of 4
     for (uint32_t i = tid; i < slice_len / 4; i += kThreads)
         z[i] = make_uint4(0, 0, 0, 0);
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int k = 0; k < KH; ++k)
         if (tok[k] != kNone)
             atomicAdd(&s_cnt[tok[k] - lo], cnt[k]);
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int k = 0; k < KH; ++k)
         if (tok[k] != kNone)
             cnt[k] = s_cnt[tok[k] - lo]; // occurrences of the token in the whole history
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int k = 0; k < KH; ++k)
         if (tok[k] != kNone)
             s_cnt[tok[k] - lo] = 0xffffffffu;
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int k = 0; k < KH; ++k)
         if (tok[k] != kNone)
             atomicMin(&s_cnt[tok[k] - lo], tid + (uint32_t)k * kThreads + 1u);
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int k = 0; k < KH; ++k)
         if (tok[k] != kNone && s_cnt[tok[k] - lo] == tid + (uint32_t)k * kThreads + 1u) {
-            ex.v[k] = penalize(rawv[k], cnt[k], P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+            float rv = rawv[k];
+            if (mrow && !((mw[k] >> bit[k]) & 1u))
+                rv = -INFINITY;
+            ex.v[k] = penalize(rv, cnt[k], P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
             ex.i[k] = tok[k];
         }
     finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv);
