@@ -75,19 +75,6 @@ __device__ __forceinline__ uint32_t block_min_u32(uint32_t v, BlockScratch& s)
     return t;
 }
 
-__device__ __forceinline__ unsigned long long block_max_u64(unsigned long long v, BlockScratch& s)
-{
-    v = __ockl_wfred_max_u64(v);
-    if (lane_id() == 0)
-        s.u64[wave_id()] = v;
-    __syncthreads();
-    unsigned long long t = 0;
-    for (int w = 0; w < kWaves; ++w)
-        t = s.u64[w] > t ? s.u64[w] : t;
-    __syncthreads();
-    return t;
-}
-
 // Exclusive prefix sum in thread order; `total` receives the workgroup sum.
 __device__ __forceinline__ uint32_t block_excl_scan_u32(uint32_t v, uint32_t& total, BlockScratch& s)
 {

@@ -404,6 +404,34 @@ def test_second_pass_piece_sizes(gpu_ctx, v):
         assert_parity(gpu_ctx, w, cap=256)
 
 
+def test_nucleus_sizes_around_path_boundaries(gpu_ctx):
+    """Nuclei just below and above the sizes at which the sorted tail changes its route (one wave up to 256 entries,
+    total and walk from LDS up to 1024, the list's head in LDS up to 2048, group maps beyond), each drawn at the
+    first entry, deep inside and at the very end."""
+    v = 129280
+    rng = np.random.default_rng(2024)
+    targets = [200, 256, 257, 300, 1000, 1024, 1025, 1100, 2040, 2048, 2049, 2100, 4096, 5000, 20000]
+    us = [0.0, 1e-7, 0.3, 0.9, 0.99999994]
+    base = -np.arange(v, dtype=np.float64) * 2e-4  # distinct, slowly falling weights
+    q = np.exp(base)
+    csum = np.cumsum(q)
+    rows = [(t, u) for t in targets for u in us]
+    b = len(rows)
+    logits = np.empty((b, v), np.float32)
+    p = api.make_params(b, 1.0, 0, 0.5)
+    uu = np.empty(b, np.float32)
+    for r, (t, u) in enumerate(rows):
+        logits[r] = base.astype(np.float32)[rng.permutation(v)]
+        p["top_p"][r] = np.float32((csum[t - 1] - 0.25 * q[t - 1]) / csum[-1])  # the nucleus ends at entry t or next to it
+        uu[r] = u
+    w = dict(name="path_boundaries", logits=logits, params=p, u=uu)
+    g = assert_parity(gpu_ctx, w, cap=64)
+    sizes = sorted(set(int(x) for x in g["n_cand"]))
+    _say("nucleus sizes: %s" % sizes)
+    assert min(sizes) <= 256 and any(256 < x <= 1024 for x in sizes) and any(1024 < x <= 2048 for x in sizes) \
+        and any(x > 2048 for x in sizes)
+
+
 def test_more_rows_than_threads():
     """1100 rows in one batch: the per-workgroup search for its piece of work loops over the rows."""
     ctx = api.SamplerContext(max_rows=1100, max_vocab=320, max_hist=0)
