@@ -851,6 +851,7 @@ struct alignas(16) FinishShared {
     uint32_t run[256];
     uint32_t flag;
     uint32_t ticket;
+    uint32_t aux;
     uint32_t soff[kMaxSlices + 1]; // first candidate of each slice in the row's flattened candidate list
 };
 
@@ -3093,39 +3094,56 @@ __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t s
     unsigned long long* sel = L.sortk + 256;                           // [kSmall]
     uint32_t* rank = reinterpret_cast<uint32_t*>(L.sortk + 256 + kSmall); // [kSmall]
     uint32_t* counter = rank + kSmall;
-    unsigned long long key[4];
-    candidate_keys<4>(sc, row, slices, n_cands, m, inv_t, floor_q, sm, key);
-    MAKO_STAMP(17);
+    // (cleared before the candidates are fetched: the barrier behind their weights then covers this too)
     if (tid < 512)
         hist[tid] = 0;
     if (tid < kSmall)
         rank[tid] = 0;
     if (tid == 0)
         *counter = 0;
-    __syncthreads();
+    unsigned long long key[4];
+    candidate_keys<4>(sc, row, slices, n_cands, m, inv_t, floor_q, sm, key);
+    MAKO_STAMP(17);
+    lds_barrier();
     uint32_t n_list;
     if (top_k > 0) {
 #pragma unroll
         for (uint32_t t = 0; t < 4; ++t)
             if (key[t])
                 atomicAdd(&hist[min((uint32_t)(key[t] >> 53), 511u)], 1u);
-        if (tid == 0) {
-            sm.flag = 0;
-            sm.ticket = 0;
+        lds_barrier();
+        if (wave_id() == 0) {
+            // one wave finds the bin of the top_k-th weight: eight bins per lane from the top down, a scan over the
+            // lanes' counts, then the lane that holds the bin goes through its eight
+            uint32_t c[8], mine = 0;
+#pragma unroll
+            for (uint32_t j = 0; j < 8; ++j) {
+                c[j] = hist[511u - (lane_id() * 8u + j)];
+                mine += c[j];
+            }
+            const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
+            const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)upto, kWave - 1);
+            uint32_t above = upto - mine, bits = 0, taken = 0;
+#pragma unroll
+            for (uint32_t j = 0; j < 8; ++j) {
+                if (above < top_k && top_k <= above + c[j]) {
+                    bits = (511u - (lane_id() * 8u + j)) << 21;
+                    taken = above + c[j];
+                }
+                above += c[j];
+            }
+            const unsigned long long hit = __ballot(taken != 0);
+            const int owner = hit ? __ffsll((long long)hit) - 1 : 0;
+            if (lane_id() == owner) {
+                sm.flag = hit ? bits : 0u; // 0 when the row has fewer than top_k candidates
+                sm.ticket = hit ? taken : 0u;
+                sm.aux = total;
+            }
         }
-        __syncthreads();
-        const uint32_t c = tid < 512 ? hist[511u - tid] : 0u;
-        uint32_t total;
-        const uint32_t above = block_excl_scan_u32(c, total, sm.bs);
-        if (tid < 512 && above < top_k && top_k <= above + c) {
-            sm.flag = (511u - tid) << 21;
-            sm.ticket = above + c;
-        }
-        __syncthreads();
-        n_valid = total;
-        thr_bits = sm.flag;                              // 0 when the row has fewer than top_k candidates
-        n_list = total < top_k ? total : sm.ticket;
-        __syncthreads();
+        lds_barrier();
+        n_valid = sm.aux;
+        thr_bits = sm.flag;
+        n_list = n_valid < top_k ? n_valid : sm.ticket;
     } else {
         uint32_t mine = 0, ge = 0;
 #pragma unroll
@@ -3350,27 +3368,25 @@ __device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uin
 __device__ float candidate_bound(const Scratch& sc, uint32_t row, uint32_t slices, float m, float inv_t, float floor_q,
                                  FinishShared& sm)
 {
-    const uint32_t tid = threadIdx.x;
-    if (tid == 0)
-        sm.flag = 0;
-    __syncthreads();
-    if (tid < slices) {
-        const SliceStat st = sc.stats[(size_t)row * kMaxSlices + tid];
-        sm.soff[tid + 1] = st.n_emit;
-        if (!(st.flags & kFlagComplete)) {
-            const float qb = weight_of(order_unkey(st.tau_key - 1u), m, inv_t, sm.tab);
-            if (qb >= floor_q && qb > 0.0f)
-                atomicMax(&sm.flag, __float_as_uint(qb)); // positive floats order like their bits
-        }
+    // lane s of every wave takes slice s, as in row_summary(); one wave leaves the offsets in LDS
+    const uint32_t s = min((uint32_t)lane_id(), slices - 1u);
+    const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
+    const bool mine = (uint32_t)lane_id() < slices;
+    uint32_t qbits = 0;
+    if (mine && !(st.flags & kFlagComplete)) {
+        const float qb = weight_of(order_unkey(st.tau_key - 1u), m, inv_t, sm.tab);
+        if (qb >= floor_q && qb > 0.0f)
+            qbits = __float_as_uint(qb); // positive floats order like their bits
     }
-    __syncthreads();
-    if (tid == 0) {
-        sm.soff[0] = 0;
-        for (uint32_t s = 0; s < slices; ++s)
-            sm.soff[s + 1] += sm.soff[s];
+    const float q_bound = __uint_as_float(__ockl_wfred_max_u32(qbits));
+    const uint32_t emitted = mine ? st.n_emit : 0u;
+    const uint32_t upto = __ockl_wfscan_add_u32(emitted, true);
+    if (wave_id() == 0) {
+        if (mine)
+            sm.soff[lane_id() + 1] = upto;
+        if (lane_id() == 0)
+            sm.soff[0] = 0;
     }
-    __syncthreads();
-    const float q_bound = __uint_as_float(sm.flag);
     __syncthreads();
     return q_bound;
 }
@@ -3708,6 +3724,9 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
     if (piece >= sc_arg.work_n[0])
         return;
+#ifdef MAKO_TIMING_SORT
+    MAKO_WG_TIMER;
+#endif
     const uint32_t item = sc_arg.work_sort[piece];
     const uint32_t row = item >> 8, w = item & 255u, tid = threadIdx.x;
     MAKO_ROW(row);
