@@ -3340,11 +3340,13 @@ __device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const 
 // First maximum of the row (std::max_element semantics, NaNs never win unless at index 0) and the totals of the
 // slices' candidate lists, from the records scan_kernel left.
 __device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uint32_t slices, float& m, uint32_t& argidx,
-                                            uint32_t& n_cands, uint32_t& any_overflow)
+                                            uint32_t& n_cands, uint32_t& any_overflow, SliceStat* lane_stat = nullptr)
 {
     // lane s of every wave takes slice s (at most kMaxSlices = 64 of them): one load each, then wave reductions
     const uint32_t s = min((uint32_t)lane_id(), slices - 1u);
     const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
+    if (lane_stat)
+        *lane_stat = st;
     const bool mine = (uint32_t)lane_id() < slices;
     const unsigned long long p =
         mine ? ((unsigned long long)order_key(st.wmax) << 32) | (unsigned long long)(kNone - st.argidx) : 0ull;
@@ -3365,12 +3367,9 @@ __device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uin
 // Where each slice's candidates start in the row's flattened candidate list (sm.soff), and the largest weight a
 // logit that was NOT emitted can have over all slices (0 if none can be a candidate): everything left behind
 // has an order key below its slice's tau_key.
-__device__ float candidate_bound(const Scratch& sc, uint32_t row, uint32_t slices, float m, float inv_t, float floor_q,
-                                 FinishShared& sm)
+__device__ float candidate_bound(const SliceStat& st, uint32_t slices, float m, float inv_t, float floor_q, FinishShared& sm)
 {
-    // lane s of every wave takes slice s, as in row_summary(); one wave leaves the offsets in LDS
-    const uint32_t s = min((uint32_t)lane_id(), slices - 1u);
-    const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
+    // `st`: the record of slice min(lane, slices - 1), as row_summary() hands it out; one wave leaves the offsets in LDS
     const bool mine = (uint32_t)lane_id() < slices;
     uint32_t qbits = 0;
     if (mine && !(st.flags & kFlagComplete)) {
@@ -3501,6 +3500,8 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     L.sortk = s_dyn64;
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
     const RowClass cls = classify(P);
+    if (cls != kNucleus)
+        MAKO_STAMP(0);
     if (d.force_token || d.close_token) { // uniform
         int32_t ftok;
         uint32_t above;
@@ -3528,7 +3529,10 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     __syncthreads();
     float m;
     uint32_t argidx, n_cands, any_overflow;
-    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
+    SliceStat lane_stat;
+    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow, &lane_stat);
+    if (cls != kNucleus)
+        MAKO_STAMP(1);
     if (cls == kGreedy) { // sampler.cpp:77-78, 88-92
         if (tid == 0) {
             RowOut o;
@@ -3557,7 +3561,7 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         // ---- top-k rows: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
         const float inv_t = 1.0f / P.temperature;
         const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
-        const float q_bound = candidate_bound(sc, row, slices, m, inv_t, floor_q, sm);
+        const float q_bound = candidate_bound(lane_stat, slices, m, inv_t, floor_q, sm);
         MAKO_STAMP(3);
         uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax); // upper half of the dynamic block
         uint32_t* jf = kf + kSortMax;
@@ -3770,10 +3774,11 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         const mako_sampling_params& P = s_args.P;
         float m;
         uint32_t argidx, n_cands, any_overflow;
-        row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
+        SliceStat lane_stat;
+        row_summary(sc, row, slices, m, argidx, n_cands, any_overflow, &lane_stat);
         const float inv_t = 1.0f / P.temperature;
         const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
-        const float q_bound = candidate_bound(sc, row, slices, m, inv_t, floor_q, sm);
+        const float q_bound = candidate_bound(lane_stat, slices, m, inv_t, floor_q, sm);
         MAKO_STAMP(3);
         uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax);
         uint32_t* jf = kf + kSortMax;
