@@ -224,6 +224,26 @@ def test_seqfp_host():
     assert " 0 failures" in out, out
 
 
+def test_generation_helpers_known_answers():
+    """LoopGuard and LookupDrafter (include/gen/) on the scenarios and numbers of the reference's own tests
+    (tests/loop_guard_test.cpp, tests/lookup_test.cpp), plus a brute-force restatement of the loop rule."""
+    exe = os.path.join(HERE, "cpu", "gen_helpers_test")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-I", os.path.join(HERE, "..", "include"),
+                    os.path.join(HERE, "cpu", "gen_helpers_test.cpp"), "-o", exe], check=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.strip().endswith("0 failures"), out.stdout
+
+
+def test_generation_helpers_equal_reference(reference):
+    """The same two classes against the unmodified reference classes compiled beside them (oracle/_ref/helpers_diff,
+    built where the reference tree is mounted): every push() / propose() / acceptance() on 360 000 random steps."""
+    exe = os.path.join(HERE, "..", "oracle", "_ref", "helpers_diff")
+    if not os.path.exists(exe):
+        pytest.skip("oracle/_ref/helpers_diff is not built (no reference tree)")
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.strip().endswith("0 differences"), out.stdout
+
+
 # ---------------------------------------------------------------- oracle vs the compiled reference, where built
 
 
