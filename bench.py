@@ -106,8 +106,9 @@ def main():
     w["u"] = np.array([orc.uniforms(int(s), 1)[0] for s in w["seeds"]], np.float32)
 
     ctx = api.SamplerContext(max_rows=rows, max_vocab=vocab, max_hist=w["hist"].shape[1] if "hist" in w else 0)
+    # (the host copy of the parameters goes along, as a serving loop that built them on the host would pass it)
     batch = api.Batch(w["logits"], w["params"], w["u"], mask=w.get("mask"), hist=w.get("hist"),
-                      hist_len=w.get("hist_len"), diagnostics=False)
+                      hist_len=w.get("hist_len"), diagnostics=False, params_host=True)
     row_bytes = workloads.bytes_per_row(w)
     batch_bytes = rows * row_bytes
     n_copies = max(2, -(-a.pool_mb * (1 << 20) // (rows * vocab * 4)))

@@ -105,6 +105,11 @@ typedef struct mako_sample_desc {
      * hist_len[r] < hist_stride (else the history is left as it is).  hist_tokens and hist_len must then be
      * writable device memory, hist_counts null, and draft null (the rows of a verify batch share one history). */
     uint32_t append_history;
+    /* Optional HOST copy of `params` (the SamplingParams originate on the host, src/gen/session.hpp:19-21).  When
+     * given, the call looks at it on the calling thread and leaves out the kernels that no row of the batch
+     * needs (a batch without top_k == 0 rows takes two launches instead of six).  It must hold the same values as
+     * the device array; the results never depend on whether it is given. */
+    const mako_sampling_params* params_host;
 } mako_sample_desc;
 
 typedef struct mako_sampler_ctx mako_sampler_ctx;

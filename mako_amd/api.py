@@ -78,6 +78,7 @@ class Desc(C.Structure):
         ("out_forced", C.c_void_p),
         ("out_above", C.c_void_p),
         ("append_history", C.c_uint32),
+        ("params_host", C.c_void_p),
     ]
 
 
@@ -177,7 +178,7 @@ class Batch:
 
     def __init__(self, logits, params, u, mask=None, hist=None, hist_len=None, hist_counts=None, draft=None, u2=None,
                  cand_cap=0, diagnostics=True, force_token=None, close_token=None, close_max_above=3,
-                 append_history=False):
+                 append_history=False, params_host=False):
         logits = np.ascontiguousarray(logits, np.float32)
         self.n_rows, self.n_vocab = logits.shape
         b = self.n_rows
@@ -186,7 +187,10 @@ class Batch:
         self.d_logits = self._up(logits)
         d.logits, d.logits_stride = self.d_logits.ptr, self.n_vocab
         d.n_rows, d.n_vocab = b, self.n_vocab
-        d.params = self._up(np.ascontiguousarray(params, PARAMS_DTYPE)).ptr
+        self.h_params = np.ascontiguousarray(params, PARAMS_DTYPE)
+        d.params = self._up(self.h_params).ptr
+        if params_host:  # the host copy, for the library to leave out kernels that have no work
+            d.params_host = self.h_params.ctypes.data
         self.d_u = self._up(np.ascontiguousarray(u, np.float32))
         d.u = self.d_u.ptr
         if mask is not None:

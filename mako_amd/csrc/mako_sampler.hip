@@ -145,7 +145,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
                              (const void*)mako::finish_kernel<true, 0>,  (const void*)mako::finish_kernel<false, 0>,
                              (const void*)mako::finish_kernel<true, 2>,  (const void*)mako::finish_kernel<false, 2>,
                              (const void*)mako::finish_kernel<true, 8>,  (const void*)mako::finish_kernel<false, 8>,
-                             (const void*)mako::sort_kernel,             (const void*)mako::plan_kernel,
+                             (const void*)mako::sort_kernel,             (const void*)mako::plan_kernel<false>,
+                             (const void*)mako::plan_kernel<true>,
                              (const void*)mako::tail_kernel};
     static_assert(mako::kSortLds >= mako::kDynLds, "sort_kernel's tail uses the finishing kernel's LDS layout");
     for (const void* k : kernels)
@@ -255,6 +256,17 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
         if (prof)                                                                                                  \
             MAKO_HIP(ctx, hipEventRecord(ctx->ev[i], st));                                                         \
     } while (0)
+    // which kernels have work: all of them unless the caller's host copy of the parameters says otherwise
+    bool any_nucleus = true, any_general = true;
+    if (d.params_host) {
+        any_nucleus = any_general = false;
+        for (uint32_t r = 0; r < d.n_rows; ++r) {
+            const mako::RowClass c = mako::classify(d.params_host[r]);
+            any_nucleus |= c == mako::kNucleus;
+            any_general |= c == mako::kGeneral;
+        }
+    }
+    const bool launch_sort = any_nucleus || any_general;
 #define MAKO_LAUNCH(V, K)                                                                                          \
     do {                                                                                                           \
         if (d.close_token)                                                                                         \
@@ -264,8 +276,9 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
             hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc_dev,        \
                                slice_len, ctx->cus);                                                               \
         MAKO_MARK(1);                                                                                              \
-        hipLaunchKernelGGL((mako::finish_kernel<V, K>), dim3(1, finish_wgs), dim3(mako::kThreads),                 \
-                           mako::kDynLds, st, d, ctx->sc_dev, slices);                                             \
+        if (any_nucleus)                                                                                           \
+            hipLaunchKernelGGL((mako::finish_kernel<V, K>), dim3(1, finish_wgs), dim3(mako::kThreads),             \
+                               mako::kDynLds, st, d, ctx->sc_dev, slices);                                         \
         MAKO_MARK(2);                                                                                              \
     } while (0)
     MAKO_MARK(0);
@@ -284,14 +297,22 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
 #undef MAKO_LAUNCH
     // top_k == 0 rows: plan from the row's histogram, sort by the plan, cut and draw; the stages talk through
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  Other rows cost a load.
-    hipLaunchKernelGGL(mako::plan_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev, slices);
+    if (launch_sort)
+        hipLaunchKernelGGL(mako::plan_kernel<false>, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev,
+                           slices);
+    else
+        hipLaunchKernelGGL(mako::plan_kernel<true>, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev,
+                           slices);
     MAKO_MARK(3);
-    hipLaunchKernelGGL(mako::partition_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), 0, st, d, ctx->sc_dev);
+    if (any_nucleus)
+        hipLaunchKernelGGL(mako::partition_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), 0, st, d, ctx->sc_dev);
     MAKO_MARK(4);
-    hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d, ctx->sc_dev,
-                       slices);
+    if (launch_sort)
+        hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d,
+                           ctx->sc_dev, slices);
     MAKO_MARK(5);
-    hipLaunchKernelGGL(mako::tail_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev);
+    if (any_nucleus)
+        hipLaunchKernelGGL(mako::tail_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev);
     MAKO_MARK(6);
 #undef MAKO_MARK
     ctx->profiled = prof;

@@ -217,7 +217,7 @@ constexpr uint32_t kKeyNegInf = 0x007fffffu; // order_key(-inf)
 
 enum RowClass { kGreedy = 0, kTopK = 1, kNucleus = 2, kGeneral = 3 };
 
-__device__ __forceinline__ RowClass classify(const mako_sampling_params& p)
+__host__ __device__ __forceinline__ RowClass classify(const mako_sampling_params& p)
 {
     if (p.temperature <= 0.0f) // Sampler::greedy, src/gen/sampler.hpp:26
         return kGreedy;
@@ -3481,8 +3481,13 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
 // from the records scan_kernel left; a top_k == 0 row's exact total, candidate count and weight histogram (from
 // finish_kernel) are summed over its pieces and the row is planned: handed to sort_kernel's workers, or, when the
 // nucleus is narrow enough to end inside the candidate lists, to its worker 0 alone.
+// INLINE_GENERAL: sort_kernel will not be launched for this batch (the host saw no row that needs it), so a row
+// that turns out to need the whole-row path after all is given it here.  (A variant of its own: the whole-row path
+// costs the kernel registers that the usual batches should not pay for.)
+template <bool INLINE_GENERAL>
 __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
 {
+    constexpr bool inline_general = INLINE_GENERAL;
     const Scratch& sc_arg = *sc_dev;
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
@@ -3549,6 +3554,10 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
 
     if (cls != kNucleus) {
         if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
+            if constexpr (inline_general) {
+                general_row(d, sc, row, P, m, argidx, L);
+                return;
+            }
             if (tid == 0) {
                 sc.plan[row].total64 = (double)m; // carries the row maximum and its first index to the whole-row path
                 sc.plan[row].n0 = argidx;
@@ -3576,6 +3585,11 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
         const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
         if (!ok) {
+            if constexpr (inline_general) {
+                __syncthreads(); // (the lists in LDS are done with)
+                general_row(d, sc, row, P, m, argidx, L);
+                return;
+            }
             if (tid == 0) {
                 sc.plan[row].total64 = (double)m;
                 sc.plan[row].n0 = argidx;

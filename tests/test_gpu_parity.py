@@ -432,6 +432,37 @@ def test_nucleus_sizes_around_path_boundaries(gpu_ctx):
         and any(x > 2048 for x in sizes)
 
 
+def test_host_parameter_copy_only_skips_work(gpu_ctx):
+    """With the host copy of the parameters the call leaves out kernels no row needs: the results are those of the
+    full pipeline and of the oracle, for batches without top_k == 0 rows (where a tied or overflowing top-k row
+    then takes the whole-row path inside plan_kernel), without any sampled row, with whole-row rows only, and mixed."""
+    rng = np.random.default_rng(77001)
+    v, b = 20000, 32
+    for case in range(8):
+        w = _random_case(rng, v, b)
+        p = w["params"]
+        if case < 3:  # top-k rows only (plus greedy ones), ties and overflows included by the generator
+            p["top_k"] = rng.choice(np.array([1, 3, 20, 50, 100, 128], np.uint32), b)
+            p["top_p"] = rng.choice(np.array([0.999, 0.95, 0.5], np.float32), b)
+            if case == 2:
+                w["logits"] = np.round(w["logits"]).astype(np.float32)  # heavy ties: uncertifiable candidate lists
+        elif case == 3:
+            p["temperature"] = np.float32(0.0)  # greedy only
+        elif case == 4:  # whole-row rows only: top_k beyond the fast path
+            p["top_k"] = np.uint32(5000)
+            p["top_p"] = np.float32(0.97)
+            p["temperature"] = np.float32(0.9)
+        _say("host parameter copy case %d" % case)
+        kw = dict(mask=w.get("mask"), hist=w.get("hist"), hist_len=w.get("hist_len"), cand_cap=64)
+        full = api.sample(gpu_ctx, w["logits"], p, w["u"], **kw)
+        lean = api.sample(gpu_ctx, w["logits"], p, w["u"], params_host=True, **kw)
+        for key in ("tokens", "n_cand", "path", "cand_idx"):
+            assert np.array_equal(full[key], lean[key]), (case, key)
+        assert np.array_equal(full["total"].view(np.uint32), lean["total"].view(np.uint32)), case
+        ref = oracle_rows(w)
+        assert [t for t, _ in ref] == [int(t) for t in lean["tokens"]], case
+
+
 def test_more_rows_than_threads():
     """1100 rows in one batch: the per-workgroup search for its piece of work loops over the rows."""
     ctx = api.SamplerContext(max_rows=1100, max_vocab=320, max_hist=0)
