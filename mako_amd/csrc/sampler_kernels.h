@@ -3494,6 +3494,9 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     __shared__ ArgsLds s_args;
     const uint32_t row = blockIdx.y;
     const uint32_t tid = threadIdx.x;
+#ifdef MAKO_TIMING_PLAN
+    MAKO_WG_TIMER;
+#endif
     MAKO_ROW(row);
     stage_args(d_arg, sc_arg, row, s_args);
     const mako_sample_desc& d = s_args.d;
