@@ -117,7 +117,7 @@ def main():
 
     def step(i):
         batch.desc.logits = pool[i % n_copies].ptr
-        ctx.sample_batch(batch.desc, stream)
+        ctx.sample_batch(batch.desc, stream, params_host=batch.params_host)
 
     if a.calibrate_copy_mb:
         n = a.calibrate_copy_mb << 20

@@ -105,11 +105,6 @@ typedef struct mako_sample_desc {
      * hist_len[r] < hist_stride (else the history is left as it is).  hist_tokens and hist_len must then be
      * writable device memory, hist_counts null, and draft null (the rows of a verify batch share one history). */
     uint32_t append_history;
-    /* Optional HOST copy of `params` (the SamplingParams originate on the host, src/gen/session.hpp:19-21).  When
-     * given, the call looks at it on the calling thread and leaves out the kernels that no row of the batch
-     * needs (a batch without top_k == 0 rows takes two launches instead of six).  It must hold the same values as
-     * the device array; the results never depend on whether it is given. */
-    const mako_sampling_params* params_host;
 } mako_sample_desc;
 
 typedef struct mako_sampler_ctx mako_sampler_ctx;
@@ -126,6 +121,13 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx);
  * stream) and returns without waiting: Sampler::sample / Sampler::verify
  * (src/gen/sampler.cpp:75-107) for every row.  One batch at a time per context. */
 int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* desc, void* stream);
+
+/* The same call for a caller that still has the batch's parameters in HOST memory (the SamplingParams originate
+ * there, src/gen/session.hpp:19-21): params_host[n_rows] must hold the same values as desc->params.  The call
+ * looks at them on the calling thread and leaves out the kernels that no row of the batch needs (a batch without
+ * top_k == 0 rows takes two launches instead of six).  The results never depend on it; null = the call above. */
+int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_desc* desc,
+                                     const mako_sampling_params* params_host, void* stream);
 
 /* Host-pointer convenience call with the reference's calling convention
  * (host logits, src/gen/session.cpp:443): copies the rows to the device,

@@ -78,7 +78,6 @@ class Desc(C.Structure):
         ("out_forced", C.c_void_p),
         ("out_above", C.c_void_p),
         ("append_history", C.c_uint32),
-        ("params_host", C.c_void_p),
     ]
 
 
@@ -86,6 +85,7 @@ EXPORTS = [
     "mako_sampler_create",
     "mako_sampler_destroy",
     "mako_sampler_sample_batch",
+    "mako_sampler_sample_batch_hinted",
     "mako_sampler_sample_host",
     "mako_sampler_last_error",
     "mako_sampler_slices",
@@ -107,6 +107,7 @@ def load():
         lib.mako_sampler_create.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_uint32, C.c_uint32, C.c_uint32]
         lib.mako_sampler_destroy.argtypes = [C.c_void_p]
         lib.mako_sampler_sample_batch.argtypes = [C.c_void_p, C.POINTER(Desc), C.c_void_p]
+        lib.mako_sampler_sample_batch_hinted.argtypes = [C.c_void_p, C.POINTER(Desc), C.c_void_p, C.c_void_p]
         lib.mako_sampler_last_error.restype = C.c_char_p
         lib.mako_sampler_last_error.argtypes = [C.c_void_p]
         lib.mako_sampler_set_profile.argtypes = [C.c_void_p, C.c_int]
@@ -167,8 +168,14 @@ class SamplerContext:
             raise MakoError("mako_sampler_kernel_times: %d %s" % (rc, self.last_error()))
         return [float(x) for x in out]
 
-    def sample_batch(self, desc, stream=None):
-        rc = self.lib.mako_sampler_sample_batch(self.ptr, C.byref(desc), stream.ptr if stream else None)
+    def sample_batch(self, desc, stream=None, params_host=None):
+        """Enqueues one batch.  params_host: address of a host copy of the rows' parameters (Batch.params_host),
+        with which the library leaves out the kernels no row needs."""
+        if params_host:
+            rc = self.lib.mako_sampler_sample_batch_hinted(self.ptr, C.byref(desc), params_host,
+                                                           stream.ptr if stream else None)
+        else:
+            rc = self.lib.mako_sampler_sample_batch(self.ptr, C.byref(desc), stream.ptr if stream else None)
         if rc != MAKO_OK:
             raise MakoError("mako_sampler_sample_batch: %d %s" % (rc, self.last_error()))
 
@@ -189,8 +196,8 @@ class Batch:
         d.n_rows, d.n_vocab = b, self.n_vocab
         self.h_params = np.ascontiguousarray(params, PARAMS_DTYPE)
         d.params = self._up(self.h_params).ptr
-        if params_host:  # the host copy, for the library to leave out kernels that have no work
-            d.params_host = self.h_params.ctypes.data
+        # the host copy's address, for the library to leave out kernels that have no work (None: not offered)
+        self.params_host = self.h_params.ctypes.data if params_host else None
         self.d_u = self._up(np.ascontiguousarray(u, np.float32))
         d.u = self.d_u.ptr
         if mask is not None:
@@ -276,5 +283,5 @@ class Batch:
 def sample(ctx, logits, params, u, **kw):
     """One batch through the device path from host arrays; returns a dict of host arrays."""
     b = Batch(logits, params, u, **kw)
-    ctx.sample_batch(b.desc)
+    ctx.sample_batch(b.desc, params_host=b.params_host)
     return b.results()

@@ -4,7 +4,12 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SRC = os.path.join(HERE, "csrc", "mako_sampler.hip")
+CSRC = os.path.join(HERE, "csrc")
+# the C ABI, and one translation unit per kernel family (a kernel's register allocation then does not depend on
+# which other kernels exist; they also compile side by side)
+SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_for_sort.hip",
+           "k_plan_alone.hip", "k_sort.hip", "k_tail.hip"]
+OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 OUT = os.path.join(HERE, "libmako_sampler.so")
 
 # Bit-exactness against the host toolchain needs: no FMA contraction, IEEE fp32
@@ -14,7 +19,6 @@ FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     "-ffp-contract=off",
     "-fhip-fp32-correctly-rounded-divide-sqrt",
     "-fno-gpu-flush-denormals-to-zero",
@@ -28,8 +32,21 @@ FLAGS = [
 ]
 
 
-def build(verbose=False, extra=()):
-    cmd = ["hipcc", *FLAGS, *extra, SRC, "-o", OUT]
+def build(verbose=False, extra=(), jobs=8):
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(OBJ_DIR, exist_ok=True)
+
+    def compile_one(name):
+        obj = os.path.join(OBJ_DIR, os.path.splitext(name)[0] + ".o")
+        cmd = ["hipcc", *FLAGS, *extra, "-c", os.path.join(CSRC, name), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", OUT]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)

@@ -1,0 +1,23 @@
+// partition_kernel and sort_kernel: the wide rows' weights handed to their workers and sorted; narrow and
+// whole-row rows finished by one worker.
+#define MAKO_EMIT_SORT_KERNELS
+#include "launch.h"
+#include "sampler_kernels.h"
+
+namespace mako {
+void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch* sc)
+{
+    hipLaunchKernelGGL(partition_kernel, dim3(kWorkers, d.n_rows), dim3(kThreads), 0, st, d, sc);
+}
+
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices)
+{
+    hipLaunchKernelGGL(sort_kernel, dim3(kWorkers, d.n_rows), dim3(kThreads), kSortLds, st, d, sc, slices);
+}
+
+hipError_t init_sort_kernels()
+{
+    static_assert(kSortLds >= kDynLds, "sort_kernel's tail uses the finishing kernels' LDS layout");
+    return hipFuncSetAttribute((const void*)sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSortLds);
+}
+} // namespace mako

@@ -1,0 +1,16 @@
+// tail_kernel: top-p cut, exact total and draw of the wide rows.
+#define MAKO_EMIT_TAIL_KERNEL
+#include "launch.h"
+#include "sampler_kernels.h"
+
+namespace mako {
+void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch* sc)
+{
+    hipLaunchKernelGGL(tail_kernel, dim3(1, d.n_rows), dim3(kThreads), kDynLds, st, d, sc);
+}
+
+hipError_t init_tail_kernels()
+{
+    return hipFuncSetAttribute((const void*)tail_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLds);
+}
+} // namespace mako

@@ -1,0 +1,34 @@
+// Launchers of the sampler's kernels.  Every kernel family is compiled as a translation unit of its own (k_*.hip):
+// the compiler's register allocation for a kernel otherwise depends on which other kernels share its inlined device
+// functions (sort_kernel lost 2.4 us per batch to spills when plan_kernel variants with the whole-row path were
+// compiled beside it).  Each init function raises the dynamic LDS limit of its family's kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mako_sampler.h"
+
+namespace mako {
+struct Scratch;
+
+hipError_t init_scan_kernels();
+hipError_t init_finish_kernels();
+hipError_t init_plan_for_sort();
+hipError_t init_plan_alone();
+hipError_t init_sort_kernels();
+hipError_t init_tail_kernels();
+
+// scan_kernel<vec, kh, above>, grid = (slices, rows), `lds` bytes of dynamic LDS
+void launch_scan(bool vec, int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d,
+                 const Scratch* sc, uint32_t slice_len, uint32_t cus);
+// finish_kernel<vec, kh> on `wgs` workgroups
+void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch* sc,
+                   uint32_t slices);
+// plan_kernel, one workgroup per row: <false> when sort_kernel follows (it has the whole-row path), <true> when
+// plan_kernel is the last kernel of the batch
+void launch_plan_for_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
+void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
+void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch* sc);
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
+void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch* sc);
+} // namespace mako

@@ -1,4 +1,5 @@
-// C ABI of include/mako_sampler.h over the kernels in sampler_kernels.h.
+// C ABI of include/mako_sampler.h over the kernels in sampler_kernels.h (launched through launch.h: every kernel
+// family is a translation unit of its own).
 #include <hip/hip_runtime.h>
 
 #include <stdint.h>
@@ -9,7 +10,24 @@
 #include <string>
 
 #include "../../include/mako_sampler.h"
+#include "launch.h"
 #include "sampler_kernels.h"
+
+namespace mako {
+__global__ void debug_expf_kernel(const float* x, float* y, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        y[i] = expf_glibc(x[i], k_exp2_tab);
+}
+
+__global__ void debug_div_kernel(const float* a, const float* b, float* y, uint32_t n)
+{
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        y[i] = a[i] / b[i];
+}
+} // namespace mako
 
 // ---------------------------------------------------------------------------------------------
 // C ABI
@@ -135,23 +153,13 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&ctx->sc_dev, 1));
     MAKO_HIP(ctx, hipMemcpy(ctx->sc_dev, &sc, sizeof sc, hipMemcpyHostToDevice));
     MAKO_HIP(ctx, hipDeviceSynchronize());
-    // both kernels overlay up to 64 KB of dynamic LDS on a few KB of static LDS
-    const void* kernels[] = {(const void*)mako::scan_kernel<true, 0>,    (const void*)mako::scan_kernel<false, 0>,
-                             (const void*)mako::scan_kernel<true, 2>,    (const void*)mako::scan_kernel<false, 2>,
-                             (const void*)mako::scan_kernel<true, 8>,    (const void*)mako::scan_kernel<false, 8>,
-                             (const void*)mako::scan_kernel<true, 0, true>, (const void*)mako::scan_kernel<false, 0, true>,
-                             (const void*)mako::scan_kernel<true, 2, true>, (const void*)mako::scan_kernel<false, 2, true>,
-                             (const void*)mako::scan_kernel<true, 8, true>, (const void*)mako::scan_kernel<false, 8, true>,
-                             (const void*)mako::finish_kernel<true, 0>,  (const void*)mako::finish_kernel<false, 0>,
-                             (const void*)mako::finish_kernel<true, 2>,  (const void*)mako::finish_kernel<false, 2>,
-                             (const void*)mako::finish_kernel<true, 8>,  (const void*)mako::finish_kernel<false, 8>,
-                             (const void*)mako::sort_kernel,             (const void*)mako::plan_kernel<false>,
-                             (const void*)mako::plan_kernel<true>,
-                             (const void*)mako::tail_kernel};
-    static_assert(mako::kSortLds >= mako::kDynLds, "sort_kernel's tail uses the finishing kernel's LDS layout");
-    for (const void* k : kernels)
-        MAKO_HIP(ctx, hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          k == (const void*)mako::sort_kernel ? (int)mako::kSortLds : (int)mako::kDynLds));
+    // the kernels overlay up to 64 KB of dynamic LDS (sort_kernel more) on a few KB of static LDS
+    MAKO_HIP(ctx, mako::init_scan_kernels());
+    MAKO_HIP(ctx, mako::init_finish_kernels());
+    MAKO_HIP(ctx, mako::init_plan_for_sort());
+    MAKO_HIP(ctx, mako::init_plan_alone());
+    MAKO_HIP(ctx, mako::init_sort_kernels());
+    MAKO_HIP(ctx, mako::init_tail_kernels());
     return MAKO_OK;
 }
 
@@ -208,6 +216,12 @@ const char* mako_sampler_last_error(const mako_sampler_ctx* ctx)
 
 int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* desc, void* stream)
 {
+    return mako_sampler_sample_batch_hinted(ctx, desc, nullptr, stream);
+}
+
+int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_desc* desc,
+                                     const mako_sampling_params* params_host, void* stream)
+{
     if (!ctx || !desc)
         return MAKO_ERR_INVALID_ARG;
     const mako_sample_desc& d = *desc;
@@ -258,61 +272,36 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
     } while (0)
     // which kernels have work: all of them unless the caller's host copy of the parameters says otherwise
     bool any_nucleus = true, any_general = true;
-    if (d.params_host) {
+    if (params_host) {
         any_nucleus = any_general = false;
         for (uint32_t r = 0; r < d.n_rows; ++r) {
-            const mako::RowClass c = mako::classify(d.params_host[r]);
+            const mako::RowClass c = mako::classify(params_host[r]);
             any_nucleus |= c == mako::kNucleus;
             any_general |= c == mako::kGeneral;
         }
     }
     const bool launch_sort = any_nucleus || any_general;
-#define MAKO_LAUNCH(V, K)                                                                                          \
-    do {                                                                                                           \
-        if (d.close_token)                                                                                         \
-            hipLaunchKernelGGL((mako::scan_kernel<V, K, true>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc_dev,   \
-                               slice_len, ctx->cus);                                                               \
-        else                                                                                                       \
-            hipLaunchKernelGGL((mako::scan_kernel<V, K>), grid, dim3(mako::kThreads), lds, st, d, ctx->sc_dev,        \
-                               slice_len, ctx->cus);                                                               \
-        MAKO_MARK(1);                                                                                              \
-        if (any_nucleus)                                                                                           \
-            hipLaunchKernelGGL((mako::finish_kernel<V, K>), dim3(1, finish_wgs), dim3(mako::kThreads),             \
-                               mako::kDynLds, st, d, ctx->sc_dev, slices);                                         \
-        MAKO_MARK(2);                                                                                              \
-    } while (0)
     MAKO_MARK(0);
-    if (vec && kh == 2)
-        MAKO_LAUNCH(true, 2);
-    else if (vec && kh == 8)
-        MAKO_LAUNCH(true, 8);
-    else if (vec)
-        MAKO_LAUNCH(true, 0);
-    else if (kh == 2)
-        MAKO_LAUNCH(false, 2);
-    else if (kh == 8)
-        MAKO_LAUNCH(false, 8);
-    else
-        MAKO_LAUNCH(false, 0);
-#undef MAKO_LAUNCH
+    mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, ctx->sc_dev, slice_len, ctx->cus);
+    MAKO_MARK(1);
+    if (any_nucleus)
+        mako::launch_finish(vec, kh, finish_wgs, st, d, ctx->sc_dev, slices);
+    MAKO_MARK(2);
     // top_k == 0 rows: plan from the row's histogram, sort by the plan, cut and draw; the stages talk through
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  Other rows cost a load.
     if (launch_sort)
-        hipLaunchKernelGGL(mako::plan_kernel<false>, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev,
-                           slices);
+        mako::launch_plan_for_sort(st, d, ctx->sc_dev, slices);
     else
-        hipLaunchKernelGGL(mako::plan_kernel<true>, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev,
-                           slices);
+        mako::launch_plan_alone(st, d, ctx->sc_dev, slices);
     MAKO_MARK(3);
     if (any_nucleus)
-        hipLaunchKernelGGL(mako::partition_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), 0, st, d, ctx->sc_dev);
+        mako::launch_partition(st, d, ctx->sc_dev);
     MAKO_MARK(4);
     if (launch_sort)
-        hipLaunchKernelGGL(mako::sort_kernel, dim3(mako::kWorkers, d.n_rows), dim3(mako::kThreads), mako::kSortLds, st, d,
-                           ctx->sc_dev, slices);
+        mako::launch_sort(st, d, ctx->sc_dev, slices);
     MAKO_MARK(5);
     if (any_nucleus)
-        hipLaunchKernelGGL(mako::tail_kernel, dim3(1, d.n_rows), dim3(mako::kThreads), mako::kDynLds, st, d, ctx->sc_dev);
+        mako::launch_tail(st, d, ctx->sc_dev);
     MAKO_MARK(6);
 #undef MAKO_MARK
     ctx->profiled = prof;
@@ -405,20 +394,6 @@ int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t
         MAKO_HIP(ctx, hipMemcpy(out_accepted, ctx->st_acc, n_rows, hipMemcpyDeviceToHost));
     return MAKO_OK;
 }
-
-#ifdef MAKO_TIMING
-int mako_sampler_debug_wg(unsigned long long* out8192)
-{
-    return hipMemcpyFromSymbol(out8192, HIP_SYMBOL(mako::g_mako_wg), 8192 * sizeof(unsigned long long)) == hipSuccess
-               ? MAKO_OK : MAKO_ERR_HIP;
-}
-// tuning builds only: copies the stage timestamps of row 0 (100 MHz wall clock) to the host
-int mako_sampler_debug_stamps(unsigned long long* out32)
-{
-    return hipMemcpyFromSymbol(out32, HIP_SYMBOL(mako::g_mako_stamp), 32 * sizeof(unsigned long long)) == hipSuccess
-               ? MAKO_OK : MAKO_ERR_HIP;
-}
-#endif
 
 int mako_sampler_debug_expf(const float* x_dev, float* y_dev, uint32_t n, void* stream)
 {

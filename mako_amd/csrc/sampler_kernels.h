@@ -56,6 +56,19 @@ struct WgTimer {
     }
 };
 #define MAKO_WG_TIMER WgTimer wg_timer_
+} // namespace mako
+// (readers of the above for the tuning scripts; one translation unit at a time is built with MAKO_TIMING)
+extern "C" int mako_sampler_debug_wg(unsigned long long* out8192)
+{
+    return hipMemcpyFromSymbol(out8192, HIP_SYMBOL(mako::g_mako_wg), 8192 * sizeof(unsigned long long)) == hipSuccess
+               ? MAKO_OK : MAKO_ERR_HIP;
+}
+extern "C" int mako_sampler_debug_stamps(unsigned long long* out32)
+{
+    return hipMemcpyFromSymbol(out32, HIP_SYMBOL(mako::g_mako_stamp), 32 * sizeof(unsigned long long)) == hipSuccess
+               ? MAKO_OK : MAKO_ERR_HIP;
+}
+namespace mako {
 #define MAKO_TIC(k)                                                                                                  \
     __builtin_amdgcn_s_waitcnt(0);                                                                                   \
     const unsigned long long tic_##k = wall_clock64()
@@ -1722,10 +1735,11 @@ __device__ __forceinline__ ChainState sum_by_quarters(Keys kf, uint32_t st, uint
 //
 // `T` (with `t_groups` records at `t_base`) describes a list whose groups were prepared by sort_kernel's workers;
 // without it the list is cut into groups of kGroup here.
-template <bool PLANNED = false>
+// SHORT_ONLY: the caller's lists never exceed kGroup entries; the code for longer ones is left out.
+template <bool PLANNED = false, bool SHORT_ONLY = false>
 __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf_ptr,
                             const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
-                            const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, GroupTable T = GroupTable{},
+                            const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, const GroupTable& T = GroupTable{},
                             size_t t_base = 0, uint32_t t_groups = 0)
 {
     using namespace seqfp;
@@ -1841,6 +1855,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         MAKO_STAMP(9);
         return sm.flag != 0;
     }
+    if constexpr (SHORT_ONLY)
+        return false; // (not reached)
 
     // group records: fp64 sums (and, from the workers, the maps of the running sum)
     MAKO_STAMP(5);
@@ -2337,6 +2353,7 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         }
         count_all += y;
     }
+    MAKO_STAMP(20);
     const double incl = pre_m + mass_w;
     const uint32_t above0 = pre_c + cnt_w - (c0 + c1), above1 = above0 + c0;
     // The nucleus ends in the first bin (from the top) at which the running mass reaches `want`.  These sums
@@ -2363,6 +2380,7 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         sm.flag = above1 + c1;
     }
     __syncthreads();
+    MAKO_STAMP(22);
     const uint32_t b_lo = sm.ticket;
     thr_bits = bin_lo_key(b_lo);
     const uint32_t n0 = sm.flag;
@@ -2383,6 +2401,7 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         atomicAdd(&w_cnt[wk1], c1);
     }
     __syncthreads();
+    MAKO_STAMP(23);
     // the mass above a worker's range, known to the thread that holds the range's highest bin
     if (wk0 != kNone && w_hi[wk0] == b0)
         plan->mass[wk0] = incl - m0 - m1;
@@ -2886,6 +2905,9 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
 // Whole-row path: exact for every parameter combination.  One workgroup rebuilds the penalised
 // row in scratch, keeps the candidates, sorts them by (q desc, idx asc) when top-k or top-p is
 // active, truncates, and draws.  src/gen/sampler.cpp:20-62.
+// (SITE: sort_kernel, its usual place, has an instance to itself, so that the compiler treats that kernel the same
+// whether or not the instances inside plan_kernel exist.)
+template <int SITE>
 __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
                             float m, uint32_t argidx, const FinishLds& L)
 {
@@ -3423,6 +3445,66 @@ __device__ __forceinline__ uint32_t row_forced(const mako_sample_desc& d, const 
     return kind;
 }
 
+// Rows other than top_k == 0 rows whose candidate lists cannot serve: top_k > kTopKFast, no truncation at all, a slice
+// that had to drop candidates.  They take the whole-row path.
+__device__ __forceinline__ bool topk_takes_whole_row(RowClass cls, uint32_t any_overflow, uint32_t n_cands)
+{
+    return cls == kGeneral || any_overflow || n_cands > kSortMax;
+}
+
+// A top-k row (top_k <= kTopKFast) from the candidates scan_kernel left: weights of the candidates, the top_k-th
+// weight's neighbourhood ordered by (q desc, idx asc) in LDS, the certificate that nothing left behind in a slice can
+// reach the top_k-th weight, then top-p, total and draw by one wave.  A row that cannot be certified takes the
+// whole-row path: here and now (INLINE_GENERAL), or through sort_kernel's work list.
+template <bool INLINE_GENERAL>
+__device__ __forceinline__ void topk_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slices,
+                                         const mako_sampling_params& P, float m, uint32_t argidx, uint32_t n_cands,
+                                         const SliceStat& lane_stat, const FinishLds& L)
+{
+    constexpr bool inline_general = INLINE_GENERAL;
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    // ---- top-k rows: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
+    const float inv_t = 1.0f / P.temperature;
+    const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
+    const float q_bound = candidate_bound(lane_stat, slices, m, inv_t, floor_q, sm);
+    MAKO_STAMP(3);
+    uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax); // upper half of the dynamic block
+    uint32_t* jf = kf + kSortMax;
+    uint32_t n_valid = 0;
+    uint32_t n_list = kNone;
+    if (!d.draft) // the top_k-th weight's neighbourhood only
+        n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, P.top_k, 0u, kf, jf, n_valid, L);
+    if (n_list == kNone)
+        n_valid = n_cands <= 1024u ? sort_candidates<1>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L)
+                                   : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
+    MAKO_STAMP(4);
+    // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
+    const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
+    if (!ok) {
+        if constexpr (inline_general) {
+            __syncthreads(); // (the lists in LDS are done with)
+            general_row<1>(d, sc, row, P, m, argidx, L);
+            return;
+        } else {
+            if (tid == 0) {
+                sc.plan[row].total64 = (double)m;
+                sc.plan[row].n0 = argidx;
+                sc.plan[row].flag = 2;
+                sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
+            }
+            return;
+        }
+    }
+    if (n_valid == 0) {
+        fallback_row(d, row, argidx);
+        return;
+    }
+    // (sampler.cpp:40-43; at most top_k <= kTopKFast <= kGroup entries)
+    static_assert(kTopKFast <= kGroup, "top-k rows end in sorted_tail's short-list path");
+    sorted_tail<false, true>(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L);
+}
+
 // Second pass over the top_k == 0 rows.  grid = (most pieces a row can have, rows) workgroups, of which workgroup i
 // serves the i-th piece of work in row order, second_pass_pieces() per top_k == 0 row (find_piece): the busy
 // workgroups are then the first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the
@@ -3556,9 +3638,9 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     }
 
     if (cls != kNucleus) {
-        if (cls == kGeneral || any_overflow || n_cands > kSortMax) {
+        if (topk_takes_whole_row(cls, any_overflow, n_cands)) {
             if constexpr (inline_general) {
-                general_row(d, sc, row, P, m, argidx, L);
+                general_row<1>(d, sc, row, P, m, argidx, L);
                 return;
             }
             if (tid == 0) {
@@ -3570,43 +3652,7 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
             return;
         }
 
-        // ---- top-k rows: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
-        const float inv_t = 1.0f / P.temperature;
-        const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
-        const float q_bound = candidate_bound(lane_stat, slices, m, inv_t, floor_q, sm);
-        MAKO_STAMP(3);
-        uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax); // upper half of the dynamic block
-        uint32_t* jf = kf + kSortMax;
-        uint32_t n_valid = 0;
-        uint32_t n_list = kNone;
-        if (!d.draft) // the top_k-th weight's neighbourhood only
-            n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, P.top_k, 0u, kf, jf, n_valid, L);
-        if (n_list == kNone)
-            n_valid = n_cands <= 1024u ? sort_candidates<1>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L)
-                                       : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
-        MAKO_STAMP(4);
-        // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
-        const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
-        if (!ok) {
-            if constexpr (inline_general) {
-                __syncthreads(); // (the lists in LDS are done with)
-                general_row(d, sc, row, P, m, argidx, L);
-                return;
-            }
-            if (tid == 0) {
-                sc.plan[row].total64 = (double)m;
-                sc.plan[row].n0 = argidx;
-                sc.plan[row].flag = 2;
-                sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
-            }
-            return;
-        }
-        if (n_valid == 0) {
-            fallback_row(d, row, argidx);
-            return;
-        }
-        sorted_tail(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L); // sampler.cpp:40-43
-
+        topk_row<inline_general>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L);
         return;
     }
 
@@ -3657,6 +3703,7 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
 }
 
+#ifdef MAKO_EMIT_SORT_KERNELS // (not templates: defined by the one translation unit that launches them)
 // grid = (kWorkers, rows) workgroups over the same work list as sort_kernel; only planned wide rows do anything.
 // Piece c of a row reads the c-th part of the row's bits(q) array once and hands every weight the plan wants to
 // the worker that will sort it: positions inside the workgroup from LDS counters, one global atomic per worker to
@@ -3772,7 +3819,7 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         __syncthreads();
         if (tid == 0)
             plan->flag = 0;
-        general_row(d, sc, row, s_args.P, m, argidx, L);
+        general_row<0>(d, sc, row, s_args.P, m, argidx, L);
         return;
     }
     const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
@@ -3840,8 +3887,12 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         MAKO_STAMP(12);
     }
 }
+#endif // MAKO_EMIT_SORT_KERNELS
 
+#ifdef MAKO_EMIT_TAIL_KERNEL
 // grid = (1, rows).  Rows whose sorted list sort_kernel's workers have prepared: top-p cut, exact total, draw.
+// (The batch's top-k rows were tried here too, beside the few long tails instead of ahead of the planning in
+// plan_kernel: 2.3 us less there, but this kernel's chains then compiled to slower code and lost twice that.)
 __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, const Scratch* sc_dev)
 {
     const Scratch& sc_arg = *sc_dev;
@@ -3850,6 +3901,9 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     __shared__ ArgsLds s_args;
     if (blockIdx.y >= sc_arg.work_n[1])
         return;
+#ifdef MAKO_TIMING_TAIL
+    MAKO_WG_TIMER;
+#endif
     const uint32_t row = sc_arg.work_tail[blockIdx.y], tid = threadIdx.x;
     MAKO_ROW(row);
     if (sc_arg.plan[row].flag != 1)
@@ -3871,20 +3925,6 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     sorted_tail<true>(d, row, s_args.P, sc.key[0] + (size_t)row * sc.vpad, sc.idx[0] + (size_t)row * sc.vpad, n0, true,
                       total64, MAKO_PATH_GENERAL, L, false, 0.0f, sc.gt, (size_t)row * sc.g_cap, groups);
 }
-
-
-__global__ void debug_expf_kernel(const float* x, float* y, uint32_t n)
-{
-    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n)
-        y[i] = expf_glibc(x[i], k_exp2_tab);
-}
-
-__global__ void debug_div_kernel(const float* a, const float* b, float* y, uint32_t n)
-{
-    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n)
-        y[i] = a[i] / b[i];
-}
+#endif // MAKO_EMIT_TAIL_KERNEL
 
 } // namespace mako
