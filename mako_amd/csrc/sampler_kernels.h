@@ -421,6 +421,7 @@ template <int KH>
 struct Extras {
     float v[KH > 0 ? KH : 1];
     uint32_t i[KH > 0 ? KH : 1];
+    bool first_moved; // in the thread that owns element 0 of the slice: that logit now lives in some thread's extra
 };
 
 // The thread's logits after the mask and the penalties (src/gen/sampler.cpp:22-28): wv[16] in the slice
@@ -429,8 +430,10 @@ struct Extras {
 // KH > 0 (histories of at most KH * 1024 entries): thread t handles history entries t, t + 1024, ...  The
 // per-token counts are accumulated in LDS; for every distinct token of the slice the thread holding its first
 // entry computes the penalised logit once (one IEEE division per history entry instead of one per logit
-// slot) and keeps it as an extra, and the logit's owner drops it (NaN).  The election of the first entry
-// makes the arrangement, and with it every later summation order, deterministic.
+// slot) and keeps it as an extra, and the logit's owner drops it (NaN).  The owner hands the masked raw logit over
+// through the token's slot of the LDS table (a gather from device memory instead would return behind every
+// streaming load in flight, and costs the slices that hold most of a Zipf history a microsecond more).  The
+// election of the first entry makes the arrangement, and with it every later summation order, deterministic.
 // KH == 0: any history length; counts in LDS, every owner penalises its own logits.
 struct NoOverlap {
     __device__ __forceinline__ void operator()() const {}
@@ -478,6 +481,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         ex.v[k] = nan;
         ex.i[k] = kNone;
     }
+    ex.first_moved = false;
     if (!pen) {
         finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv);
         return;
@@ -487,27 +491,11 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         finish_slice<VEC>(raw, lo, hi, P, true, s_cnt, wv);
         return;
     }
-    // the masked raw logits of the entries that fall into this slice (asked for now, looked at after the counting)
-    const float* lrow = d.logits + (int64_t)row * d.logits_stride;
-    const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
-    float rawv[KH > 0 ? KH : 1];
-    uint32_t mw[KH > 0 ? KH : 1];
 #pragma unroll
     for (int k = 0; k < KH; ++k) {
         have[k] = have[k] && tok[k] >= lo && tok[k] < hi;
-        rawv[k] = lrow[have[k] ? tok[k] : lo];
-    }
-    if (mrow) {
-#pragma unroll
-        for (int k = 0; k < KH; ++k)
-            mw[k] = mrow[(have[k] ? tok[k] : lo) >> 5];
-    }
-    uint32_t bit[KH > 0 ? KH : 1];
-#pragma unroll
-    for (int k = 0; k < KH; ++k) {
         if (!hc)
             cnt[k] = 1;
-        bit[k] = tok[k] & 31u;
         if (!have[k]) {
             tok[k] = kNone;
             cnt[k] = 1;
@@ -538,37 +526,52 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         if (tok[k] != kNone)
             atomicMin(&s_cnt[tok[k] - lo], tid + (uint32_t)k * kThreads + 1u);
     lds_barrier();
+    bool elected[KH > 0 ? KH : 1];
 #pragma unroll
     for (int k = 0; k < KH; ++k)
-        if (tok[k] != kNone && s_cnt[tok[k] - lo] == tid + (uint32_t)k * kThreads + 1u) {
-            float rv = rawv[k];
-            if (mrow && !((mw[k] >> bit[k]) & 1u))
-                rv = -INFINITY;
-            ex.v[k] = penalize(rv, cnt[k], P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
-            ex.i[k] = tok[k];
-        }
+        elected[k] = tok[k] != kNone && s_cnt[tok[k] - lo] == tid + (uint32_t)k * kThreads + 1u;
+    lds_barrier(); // (the slots are about to be overwritten)
     finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv);
-    // owners drop the logits that now live in an extra
+    // owners: a logit whose slot is taken goes into the slot (its bits) and out of the owner's registers
     if (VEC) {
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k) {
             const uint32_t i = lo + k * 4096u + tid * 4u;
             if (i < hi) {
-                const uint4 n = *reinterpret_cast<const uint4*>(s_cnt + (i - lo));
-                wv[4 * k + 0] = n.x ? nan : wv[4 * k + 0];
-                wv[4 * k + 1] = n.y ? nan : wv[4 * k + 1];
-                wv[4 * k + 2] = n.z ? nan : wv[4 * k + 2];
-                wv[4 * k + 3] = n.w ? nan : wv[4 * k + 3];
+                uint4* slot = reinterpret_cast<uint4*>(s_cnt + (i - lo));
+                const uint4 n = *slot;
+                if (n.x | n.y | n.z | n.w) {
+                    *slot = make_uint4(n.x ? __float_as_uint(wv[4 * k + 0]) : 0u, n.y ? __float_as_uint(wv[4 * k + 1]) : 0u,
+                                       n.z ? __float_as_uint(wv[4 * k + 2]) : 0u, n.w ? __float_as_uint(wv[4 * k + 3]) : 0u);
+                    if (k == 0 && tid == 0)
+                        ex.first_moved = n.x != 0;
+                    wv[4 * k + 0] = n.x ? nan : wv[4 * k + 0];
+                    wv[4 * k + 1] = n.y ? nan : wv[4 * k + 1];
+                    wv[4 * k + 2] = n.z ? nan : wv[4 * k + 2];
+                    wv[4 * k + 3] = n.w ? nan : wv[4 * k + 3];
+                }
             }
         }
     } else {
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j) {
             const uint32_t i = lo + j * (uint32_t)kThreads + tid;
-            if (i < hi && s_cnt[i - lo])
+            if (i < hi && s_cnt[i - lo]) {
+                s_cnt[i - lo] = __float_as_uint(wv[j]);
+                if (j == 0 && tid == 0)
+                    ex.first_moved = true;
                 wv[j] = nan;
+            }
         }
     }
+    lds_barrier();
+#pragma unroll
+    for (int k = 0; k < KH; ++k)
+        if (elected[k]) {
+            const float rv = __uint_as_float(s_cnt[tok[k] - lo]); // (already -inf where the mask clears the token)
+            ex.v[k] = penalize(rv, cnt[k], P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+            ex.i[k] = tok[k];
+        }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -796,7 +799,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
     st.above = above_slice;
     st.pad[0] = st.pad[1] = 0;
     // element 0 of the row is NaN (it may have moved to an extra): only its holder raises the flag
-    bool first_nan = slice == 0 && tid == 0 && wv[0] != wv[0] && !(pen && KH > 0 && s_dyn[0]);
+    bool first_nan = slice == 0 && tid == 0 && wv[0] != wv[0] && !(pen && KH > 0 && ex.first_moved);
 #pragma unroll
     for (int k = 0; k < KH; ++k)
         first_nan = first_nan || (ex.i[k] == 0 && ex.v[k] != ex.v[k]);
