@@ -502,10 +502,12 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         }
     }
     // (barriers that order LDS traffic only: the logits stay in flight)
+    MAKO_STAMP(20);
     uint4* z = reinterpret_cast<uint4*>(s_cnt); // slice_len is a multiple of 4
     for (uint32_t i = tid; i < slice_len / 4; i += kThreads)
         z[i] = make_uint4(0, 0, 0, 0);
     lds_barrier();
+    MAKO_STAMP(21);
 #pragma unroll
     for (int k = 0; k < KH; ++k)
         if (tok[k] != kNone)
@@ -531,7 +533,9 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     for (int k = 0; k < KH; ++k)
         elected[k] = tok[k] != kNone && s_cnt[tok[k] - lo] == tid + (uint32_t)k * kThreads + 1u;
     lds_barrier(); // (the slots are about to be overwritten)
+    MAKO_STAMP(22);
     finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv);
+    MAKO_STAMP(23);
     // owners: a logit whose slot is taken goes into the slot (its bits) and out of the owner's registers
     if (VEC) {
 #pragma unroll
@@ -663,13 +667,15 @@ __device__ bool find_piece(const mako_sample_desc& d, uint32_t piece, uint32_t p
     return false;
 }
 
-// The j-th largest of the wavefront's 64 keys (j >= 1): the largest v with at least j keys >= v, built
-// bit by bit from the top.  One vector compare per bit; the rest is scalar.
+// A lower bound, tight to 2^-9 relative, of the j-th largest of the wavefront's 64 order keys (j >= 1): the largest
+// v with at least j keys >= v, built bit by bit from the top down to bit 14 (the low fourteen bits stay zero: whoever
+// uses the result as a threshold keeps at least j keys, and a handful more at most).  One vector compare per bit;
+// the rest is scalar.
 __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 {
     uint32_t prefix = 0;
 #pragma unroll
-    for (int b = 31; b >= 0; --b) {
+    for (int b = 31; b >= 14; --b) {
         const uint32_t cand = prefix | (1u << b);
         const uint32_t c = (uint32_t)__popcll(__ballot(key >= cand));
         prefix = c >= j ? cand : prefix;
@@ -813,26 +819,43 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
         }
         // w >= tau and w > -inf in one compare: -inf itself is below the most negative finite float
         const float tau = fmaxf(order_unkey(tau_key), -3.402823466e38f);
+        // slots in the slice's list: the wave counts its candidates, one lane reserves the wave's run with a single
+        // LDS atomic, and every thread fills its part of the run (one atomic per candidate cost a round trip each)
+        uint32_t mine = 0;
 #pragma unroll
-        for (uint32_t j = 0; j < 16; ++j) {
-            const float w = wv[j];
-            if (w >= tau) {
-                const uint32_t pos = atomicAdd(&sm.emit_n, 1u);
-                if (pos < kCap) {
-                    sm.cw[pos] = w;
-                    sm.ci[pos] = elem_index<VEC>(lo, tid, j);
-                }
-            }
-        }
+        for (uint32_t j = 0; j < 16; ++j)
+            mine += wv[j] >= tau ? 1u : 0u;
 #pragma unroll
         for (int k = 0; k < KH; ++k)
-            if (ex.v[k] >= tau) {
-                const uint32_t pos = atomicAdd(&sm.emit_n, 1u);
-                if (pos < kCap) {
-                    sm.cw[pos] = ex.v[k];
-                    sm.ci[pos] = ex.i[k];
+            mine += ex.v[k] >= tau ? 1u : 0u;
+        const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
+        const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)upto, kWave - 1);
+        if (wave_total) { // uniform
+            uint32_t base = 0;
+            if (lane_id() == 0)
+                base = atomicAdd(&sm.emit_n, wave_total);
+            uint32_t pos = (uint32_t)__builtin_amdgcn_readfirstlane((int)base) + upto - mine;
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j) {
+                const float w = wv[j];
+                if (w >= tau) {
+                    if (pos < kCap) {
+                        sm.cw[pos] = w;
+                        sm.ci[pos] = elem_index<VEC>(lo, tid, j);
+                    }
+                    ++pos;
                 }
             }
+#pragma unroll
+            for (int k = 0; k < KH; ++k)
+                if (ex.v[k] >= tau) {
+                    if (pos < kCap) {
+                        sm.cw[pos] = ex.v[k];
+                        sm.ci[pos] = ex.i[k];
+                    }
+                    ++pos;
+                }
+        }
     }
     __syncthreads();
     MAKO_STAMP(31);
