@@ -363,10 +363,20 @@ __device__ __forceinline__ uint32_t count_above(const RawSlice<VEC>& r, uint32_t
 // slice hold NaN, which never wins a comparison and never becomes a candidate.
 template <bool VEC>
 __device__ __forceinline__ void finish_slice(const RawSlice<VEC>& r, uint32_t lo, uint32_t hi, const mako_sampling_params& P,
-                                             bool pen, const uint32_t* s_cnt, float (&wv)[16])
+                                             bool pen, const uint32_t* s_cnt, float (&wv)[16], bool masked)
 {
     const uint32_t tid = threadIdx.x;
-    if (VEC) {
+    if (VEC && !masked) { // uniform: no mask, nothing to clear
+        const float nan = __uint_as_float(0x7fc00000u);
+#pragma unroll
+        for (uint32_t k = 0; k < 4; ++k) {
+            const bool inside = lo + k * 4096u + tid * 4u < hi;
+            wv[4 * k + 0] = !inside ? nan : r.v[k].x;
+            wv[4 * k + 1] = !inside ? nan : r.v[k].y;
+            wv[4 * k + 2] = !inside ? nan : r.v[k].z;
+            wv[4 * k + 3] = !inside ? nan : r.v[k].w;
+        }
+    } else if (VEC) {
         const float nan = __uint_as_float(0x7fc00000u);
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k) {
@@ -483,12 +493,12 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     }
     ex.first_moved = false;
     if (!pen) {
-        finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv);
+        finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv, d.mask != nullptr);
         return;
     }
     if (KH == 0) {
         build_counts(d, row, hl, lo, hi, slice_len, s_cnt);
-        finish_slice<VEC>(raw, lo, hi, P, true, s_cnt, wv);
+        finish_slice<VEC>(raw, lo, hi, P, true, s_cnt, wv, d.mask != nullptr);
         return;
     }
 #pragma unroll
@@ -534,7 +544,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         elected[k] = tok[k] != kNone && s_cnt[tok[k] - lo] == tid + (uint32_t)k * kThreads + 1u;
     lds_barrier(); // (the slots are about to be overwritten)
     MAKO_STAMP(22);
-    finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv);
+    finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv, d.mask != nullptr);
     MAKO_STAMP(23);
     // owners: a logit whose slot is taken goes into the slot (its bits) and out of the owner's registers
     if (VEC) {
@@ -838,23 +848,22 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
 #pragma unroll
             for (uint32_t j = 0; j < 16; ++j) {
                 const float w = wv[j];
-                if (w >= tau) {
-                    if (pos < kCap) {
-                        sm.cw[pos] = w;
-                        sm.ci[pos] = elem_index<VEC>(lo, tid, j);
-                    }
-                    ++pos;
+                const bool take = w >= tau;
+                if (take && pos < kCap) {
+                    sm.cw[pos] = w;
+                    sm.ci[pos] = elem_index<VEC>(lo, tid, j);
                 }
+                pos += take ? 1u : 0u;
             }
 #pragma unroll
-            for (int k = 0; k < KH; ++k)
-                if (ex.v[k] >= tau) {
-                    if (pos < kCap) {
-                        sm.cw[pos] = ex.v[k];
-                        sm.ci[pos] = ex.i[k];
-                    }
-                    ++pos;
+            for (int k = 0; k < KH; ++k) {
+                const bool take = ex.v[k] >= tau;
+                if (take && pos < kCap) {
+                    sm.cw[pos] = ex.v[k];
+                    sm.ci[pos] = ex.i[k];
                 }
+                pos += take ? 1u : 0u;
+            }
         }
     }
     __syncthreads();
