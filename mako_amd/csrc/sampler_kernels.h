@@ -3110,6 +3110,45 @@ __device__ __forceinline__ void candidate_keys(const Scratch& sc, uint32_t row, 
     }
 }
 
+// The same keys from the candidate lists read as SLOTS: thread tid takes entries (tid % 128) + 128 t, t < 4, of slice
+// tid / 128, whether or not the slice emitted that many.  Where the lists end is not needed to ask for them, so the
+// loads go out together with the loads of the slices' records instead of one trip to memory behind them; and
+// since every slice's list starts at t = 0, the trips past the longest list are skipped by whole waves.
+// For rows of at most eight slices.
+constexpr int kPrefetchItems = 4;
+struct CandSlots {
+    float w[kPrefetchItems];
+    uint32_t id[kPrefetchItems];
+};
+__device__ __forceinline__ bool slots_cover(uint32_t slices) { return slices <= 8u; }
+__device__ __forceinline__ void fetch_candidate_slots(const Scratch& sc, uint32_t row, uint32_t slices, CandSlots& c)
+{
+    static_assert(kCap == (uint32_t)kPrefetchItems * 128u && kThreads == 1024, "eight slices of 128 threads, four entries each");
+    const uint32_t sl = min(threadIdx.x >> 7, slices - 1u), i0 = threadIdx.x & 127u;
+    const size_t base = ((size_t)row * sc.slices_cap + sl) * kCap + i0;
+#pragma unroll
+    for (uint32_t t = 0; t < (uint32_t)kPrefetchItems; ++t) {
+        c.w[t] = sc.cand_w[base + 128u * t];
+        c.id[t] = sc.cand_i[base + 128u * t];
+    }
+}
+// (sm.soff as candidate_bound() leaves it)
+__device__ __forceinline__ void keys_from_slots(const CandSlots& c, uint32_t slices, float m, float inv_t, float floor_q,
+                                                const FinishShared& sm, unsigned long long (&key)[kPrefetchItems])
+{
+    const uint32_t sl = min(threadIdx.x >> 7, slices - 1u), i0 = threadIdx.x & 127u;
+    const uint32_t emitted = (threadIdx.x >> 7) < slices ? sm.soff[sl + 1] - sm.soff[sl] : 0u;
+#pragma unroll
+    for (uint32_t t = 0; t < (uint32_t)kPrefetchItems; ++t) {
+        key[t] = 0;
+        if (i0 + 128u * t < emitted) {
+            const float q = weight_of(c.w[t], m, inv_t, sm.tab);
+            if (q >= floor_q && q > 0.0f)
+                key[t] = ((unsigned long long)__float_as_uint(q) << 32) | (unsigned long long)(kNone - c.id[t]);
+        }
+    }
+}
+
 // The row's candidates (all slices) weighted, sorted by (q desc, idx asc) and left in LDS as kf[i] = ~bits(q_i),
 // jf[i] = token id, invalid ones (q not a candidate) last.  Returns the number of valid candidates.
 template <int ITEMS>
@@ -3141,9 +3180,11 @@ constexpr uint32_t kSmall = 256; // lists of up to this many entries are ordered
 //   top_k == 0: the threshold is thr_bits, below which the nucleus cannot reach (from the row's histogram).
 // Returns the number of entries in the list, or kNone when they exceed kSmall (nothing is written then);
 // n_valid receives the number of candidates that have a weight at all.
+// `pre` (when have_pre): the row's candidate slots as fetch_candidate_slots() loaded them.
 __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_cands, float m, float inv_t,
                                      float floor_q, uint32_t top_k, uint32_t thr_bits, uint32_t* kf, uint32_t* jf,
-                                     uint32_t& n_valid, const FinishLds& L)
+                                     uint32_t& n_valid, const FinishLds& L, bool have_pre = false,
+                                     const CandSlots& pre = CandSlots{})
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
@@ -3159,7 +3200,11 @@ __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t s
     if (tid == 0)
         *counter = 0;
     unsigned long long key[4];
-    candidate_keys<4>(sc, row, slices, n_cands, m, inv_t, floor_q, sm, key);
+    static_assert(kPrefetchItems == 4, "one key array for both routes");
+    if (have_pre) // uniform
+        keys_from_slots(pre, slices, m, inv_t, floor_q, sm, key);
+    else
+        candidate_keys<4>(sc, row, slices, n_cands, m, inv_t, floor_q, sm, key);
     MAKO_STAMP(17);
     lds_barrier();
     uint32_t n_list;
@@ -3494,7 +3539,8 @@ __device__ __forceinline__ bool topk_takes_whole_row(RowClass cls, uint32_t any_
 template <bool INLINE_GENERAL>
 __device__ __forceinline__ void topk_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slices,
                                          const mako_sampling_params& P, float m, uint32_t argidx, uint32_t n_cands,
-                                         const SliceStat& lane_stat, const FinishLds& L)
+                                         const SliceStat& lane_stat, const FinishLds& L, bool have_pre = false,
+                                         const CandSlots& pre = CandSlots{})
 {
     constexpr bool inline_general = INLINE_GENERAL;
     FinishShared& sm = *L.sm;
@@ -3509,7 +3555,7 @@ __device__ __forceinline__ void topk_row(const mako_sample_desc& d, const Scratc
     uint32_t n_valid = 0;
     uint32_t n_list = kNone;
     if (!d.draft) // the top_k-th weight's neighbourhood only
-        n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, P.top_k, 0u, kf, jf, n_valid, L);
+        n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, P.top_k, 0u, kf, jf, n_valid, L, have_pre, pre);
     if (n_list == kNone)
         n_valid = n_cands <= 1024u ? sort_candidates<1>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L)
                                    : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
@@ -3652,6 +3698,11 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     if (tid < 32)
         sm.tab[tid] = k_exp2_tab[tid];
     __syncthreads();
+    // a top-k row's candidates are asked for together with the slices' records
+    CandSlots pre;
+    const bool prefetched = cls == kTopK && !d.draft && slots_cover(slices); // uniform
+    if (prefetched)
+        fetch_candidate_slots(sc, row, slices, pre);
     float m;
     uint32_t argidx, n_cands, any_overflow;
     SliceStat lane_stat;
@@ -3687,7 +3738,7 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
             return;
         }
 
-        topk_row<inline_general>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L);
+        topk_row<inline_general>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
         return;
     }
 
