@@ -425,25 +425,15 @@ __device__ __forceinline__ void finish_slice(const RawSlice<VEC>& r, uint32_t lo
     }
 }
 
-// Logits that moved out of their owner's registers: the thread that handles history entry h keeps the
-// penalised logit of that token (if it is the token's first entry) as an extra element of its own.
-template <int KH>
-struct Extras {
-    float v[KH > 0 ? KH : 1];
-    uint32_t i[KH > 0 ? KH : 1];
-    bool first_moved; // in the thread that owns element 0 of the slice: that logit now lives in some thread's extra
-};
-
-// The thread's logits after the mask and the penalties (src/gen/sampler.cpp:22-28): wv[16] in the slice
-// layout plus up to KH extras.
+// The thread's logits after the mask and the penalties (src/gen/sampler.cpp:22-28): wv[16] in the slice layout.
 //
 // KH > 0 (histories of at most KH * 1024 entries): thread t handles history entries t, t + 1024, ...  The
 // per-token counts are accumulated in LDS; for every distinct token of the slice the thread holding its first
-// entry computes the penalised logit once (one IEEE division per history entry instead of one per logit
-// slot) and keeps it as an extra, and the logit's owner drops it (NaN).  The owner hands the masked raw logit over
-// through the token's slot of the LDS table (a gather from device memory instead would return behind every
-// streaming load in flight, and costs the slices that hold most of a Zipf history a microsecond more).  The
-// election of the first entry makes the arrangement, and with it every later summation order, deterministic.
+// entry (an election, so that each token is handled once) computes the penalised logit: one IEEE division per
+// history entry instead of one per logit slot.  The logit travels through the token's slot of the LDS table:
+// its owner puts the masked raw value there, the elected thread replaces it by the penalised one, the owner
+// takes it back.  (A gather from device memory instead would return behind every streaming load in flight, and
+// costs the slices that hold most of a Zipf history a microsecond more.)
 // KH == 0: any history length; counts in LDS, every owner penalises its own logits.
 struct NoOverlap {
     __device__ __forceinline__ void operator()() const {}
@@ -454,11 +444,10 @@ struct NoOverlap {
 template <bool VEC, int KH, typename Overlap = NoOverlap>
 __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi,
                                                uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, bool pen,
-                                               uint32_t* s_cnt, float (&wv)[16], Extras<KH>& ex, Overlap overlap = Overlap(),
+                                               uint32_t* s_cnt, float (&wv)[16], Overlap overlap = Overlap(),
                                                bool want_above = false, float close_v = 0.0f, uint32_t* above = nullptr)
 {
     const uint32_t tid = threadIdx.x;
-    const float nan = __uint_as_float(0x7fc00000u);
     // My history entries go first: loads return in the order they were issued, so whatever waits for these does not
     // wait for the logits behind them, and the counting in LDS below runs while the logits are still on their way.
     // (Loads from clamped positions, issued without branches between them; what was not wanted is dropped
@@ -486,12 +475,6 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     overlap();
     if (want_above) // uniform
         *above = count_above<VEC>(raw, lo, hi, close_v);
-#pragma unroll
-    for (int k = 0; k < (KH > 0 ? KH : 1); ++k) {
-        ex.v[k] = nan;
-        ex.i[k] = kNone;
-    }
-    ex.first_moved = false;
     if (!pen) {
         finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv, d.mask != nullptr);
         return;
@@ -546,7 +529,8 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     MAKO_STAMP(22);
     finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv, d.mask != nullptr);
     MAKO_STAMP(23);
-    // owners: a logit whose slot is taken goes into the slot (its bits) and out of the owner's registers
+    // owners: a logit whose slot is taken goes into the slot (its bits); `moved` remembers which of the sixteen
+    uint32_t moved = 0;
     if (VEC) {
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k) {
@@ -557,12 +541,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
                 if (n.x | n.y | n.z | n.w) {
                     *slot = make_uint4(n.x ? __float_as_uint(wv[4 * k + 0]) : 0u, n.y ? __float_as_uint(wv[4 * k + 1]) : 0u,
                                        n.z ? __float_as_uint(wv[4 * k + 2]) : 0u, n.w ? __float_as_uint(wv[4 * k + 3]) : 0u);
-                    if (k == 0 && tid == 0)
-                        ex.first_moved = n.x != 0;
-                    wv[4 * k + 0] = n.x ? nan : wv[4 * k + 0];
-                    wv[4 * k + 1] = n.y ? nan : wv[4 * k + 1];
-                    wv[4 * k + 2] = n.z ? nan : wv[4 * k + 2];
-                    wv[4 * k + 3] = n.w ? nan : wv[4 * k + 3];
+                    moved |= ((n.x ? 1u : 0u) | (n.y ? 2u : 0u) | (n.z ? 4u : 0u) | (n.w ? 8u : 0u)) << (4u * k);
                 }
             }
         }
@@ -572,9 +551,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
             const uint32_t i = lo + j * (uint32_t)kThreads + tid;
             if (i < hi && s_cnt[i - lo]) {
                 s_cnt[i - lo] = __float_as_uint(wv[j]);
-                if (j == 0 && tid == 0)
-                    ex.first_moved = true;
-                wv[j] = nan;
+                moved |= 1u << j;
             }
         }
     }
@@ -583,9 +560,28 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     for (int k = 0; k < KH; ++k)
         if (elected[k]) {
             const float rv = __uint_as_float(s_cnt[tok[k] - lo]); // (already -inf where the mask clears the token)
-            ex.v[k] = penalize(rv, cnt[k], P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
-            ex.i[k] = tok[k];
+            s_cnt[tok[k] - lo] =
+                __float_as_uint(penalize(rv, cnt[k], P.repetition_penalty, P.presence_penalty, P.frequency_penalty));
         }
+    lds_barrier();
+    if (moved) {
+        if (VEC) {
+#pragma unroll
+            for (uint32_t k = 0; k < 4; ++k)
+                if ((moved >> (4u * k)) & 0xfu) {
+                    const uint4 v = *reinterpret_cast<const uint4*>(s_cnt + (lo + k * 4096u + tid * 4u - lo));
+                    wv[4 * k + 0] = (moved >> (4u * k)) & 1u ? __uint_as_float(v.x) : wv[4 * k + 0];
+                    wv[4 * k + 1] = (moved >> (4u * k)) & 2u ? __uint_as_float(v.y) : wv[4 * k + 1];
+                    wv[4 * k + 2] = (moved >> (4u * k)) & 4u ? __uint_as_float(v.z) : wv[4 * k + 2];
+                    wv[4 * k + 3] = (moved >> (4u * k)) & 8u ? __uint_as_float(v.w) : wv[4 * k + 3];
+                }
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j)
+                if ((moved >> j) & 1u)
+                    wv[j] = __uint_as_float(s_cnt[j * (uint32_t)kThreads + tid]);
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -746,13 +742,12 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
     }
     uint32_t above = 0;
     float wv[16];
-    Extras<KH> ex;
     if (ABOVE) {
-        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv, ex, NoOverlap(), want_above, close_v, &above);
+        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv, NoOverlap(), want_above, close_v, &above);
         if (want_above) // uniform
             above = __ockl_wfred_add_u32(above);
     } else {
-        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv, ex);
+        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv);
     }
 
     MAKO_STAMP(29);
@@ -761,9 +756,6 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j)
         best = fmaxf(best, wv[j]);
-#pragma unroll
-    for (int k = 0; k < KH; ++k)
-        best = fmaxf(best, ex.v[k]);
     const uint32_t bkey = order_key(best);
     const bool emits = cls == kTopK || cls == kNucleus;
     const uint32_t wmax = __ockl_wfred_max_u32(bkey);
@@ -799,10 +791,6 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
         for (int j = 15; j >= 0; --j)
             if (wv[j] == M)
                 first = elem_index<VEC>(lo, tid, (uint32_t)j);
-#pragma unroll
-        for (int k = 0; k < KH; ++k)
-            if (ex.v[k] == M)
-                first = min(first, ex.i[k]);
         if (first != kNone)
             atomicMin(&sm.argidx, first);
     }
@@ -814,11 +802,8 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
     st.tau_key = 0;
     st.above = above_slice;
     st.pad[0] = st.pad[1] = 0;
-    // element 0 of the row is NaN (it may have moved to an extra): only its holder raises the flag
-    bool first_nan = slice == 0 && tid == 0 && wv[0] != wv[0] && !(pen && KH > 0 && ex.first_moved);
-#pragma unroll
-    for (int k = 0; k < KH; ++k)
-        first_nan = first_nan || (ex.i[k] == 0 && ex.v[k] != ex.v[k]);
+    // element 0 of the row is NaN: its holder raises the flag
+    const bool first_nan = slice == 0 && tid == 0 && wv[0] != wv[0];
     if (first_nan)
         atomicOr(&sm.emit_flags, kFlagFirstNan);
 
@@ -835,9 +820,6 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j)
             mine += wv[j] >= tau ? 1u : 0u;
-#pragma unroll
-        for (int k = 0; k < KH; ++k)
-            mine += ex.v[k] >= tau ? 1u : 0u;
         const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
         const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)upto, kWave - 1);
         if (wave_total) { // uniform
@@ -852,15 +834,6 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
                 if (take && pos < kCap) {
                     sm.cw[pos] = w;
                     sm.ci[pos] = elem_index<VEC>(lo, tid, j);
-                }
-                pos += take ? 1u : 0u;
-            }
-#pragma unroll
-            for (int k = 0; k < KH; ++k) {
-                const bool take = ex.v[k] >= tau;
-                if (take && pos < kCap) {
-                    sm.cw[pos] = ex.v[k];
-                    sm.ci[pos] = ex.i[k];
                 }
                 pos += take ? 1u : 0u;
             }
@@ -3313,14 +3286,13 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
     constexpr bool pen = PEN;
     float wv[16];
-    Extras<KH> ex;
-    load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, ex);
+    load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv);
     MAKO_STAMP(24);
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
     double sum = 0;
     uint32_t n = 0;
-    uint32_t qb[16], qe[KH > 0 ? KH : 1]; // bits(q), 0 where q is not a candidate
+    uint32_t qb[16]; // bits(q), 0 where q is not a candidate
     // (a piece may be shorter than the sixteen logits per thread: whole blocks past its end are skipped; the test is
     // the same for every thread)
 #pragma unroll
@@ -3333,15 +3305,6 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
                 sum += (double)q;
                 ++n;
             }
-        }
-    }
-#pragma unroll
-    for (int k = 0; k < (PEN ? KH : 0); ++k) {
-        const float q = weight_of(ex.v[k], m, inv_t, sm.tab);
-        qe[k] = (q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
-        if (qe[k]) {
-            sum += (double)q;
-            ++n;
         }
     }
     MAKO_STAMP(25);
@@ -3386,14 +3349,6 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
                 qk[i] = qb[j];
         }
     }
-    __syncthreads(); // the owners' stores land before the holders of moved logits overwrite theirs
-#pragma unroll
-    for (int k = 0; k < (PEN ? KH : 0); ++k)
-        if (ex.i[k] != kNone) {
-            qk[ex.i[k]] = qe[k];
-            if (qe[k])
-                atomicAdd(&hist[weight_bin(qe[k])], record(qe[k]));
-        }
     lds_barrier(); // (the histogram is complete; nobody waits for the stores above)
     MAKO_STAMP(27);
     // the slice's non-empty bins are added to the row's histogram (a few hundred atomics per slice, none waited for)
