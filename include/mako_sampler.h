@@ -69,7 +69,8 @@ typedef struct mako_sample_desc {
     const int32_t* hist_tokens; /* optional [n_rows][hist_stride]: the tokens passed to accept(), sampler.cpp:15-18;
                                    ids outside [0, n_vocab) are ignored */
     const uint32_t* hist_counts; /* optional, same shape: if non-null entry j counts hist_counts[j] occurrences
-                                    (pre-aggregated (id, count) pairs, the reference's counts_ map) */
+                                    (pre-aggregated (id, count) pairs, the reference's counts_ map); an entry
+                                    that counts 0 occurrences is ignored, like a token accept() never saw */
     int64_t hist_stride;
     const uint32_t* hist_len;   /* [n_rows] valid entries per row (required when hist_tokens is given) */
     /* speculative verification, sampler.cpp:86-107 (optional: all three or none) */

@@ -486,12 +486,12 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     }
 #pragma unroll
     for (int k = 0; k < KH; ++k) {
-        have[k] = have[k] && tok[k] >= lo && tok[k] < hi;
         if (!hc)
             cnt[k] = 1;
-        if (!have[k]) {
+        // (an entry that counts no occurrence is no entry: the reference's table holds what accept() has seen)
+        if (!(have[k] && tok[k] >= lo && tok[k] < hi && cnt[k] != 0u)) {
             tok[k] = kNone;
-            cnt[k] = 1;
+            cnt[k] = 0;
         }
     }
     // (barriers that order LDS traffic only: the logits stay in flight)
@@ -501,30 +501,21 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         z[i] = make_uint4(0, 0, 0, 0);
     lds_barrier();
     MAKO_STAMP(21);
-#pragma unroll
-    for (int k = 0; k < KH; ++k)
-        if (tok[k] != kNone)
-            atomicAdd(&s_cnt[tok[k] - lo], cnt[k]);
-    lds_barrier();
-#pragma unroll
-    for (int k = 0; k < KH; ++k)
-        if (tok[k] != kNone)
-            cnt[k] = s_cnt[tok[k] - lo]; // occurrences of the token in the whole history
-    lds_barrier();
-#pragma unroll
-    for (int k = 0; k < KH; ++k)
-        if (tok[k] != kNone)
-            s_cnt[tok[k] - lo] = 0xffffffffu;
-    lds_barrier();
-#pragma unroll
-    for (int k = 0; k < KH; ++k)
-        if (tok[k] != kNone)
-            atomicMin(&s_cnt[tok[k] - lo], tid + (uint32_t)k * kThreads + 1u);
-    lds_barrier();
+    // every entry adds its occurrences to its token's slot; the entry that finds the slot empty speaks for the
+    // token from here on (which of a token's entries that is does not matter: it only carries the logit through
+    // penalize() once)
     bool elected[KH > 0 ? KH : 1];
 #pragma unroll
+    for (int k = 0; k < KH; ++k) {
+        elected[k] = false;
+        if (tok[k] != kNone)
+            elected[k] = atomicAdd(&s_cnt[tok[k] - lo], cnt[k]) == 0u;
+    }
+    lds_barrier();
+#pragma unroll
     for (int k = 0; k < KH; ++k)
-        elected[k] = tok[k] != kNone && s_cnt[tok[k] - lo] == tid + (uint32_t)k * kThreads + 1u;
+        if (elected[k])
+            cnt[k] = s_cnt[tok[k] - lo]; // occurrences of the token in the whole history
     lds_barrier(); // (the slots are about to be overwritten)
     MAKO_STAMP(22);
     finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv, d.mask != nullptr);
