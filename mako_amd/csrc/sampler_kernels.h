@@ -452,22 +452,22 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     // wait for the logits behind them, and the counting in LDS below runs while the logits are still on their way.
     // (Loads from clamped positions, issued without branches between them; what was not wanted is dropped
     // afterwards: a branch around each load would make every load wait for the one before.)
-    const bool extras = KH > 0 && pen; // uniform
+    // Whether they are asked for depends on the kernel's arguments alone, not on the row's parameters or its history
+    // length (`hl`, `pen`): a caller may still be waiting for those when these loads and the logits' go out.
+    const bool may_penalise = KH > 0 && d.hist_tokens != nullptr && d.hist_stride > 0; // uniform
     const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
     const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
     uint32_t tok[KH > 0 ? KH : 1], cnt[KH > 0 ? KH : 1];
     bool have[KH > 0 ? KH : 1];
-    if (extras) {
+    if (may_penalise) {
+        const uint32_t last = (uint32_t)d.hist_stride - 1u; // (entries past the row's length are read and dropped)
 #pragma unroll
-        for (int k = 0; k < KH; ++k) {
-            const uint32_t h = tid + (uint32_t)k * kThreads;
-            have[k] = h < hl;
-            tok[k] = (uint32_t)ht[have[k] ? h : 0u]; // hl > 0 here
-        }
+        for (int k = 0; k < KH; ++k)
+            tok[k] = (uint32_t)ht[min(tid + (uint32_t)k * kThreads, last)];
         if (hc) {
 #pragma unroll
             for (int k = 0; k < KH; ++k)
-                cnt[k] = hc[have[k] ? tid + (uint32_t)k * kThreads : 0u];
+                cnt[k] = hc[min(tid + (uint32_t)k * kThreads, last)];
         }
     }
     RawSlice<VEC> raw;
@@ -489,6 +489,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         if (!hc)
             cnt[k] = 1;
         // (an entry that counts no occurrence is no entry: the reference's table holds what accept() has seen)
+        have[k] = tid + (uint32_t)k * kThreads < hl;
         if (!(have[k] && tok[k] >= lo && tok[k] < hi && cnt[k] != 0u)) {
             tok[k] = kNone;
             cnt[k] = 0;
@@ -700,10 +701,12 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, cons
     MAKO_STAMP(28);
     const uint32_t lo = slice * slice_len;
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
+    // (the history's length is asked for whatever the parameters say: its load then leaves together with theirs)
+    const uint32_t hl_row = d.hist_tokens ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
     const mako_sampling_params P = d.params[row];
     const RowClass cls = classify(P);
     // Greedy rows ignore the penalties (src/gen/sampler.cpp:77-78).
-    const uint32_t hl = (d.hist_tokens && cls != kGreedy) ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
+    const uint32_t hl = cls != kGreedy ? hl_row : 0u;
     const bool pen = hl > 0 && !penalties_neutral(P);
     if (tid == 0) {
         sm.argidx = kNone;
@@ -3265,19 +3268,29 @@ __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t s
     return n_list;
 }
 
+__device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uint32_t slices, float& m, uint32_t& argidx,
+                                            uint32_t& n_cands, uint32_t& any_overflow, SliceStat* lane_stat = nullptr);
+
 // Exact fp64 sum of q over one slice, and the number of candidates in it (q > 0 and q >= min_p).
 // The summation order is fixed: each thread adds its logits in index order, then lanes, then waves.
 // (PEN: the row has penalties to apply; a compile-time fact so that each case gets straight-line code of its own.)
+// (`slices`: of scan_kernel, whose records give the row maximum; they are asked for behind the piece's own loads)
 template <bool VEC, int KH, bool PEN>
 __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slice,
-                              uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, float m, const FinishLds& L)
+                              uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, uint32_t slices,
+                              const FinishLds& L)
 {
     FinishShared& sm = *L.sm;
     const uint32_t lo = slice * slice_len;
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
     constexpr bool pen = PEN;
     float wv[16];
-    load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv);
+    float m = 0.0f;
+    load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, [&]() {
+        uint32_t argidx, n_cands, any_overflow;
+        row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
+    });
+    MAKO_STAMP(1);
     MAKO_STAMP(24);
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
@@ -3367,6 +3380,25 @@ struct alignas(16) ArgsLds {
     mako_sampling_params P; // the row's parameters
 };
 
+// The same in two steps for a kernel that learns its row late: the arguments first (no barrier), the row's parameters
+// (already in registers, the same in every lane) afterwards; the caller's next barrier publishes both.
+__device__ __forceinline__ void stage_args_only(const mako_sample_desc& d_arg, const Scratch& sc_arg, ArgsLds& a)
+{
+    const uint32_t* src_d = reinterpret_cast<const uint32_t*>(&d_arg);
+    const uint32_t* src_s = reinterpret_cast<const uint32_t*>(&sc_arg);
+    uint32_t* dst_d = reinterpret_cast<uint32_t*>(&a.d);
+    uint32_t* dst_s = reinterpret_cast<uint32_t*>(&a.sc);
+    for (uint32_t i = threadIdx.x; i < sizeof(mako_sample_desc) / 4; i += kThreads)
+        dst_d[i] = src_d[i];
+    for (uint32_t i = threadIdx.x; i < sizeof(Scratch) / 4; i += kThreads)
+        dst_s[i] = src_s[i];
+}
+__device__ __forceinline__ void stage_params(const mako_sampling_params& P, ArgsLds& a)
+{
+    if (threadIdx.x == 0)
+        a.P = P;
+}
+
 __device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const Scratch& sc_arg, uint32_t row, ArgsLds& a)
 {
     static_assert(sizeof(mako_sample_desc) % 4 == 0 && sizeof(Scratch) % 4 == 0, "word copies");
@@ -3388,7 +3420,7 @@ __device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const 
 // First maximum of the row (std::max_element semantics, NaNs never win unless at index 0) and the totals of the
 // slices' candidate lists, from the records scan_kernel left.
 __device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uint32_t slices, float& m, uint32_t& argidx,
-                                            uint32_t& n_cands, uint32_t& any_overflow, SliceStat* lane_stat = nullptr)
+                                            uint32_t& n_cands, uint32_t& any_overflow, SliceStat* lane_stat)
 {
     // lane s of every wave takes slice s (at most kMaxSlices = 64 of them): one load each, then wave reductions
     const uint32_t s = min((uint32_t)lane_id(), slices - 1u);
@@ -3546,17 +3578,48 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
 #ifdef MAKO_TIMING_FINISH
     MAKO_WG_TIMER;
 #endif
+    // What the workgroup needs before it can ask for its logits is asked for in as few trips to memory as possible
+    // (each costs most of a microsecond here, and the pass starts with nothing else to do): the rows' parameters
+    // for find_piece() and the arguments' copy go out together with the cut, and the row's own parameters are then
+    // taken from the lane that loaded them.
+    const uint32_t wg = blockIdx.y * gridDim.x + blockIdx.x, tid = threadIdx.x;
+    const bool by_lane = d_arg.n_rows <= (uint32_t)kWave; // uniform
+    mako_sampling_params P_lane = mako_sampling_params{};
+    if (by_lane)
+        P_lane = d_arg.params[min((uint32_t)lane_id(), d_arg.n_rows - 1u)];
+    stage_args_only(d_arg, sc_arg, s_args);
     // (pieces per row, their length, workgroups with work: the others leave at once)
     const uint4 cut = *reinterpret_cast<const uint4*>(sc_arg.work_n + 4);
-    if (blockIdx.y * gridDim.x + blockIdx.x >= cut.z)
+    if (wg >= cut.z)
         return;
     const uint32_t pieces = cut.x, piece_len = cut.y;
     uint32_t row, piece;
-    if (!find_piece(d_arg, blockIdx.y * gridDim.x + blockIdx.x, pieces, 0u, row, piece, sm.bs))
-        return;
-    const uint32_t tid = threadIdx.x;
+    if (by_lane) {
+        // find_piece() over the parameters already here: one row per lane, every wave for itself
+        const uint32_t mine = ((uint32_t)lane_id() < d_arg.n_rows && classify(P_lane) == kNucleus) ? pieces : 0u;
+        const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
+        const unsigned long long bal = __ballot(wg >= upto - mine && wg < upto);
+        if (bal == 0ull)
+            return;
+        const int owner = __ffsll((long long)bal) - 1;
+        row = (uint32_t)owner;
+        piece = wg - (uint32_t)__builtin_amdgcn_readlane((int)(upto - mine), owner);
+        mako_sampling_params P_row;
+        uint32_t* dst = reinterpret_cast<uint32_t*>(&P_row);
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(&P_lane);
+#pragma unroll
+        for (uint32_t i = 0; i < sizeof(mako_sampling_params) / 4; ++i)
+            dst[i] = (uint32_t)__builtin_amdgcn_readlane((int)src[i], owner);
+        stage_params(P_row, s_args);
+    } else {
+        if (!find_piece(d_arg, wg, pieces, 0u, row, piece, sm.bs))
+            return;
+        stage_params(d_arg.params[row], s_args);
+    }
     MAKO_ROW(row);
-    stage_args(d_arg, sc_arg, row, s_args);
+    if (tid < 32)
+        sm.tab[tid] = k_exp2_tab[tid];
+    __syncthreads(); // (publishes the arguments, the parameters and the table)
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
     FinishLds L;
@@ -3572,18 +3635,14 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
         if (row_forced(d, sc, row, slices, ftok, above) != MAKO_FORCED_NONE)
             return;
     }
-    if (tid < 32)
-        sm.tab[tid] = k_exp2_tab[tid];
-    __syncthreads();
-    float m;
-    uint32_t argidx, n_cands, any_overflow;
-    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
-    MAKO_STAMP(1);
+    // (the history's length and, inside slice_partial, the history, the logits and the slices' records: one trip)
     const uint32_t hl = d.hist_tokens ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
-    if (hl > 0 && !penalties_neutral(P))
-        slice_partial<VEC, KH, true>(d, sc, row, piece, piece_len, P, hl, m, L);
+    // (a row without history entries takes the penalising variant too when it has penalties: it finds nothing to
+    // penalise, and nothing here waits for the length)
+    if (d.hist_tokens && !penalties_neutral(P))
+        slice_partial<VEC, KH, true>(d, sc, row, piece, piece_len, P, hl, slices, L);
     else
-        slice_partial<VEC, KH, false>(d, sc, row, piece, piece_len, P, hl, m, L);
+        slice_partial<VEC, KH, false>(d, sc, row, piece, piece_len, P, hl, slices, L);
 }
 
 // grid = (1, rows), one workgroup per row.  Rows whose token is forced, greedy rows and top-k rows are finished here
