@@ -24,7 +24,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per batch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
 # for a device-to-device copy of known size (see the traffic summary under profiles/)
-MEASURED_TRAFFIC_BYTES = {"config3": 74.6e6}
+MEASURED_TRAFFIC_BYTES = {"config3": 74.8e6}
 
 
 def make_workload(name):

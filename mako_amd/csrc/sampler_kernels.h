@@ -683,7 +683,7 @@ __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 
 // grid = (slices, rows).
 // (ABOVE: the batch has close tokens, whose logits' ranks are counted on the way; a variant of its own because the
-// count's registers would cost every other batch half its occupancy)
+// count takes sixteen more registers, up to the limit for two workgroups per CU, which no other batch should pay)
 template <bool VEC, int KH, bool ABOVE = false>
 __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, const Scratch* sc_dev, uint32_t slice_len,
                                                         uint32_t cus)
