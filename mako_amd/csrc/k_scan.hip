@@ -5,13 +5,13 @@
 namespace mako {
 namespace {
 template <bool VEC, int KH, bool ABOVE>
-void launch_one(dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slice_len,
+void launch_one(dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slice_len,
                 uint32_t cus)
 {
     hipLaunchKernelGGL((scan_kernel<VEC, KH, ABOVE>), grid, dim3(kThreads), lds, st, d, sc, slice_len, cus);
 }
 template <bool VEC, int KH>
-void launch_kh(bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d, const Scratch* sc,
+void launch_kh(bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d, const Scratch& sc,
                uint32_t slice_len, uint32_t cus)
 {
     if (above)
@@ -20,7 +20,7 @@ void launch_kh(bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sam
         launch_one<VEC, KH, false>(grid, lds, st, d, sc, slice_len, cus);
 }
 template <bool VEC>
-void launch_vec(int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d, const Scratch* sc,
+void launch_vec(int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d, const Scratch& sc,
                 uint32_t slice_len, uint32_t cus)
 {
     if (kh == 2)
@@ -33,7 +33,7 @@ void launch_vec(int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const
 } // namespace
 
 void launch_scan(bool vec, int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d,
-                 const Scratch* sc, uint32_t slice_len, uint32_t cus)
+                 const Scratch& sc, uint32_t slice_len, uint32_t cus)
 {
     if (vec)
         launch_vec<true>(kh, above, grid, lds, st, d, sc, slice_len, cus);

@@ -282,7 +282,7 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
     }
     const bool launch_sort = any_nucleus || any_general;
     MAKO_MARK(0);
-    mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, ctx->sc_dev, slice_len, ctx->cus);
+    mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, ctx->sc, slice_len, ctx->cus);
     MAKO_MARK(1);
     if (any_nucleus)
         mako::launch_finish(vec, kh, finish_wgs, st, d, ctx->sc_dev, slices);

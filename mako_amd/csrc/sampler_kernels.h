@@ -685,10 +685,11 @@ __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 // (ABOVE: the batch has close tokens, whose logits' ranks are counted on the way; a variant of its own because the
 // count takes sixteen more registers, up to the limit for two workgroups per CU, which no other batch should pay)
 template <bool VEC, int KH, bool ABOVE = false>
-__global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, const Scratch* sc_dev, uint32_t slice_len,
+__global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scratch sc_arg, uint32_t slice_len,
                                                         uint32_t cus)
 {
-    const Scratch& sc = *sc_dev;
+    // (scan_kernel takes the context's record by value: its first loads then need no trip to memory for a pointer)
+    const Scratch& sc = sc_arg;
     MAKO_ROW(blockIdx.y);
 #ifdef MAKO_TIMING_SCAN
     MAKO_WG_TIMER;
