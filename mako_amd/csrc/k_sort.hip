@@ -5,7 +5,7 @@
 #include "sampler_kernels.h"
 
 namespace mako {
-void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch* sc)
+void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc)
 {
     hipLaunchKernelGGL(partition_kernel, dim3(kWorkers, d.n_rows), dim3(kThreads), 0, st, d, sc);
 }

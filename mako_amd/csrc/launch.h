@@ -29,7 +29,7 @@ void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sa
 // plan_kernel is the last kernel of the batch
 void launch_plan_for_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
 void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
-void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch* sc);
+void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc); // (host copy, by value)
 void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
 void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch* sc);
 } // namespace mako

@@ -295,7 +295,7 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
         mako::launch_plan_alone(st, d, ctx->sc_dev, slices);
     MAKO_MARK(3);
     if (any_nucleus)
-        mako::launch_partition(st, d, ctx->sc_dev);
+        mako::launch_partition(st, d, ctx->sc);
     MAKO_MARK(4);
     if (launch_sort)
         mako::launch_sort(st, d, ctx->sc_dev, slices);

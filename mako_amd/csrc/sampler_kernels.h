@@ -3801,39 +3801,52 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
 // the worker that will sort it: positions inside the workgroup from LDS counters, one global atomic per worker to
 // reserve the workgroup's run in that worker's share.  (Without this step each of the 32 workers would sweep the
 // whole row to find its own weights.)
-__global__ __launch_bounds__(kThreads) void partition_kernel(mako_sample_desc d, const Scratch* sc_dev)
+__global__ __launch_bounds__(kThreads) void partition_kernel(mako_sample_desc d, Scratch sc_arg)
 {
-    const Scratch& sc = *sc_dev;
+    // (the context's record by value, and loads asked for in groups: a workgroup here lives four microseconds, and
+    // every dependent trip to memory is most of one)
+    const Scratch& sc = sc_arg;
     __shared__ uint32_t s_count[kWorkers], s_base[kWorkers], s_off[kWorkers], s_cnt[kWorkers];
     __shared__ uint32_t s_table[kBins / 4];
     const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
-    if (piece >= sc.work_n[0])
-        return;
+    // first trip: the list's length and this workgroup's entry of it (the list has room for every workgroup of the
+    // grid; what the entry says is looked at only if the length covers it)
+    const uint32_t n_work = sc.work_n[0];
     const uint32_t item = sc.work_sort[piece];
+    if (piece >= n_work)
+        return;
     const uint32_t row = item >> 8, c = item & 255u, tid = threadIdx.x;
     MAKO_ROW(row);
     BigPlan* plan = sc.plan + row;
-    if (plan->flag != 1)
-        return;
     const uint32_t V = d.n_vocab;
     const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
     uint32_t* kstage = sc.key[1] + (size_t)row * sc.vpad;
     uint32_t* istage = sc.idx[1] + (size_t)row * sc.vpad;
     const uint32_t part = (((V + kWorkers - 1u) / kWorkers) + 3u) & ~3u; // entries per piece, a multiple of 4
     const uint32_t lo = min(V, c * part), hi = min(V, lo + part);
-    // the first loads go out before anything else
+    // second trip: the row's flag, the piece's first weights, the bin -> worker table and the workers' ranges
+    const uint32_t flag = plan->flag;
     uint4 x = make_uint4(0, 0, 0, 0);
     {
         const uint32_t i = lo + tid * 4u;
         if (i < hi)
             x = *reinterpret_cast<const uint4*>(qk + i); // (the array is padded to a multiple of 1024 entries past V)
     }
+    uint32_t table_word = 0, off_w = 0, cnt_w = 0;
     if (tid < kBins / 4)
-        s_table[tid] = reinterpret_cast<const uint32_t*>(sc.bin_worker + (size_t)row * kBins)[tid];
+        table_word = reinterpret_cast<const uint32_t*>(sc.bin_worker + (size_t)row * kBins)[tid];
+    if (tid < kWorkers) {
+        off_w = plan->off[tid];
+        cnt_w = plan->cnt[tid];
+    }
+    if (flag != 1)
+        return;
+    if (tid < kBins / 4)
+        s_table[tid] = table_word;
     if (tid < kWorkers) {
         s_count[tid] = 0;
-        s_off[tid] = plan->off[tid];
-        s_cnt[tid] = plan->cnt[tid];
+        s_off[tid] = off_w;
+        s_cnt[tid] = cnt_w;
     }
     __syncthreads();
     const uint8_t* table = reinterpret_cast<const uint8_t*>(s_table);
