@@ -148,7 +148,10 @@ constexpr uint32_t kGroup = 256;      // a sorted list is processed in groups of
 constexpr uint32_t kMaxGroups = 1024; // groups per list
 constexpr uint32_t kSegCap = 6144;    // entries a worker sorts in LDS
 constexpr uint32_t kFine = 2048;      // value buckets of that sort
-constexpr uint32_t kSortLds = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u; // dynamic LDS of sort_kernel
+// dynamic LDS of sort_kernel: the entries, their order, the buckets, and a copy of the sorted weights for the group
+// records
+constexpr uint32_t kSortLds = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u + kSegCap * 4u;
+constexpr uint32_t kSortedCopyAt = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u; // byte offset of that copy
 
 // Work order for a top_k == 0 row whose nucleus is too wide for the per-slice candidate lists: the weights
 // with bits(q) >= key_lo (n0 of them) are split by value into kWorkers contiguous ranges of about equal size.
@@ -2544,7 +2547,7 @@ __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t*
 }
 
 __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, uint32_t* kout, uint32_t* iout,
-                                unsigned long long* dyn, FinishShared& sm);
+                                unsigned long long* dyn, FinishShared& sm, uint32_t* sorted_lds = nullptr);
 
 // Worker's sort, LDS-resident: the weights of the row with key_lo <= bits(q) < key_hi (at most kSegCap of them)
 // are collected from the row's bits(q) array in one sweep, dropped into kFine value buckets (descending), and
@@ -2622,8 +2625,11 @@ __device__ bool lds_sort_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, 
 
 // Second half of the workers' sort: the n entries (bits(q), idx) in LDS at A, all with key_lo <= bits(q) < key_hi,
 // go to kout / iout ordered by (q desc, idx asc).  hist must be zero and sm.flag 0 on entry.
+// sorted_lds (optional, n words of LDS outside the sort's own): receives the sorted ~bits(q) as well, and the
+// function then returns behind a barrier that orders LDS only: the caller goes on from the copy instead of waiting
+// for the stores to kout and reading them back.
 __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, uint32_t* kout, uint32_t* iout,
-                                unsigned long long* dyn, FinishShared& sm)
+                                unsigned long long* dyn, FinishShared& sm, uint32_t* sorted_lds)
 {
     uint2* A = reinterpret_cast<uint2*>(dyn);
     uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
@@ -2679,16 +2685,22 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
             }
             kout[lo + r] = ~me.x;
             iout[lo + r] = me.y;
+            if (sorted_lds)
+                sorted_lds[lo + r] = ~me.x;
         }
     }
-    __syncthreads();
+    if (sorted_lds) // uniform
+        lds_barrier();
+    else
+        __syncthreads();
     return true;
 }
 
 // The worker's share as partition_kernel left it (cnt <= kSegCap entries, bits(q) in ks and token ids in is, any
 // order), sorted into kout / iout.
 __device__ bool lds_sort_staged(const uint32_t* ks, const uint32_t* is, uint32_t key_lo, uint32_t key_hi, uint32_t cnt,
-                                uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm)
+                                uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm,
+                                uint32_t* sorted_lds = nullptr)
 {
     uint2* A = reinterpret_cast<uint2*>(dyn);
     uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
@@ -2713,7 +2725,7 @@ __device__ bool lds_sort_staged(const uint32_t* ks, const uint32_t* is, uint32_t
             A[e] = make_uint2(min(max(k[t], key_lo), key_hi - 1u), id[t]); // (clamped: a bucket index is always valid)
     }
     __syncthreads();
-    return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm);
+    return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm, sorted_lds);
 }
 
 // A share too large for one LDS sort is cut by value into runs that fit: one counting sweep over the share (the
@@ -2853,18 +2865,23 @@ __device__ bool lds_sort_staged_runs(const uint32_t* ks, const uint32_t* is, uin
 
 // Group records of a worker's sorted range (cnt entries from position off of the list kf): fp64 sums, and the
 // maps of the running fp32 sum for the epoch guessed from the mass above the range plus the sums before the group.
+// kf_lds (optional): the worker's cnt sorted weights in LDS (outside L.sortk's first 16 KB), read instead of kf + off.
 __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, size_t t_at, double mass, const GroupTable& T,
-                              const FinishLds& L)
+                              const FinishLds& L, const uint32_t* kf_lds = nullptr)
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
+    const uint32_t* src = kf_lds ? kf_lds : kf + off; // uniform
     double* gs = reinterpret_cast<double*>(L.sortk); // [groups] estimate of the sum before each group
     double* ge = gs + kMaxGroups;                    // [groups] and after it
     const uint32_t groups = (cnt + kGroup - 1u) / kGroup;
-    __syncthreads();
+    if (kf_lds) // uniform: the copy is in place (its writers' barrier), nothing in device memory is waited for
+        lds_barrier();
+    else
+        __syncthreads();
     for (uint32_t g = wave_id(); g < groups; g += kWaves) {
         float q[4];
-        load_span(kf, off + g * kGroup, min(kGroup, cnt - g * kGroup), q);
+        load_span(src, g * kGroup, min(kGroup, cnt - g * kGroup), q);
         const double s = __ockl_wfred_add_f64((((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3]);
         if (lane_id() == 0)
             gs[g] = s;
@@ -2886,7 +2903,7 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
     for (uint32_t g = wave_id(); g < groups; g += kWaves) {
         const uint32_t len = min(kGroup, cnt - g * kGroup);
         float q[4];
-        load_span(kf, off + g * kGroup, len, q);
+        load_span(src, g * kGroup, len, q);
         const double guess = gs[g];
         const int eg = guess > 0 ? exponent_of((float)guess) : 0;
         const seqfp::Step32 st = span_map(q, len, eg);
@@ -3976,8 +3993,11 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         MAKO_STAMP(10);
         MAKO_COUNT(31, threadIdx.x == 0 && cnt > kSegCap ? 1 : 0);
         MAKO_COUNT(21, threadIdx.x == 0 ? cnt : 0);
-        const bool sorted = cnt <= kSegCap
-                                ? lds_sort_staged(key1 + off, idx1 + off, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm)
+        uint32_t* sorted_copy = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(s_dyn64) + kSortedCopyAt);
+        const bool in_lds = cnt <= kSegCap; // uniform
+        const bool sorted = in_lds
+                                ? lds_sort_staged(key1 + off, idx1 + off, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm,
+                                                  sorted_copy)
                                 : lds_sort_staged_runs(key1 + off, idx1 + off, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm);
         if (cnt > kSegCap)
             MAKO_STAMP(18);
@@ -3988,7 +4008,7 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
             sort_segment(key0 + off, idx0 + off, key1 + off, idx1 + off, cnt, L);
         }
         MAKO_STAMP(11);
-        worker_groups(key0, off, cnt, t_row + gbase, plan->mass[w], sc.gt, L);
+        worker_groups(key0, off, cnt, t_row + gbase, plan->mass[w], sc.gt, L, (in_lds && sorted) ? sorted_copy : nullptr);
         MAKO_STAMP(12);
     }
 }
