@@ -3958,6 +3958,11 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         if (tid == 0)
             plan->flag = 0;
         const mako_sampling_params& P = s_args.P;
+        // (the candidate lists are asked for together with the slices' records, as for a top-k row)
+        CandSlots pre;
+        const bool prefetched = slots_cover(slices); // uniform
+        if (prefetched)
+            fetch_candidate_slots(sc, row, slices, pre);
         float m;
         uint32_t argidx, n_cands, any_overflow;
         SliceStat lane_stat;
@@ -3969,7 +3974,8 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         uint32_t* kf = reinterpret_cast<uint32_t*>(L.sortk + kSortMax);
         uint32_t* jf = kf + kSortMax;
         uint32_t n_valid = 0;
-        const uint32_t n_list = small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, 0u, thr_bits, kf, jf, n_valid, L);
+        const uint32_t n_list =
+            small_candidates(sc, row, slices, n_cands, m, inv_t, floor_q, 0u, thr_bits, kf, jf, n_valid, L, prefetched, pre);
         MAKO_STAMP(4);
         if (n_list != kNone && n_list > 0 &&
             sorted_tail(d, row, P, kf, jf, n_list, true, total64, MAKO_PATH_NUCLEUS, L, true, q_bound))
