@@ -2279,6 +2279,164 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 
 __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t* i1, uint32_t n, const FinishLds& L);
 
+// std::ranges::nth_element(cand, cand + nth, desc) of src/gen/sampler.cpp:41 as libstdc++ 11 runs it (introselect,
+// bits/stl_algo.h:1964), leaving the candidates in exactly the arrangement that library leaves: the reference sums
+// and walks the top_k survivors in that order when no top-p follows.  key/idx hold n candidates (~bits(q), token
+// id); `desc` is the order of the 64-bit values key << 32 | idx, all distinct.
+// One round = median of three to the front, then the unguarded Hoare partition of the rest around it.  That
+// partition swaps the t-th entry from the left that belongs right with the t-th entry from the right that belongs
+// left for as long as the former lies before the latter, and cuts behind the entries that belong left: the two
+// position lists come from ballots (wave w owns the w-th sixteenth of the range), the swaps are independent.
+// lsta / lstb: room for n positions each.  The depth limit's heap select and the last insertion sort (at most three
+// entries) are sequential code on one thread.
+__device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32_t nth, uint32_t* lsta, uint32_t* lstb,
+                                FinishShared& sm)
+{
+    typedef unsigned long long u64;
+    const uint32_t tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+    auto get = [&](uint32_t i) { return ((u64)key[i] << 32) | (u64)idx[i]; };
+    auto put = [&](uint32_t i, u64 v) {
+        key[i] = (uint32_t)(v >> 32);
+        idx[i] = (uint32_t)v;
+    };
+    if (n == 0 || nth >= n)
+        return;
+    uint32_t first = 0, last = n;
+    uint32_t depth = 2u * (31u - (uint32_t)__clz((int)n));
+    __syncthreads();
+    while (last - first > 3u) {
+        if (depth == 0) {
+            // __heap_select(first, nth + 1, last) and iter_swap(first, nth): bits/stl_algo.h:1956-1960, stl_heap.h
+            if (tid == 0) {
+                const uint32_t middle = nth + 1u - first, len = last - first;
+                auto sift = [&](uint32_t hole, u64 v) { // __adjust_heap: the hole sinks to a leaf, v rises from there
+                    const uint32_t top = hole;
+                    uint32_t child = hole;
+                    while (child < (middle - 1u) / 2u) {
+                        child = 2u * (child + 1u);
+                        if (get(first + child) < get(first + child - 1u))
+                            --child;
+                        put(first + hole, get(first + child));
+                        hole = child;
+                    }
+                    if ((middle & 1u) == 0 && middle >= 2u && child == (middle - 2u) / 2u) {
+                        child = 2u * (child + 1u);
+                        put(first + hole, get(first + child - 1u));
+                        hole = child - 1u;
+                    }
+                    while (hole > top) {
+                        const uint32_t parent = (hole - 1u) / 2u;
+                        if (!(get(first + parent) < v))
+                            break;
+                        put(first + hole, get(first + parent));
+                        hole = parent;
+                    }
+                    put(first + hole, v);
+                };
+                if (middle >= 2u)
+                    for (uint32_t parent = (middle - 2u) / 2u;; --parent) {
+                        sift(parent, get(first + parent));
+                        if (parent == 0)
+                            break;
+                    }
+                for (uint32_t i = middle; i < len; ++i) {
+                    const u64 v = get(first + i);
+                    if (v < get(first)) {
+                        put(first + i, get(first));
+                        sift(0u, v);
+                    }
+                }
+                const u64 a = get(first), b = get(nth);
+                put(first, b);
+                put(nth, a);
+            }
+            __syncthreads();
+            return;
+        }
+        --depth;
+        if (tid == 0) { // __move_median_to_first(first, first + 1, mid, last - 1)
+            const uint32_t ix = first + 1u, iy = first + (last - first) / 2u, iz = last - 1u;
+            const u64 x = get(ix), y = get(iy), z = get(iz);
+            uint32_t im;
+            if (x < y)
+                im = y < z ? iy : (x < z ? iz : ix);
+            else
+                im = x < z ? ix : (y < z ? iz : iy);
+            const u64 r = get(first), med = get(im);
+            put(first, med);
+            put(im, r);
+        }
+        __syncthreads();
+        const u64 pivot = get(first);
+        const uint32_t lo0 = first + 1u, len = last - lo0;
+        const uint32_t chunk = ((len + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
+        const uint32_t beg = min(last, lo0 + wave * chunk), end = min(last, beg + chunk);
+        // entries of the wave's chunk that belong left of the cut
+        uint32_t mine = 0;
+        for (uint32_t base = beg; base < end; base += kWave) {
+            const uint32_t pos = base + lane;
+            const bool small = pos < end && get(min(pos, last - 1u)) < pivot;
+            mine += (uint32_t)__popcll(__ballot(small));
+        }
+        if (lane == 0)
+            sm.bs.u64[wave] = mine;
+        __syncthreads();
+        uint32_t small_before = 0, smalls = 0;
+        for (int w = 0; w < kWaves; ++w) {
+            const uint32_t x = (uint32_t)sm.bs.u64[w];
+            if (w < (int)wave)
+                small_before += x;
+            smalls += x;
+        }
+        const uint32_t bigs = len - smalls;
+        uint32_t big_before = (beg - lo0) - small_before;
+        // position lists: lsta[t] = the t-th big entry from the left, lstb[t] = the t-th small entry from the left
+        const u64 lower = (1ull << lane) - 1ull;
+        for (uint32_t base = beg; base < end; base += kWave) {
+            const uint32_t pos = base + lane;
+            const bool in = pos < end;
+            const bool small = in && get(min(pos, last - 1u)) < pivot;
+            const u64 bs = __ballot(small), bb = __ballot(in && !small);
+            if (small)
+                lstb[small_before + (uint32_t)__popcll(bs & lower)] = pos;
+            else if (in)
+                lsta[big_before + (uint32_t)__popcll(bb & lower)] = pos;
+            small_before += (uint32_t)__popcll(bs);
+            big_before += (uint32_t)__popcll(bb);
+        }
+        __syncthreads();
+        const uint32_t pairs = min(bigs, smalls);
+        for (uint32_t t = tid; t < pairs; t += kThreads) {
+            const uint32_t a = lsta[t], b = lstb[smalls - 1u - t];
+            if (a < b) {
+                const u64 va = get(a), vb = get(b);
+                put(a, vb);
+                put(b, va);
+            }
+        }
+        __syncthreads();
+        const uint32_t cut = lo0 + smalls;
+        if (cut <= nth)
+            first = cut;
+        else
+            last = cut;
+    }
+    if (tid == 0) // __insertion_sort(first, last)
+        for (uint32_t i = first + 1u; i < last; ++i) {
+            const u64 v = get(i);
+            uint32_t j = i;
+            if (v < get(first)) {
+                for (; j > first; --j)
+                    put(j, get(j - 1u));
+            } else {
+                for (; v < get(j - 1u); --j)
+                    put(j, get(j - 1u));
+            }
+            put(j, v);
+        }
+    __syncthreads();
+}
+
 // Common tail of the whole-row paths.  key[0]/idx[0] of the row hold n0 candidates (~bits(q), token id) in index
 // order.  Sorts them by (q desc, idx asc) when top-k or top-p is active, truncates (src/gen/sampler.cpp:39-61)
 // and draws.  `total64` (when have_total) is the fp64 sum of q over all candidates of the row, of which the list
@@ -2295,6 +2453,15 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
     // order by (q desc, idx asc): stable LSD radix sort of ~bits(q), ascending
     const bool topk_active = P.top_k > 0 && P.top_k < n0;
     const bool topp_active = P.top_p < 1.0f;
+    if (topk_active && !topp_active) {
+        // top-k alone: the survivors stay in the order nth_element leaves them (sampler.cpp:39-43, then :79-83)
+        nth_element_row(key0, idx0, n0, P.top_k, key1, idx1, sm);
+        const uint32_t* kf = key0;
+        const uint32_t* jf = idx0;
+        draw_from_list(
+            d, row, [=](uint32_t i) { return __uint_as_float(~kf[i]); }, [=](uint32_t i) { return jf[i]; }, P.top_k, path, sm);
+        return;
+    }
     if (topk_active || topp_active)
         sort_segment(key0, idx0, key1, idx1, n0, L);
     const uint32_t *ks = key0, *is = idx0;

@@ -128,7 +128,7 @@ class _Oracle:
             maskp = _up(mask)
         return logits, hist, mask, maskp
 
-    def sample(self, logits, params, u, hist=None, mask=None, order_mode=1, cap=0):
+    def sample(self, logits, params, u, hist=None, mask=None, order_mode=0, cap=0):
         """Returns (token, dict trace)."""
         logits, hist, mask, maskp = self._args(logits, hist, mask)
         tr = Trace()
@@ -141,7 +141,7 @@ class _Oracle:
         return t, dict(n_cand=tr.n_cand, total=np.float32(tr.total), q_chosen=np.float32(tr.q_chosen),
                        max_logit=np.float32(tr.max_logit), cand_idx=ci[:n].copy(), cand_q=cq[:n].copy())
 
-    def verify(self, logits, params, draft, u1, u2, hist=None, mask=None, order_mode=1):
+    def verify(self, logits, params, draft, u1, u2, hist=None, mask=None, order_mode=0):
         logits, hist, mask, maskp = self._args(logits, hist, mask)
         acc = C.c_int(0)
         t = self.lib.or_verify(_fp(logits), logits.size, C.byref(params), _ip(hist), hist.size, maskp, draft,

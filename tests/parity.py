@@ -7,7 +7,7 @@ from mako_amd import api
 from oracle import pyoracle
 
 
-def oracle_rows(w, rows=None, cap=0, order_mode=1, draft=None, u2=None):
+def oracle_rows(w, rows=None, cap=0, order_mode=0, draft=None, u2=None):
     o = pyoracle.oracle()
     b = w["logits"].shape[0]
     rows = range(b) if rows is None else rows

@@ -31,12 +31,12 @@ def expected(oracle, logits, seed, mode, prm):
     p = pyoracle.make_params(*prm)
     for i in range(steps):
         if mode == 0:
-            t, _ = oracle.sample(logits[i], p, float(us[k]), hist, order_mode=1)
+            t, _ = oracle.sample(logits[i], p, float(us[k]), hist, order_mode=0)
             acc = False
             k += 0 if p.temperature <= 0 else 1
         else:
             draft = int(np.argmax(logits[i]))
-            t, acc = oracle.verify(logits[i], p, draft, float(us[k]), float(us[k + 1]), hist, order_mode=1)
+            t, acc = oracle.verify(logits[i], p, draft, float(us[k]), float(us[k + 1]), hist, order_mode=0)
             if p.temperature > 0:
                 k += 1 if (acc or t == draft) else 2
         hist.append(t)

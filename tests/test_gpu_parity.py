@@ -100,9 +100,6 @@ def _random_case(rng, v, b):
     p["presence_penalty"] = rng.choice(np.array([0.0, 0.3, -0.5], np.float32), b)
     p["frequency_penalty"] = rng.choice(np.array([0.0, 0.2], np.float32), b)
     p["repetition_penalty"] = rng.choice(np.array([1.0, 1.1, 2.0, 0.5, 0.0], np.float32), b)
-    # the candidate order after top-k alone is the reference library's nth_element order: not compared here
-    both = (p["top_k"] > 0) & ~(p["top_p"] < 1.0)
-    p["top_p"][both] = np.float32(0.97)
     w = dict(name="random_v%d" % v, logits=logits, params=p, u=rng.random(b).astype(np.float32))
     hl = int(rng.choice([0, 1, 17, 600]))
     if hl:
@@ -122,6 +119,80 @@ def test_random_parameters(gpu_ctx, v):
         w = _random_case(rng, v, 24 if v < 100000 else 8)
         _say("random case v=%d it=%d" % (v, it))
         assert_parity(gpu_ctx, w, cap=min(v, 512))
+
+
+@pytest.mark.parametrize("v", [65, 4096, 40000, 129280])
+def test_random_parameters_with_zipf_histories(gpu_ctx, v):
+    """The same random mixes with Zipf(1.1) histories (most of a history in the first slice, few distinct tokens
+    many times over) and, now and then, a NaN logit at a penalised position."""
+    rng = np.random.default_rng(3000 + v)
+    done = 0
+    while done < 4:
+        w = _random_case(rng, v, 24 if v < 100000 else 8)
+        if "hist" not in w:
+            continue
+        b, hl = w["hist"].shape
+        w["hist"] = np.minimum(v - 1, rng.zipf(1.1, (b, hl)) - 1).astype(np.int32)
+        if done % 2:
+            w["logits"][0, int(w["hist"][0, 0])] = np.nan
+        _say("zipf history case v=%d it=%d" % (v, done))
+        assert_parity(gpu_ctx, w, cap=min(v, 512))
+        done += 1
+
+
+def _topk_only_case(rng, v, b, ks):
+    w = _random_case(rng, v, b)
+    p = w["params"]
+    p["temperature"] = rng.choice(np.array([0.3, 0.7, 1.0, 2.5], np.float32), b)
+    p["top_k"] = rng.choice(np.array(ks, np.uint32), b)
+    p["top_p"] = rng.choice(np.array([1.0, 1.5], np.float32), b)
+    return w
+
+
+@pytest.mark.parametrize("v", [4, 5, 8, 65, 1000, 16385, 40000, 129280, 151552])
+def test_topk_alone_keeps_nth_element_order(gpu_ctx, v):
+    """top_k without top-p: the survivors are summed and walked in the order libstdc++'s nth_element leaves
+    (src/gen/sampler.cpp:39-43, 79-83); candidate lists, fp32 totals and tokens equal the oracle's, whose
+    introselect is pinned against std::nth_element itself on the CPU."""
+    rng = np.random.default_rng(4100 + v)
+    ks = [1, 2, 3, 7, 40, 100, 129, 1000, 5000, v // 2, v - 1, v]
+    for it in range(3):
+        w = _topk_only_case(rng, v, 24 if v < 100000 else 6, [k for k in ks if 0 < k])
+        _say("top-k alone v=%d it=%d" % (v, it))
+        assert_parity(gpu_ctx, w, cap=min(v, 512))
+
+
+def test_topk_alone_verify(gpu_ctx):
+    """Sampler::verify over the nth_element order: the draft's weight, and the redraw over the list without it."""
+    rng = np.random.default_rng(4200)
+    v, b = 20000, 32
+    w = _topk_only_case(rng, v, b, [3, 40, 100, 1000])
+    first = oracle_rows(w)
+    draft = np.array([t for t, _ in first], np.int32)
+    draft[::3] = rng.integers(0, v, len(draft[::3]))
+    u2 = rng.random(b).astype(np.float32)
+    g = gpu_rows(gpu_ctx, w, draft=draft, u2=u2)
+    ref = oracle_rows(w, draft=draft, u2=u2)
+    for r, (t, tr) in enumerate(ref):
+        assert g["tokens"][r] == t and bool(g["accepted"][r]) == tr["accepted"], (r, g["tokens"][r], t)
+
+
+def test_topk_alone_depth_limit(gpu_ctx, oracle):
+    """Worst-case orders recorded from libstdc++ (tests/golden: nth_killers) drive introselect to its depth limit:
+    the heap select must leave the library's arrangement too.  The logits keep the recorded weights' order."""
+    import json
+    import os
+    golden = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")))
+    for k in golden["nth_killers"]:
+        q = np.array(k["q"], np.float32)
+        ranks = np.unique(-q, return_inverse=True)[1]  # 0 = heaviest; equal weights keep equal logits
+        logits = (-(ranks.astype(np.float32)) * np.float32(0.002)).reshape(1, -1)
+        p = api.make_params(1, 1.0, top_k=int(k["nth"]))
+        w = dict(name="nth_killer_%d" % k["n"], logits=logits, params=p, u=np.array([0.61], np.float32))
+        before = oracle.heap_selects()
+        _say("depth limit case n=%d nth=%d" % (k["n"], k["nth"]))
+        assert_parity(gpu_ctx, w, cap=int(k["n"]))
+        assert oracle.heap_selects() > before, "the case no longer reaches the depth limit"
 
 
 def test_special_values(gpu_ctx):
