@@ -2287,24 +2287,19 @@ __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t*
 // partition swaps the t-th entry from the left that belongs right with the t-th entry from the right that belongs
 // left for as long as the former lies before the latter, and cuts behind the entries that belong left: the two
 // position lists come from ballots (wave w owns the w-th sixteenth of the range), the swaps are independent.
-// lsta / lstb: room for n positions each.  The depth limit's heap select and the last insertion sort (at most three
-// entries) are sequential code on one thread.
-__device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32_t nth, uint32_t* lsta, uint32_t* lstb,
-                                FinishShared& sm)
+// The depth limit's heap select and the last insertion sort (at most three entries) are sequential code on one
+// thread.
+//
+// introselect_rounds runs the rounds on [first, last) through get(i) / put(i, v) until the range is no longer than
+// `until` (3 = to the end, insertion sort included).  lsta / lstb: room for last - first positions each.  Returns
+// true when nothing is left to do.
+template <typename Get, typename Put>
+__device__ bool introselect_rounds(Get get, Put put, uint32_t& first, uint32_t& last, uint32_t nth, uint32_t& depth,
+                                   uint32_t until, uint32_t* lsta, uint32_t* lstb, FinishShared& sm)
 {
     typedef unsigned long long u64;
     const uint32_t tid = threadIdx.x, lane = lane_id(), wave = wave_id();
-    auto get = [&](uint32_t i) { return ((u64)key[i] << 32) | (u64)idx[i]; };
-    auto put = [&](uint32_t i, u64 v) {
-        key[i] = (uint32_t)(v >> 32);
-        idx[i] = (uint32_t)v;
-    };
-    if (n == 0 || nth >= n)
-        return;
-    uint32_t first = 0, last = n;
-    uint32_t depth = 2u * (31u - (uint32_t)__clz((int)n));
-    __syncthreads();
-    while (last - first > 3u) {
+    while (last - first > until) {
         if (depth == 0) {
             // __heap_select(first, nth + 1, last) and iter_swap(first, nth): bits/stl_algo.h:1956-1960, stl_heap.h
             if (tid == 0) {
@@ -2351,7 +2346,7 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
                 put(nth, a);
             }
             __syncthreads();
-            return;
+            return true;
         }
         --depth;
         if (tid == 0) { // __move_median_to_first(first, first + 1, mid, last - 1)
@@ -2372,11 +2367,17 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
         const uint32_t chunk = ((len + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
         const uint32_t beg = min(last, lo0 + wave * chunk), end = min(last, beg + chunk);
         // entries of the wave's chunk that belong left of the cut
+        // (kTrip loads in flight per lane: a trip costs one round trip to memory, not kTrip)
+        constexpr uint32_t kTrip = 4;
         uint32_t mine = 0;
-        for (uint32_t base = beg; base < end; base += kWave) {
-            const uint32_t pos = base + lane;
-            const bool small = pos < end && get(min(pos, last - 1u)) < pivot;
-            mine += (uint32_t)__popcll(__ballot(small));
+        for (uint32_t base = beg; base < end; base += kWave * kTrip) {
+            u64 v[kTrip];
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u)
+                v[u] = get(min(base + u * kWave + lane, last - 1u));
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u)
+                mine += (uint32_t)__popcll(__ballot(base + u * kWave + lane < end && v[u] < pivot));
         }
         if (lane == 0)
             sm.bs.u64[wave] = mine;
@@ -2392,17 +2393,24 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
         uint32_t big_before = (beg - lo0) - small_before;
         // position lists: lsta[t] = the t-th big entry from the left, lstb[t] = the t-th small entry from the left
         const u64 lower = (1ull << lane) - 1ull;
-        for (uint32_t base = beg; base < end; base += kWave) {
-            const uint32_t pos = base + lane;
-            const bool in = pos < end;
-            const bool small = in && get(min(pos, last - 1u)) < pivot;
-            const u64 bs = __ballot(small), bb = __ballot(in && !small);
-            if (small)
-                lstb[small_before + (uint32_t)__popcll(bs & lower)] = pos;
-            else if (in)
-                lsta[big_before + (uint32_t)__popcll(bb & lower)] = pos;
-            small_before += (uint32_t)__popcll(bs);
-            big_before += (uint32_t)__popcll(bb);
+        for (uint32_t base = beg; base < end; base += kWave * kTrip) {
+            u64 v[kTrip];
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u)
+                v[u] = get(min(base + u * kWave + lane, last - 1u));
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u) {
+                const uint32_t pos = base + u * kWave + lane;
+                const bool in = pos < end;
+                const bool small = in && v[u] < pivot;
+                const u64 bs = __ballot(small), bb = __ballot(in && !small);
+                if (small)
+                    lstb[small_before + (uint32_t)__popcll(bs & lower)] = pos;
+                else if (in)
+                    lsta[big_before + (uint32_t)__popcll(bb & lower)] = pos;
+                small_before += (uint32_t)__popcll(bs);
+                big_before += (uint32_t)__popcll(bb);
+            }
         }
         __syncthreads();
         const uint32_t pairs = min(bigs, smalls);
@@ -2421,6 +2429,8 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
         else
             last = cut;
     }
+    if (last - first > 3u)
+        return false;
     if (tid == 0) // __insertion_sort(first, last)
         for (uint32_t i = first + 1u; i < last; ++i) {
             const u64 v = get(i);
@@ -2435,12 +2445,53 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
             put(j, v);
         }
     __syncthreads();
+    return true;
+}
+
+// The row's candidates in device memory (key[i], idx[i]; lsta / lstb: room for n positions each).  The rounds run on
+// device memory, ten or so dependent trips to memory each, until the range fits the dynamic LDS block (kSortMax
+// entries and two position lists); the remaining dozen rounds run on a copy there.
+__device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32_t nth, uint32_t* lsta, uint32_t* lstb,
+                                const FinishLds& L)
+{
+    typedef unsigned long long u64;
+    const uint32_t tid = threadIdx.x;
+    if (n == 0 || nth >= n)
+        return;
+    uint32_t first = 0, last = n;
+    uint32_t depth = 2u * (31u - (uint32_t)__clz((int)n));
+    __syncthreads();
+    auto get = [=](uint32_t i) { return ((u64)key[i] << 32) | (u64)idx[i]; };
+    auto put = [=](uint32_t i, u64 v) {
+        key[i] = (uint32_t)(v >> 32);
+        idx[i] = (uint32_t)v;
+    };
+    if (introselect_rounds(get, put, first, last, nth, depth, kSortMax, lsta, lstb, *L.sm))
+        return;
+    MAKO_STAMP(28);
+    u64* lds = L.sortk;
+    uint32_t* la = reinterpret_cast<uint32_t*>(L.sortk + kSortMax);
+    uint32_t* lb = la + kSortMax;
+    static_assert(kSortMax * 16u <= kDynLds, "the range and its two position lists fit the dynamic LDS block");
+    const uint32_t base = first, len = last - first;
+    for (uint32_t i = tid; i < len; i += kThreads)
+        lds[i] = get(base + i);
+    __syncthreads();
+    introselect_rounds([=](uint32_t i) { return lds[i - base]; }, [=](uint32_t i, u64 v) { lds[i - base] = v; }, first, last,
+                       nth, depth, 3u, la, lb, *L.sm);
+    for (uint32_t i = tid; i < len; i += kThreads)
+        put(base + i, lds[i]);
+    __syncthreads();
 }
 
 // Common tail of the whole-row paths.  key[0]/idx[0] of the row hold n0 candidates (~bits(q), token id) in index
 // order.  Sorts them by (q desc, idx asc) when top-k or top-p is active, truncates (src/gen/sampler.cpp:39-61)
 // and draws.  `total64` (when have_total) is the fp64 sum of q over all candidates of the row, of which the list
 // may be only the heaviest part; otherwise it is summed from the list.
+// (TOPK_ALONE = false leaves the top-k-without-top-p branch out of the instance inside plan_kernel<true>: that kernel is
+// only launched for batches whose host copy of the parameters shows a top-p on every sampled row, and the branch's
+// registers would be spilled around the top-k rows' fast path, +3.5 us on a 256-row batch.)
+template <bool TOPK_ALONE>
 __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
                                    uint32_t n0, bool have_total, double total64, uint32_t path, const FinishLds& L)
 {
@@ -2453,25 +2504,22 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
     // order by (q desc, idx asc): stable LSD radix sort of ~bits(q), ascending
     const bool topk_active = P.top_k > 0 && P.top_k < n0;
     const bool topp_active = P.top_p < 1.0f;
-    if (topk_active && !topp_active) {
-        // top-k alone: the survivors stay in the order nth_element leaves them (sampler.cpp:39-43, then :79-83)
-        nth_element_row(key0, idx0, n0, P.top_k, key1, idx1, sm);
-        const uint32_t* kf = key0;
-        const uint32_t* jf = idx0;
-        draw_from_list(
-            d, row, [=](uint32_t i) { return __uint_as_float(~kf[i]); }, [=](uint32_t i) { return jf[i]; }, P.top_k, path, sm);
-        return;
-    }
-    if (topk_active || topp_active)
+    // top-k alone: the survivors stay in the order nth_element leaves them (sampler.cpp:39-43, then :79-83)
+    const bool nth_order = TOPK_ALONE && topk_active && !topp_active;
+    if (nth_order)
+        nth_element_row(key0, idx0, n0, P.top_k, key1, idx1, L);
+    else if (topk_active || topp_active)
         sort_segment(key0, idx0, key1, idx1, n0, L);
     const uint32_t *ks = key0, *is = idx0;
     MAKO_STAMP(12);
     const uint32_t n1 = topk_active ? P.top_k : n0; // sampler.cpp:40-43
-    if (topk_active || topp_active) {
+    // (sorted_tail's one-wave path for lists of up to kGroup entries adds and walks them in the order given, whatever
+    // it is, and without a top-p it cuts nothing: nth_element's survivors take it too)
+    if (nth_order ? (!d.draft && n1 <= kGroup) : (topk_active || topp_active)) {
         sorted_tail(d, row, P, ks, is, n1, have_total, total64, path, L);
         return;
     }
-    // neither top-k nor top-p: the candidates stay in index order
+    // nth_element's order (long lists, verification), or neither top-k nor top-p: the candidates stay in index order
     const uint32_t* kf = ks;
     const uint32_t* jf = is;
     draw_from_list(
@@ -3108,6 +3156,7 @@ __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32
     const float* lrow = d.logits + (int64_t)row * d.logits_stride;
     const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
 
+    MAKO_STAMP(24);
     // 1. masked copy, then the penalties once per distinct history token
     for (uint32_t i = tid; i < V; i += kThreads) {
         float v = lrow[i];
@@ -3137,6 +3186,7 @@ __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32
         __syncthreads();
     }
 
+    MAKO_STAMP(25);
     // 2. weights and the min_p / q > 0 filter, compacted in index order (sampler.cpp:29-36)
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p; // std::min(min_p, 1.0f)
@@ -3169,11 +3219,12 @@ __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32
     }
     __syncthreads();
 
+    MAKO_STAMP(26);
     if (n0 == 0) {
         fallback_row(d, row, argidx);
         return;
     }
-    sort_truncate_draw(d, sc, row, P, n0, false, 0.0, MAKO_PATH_GENERAL, L);
+    sort_truncate_draw<SITE == 0>(d, sc, row, P, n0, false, 0.0, MAKO_PATH_GENERAL, L);
 }
 
 // Bitonic sort, descending, of 1024 * ITEMS keys held ITEMS per thread: key[t] is element t * 1024 + tid.
