@@ -2468,7 +2468,6 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
     };
     if (introselect_rounds(get, put, first, last, nth, depth, kSortMax, lsta, lstb, *L.sm))
         return;
-    MAKO_STAMP(28);
     u64* lds = L.sortk;
     uint32_t* la = reinterpret_cast<uint32_t*>(L.sortk + kSortMax);
     uint32_t* lb = la + kSortMax;
@@ -3156,7 +3155,6 @@ __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32
     const float* lrow = d.logits + (int64_t)row * d.logits_stride;
     const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
 
-    MAKO_STAMP(24);
     // 1. masked copy, then the penalties once per distinct history token
     for (uint32_t i = tid; i < V; i += kThreads) {
         float v = lrow[i];
@@ -3186,28 +3184,72 @@ __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32
         __syncthreads();
     }
 
-    MAKO_STAMP(25);
-    // 2. weights and the min_p / q > 0 filter, compacted in index order (sampler.cpp:29-36)
+    // 2. weights and the min_p / q > 0 filter, compacted in index order (sampler.cpp:29-36).  Wave w owns the w-th
+    // sixteenth of the row (a multiple of 256 logits, lane l entries 4l..4l+3 of each 256): a sweep that leaves bits(q)
+    // of every candidate (0 otherwise) in place of the logit and counts them, one exchange of the waves' totals, and
+    // a sweep in which every lane reads back what it wrote and a wave scan ranks it.  No barrier inside the sweeps.
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p; // std::min(min_p, 1.0f)
-    uint32_t n0 = 0;
-    for (uint32_t base = 0; base < V; base += kThreads * 4u) {
-        const uint32_t i = base + tid * 4u;
+    uint32_t* qb = reinterpret_cast<uint32_t*>(wbuf);
+    const uint32_t lane = lane_id(), wave = wave_id();
+    const uint32_t chunk = ((V + kThreads * 4u - 1u) / (kThreads * 4u)) * kGroup;
+    const uint32_t beg = min(V, wave * chunk), end = min(V, beg + chunk);
+    uint32_t mine = 0;
+    for (uint32_t base = beg; base < end; base += kGroup) {
+        const uint32_t i = base + lane * 4u;
+        float w[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        const bool whole = i + 3u < end;
+        if (whole) {
+            const float4 x = *reinterpret_cast<const float4*>(wbuf + i);
+            w[0] = x.x, w[1] = x.y, w[2] = x.z, w[3] = x.w;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (i + j < end)
+                    w[j] = wbuf[i + j];
+        }
         uint32_t k[4];
-        uint32_t c = 0;
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            k[j] = 0;
-            if (i + j < V) {
-                const float q = weight_of(wbuf[i + j], m, inv_t, sm.tab);
-                if (q >= floor_q && q > 0.0f) {
-                    k[j] = __float_as_uint(q);
-                    ++c;
-                }
-            }
+            const float q = weight_of(w[j], m, inv_t, sm.tab);
+            k[j] = (i + j < end && q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
+            mine += k[j] ? 1u : 0u;
         }
-        uint32_t tot;
-        uint32_t pos = n0 + block_excl_scan_u32(c, tot, sm.bs);
+        if (whole) {
+            *reinterpret_cast<uint4*>(qb + i) = make_uint4(k[0], k[1], k[2], k[3]);
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (i + j < end)
+                    qb[i + j] = k[j];
+        }
+    }
+    mine = __ockl_wfred_add_u32(mine);
+    if (lane == 0)
+        sm.bs.u64[wave] = mine;
+    __syncthreads();
+    uint32_t n0 = 0, at = 0;
+    for (int w = 0; w < kWaves; ++w) {
+        const uint32_t x = (uint32_t)sm.bs.u64[w];
+        if (w < (int)wave)
+            at += x;
+        n0 += x;
+    }
+    for (uint32_t base = beg; base < end; base += kGroup) {
+        const uint32_t i = base + lane * 4u;
+        uint32_t k[4] = {0u, 0u, 0u, 0u};
+        if (i + 3u < end) {
+            const uint4 x = *reinterpret_cast<const uint4*>(qb + i);
+            k[0] = x.x, k[1] = x.y, k[2] = x.z, k[3] = x.w;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (i + j < end)
+                    k[j] = qb[i + j];
+        }
+        const uint32_t c = (k[0] ? 1u : 0u) + (k[1] ? 1u : 0u) + (k[2] ? 1u : 0u) + (k[3] ? 1u : 0u);
+        const uint32_t incl = __ockl_wfscan_add_u32(c, true);
+        uint32_t pos = at + incl - c;
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
             if (k[j]) {
@@ -3215,11 +3257,10 @@ __device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32
                 idx0[pos] = i + j;
                 ++pos;
             }
-        n0 += tot;
+        at += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
     }
     __syncthreads();
 
-    MAKO_STAMP(26);
     if (n0 == 0) {
         fallback_row(d, row, argidx);
         return;
