@@ -523,6 +523,10 @@ def test_host_parameter_copy_only_skips_work(gpu_ctx):
             p["top_k"] = np.uint32(5000)
             p["top_p"] = np.float32(0.97)
             p["temperature"] = np.float32(0.9)
+        elif case == 5:  # top-k alone: whole-row rows in nth_element's order
+            p["top_k"] = rng.choice(np.array([3, 40, 1000], np.uint32), b)
+            p["top_p"] = np.float32(1.0)
+            p["temperature"] = np.float32(0.9)
         _say("host parameter copy case %d" % case)
         kw = dict(mask=w.get("mask"), hist=w.get("hist"), hist_len=w.get("hist_len"), cand_cap=64)
         full = api.sample(gpu_ctx, w["logits"], p, w["u"], **kw)
