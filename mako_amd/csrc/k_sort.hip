@@ -5,14 +5,14 @@
 #include "sampler_kernels.h"
 
 namespace mako {
-void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc)
+void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows)
 {
-    hipLaunchKernelGGL(partition_kernel, dim3(kWorkers, d.n_rows), dim3(kThreads), 0, st, d, sc);
+    hipLaunchKernelGGL(partition_kernel, dim3(kWorkers, grid_rows), dim3(kThreads), 0, st, d, sc);
 }
 
-void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices)
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices, uint32_t grid_rows)
 {
-    hipLaunchKernelGGL(sort_kernel, dim3(kWorkers, d.n_rows), dim3(kThreads), kSortLds, st, d, sc, slices);
+    hipLaunchKernelGGL(sort_kernel, dim3(kWorkers, grid_rows), dim3(kThreads), kSortLds, st, d, sc, slices);
 }
 
 hipError_t init_sort_kernels()

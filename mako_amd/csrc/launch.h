@@ -29,7 +29,11 @@ void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sa
 // plan_kernel is the last kernel of the batch
 void launch_plan_for_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
 void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
-void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc); // (host copy, by value)
-void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
-void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch* sc);
+// partition_kernel and sort_kernel serve the same work list, workgroup i its entry i: `grid_rows` * kWorkers workgroups
+// must cover the longest list the batch can produce (kWorkers entries per top_k == 0 row, one per other sampled
+// row); tail_kernel takes one workgroup per possible wide row.  Workgroups beyond the lists leave at once, but each
+// of them still has to be dispatched.
+void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows); // (host copy, by value)
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices, uint32_t grid_rows);
+void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t grid_rows);
 } // namespace mako

@@ -271,14 +271,22 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
             MAKO_HIP(ctx, hipEventRecord(ctx->ev[i], st));                                                         \
     } while (0)
     // which kernels have work: all of them unless the caller's host copy of the parameters says otherwise
+    // and how long the finishing kernels' work lists can get: kWorkers entries per top_k == 0 row, one per other
+    // sampled row (whole-row rows, top-k rows that cannot be certified from their candidates)
     bool any_nucleus = true, any_general = true;
+    uint32_t nucleus_rows = d.n_rows, list_rows = d.n_rows;
     if (params_host) {
         any_nucleus = any_general = false;
+        uint32_t n_nucleus = 0, n_other = 0;
         for (uint32_t r = 0; r < d.n_rows; ++r) {
             const mako::RowClass c = mako::classify(params_host[r]);
             any_nucleus |= c == mako::kNucleus;
             any_general |= c == mako::kGeneral;
+            n_nucleus += c == mako::kNucleus;
+            n_other += c == mako::kTopK || c == mako::kGeneral;
         }
+        nucleus_rows = std::max(n_nucleus, 1u);
+        list_rows = std::max(n_nucleus + (n_other + mako::kWorkers - 1u) / mako::kWorkers, 1u);
     }
     const bool launch_sort = any_nucleus || any_general;
     MAKO_MARK(0);
@@ -295,13 +303,13 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
         mako::launch_plan_alone(st, d, ctx->sc_dev, slices);
     MAKO_MARK(3);
     if (any_nucleus)
-        mako::launch_partition(st, d, ctx->sc);
+        mako::launch_partition(st, d, ctx->sc, list_rows);
     MAKO_MARK(4);
     if (launch_sort)
-        mako::launch_sort(st, d, ctx->sc_dev, slices);
+        mako::launch_sort(st, d, ctx->sc_dev, slices, list_rows);
     MAKO_MARK(5);
     if (any_nucleus)
-        mako::launch_tail(st, d, ctx->sc_dev);
+        mako::launch_tail(st, d, ctx->sc_dev, nucleus_rows);
     MAKO_MARK(6);
 #undef MAKO_MARK
     ctx->profiled = prof;
