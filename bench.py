@@ -102,8 +102,8 @@ def main():
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
     a = ap.parse_args()
     if a.gpus != 1:
-        raise SystemExit("bench.py measures one GPU: rows are independent, a multi-GPU run is a plain batch split "
-                         "(see DESIGN.md); run with --gpus 1")
+        raise SystemExit("bench.py measures one GPU: rows are independent, so a multi-GPU run is a plain split of "
+                         "the batch by rows with nothing exchanged; run with --gpus 1")
 
     from mako_amd import api, hip, workloads
     from oracle import pyoracle
