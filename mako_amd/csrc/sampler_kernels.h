@@ -1892,14 +1892,22 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             G.cmax()[tid] = T.cmax[t_base + tid];
             // (clamped into the list: a record is only ever read, never trusted for addressing)
             const uint32_t st = min(T.start[t_base + tid], n1), pk = T.pack[t_base + tid];
+            // (the quarter records are asked for together with the rest, whether or not the group has any: asking
+            // only once `pk` is known would be one more trip to memory for every row)
+            const uint4* tq = T.quarters + (t_base + tid) * 4u;
+            const uint4 qr0 = tq[0], qr1 = tq[1], qr2 = tq[2], qr3 = tq[3];
             uint32_t slot = 0;
             if (pk & kHasQuarters) {
                 slot = atomicAdd(&G.misc()[3], 1u) + 1u;
                 if (slot > kQuarterSlots)
                     slot = 0;
-                else
-                    for (uint32_t k = 0; k < 4; ++k)
-                        G.quarters()[(slot - 1u) * 4u + k] = T.quarters[(t_base + tid) * 4u + k];
+            }
+            if (slot) {
+                uint4* gq = G.quarters() + (slot - 1u) * 4u;
+                gq[0] = qr0;
+                gq[1] = qr1;
+                gq[2] = qr2;
+                gq[3] = qr3;
             }
             G.start()[tid] = st;
             G.pack()[tid] = min(pk & kLenMask, min(kGroup, n1 - st)) | (slot << 9) | (pk & 0x00ff0000u);
