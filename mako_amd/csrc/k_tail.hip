@@ -4,7 +4,7 @@
 #include "sampler_kernels.h"
 
 namespace mako {
-void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t grid_rows)
+void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows)
 {
     hipLaunchKernelGGL(tail_kernel, dim3(1, grid_rows), dim3(kThreads), kDynLds, st, d, sc);
 }

@@ -309,7 +309,7 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
         mako::launch_sort(st, d, ctx->sc_dev, slices, list_rows);
     MAKO_MARK(5);
     if (any_nucleus)
-        mako::launch_tail(st, d, ctx->sc_dev, nucleus_rows);
+        mako::launch_tail(st, d, ctx->sc, nucleus_rows);
     MAKO_MARK(6);
 #undef MAKO_MARK
     ctx->profiled = prof;
