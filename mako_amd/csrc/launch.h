@@ -34,6 +34,6 @@ void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch*
 // row); tail_kernel takes one workgroup per possible wide row.  Workgroups beyond the lists leave at once, but each
 // of them still has to be dispatched.
 void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows); // (host copy, by value)
-void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices, uint32_t grid_rows);
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows); // (host copy)
 void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows); // (host copy, by value)
 } // namespace mako

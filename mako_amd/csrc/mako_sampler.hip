@@ -306,7 +306,7 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
         mako::launch_partition(st, d, ctx->sc, list_rows);
     MAKO_MARK(4);
     if (launch_sort)
-        mako::launch_sort(st, d, ctx->sc_dev, slices, list_rows);
+        mako::launch_sort(st, d, ctx->sc, slices, list_rows);
     MAKO_MARK(5);
     if (any_nucleus)
         mako::launch_tail(st, d, ctx->sc, nucleus_rows);

@@ -4172,19 +4172,22 @@ __global__ __launch_bounds__(kThreads) void partition_kernel(mako_sample_desc d,
 // grid = (kWorkers, rows) workgroups, of which workgroup i serves entry i of the work list.  Worker w gathers its range of weights from
 // the row's bits(q) array, sorts it and stores it at its place in the row's sorted list; the last worker to
 // finish cuts the nucleus and draws.
-__global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
+__global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
 {
-    const Scratch& sc_arg = *sc_dev;
+    // (the context's record by value: its first loads, the list's length and this workgroup's entry, go out together
+    // and at once; the list has room for every workgroup of the grid)
+    const Scratch& sc_arg = sc_val;
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
     const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
-    if (piece >= sc_arg.work_n[0])
+    const uint32_t n_work = sc_arg.work_n[0];
+    const uint32_t item = sc_arg.work_sort[piece];
+    if (piece >= n_work)
         return;
 #ifdef MAKO_TIMING_SORT
     MAKO_WG_TIMER;
 #endif
-    const uint32_t item = sc_arg.work_sort[piece];
     const uint32_t row = item >> 8, w = item & 255u, tid = threadIdx.x;
     MAKO_ROW(row);
     const uint32_t flag = sc_arg.plan[row].flag;
