@@ -19,7 +19,8 @@ hipError_t init_sort_kernels();
 hipError_t init_tail_kernels();
 
 // scan_kernel<vec, kh, above>, grid = (slices, rows), `lds` bytes of dynamic LDS
-// (`sc`: the HOST copy of the context's record; this kernel takes it by value, the others by device pointer)
+// (`sc`: the HOST copy of the context's record; scan, partition, sort and tail kernels take it by value, so that their
+// first loads need no trip to memory for the record itself; finish and plan kernels take the device copy's address)
 void launch_scan(bool vec, int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d,
                  const Scratch& sc, uint32_t slice_len, uint32_t cus);
 // finish_kernel<vec, kh> on `wgs` workgroups
