@@ -1,0 +1,172 @@
+// Constants, the context's scratch layout, order keys and the classification of rows: shared by every kernel
+// of the sampler.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <type_traits>
+#include "../../include/mako_sampler.h"
+#include "block_prims.h"
+#include "device_math.h"
+#include "seqfp.h"
+#include "tuning_stamps.h"
+
+namespace mako {
+
+constexpr uint32_t kNone = 0xffffffffu;
+
+constexpr uint32_t kSliceMax = 16384; // elements per slice: 16 per thread
+constexpr uint32_t kMaxSlices = 64;
+constexpr uint32_t kCap = 512;       // candidates kept per slice
+constexpr uint32_t kTopKFast = 128;  // largest top_k resolved from the per-slice candidates
+constexpr uint32_t kSortMax = 4096;  // candidates the finisher sorts in LDS
+constexpr uint32_t kDynLds = 65536;  // dynamic LDS of both kernels
+constexpr uint32_t kBins = 2048;     // weight histogram of top_k == 0 rows, see weight_bin()
+constexpr uint32_t kBinSumBits = 44; // a bin's record: count << 44 | sum of 24-bit significands
+
+// Histogram bin of a weight q in (0, 1], by its bits: 128 bins per binade for the eight binades below 1.0 (bins
+// 1024..2047) and 8 per binade for everything smaller, subnormals included (bins 71..1023; bins below 71 stay
+// empty).  Bin edges include every binade boundary, so all weights of a bin share their exponent and the bin's
+// mass is exactly (sum of 24-bit significands) * 2^(exponent - 150).  The fine bins keep near-flat rows, whose
+// weights all lie within a factor of two, spread over all workers.
+constexpr uint32_t kFineFrom = 0x3b810000u; // bits(2^-8) + 0x10000: the top fine bin holds 1.0 alone
+constexpr uint32_t kCoarseShift = 20;       // 8 bins per binade
+constexpr uint32_t kCoarseBase = 1023u - ((kFineFrom - 1u) >> kCoarseShift); // 71
+__device__ __forceinline__ uint32_t weight_bin(uint32_t bits)
+{
+    return bits >= kFineFrom ? min(1024u + ((bits - kFineFrom) >> 16), kBins - 1u) : (bits >> kCoarseShift) + kCoarseBase;
+}
+// Smallest bits(q) of a bin, and one past the largest.
+__device__ __forceinline__ uint32_t bin_lo_key(uint32_t b)
+{
+    if (b >= 1024u)
+        return kFineFrom + ((b - 1024u) << 16);
+    return b > kCoarseBase ? (b - kCoarseBase) << kCoarseShift : 0u;
+}
+__device__ __forceinline__ uint32_t bin_hi_key(uint32_t b)
+{
+    return b + 1u < kBins ? bin_lo_key(b + 1u) : kFineFrom + (1024u << 16); // (just above bits(1.0f))
+}
+
+constexpr uint32_t kFlagFirstNan = 1u; // element 0 of the row is NaN (slice 0 only)
+constexpr uint32_t kFlagOverflow = 2u; // more than kCap logits reached the slice's threshold
+constexpr uint32_t kFlagComplete = 4u; // every logit above -inf was emitted
+
+struct SliceStat {
+    float wmax;       // max of the slice's penalised logits (-inf if none compares greater)
+    uint32_t argidx;  // first index holding it, kNone if nothing exceeded -inf
+    uint32_t flags;
+    uint32_t n_emit;  // candidates written for this slice
+    uint32_t tau_key; // order key of the emission threshold: every logit with key >= tau_key was emitted
+    uint32_t above;   // logits of the slice strictly above the row's close_token logit (0 without one)
+    uint32_t pad[2];
+};
+
+constexpr uint32_t kWorkers = 32;  // workgroups that share the sort of one wide-nucleus row
+constexpr uint32_t kGroup = 256;      // a sorted list is processed in groups of one wave x four entries per lane
+constexpr uint32_t kMaxGroups = 1024; // groups per list
+constexpr uint32_t kSegCap = 6144;    // entries a worker sorts in LDS
+constexpr uint32_t kFine = 2048;      // value buckets of that sort
+// dynamic LDS of sort_kernel: the entries, their order, the buckets, and a copy of the sorted weights for the group
+// records
+constexpr uint32_t kSortLds = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u + kSegCap * 4u;
+constexpr uint32_t kSortedCopyAt = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u; // byte offset of that copy
+
+// Work order for a top_k == 0 row whose nucleus is too wide for the per-slice candidate lists: the weights
+// with bits(q) >= key_lo (n0 of them) are split by value into kWorkers contiguous ranges of about equal size.
+struct BigPlan {
+    uint32_t flag;   // 1: the row waits for sort_kernel's workers; 2: for its whole-row path (worker 0 alone);
+                     // 3: a narrow nucleus, finished by worker 0 from the candidate lists
+    uint32_t n0;     // entries to sort
+    uint32_t pad0;
+    uint32_t groups; // groups of the whole list: each worker's range is cut into groups of kGroup on its own
+    double total64;  // exact fp64 sum of q over the row's candidates
+    uint32_t thr;    // bits(q) below which the nucleus cannot reach
+    uint32_t pad;
+    uint32_t key_lo[kWorkers]; // worker w takes bits(q) in [key_lo[w], key_hi[w])
+    uint32_t key_hi[kWorkers];
+    uint32_t off[kWorkers];    // and writes them from position off[w] of the sorted list
+    uint32_t cnt[kWorkers];
+    uint32_t gbase[kWorkers];  // first group of worker w
+    uint32_t cursor[kWorkers]; // entries partition_kernel has handed to worker w so far
+    double mass[kWorkers];     // sum of the weights above worker w's range
+};
+
+// Per-group records of a planned row's sorted list, written by the workers and read by the last of them.
+struct GroupTable {
+    double* sum;     // fp64 sum of the group's weights
+    uint32_t* d0;    // the group's map for the running fp32 sum in the epoch guessed from the mass before it
+    uint32_t* d1;
+    uint32_t* cmax;
+    uint32_t* start; // first entry of the group in the sorted list
+    uint32_t* pack;  // entries | guessed exponent << 16 | kHasQuarters if `quarters` holds records for the group
+    uint4* quarters; // [4] per group: the maps of the group's four quarters (see build_quarters)
+};
+
+struct Scratch {
+    SliceStat* stats;  // [max_rows][kMaxSlices]
+    float* cand_w;     // [max_rows][slices_cap][kCap] penalised logits of the slice's candidates
+    uint32_t* cand_i;  // [max_rows][slices_cap][kCap] their token ids
+    double* part_sum;  // [max_rows][kMaxSlices] exact fp64 sum of q over the slice (top_k == 0 rows)
+    uint32_t* part_n;  // [max_rows][kMaxSlices] candidates (q > 0, q >= min_p) in the slice
+    BigPlan* plan;     // [max_rows]; flag zero between calls
+    unsigned long long* bins; // [max_rows][kBins] weight histogram of top_k == 0 rows: candidates in the bin << 44 |
+                              // sum of their 24-bit significands (kBinSumBits: at most 2^20 - 1 logits per row).
+                              // A bin's exact mass is that sum * 2^(e - 150), e being the bin's exponent.  The
+                              // slices add with one atomic per non-empty bin; plan_kernel reads the row's bins
+                              // and leaves them zero
+    float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path; top_k == 0 rows keep
+                       // bits(q) of every logit here instead (0 where q is not a candidate)
+    uint32_t* cnt;     // [max_rows][vpad] token counts; all zero between calls
+    uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong; [1] also takes the workers' unsorted
+                       // shares (bits(q)) from partition_kernel
+    uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, likewise
+    uint8_t* bin_worker; // [max_rows][kBins] the worker that takes the weights of each histogram bin (0xff: none)
+    GroupTable gt;     // [max_rows][g_cap] each
+    // Work lists.  sort_kernel and tail_kernel are launched with one workgroup per POSSIBLE piece of work, but
+    // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
+    // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
+    // (finish_kernel and plan_kernel get the same effect from find_piece().)
+    uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); then, 16-byte aligned at [4],
+                           // the second pass's pieces per top_k == 0 row, their length and the number of workgroups
+                           // with work (scan_kernel's first workgroup decides, see second_pass_pieces())
+    uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel and plan_kernel
+    uint32_t* work_tail;   // [max_rows] row; appended by plan_kernel
+    uint64_t vpad;
+    uint32_t slices_cap;
+    uint32_t g_cap;    // vpad / kGroup + kWorkers
+};
+
+// Total order on floats as unsigned keys: -inf < ... < -0 = +0 < ... < +inf.  Never called on NaN.
+__device__ __forceinline__ uint32_t order_key(float f)
+{
+    const uint32_t b = __float_as_uint(f + 0.0f); // -0 -> +0
+    return b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u);
+}
+__device__ __forceinline__ float order_unkey(uint32_t k)
+{
+    const uint32_t b = (k & 0x80000000u) ? (k ^ 0x80000000u) : ~k;
+    return __uint_as_float(b);
+}
+constexpr uint32_t kKeyNegInf = 0x007fffffu; // order_key(-inf)
+
+enum RowClass { kGreedy = 0, kTopK = 1, kNucleus = 2, kGeneral = 3 };
+
+__host__ __device__ __forceinline__ RowClass classify(const mako_sampling_params& p)
+{
+    if (p.temperature <= 0.0f) // Sampler::greedy, src/gen/sampler.hpp:26
+        return kGreedy;
+    if (!(p.top_p < 1.0f)) // no top-p: the candidate order is not the sorted one (sampler.cpp:44)
+        return kGeneral;
+    if (p.top_k == 0)
+        return kNucleus;
+    return p.top_k <= kTopKFast ? kTopK : kGeneral;
+}
+
+__device__ __forceinline__ bool penalties_neutral(const mako_sampling_params& p)
+{
+    return p.repetition_penalty == 1.0f && p.presence_penalty == 0.0f && p.frequency_penalty == 0.0f;
+}
+
+} // namespace mako

@@ -1,0 +1,211 @@
+// scan_kernel: the single pass over the logits in device memory.
+#pragma once
+
+#include "slice_load.h"
+#include "work_split.h"
+
+namespace mako {
+
+struct alignas(16) ScanShared {
+    uint32_t wave_max[kWaves]; // order keys
+    uint32_t wave_kth[kWaves];
+    uint32_t wave_above[kWaves];
+    uint32_t argidx;
+    uint32_t emit_n;
+    uint32_t emit_flags;
+    float cw[kCap];
+    uint32_t ci[kCap];
+};
+
+// A lower bound, tight to 2^-9 relative, of the j-th largest of the wavefront's 64 order keys (j >= 1): the largest
+// v with at least j keys >= v, built bit by bit from the top down to bit 14 (the low fourteen bits stay zero: whoever
+// uses the result as a threshold keeps at least j keys, and a handful more at most).  One vector compare per bit;
+// the rest is scalar.
+__device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
+{
+    uint32_t prefix = 0;
+#pragma unroll
+    for (int b = 31; b >= 14; --b) {
+        const uint32_t cand = prefix | (1u << b);
+        const uint32_t c = (uint32_t)__popcll(__ballot(key >= cand));
+        prefix = c >= j ? cand : prefix;
+    }
+    return prefix;
+}
+
+// grid = (slices, rows).
+// (ABOVE: the batch has close tokens, whose logits' ranks are counted on the way; a variant of its own because the
+// count takes sixteen more registers, up to the limit for two workgroups per CU, which no other batch should pay)
+template <bool VEC, int KH, bool ABOVE = false>
+__global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scratch sc_arg, uint32_t slice_len,
+                                                        uint32_t cus)
+{
+    // (scan_kernel takes the context's record by value: its first loads then need no trip to memory for a pointer)
+    const Scratch& sc = sc_arg;
+    MAKO_ROW(blockIdx.y);
+#ifdef MAKO_TIMING_SCAN
+    MAKO_WG_TIMER;
+#endif
+    // (16-byte alignment: the table is cleared and read with 128-bit LDS operations, which crawl when misaligned)
+    extern __shared__ __align__(16) uint32_t s_dyn[]; // [slice_len] token counts when the row has penalties
+    __shared__ ScanShared sm;
+
+    const uint32_t row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
+    MAKO_STAMP(28);
+    const uint32_t lo = slice * slice_len;
+    const uint32_t hi = min(d.n_vocab, lo + slice_len);
+    // (the history's length is asked for whatever the parameters say: its load then leaves together with theirs)
+    const uint32_t hl_row = d.hist_tokens ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
+    const mako_sampling_params P = d.params[row];
+    const RowClass cls = classify(P);
+    // Greedy rows ignore the penalties (src/gen/sampler.cpp:77-78).
+    const uint32_t hl = cls != kGreedy ? hl_row : 0u;
+    const bool pen = hl > 0 && !penalties_neutral(P);
+    if (tid == 0) {
+        sm.argidx = kNone;
+        sm.emit_n = 0;
+        sm.emit_flags = 0;
+        if (row == 0 && slice == 0) { // the lists finish_kernel and plan_kernel append to start empty
+            sc.work_n[0] = 0;
+            sc.work_n[1] = 0;
+        }
+    }
+    if (row == 0 && slice == 0 && wave_id() == 1) { // how the second pass will be cut up
+        uint32_t piece_len, busy;
+        const uint32_t pieces = second_pass_pieces(d, gridDim.x, slice_len, cus, piece_len, busy);
+        if (lane_id() == 0)
+            *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(pieces, piece_len, busy, 0u);
+    }
+    // ReasoningBudget::forced's question (src/server/openai.cpp:598-602), answered in the same pass over the logits
+    bool want_above = false;
+    float close_v = 0.0f;
+    if (ABOVE && d.close_token) {
+        const int32_t ct = d.close_token[row];
+        if (ct >= 0 && (uint32_t)ct < d.n_vocab &&
+            (!d.mask || ((d.mask[(int64_t)row * d.mask_stride + ((uint32_t)ct >> 5)] >> ((uint32_t)ct & 31u)) & 1u))) {
+            want_above = true;
+            close_v = d.logits[(int64_t)row * d.logits_stride + ct];
+        }
+    }
+    uint32_t above = 0;
+    float wv[16];
+    if (ABOVE) {
+        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv, NoOverlap(), want_above, close_v, &above);
+        if (want_above) // uniform
+            above = __ockl_wfred_add_u32(above);
+    } else {
+        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, s_dyn, wv);
+    }
+
+    MAKO_STAMP(29);
+    // maximum of the thread's logits (NaNs ignored), then of the wave, then of the slice
+    float best = -INFINITY;
+#pragma unroll
+    for (uint32_t j = 0; j < 16; ++j)
+        best = fmaxf(best, wv[j]);
+    const uint32_t bkey = order_key(best);
+    const bool emits = cls == kTopK || cls == kNucleus;
+    const uint32_t wmax = __ockl_wfred_max_u32(bkey);
+    uint32_t wkth = 0;
+    if (emits) {
+        // Every logit that can be among the row's K largest is among this slice's K largest.  Each wave
+        // takes the ceil(K/16)-th largest of its per-thread maxima; at least K logits of the slice are >= the
+        // smallest of those 16 values, which becomes the emission threshold.
+        const uint32_t K = cls == kTopK ? P.top_k : kTopKFast;
+        wkth = wave_kth_largest(bkey, (K + kWaves - 1) / kWaves);
+    }
+    if (lane_id() == 0) {
+        sm.wave_max[wave_id()] = wmax;
+        sm.wave_kth[wave_id()] = wkth;
+        if (ABOVE)
+            sm.wave_above[wave_id()] = above;
+    }
+    __syncthreads();
+    MAKO_STAMP(30);
+    uint32_t mkey = 0, tau_key = 0xffffffffu, above_slice = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        mkey = max(mkey, sm.wave_max[w]);
+        tau_key = min(tau_key, sm.wave_kth[w]);
+        if (ABOVE)
+            above_slice += sm.wave_above[w];
+    }
+    // first index holding the maximum
+    if (bkey == mkey) {
+        const float M = order_unkey(mkey);
+        uint32_t first = kNone;
+#pragma unroll
+        for (int j = 15; j >= 0; --j)
+            if (wv[j] == M)
+                first = elem_index<VEC>(lo, tid, (uint32_t)j);
+        if (first != kNone)
+            atomicMin(&sm.argidx, first);
+    }
+
+    SliceStat st;
+    st.wmax = order_unkey(mkey);
+    st.flags = 0;
+    st.n_emit = 0;
+    st.tau_key = 0;
+    st.above = above_slice;
+    st.pad[0] = st.pad[1] = 0;
+    // element 0 of the row is NaN: its holder raises the flag
+    const bool first_nan = slice == 0 && tid == 0 && wv[0] != wv[0];
+    if (first_nan)
+        atomicOr(&sm.emit_flags, kFlagFirstNan);
+
+    if (emits) {
+        if (tau_key <= kKeyNegInf) {
+            tau_key = kKeyNegInf;
+            st.flags |= kFlagComplete;
+        }
+        // w >= tau and w > -inf in one compare: -inf itself is below the most negative finite float
+        const float tau = fmaxf(order_unkey(tau_key), -3.402823466e38f);
+        // slots in the slice's list: the wave counts its candidates, one lane reserves the wave's run with a single
+        // LDS atomic, and every thread fills its part of the run (one atomic per candidate cost a round trip each)
+        uint32_t mine = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j)
+            mine += wv[j] >= tau ? 1u : 0u;
+        const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
+        const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)upto, kWave - 1);
+        if (wave_total) { // uniform
+            uint32_t base = 0;
+            if (lane_id() == 0)
+                base = atomicAdd(&sm.emit_n, wave_total);
+            uint32_t pos = (uint32_t)__builtin_amdgcn_readfirstlane((int)base) + upto - mine;
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j) {
+                const float w = wv[j];
+                const bool take = w >= tau;
+                if (take && pos < kCap) {
+                    sm.cw[pos] = w;
+                    sm.ci[pos] = elem_index<VEC>(lo, tid, j);
+                }
+                pos += take ? 1u : 0u;
+            }
+        }
+    }
+    __syncthreads();
+    MAKO_STAMP(31);
+    if (emits) {
+        const uint32_t n = sm.emit_n;
+        if (n > kCap)
+            st.flags |= kFlagOverflow;
+        st.n_emit = min(n, kCap);
+        st.tau_key = tau_key;
+        const size_t base = ((size_t)row * sc.slices_cap + slice) * kCap;
+        if (tid < st.n_emit) {
+            sc.cand_w[base + tid] = sm.cw[tid];
+            sc.cand_i[base + tid] = sm.ci[tid];
+        }
+    }
+    if (tid == 0) {
+        st.argidx = sm.argidx;
+        st.flags |= sm.emit_flags;
+        sc.stats[(size_t)row * kMaxSlices + slice] = st;
+    }
+    MAKO_STAMP(27);
+}
+
+} // namespace mako

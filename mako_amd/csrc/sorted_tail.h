@@ -1,0 +1,1088 @@
+// Sorted candidate lists: top-p cut, exact fp32 total and walk in groups of 256 entries.
+#pragma once
+
+#include "generic_replay.h"
+
+namespace mako {
+
+constexpr uint32_t kWalkSeqGroups = 8; // a walk expected to end within this many groups goes entry by entry from LDS
+struct GroupLds { // carved from the dynamic LDS block once sorting is over; one pointer, the rest is offsets
+    unsigned long long* base;
+    __device__ __forceinline__ double* pg() const { return reinterpret_cast<double*>(base); } // [kMaxGroups + 2] fp64 sum of the entries before each group
+    __device__ __forceinline__ uint32_t* d0() const { return reinterpret_cast<uint32_t*>(base + kMaxGroups + 2); } // [kMaxGroups] the group's map for the guessed epoch
+    __device__ __forceinline__ uint32_t* d1() const { return d0() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* cmax() const { return d1() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* start() const { return cmax() + kMaxGroups; } // first entry of the group
+    // entries (bits 0-8) | quarter-record slot + 1 (bits 9-15) | guessed exponent << 16
+    __device__ __forceinline__ uint32_t* pack() const { return start() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* misc() const { return pack() + kMaxGroups; } // [4]; misc[3] counts the quarter-record slots in use
+    // [kQuarterSlots][4], in the upper half of the dynamic LDS block
+    __device__ __forceinline__ uint4* quarters() const { return reinterpret_cast<uint4*>(base + kSortMax); }
+    // the walk's maps, bounds and packs ([kMaxGroups] each, behind the quarter records): built while the running
+    // sum is still being chained, so they cannot share the arrays above
+    __device__ __forceinline__ uint32_t* w_d0() const { return reinterpret_cast<uint32_t*>(base + kSortMax) + 1536; }
+    __device__ __forceinline__ uint32_t* w_d1() const { return w_d0() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* w_need() const { return w_d1() + kMaxGroups; }
+    __device__ __forceinline__ uint32_t* w_pack() const { return w_need() + kMaxGroups; }
+    // [kWalkSeqGroups * kGroup + kWave] the head of the list as floats, for a walk that ends within it
+    __device__ __forceinline__ float* head() const { return reinterpret_cast<float*>(w_pack() + kMaxGroups); }
+};
+constexpr uint32_t kLenMask = 0x1ffu;
+constexpr uint32_t kHasQuarters = 1u << 31;
+constexpr uint32_t kQuarterSlots = 96;
+constexpr uint32_t kQuarter = kGroup / 4;
+constexpr uint32_t kSeqMax = 1024; // sorted lists up to this long get their total and walk entry by entry
+
+__device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
+{
+    static_assert((kMaxGroups + 2) * 8 + 5 * kMaxGroups * 4 + 16 <= kSortMax * 8, "group records fit below the LDS lists");
+    static_assert(kQuarterSlots * 16 == 1536 &&
+                      kSortMax * 8 + 1536 * 4 + 4 * kMaxGroups * 4 + (kWalkSeqGroups * kGroup + kWave) * 4 <= kDynLds,
+                  "the walk's records sit behind the quarter records and fit the dynamic LDS block");
+    return GroupLds{L.sortk};
+}
+
+// Values every lane of the wave holds alike, moved to scalar registers so that loops and branches on them
+// compile to scalar control flow.
+// A double from a lane whose number is the same for the whole wave.
+__device__ __forceinline__ double readlane_f64(double v, uint32_t lane)
+{
+    const long long b = __double_as_longlong(v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, (int)lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), (int)lane);
+    return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
+__device__ __forceinline__ uint32_t uniform_u32(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
+}
+
+// Cross-lane moves on the VALU data path (DPP) instead of through the LDS crossbar: a dependent chain of six
+// of them costs tens of cycles, not hundreds.  Lanes without a source lane receive 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_or_zero(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+
+// Inclusive scan, in lane order, of the 64 lanes' maps under composition (cmax is not touched).
+__device__ __forceinline__ void wave_scan_maps(uint32_t& d0, uint32_t& d1)
+{
+    using seqfp::Step32;
+#define MAKO_SCAN_STEP(CTRL, ROW_MASK)                                                                               \
+    {                                                                                                                \
+        const Step32 t = Step32{dpp_or_zero<CTRL, ROW_MASK>(d0), dpp_or_zero<CTRL, ROW_MASK>(d1), 0u};               \
+        const Step32 r = seqfp::compose32(t, Step32{d0, d1, 0u}); /* earlier lanes first; {0, 0} is the identity */  \
+        d0 = r.d0;                                                                                                   \
+        d1 = r.d1;                                                                                                   \
+    }
+    MAKO_SCAN_STEP(0x111, 0xf) // row_shr:1
+    MAKO_SCAN_STEP(0x112, 0xf) // row_shr:2
+    MAKO_SCAN_STEP(0x114, 0xf) // row_shr:4
+    MAKO_SCAN_STEP(0x118, 0xf) // row_shr:8
+    MAKO_SCAN_STEP(0x142, 0xa) // row_bcast:15 into rows 1 and 3
+    MAKO_SCAN_STEP(0x143, 0xc) // row_bcast:31 into rows 2 and 3
+#undef MAKO_SCAN_STEP
+}
+
+__device__ __forceinline__ int exponent_of(float x)
+{
+    uint32_t M;
+    int e;
+    seqfp::split(x, M, e);
+    return e;
+}
+
+// A sorted list's keys, wherever they are (LDS or device memory: loads through a generic pointer, which the
+// hardware completes in no particular order, so that the code has to wait for all of them at once) ...
+struct AnyKeys {
+    const uint32_t* p;
+    __device__ __forceinline__ uint32_t operator[](uint32_t i) const { return p[i]; }
+    __device__ __forceinline__ uint4 vec(uint32_t i) const { return *reinterpret_cast<const uint4*>(p + i); }
+};
+// ... or known to be in device memory: plain global loads, which can be left in flight and waited for one by one.
+struct GlobalKeys {
+    const uint32_t* p;
+    __device__ __forceinline__ uint32_t operator[](uint32_t i) const
+    {
+        return ((const __attribute__((address_space(1))) uint32_t*)p)[i];
+    }
+    __device__ __forceinline__ uint4 vec(uint32_t i) const
+    {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 v = *((const __attribute__((address_space(1))) u32x4*)(p + i));
+        return make_uint4(v.x, v.y, v.z, v.w);
+    }
+};
+
+// The four weights a lane owns in the span of `len` (<= kGroup) entries that starts at kf[start]: entries
+// 4 * lane .. 4 * lane + 3, 0.0f past the end.  kf itself is 16-byte aligned.
+template <typename Keys>
+__device__ __forceinline__ void load_span(Keys kf, uint32_t start, uint32_t len, float (&q)[4])
+{
+    const uint32_t i = lane_id() * 4u;
+    uint32_t k[4] = {0u, 0u, 0u, 0u}; // bits(0.0f)
+    if ((start & 3u) == 0 && i + 3 < len) {
+        const uint4 x = kf.vec(start + i);
+        k[0] = ~x.x;
+        k[1] = ~x.y;
+        k[2] = ~x.z;
+        k[3] = ~x.w;
+    } else if (len) {
+        // (every load from a position inside the span, and what lies past the end masked with an AND: a select
+        // would be turned into a branch around each load, and each would wait for the one before)
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            k[j] = ~kf[start + min(i + j, len - 1u)] & (i + j < len ? 0xffffffffu : 0u);
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j)
+        q[j] = __uint_as_float(k[j]);
+}
+__device__ __forceinline__ void load_span(const uint32_t* kf, uint32_t start, uint32_t len, float (&q)[4])
+{
+    load_span(AnyKeys{kf}, start, len, q);
+}
+
+// Composition of the 64 lanes' maps in lane order; every lane receives the result.
+__device__ __forceinline__ seqfp::Step32 wave_compose_step32(seqfp::Step32 v)
+{
+    wave_scan_maps(v.d0, v.d1);
+    seqfp::Step32 r;
+    r.d0 = (uint32_t)__builtin_amdgcn_readlane((int)v.d0, kWave - 1);
+    r.d1 = (uint32_t)__builtin_amdgcn_readlane((int)v.d1, kWave - 1);
+    r.cmax = __ockl_wfred_max_u32(v.cmax);
+    return r;
+}
+
+// The map of one span for the epoch with exponent eg (eg == 0: no usable guess, the map is marked unusable).
+__device__ __forceinline__ seqfp::Step32 span_map(const float (&q)[4], uint32_t len, int eg)
+{
+    using namespace seqfp;
+    Step32 st = Step32{kSat, kSat, kSat};
+    if (eg > 0) { // uniform per wave
+        st = identity32();
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (lane_id() * 4u + j < len)
+                st = compose32(st, step32(q[j], eg));
+        st = wave_compose_step32(st);
+    }
+    return st;
+}
+
+// A group inside which the running sum is expected to change binade cannot be applied as one map.  Its four
+// quarters (64 entries = the 16 lanes of one DPP row each) get maps of their own, each for the binade guessed from
+// the fp64 sum up to ITS first entry: the chain then replays only the quarter in which the change happens.
+// `at_start` is the estimate of the sum at the group's first entry.  One wave; the four records (d0, d1, cmax,
+// exponent) go to out[0..3].
+__device__ void build_quarters(const float (&q)[4], uint32_t len, double at_start, uint4* out)
+{
+    using namespace seqfp;
+    const uint32_t lane = lane_id(), quarter = lane >> 4;
+    double rs = (((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3];
+    for (int o = 1; o < 16; o <<= 1)
+        rs += __shfl_xor(rs, o);
+    const double s0 = __shfl(rs, 0), s1 = __shfl(rs, 16), s2 = __shfl(rs, 32);
+    const double before = quarter == 0 ? 0.0 : (quarter == 1 ? s0 : (quarter == 2 ? s0 + s1 : (s0 + s1) + s2));
+    const double guess = at_start + before;
+    const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+    Step32 v = Step32{kSat, kSat, kSat};
+    if (eg > 0) {
+        v = identity32();
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (lane * 4u + j < len)
+                v = compose32(v, step32(q[j], eg));
+    }
+    uint32_t cm = v.cmax;
+    for (int o = 1; o < 16; o <<= 1)
+        cm = max(cm, (uint32_t)__shfl_xor((int)cm, o));
+    // inclusive scan inside the row of 16 lanes
+#define MAKO_ROW_STEP(CTRL)                                                                                          \
+    {                                                                                                                \
+        const Step32 t = Step32{dpp_or_zero<CTRL, 0xf>(v.d0), dpp_or_zero<CTRL, 0xf>(v.d1), 0u};                     \
+        const Step32 r = compose32(t, Step32{v.d0, v.d1, 0u});                                                       \
+        v.d0 = r.d0;                                                                                                 \
+        v.d1 = r.d1;                                                                                                 \
+    }
+    MAKO_ROW_STEP(0x111)
+    MAKO_ROW_STEP(0x112)
+    MAKO_ROW_STEP(0x114)
+    MAKO_ROW_STEP(0x118)
+#undef MAKO_ROW_STEP
+    if ((lane & 15u) == 15u)
+        out[quarter] = make_uint4(v.d0, v.d1, cm, (uint32_t)eg);
+}
+
+// Group maps of groups [0, groups) for epochs guessed from pg: of the running sum (walk == false, into G.d0 / d1 /
+// cmax / pack) or of the walk from r0 (into G.w_d0 / w_d1 / w_need / w_pack).  The calling wave is number `part` of
+// `parts` that share the work.
+template <typename Keys>
+__device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0, const GroupLds G,
+                                 uint32_t part = wave_id(), uint32_t parts = kWaves)
+{
+    using namespace seqfp;
+    uint32_t* const o_d0 = walk ? G.w_d0() : G.d0();
+    uint32_t* const o_d1 = walk ? G.w_d1() : G.d1();
+    uint32_t* const o_c = walk ? G.w_need() : G.cmax();
+    uint32_t* const o_pack = walk ? G.w_pack() : G.pack();
+    // Up to four groups per trip and wave, their loads issued together; a wave's groups lie `parts` apart, so that a
+    // short list is spread over all the waves (a map costs a wave about a microsecond).
+    for (uint32_t g0 = part; g0 < groups; g0 += parts * 4u) {
+        float q[4][4];
+        uint32_t len[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t g = min(g0 + u * parts, groups - 1u);
+            len[u] = uniform_u32(G.pack()[g] & kLenMask);
+            load_span(kf, uniform_u32(G.start()[g]), len[u], q[u]);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t g = g0 + u * parts;
+            if (g >= groups) // uniform
+                break;
+            const double guess = g < groups ? (walk ? r0 - G.pg()[g] : G.pg()[g]) : 0.0;
+            const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+            const Step32 st = span_map(q[u], len[u], eg);
+            // a group in which the running sum is expected to change binade (or starts from zero) gets quarter
+            // records; the walk replays such groups whole
+            uint32_t slot = 0;
+            if (!walk && g < groups) { // uniform
+                const double at_end = G.pg()[g + 1];
+                const int e_end = at_end > 0 ? exponent_of((float)at_end) : 0;
+                if (uniform_u32((uint32_t)(e_end != eg)) || g == 0) {
+                    if (lane_id() == 0)
+                        slot = atomicAdd(&G.misc()[3], 1u) + 1u;
+                    slot = uniform_u32(slot);
+                    if (slot > kQuarterSlots)
+                        slot = 0;
+                    else
+                        build_quarters(q[u], len[u], G.pg()[g], G.quarters() + (slot - 1u) * 4u);
+                }
+            }
+            if (lane_id() == 0 && g < groups) {
+                uint32_t third = st.cmax;
+                if (walk) {
+                    // group_sub_ok as one bound (lane 0 holds the group's first, largest weight): the state after
+                    // the group must be at least `third`, which keeps it inside the binade with room for one
+                    // more decrement and at or above that weight, so that nothing in the group stopped the walk
+                    uint32_t Mq;
+                    int eq;
+                    split(q[u][0], Mq, eq);
+                    const int dl = eg - eq;
+                    third = 1u;
+                    if (dl < 0)
+                        third = 1u << 31;
+                    else if (dl <= 25)
+                        third = max(1u, (uint32_t)(((unsigned long long)Mq + (1ull << dl) - 1ull) >> dl));
+                    if (eg > 1)
+                        third = max(third, min(st.cmax, 1u << 30) + (1u << 23) + 1u);
+                }
+                o_d0[g] = st.d0;
+                o_d1[g] = st.d1;
+                o_c[g] = third;
+                o_pack[g] = len[u] | (slot << 9) | ((uint32_t)eg << 16);
+            }
+        }
+    }
+}
+
+// The entries of one span (at most 256), one per lane and register: x[j] of lane l is entry 64 * j + l, 0.0f past
+// the end.
+template <typename Keys>
+__device__ __forceinline__ void load_span_lanes(Keys kf, uint32_t start, uint32_t len, float (&x)[4])
+{
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j) {
+        const uint32_t i = j * kWave + lane_id();
+        // (every lane loads, from inside the span; masked with an AND, as in load_span)
+        x[j] = __uint_as_float(~kf[start + min(i, len - 1u)] & (i < len ? 0xffffffffu : 0u));
+    }
+}
+// The same in two steps, for loads that are to stay in flight while other work goes on: the words as loaded
+// (nothing touches them here), and their conversion once they are wanted.
+template <typename Keys>
+__device__ __forceinline__ void fetch_span_lanes(Keys kf, uint32_t start, uint32_t len, uint32_t (&raw)[4])
+{
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j)
+        raw[j] = kf[start + min(j * kWave + lane_id(), len - 1u)];
+}
+__device__ __forceinline__ void take_span_lanes(const uint32_t (&raw)[4], uint32_t len, float (&x)[4])
+{
+#pragma unroll
+    for (uint32_t j = 0; j < 4; ++j)
+        x[j] = __uint_as_float(~raw[j] & (j * kWave + lane_id() < len ? 0xffffffffu : 0u));
+}
+
+// One step of a chain that travels across the lanes: every lane takes the value of the lane below it (lane 0:
+// of lane 63) and subtracts / adds its own entry.  Started from a uniform value, lane t holds after t + 1 steps
+// the value a sequential loop would hold after entries 0..t; the other lanes hold values nobody reads.  One
+// dependent instruction per entry, where a broadcast per entry costs three.
+__device__ __forceinline__ float ror_sub(float v, float x)
+{
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), 0x13C /* wave_ror:1 */,
+                                                                 0xf, 0xf, false)) - x;
+}
+__device__ __forceinline__ float ror_add(float v, float x)
+{
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), 0x13C /* wave_ror:1 */,
+                                                                 0xf, 0xf, false)) + x;
+}
+
+// S plus the entries of one span (len in 1..256), added one by one in fp32 (src/gen/sampler.cpp:80-82).  One wave.
+template <typename Keys>
+__device__ float exact_span_sum(Keys kf, uint32_t start, uint32_t len, float S)
+{
+    float x[4];
+    const uint32_t n = uniform_u32(len);
+    if (n == 0)
+        return S;
+    load_span_lanes(kf, uniform_u32(start), n, x);
+    float v = S; // uniform
+    for (uint32_t base = 0; base < n; base += kWave) {
+        const float cur = x[0];
+        for (uint32_t b = 0; b < kWave && base + b < n; b += 16u) {
+#pragma unroll
+            for (uint32_t k = 0; k < 16; ++k)
+                v = ror_add(v, cur);
+        }
+        x[0] = x[1];
+        x[1] = x[2];
+        x[2] = x[3];
+    }
+    // entries past the end added 0.0f: the lane of the last step holds the sum
+    const uint32_t steps = (n + 15u) & ~15u;
+    return __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), (steps - 1u) & 63u));
+}
+
+// The entries of one span (n in 1..256, in registers as load_span_lanes() leaves them; the span starts at entry
+// `beg` of the list) subtracted from r one by one (src/gen/sampler.cpp:67-71).  Returns true and the entry's
+// position in the list when the walk stops inside the span, else false and the new r.  One wave.
+//
+// The walk stops at the first entry with r < x, which is the first entry whose subtraction turns r negative (x != r
+// gives a nonzero difference, denormals kept), and a negative r stays negative under every later subtraction of a
+// weight.  So 64 entries are subtracted without looking; only a block that ends negative is gone through again,
+// sixteen entries at a time, and the sixteen that turn r negative one by one.
+__device__ __forceinline__ bool walk_lanes(float (&x)[4], uint32_t n, uint32_t beg, float& r, uint32_t& pos)
+{
+    float v = r;    // uniform
+    float r_in = r; // the walk's value in front of the current block
+    for (uint32_t base = 0; base < n; base += kWave) {
+        const float cur = x[0];
+        const bool whole = n - base > 48u; // (a short rest goes sixteen at a time straight away)
+        uint32_t out = 0x80000000u;
+        if (whole) {
+#pragma unroll
+            for (uint32_t k = 0; k < kWave; ++k)
+                v = ror_sub(v, cur);
+            out = (uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), kWave - 1);
+        }
+        if (out >> 31) {
+            v = r_in;
+            for (uint32_t b = 0; b < kWave && base + b < n; b += 16u) {
+#pragma unroll
+                for (uint32_t k = 0; k < 16; ++k)
+                    v = ror_sub(v, cur);
+                const uint32_t o16 = (uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), (b + 15u) & 63u);
+                if (o16 >> 31) {
+                    float rr = r_in;
+                    for (uint32_t l = b; l < b + 16u; ++l) {
+                        const float xv =
+                            __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(cur), l & 63u));
+                        if (__ballot(rr < xv) != 0ull) {
+                            pos = beg + base + l;
+                            return true;
+                        }
+                        rr -= xv;
+                    }
+                }
+                r_in = __uint_as_float(o16);
+            }
+        }
+        if (whole)
+            r_in = __uint_as_float(out);
+        x[0] = x[1];
+        x[1] = x[2];
+        x[2] = x[3];
+    }
+    r = r_in;
+    return false;
+}
+
+template <typename Keys>
+__device__ bool exact_span_walk(Keys kf, uint32_t start, uint32_t len, float& r, uint32_t& pos)
+{
+    float x[4];
+    const uint32_t n = uniform_u32(len);
+    const uint32_t beg = uniform_u32(start);
+    if (n == 0)
+        return false;
+    load_span_lanes(kf, beg, n, x);
+    return walk_lanes(x, n, beg, r, pos);
+}
+
+// The walk over the first `n` entries of the list, staged in LDS as floats (16-byte aligned): every lane of the
+// wave reads the same four entries with one broadcast load and subtracts them in turn, three nanoseconds an entry
+// (the travelling chain of walk_lanes() takes five).  Blocks of 64 blind, then of 16, then entry by entry, as there.
+// Returns true and the position when the walk stops, else false and the new r.
+__device__ __forceinline__ bool walk_lds(const float* sx, uint32_t n, float& r, uint32_t& pos)
+{
+    float v = r;
+    uint32_t base = 0;
+    for (; base + kWave <= n; base += kWave) {
+        const float4* p = reinterpret_cast<const float4*>(sx + base);
+        float t = v;
+#pragma unroll
+        for (uint32_t i = 0; i < kWave / 4u; ++i) {
+            const float4 x = p[i];
+            t -= x.x;
+            t -= x.y;
+            t -= x.z;
+            t -= x.w;
+        }
+        if (__ballot(t < 0.0f) != 0ull)
+            break; // the walk stops in this block: found below
+        v = t;
+    }
+    for (; base + 16u <= n; base += 16u) {
+        const float4* p = reinterpret_cast<const float4*>(sx + base);
+        float t = v;
+#pragma unroll
+        for (uint32_t i = 0; i < 4u; ++i) {
+            const float4 x = p[i];
+            t -= x.x;
+            t -= x.y;
+            t -= x.z;
+            t -= x.w;
+        }
+        if (__ballot(t < 0.0f) != 0ull)
+            break;
+        v = t;
+    }
+    for (const uint32_t end = min(n, base + 16u); base < end; ++base) {
+        const float x = sx[base];
+        if (__ballot(v < x) != 0ull) {
+            pos = base;
+            return true;
+        }
+        v -= x;
+    }
+    r = v;
+    return false;
+}
+
+// S plus the first `n` entries of a list staged in LDS as for walk_lds(), added one by one in fp32.
+__device__ __forceinline__ float sum_lds(const float* sx, uint32_t n, float S)
+{
+    uint32_t base = 0;
+    for (; base + 16u <= n; base += 16u) {
+        const float4* p = reinterpret_cast<const float4*>(sx + base);
+#pragma unroll
+        for (uint32_t i = 0; i < 4u; ++i) {
+            const float4 x = p[i];
+            S += x.x;
+            S += x.y;
+            S += x.z;
+            S += x.w;
+        }
+    }
+    for (; base < n; ++base)
+        S += sx[base];
+    return S;
+}
+
+// State of a chain between groups: significand and exponent of the running value, and where the walk stopped.
+struct ChainState {
+    uint32_t M;
+    int e;
+    uint32_t pos; // kNone while the walk goes on
+};
+
+// One group applied to the running sum quarter by quarter (records at `rec`), replaying only the quarters whose
+// map does not apply.  One wave.  (State by value: the chain keeps it in scalar registers.)
+template <typename Keys>
+__device__ __forceinline__ ChainState sum_by_quarters(Keys kf, uint32_t st, uint32_t len, const uint4* rec, ChainState c)
+{
+    using namespace seqfp;
+#pragma unroll 1
+    for (uint32_t k = 0; k < 4u; ++k) {
+        if (k * kQuarter < len) { // uniform
+            const uint4 r = rec[k];
+            const uint32_t d0 = uniform_u32(r.x), d1 = uniform_u32(r.y), cm = uniform_u32(r.z), eg = uniform_u32(r.w);
+            const uint32_t dd = (c.M & 1u) ? d1 : d0;
+            const uint32_t lim = cm >= (1u << 24) - 1u ? 0u : (1u << 24) - 1u - cm;
+            if ((uint32_t)c.e == eg && c.M + dd < lim) {
+                c.M += dd;
+            } else {
+                const float S = exact_span_sum(kf, st + k * kQuarter, min(kQuarter, len - k * kQuarter), join(c.M, c.e));
+                uint32_t Mv;
+                int ev;
+                split(S, Mv, ev);
+                c.M = uniform_u32(Mv);
+                c.e = (int)uniform_u32((uint32_t)ev);
+            }
+        }
+    }
+    return c;
+}
+
+// Tail of every path that ends with a list sorted by (q desc, idx asc): kf[i] = ~bits(q_i), jf[i] = token id,
+// n1 entries (already cut to top_k).  Applies top-p (src/gen/sampler.cpp:44-61) against total64 (the fp64 sum over
+// the row's candidates; summed from the list when !have_total), then the exact fp32 total (:80-82) and walk
+// (:64-73).  All 1024 threads must call it.
+//
+// When `need_cut` the list is only the heaviest part of the row's candidates and every candidate missing from
+// it weighs at most q_bound: the nucleus must then end inside the list, at an entry strictly heavier than
+// q_bound.  If it does not, nothing is written and false is returned (the caller widens the list).
+//
+// `T` (with `t_groups` records at `t_base`) describes a list whose groups were prepared by sort_kernel's workers;
+// without it the list is cut into groups of kGroup here.
+// SHORT_ONLY: the caller's lists never exceed kGroup entries; the code for longer ones is left out.
+template <bool PLANNED = false, bool SHORT_ONLY = false>
+__device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf_ptr,
+                            const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
+                            const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, const GroupTable& T = GroupTable{},
+                            size_t t_base = 0, uint32_t t_groups = 0)
+{
+    using namespace seqfp;
+    // (a planned row's list is in device memory; the other callers may hand over a list in LDS)
+    const typename std::conditional<PLANNED, GlobalKeys, AnyKeys>::type kf{kf_ptr};
+    const float u_row = d.u[row]; // (asked for here, wanted much later)
+    const uint32_t n1 = uniform_u32(n1_arg);
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    auto qat = [=](uint32_t i) { return __uint_as_float(~kf[i]); };
+    auto idat = [=](uint32_t i) { return jf[i]; };
+    const GroupLds G = group_lds(L);
+    const bool topp_active = P.top_p < 1.0f;
+    if (d.draft || (!PLANNED && n1 > kGroup * kMaxGroups)) {
+        // verification and oversized lists take the generic windowed replay
+        uint32_t n = n1;
+        if (topp_active) {
+            if (!have_total) {
+                double part = 0;
+                for (uint32_t i = tid; i < n; i += kThreads)
+                    part += (double)qat(i);
+                total64 = block_sum_f64(part, sm.bs);
+            }
+            const double want = (double)P.top_p * total64;
+            double carry = 0;
+            uint32_t keep = kNone;
+            for (uint32_t base = 0; base < n; base += kThreads) {
+                const uint32_t i = base + tid;
+                const double q = i < n ? (double)qat(i) : 0.0;
+                double tile;
+                const double incl = carry + block_incl_scan_f64(q, tile, sm.bs);
+                const uint32_t hit = (i < n && incl >= want) ? i : kNone;
+                const uint32_t first = block_min_u32(hit, sm.bs);
+                if (first != kNone) {
+                    keep = first + 1;
+                    break;
+                }
+                carry += tile;
+            }
+            if (need_cut && keep == kNone)
+                return false;
+            n = keep == kNone ? n : keep;
+        }
+        if (need_cut && !(q_bound < qat(n - 1)))
+            return false;
+        draw_from_list(d, row, qat, idat, n, path, sm);
+        return true;
+    }
+
+    if (!PLANNED && n1 <= kGroup) {
+        // short list: one wave does everything, the chain of fp32 roundings replayed with real additions
+        MAKO_STAMP(5);
+        __syncthreads(); // the list is published; sm.flag is free
+        if (wave_id() == 0) {
+            float q[4];
+            load_span(kf, 0, n1, q);
+            double p[4];
+            p[0] = (double)q[0];
+            p[1] = p[0] + (double)q[1];
+            p[2] = p[1] + (double)q[2];
+            p[3] = p[2] + (double)q[3];
+            const double incl = __ockl_wfscan_add_f64(p[3], true);
+            if (!have_total)
+                total64 = readlane_f64(incl, kWave - 1);
+            uint32_t n = n1;
+            bool ok = true;
+            if (topp_active) {
+                const double want = (double)P.top_p * total64;
+                const double base = incl - p[3];
+                uint32_t hit = kNone;
+#pragma unroll
+                for (int j = 3; j >= 0; --j)
+                    if (base + p[j] >= want)
+                        hit = lane_id() * 4u + (uint32_t)j;
+                const unsigned long long bal = __ballot(hit != kNone && hit < n1);
+                if (bal)
+                    n = (uint32_t)__builtin_amdgcn_readlane((int)hit, __ffsll((long long)bal) - 1) + 1u;
+                else
+                    ok = !need_cut;
+            }
+            if (ok && need_cut && !(q_bound < qat(n - 1)))
+                ok = false;
+            if (ok) {
+                const float total = exact_span_sum(kf, 0, n, 0.0f);
+                const float span = total - 0.0f;
+                const float prod = u_row * span;
+                float r = prod + 0.0f;
+                uint32_t pos = n - 1;
+                if (r < 0.0f)
+                    pos = 0;
+                else if (r == r && r != INFINITY)
+                    exact_span_walk(kf, 0, n, r, pos);
+                if (d.out_cand_idx && d.out_cand_q)
+                    for (uint32_t j = lane_id(); j < n && j < d.cand_cap; j += kWave) {
+                        d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
+                        d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
+                    }
+                if (lane_id() == 0) {
+                    RowOut o;
+                    o.token = (int32_t)idat(pos);
+                    o.n_cand = n;
+                    o.total = total;
+                    o.q = qat(pos);
+                    o.path = path;
+                    o.accepted = 0;
+                    write_row(d, row, o);
+                }
+            }
+            if (lane_id() == 0)
+                sm.flag = ok;
+        }
+        __syncthreads();
+        MAKO_STAMP(9);
+        return sm.flag != 0;
+    }
+    if constexpr (SHORT_ONLY)
+        return false; // (not reached)
+
+    // group records: fp64 sums (and, from the workers, the maps of the running sum)
+    MAKO_STAMP(5);
+    const uint32_t groups1 = PLANNED ? t_groups : (n1 + kGroup - 1) / kGroup;
+    if (tid == 0)
+        G.misc()[3] = 0;
+    // The head of the list as floats in LDS (loads set out now, wanted after the cut): where the running sum and
+    // the walk change binade every few entries, both go through it entry by entry.
+    constexpr uint32_t kHead = kWalkSeqGroups * kGroup;
+    {
+        uint32_t raw[kHead / kThreads];
+#pragma unroll
+        for (uint32_t t = 0; t < kHead / kThreads; ++t)
+            raw[t] = kf[min(t * kThreads + tid, n1 - 1u)];
+#pragma unroll
+        for (uint32_t t = 0; t < kHead / kThreads; ++t)
+            G.head()[t * kThreads + tid] = __uint_as_float(~raw[t] & (t * kThreads + tid < n1 ? 0xffffffffu : 0u));
+        if (tid < kWave)
+            G.head()[kHead + tid] = 0.0f;
+    }
+    __syncthreads();
+    if constexpr (PLANNED) {
+        if (tid < groups1) {
+            G.pg()[tid + 1] = T.sum[t_base + tid];
+            G.d0()[tid] = T.d0[t_base + tid];
+            G.d1()[tid] = T.d1[t_base + tid];
+            G.cmax()[tid] = T.cmax[t_base + tid];
+            // (clamped into the list: a record is only ever read, never trusted for addressing)
+            const uint32_t st = min(T.start[t_base + tid], n1), pk = T.pack[t_base + tid];
+            // (the quarter records are asked for together with the rest, whether or not the group has any: asking
+            // only once `pk` is known would be one more trip to memory for every row)
+            const uint4* tq = T.quarters + (t_base + tid) * 4u;
+            const uint4 qr0 = tq[0], qr1 = tq[1], qr2 = tq[2], qr3 = tq[3];
+            uint32_t slot = 0;
+            if (pk & kHasQuarters) {
+                slot = atomicAdd(&G.misc()[3], 1u) + 1u;
+                if (slot > kQuarterSlots)
+                    slot = 0;
+            }
+            if (slot) {
+                uint4* gq = G.quarters() + (slot - 1u) * 4u;
+                gq[0] = qr0;
+                gq[1] = qr1;
+                gq[2] = qr2;
+                gq[3] = qr3;
+            }
+            G.start()[tid] = st;
+            G.pack()[tid] = min(pk & kLenMask, min(kGroup, n1 - st)) | (slot << 9) | (pk & 0x00ff0000u);
+        }
+    } else {
+        if (tid < groups1) {
+            G.start()[tid] = tid * kGroup;
+            G.pack()[tid] = min(kGroup, n1 - tid * kGroup);
+        }
+        for (uint32_t g0 = wave_id() * 4u; g0 < groups1; g0 += kWaves * 4u) {
+            float q[4][4];
+#pragma unroll
+            for (uint32_t u = 0; u < 4; ++u) {
+                const uint32_t g = min(g0 + u, groups1 - 1u);
+                load_span(kf, g * kGroup, min(kGroup, n1 - g * kGroup), q[u]);
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 4; ++u) {
+                const double s = __ockl_wfred_add_f64((((double)q[u][0] + (double)q[u][1]) + (double)q[u][2]) + (double)q[u][3]);
+                if (lane_id() == 0 && g0 + u < groups1)
+                    G.pg()[g0 + u + 1] = s;
+            }
+        }
+    }
+    __syncthreads();
+    {
+        const double v = tid < groups1 ? G.pg()[tid + 1] : 0.0;
+        double all;
+        const double incl = block_incl_scan_f64(v, all, sm.bs);
+        if (tid < groups1)
+            G.pg()[tid + 1] = incl;
+        if (tid == 0)
+            G.pg()[0] = 0.0;
+        if (!have_total)
+            total64 = all;
+    }
+    __syncthreads();
+
+    // top-p: first entry at which the running fp64 sum reaches top_p * total
+    MAKO_STAMP(6);
+    uint32_t n = n1, groups = uniform_u32(groups1);
+    if (topp_active) {
+        const double want = (double)P.top_p * total64;
+        const uint32_t hitg = (tid < groups1 && G.pg()[tid + 1] >= want) ? tid : kNone;
+        const uint32_t gs = block_min_u32(hitg, sm.bs);
+        if (need_cut && gs == kNone)
+            return false;
+        if (gs != kNone) {
+            if (wave_id() == 0) {
+                const uint32_t st = G.start()[gs], len = G.pack()[gs] & kLenMask;
+                float q[4];
+                load_span(kf, st, len, q);
+                double p[4];
+                p[0] = (double)q[0];
+                p[1] = p[0] + (double)q[1];
+                p[2] = p[1] + (double)q[2];
+                p[3] = p[2] + (double)q[3];
+                const double incl = __ockl_wfscan_add_f64(p[3], true);
+                const double base = G.pg()[gs] + (incl - p[3]);
+                uint32_t hit = kNone;
+#pragma unroll
+                for (int j = 3; j >= 0; --j)
+                    if (base + p[j] >= want)
+                        hit = lane_id() * 4u + (uint32_t)j;
+                const unsigned long long bal = __ballot(hit != kNone && hit < len);
+                uint32_t keep = len;
+                if (bal)
+                    keep = (uint32_t)__builtin_amdgcn_readlane((int)hit, __ffsll((long long)bal) - 1) + 1u;
+                if (lane_id() == 0) {
+                    G.misc()[0] = st + keep;
+                    if (keep != len)
+                        G.pack()[gs] = keep; // shortened: the prepared map no longer applies (exponent 0)
+                }
+            }
+            __syncthreads();
+            n = uniform_u32(G.misc()[0]);
+            groups = uniform_u32(gs + 1u);
+        }
+    }
+    if (n < 1)
+        n = 1;
+    // (values merged over branches the compiler cannot see as uniform: back to scalar registers)
+    n = uniform_u32(n);
+    groups = uniform_u32(groups);
+    if (need_cut && !(q_bound < qat(n - 1)))
+        return false;
+    __syncthreads();
+
+    // candidates and the row's results, once total and position are known
+    auto emit = [&](float total, uint32_t pos) {
+        if (d.out_cand_idx && d.out_cand_q)
+            for (uint32_t j = tid; j < n && j < d.cand_cap; j += kThreads) {
+                d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
+                d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
+            }
+        if (tid == 0) {
+            RowOut o;
+            o.token = (int32_t)idat(pos);
+            o.n_cand = n;
+            o.total = total;
+            o.q = qat(pos);
+            o.path = path;
+            o.accepted = 0;
+            write_row(d, row, o);
+        }
+    };
+
+    MAKO_STAMP(7);
+    if (n <= kSeqMax) {
+        // A nucleus this short is copied to LDS and gone through entry by entry, once for the total and once for the
+        // walk (three nanoseconds an entry each way): the group maps below only pay on longer lists.
+        if (wave_id() == 0) {
+            const float S = sum_lds(G.head(), n, 0.0f);
+            const float span = S - 0.0f;
+            const float prod = u_row * span;
+            const float r0 = prod + 0.0f;
+            uint32_t at = n - 1;
+            if (r0 < 0.0f) {
+                at = 0;
+            } else if (r0 == r0 && r0 != INFINITY) {
+                float r = r0;
+                walk_lds(G.head(), n, r, at);
+            }
+            if (lane_id() == 0) {
+                G.misc()[1] = __float_as_uint(S);
+                G.misc()[2] = at;
+            }
+        }
+        __syncthreads();
+        MAKO_STAMP(9);
+        emit(__uint_as_float(G.misc()[1]), G.misc()[2]);
+        return true;
+    }
+
+    // exact fp32 total: group maps in parallel (here, or already by the workers), then one wave chains them
+    if (!PLANNED)
+        build_group_maps(kf, groups, false, 0.0, G);
+    __syncthreads();
+    MAKO_STAMP(13);
+    // While one wave chains the running sum, the others already prepare the walk: its maps only need the binade r is
+    // expected to be in at each group, and the fp64 sums give that (a wrong guess costs a replay, never the result).
+    // Groups that start after the mass r0 could have is used up get no map.
+    const double r0_guess = (double)u_row * G.pg()[groups];
+    uint32_t reach;
+    {
+        const uint32_t beyond = (tid < groups && !(r0_guess * 1.001 - G.pg()[tid] > 0)) ? tid : kNone;
+        reach = min(groups, block_min_u32(beyond, sm.bs));
+        if (tid < groups)
+            G.w_pack()[tid] = G.pack()[tid] & kLenMask;
+        __syncthreads();
+    }
+#ifdef MAKO_TIMING
+    if (tid == 0 && s_mako_row == 0) {
+        g_mako_stamp[20] = groups;
+        g_mako_stamp[21] = reach;
+        g_mako_stamp[22] = n;
+    }
+    const unsigned long long tb0 = wall_clock64();
+#endif
+    // A walk that will end within a few groups goes through them entry by entry, from a copy in LDS: faster than
+    // the groups' maps would be to build.
+    const bool head_walk = reach <= kWalkSeqGroups; // uniform
+    const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
+    if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && !head_walk) {
+        // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
+        build_group_maps(kf, reach, true, r0_guess, G, (uint32_t)(wave_id() >> 2) * 3u + (uint32_t)(wave_id() & 3) - 1u,
+                         3u * kWaves / 4u);
+#ifdef MAKO_TIMING
+        if (tid == 64 && s_mako_row == 0)
+            g_mako_stamp[23] = wall_clock64() - tb0;
+#endif
+    }
+    if (wave_id() == 0) {
+        // 64 groups at a time, one per lane.  A scan composes the lanes' maps; every lane then knows the state after
+        // its group, provided all groups so far share the running epoch and stay inside the binade.  The run up to the
+        // first group that cannot promise this is applied in one step, that group is replayed entry by entry, and
+        // the scan resumes behind it.  The state (significand M, exponent e) lives in scalar registers.
+        uint32_t M = 0;
+        int e = 1; // 0.0f
+        // The sum changes binade every few entries at first.  The leading groups, up to the last of the first few in
+        // which the fp64 sums expect a change, are added entry by entry from the copy in LDS.
+        uint32_t first = 0;
+        MAKO_TIC(0);
+        {
+            const uint32_t gq = min((uint32_t)lane_id(), groups - 1u);
+            const bool cross = (uint32_t)lane_id() < min(groups, kWalkSeqGroups) &&
+                               (lane_id() == 0 || exponent_of((float)G.pg()[gq]) != exponent_of((float)G.pg()[gq + 1u]));
+            const unsigned long long bal = __ballot(cross);
+            first = bal ? 64u - (uint32_t)__clzll((long long)bal) : 0u;
+            if (first) {
+                const uint32_t hs = first == groups ? n : uniform_u32(G.start()[min(first, groups - 1u)]);
+                const float S = sum_lds(G.head(), min(hs, kHead), 0.0f);
+                uint32_t Mv;
+                int ev;
+                split(S, Mv, ev);
+                M = uniform_u32(Mv);
+                e = (int)uniform_u32((uint32_t)ev);
+            }
+        }
+        MAKO_TOC(0, 17);
+#ifdef MAKO_TIMING
+        if (lane_id() == 0)
+            g_mako_stamp[19] = first;
+#endif
+        MAKO_TIC(1);
+        for (uint32_t base = 0; base < groups; base += kWave) {
+            const uint32_t gl = min(base + lane_id(), groups - 1u);
+            const uint32_t pk_l = G.pack()[gl], st_l = G.start()[gl];
+            const uint32_t d0_l = G.d0()[gl], d1_l = G.d1()[gl], cm_l = G.cmax()[gl];
+            const uint32_t cnt = min((uint32_t)kWave, groups - base);
+            uint32_t done = base == 0 ? first : 0u; // (first <= kWalkSeqGroups)
+            while (done < cnt) {
+                const bool live = lane_id() >= done && lane_id() < cnt;
+                const bool same = live && (pk_l >> 16) == (uint32_t)e;
+                Step32 v = lane_id() < done ? identity32() : (same ? Step32{d0_l, d1_l, 0u} : Step32{kSat, kSat, 0u});
+                wave_scan_maps(v.d0, v.d1);
+                const uint32_t after = M + ((M & 1u) ? v.d1 : v.d0); // < 2^29: no wrap
+                const bool ok = same && after + cm_l + 1u < (1u << 24); // group_add_ok for every group so far
+                const unsigned long long bad = __ballot(live && !ok);
+                const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : cnt;
+                if (f > done)
+                    M = (uint32_t)__builtin_amdgcn_readlane((int)after, (int)f - 1);
+                if (f < cnt) {
+                    const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
+                    const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
+#ifdef MAKO_TIMING
+                    if (lane_id() == 0)
+                        g_mako_stamp[21] += 1;
+#endif
+                    const uint32_t slot = (pk >> 9) & 0x7fu;
+                    if (slot) {
+                        const ChainState c = sum_by_quarters(kf, st, pk & kLenMask, G.quarters() + (slot - 1u) * 4u,
+                                                             ChainState{M, e, kNone});
+                        M = c.M;
+                        e = c.e;
+                    } else {
+                        const float S = exact_span_sum(kf, st, pk & kLenMask, join(M, e));
+                        uint32_t Mv;
+                        int ev;
+                        split(S, Mv, ev);
+                        M = uniform_u32(Mv);
+                        e = (int)uniform_u32((uint32_t)ev);
+                    }
+                }
+                done = f + 1u;
+            }
+        }
+        MAKO_TOC(1, 18);
+        if (lane_id() == 0)
+            G.misc()[1] = __float_as_uint(join(M, e));
+    }
+    __syncthreads();
+    MAKO_STAMP(8);
+    const float total = __uint_as_float(G.misc()[1]);
+    const float span = total - 0.0f;
+    const float prod = u_row * span;
+    const float r0 = prod + 0.0f;
+    __syncthreads();
+
+    // exact walk
+    uint32_t pos = n - 1;
+    if (r0 < 0.0f) {
+        pos = 0;
+    } else if (r0 == r0 && r0 != INFINITY) {
+        MAKO_STAMP(14);
+        if (wave_id() == 0) {
+            uint32_t M;
+            int e;
+            {
+                uint32_t Mv;
+                int ev;
+                split(r0, Mv, ev);
+                M = uniform_u32(Mv);
+                e = (int)uniform_u32((uint32_t)ev);
+            }
+            uint32_t at = n - 1;
+            bool stopped = false;
+            uint32_t first = 0; // groups already walked
+            if (head_walk && head_n) {
+                float r = r0;
+                stopped = walk_lds(G.head(), head_n, r, at);
+                uint32_t Mv;
+                int ev;
+                split(r, Mv, ev);
+                M = uniform_u32(Mv);
+                e = (int)uniform_u32((uint32_t)ev);
+                first = reach;
+            }
+            for (uint32_t base = 0; base < groups && !stopped; base += kWave) {
+                const uint32_t gl = min(base + lane_id(), groups - 1u);
+                const uint32_t pk_l = G.w_pack()[gl], st_l = G.start()[gl];
+                const uint32_t d0_l = G.w_d0()[gl], d1_l = G.w_d1()[gl], need_l = G.w_need()[gl]; // (the bound, see build_group_maps)
+                const uint32_t cnt = min((uint32_t)kWave, groups - base);
+                uint32_t done = base == 0 ? first : 0u; // (first <= kWalkSeqGroups)
+                while (done < cnt) {
+                    MAKO_COUNT(30, 1);
+                    const bool live = lane_id() >= done && lane_id() < cnt;
+                    const bool same = live && (pk_l >> 16) == (uint32_t)e;
+                    Step32 v = lane_id() < done ? identity32() : (same ? Step32{d0_l, d1_l, 0u} : Step32{kSat, kSat, 0u});
+                    wave_scan_maps(v.d0, v.d1);
+                    const uint32_t dd = (M & 1u) ? v.d1 : v.d0;
+                    const bool ok = same && dd <= M && M - dd >= need_l; // group_sub_ok for every group so far
+                    const unsigned long long bad = __ballot(live && !ok);
+                    const uint32_t f = bad ? (uint32_t)__ffsll((long long)bad) - 1u : cnt;
+                    if (f > done)
+                        M = (uint32_t)__builtin_amdgcn_readlane((int)(M - dd), (int)f - 1);
+                    if (f >= cnt)
+                        break;
+                    // Group f goes entry by entry.  Where one group does, its neighbours tend to follow (r is down
+                    // among the weights and changes binade every few entries), so the groups behind it are tried one
+                    // at a time with a few scalar operations each, the next one's entries already on their way,
+                    // and the scan takes over again once four in a row have gone through as maps.
+                    uint32_t g = f, passed = 0;
+                    uint32_t raw[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu}; // the entries of group g
+                    {
+                        const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g);
+                        const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g);
+                        if (pk & kLenMask)
+                            fetch_span_lanes(kf, st, pk & kLenMask, raw);
+                    }
+                    while (g < cnt && passed < 4u) {
+                        const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g);
+                        const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g);
+                        float xa[4];
+                        take_span_lanes(raw, pk & kLenMask, xa);
+                        // (the next group's entries set out now; they are used only if that group is replayed too)
+                        const uint32_t g1 = min(g + 1u, cnt - 1u);
+                        const uint32_t st1 = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g1);
+                        const uint32_t pk1 = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g1);
+                        if (pk1 & kLenMask)
+                            fetch_span_lanes(kf, st1, pk1 & kLenMask, raw);
+                        bool by_map = false;
+                        if (g != f && (pk >> 16) == (uint32_t)e) {
+                            const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, g);
+                            const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d1_l, g);
+                            const uint32_t need = (uint32_t)__builtin_amdgcn_readlane((int)need_l, g);
+                            const uint32_t d1g = (M & 1u) ? d1 : d0;
+                            if (d1g <= M && M - d1g >= need) { // group_sub_ok
+                                M -= d1g;
+                                by_map = true;
+                            }
+                        }
+                        if (by_map) {
+                            ++passed;
+                        } else {
+                            MAKO_COUNT(22, 1);
+                            passed = 0;
+                            float r = join(M, e);
+                            if ((pk & kLenMask) && walk_lanes(xa, pk & kLenMask, st, r, at)) {
+                                stopped = true;
+                                break;
+                            }
+                            uint32_t Mv;
+                            int ev;
+                            split(r, Mv, ev);
+                            M = uniform_u32(Mv);
+                            e = (int)uniform_u32((uint32_t)ev);
+                        }
+                        ++g;
+                    }
+                    if (stopped)
+                        break;
+                    done = g;
+                }
+            }
+            if (lane_id() == 0)
+                G.misc()[2] = at;
+        }
+        __syncthreads();
+        pos = G.misc()[2];
+    }
+
+    MAKO_STAMP(9);
+    emit(total, pos);
+    return true;
+}
+
+} // namespace mako

@@ -1,0 +1,51 @@
+// tail_kernel: the wide rows' cut, total and draw.
+#pragma once
+
+#include "sorted_tail.h"
+
+namespace mako {
+
+#ifdef MAKO_EMIT_TAIL_KERNEL
+// grid = (1, rows).  Rows whose sorted list sort_kernel's workers have prepared: top-p cut, exact total, draw.
+// (The batch's top-k rows were tried here too, beside the few long tails instead of ahead of the planning in
+// plan_kernel: 2.3 us less there, but this kernel's chains then compiled to slower code and lost twice that.)
+// (The context's record by value: with a pointer to it the first loads would have to wait for a trip to memory.  The
+// list's length and this workgroup's entry are asked for together, then everything the row's plan holds.)
+__global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_val)
+{
+    const Scratch& sc_arg = sc_val;
+    extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
+    __shared__ FinishShared sm;
+    __shared__ ArgsLds s_args;
+    const uint32_t n_work = sc_arg.work_n[1];
+    const uint32_t row = sc_arg.work_tail[blockIdx.y], tid = threadIdx.x; // (the list has room for every workgroup)
+    if (blockIdx.y >= n_work)
+        return;
+#ifdef MAKO_TIMING_TAIL
+    MAKO_WG_TIMER;
+#endif
+    MAKO_ROW(row);
+    const BigPlan* planned = sc_arg.plan + row;
+    const uint32_t flag = planned->flag, plan_n0 = planned->n0, plan_groups = planned->groups;
+    const double total64 = planned->total64;
+    if (flag != 1)
+        return;
+    stage_args(d_arg, sc_arg, row, s_args);
+    const mako_sample_desc& d = s_args.d;
+    const Scratch& sc = s_args.sc;
+    BigPlan* plan = sc.plan + row;
+    FinishLds L;
+    L.sm = &sm;
+    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
+    L.sortk = s_dyn64;
+    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
+    const uint32_t n0 = min(plan_n0, d.n_vocab), groups = min(plan_groups, min(kMaxGroups, sc.g_cap));
+    __syncthreads();
+    if (tid == 0)
+        plan->flag = 0;
+    sorted_tail<true>(d, row, s_args.P, sc.key[0] + (size_t)row * sc.vpad, sc.idx[0] + (size_t)row * sc.vpad, n0, true,
+                      total64, MAKO_PATH_GENERAL, L, false, 0.0f, sc.gt, (size_t)row * sc.g_cap, groups);
+}
+#endif // MAKO_EMIT_TAIL_KERNEL
+
+} // namespace mako

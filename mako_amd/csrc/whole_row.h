@@ -1,0 +1,590 @@
+// The whole-row path: exact for every parameter combination, one workgroup per row.
+#pragma once
+
+#include "sorted_tail.h"
+
+namespace mako {
+
+// Lanes of this wave whose `digit` equals mine, restricted to `valid` lanes.
+__device__ __forceinline__ unsigned long long match_digit(uint32_t digit, bool valid)
+{
+    unsigned long long m = __ballot(valid);
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+        const bool bit = (digit >> b) & 1u;
+        const unsigned long long bal = __ballot(bit);
+        m &= bit ? bal : ~bal;
+    }
+    return m;
+}
+
+// One stable counting-sort pass on bits [shift, shift + 8) of the keys, ascending, by one workgroup.
+// Wave w owns the contiguous chunk [w * C, (w + 1) * C) of the input and walks it 64 pairs at a time: lanes
+// with equal digits find each other with ballots (match_digit), so ranks inside a group need no atomics, and
+// the wave's running output offsets per digit live in its private row of LDS.  Three barriers per pass.
+// Returns false (and moves nothing) when every key has the same digit.
+__device__ bool radix_pass(const uint32_t* ksrc, const uint32_t* isrc, uint32_t* kdst, uint32_t* idst, uint32_t n,
+                           uint32_t shift, const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+    const uint32_t chunk = ((n + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
+    const uint32_t beg = min(n, wave * chunk), end = min(n, beg + chunk);
+    uint32_t* woff = L.wcount + wave * 256u;
+    for (uint32_t j = lane; j < 256u; j += kWave)
+        woff[j] = 0;
+    if (tid == 0)
+        sm.flag = 0;
+    const unsigned long long lower = (1ull << lane) - 1ull;
+    // per-wave digit counts (the row is private to the wave: in-order LDS, no barrier needed).  Four groups
+    // are fetched per trip, from clamped positions, so that their latencies overlap.
+    for (uint32_t base = beg; base < end; base += 4u * kWave) {
+        uint32_t key[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+            key[u] = ksrc[min(base + u * kWave + lane, end - 1u)];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const bool valid = base + u * kWave + lane < end;
+            const uint32_t dg = valid ? ((key[u] >> shift) & 255u) : 0u;
+            const unsigned long long mm = match_digit(dg, valid);
+            if (valid && (mm & lower) == 0)
+                woff[dg] += (uint32_t)__popcll(mm);
+        }
+    }
+    __syncthreads();
+    // digit totals -> global offsets; wave rows become each wave's first output position per digit
+    uint32_t mine = 0;
+    if (tid < 256)
+        for (int w = 0; w < kWaves; ++w)
+            mine += L.wcount[w * 256 + tid];
+    if (tid < 256 && mine == n)
+        sm.flag = 1;
+    uint32_t tot;
+    uint32_t acc = block_excl_scan_u32(mine, tot, sm.bs); // its barriers publish sm.flag
+    if (sm.flag)
+        return false;
+    if (tid < 256)
+        for (int w = 0; w < kWaves; ++w) {
+            const uint32_t t = L.wcount[w * 256 + tid];
+            L.wcount[w * 256 + tid] = acc;
+            acc += t;
+        }
+    __syncthreads();
+    for (uint32_t base = beg; base < end; base += 4u * kWave) {
+        uint32_t key[4], id[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t i = min(base + u * kWave + lane, end - 1u);
+            key[u] = ksrc[i];
+            id[u] = isrc[i];
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const bool valid = base + u * kWave + lane < end;
+            const uint32_t dg = valid ? ((key[u] >> shift) & 255u) : 0u;
+            const unsigned long long mm = match_digit(dg, valid);
+            const uint32_t off = woff[dg];
+            if (valid) {
+                const uint32_t pos = off + (uint32_t)__popcll(mm & lower);
+                kdst[pos] = key[u];
+                idst[pos] = id[u];
+                if ((mm & lower) == 0)
+                    woff[dg] = off + (uint32_t)__popcll(mm);
+            }
+        }
+    }
+    __syncthreads();
+    return true;
+}
+
+__device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t* i1, uint32_t n, const FinishLds& L);
+
+// std::ranges::nth_element(cand, cand + nth, desc) of src/gen/sampler.cpp:41 as libstdc++ 11 runs it (introselect,
+// bits/stl_algo.h:1964), leaving the candidates in exactly the arrangement that library leaves: the reference sums
+// and walks the top_k survivors in that order when no top-p follows.  key/idx hold n candidates (~bits(q), token
+// id); `desc` is the order of the 64-bit values key << 32 | idx, all distinct.
+// One round = median of three to the front, then the unguarded Hoare partition of the rest around it.  That
+// partition swaps the t-th entry from the left that belongs right with the t-th entry from the right that belongs
+// left for as long as the former lies before the latter, and cuts behind the entries that belong left: the two
+// position lists come from ballots (wave w owns the w-th sixteenth of the range), the swaps are independent.
+// The depth limit's heap select and the last insertion sort (at most three entries) are sequential code on one
+// thread.
+//
+// introselect_rounds runs the rounds on [first, last) through get(i) / put(i, v) until the range is no longer than
+// `until` (3 = to the end, insertion sort included).  lsta / lstb: room for last - first positions each.  Returns
+// true when nothing is left to do.
+template <typename Get, typename Put>
+__device__ bool introselect_rounds(Get get, Put put, uint32_t& first, uint32_t& last, uint32_t nth, uint32_t& depth,
+                                   uint32_t until, uint32_t* lsta, uint32_t* lstb, FinishShared& sm)
+{
+    typedef unsigned long long u64;
+    const uint32_t tid = threadIdx.x, lane = lane_id(), wave = wave_id();
+    while (last - first > until) {
+        if (depth == 0) {
+            // __heap_select(first, nth + 1, last) and iter_swap(first, nth): bits/stl_algo.h:1956-1960, stl_heap.h
+            if (tid == 0) {
+                const uint32_t middle = nth + 1u - first, len = last - first;
+                auto sift = [&](uint32_t hole, u64 v) { // __adjust_heap: the hole sinks to a leaf, v rises from there
+                    const uint32_t top = hole;
+                    uint32_t child = hole;
+                    while (child < (middle - 1u) / 2u) {
+                        child = 2u * (child + 1u);
+                        if (get(first + child) < get(first + child - 1u))
+                            --child;
+                        put(first + hole, get(first + child));
+                        hole = child;
+                    }
+                    if ((middle & 1u) == 0 && middle >= 2u && child == (middle - 2u) / 2u) {
+                        child = 2u * (child + 1u);
+                        put(first + hole, get(first + child - 1u));
+                        hole = child - 1u;
+                    }
+                    while (hole > top) {
+                        const uint32_t parent = (hole - 1u) / 2u;
+                        if (!(get(first + parent) < v))
+                            break;
+                        put(first + hole, get(first + parent));
+                        hole = parent;
+                    }
+                    put(first + hole, v);
+                };
+                if (middle >= 2u)
+                    for (uint32_t parent = (middle - 2u) / 2u;; --parent) {
+                        sift(parent, get(first + parent));
+                        if (parent == 0)
+                            break;
+                    }
+                for (uint32_t i = middle; i < len; ++i) {
+                    const u64 v = get(first + i);
+                    if (v < get(first)) {
+                        put(first + i, get(first));
+                        sift(0u, v);
+                    }
+                }
+                const u64 a = get(first), b = get(nth);
+                put(first, b);
+                put(nth, a);
+            }
+            __syncthreads();
+            return true;
+        }
+        --depth;
+        if (tid == 0) { // __move_median_to_first(first, first + 1, mid, last - 1)
+            const uint32_t ix = first + 1u, iy = first + (last - first) / 2u, iz = last - 1u;
+            const u64 x = get(ix), y = get(iy), z = get(iz);
+            uint32_t im;
+            if (x < y)
+                im = y < z ? iy : (x < z ? iz : ix);
+            else
+                im = x < z ? ix : (y < z ? iz : iy);
+            const u64 r = get(first), med = get(im);
+            put(first, med);
+            put(im, r);
+        }
+        __syncthreads();
+        const u64 pivot = get(first);
+        const uint32_t lo0 = first + 1u, len = last - lo0;
+        const uint32_t chunk = ((len + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
+        const uint32_t beg = min(last, lo0 + wave * chunk), end = min(last, beg + chunk);
+        // entries of the wave's chunk that belong left of the cut
+        // (kTrip loads in flight per lane: a trip costs one round trip to memory, not kTrip)
+        constexpr uint32_t kTrip = 4;
+        uint32_t mine = 0;
+        for (uint32_t base = beg; base < end; base += kWave * kTrip) {
+            u64 v[kTrip];
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u)
+                v[u] = get(min(base + u * kWave + lane, last - 1u));
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u)
+                mine += (uint32_t)__popcll(__ballot(base + u * kWave + lane < end && v[u] < pivot));
+        }
+        if (lane == 0)
+            sm.bs.u64[wave] = mine;
+        __syncthreads();
+        uint32_t small_before = 0, smalls = 0;
+        for (int w = 0; w < kWaves; ++w) {
+            const uint32_t x = (uint32_t)sm.bs.u64[w];
+            if (w < (int)wave)
+                small_before += x;
+            smalls += x;
+        }
+        const uint32_t bigs = len - smalls;
+        uint32_t big_before = (beg - lo0) - small_before;
+        // position lists: lsta[t] = the t-th big entry from the left, lstb[t] = the t-th small entry from the left
+        const u64 lower = (1ull << lane) - 1ull;
+        for (uint32_t base = beg; base < end; base += kWave * kTrip) {
+            u64 v[kTrip];
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u)
+                v[u] = get(min(base + u * kWave + lane, last - 1u));
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u) {
+                const uint32_t pos = base + u * kWave + lane;
+                const bool in = pos < end;
+                const bool small = in && v[u] < pivot;
+                const u64 bs = __ballot(small), bb = __ballot(in && !small);
+                if (small)
+                    lstb[small_before + (uint32_t)__popcll(bs & lower)] = pos;
+                else if (in)
+                    lsta[big_before + (uint32_t)__popcll(bb & lower)] = pos;
+                small_before += (uint32_t)__popcll(bs);
+                big_before += (uint32_t)__popcll(bb);
+            }
+        }
+        __syncthreads();
+        const uint32_t pairs = min(bigs, smalls);
+        for (uint32_t t = tid; t < pairs; t += kThreads) {
+            const uint32_t a = lsta[t], b = lstb[smalls - 1u - t];
+            if (a < b) {
+                const u64 va = get(a), vb = get(b);
+                put(a, vb);
+                put(b, va);
+            }
+        }
+        __syncthreads();
+        const uint32_t cut = lo0 + smalls;
+        if (cut <= nth)
+            first = cut;
+        else
+            last = cut;
+    }
+    if (last - first > 3u)
+        return false;
+    if (tid == 0) // __insertion_sort(first, last)
+        for (uint32_t i = first + 1u; i < last; ++i) {
+            const u64 v = get(i);
+            uint32_t j = i;
+            if (v < get(first)) {
+                for (; j > first; --j)
+                    put(j, get(j - 1u));
+            } else {
+                for (; v < get(j - 1u); --j)
+                    put(j, get(j - 1u));
+            }
+            put(j, v);
+        }
+    __syncthreads();
+    return true;
+}
+
+// The row's candidates in device memory (key[i], idx[i]; lsta / lstb: room for n positions each).  The rounds run on
+// device memory, ten or so dependent trips to memory each, until the range fits the dynamic LDS block (kSortMax
+// entries and two position lists); the remaining dozen rounds run on a copy there.
+__device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32_t nth, uint32_t* lsta, uint32_t* lstb,
+                                const FinishLds& L)
+{
+    typedef unsigned long long u64;
+    const uint32_t tid = threadIdx.x;
+    if (n == 0 || nth >= n)
+        return;
+    uint32_t first = 0, last = n;
+    uint32_t depth = 2u * (31u - (uint32_t)__clz((int)n));
+    __syncthreads();
+    auto get = [=](uint32_t i) { return ((u64)key[i] << 32) | (u64)idx[i]; };
+    auto put = [=](uint32_t i, u64 v) {
+        key[i] = (uint32_t)(v >> 32);
+        idx[i] = (uint32_t)v;
+    };
+    if (introselect_rounds(get, put, first, last, nth, depth, kSortMax, lsta, lstb, *L.sm))
+        return;
+    u64* lds = L.sortk;
+    uint32_t* la = reinterpret_cast<uint32_t*>(L.sortk + kSortMax);
+    uint32_t* lb = la + kSortMax;
+    static_assert(kSortMax * 16u <= kDynLds, "the range and its two position lists fit the dynamic LDS block");
+    const uint32_t base = first, len = last - first;
+    for (uint32_t i = tid; i < len; i += kThreads)
+        lds[i] = get(base + i);
+    __syncthreads();
+    introselect_rounds([=](uint32_t i) { return lds[i - base]; }, [=](uint32_t i, u64 v) { lds[i - base] = v; }, first, last,
+                       nth, depth, 3u, la, lb, *L.sm);
+    for (uint32_t i = tid; i < len; i += kThreads)
+        put(base + i, lds[i]);
+    __syncthreads();
+}
+
+// Common tail of the whole-row paths.  key[0]/idx[0] of the row hold n0 candidates (~bits(q), token id) in index
+// order.  Sorts them by (q desc, idx asc) when top-k or top-p is active, truncates (src/gen/sampler.cpp:39-61)
+// and draws.  `total64` (when have_total) is the fp64 sum of q over all candidates of the row, of which the list
+// may be only the heaviest part; otherwise it is summed from the list.
+// (TOPK_ALONE = false leaves the top-k-without-top-p branch out of the instance inside plan_kernel<true>: that kernel is
+// only launched for batches whose host copy of the parameters shows a top-p on every sampled row, and the branch's
+// registers would be spilled around the top-k rows' fast path, +3.5 us on a 256-row batch.)
+template <bool TOPK_ALONE>
+__device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
+                                   uint32_t n0, bool have_total, double total64, uint32_t path, const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
+    uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
+    uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
+    uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
+
+    // order by (q desc, idx asc): stable LSD radix sort of ~bits(q), ascending
+    const bool topk_active = P.top_k > 0 && P.top_k < n0;
+    const bool topp_active = P.top_p < 1.0f;
+    // top-k alone: the survivors stay in the order nth_element leaves them (sampler.cpp:39-43, then :79-83)
+    const bool nth_order = TOPK_ALONE && topk_active && !topp_active;
+    if (nth_order)
+        nth_element_row(key0, idx0, n0, P.top_k, key1, idx1, L);
+    else if (topk_active || topp_active)
+        sort_segment(key0, idx0, key1, idx1, n0, L);
+    const uint32_t *ks = key0, *is = idx0;
+    MAKO_STAMP(12);
+    const uint32_t n1 = topk_active ? P.top_k : n0; // sampler.cpp:40-43
+    // (sorted_tail's one-wave path for lists of up to kGroup entries adds and walks them in the order given, whatever
+    // it is, and without a top-p it cuts nothing: nth_element's survivors take it too)
+    if (nth_order ? (!d.draft && n1 <= kGroup) : (topk_active || topp_active)) {
+        sorted_tail(d, row, P, ks, is, n1, have_total, total64, path, L);
+        return;
+    }
+    // nth_element's order (long lists, verification), or neither top-k nor top-p: the candidates stay in index order
+    const uint32_t* kf = ks;
+    const uint32_t* jf = is;
+    draw_from_list(
+        d, row, [=](uint32_t i) { return __uint_as_float(~kf[i]); }, [=](uint32_t i) { return jf[i]; }, n1, path, sm);
+}
+
+// Copies the weights of the row with key_lo <= bits(q) < key_hi, in index order, to kout / iout (as ~bits(q) and
+// token id).  Wave w owns a contiguous chunk of the row: a counting sweep, one exchange of the 16 wave totals,
+// then a writing sweep in which ranks come from ballots.  Lane l holds entries 4l..4l+3 of each 256-entry group.
+// Returns the number of entries written.
+__device__ uint32_t gather_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, uint32_t key_hi, uint32_t* kout,
+                                 uint32_t* iout, uint32_t cap, FinishShared& sm)
+{
+    const uint32_t lane = lane_id(), wave = wave_id();
+    const uint32_t chunk = ((V + kThreads * 4u - 1u) / (kThreads * 4u)) * kGroup; // per wave, a multiple of 256
+    const uint32_t beg = min(V, wave * chunk), end = min(V, beg + chunk);
+    auto fetch = [&](uint32_t i, uint32_t (&k)[4]) {
+        if (i + 3 < end) {
+            const uint4 x = *reinterpret_cast<const uint4*>(qk + i);
+            k[0] = x.x;
+            k[1] = x.y;
+            k[2] = x.z;
+            k[3] = x.w;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                k[j] = i + j < end ? qk[i + j] : 0u;
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (k[j] < key_lo || k[j] >= key_hi)
+                k[j] = 0;
+    };
+    uint32_t mine = 0;
+    for (uint32_t base = beg; base < end; base += 4u * kGroup) {
+        uint32_t k[4][4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+            fetch(base + u * kGroup + lane * 4u, k[u]);
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u)
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                mine += k[u][j] != 0;
+    }
+    mine = __ockl_wfred_add_u32(mine);
+    __syncthreads();
+    if (lane == 0)
+        sm.bs.u64[wave] = mine;
+    __syncthreads();
+    uint32_t out = 0, n0 = 0;
+    for (int w = 0; w < kWaves; ++w) {
+        const uint32_t x = (uint32_t)sm.bs.u64[w];
+        if (w < (int)wave)
+            out += x;
+        n0 += x;
+    }
+    const unsigned long long lower = (1ull << lane) - 1ull;
+    for (uint32_t base = beg; base < end; base += 2u * kGroup) {
+        uint32_t k[2][4];
+        fetch(base + lane * 4u, k[0]);
+        fetch(base + kGroup + lane * 4u, k[1]);
+#pragma unroll
+        for (uint32_t u = 0; u < 2; ++u) {
+            uint32_t before = 0, total = 0;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                const unsigned long long bal = __ballot(k[u][j] != 0);
+                before += (uint32_t)__popcll(bal & lower);
+                total += (uint32_t)__popcll(bal);
+            }
+            uint32_t pos = out + before;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (k[u][j]) {
+                    if (pos < cap) { // (the caller's count of the range; never exceeded when the plan is sound)
+                        kout[pos] = ~k[u][j];
+                        iout[pos] = base + u * kGroup + lane * 4u + j;
+                    }
+                    ++pos;
+                }
+            out += total;
+        }
+    }
+    __syncthreads();
+    return n0;
+}
+
+// Sorts n (key, id) pairs at (k0, i0) by key ascending, stably, with (k1, i1) as the second buffer; the result
+// ends in (k0, i0).
+__device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t* i1, uint32_t n, const FinishLds& L)
+{
+    if (n < 2)
+        return;
+    uint32_t *ks = k0, *is = i0, *kd = k1, *id = i1;
+    for (uint32_t shift = 0; shift < 32; shift += 8) {
+        if (radix_pass(ks, is, kd, id, n, shift, L)) {
+            uint32_t* t = ks;
+            ks = kd;
+            kd = t;
+            t = is;
+            is = id;
+            id = t;
+        }
+        __syncthreads();
+    }
+    if (ks != k0) {
+        for (uint32_t i = threadIdx.x; i < n; i += kThreads) {
+            k0[i] = ks[i];
+            i0[i] = is[i];
+        }
+        __syncthreads();
+    }
+}
+
+// Whole-row path: exact for every parameter combination.  One workgroup rebuilds the penalised
+// row in scratch, keeps the candidates, sorts them by (q desc, idx asc) when top-k or top-p is
+// active, truncates, and draws.  src/gen/sampler.cpp:20-62.
+// (SITE: sort_kernel, its usual place, has an instance to itself, so that the compiler treats that kernel the same
+// whether or not the instances inside plan_kernel exist.)
+template <int SITE>
+__device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
+                            float m, uint32_t argidx, const FinishLds& L)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t V = d.n_vocab;
+    float* wbuf = sc.wbuf + (size_t)row * sc.vpad;
+    uint32_t* cnt = sc.cnt + (size_t)row * sc.vpad;
+    uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
+    uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
+    const float* lrow = d.logits + (int64_t)row * d.logits_stride;
+    const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
+
+    // 1. masked copy, then the penalties once per distinct history token
+    for (uint32_t i = tid; i < V; i += kThreads) {
+        float v = lrow[i];
+        if (mrow && !((mrow[i >> 5] >> (i & 31u)) & 1u))
+            v = -INFINITY;
+        wbuf[i] = v;
+    }
+    __syncthreads();
+    const uint32_t hl = d.hist_tokens ? d.hist_len[row] : 0u;
+    if (hl > 0 && !penalties_neutral(P)) {
+        const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
+        const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
+        for (uint32_t h = tid; h < hl; h += kThreads) {
+            const uint32_t t = (uint32_t)ht[h];
+            if (t < V)
+                atomicAdd(&cnt[t], hc ? hc[h] : 1u);
+        }
+        __syncthreads();
+        for (uint32_t h = tid; h < hl; h += kThreads) {
+            const uint32_t t = (uint32_t)ht[h];
+            if (t < V) {
+                const uint32_t c = atomicExch(&cnt[t], 0u); // claims the token and restores the zero
+                if (c)
+                    wbuf[t] = penalize(wbuf[t], c, P.repetition_penalty, P.presence_penalty, P.frequency_penalty);
+            }
+        }
+        __syncthreads();
+    }
+
+    // 2. weights and the min_p / q > 0 filter, compacted in index order (sampler.cpp:29-36).  Wave w owns the w-th
+    // sixteenth of the row (a multiple of 256 logits, lane l entries 4l..4l+3 of each 256): a sweep that leaves bits(q)
+    // of every candidate (0 otherwise) in place of the logit and counts them, one exchange of the waves' totals, and
+    // a sweep in which every lane reads back what it wrote and a wave scan ranks it.  No barrier inside the sweeps.
+    const float inv_t = 1.0f / P.temperature;
+    const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p; // std::min(min_p, 1.0f)
+    uint32_t* qb = reinterpret_cast<uint32_t*>(wbuf);
+    const uint32_t lane = lane_id(), wave = wave_id();
+    const uint32_t chunk = ((V + kThreads * 4u - 1u) / (kThreads * 4u)) * kGroup;
+    const uint32_t beg = min(V, wave * chunk), end = min(V, beg + chunk);
+    uint32_t mine = 0;
+    for (uint32_t base = beg; base < end; base += kGroup) {
+        const uint32_t i = base + lane * 4u;
+        float w[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        const bool whole = i + 3u < end;
+        if (whole) {
+            const float4 x = *reinterpret_cast<const float4*>(wbuf + i);
+            w[0] = x.x, w[1] = x.y, w[2] = x.z, w[3] = x.w;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (i + j < end)
+                    w[j] = wbuf[i + j];
+        }
+        uint32_t k[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const float q = weight_of(w[j], m, inv_t, sm.tab);
+            k[j] = (i + j < end && q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
+            mine += k[j] ? 1u : 0u;
+        }
+        if (whole) {
+            *reinterpret_cast<uint4*>(qb + i) = make_uint4(k[0], k[1], k[2], k[3]);
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (i + j < end)
+                    qb[i + j] = k[j];
+        }
+    }
+    mine = __ockl_wfred_add_u32(mine);
+    if (lane == 0)
+        sm.bs.u64[wave] = mine;
+    __syncthreads();
+    uint32_t n0 = 0, at = 0;
+    for (int w = 0; w < kWaves; ++w) {
+        const uint32_t x = (uint32_t)sm.bs.u64[w];
+        if (w < (int)wave)
+            at += x;
+        n0 += x;
+    }
+    for (uint32_t base = beg; base < end; base += kGroup) {
+        const uint32_t i = base + lane * 4u;
+        uint32_t k[4] = {0u, 0u, 0u, 0u};
+        if (i + 3u < end) {
+            const uint4 x = *reinterpret_cast<const uint4*>(qb + i);
+            k[0] = x.x, k[1] = x.y, k[2] = x.z, k[3] = x.w;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (i + j < end)
+                    k[j] = qb[i + j];
+        }
+        const uint32_t c = (k[0] ? 1u : 0u) + (k[1] ? 1u : 0u) + (k[2] ? 1u : 0u) + (k[3] ? 1u : 0u);
+        const uint32_t incl = __ockl_wfscan_add_u32(c, true);
+        uint32_t pos = at + incl - c;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (k[j]) {
+                key0[pos] = ~k[j];
+                idx0[pos] = i + j;
+                ++pos;
+            }
+        at += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+    }
+    __syncthreads();
+
+    if (n0 == 0) {
+        fallback_row(d, row, argidx);
+        return;
+    }
+    sort_truncate_draw<SITE == 0>(d, sc, row, P, n0, false, 0.0, MAKO_PATH_GENERAL, L);
+}
+
+} // namespace mako

@@ -1,0 +1,385 @@
+// The workers' LDS sorts of their shares of a wide nucleus, and the group records they leave for the tail.
+#pragma once
+
+#include "sorted_tail.h"
+#include "whole_row.h"
+
+namespace mako {
+
+__device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, uint32_t* kout, uint32_t* iout,
+                                unsigned long long* dyn, FinishShared& sm, uint32_t* sorted_lds = nullptr);
+
+// Worker's sort, LDS-resident: the weights of the row with key_lo <= bits(q) < key_hi (at most kSegCap of them)
+// are collected from the row's bits(q) array in one sweep, dropped into kFine value buckets (descending), and
+// every entry then finds its place by counting the entries of its own bucket that precede it under
+// (q desc, idx asc).  The sorted range is written to kout / iout as ~bits(q) and token id.  Returns false, having
+// written nothing, when the range does not fit or a bucket is too crowded to be ranked by counting.
+__device__ bool lds_sort_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, uint32_t key_hi, uint32_t cnt, uint32_t* kout,
+                               uint32_t* iout, unsigned long long* dyn, FinishShared& sm)
+{
+    uint2* A = reinterpret_cast<uint2*>(dyn);                       // [kSegCap] (bits(q), idx), any order
+    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);         // [kSegCap] entry of A at each bucket-ordered slot
+    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap);      // [kFine + 1] bucket counts, then bucket starts
+    const uint32_t tid = threadIdx.x, lane = lane_id();
+    if (cnt > kSegCap)
+        return false;
+    for (uint32_t b = tid; b <= kFine; b += kThreads)
+        hist[b] = 0;
+    if (tid == 0) {
+        sm.ticket = 0;
+        sm.flag = 0;
+    }
+    __syncthreads();
+    // 1. collect: a slot range per wave and trip from one LDS atomic
+    for (uint32_t base = 0; base < V; base += 4u * kThreads * 4u) {
+        uint32_t k[4][4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint32_t i = base + u * kThreads * 4u + tid * 4u;
+            if (i + 3 < V) {
+                const uint4 x = *reinterpret_cast<const uint4*>(qk + i);
+                k[u][0] = x.x;
+                k[u][1] = x.y;
+                k[u][2] = x.z;
+                k[u][3] = x.w;
+            } else {
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j)
+                    k[u][j] = i + j < V ? qk[i + j] : 0u;
+            }
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            // ranks inside the wave from ballots (any order will do), one LDS atomic per wave for the slots
+            uint32_t before = 0, wave_total = 0;
+            const unsigned long long lower = (1ull << lane) - 1ull;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+                if (k[u][j] < key_lo || k[u][j] >= key_hi)
+                    k[u][j] = 0; // 0 is never a candidate's weight
+                const unsigned long long bal = __ballot(k[u][j] != 0);
+                before += (uint32_t)__popcll(bal & lower);
+                wave_total += (uint32_t)__popcll(bal);
+            }
+            if (wave_total) { // uniform
+                uint32_t slot = 0;
+                if (lane == 0)
+                    slot = atomicAdd(&sm.ticket, wave_total);
+                slot = uniform_u32(slot) + before;
+                const uint32_t i = base + u * kThreads * 4u + tid * 4u;
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j)
+                    if (k[u][j]) {
+                        if (slot < kSegCap)
+                            A[slot] = make_uint2(k[u][j], i + j);
+                        ++slot;
+                    }
+            }
+        }
+    }
+    __syncthreads();
+    if (sm.ticket != cnt) // (cannot happen: the plan counted the same array)
+        return false;
+    return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm);
+}
+
+// Second half of the workers' sort: the n entries (bits(q), idx) in LDS at A, all with key_lo <= bits(q) < key_hi,
+// go to kout / iout ordered by (q desc, idx asc).  hist must be zero and sm.flag 0 on entry.
+// sorted_lds (optional, n words of LDS outside the sort's own): receives the sorted ~bits(q) as well, and the
+// function then returns behind a barrier that orders LDS only: the caller goes on from the copy instead of waiting
+// for the stores to kout and reading them back.
+__device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, uint32_t* kout, uint32_t* iout,
+                                unsigned long long* dyn, FinishShared& sm, uint32_t* sorted_lds)
+{
+    uint2* A = reinterpret_cast<uint2*>(dyn);
+    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap);
+    const uint32_t tid = threadIdx.x;
+    // 2. buckets by value, heaviest first
+    const uint32_t range = key_hi - key_lo; // > 0
+    const uint32_t shift = range > kFine ? 32u - (uint32_t)__clz((range - 1u) >> 11) : 0u; // (range - 1) >> shift < kFine
+    constexpr uint32_t kPer = kSegCap / kThreads;
+    uint32_t bucket[kPer], pib[kPer];
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t) {
+        const uint32_t e = t * kThreads + tid;
+        bucket[t] = kNone;
+        pib[t] = 0;
+        if (e < n) {
+            bucket[t] = (key_hi - 1u - A[e].x) >> shift;
+            pib[t] = atomicAdd(&hist[bucket[t]], 1u);
+        }
+    }
+    __syncthreads();
+    {
+        const uint32_t c0 = hist[2u * tid], c1 = hist[2u * tid + 1u];
+        if (max(c0, c1) > 64u)
+            sm.flag = 1;
+        uint32_t total;
+        const uint32_t ex = block_excl_scan_u32(c0 + c1, total, sm.bs); // (barriers: all counts are read before)
+        hist[2u * tid] = ex;
+        hist[2u * tid + 1u] = ex + c0;
+        if (tid == 0)
+            hist[kFine] = total;
+    }
+    __syncthreads();
+    if (sm.flag)
+        return false;
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t)
+        if (bucket[t] != kNone)
+            B[hist[bucket[t]] + pib[t]] = (uint16_t)(t * kThreads + tid);
+    __syncthreads();
+    // 3. rank inside the bucket, and out
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t) {
+        const uint32_t s = t * kThreads + tid;
+        if (s < n) {
+            const uint2 me = A[B[s]];
+            const uint32_t b = (key_hi - 1u - me.x) >> shift;
+            const uint32_t lo = hist[b], hi = hist[b + 1u];
+            uint32_t r = 0;
+            for (uint32_t x = lo; x < hi; ++x) {
+                const uint2 o = A[B[x]];
+                r += (o.x > me.x) || (o.x == me.x && o.y < me.y);
+            }
+            kout[lo + r] = ~me.x;
+            iout[lo + r] = me.y;
+            if (sorted_lds)
+                sorted_lds[lo + r] = ~me.x;
+        }
+    }
+    if (sorted_lds) // uniform
+        lds_barrier();
+    else
+        __syncthreads();
+    return true;
+}
+
+// The worker's share as partition_kernel left it (cnt <= kSegCap entries, bits(q) in ks and token ids in is, any
+// order), sorted into kout / iout.
+__device__ bool lds_sort_staged(const uint32_t* ks, const uint32_t* is, uint32_t key_lo, uint32_t key_hi, uint32_t cnt,
+                                uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm,
+                                uint32_t* sorted_lds = nullptr)
+{
+    uint2* A = reinterpret_cast<uint2*>(dyn);
+    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap);
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t b = tid; b <= kFine; b += kThreads)
+        hist[b] = 0;
+    if (tid == 0)
+        sm.flag = 0;
+    constexpr uint32_t kPer = kSegCap / kThreads;
+    uint32_t k[kPer], id[kPer];
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t) { // (all loads first, from clamped positions)
+        const uint32_t e = min(t * kThreads + tid, cnt - 1u);
+        k[t] = ks[e];
+        id[t] = is[e];
+    }
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t) {
+        const uint32_t e = t * kThreads + tid;
+        if (e < cnt)
+            A[e] = make_uint2(min(max(k[t], key_lo), key_hi - 1u), id[t]); // (clamped: a bucket index is always valid)
+    }
+    __syncthreads();
+    return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm, sorted_lds);
+}
+
+// A share too large for one LDS sort is cut by value into runs that fit: one counting sweep over the share (the
+// same kFine buckets as the sort uses) finds run boundaries at bucket edges, then each run is collected from the
+// share and sorted on its own.  Returns false (the caller falls back to the radix sort through global memory)
+// when a single bucket holds more than fits.
+__device__ bool lds_sort_staged_runs(const uint32_t* ks, const uint32_t* is, uint32_t key_lo, uint32_t key_hi, uint32_t cnt,
+                                     uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm)
+{
+    uint2* A = reinterpret_cast<uint2*>(dyn);
+    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap); // [kFine + 1]
+    const uint32_t tid = threadIdx.x, lane = lane_id();
+    const uint32_t range = key_hi - key_lo;
+    const uint32_t shift = range > kFine ? 32u - (uint32_t)__clz((range - 1u) >> 11) : 0u;
+    for (uint32_t b = tid; b <= kFine; b += kThreads)
+        hist[b] = 0;
+    __syncthreads();
+    constexpr uint32_t kTrip = 8; // loads in flight per thread: the sweeps below are bound by memory latency
+    for (uint32_t base = 0; base < cnt; base += kTrip * kThreads) {
+        uint32_t k[kTrip];
+#pragma unroll
+        for (uint32_t u = 0; u < kTrip; ++u)
+            k[u] = ks[min(base + u * kThreads + tid, cnt - 1u)];
+#pragma unroll
+        for (uint32_t u = 0; u < kTrip; ++u)
+            if (base + u * kThreads + tid < cnt)
+                atomicAdd(&hist[(key_hi - 1u - min(max(k[u], key_lo), key_hi - 1u)) >> shift], 1u);
+    }
+    __syncthreads();
+    // bucket starts (exclusive scan), kept in sm.hist / sm.run as run boundaries below
+    uint32_t total;
+    const uint32_t c0 = hist[2u * tid], c1 = hist[2u * tid + 1u];
+    const uint32_t ex = block_excl_scan_u32(c0 + c1, total, sm.bs);
+    __syncthreads();
+    hist[2u * tid] = ex;
+    hist[2u * tid + 1u] = ex + c0;
+    if (tid == 0) {
+        hist[kFine] = total;
+        sm.flag = 0;
+    }
+    __syncthreads();
+    // runs: greedily as many whole buckets as fit (thread 0; a handful of runs).  Run r covers buckets
+    // [sm.hist[r], sm.hist[64 + r]) = entries [sm.run[r], sm.run[r] + sm.run[64 + r]) of the sorted share.
+    if (tid == 0) {
+        uint32_t runs = 0, b0 = 0;
+        while (b0 < kFine && runs < 64u) {
+            uint32_t b1 = b0 + 1u;
+            if (hist[b1] - hist[b0] > kSegCap) { // one bucket alone is too much
+                runs = 0xffffffffu;
+                break;
+            }
+            { // the last bucket edge within reach: the bucket starts never decrease, so bisect
+                uint32_t lo = b1, hi = kFine;
+                while (lo < hi) {
+                    const uint32_t mid = (lo + hi + 1u) / 2u;
+                    if (hist[mid] - hist[b0] <= kSegCap)
+                        lo = mid;
+                    else
+                        hi = mid - 1u;
+                }
+                b1 = lo;
+            }
+            if (hist[b1] != hist[b0]) {
+                sm.hist[runs] = b0;
+                sm.hist[64u + runs] = b1;
+                sm.run[runs] = hist[b0];
+                sm.run[64u + runs] = hist[b1] - hist[b0];
+                ++runs;
+            }
+            b0 = b1;
+        }
+        if (runs != 0xffffffffu && b0 < kFine)
+            runs = 0xffffffffu;
+        sm.ticket = runs;
+    }
+    __syncthreads();
+    const uint32_t runs = sm.ticket;
+    if (runs == 0xffffffffu)
+        return false;
+    for (uint32_t r = 0; r < runs; ++r) {
+        const uint32_t b0 = sm.hist[r], b1 = sm.hist[64u + r];
+        const uint32_t at = sm.run[r], n = sm.run[64u + r];
+        // keys of buckets [b0, b1): (key_hi - 1 - k) >> shift in [b0, b1)
+        const uint32_t hi_r = key_hi - (b0 << shift);
+        const uint32_t lo_r = ((unsigned long long)b1 << shift) >= range ? key_lo : key_hi - (b1 << shift);
+        __syncthreads();
+        for (uint32_t b = tid; b <= kFine; b += kThreads)
+            hist[b] = 0;
+        if (tid == 0) {
+            sm.ticket = 0;
+            sm.flag = 0;
+        }
+        __syncthreads();
+        const unsigned long long lower = (1ull << lane) - 1ull;
+        for (uint32_t base = 0; base < cnt; base += kTrip * kThreads) {
+            uint32_t k[kTrip], id[kTrip];
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u) {
+                const uint32_t e = min(base + u * kThreads + tid, cnt - 1u);
+                k[u] = ks[e];
+                id[u] = is[e];
+            }
+            // slots for the whole trip from one LDS atomic per wave
+            bool mine[kTrip];
+            uint32_t before = 0, wave_total = 0;
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u) {
+                k[u] = min(max(k[u], key_lo), key_hi - 1u);
+                mine[u] = base + u * kThreads + tid < cnt && k[u] >= lo_r && k[u] < hi_r;
+                const unsigned long long bal = __ballot(mine[u]);
+                before += (uint32_t)__popcll(bal & lower);
+                wave_total += (uint32_t)__popcll(bal);
+            }
+            if (wave_total) { // uniform
+                uint32_t slot = 0;
+                if (lane == 0)
+                    slot = atomicAdd(&sm.ticket, wave_total);
+                slot = uniform_u32(slot) + before;
+#pragma unroll
+                for (uint32_t u = 0; u < kTrip; ++u)
+                    if (mine[u]) {
+                        if (slot < kSegCap)
+                            A[slot] = make_uint2(k[u], id[u]);
+                        ++slot;
+                    }
+            }
+        }
+        __syncthreads();
+        if (sm.ticket != n) // (cannot happen: the same keys were counted above)
+            return false;
+        if (!lds_bucket_sort(n, lo_r, hi_r, kout + at, iout + at, dyn, sm))
+            return false; // (a crowded bucket: ties)
+    }
+    return true;
+}
+
+// Group records of a worker's sorted range (cnt entries from position off of the list kf): fp64 sums, and the
+// maps of the running fp32 sum for the epoch guessed from the mass above the range plus the sums before the group.
+// kf_lds (optional): the worker's cnt sorted weights in LDS (outside L.sortk's first 16 KB), read instead of kf + off.
+__device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, size_t t_at, double mass, const GroupTable& T,
+                              const FinishLds& L, const uint32_t* kf_lds = nullptr)
+{
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t* src = kf_lds ? kf_lds : kf + off; // uniform
+    double* gs = reinterpret_cast<double*>(L.sortk); // [groups] estimate of the sum before each group
+    double* ge = gs + kMaxGroups;                    // [groups] and after it
+    const uint32_t groups = (cnt + kGroup - 1u) / kGroup;
+    if (kf_lds) // uniform: the copy is in place (its writers' barrier), nothing in device memory is waited for
+        lds_barrier();
+    else
+        __syncthreads();
+    for (uint32_t g = wave_id(); g < groups; g += kWaves) {
+        float q[4];
+        load_span(src, g * kGroup, min(kGroup, cnt - g * kGroup), q);
+        const double s = __ockl_wfred_add_f64((((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3]);
+        if (lane_id() == 0)
+            gs[g] = s;
+    }
+    __syncthreads();
+    for (uint32_t g0 = 0; g0 < groups; g0 += kThreads) { // (one trip unless the range is the fallback's)
+        const uint32_t g = g0 + tid;
+        const double v = g < groups ? gs[g] : 0.0;
+        double all;
+        const double incl = block_incl_scan_f64(v, all, sm.bs);
+        if (g < groups) {
+            T.sum[t_at + g] = v;
+            gs[g] = mass + (incl - v);
+            ge[g] = mass + incl;
+        }
+        mass += all;
+    }
+    __syncthreads();
+    for (uint32_t g = wave_id(); g < groups; g += kWaves) {
+        const uint32_t len = min(kGroup, cnt - g * kGroup);
+        float q[4];
+        load_span(src, g * kGroup, len, q);
+        const double guess = gs[g];
+        const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+        const seqfp::Step32 st = span_map(q, len, eg);
+        // the sum is expected to change binade inside the group (or starts at zero): records for its quarters
+        const double at_end = ge[g];
+        const bool split4 = uniform_u32((uint32_t)(eg == 0 || exponent_of((float)at_end) != eg)) != 0;
+        if (split4)
+            build_quarters(q, len, guess, T.quarters + (t_at + g) * 4u);
+        if (lane_id() == 0) {
+            T.d0[t_at + g] = st.d0;
+            T.d1[t_at + g] = st.d1;
+            T.cmax[t_at + g] = st.cmax;
+            T.start[t_at + g] = off + g * kGroup;
+            T.pack[t_at + g] = len | ((uint32_t)eg << 16) | (split4 ? kHasQuarters : 0u);
+        }
+    }
+}
+
+} // namespace mako

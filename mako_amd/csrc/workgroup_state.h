@@ -1,0 +1,73 @@
+// LDS records shared by the finishing kernels: the workgroup's scratch, views into the dynamic LDS block, and
+// the kernel arguments staged in LDS.
+#pragma once
+
+#include "sampler_common.h"
+
+namespace mako {
+
+struct alignas(16) FinishShared {
+    BlockScratch bs;
+    uint64_t tab[32];
+    uint32_t hist[256];
+    uint32_t run[256];
+    uint32_t flag;
+    uint32_t ticket;
+    uint32_t aux;
+    uint32_t soff[kMaxSlices + 1]; // first candidate of each slice in the row's flattened candidate list
+};
+
+// Views into the 64 KB dynamic LDS block; `cnt` (first pass) overlaps the two others (second pass).
+struct FinishLds {
+    FinishShared* sm;
+    uint32_t* cnt;              // [kSliceMax]
+    unsigned long long* sortk;  // [kSortMax]
+    uint32_t* wcount;           // [kWaves * 256]
+};
+
+// Kernel arguments that are handed on by reference to out-of-line device functions would be spilled to scratch
+// memory (a microsecond per access); the two finishing kernels keep their copies in LDS instead.
+struct alignas(16) ArgsLds {
+    mako_sample_desc d;
+    Scratch sc;
+    mako_sampling_params P; // the row's parameters
+};
+
+// The same in two steps for a kernel that learns its row late: the arguments first (no barrier), the row's parameters
+// (already in registers, the same in every lane) afterwards; the caller's next barrier publishes both.
+__device__ __forceinline__ void stage_args_only(const mako_sample_desc& d_arg, const Scratch& sc_arg, ArgsLds& a)
+{
+    const uint32_t* src_d = reinterpret_cast<const uint32_t*>(&d_arg);
+    const uint32_t* src_s = reinterpret_cast<const uint32_t*>(&sc_arg);
+    uint32_t* dst_d = reinterpret_cast<uint32_t*>(&a.d);
+    uint32_t* dst_s = reinterpret_cast<uint32_t*>(&a.sc);
+    for (uint32_t i = threadIdx.x; i < sizeof(mako_sample_desc) / 4; i += kThreads)
+        dst_d[i] = src_d[i];
+    for (uint32_t i = threadIdx.x; i < sizeof(Scratch) / 4; i += kThreads)
+        dst_s[i] = src_s[i];
+}
+__device__ __forceinline__ void stage_params(const mako_sampling_params& P, ArgsLds& a)
+{
+    if (threadIdx.x == 0)
+        a.P = P;
+}
+
+__device__ __forceinline__ void stage_args(const mako_sample_desc& d_arg, const Scratch& sc_arg, uint32_t row, ArgsLds& a)
+{
+    static_assert(sizeof(mako_sample_desc) % 4 == 0 && sizeof(Scratch) % 4 == 0, "word copies");
+    const uint32_t* src_d = reinterpret_cast<const uint32_t*>(&d_arg);
+    const uint32_t* src_s = reinterpret_cast<const uint32_t*>(&sc_arg);
+    uint32_t* dst_d = reinterpret_cast<uint32_t*>(&a.d);
+    uint32_t* dst_s = reinterpret_cast<uint32_t*>(&a.sc);
+    for (uint32_t i = threadIdx.x; i < sizeof(mako_sample_desc) / 4; i += kThreads)
+        dst_d[i] = src_d[i];
+    for (uint32_t i = threadIdx.x; i < sizeof(Scratch) / 4; i += kThreads)
+        dst_s[i] = src_s[i];
+    const uint32_t* src_p = reinterpret_cast<const uint32_t*>(d_arg.params + row);
+    uint32_t* dst_p = reinterpret_cast<uint32_t*>(&a.P);
+    if (threadIdx.x < sizeof(mako_sampling_params) / 4)
+        dst_p[threadIdx.x] = src_p[threadIdx.x];
+    __syncthreads();
+}
+
+} // namespace mako
