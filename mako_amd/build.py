@@ -7,8 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 # the C ABI, and one translation unit per kernel family (a kernel's register allocation then does not depend on
 # which other kernels exist; they also compile side by side)
-SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_for_sort.hip",
-           "k_plan_alone.hip", "k_sort.hip", "k_tail.hip"]
+SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_second.hip", "k_rows.hip", "k_sort.hip", "k_tail.hip"]
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 OUT = os.path.join(HERE, "libmako_sampler.so")
 
@@ -24,12 +23,14 @@ FLAGS = [
     "-fno-gpu-flush-denormals-to-zero",
     "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # every device function inlined into its kernel: no call stack, so the finishing kernels need no
-    # scratch memory (kernels that use scratch run far fewer workgroups at a time on this chip)
-    "-mllvm", "-amdgpu-function-calls=false",
     "-Wall",
     "-Wno-unused-command-line-argument",
 ]
+# every device function inlined into its kernel: no call stack, no scratch memory
+INLINE_ALL = ["-mllvm", "-amdgpu-function-calls=false"]
+# sort_kernel keeps the whole-row path, which it runs for a rare row only, out of line: inlined, it costs the
+# workers' sort 70 spilled vector registers
+PER_SOURCE = {"k_sort.hip": ["-DMAKO_WHOLE_ROW_CALL=__attribute__((noinline))"]}
 
 
 def build(verbose=False, extra=(), jobs=8):
@@ -38,7 +39,7 @@ def build(verbose=False, extra=(), jobs=8):
 
     def compile_one(name):
         obj = os.path.join(OBJ_DIR, os.path.splitext(name)[0] + ".o")
-        cmd = ["hipcc", *FLAGS, *extra, "-c", os.path.join(CSRC, name), "-o", obj]
+        cmd = ["hipcc", *FLAGS, *PER_SOURCE.get(name, INLINE_ALL), *extra, "-c", os.path.join(CSRC, name), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)

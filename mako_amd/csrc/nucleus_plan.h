@@ -8,10 +8,14 @@ namespace mako {
 // Plans a top_k == 0 row from the histogram of its weights (weight_bin(), exact masses): finds the bin by
 // which the nucleus must have ended and splits the weights above it over kWorkers workers by value.
 // Thread t brings the counts (c0, c1) and significand sums (s0, s1) of bins kBins-1-2t and kBins-2-2t.
-// Returns n0, the number of weights to sort; the plan is written to `plan` (flag left untouched).
-__device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, uint32_t c0, uint32_t c1,
-                                 unsigned long long s0, unsigned long long s1, BigPlan* plan, uint8_t* bin_worker,
-                                 const FinishLds& L, uint32_t& thr_bits)
+// `b_prune`: bins below it hold weights the nucleus cannot reach (prune_bin()); the second pass kept none of them,
+// so the list never extends below it.
+// Returns n0, the number of weights to sort; the plan is written to `plan` (in LDS; flag left untouched).
+// total64 receives the sum of q over the row's candidates (the bins' exact masses, added from the top bin down in a
+// fixed order), count_all their number; with no candidate at all nothing else is done and 0 is returned.
+__device__ uint32_t plan_nucleus(const mako_sampling_params& P, uint32_t c0, uint32_t c1, unsigned long long s0,
+                                 unsigned long long s1, uint32_t b_prune, BigPlan* plan, const FinishLds& L,
+                                 uint32_t& thr_bits, double& total64, uint32_t& count_all_out)
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
@@ -22,7 +26,6 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         return __longlong_as_double((long long)(1023ull + e - 150ull) << 52);
     };
     const double m0 = (double)s0 * scale(b0), m1 = (double)s1 * scale(b1);
-    const double want = (double)P.top_p * total64;
     uint32_t* w_hi = L.wcount;            // highest bin of each worker
     uint32_t* w_lo = L.wcount + kWorkers; // lowest bin
     uint32_t* w_off = L.wcount + 2 * kWorkers;
@@ -42,7 +45,7 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         sm.bs.u64[wave_id()] = cnt_w;
     }
     __syncthreads();
-    double pre_m = 0;
+    double pre_m = 0, all_m = 0;
     uint32_t pre_c = 0, count_all = 0;
     for (int w = 0; w < kWaves; ++w) {
         const double x = sm.bs.f64[w];
@@ -51,8 +54,14 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
             pre_m += x;
             pre_c += y;
         }
+        all_m += x;
         count_all += y;
     }
+    total64 = all_m;
+    count_all_out = count_all;
+    if (count_all == 0)
+        return 0;
+    const double want = (double)P.top_p * total64;
     MAKO_STAMP(20);
     const double incl = pre_m + mass_w;
     const uint32_t above0 = pre_c + cnt_w - (c0 + c1), above1 = above0 + c0;
@@ -72,16 +81,19 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
     uint32_t before = reached_w - reached;
     for (int w = 0; w < kWaves; ++w)
         before += w < wave_id() ? sm.hist[w] : 0u;
-    if (r0 && before + 1 == 2) {
+    if (r0 && before + 1 == 2)
         sm.ticket = b0;
-        sm.flag = above0 + c0;
-    } else if (r1 && before + (uint32_t)r0 + 1 == 2) {
+    else if (r1 && before + (uint32_t)r0 + 1 == 2)
         sm.ticket = b1;
+    __syncthreads();
+    const uint32_t b_lo = max(sm.ticket, b_prune);
+    // (every bin has one holder: the holder of the lowest bin taken knows how many weights lie at or above it)
+    if (b0 == b_lo)
+        sm.flag = above0 + c0;
+    else if (b1 == b_lo)
         sm.flag = above1 + c1;
-    }
     __syncthreads();
     MAKO_STAMP(22);
-    const uint32_t b_lo = sm.ticket;
     thr_bits = bin_lo_key(b_lo);
     const uint32_t n0 = sm.flag;
     auto worker_of = [&](uint32_t b, uint32_t c, uint32_t above) {
@@ -107,10 +119,9 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         plan->mass[wk0] = incl - m0 - m1;
     if (wk1 != kNone && w_hi[wk1] == b1)
         plan->mass[wk1] = incl - m1;
-    bin_worker[b0] = (uint8_t)wk0; // (kNone -> 0xff)
-    bin_worker[b1] = (uint8_t)wk1;
     if (tid < kWorkers) {
-        plan->cursor[tid] = 0;
+        plan->bin_lo[tid] = w_lo[tid]; // (kNone for a worker without weights: bin_lo > bin_hi)
+        plan->bin_hi[tid] = w_hi[tid];
         plan->key_lo[tid] = bin_lo_key(min(w_lo[tid], kBins - 1u));
         plan->key_hi[tid] = bin_hi_key(w_hi[tid]);
         plan->off[tid] = w_cnt[tid] ? w_off[tid] : 0u;

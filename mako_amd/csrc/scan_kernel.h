@@ -71,10 +71,15 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
         }
     }
     if (row == 0 && slice == 0 && wave_id() == 1) { // how the second pass will be cut up
-        uint32_t piece_len, busy;
-        const uint32_t pieces = second_pass_pieces(d, gridDim.x, slice_len, cus, piece_len, busy);
+        uint32_t piece_len, busy, rows;
+        const uint32_t pieces = second_pass_pieces(d, gridDim.x, slice_len, cus, sc.work_rows, piece_len, busy, rows);
         if (lane_id() == 0)
-            *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(pieces, piece_len, busy, 0u);
+            *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(pieces, piece_len, busy, rows);
+    }
+    if (cls == kNucleus) { // the row's weight histogram starts empty: every slice clears its share of the bins
+        const uint32_t per = (kBins + gridDim.x - 1u) / gridDim.x;
+        for (uint32_t b = slice * per + tid; b < min((slice + 1u) * per, kBins); b += kThreads)
+            sc.bins[(size_t)row * kBins + b] = 0ull;
     }
     // ReasoningBudget::forced's question (src/server/openai.cpp:598-602), answered in the same pass over the logits
     bool want_above = false;

@@ -323,7 +323,7 @@ __device__ __forceinline__ void topk_row(const mako_sample_desc& d, const Scratc
                 sc.plan[row].total64 = (double)m;
                 sc.plan[row].n0 = argidx;
                 sc.plan[row].flag = 2;
-                sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
+                sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = (row << 8) | kItemWhole;
             }
             return;
         }
