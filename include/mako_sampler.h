@@ -46,7 +46,7 @@ typedef struct mako_sampling_params {
 #define MAKO_PATH_GREEDY 1u   /* argmax of the (masked) raw logits */
 #define MAKO_PATH_FALLBACK 2u /* no candidate survived: most likely token (sampler.cpp:37-38) */
 #define MAKO_PATH_TOPK 3u     /* resolved from the per-slice top-k candidates */
-#define MAKO_PATH_NUCLEUS 4u  /* top_k == 0: nucleus resolved from the per-slice candidates */
+#define MAKO_PATH_NUCLEUS 4u  /* top_k == 0: second pass over the row, nucleus sorted by the row's workers */
 #define MAKO_PATH_GENERAL 5u  /* whole-row sort path */
 #define MAKO_PATH_FORCED 6u   /* not sampled: force_token / close_token took the row */
 

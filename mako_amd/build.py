@@ -28,9 +28,12 @@ FLAGS = [
 ]
 # every device function inlined into its kernel: no call stack, no scratch memory
 INLINE_ALL = ["-mllvm", "-amdgpu-function-calls=false"]
-# sort_kernel keeps the whole-row path, which it runs for a rare row only, out of line: inlined, it costs the
-# workers' sort 70 spilled vector registers
-PER_SOURCE = {"k_sort.hip": ["-DMAKO_WHOLE_ROW_CALL=__attribute__((noinline))"]}
+# Kernels that run the whole-row path for a rare row only keep it out of line (inlined, it costs sort_kernel's workers
+# 70 spilled vector registers); tail_kernel keeps the rows it finishes beside its tails out of line as well
+NOINLINE = "__attribute__((noinline))"
+PER_SOURCE = {"k_sort.hip": ["-DMAKO_WHOLE_ROW_CALL=" + NOINLINE],
+              "k_rows.hip": ["-DMAKO_WHOLE_ROW_CALL=" + NOINLINE],
+              "k_tail.hip": ["-DMAKO_WHOLE_ROW_CALL=" + NOINLINE, "-DMAKO_ROWS_CALL=" + NOINLINE]}
 
 
 def build(verbose=False, extra=(), jobs=8):

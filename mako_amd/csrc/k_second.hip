@@ -1,4 +1,4 @@
-// second_kernel's variants: the second pass over the top_k == 0 rows, and beside it the rows that need none.
+// second_kernel's variants: the second pass over the top_k == 0 rows.
 #include "launch.h"
 #include "sampler_kernels.h"
 
@@ -7,7 +7,8 @@ namespace {
 template <bool VEC, int KH>
 void launch_one(uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices)
 {
-    hipLaunchKernelGGL((second_kernel<VEC, KH>), dim3(wgs), dim3(kThreads), kSecondLds, st, d, sc, slices);
+    hipLaunchKernelGGL((second_kernel<VEC, KH>), dim3(wgs), dim3(kThreads), kSecondLds, st, d, sc, slices,
+                       (d.n_vocab + kPieceLen - 1u) / kPieceLen);
 }
 template <bool VEC>
 void launch_vec(int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices)
@@ -32,7 +33,6 @@ void launch_second(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sa
 
 hipError_t init_second_kernels()
 {
-    static_assert(kSecondLds >= kDynLds, "finish_row() uses the finishing kernels' LDS layout");
     const void* kernels[] = {(const void*)second_kernel<true, 0>, (const void*)second_kernel<false, 0>,
                              (const void*)second_kernel<true, 2>, (const void*)second_kernel<false, 2>,
                              (const void*)second_kernel<true, 8>, (const void*)second_kernel<false, 8>};

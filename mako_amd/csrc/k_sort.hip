@@ -5,10 +5,9 @@
 #include "sampler_kernels.h"
 
 namespace mako {
-void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t nucleus_rows,
-                 uint32_t list_rows)
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t list_cap)
 {
-    hipLaunchKernelGGL(sort_kernel, dim3(nucleus_rows * kWorkers + list_rows), dim3(kThreads), kSortLds, st, d, sc, slices);
+    hipLaunchKernelGGL(sort_kernel, dim3(list_cap), dim3(kThreads), kSortLds, st, d, sc, slices);
 }
 
 hipError_t init_sort_kernels()

@@ -22,16 +22,15 @@ hipError_t init_tail_kernels();
 // scan_kernel<vec, kh, above>, grid = (slices, rows), `lds` bytes of dynamic LDS
 void launch_scan(bool vec, int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d,
                  const Scratch& sc, uint32_t slice_len, uint32_t cus);
-// second_kernel<vec, kh> on `wgs` workgroups: the second pass's pieces, then one workgroup per row
+// second_kernel<vec, kh> on `wgs` workgroups: the second pass's pieces
 void launch_second(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc,
                    uint32_t slices);
-// rows_kernel, one workgroup per row, for a batch without top_k == 0 rows: <false> when sort_kernel follows (it has
-// the whole-row path), <true> when rows_kernel is the last kernel of the batch
-void launch_rows(bool inline_general, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices);
-// sort_kernel: kWorkers workgroups per top_k == 0 row (`nucleus_rows` of them at most), then one per row that can
-// be on the whole-row list (`list_rows`).  Workgroups beyond the lists leave at once, but each of them still has to
-// be dispatched.  tail_kernel takes one workgroup per possible wide row.
-void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t nucleus_rows,
-                 uint32_t list_rows);
-void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows);
+// rows_kernel, one workgroup per row, for a batch without top_k == 0 rows; `any_general`: some row may be without a
+// top-p (the whole-row path then has to keep the order of top-k alone)
+void launch_rows(bool any_general, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices);
+// sort_kernel: `list_cap` workgroups for its work list (room for the longest list the batch can produce; workgroups
+// beyond the list leave at once, but each of them still has to be dispatched).  tail_kernel takes one workgroup per
+// possible top_k == 0 row (`tail_cap`), then one per row for the rows that need no second pass.
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t list_cap);
+void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t tail_cap);
 } // namespace mako

@@ -83,12 +83,10 @@ uint32_t slice_len_for(uint32_t n_vocab, uint32_t slices)
     return (len + 3u) & ~3u;
 }
 
-// Most pieces the second pass cuts a row of n_vocab logits into: slices, or blocks of 4096 logits when that many
-// workgroups fit one round (decided on the device, see second_pass_pieces()).
-uint32_t pieces_max_for(uint32_t n_vocab)
+// Pieces the second pass cuts a row of n_vocab logits into.
+uint32_t pieces_for(uint32_t n_vocab)
 {
-    const uint32_t slices = std::max(1u, (n_vocab + mako::kSliceMax - 1) / mako::kSliceMax);
-    return std::min<uint32_t>(mako::kMaxSlices, std::max(slices, (n_vocab + 4095u) / 4096u));
+    return std::max(1u, (n_vocab + mako::kPieceLen - 1u) / mako::kPieceLen);
 }
 
 } // namespace
@@ -105,8 +103,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
 {
     if (!out || max_rows == 0 || max_vocab == 0)
         return MAKO_ERR_INVALID_ARG;
-    // (kMaxSlices slices of kSliceMax logits; one logit fewer so that a histogram bin's count fits its 20 bits)
-    if (mako_sampler_slices(max_vocab) > mako::kMaxSlices || max_vocab >= (1u << (64 - mako::kBinSumBits)))
+    // (kMaxSlices slices of kSliceMax logits)
+    if (mako_sampler_slices(max_vocab) > mako::kMaxSlices || pieces_for(max_vocab) > 64u || max_vocab >= (1u << 20))
         return MAKO_ERR_INVALID_ARG;
     mako_sampler_ctx* ctx = new (std::nothrow) mako_sampler_ctx;
     if (!ctx)
@@ -132,8 +130,6 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap));
     MAKO_HIP(ctx, dev_alloc(&sc.plan, (size_t)max_rows));
     MAKO_HIP(ctx, hipMemset(sc.plan, 0, (size_t)max_rows * sizeof(mako::BigPlan)));
-    MAKO_HIP(ctx, dev_alloc(&sc.bins, (size_t)max_rows * mako::kBins));
-    MAKO_HIP(ctx, hipMemset(sc.bins, 0, (size_t)max_rows * mako::kBins * sizeof(unsigned long long)));
     MAKO_HIP(ctx, dev_alloc(&sc.wbuf, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.cnt, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.key[0], rv));
@@ -150,17 +146,18 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.gt.start, rg));
     MAKO_HIP(ctx, dev_alloc(&sc.gt.pack, rg));
     MAKO_HIP(ctx, dev_alloc(&sc.gt.quarters, rg * 4));
-    sc.pieces_cap = pieces_max_for(max_vocab);
+    sc.pieces_cap = pieces_for(max_vocab);
     MAKO_HIP(ctx, dev_alloc(&sc.piece_idx, rv));
-    MAKO_HIP(ctx, dev_alloc(&sc.piece_tab, (size_t)max_rows * sc.pieces_cap * (mako::kBins + 1u)));
+    MAKO_HIP(ctx, dev_alloc(&sc.piece_tab, (size_t)max_rows * sc.pieces_cap * (mako::kWorkers + 1u)));
+    MAKO_HIP(ctx, dev_alloc(&sc.piece_mass, (size_t)max_rows * sc.pieces_cap * mako::kWorkers));
+    MAKO_HIP(ctx, dev_alloc(&sc.piece_sum, (size_t)max_rows * sc.pieces_cap));
+    MAKO_HIP(ctx, dev_alloc(&sc.piece_cnt, (size_t)max_rows * sc.pieces_cap));
     MAKO_HIP(ctx, dev_alloc(&sc.work_n, 8));
     MAKO_HIP(ctx, hipMemset(sc.work_n, 0, 8 * sizeof(uint32_t)));
     MAKO_HIP(ctx, dev_alloc(&sc.work_rows, (size_t)max_rows));
     MAKO_HIP(ctx, hipMemset(sc.work_rows, 0, (size_t)max_rows * sizeof(uint32_t)));
     MAKO_HIP(ctx, dev_alloc(&sc.work_sort, (size_t)max_rows * mako::kWorkers));
     MAKO_HIP(ctx, dev_alloc(&sc.work_tail, (size_t)max_rows));
-    MAKO_HIP(ctx, dev_alloc(&sc.row_ticket, (size_t)max_rows));
-    MAKO_HIP(ctx, hipMemset(sc.row_ticket, 0, (size_t)max_rows * sizeof(uint32_t)));
     MAKO_HIP(ctx, hipDeviceSynchronize());
     // the kernels overlay up to 64 KB of dynamic LDS (second_kernel and sort_kernel more) on a few KB of static LDS
     MAKO_HIP(ctx, mako::init_scan_kernels());
@@ -177,8 +174,8 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {sc.piece_idx, sc.piece_tab, sc.row_ticket, sc.work_n, sc.work_rows, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
-                    sc.cand_w, sc.cand_i, sc.bins, sc.plan,
+    void* ptrs[] = {sc.piece_idx, sc.piece_tab, sc.piece_mass, sc.piece_sum, sc.piece_cnt, sc.work_n, sc.work_rows, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
+                    sc.cand_w, sc.cand_i, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
                     ctx->st_hist,  ctx->st_hcnt, ctx->st_hlen,  ctx->st_draft, ctx->st_tokens, ctx->st_acc};
@@ -276,42 +273,36 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
     // which kernels have work: all of them unless the caller's host copy of the parameters says otherwise; and how
     // many workgroups the launches behind the scan can need
     bool any_nucleus = true, any_general = true;
-    uint32_t nucleus_rows = d.n_rows, list_rows = d.n_rows;
+    uint32_t nucleus_rows = d.n_rows;
     if (params_host) {
         any_nucleus = any_general = false;
-        uint32_t n_nucleus = 0, n_other = 0;
+        uint32_t n_nucleus = 0;
         for (uint32_t r = 0; r < d.n_rows; ++r) {
             const mako::RowClass c = mako::classify(params_host[r]);
             any_nucleus |= c == mako::kNucleus;
             any_general |= c == mako::kGeneral;
             n_nucleus += c == mako::kNucleus;
-            n_other += c == mako::kTopK || c == mako::kGeneral;
         }
         nucleus_rows = n_nucleus;
-        list_rows = n_other;
     }
-    const bool launch_sort = any_nucleus || any_general;
-    // The second pass cuts top_k == 0 rows into pieces of one to four blocks of 4096 logits (decided on the device:
-    // pieces finer than slices only while all of them fit one round of workgroups), so this many of its workgroups
-    // can have work; one more per row follows them.
-    const uint32_t pieces_max = pieces_max_for(d.n_vocab);
-    const uint32_t second_wgs = std::max(nucleus_rows * slices, std::min(ctx->cus, nucleus_rows * pieces_max)) + d.n_rows;
     MAKO_MARK(0);
     mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, ctx->sc, slice_len, ctx->cus);
     MAKO_MARK(1);
-    // top_k == 0 rows: second pass, then planned and sorted by the rows' workers, then cut and drawn from; the stages
-    // talk through kernel boundaries (handing over inside a kernel costs as much as a launch on this chip).  The
-    // other rows are finished beside the second pass.
-    if (any_nucleus)
-        mako::launch_second(vec, kh, second_wgs, st, d, ctx->sc, slices);
-    else
-        mako::launch_rows(!launch_sort, st, d, ctx->sc, slices);
-    MAKO_MARK(2);
-    if (launch_sort)
-        mako::launch_sort(st, d, ctx->sc, slices, nucleus_rows, std::max(list_rows, 1u));
-    MAKO_MARK(3);
-    if (any_nucleus)
-        mako::launch_tail(st, d, ctx->sc, std::max(nucleus_rows, 1u));
+    // top_k == 0 rows: second pass, then sorted by the rows' workers, then cut and drawn from; the stages talk
+    // through kernel boundaries (handing over inside a kernel costs as much as a launch on this chip).  The other
+    // rows are finished beside the tails, or, in a batch without top_k == 0 rows, by a launch of their own.
+    if (any_nucleus) {
+        mako::launch_second(vec, kh, nucleus_rows * pieces_for(d.n_vocab), st, d, ctx->sc, slices);
+        MAKO_MARK(2);
+        // (the work list: up to kWorkers entries per top_k == 0 row)
+        mako::launch_sort(st, d, ctx->sc, slices, std::max(nucleus_rows, 1u) * mako::kWorkers);
+        MAKO_MARK(3);
+        mako::launch_tail(st, d, ctx->sc, slices, nucleus_rows);
+    } else {
+        mako::launch_rows(any_general, st, d, ctx->sc, slices);
+        MAKO_MARK(2);
+        MAKO_MARK(3);
+    }
     MAKO_MARK(4);
 #undef MAKO_MARK
     ctx->profiled = prof;

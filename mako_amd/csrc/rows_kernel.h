@@ -9,14 +9,15 @@ namespace mako {
 // One workgroup finishes row `row`: a forced token is written; a greedy row takes its argmax; a top-k row is
 // resolved from the candidate lists.  A top_k == 0 row is only looked at for a forced token: its weights take the
 // second pass and sort_kernel.  (sm.tab must hold the exp2 table; all threads call.)
-// INLINE_GENERAL: sort_kernel will not be launched for this batch (the host saw no row that needs it), so a row
-// that turns out to need the whole-row path after all is given it here; otherwise such a row is put on sort_kernel's
-// list.
-template <bool INLINE_GENERAL>
-__device__ __forceinline__ void finish_row(const mako_sample_desc& d, const Scratch& sc, const mako_sampling_params& P,
+// A row that needs the whole-row path is given it here (general_row<SITE>; SITE 1 leaves out the order of top-k without
+// top-p, for batches whose host copy of the parameters shows a top-p on every sampled row).
+#ifndef MAKO_ROWS_CALL
+#define MAKO_ROWS_CALL __forceinline__
+#endif
+template <int SITE>
+__device__ MAKO_ROWS_CALL void finish_row(const mako_sample_desc& d, const Scratch& sc, const mako_sampling_params& P,
                                            uint32_t row, uint32_t slices, const FinishLds& L)
 {
-    constexpr bool inline_general = INLINE_GENERAL;
     const uint32_t tid = threadIdx.x;
     const RowClass cls = classify(P);
     MAKO_STAMP(0);
@@ -68,23 +69,14 @@ __device__ __forceinline__ void finish_row(const mako_sample_desc& d, const Scra
         return;
     }
     if (topk_takes_whole_row(cls, any_overflow, n_cands)) {
-        if constexpr (inline_general) {
-            general_row<1>(d, sc, row, P, m, argidx, L);
-            return;
-        }
-        if (tid == 0) {
-            sc.plan[row].total64 = (double)m; // carries the row maximum and its first index to the whole-row path
-            sc.plan[row].n0 = argidx;
-            sc.plan[row].flag = 2;
-            sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = (row << 8) | kItemWhole;
-        }
+        general_row<SITE>(d, sc, row, P, m, argidx, L);
         return;
     }
-    topk_row<inline_general>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
+    topk_row<SITE>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
 }
 
 // grid = rows workgroups: batches without top_k == 0 rows (the host's copy of the parameters says so).
-template <bool INLINE_GENERAL>
+template <int SITE>
 __global__ __launch_bounds__(kThreads) void rows_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
 {
     const Scratch& sc_arg = sc_val;
@@ -105,7 +97,7 @@ __global__ __launch_bounds__(kThreads) void rows_kernel(mako_sample_desc d_arg, 
     L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
     L.sortk = s_dyn64;
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
-    finish_row<INLINE_GENERAL>(s_args.d, s_args.sc, s_args.P, row, slices, L);
+    finish_row<SITE>(s_args.d, s_args.sc, s_args.P, row, slices, L);
 }
 
 } // namespace mako

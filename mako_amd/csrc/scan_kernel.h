@@ -70,16 +70,10 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
             sc.work_n[1] = 0;
         }
     }
-    if (row == 0 && slice == 0 && wave_id() == 1) { // how the second pass will be cut up
-        uint32_t piece_len, busy, rows;
-        const uint32_t pieces = second_pass_pieces(d, gridDim.x, slice_len, cus, sc.work_rows, piece_len, busy, rows);
+    if (row == 0 && slice == 0 && wave_id() == 1) { // the rows that take the second pass
+        const uint32_t rows = nucleus_rows(d, sc.work_rows);
         if (lane_id() == 0)
-            *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(pieces, piece_len, busy, rows);
-    }
-    if (cls == kNucleus) { // the row's weight histogram starts empty: every slice clears its share of the bins
-        const uint32_t per = (kBins + gridDim.x - 1u) / gridDim.x;
-        for (uint32_t b = slice * per + tid; b < min((slice + 1u) * per, kBins); b += kThreads)
-            sc.bins[(size_t)row * kBins + b] = 0ull;
+            sc.work_n[4] = rows;
     }
     // ReasoningBudget::forced's question (src/server/openai.cpp:598-602), answered in the same pass over the logits
     bool want_above = false;
@@ -109,7 +103,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
     for (uint32_t j = 0; j < 16; ++j)
         best = fmaxf(best, wv[j]);
     const uint32_t bkey = order_key(best);
-    const bool emits = cls == kTopK || cls == kNucleus;
+    const bool emits = cls == kTopK; // (top_k == 0 rows take the second pass: nobody reads candidates of theirs)
     const uint32_t wmax = __ockl_wfred_max_u32(bkey);
     uint32_t wkth = 0;
     if (emits) {
