@@ -155,7 +155,7 @@ def main():
 
     # per-kernel split of a batch: HIP events recorded by the library on the launch stream, a few extra steps
     ctx.set_profile(True)
-    split = np.zeros(api.KERNEL_COUNT)
+    split = np.zeros(6)
     n_split = min(a.steps, 50)
     for i in range(n_split):
         step(a.warmup + a.steps + i)
@@ -255,9 +255,10 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
                      "bytes_per_launch": batch_bytes,
-                     "kernel": "scan + second + sort + tail kernels (the four launches of one batch)",
+                     "kernel": "scan + finish + plan + partition + sort + tail kernels (the six launches of one batch)",
                      "launch_ms": ms_per_step,
-                     "kernel_ms": dict(zip(api.KERNEL_NAMES, [float(x) for x in split])),
+                     "kernel_ms": dict(zip(["scan_kernel", "finish_kernel", "plan_kernel", "partition_kernel", "sort_kernel", "tail_kernel"],
+                                           [float(x) for x in split])),
                      "scan_kernel_gbs": batch_bytes / (split[0] * 1e-3) / 1e9},
         "host_pointer_rows_per_s": host_rate,
         "overlapped_batches": overlapped,

@@ -46,7 +46,7 @@ typedef struct mako_sampling_params {
 #define MAKO_PATH_GREEDY 1u   /* argmax of the (masked) raw logits */
 #define MAKO_PATH_FALLBACK 2u /* no candidate survived: most likely token (sampler.cpp:37-38) */
 #define MAKO_PATH_TOPK 3u     /* resolved from the per-slice top-k candidates */
-#define MAKO_PATH_NUCLEUS 4u  /* top_k == 0: second pass over the row, nucleus sorted by the row's workers */
+#define MAKO_PATH_NUCLEUS 4u  /* top_k == 0: nucleus resolved from the per-slice candidates */
 #define MAKO_PATH_GENERAL 5u  /* whole-row sort path */
 #define MAKO_PATH_FORCED 6u   /* not sampled: force_token / close_token took the row */
 
@@ -126,7 +126,7 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
 /* The same call for a caller that still has the batch's parameters in HOST memory (the SamplingParams originate
  * there, src/gen/session.hpp:19-21): params_host[n_rows] must hold the same values as desc->params.  The call
  * looks at them on the calling thread and leaves out the kernels that no row of the batch needs (a batch without
- * top_k == 0 rows takes two launches instead of four).  The results never depend on it; null = the call above. */
+ * top_k == 0 rows takes two launches instead of six).  The results never depend on it; null = the call above. */
 int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_desc* desc,
                                      const mako_sampling_params* params_host, void* stream);
 
@@ -144,11 +144,11 @@ int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t
 const char* mako_sampler_last_error(const mako_sampler_ctx* ctx);
 
 /* Per-kernel timing for benchmarks (no counterpart in the reference).  While enabled, every
- * mako_sampler_sample_batch records HIP events on its stream around its four kernels;
+ * mako_sampler_sample_batch records HIP events on its stream around its six kernels;
  * mako_sampler_kernel_times waits for the last recorded batch and returns the milliseconds of
- * scan_kernel, second_kernel (rows_kernel for a batch without top_k == 0 rows), sort_kernel and
- * tail_kernel in out_ms[0..3].  Off by default. */
-#define MAKO_SAMPLER_KERNELS 4
+ * scan_kernel, finish_kernel, plan_kernel, partition_kernel, sort_kernel and tail_kernel in
+ * out_ms[0..5].  Off by default. */
+#define MAKO_SAMPLER_KERNELS 6
 int mako_sampler_set_profile(mako_sampler_ctx* ctx, int enabled);
 int mako_sampler_kernel_times(mako_sampler_ctx* ctx, float* out_ms);
 

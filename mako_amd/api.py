@@ -81,9 +81,6 @@ class Desc(C.Structure):
     ]
 
 
-KERNEL_COUNT = 4  # MAKO_SAMPLER_KERNELS
-KERNEL_NAMES = ["scan_kernel", "second_kernel", "sort_kernel", "tail_kernel"]
-
 EXPORTS = [
     "mako_sampler_create",
     "mako_sampler_destroy",
@@ -164,8 +161,8 @@ class SamplerContext:
             raise MakoError("mako_sampler_set_profile: %d %s" % (rc, self.last_error()))
 
     def kernel_times_ms(self):
-        """(scan, second / rows, sort, tail) kernel milliseconds of the last batch sampled while profiling was on."""
-        out = (C.c_float * KERNEL_COUNT)()
+        """(scan, finish, plan, partition, sort, tail) kernel milliseconds of the last batch sampled while profiling was on."""
+        out = (C.c_float * 6)()
         rc = self.lib.mako_sampler_kernel_times(self.ptr, out)
         if rc != MAKO_OK:
             raise MakoError("mako_sampler_kernel_times: %d %s" % (rc, self.last_error()))

@@ -7,7 +7,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 # the C ABI, and one translation unit per kernel family (a kernel's register allocation then does not depend on
 # which other kernels exist; they also compile side by side)
-SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_second.hip", "k_rows.hip", "k_sort.hip", "k_tail.hip"]
+SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_for_sort.hip",
+           "k_plan_alone.hip", "k_sort.hip", "k_tail.hip"]
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 OUT = os.path.join(HERE, "libmako_sampler.so")
 
@@ -23,17 +24,12 @@ FLAGS = [
     "-fno-gpu-flush-denormals-to-zero",
     "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # every device function inlined into its kernel: no call stack, so the finishing kernels need no
+    # scratch memory (kernels that use scratch run far fewer workgroups at a time on this chip)
+    "-mllvm", "-amdgpu-function-calls=false",
     "-Wall",
     "-Wno-unused-command-line-argument",
 ]
-# every device function inlined into its kernel: no call stack, no scratch memory
-INLINE_ALL = ["-mllvm", "-amdgpu-function-calls=false"]
-# Kernels that run the whole-row path for a rare row only keep it out of line (inlined, it costs sort_kernel's workers
-# 70 spilled vector registers); tail_kernel keeps the rows it finishes beside its tails out of line as well
-NOINLINE = "__attribute__((noinline))"
-PER_SOURCE = {"k_sort.hip": ["-DMAKO_WHOLE_ROW_CALL=" + NOINLINE],
-              "k_rows.hip": ["-DMAKO_WHOLE_ROW_CALL=" + NOINLINE],
-              "k_tail.hip": ["-DMAKO_WHOLE_ROW_CALL=" + NOINLINE, "-DMAKO_ROWS_CALL=" + NOINLINE]}
 
 
 def build(verbose=False, extra=(), jobs=8):
@@ -42,7 +38,7 @@ def build(verbose=False, extra=(), jobs=8):
 
     def compile_one(name):
         obj = os.path.join(OBJ_DIR, os.path.splitext(name)[0] + ".o")
-        cmd = ["hipcc", *FLAGS, *PER_SOURCE.get(name, INLINE_ALL), *extra, "-c", os.path.join(CSRC, name), "-o", obj]
+        cmd = ["hipcc", *FLAGS, *extra, "-c", os.path.join(CSRC, name), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)

@@ -10,7 +10,6 @@
 // Wavefront reductions and scans of the device library (DPP row shifts and broadcasts: a dozen instructions where
 // a shuffle-based butterfly pays six trips through the LDS crossbar).
 extern "C" __device__ uint32_t __ockl_wfred_add_u32(uint32_t);
-extern "C" __device__ unsigned long long __ockl_wfred_add_u64(unsigned long long);
 extern "C" __device__ uint32_t __ockl_wfred_min_u32(uint32_t);
 extern "C" __device__ uint32_t __ockl_wfred_max_u32(uint32_t);
 extern "C" __device__ unsigned long long __ockl_wfred_max_u64(unsigned long long);

@@ -1,13 +1,18 @@
-// sort_kernel: the top_k == 0 rows planned and their nuclei sorted by the rows' workers; narrow and whole-row rows
-// finished by one worker.
+// partition_kernel and sort_kernel: the wide rows' weights handed to their workers and sorted; narrow and
+// whole-row rows finished by one worker.
 #define MAKO_EMIT_SORT_KERNELS
 #include "launch.h"
 #include "sampler_kernels.h"
 
 namespace mako {
-void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t list_cap)
+void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows)
 {
-    hipLaunchKernelGGL(sort_kernel, dim3(list_cap), dim3(kThreads), kSortLds, st, d, sc, slices);
+    hipLaunchKernelGGL(partition_kernel, dim3(kWorkers, grid_rows), dim3(kThreads), 0, st, d, sc);
+}
+
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows)
+{
+    hipLaunchKernelGGL(sort_kernel, dim3(kWorkers, grid_rows), dim3(kThreads), kSortLds, st, d, sc, slices);
 }
 
 hipError_t init_sort_kernels()

@@ -1,9 +1,7 @@
 // Launchers of the sampler's kernels.  Every kernel family is compiled as a translation unit of its own (k_*.hip):
 // the compiler's register allocation for a kernel otherwise depends on which other kernels share its inlined device
-// functions (sort_kernel lost 2.4 us per batch to spills when kernels with the whole-row path were compiled beside
-// it).  Each init function raises the dynamic LDS limit of its family's kernels.
-// Every kernel takes the context's record (`sc`, the host copy) by value: its first loads then need no trip to
-// memory for the record itself, and no launch depends on a copy of it in device memory.
+// functions (sort_kernel lost 2.4 us per batch to spills when plan_kernel variants with the whole-row path were
+// compiled beside it).  Each init function raises the dynamic LDS limit of its family's kernels.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -14,23 +12,29 @@ namespace mako {
 struct Scratch;
 
 hipError_t init_scan_kernels();
-hipError_t init_second_kernels();
-hipError_t init_rows_kernels();
+hipError_t init_finish_kernels();
+hipError_t init_plan_for_sort();
+hipError_t init_plan_alone();
 hipError_t init_sort_kernels();
 hipError_t init_tail_kernels();
 
 // scan_kernel<vec, kh, above>, grid = (slices, rows), `lds` bytes of dynamic LDS
+// (`sc`: the HOST copy of the context's record; scan, partition, sort and tail kernels take it by value, so that their
+// first loads need no trip to memory for the record itself; finish and plan kernels take the device copy's address)
 void launch_scan(bool vec, int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d,
                  const Scratch& sc, uint32_t slice_len, uint32_t cus);
-// second_kernel<vec, kh> on `wgs` workgroups: the second pass's pieces
-void launch_second(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc,
+// finish_kernel<vec, kh> on `wgs` workgroups
+void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch* sc,
                    uint32_t slices);
-// rows_kernel, one workgroup per row, for a batch without top_k == 0 rows; `any_general`: some row may be without a
-// top-p (the whole-row path then has to keep the order of top-k alone)
-void launch_rows(bool any_general, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices);
-// sort_kernel: `list_cap` workgroups for its work list (room for the longest list the batch can produce; workgroups
-// beyond the list leave at once, but each of them still has to be dispatched).  tail_kernel takes one workgroup per
-// possible top_k == 0 row (`tail_cap`), then one per row for the rows that need no second pass.
-void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t list_cap);
-void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t tail_cap);
+// plan_kernel, one workgroup per row: <false> when sort_kernel follows (it has the whole-row path), <true> when
+// plan_kernel is the last kernel of the batch
+void launch_plan_for_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
+void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
+// partition_kernel and sort_kernel serve the same work list, workgroup i its entry i: `grid_rows` * kWorkers workgroups
+// must cover the longest list the batch can produce (kWorkers entries per top_k == 0 row, one per other sampled
+// row); tail_kernel takes one workgroup per possible wide row.  Workgroups beyond the lists leave at once, but each
+// of them still has to be dispatched.
+void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows); // (host copy, by value)
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows); // (host copy)
+void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows); // (host copy, by value)
 } // namespace mako

@@ -36,7 +36,8 @@ __global__ void debug_div_kernel(const float* a, const float* b, float* y, uint3
 struct mako_sampler_ctx {
     int device = 0;
     uint32_t max_rows = 0, max_vocab = 0, max_hist = 0;
-    mako::Scratch sc{}; // handed to every kernel by value
+    mako::Scratch sc{};
+    mako::Scratch* sc_dev = nullptr; // the same record in device memory: the kernels take a pointer to it
     // staging for the host-pointer call
     float* st_logits = nullptr;
     mako_sampling_params* st_params = nullptr;
@@ -83,12 +84,6 @@ uint32_t slice_len_for(uint32_t n_vocab, uint32_t slices)
     return (len + 3u) & ~3u;
 }
 
-// Pieces the second pass cuts a row of n_vocab logits into.
-uint32_t pieces_for(uint32_t n_vocab)
-{
-    return std::max(1u, (n_vocab + mako::kPieceLen - 1u) / mako::kPieceLen);
-}
-
 } // namespace
 
 extern "C" {
@@ -103,8 +98,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
 {
     if (!out || max_rows == 0 || max_vocab == 0)
         return MAKO_ERR_INVALID_ARG;
-    // (kMaxSlices slices of kSliceMax logits)
-    if (mako_sampler_slices(max_vocab) > mako::kMaxSlices || pieces_for(max_vocab) > 64u || max_vocab >= (1u << 20))
+    // (kMaxSlices slices of kSliceMax logits; one logit fewer so that a histogram bin's count fits its 20 bits)
+    if (mako_sampler_slices(max_vocab) > mako::kMaxSlices || max_vocab >= (1u << (64 - mako::kBinSumBits)))
         return MAKO_ERR_INVALID_ARG;
     mako_sampler_ctx* ctx = new (std::nothrow) mako_sampler_ctx;
     if (!ctx)
@@ -128,8 +123,12 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.stats, (size_t)max_rows * mako::kMaxSlices));
     MAKO_HIP(ctx, dev_alloc(&sc.cand_w, (size_t)max_rows * sc.slices_cap * mako::kCap));
     MAKO_HIP(ctx, dev_alloc(&sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap));
+    MAKO_HIP(ctx, dev_alloc(&sc.part_sum, (size_t)max_rows * mako::kMaxSlices));
+    MAKO_HIP(ctx, dev_alloc(&sc.part_n, (size_t)max_rows * mako::kMaxSlices));
     MAKO_HIP(ctx, dev_alloc(&sc.plan, (size_t)max_rows));
     MAKO_HIP(ctx, hipMemset(sc.plan, 0, (size_t)max_rows * sizeof(mako::BigPlan)));
+    MAKO_HIP(ctx, dev_alloc(&sc.bins, (size_t)max_rows * mako::kBins));
+    MAKO_HIP(ctx, hipMemset(sc.bins, 0, (size_t)max_rows * mako::kBins * sizeof(unsigned long long)));
     MAKO_HIP(ctx, dev_alloc(&sc.wbuf, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.cnt, rv));
     MAKO_HIP(ctx, dev_alloc(&sc.key[0], rv));
@@ -146,23 +145,19 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, dev_alloc(&sc.gt.start, rg));
     MAKO_HIP(ctx, dev_alloc(&sc.gt.pack, rg));
     MAKO_HIP(ctx, dev_alloc(&sc.gt.quarters, rg * 4));
-    sc.pieces_cap = pieces_for(max_vocab);
-    MAKO_HIP(ctx, dev_alloc(&sc.piece_idx, rv));
-    MAKO_HIP(ctx, dev_alloc(&sc.piece_tab, (size_t)max_rows * sc.pieces_cap * (mako::kWorkers + 1u)));
-    MAKO_HIP(ctx, dev_alloc(&sc.piece_mass, (size_t)max_rows * sc.pieces_cap * mako::kWorkers));
-    MAKO_HIP(ctx, dev_alloc(&sc.piece_sum, (size_t)max_rows * sc.pieces_cap));
-    MAKO_HIP(ctx, dev_alloc(&sc.piece_cnt, (size_t)max_rows * sc.pieces_cap));
+    MAKO_HIP(ctx, dev_alloc(&sc.bin_worker, (size_t)max_rows * mako::kBins));
     MAKO_HIP(ctx, dev_alloc(&sc.work_n, 8));
     MAKO_HIP(ctx, hipMemset(sc.work_n, 0, 8 * sizeof(uint32_t)));
-    MAKO_HIP(ctx, dev_alloc(&sc.work_rows, (size_t)max_rows));
-    MAKO_HIP(ctx, hipMemset(sc.work_rows, 0, (size_t)max_rows * sizeof(uint32_t)));
     MAKO_HIP(ctx, dev_alloc(&sc.work_sort, (size_t)max_rows * mako::kWorkers));
     MAKO_HIP(ctx, dev_alloc(&sc.work_tail, (size_t)max_rows));
+    MAKO_HIP(ctx, dev_alloc(&ctx->sc_dev, 1));
+    MAKO_HIP(ctx, hipMemcpy(ctx->sc_dev, &sc, sizeof sc, hipMemcpyHostToDevice));
     MAKO_HIP(ctx, hipDeviceSynchronize());
-    // the kernels overlay up to 64 KB of dynamic LDS (second_kernel and sort_kernel more) on a few KB of static LDS
+    // the kernels overlay up to 64 KB of dynamic LDS (sort_kernel more) on a few KB of static LDS
     MAKO_HIP(ctx, mako::init_scan_kernels());
-    MAKO_HIP(ctx, mako::init_second_kernels());
-    MAKO_HIP(ctx, mako::init_rows_kernels());
+    MAKO_HIP(ctx, mako::init_finish_kernels());
+    MAKO_HIP(ctx, mako::init_plan_for_sort());
+    MAKO_HIP(ctx, mako::init_plan_alone());
     MAKO_HIP(ctx, mako::init_sort_kernels());
     MAKO_HIP(ctx, mako::init_tail_kernels());
     return MAKO_OK;
@@ -174,8 +169,8 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {sc.piece_idx, sc.piece_tab, sc.piece_mass, sc.piece_sum, sc.piece_cnt, sc.work_n, sc.work_rows, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
-                    sc.cand_w, sc.cand_i, sc.plan,
+    void* ptrs[] = {ctx->sc_dev, sc.bin_worker, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
+                    sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.bins, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
                     ctx->st_hist,  ctx->st_hcnt, ctx->st_hlen,  ctx->st_draft, ctx->st_tokens, ctx->st_acc};
@@ -262,6 +257,11 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
     const bool vec = d.n_vocab % 4 == 0 && d.logits_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(d.logits) & 15u) == 0;
     const size_t lds = d.hist_tokens ? (size_t)slice_len * sizeof(uint32_t) : 0;
     const dim3 grid(slices, d.n_rows);
+    // The second pass cuts top_k == 0 rows into pieces of one to four blocks of 4096 logits (decided on the device:
+    // pieces finer than slices only while all of them fit one round of workgroups), so this many workgroups can
+    // have work; the others leave after a look at the rows' parameters.
+    const uint32_t pieces_max = std::min<uint32_t>(mako::kMaxSlices, std::max(slices, (d.n_vocab + 4095u) / 4096u));
+    const uint32_t finish_wgs = std::max(d.n_rows * slices, std::min(ctx->cus, d.n_rows * pieces_max));
     // histories of up to 2 (8) entries per thread stay in registers; longer ones take the generic route
     const int kh = !d.hist_tokens ? 2 : (d.hist_stride <= 2 * mako::kThreads ? 2 : (d.hist_stride <= 8 * mako::kThreads ? 8 : 0));
     const bool prof = ctx->profile;
@@ -270,40 +270,47 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
         if (prof)                                                                                                  \
             MAKO_HIP(ctx, hipEventRecord(ctx->ev[i], st));                                                         \
     } while (0)
-    // which kernels have work: all of them unless the caller's host copy of the parameters says otherwise; and how
-    // many workgroups the launches behind the scan can need
+    // which kernels have work: all of them unless the caller's host copy of the parameters says otherwise
+    // and how long the finishing kernels' work lists can get: kWorkers entries per top_k == 0 row, one per other
+    // sampled row (whole-row rows, top-k rows that cannot be certified from their candidates)
     bool any_nucleus = true, any_general = true;
-    uint32_t nucleus_rows = d.n_rows;
+    uint32_t nucleus_rows = d.n_rows, list_rows = d.n_rows;
     if (params_host) {
         any_nucleus = any_general = false;
-        uint32_t n_nucleus = 0;
+        uint32_t n_nucleus = 0, n_other = 0;
         for (uint32_t r = 0; r < d.n_rows; ++r) {
             const mako::RowClass c = mako::classify(params_host[r]);
             any_nucleus |= c == mako::kNucleus;
             any_general |= c == mako::kGeneral;
             n_nucleus += c == mako::kNucleus;
+            n_other += c == mako::kTopK || c == mako::kGeneral;
         }
-        nucleus_rows = n_nucleus;
+        nucleus_rows = std::max(n_nucleus, 1u);
+        list_rows = std::max(n_nucleus + (n_other + mako::kWorkers - 1u) / mako::kWorkers, 1u);
     }
+    const bool launch_sort = any_nucleus || any_general;
     MAKO_MARK(0);
     mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, ctx->sc, slice_len, ctx->cus);
     MAKO_MARK(1);
-    // top_k == 0 rows: second pass, then sorted by the rows' workers, then cut and drawn from; the stages talk
-    // through kernel boundaries (handing over inside a kernel costs as much as a launch on this chip).  The other
-    // rows are finished beside the tails, or, in a batch without top_k == 0 rows, by a launch of their own.
-    if (any_nucleus) {
-        mako::launch_second(vec, kh, nucleus_rows * pieces_for(d.n_vocab), st, d, ctx->sc, slices);
-        MAKO_MARK(2);
-        // (the work list: up to kWorkers entries per top_k == 0 row)
-        mako::launch_sort(st, d, ctx->sc, slices, std::max(nucleus_rows, 1u) * mako::kWorkers);
-        MAKO_MARK(3);
-        mako::launch_tail(st, d, ctx->sc, slices, nucleus_rows);
-    } else {
-        mako::launch_rows(any_general, st, d, ctx->sc, slices);
-        MAKO_MARK(2);
-        MAKO_MARK(3);
-    }
+    if (any_nucleus)
+        mako::launch_finish(vec, kh, finish_wgs, st, d, ctx->sc_dev, slices);
+    MAKO_MARK(2);
+    // top_k == 0 rows: plan from the row's histogram, sort by the plan, cut and draw; the stages talk through
+    // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  Other rows cost a load.
+    if (launch_sort)
+        mako::launch_plan_for_sort(st, d, ctx->sc_dev, slices);
+    else
+        mako::launch_plan_alone(st, d, ctx->sc_dev, slices);
+    MAKO_MARK(3);
+    if (any_nucleus)
+        mako::launch_partition(st, d, ctx->sc, list_rows);
     MAKO_MARK(4);
+    if (launch_sort)
+        mako::launch_sort(st, d, ctx->sc, slices, list_rows);
+    MAKO_MARK(5);
+    if (any_nucleus)
+        mako::launch_tail(st, d, ctx->sc, nucleus_rows);
+    MAKO_MARK(6);
 #undef MAKO_MARK
     ctx->profiled = prof;
     MAKO_HIP(ctx, hipGetLastError());

@@ -1,127 +1,134 @@
-// Splitting a top_k == 0 row among the workers that sort its nucleus, from a sample of the row's weights.
+// Planning a top_k == 0 row from the exact histogram of its weights.
 #pragma once
 
 #include "workgroup_state.h"
 
 namespace mako {
 
-// The whole workgroup turns the histogram of the row's sampled weights (shist[b]; only bins >= b_prune were counted)
-// into (1) a guess of how far down the nucleus reaches and (2) the workers' value ranges.
-//
-// (1) Every sample stands for n_vocab / kSamples weights of about its size, except the eight heaviest, which stand for
-// themselves (where the row's weights are sparse a sample has no neighbours, and counting it many times over would
-// put the cut too high).  From the samples' masses (count x the bin's middle weight) the bin in which the running
-// mass reaches top_p x total is found, and the row keeps the weights down to HALF the lower edge of that bin (never
-// below b_prune).  This is a guess: the kept set is exactly the weights in bins >= b_keep, and tail_kernel checks that
-// the nucleus ends inside it; a row whose nucleus does not takes the whole-row path instead.
-// (2) The kept weights are cut by value into `workers` contiguous ranges, heaviest first, that hold about the same
-// number of samples each.  A cut that falls inside a bin is placed by interpolation between the bin's edges, so a
-// crowded bin is shared by several workers.
-//   table[b]   the worker that takes the heaviest weights of bin b
-//   cut[j]     (1 <= j < workers) bits(q) of the cut between workers j - 1 and j: weights with bits(q) below it go
-//              to worker j or beyond; 0 where no cut was placed (cleared by the caller)
-// `workers` is chosen so that a worker's share stays near kShareTarget.  Every piece of the row sees the same samples
-// and arrives at the same answers; no result depends on them, only the work does.  Thread t holds bins
-// kBins - 1 - 2t and kBins - 2 - 2t.  Three barriers inside (LDS only); the caller's next barrier publishes table and
-// cut.  Returns the number of workers; b_keep receives the lowest bin kept.
-struct SamplePlanLds {
-    uint32_t wave_cnt[kWaves];
-    float wave_mass[kWaves];
-    uint32_t edge_bin;
-    uint32_t kept_samples;
-};
-__device__ __forceinline__ uint32_t sample_plan(const uint32_t* shist, uint8_t* table, uint32_t* cut, uint32_t n_vocab,
-                                                float top_p, uint32_t b_prune, SamplePlanLds& pl, uint32_t& b_keep)
+// Plans a top_k == 0 row from the histogram of its weights (weight_bin(), exact masses): finds the bin by
+// which the nucleus must have ended and splits the weights above it over kWorkers workers by value.
+// Thread t brings the counts (c0, c1) and significand sums (s0, s1) of bins kBins-1-2t and kBins-2-2t.
+// Returns n0, the number of weights to sort; the plan is written to `plan` (flag left untouched).
+__device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, uint32_t c0, uint32_t c1,
+                                 unsigned long long s0, unsigned long long s1, BigPlan* plan, uint8_t* bin_worker,
+                                 const FinishLds& L, uint32_t& thr_bits)
 {
-    const uint32_t b0 = kBins - 1u - 2u * threadIdx.x, b1 = b0 - 1u;
-    const uint32_t c0 = shist[b0], c1 = shist[b1];
-    const uint32_t incl = __ockl_wfscan_add_u32(c0 + c1, true);
-    if (lane_id() == kWave - 1)
-        pl.wave_cnt[wave_id()] = incl;
-    if (threadIdx.x == 0)
-        pl.edge_bin = 0u; // (no bin reaches the cut: everything above b_prune is kept)
-    lds_barrier();
-    uint32_t above0 = incl - (c0 + c1);
-    for (int w = 0; w < wave_id(); ++w)
-        above0 += pl.wave_cnt[w];
-    const uint32_t above1 = above0 + c0;
-    // (1) masses: the samples ranked 0..7 count once, the others n_vocab / kSamples times
-    const float each = fmaxf(1.0f, (float)n_vocab / (float)kSamples);
-    auto weighted = [&](uint32_t above, uint32_t c) {
-        const uint32_t solo = above < 8u ? min(c, 8u - above) : 0u;
-        return (float)solo + (float)(c - solo) * each;
+    FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t b0 = kBins - 1u - 2u * tid, b1 = b0 - 1u;
+    // exact mass of a bin: sum of significands times the bin's power of two (bins never straddle a binade)
+    auto scale = [](uint32_t b) {
+        const uint32_t e = max(bin_lo_key(b) >> 23, 1u); // biased exponent of the bin's weights (subnormals: 1)
+        return __longlong_as_double((long long)(1023ull + e - 150ull) << 52);
     };
-    auto middle = [](uint32_t b) { return __uint_as_float((bin_lo_key(b) >> 1) + (bin_hi_key(b) >> 1)); };
-    const float m0 = c0 ? weighted(above0, c0) * middle(b0) : 0.0f, m1 = c1 ? weighted(above1, c1) * middle(b1) : 0.0f;
-    float mincl = m0 + m1; // inclusive scan over the wave, then the waves' totals
-    for (int o = 1; o < kWave; o <<= 1) {
-        const float t = __shfl_up(mincl, o);
-        mincl += lane_id() >= o ? t : 0.0f;
+    const double m0 = (double)s0 * scale(b0), m1 = (double)s1 * scale(b1);
+    const double want = (double)P.top_p * total64;
+    uint32_t* w_hi = L.wcount;            // highest bin of each worker
+    uint32_t* w_lo = L.wcount + kWorkers; // lowest bin
+    uint32_t* w_off = L.wcount + 2 * kWorkers;
+    uint32_t* w_cnt = L.wcount + 3 * kWorkers;
+    if (tid < kWorkers) {
+        w_hi[tid] = 0;
+        w_lo[tid] = kNone;
+        w_off[tid] = kNone;
+        w_cnt[tid] = 0;
     }
-    if (lane_id() == kWave - 1)
-        pl.wave_mass[wave_id()] = mincl;
-    lds_barrier();
-    float mabove0 = mincl - (m0 + m1), mtotal = 0.0f;
+    // running mass (inclusive) and candidates above each bin (exclusive), from the top bin down: wave scans, and
+    // one exchange of the sixteen waves' totals for both
+    const double mass_w = __ockl_wfscan_add_f64(m0 + m1, true);
+    const uint32_t cnt_w = __ockl_wfscan_add_u32(c0 + c1, true);
+    if (lane_id() == kWave - 1) {
+        sm.bs.f64[wave_id()] = mass_w;
+        sm.bs.u64[wave_id()] = cnt_w;
+    }
+    __syncthreads();
+    double pre_m = 0;
+    uint32_t pre_c = 0, count_all = 0;
     for (int w = 0; w < kWaves; ++w) {
-        const float x = pl.wave_mass[w];
-        mabove0 += w < wave_id() ? x : 0.0f;
-        mtotal += x;
-    }
-    const float want = top_p * mtotal;
-    // the first bin (from the top) at which the running mass reaches `want` (the largest bin index among those that do)
-    if (c0 && mabove0 + m0 >= want)
-        atomicMax(&pl.edge_bin, b0);
-    else if (c1 && mabove0 + m0 + m1 >= want)
-        atomicMax(&pl.edge_bin, b1);
-    lds_barrier();
-    {
-        const uint32_t edge = pl.edge_bin;
-        uint32_t keep = b_prune;
-        if (edge > 0u) {
-            const uint32_t lo = bin_lo_key(edge);
-            keep = max(b_prune, lo > (1u << 23) ? weight_bin(lo - (1u << 23)) : 0u); // (half the edge bin's lower edge)
+        const double x = sm.bs.f64[w];
+        const uint32_t y = (uint32_t)sm.bs.u64[w];
+        if (w < wave_id()) {
+            pre_m += x;
+            pre_c += y;
         }
-        b_keep = keep;
+        count_all += y;
     }
-    // samples kept: those in bins >= b_keep (the holder of bin b_keep knows)
-    if (b0 == b_keep)
-        pl.kept_samples = above0 + c0;
-    else if (b1 == b_keep)
-        pl.kept_samples = above1 + c1;
-    lds_barrier();
-    const uint32_t kept = pl.kept_samples;
-    // (2) (samples * n_vocab stays below 2^32: kSamples = 2^10 samples, n_vocab below 2^20)
-    const uint32_t est = (kept * n_vocab + kSamples - 1u) / kSamples;
-    const uint32_t workers = min(kWorkers, max(1u, (est + kShareTarget - 1u) / kShareTarget));
-    const float per = (float)max(kept, 1u) / (float)workers; // samples per worker
-    const float inv_per = (float)workers / (float)max(kept, 1u);
-    // cuts lie at sample counts j * per, j = 1 .. workers - 1: those at or before `above` lie in higher bins
-    auto place = [&](uint32_t b, uint32_t above, uint32_t c) {
-        const uint32_t j0 = min(workers - 1u, (uint32_t)((float)above * inv_per));
-        table[b] = (uint8_t)j0;
-        const uint32_t j1 = min(workers - 1u, (uint32_t)((float)(above + c) * inv_per));
-        if (j1 > j0 && b >= b_keep) { // (few bins hold a cut)
-            const uint32_t hi = bin_hi_key(b), lo = bin_lo_key(b);
-            const float width = (float)(hi - lo), inv_c = 1.0f / (float)c;
-            for (uint32_t j = j0 + 1u; j <= j1; ++j) {
-                const float frac = ((float)j * per - (float)above) * inv_c; // from the bin's top down
-                cut[j] = hi - min(hi - lo, (uint32_t)(fminf(fmaxf(frac, 0.0f), 1.0f) * width));
-            }
-        }
+    MAKO_STAMP(20);
+    const double incl = pre_m + mass_w;
+    const uint32_t above0 = pre_c + cnt_w - (c0 + c1), above1 = above0 + c0;
+    // The nucleus ends in the first bin (from the top) at which the running mass reaches `want`.  These sums
+    // associate differently from the sorted prefix sums that make the final decision, so one more non-empty
+    // bin is taken along: the list stops at the SECOND bin that satisfies the test.
+    const bool r0 = c0 && incl - m1 >= want, r1 = c1 && incl >= want;
+    const uint32_t reached = (uint32_t)r0 + (uint32_t)r1;
+    const uint32_t reached_w = __ockl_wfscan_add_u32(reached, true);
+    if (lane_id() == kWave - 1)
+        sm.hist[wave_id()] = reached_w;
+    if (tid == 0) {
+        sm.ticket = 0;        // the lowest bin taken; not reached twice: every candidate is kept
+        sm.flag = count_all;  // the number of weights to sort
+    }
+    __syncthreads();
+    uint32_t before = reached_w - reached;
+    for (int w = 0; w < kWaves; ++w)
+        before += w < wave_id() ? sm.hist[w] : 0u;
+    if (r0 && before + 1 == 2) {
+        sm.ticket = b0;
+        sm.flag = above0 + c0;
+    } else if (r1 && before + (uint32_t)r0 + 1 == 2) {
+        sm.ticket = b1;
+        sm.flag = above1 + c1;
+    }
+    __syncthreads();
+    MAKO_STAMP(22);
+    const uint32_t b_lo = sm.ticket;
+    thr_bits = bin_lo_key(b_lo);
+    const uint32_t n0 = sm.flag;
+    auto worker_of = [&](uint32_t b, uint32_t c, uint32_t above) {
+        return (c == 0 || b < b_lo) ? kNone : min(kWorkers - 1u, (uint32_t)(((unsigned long long)above * kWorkers) / n0));
     };
-    place(b0, above0, c0);
-    place(b1, above1, c1);
-    return workers;
-}
-
-// The worker that takes the weight with these bits(q), in bin b.
-__device__ __forceinline__ uint32_t worker_of_weight(uint32_t bits, uint32_t b, const uint8_t* table, const uint32_t* cut,
-                                                     uint32_t workers)
-{
-    uint32_t dest = table[b];
-    while (dest + 1u < workers && bits < cut[dest + 1u])
-        ++dest;
-    return dest;
+    const uint32_t wk0 = worker_of(b0, c0, above0), wk1 = worker_of(b1, c1, above1);
+    if (wk0 != kNone) {
+        atomicMax(&w_hi[wk0], b0);
+        atomicMin(&w_lo[wk0], b0);
+        atomicMin(&w_off[wk0], above0);
+        atomicAdd(&w_cnt[wk0], c0);
+    }
+    if (wk1 != kNone) {
+        atomicMax(&w_hi[wk1], b1);
+        atomicMin(&w_lo[wk1], b1);
+        atomicMin(&w_off[wk1], above1);
+        atomicAdd(&w_cnt[wk1], c1);
+    }
+    __syncthreads();
+    MAKO_STAMP(23);
+    // the mass above a worker's range, known to the thread that holds the range's highest bin
+    if (wk0 != kNone && w_hi[wk0] == b0)
+        plan->mass[wk0] = incl - m0 - m1;
+    if (wk1 != kNone && w_hi[wk1] == b1)
+        plan->mass[wk1] = incl - m1;
+    bin_worker[b0] = (uint8_t)wk0; // (kNone -> 0xff)
+    bin_worker[b1] = (uint8_t)wk1;
+    if (tid < kWorkers) {
+        plan->cursor[tid] = 0;
+        plan->key_lo[tid] = bin_lo_key(min(w_lo[tid], kBins - 1u));
+        plan->key_hi[tid] = bin_hi_key(w_hi[tid]);
+        plan->off[tid] = w_cnt[tid] ? w_off[tid] : 0u;
+        plan->cnt[tid] = w_cnt[tid];
+    }
+    if (wave_id() == 0) { // the workers' first group records: a scan over their group counts
+        const uint32_t mine = lane_id() < (int)kWorkers ? (w_cnt[lane_id()] + kGroup - 1u) / kGroup : 0u;
+        const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
+        if (lane_id() < (int)kWorkers)
+            plan->gbase[lane_id()] = upto - mine;
+        if (lane_id() == kWave - 1) {
+            plan->groups = upto;
+            plan->n0 = n0;
+            plan->total64 = total64;
+        }
+    }
+    __syncthreads();
+    return n0;
 }
 
 } // namespace mako

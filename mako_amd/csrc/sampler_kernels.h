@@ -4,14 +4,12 @@
 //   scan_kernel       one workgroup per (row, slice): the single coalesced pass over the fp32 logits.  The token
 //                     mask and the history penalties are applied in registers; the slice's maximum and its largest
 //                     logits (a superset of what top-k can need) go to scratch.
-//   second_kernel     the second, cache-resident pass over top_k == 0 rows: exact sums and the histogram of
-//                     q = expf((w - m) / T), each piece's weights left ordered by histogram bin; beside it, one
-//                     workgroup per other row: greedy and forced rows, top-k rows from the candidate lists, ordered
-//                     by (q desc, idx asc) and drawn from with the reference's exact fp32 rounding order.
-//                     (rows_kernel: the same for a batch without top_k == 0 rows.)
-//   sort_kernel       every top_k == 0 row planned from its histogram by each of its 32 workers; narrow nuclei
-//                     finished from the candidate lists, wide ones gathered by value range and sorted.
-//   tail_kernel       the wide nuclei cut and drawn from.
+//   finish_kernel     the second, cache-resident pass over top_k == 0 rows: exact sums and the histogram of
+//                     q = expf((w - m) / T).
+//   plan_kernel       greedy and forced rows; top-k rows from the candidate lists, ordered by (q desc, idx asc) and
+//                     drawn from with the reference's exact fp32 rounding order; the plan of every top_k == 0 row.
+//   partition_kernel, sort_kernel, tail_kernel
+//                     the wide nuclei: weights handed to 32 workers per row, sorted, cut and drawn from.
 //   Whatever the candidate lists cannot certify falls to a whole-row path that is exact for every parameter
 //   combination.
 #pragma once
@@ -30,7 +28,7 @@
 #include "worker_sort.h"
 #include "row_records.h"
 #include "topk_candidates.h"
-#include "rows_kernel.h"
 #include "second_pass.h"
+#include "plan_kernel.h"
 #include "sort_kernels.h"
 #include "tail_kernel.h"

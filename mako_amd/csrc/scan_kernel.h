@@ -70,10 +70,11 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
             sc.work_n[1] = 0;
         }
     }
-    if (row == 0 && slice == 0 && wave_id() == 1) { // the rows that take the second pass
-        const uint32_t rows = nucleus_rows(d, sc.work_rows);
+    if (row == 0 && slice == 0 && wave_id() == 1) { // how the second pass will be cut up
+        uint32_t piece_len, busy;
+        const uint32_t pieces = second_pass_pieces(d, gridDim.x, slice_len, cus, piece_len, busy);
         if (lane_id() == 0)
-            sc.work_n[4] = rows;
+            *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(pieces, piece_len, busy, 0u);
     }
     // ReasoningBudget::forced's question (src/server/openai.cpp:598-602), answered in the same pass over the logits
     bool want_above = false;
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
     for (uint32_t j = 0; j < 16; ++j)
         best = fmaxf(best, wv[j]);
     const uint32_t bkey = order_key(best);
-    const bool emits = cls == kTopK; // (top_k == 0 rows take the second pass: nobody reads candidates of theirs)
+    const bool emits = cls == kTopK || cls == kNucleus;
     const uint32_t wmax = __ockl_wfred_max_u32(bkey);
     uint32_t wkth = 0;
     if (emits) {

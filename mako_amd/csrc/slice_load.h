@@ -36,14 +36,14 @@ __device__ __forceinline__ void build_counts(const mako_sample_desc& d, uint32_t
 
 // The thread's 16 logits, raw, plus the mask bits of each group of four (VEC) or of each logit (scalar).
 // Issued before anything else so that the HBM latency overlaps the LDS work that follows.
-template <bool VEC, int NB = 4>
+template <bool VEC>
 struct RawSlice {
-    float4 v[NB];
-    uint32_t bits[NB]; // VEC: bit c of bits[k] = logit 4k+c allowed; scalar: bit j of bits[0] = logit j allowed
+    float4 v[4];
+    uint32_t bits[4]; // VEC: bit c of bits[k] = logit 4k+c allowed; scalar: bit j of bits[0] = logit j allowed
 };
 
-template <bool VEC, int NB = 4>
-__device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi, RawSlice<VEC, NB>& r)
+template <bool VEC>
+__device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi, RawSlice<VEC>& r)
 {
     const uint32_t tid = threadIdx.x;
     const float* lrow = d.logits + (int64_t)row * d.logits_stride;
@@ -52,21 +52,21 @@ __device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row
     if (VEC) {
         // all four loads go out back to back, from clamped addresses and without a branch between them (a branch
         // would make the compiler wait for each load before the next); what lies past the slice is dropped after
-        uint32_t at[NB];
+        uint32_t at[4];
 #pragma unroll
-        for (uint32_t k = 0; k < (uint32_t)NB; ++k) {
+        for (uint32_t k = 0; k < 4; ++k) {
             const uint32_t i = lo + k * 4096u + tid * 4u;
             at[k] = i < hi ? i : hi - 4u; // hi - lo is a positive multiple of 4 in this mode
             r.v[k] = *reinterpret_cast<const float4*>(lrow + at[k]);
         }
         if (mrow) {
 #pragma unroll
-            for (uint32_t k = 0; k < (uint32_t)NB; ++k)
+            for (uint32_t k = 0; k < 4; ++k)
                 r.bits[k] = mrow[at[k] >> 5] >> (at[k] & 31u);
         }
         if (!mrow) {
 #pragma unroll
-            for (uint32_t k = 0; k < (uint32_t)NB; ++k)
+            for (uint32_t k = 0; k < 4; ++k)
                 r.bits[k] = 0xfu;
         }
         // (finish_slice() replaces what was read past the slice: nothing here touches the loaded values, so the
@@ -75,7 +75,7 @@ __device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row
         float* f = reinterpret_cast<float*>(r.v);
         uint32_t allowed = 0xffffu;
 #pragma unroll
-        for (uint32_t j = 0; j < 4u * NB; ++j) {
+        for (uint32_t j = 0; j < 16; ++j) {
             const uint32_t i = lo + j * (uint32_t)kThreads + tid;
             f[j] = nan;
             if (i < hi) {
@@ -90,14 +90,14 @@ __device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row
 
 // How many of the thread's logits (as the sampler is given them: a token the mask clears is -inf) are strictly
 // greater than v: the count of ReasoningBudget::forced, src/server/openai.cpp:599-602.
-template <bool VEC, int NB = 4>
-__device__ __forceinline__ uint32_t count_above(const RawSlice<VEC, NB>& r, uint32_t lo, uint32_t hi, float v)
+template <bool VEC>
+__device__ __forceinline__ uint32_t count_above(const RawSlice<VEC>& r, uint32_t lo, uint32_t hi, float v)
 {
     const uint32_t tid = threadIdx.x;
     uint32_t c = 0;
     if (VEC) {
 #pragma unroll
-        for (uint32_t k = 0; k < (uint32_t)NB; ++k) {
+        for (uint32_t k = 0; k < 4; ++k) {
             if (lo + k * 4096u + tid * 4u < hi) {
                 c += ((r.bits[k] & 1u) && r.v[k].x > v) ? 1u : 0u;
                 c += ((r.bits[k] & 2u) && r.v[k].y > v) ? 1u : 0u;
@@ -108,7 +108,7 @@ __device__ __forceinline__ uint32_t count_above(const RawSlice<VEC, NB>& r, uint
     } else {
         const float* f = reinterpret_cast<const float*>(r.v);
 #pragma unroll
-        for (uint32_t j = 0; j < 4u * NB; ++j)
+        for (uint32_t j = 0; j < 16; ++j)
             c += (lo + j * (uint32_t)kThreads + tid < hi && ((r.bits[0] >> j) & 1u) && f[j] > v) ? 1u : 0u;
     }
     return c;
@@ -116,15 +116,15 @@ __device__ __forceinline__ uint32_t count_above(const RawSlice<VEC, NB>& r, uint
 
 // Mask and penalties (src/gen/sampler.cpp:22-28) applied to the raw logits; slots past the end of the
 // slice hold NaN, which never wins a comparison and never becomes a candidate.
-template <bool VEC, int NB = 4>
-__device__ __forceinline__ void finish_slice(const RawSlice<VEC, NB>& r, uint32_t lo, uint32_t hi, const mako_sampling_params& P,
-                                             bool pen, const uint32_t* s_cnt, float (&wv)[4 * NB], bool masked)
+template <bool VEC>
+__device__ __forceinline__ void finish_slice(const RawSlice<VEC>& r, uint32_t lo, uint32_t hi, const mako_sampling_params& P,
+                                             bool pen, const uint32_t* s_cnt, float (&wv)[16], bool masked)
 {
     const uint32_t tid = threadIdx.x;
     if (VEC && !masked) { // uniform: no mask, nothing to clear
         const float nan = __uint_as_float(0x7fc00000u);
 #pragma unroll
-        for (uint32_t k = 0; k < (uint32_t)NB; ++k) {
+        for (uint32_t k = 0; k < 4; ++k) {
             const bool inside = lo + k * 4096u + tid * 4u < hi;
             wv[4 * k + 0] = !inside ? nan : r.v[k].x;
             wv[4 * k + 1] = !inside ? nan : r.v[k].y;
@@ -134,7 +134,7 @@ __device__ __forceinline__ void finish_slice(const RawSlice<VEC, NB>& r, uint32_
     } else if (VEC) {
         const float nan = __uint_as_float(0x7fc00000u);
 #pragma unroll
-        for (uint32_t k = 0; k < (uint32_t)NB; ++k) {
+        for (uint32_t k = 0; k < 4; ++k) {
             const bool inside = lo + k * 4096u + tid * 4u < hi;
             wv[4 * k + 0] = !inside ? nan : ((r.bits[k] & 1u) ? r.v[k].x : -INFINITY);
             wv[4 * k + 1] = !inside ? nan : ((r.bits[k] & 2u) ? r.v[k].y : -INFINITY);
@@ -144,13 +144,13 @@ __device__ __forceinline__ void finish_slice(const RawSlice<VEC, NB>& r, uint32_
     } else {
         const float* f = reinterpret_cast<const float*>(r.v);
 #pragma unroll
-        for (uint32_t j = 0; j < 4u * NB; ++j)
+        for (uint32_t j = 0; j < 16; ++j)
             wv[j] = ((r.bits[0] >> j) & 1u) ? f[j] : -INFINITY;
     }
     if (pen) {
         if (VEC) {
 #pragma unroll
-            for (uint32_t k = 0; k < (uint32_t)NB; ++k) {
+            for (uint32_t k = 0; k < 4; ++k) {
                 const uint32_t i = lo + k * 4096u + tid * 4u;
                 if (i < hi) {
                     const uint4 n = *reinterpret_cast<const uint4*>(s_cnt + (i - lo));
@@ -168,7 +168,7 @@ __device__ __forceinline__ void finish_slice(const RawSlice<VEC, NB>& r, uint32_
             }
         } else {
 #pragma unroll
-            for (uint32_t j = 0; j < 4u * NB; ++j) {
+            for (uint32_t j = 0; j < 16; ++j) {
                 const uint32_t i = lo + j * (uint32_t)kThreads + tid;
                 if (i < hi) {
                     const uint32_t n = s_cnt[i - lo];
@@ -196,10 +196,10 @@ struct NoOverlap {
 
 // `overlap` runs right after the slice's loads have been issued: work that does not depend on them hides
 // behind their latency.  It must be reached by the whole workgroup or by none of it.
-template <bool VEC, int KH, int NB = 4, typename Overlap = NoOverlap>
+template <bool VEC, int KH, typename Overlap = NoOverlap>
 __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi,
                                                uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, bool pen,
-                                               uint32_t* s_cnt, float (&wv)[4 * NB], Overlap overlap = Overlap(),
+                                               uint32_t* s_cnt, float (&wv)[16], Overlap overlap = Overlap(),
                                                bool want_above = false, float close_v = 0.0f, uint32_t* above = nullptr)
 {
     const uint32_t tid = threadIdx.x;
@@ -225,18 +225,18 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
                 cnt[k] = hc[min(tid + (uint32_t)k * kThreads, last)];
         }
     }
-    RawSlice<VEC, NB> raw;
-    load_raw<VEC, NB>(d, row, lo, hi, raw);
+    RawSlice<VEC> raw;
+    load_raw<VEC>(d, row, lo, hi, raw);
     overlap();
     if (want_above) // uniform
-        *above = count_above<VEC, NB>(raw, lo, hi, close_v);
+        *above = count_above<VEC>(raw, lo, hi, close_v);
     if (!pen) {
-        finish_slice<VEC, NB>(raw, lo, hi, P, false, s_cnt, wv, d.mask != nullptr);
+        finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv, d.mask != nullptr);
         return;
     }
     if (KH == 0) {
         build_counts(d, row, hl, lo, hi, slice_len, s_cnt);
-        finish_slice<VEC, NB>(raw, lo, hi, P, true, s_cnt, wv, d.mask != nullptr);
+        finish_slice<VEC>(raw, lo, hi, P, true, s_cnt, wv, d.mask != nullptr);
         return;
     }
 #pragma unroll
@@ -274,13 +274,13 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
             cnt[k] = s_cnt[tok[k] - lo]; // occurrences of the token in the whole history
     lds_barrier(); // (the slots are about to be overwritten)
     MAKO_STAMP(22);
-    finish_slice<VEC, NB>(raw, lo, hi, P, false, s_cnt, wv, d.mask != nullptr);
+    finish_slice<VEC>(raw, lo, hi, P, false, s_cnt, wv, d.mask != nullptr);
     MAKO_STAMP(23);
     // owners: a logit whose slot is taken goes into the slot (its bits); `moved` remembers which of the sixteen
     uint32_t moved = 0;
     if (VEC) {
 #pragma unroll
-        for (uint32_t k = 0; k < (uint32_t)NB; ++k) {
+        for (uint32_t k = 0; k < 4; ++k) {
             const uint32_t i = lo + k * 4096u + tid * 4u;
             if (i < hi) {
                 uint4* slot = reinterpret_cast<uint4*>(s_cnt + (i - lo));
@@ -294,7 +294,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
         }
     } else {
 #pragma unroll
-        for (uint32_t j = 0; j < 4u * NB; ++j) {
+        for (uint32_t j = 0; j < 16; ++j) {
             const uint32_t i = lo + j * (uint32_t)kThreads + tid;
             if (i < hi && s_cnt[i - lo]) {
                 s_cnt[i - lo] = __float_as_uint(wv[j]);
@@ -314,7 +314,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     if (moved) {
         if (VEC) {
 #pragma unroll
-            for (uint32_t k = 0; k < (uint32_t)NB; ++k)
+            for (uint32_t k = 0; k < 4; ++k)
                 if ((moved >> (4u * k)) & 0xfu) {
                     const uint4 v = *reinterpret_cast<const uint4*>(s_cnt + (lo + k * 4096u + tid * 4u - lo));
                     wv[4 * k + 0] = (moved >> (4u * k)) & 1u ? __uint_as_float(v.x) : wv[4 * k + 0];
@@ -324,7 +324,7 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
                 }
         } else {
 #pragma unroll
-            for (uint32_t j = 0; j < 4u * NB; ++j)
+            for (uint32_t j = 0; j < 16; ++j)
                 if ((moved >> j) & 1u)
                     wv[j] = __uint_as_float(s_cnt[j * (uint32_t)kThreads + tid]);
         }

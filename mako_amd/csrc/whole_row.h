@@ -23,12 +23,9 @@ __device__ __forceinline__ unsigned long long match_digit(uint32_t digit, bool v
 // with equal digits find each other with ballots (match_digit), so ranks inside a group need no atomics, and
 // the wave's running output offsets per digit live in its private row of LDS.  Three barriers per pass.
 // Returns false (and moves nothing) when every key has the same digit.
-// (BY_ID: the digit is taken from the token id instead of the key.)
-template <bool BY_ID = false>
 __device__ bool radix_pass(const uint32_t* ksrc, const uint32_t* isrc, uint32_t* kdst, uint32_t* idst, uint32_t n,
                            uint32_t shift, const FinishLds& L)
 {
-    const uint32_t* dsrc = BY_ID ? isrc : ksrc; // where the digits come from
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x, lane = lane_id(), wave = wave_id();
     const uint32_t chunk = ((n + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
@@ -45,7 +42,7 @@ __device__ bool radix_pass(const uint32_t* ksrc, const uint32_t* isrc, uint32_t*
         uint32_t key[4];
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u)
-            key[u] = dsrc[min(base + u * kWave + lane, end - 1u)];
+            key[u] = ksrc[min(base + u * kWave + lane, end - 1u)];
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
             const bool valid = base + u * kWave + lane < end;
@@ -85,7 +82,7 @@ __device__ bool radix_pass(const uint32_t* ksrc, const uint32_t* isrc, uint32_t*
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
             const bool valid = base + u * kWave + lane < end;
-            const uint32_t dg = valid ? (((BY_ID ? id[u] : key[u]) >> shift) & 255u) : 0u;
+            const uint32_t dg = valid ? ((key[u] >> shift) & 255u) : 0u;
             const unsigned long long mm = match_digit(dg, valid);
             const uint32_t off = woff[dg];
             if (valid) {
@@ -458,44 +455,13 @@ __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t*
     }
 }
 
-// The same for pairs in any order: sorted by (key ascending, id ascending), the ids (below 2^24) first.
-__device__ void sort_segment_unordered(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t* i1, uint32_t n, const FinishLds& L)
-{
-    if (n < 2)
-        return;
-    uint32_t *ks = k0, *is = i0, *kd = k1, *id = i1;
-    for (uint32_t pass = 0; pass < 7; ++pass) {
-        const bool moved = pass < 3 ? radix_pass<true>(ks, is, kd, id, n, pass * 8u, L)
-                                    : radix_pass<false>(ks, is, kd, id, n, (pass - 3u) * 8u, L);
-        if (moved) {
-            uint32_t* t = ks;
-            ks = kd;
-            kd = t;
-            t = is;
-            is = id;
-            id = t;
-        }
-        __syncthreads();
-    }
-    if (ks != k0) {
-        for (uint32_t i = threadIdx.x; i < n; i += kThreads) {
-            k0[i] = ks[i];
-            i0[i] = is[i];
-        }
-        __syncthreads();
-    }
-}
-
 // Whole-row path: exact for every parameter combination.  One workgroup rebuilds the penalised
 // row in scratch, keeps the candidates, sorts them by (q desc, idx asc) when top-k or top-p is
 // active, truncates, and draws.  src/gen/sampler.cpp:20-62.
 // (SITE: sort_kernel, its usual place, has an instance to itself, so that the compiler treats that kernel the same
 // whether or not the instances inside plan_kernel exist.)
-#ifndef MAKO_WHOLE_ROW_CALL
-#define MAKO_WHOLE_ROW_CALL
-#endif
 template <int SITE>
-__device__ MAKO_WHOLE_ROW_CALL void general_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
+__device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
                             float m, uint32_t argidx, const FinishLds& L)
 {
     FinishShared& sm = *L.sm;

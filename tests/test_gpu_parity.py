@@ -439,8 +439,9 @@ def test_tied_wide_nucleus(gpu_ctx):
 
 
 def test_narrow_nucleus_inside_one_slice(gpu_ctx):
-    """A nucleus of ~200 tokens that all live in one 16K-token slice, 14 to each wavefront of the scan: one piece of
-    the second pass holds the whole nucleus, one worker sorts it."""
+    """A nucleus of ~200 tokens that all live in one 16K-token slice, 14 to each wavefront of the scan: the slice
+    keeps only those at or above the smallest of the wavefronts' 8th largest, the certificate of the candidate
+    list fails, and the row is rebuilt from its weight array."""
     rng = np.random.default_rng(4444)
     b, v = 4, 129280
     slice_len = 16160  # ceil(129280 / 8)
@@ -455,7 +456,7 @@ def test_narrow_nucleus_inside_one_slice(gpu_ctx):
     w = dict(name="one_slice", logits=logits, params=p, u=rng.random(b).astype(np.float32))
     g = assert_parity(gpu_ctx, w, cap=512)
     _say("one-slice nuclei: %s paths %s" % (g["n_cand"].tolist(), g["path"].tolist()))
-    assert (g["path"] == api.PATH_NUCLEUS).all()
+    assert (g["path"] == api.PATH_GENERAL).any() and (g["path"] == api.PATH_NUCLEUS).any()
 
 
 @pytest.mark.parametrize("v", [40000, 129280])
