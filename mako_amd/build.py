@@ -24,12 +24,17 @@ FLAGS = [
     "-fno-gpu-flush-denormals-to-zero",
     "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # every device function inlined into its kernel: no call stack, so the finishing kernels need no
-    # scratch memory (kernels that use scratch run far fewer workgroups at a time on this chip)
-    "-mllvm", "-amdgpu-function-calls=false",
     "-Wall",
     "-Wno-unused-command-line-argument",
 ]
+# Every device function inlined into its kernel: no call stack, so the kernel needs no scratch memory (kernels
+# that use scratch run far fewer workgroups at a time on this chip).
+INLINE_ALL = ["-mllvm", "-amdgpu-function-calls=false"]
+# Per source.  tail_kernel calls the top-k row finisher out of line: few workgroups run it, and inlined it costs the
+# tails' own code registers and spills.
+SOURCE_FLAGS = {
+    "k_tail.hip": ["-DMAKO_ROWS_CALL=__attribute__((noinline))"],
+}
 
 
 def build(verbose=False, extra=(), jobs=8):
@@ -38,7 +43,7 @@ def build(verbose=False, extra=(), jobs=8):
 
     def compile_one(name):
         obj = os.path.join(OBJ_DIR, os.path.splitext(name)[0] + ".o")
-        cmd = ["hipcc", *FLAGS, *extra, "-c", os.path.join(CSRC, name), "-o", obj]
+        cmd = ["hipcc", *FLAGS, *SOURCE_FLAGS.get(name, INLINE_ALL), *extra, "-c", os.path.join(CSRC, name), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)

@@ -4,9 +4,9 @@
 #include "sampler_kernels.h"
 
 namespace mako {
-void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows)
+void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t tail_cap)
 {
-    hipLaunchKernelGGL(tail_kernel, dim3(1, grid_rows), dim3(kThreads), kDynLds, st, d, sc);
+    hipLaunchKernelGGL(tail_kernel, dim3(1, tail_cap + d.n_rows), dim3(kThreads), kDynLds, st, d, sc, slices, tail_cap);
 }
 
 hipError_t init_tail_kernels()

@@ -36,5 +36,6 @@ void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch*
 // of them still has to be dispatched.
 void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows); // (host copy, by value)
 void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows); // (host copy)
-void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows); // (host copy, by value)
+// (tail_kernel: `tail_cap` workgroups for the possible wide rows, then one per row for the batch's top-k rows)
+void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t tail_cap); // (host copy, by value)
 } // namespace mako

@@ -308,8 +308,8 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
     if (launch_sort)
         mako::launch_sort(st, d, ctx->sc, slices, list_rows);
     MAKO_MARK(5);
-    if (any_nucleus)
-        mako::launch_tail(st, d, ctx->sc, nucleus_rows);
+    if (launch_sort) // (also finishes the top-k rows that plan_kernel<false> leaves)
+        mako::launch_tail(st, d, ctx->sc, slices, nucleus_rows);
     MAKO_MARK(6);
 #undef MAKO_MARK
     ctx->profiled = prof;

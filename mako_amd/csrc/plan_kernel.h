@@ -6,8 +6,39 @@
 
 namespace mako {
 
-// grid = (1, rows), one workgroup per row.  Rows whose token is forced, greedy rows and top-k rows are finished here
-// from the records scan_kernel left; a top_k == 0 row's exact total, candidate count and weight histogram (from
+// A top-k row finished by one workgroup from the records and candidate lists scan_kernel left (all threads call;
+// sm.tab must hold the exp2 table): what plan_kernel<true> does for such a row, for tail_kernel's launch.  Rows that
+// plan_kernel<false> has dealt with (forced rows, rows it put on sort_kernel's whole-row list) are left alone.
+#ifndef MAKO_ROWS_CALL
+#define MAKO_ROWS_CALL __forceinline__
+#endif
+__device__ MAKO_ROWS_CALL void finish_topk_row(const mako_sample_desc& d, const Scratch& sc, const mako_sampling_params& P,
+                                               uint32_t row, uint32_t slices, const FinishLds& L)
+{
+    if (classify(P) != kTopK)
+        return;
+    if (d.force_token || d.close_token) { // uniform
+        int32_t ftok;
+        uint32_t above;
+        if (row_forced(d, sc, row, slices, ftok, above) != MAKO_FORCED_NONE)
+            return;
+    }
+    CandSlots pre;
+    const bool prefetched = !d.draft && slots_cover(slices); // uniform
+    if (prefetched)
+        fetch_candidate_slots(sc, row, slices, pre);
+    float m;
+    uint32_t argidx, n_cands, any_overflow;
+    SliceStat lane_stat;
+    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow, &lane_stat);
+    if (topk_takes_whole_row(kTopK, any_overflow, n_cands))
+        return;
+    topk_row<true>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
+}
+
+// grid = (1, rows), one workgroup per row.  Rows whose token is forced, greedy rows and (INLINE_GENERAL only: in a
+// batch that goes on to sort_kernel and tail_kernel the top-k rows are finished beside the tails) top-k rows are
+// finished here from the records scan_kernel left; a top_k == 0 row's exact total, candidate count and weight histogram (from
 // finish_kernel) are summed over its pieces and the row is planned: handed to sort_kernel's workers, or, when the
 // nucleus is narrow enough to end inside the candidate lists, to its worker 0 alone.
 // INLINE_GENERAL: sort_kernel will not be launched for this batch (the host saw no row that needs it), so a row
@@ -66,7 +97,7 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     __syncthreads();
     // a top-k row's candidates are asked for together with the slices' records
     CandSlots pre;
-    const bool prefetched = cls == kTopK && !d.draft && slots_cover(slices); // uniform
+    const bool prefetched = inline_general && cls == kTopK && !d.draft && slots_cover(slices); // uniform
     if (prefetched)
         fetch_candidate_slots(sc, row, slices, pre);
     float m;
@@ -104,7 +135,10 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
             return;
         }
 
-        topk_row<inline_general>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
+        if constexpr (!inline_general)
+            return; // (tail_kernel's launch finishes the batch's top-k rows beside the tails: finish_topk_row())
+        else
+            topk_row<inline_general>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
         return;
     }
 

@@ -2,6 +2,7 @@
 #pragma once
 
 #include "sorted_tail.h"
+#include "plan_kernel.h"
 
 namespace mako {
 
@@ -11,12 +12,31 @@ namespace mako {
 // plan_kernel: 2.3 us less there, but this kernel's chains then compiled to slower code and lost twice that.)
 // (The context's record by value: with a pointer to it the first loads would have to wait for a trip to memory.  The
 // list's length and this workgroup's entry are asked for together, then everything the row's plan holds.)
-__global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_val)
+// Workgroups from tail_cap on: workgroup tail_cap + r finishes row r if it is a top-k row (finish_topk_row()), beside
+// the few long tails, on CUs that would otherwise idle.  (That code is kept out of line: inlined, it made this kernel's
+// chains compile to slower code.)
+__global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices,
+                                                        uint32_t tail_cap)
 {
     const Scratch& sc_arg = sc_val;
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
+    if (blockIdx.y >= tail_cap) {
+        const uint32_t r = blockIdx.y - tail_cap;
+        if (r >= d_arg.n_rows)
+            return;
+        if (threadIdx.x < 32)
+            sm.tab[threadIdx.x] = k_exp2_tab[threadIdx.x];
+        stage_args(d_arg, sc_arg, r, s_args); // (its barrier publishes the table too)
+        FinishLds Lr;
+        Lr.sm = &sm;
+        Lr.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
+        Lr.sortk = s_dyn64;
+        Lr.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
+        finish_topk_row(s_args.d, s_args.sc, s_args.P, r, slices, Lr);
+        return;
+    }
     const uint32_t n_work = sc_arg.work_n[1];
     const uint32_t row = sc_arg.work_tail[blockIdx.y], tid = threadIdx.x; // (the list has room for every workgroup)
     if (blockIdx.y >= n_work)
