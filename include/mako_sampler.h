@@ -11,9 +11,11 @@
  * draws replaced by the caller's u (and u2).
  *
  * Every pointer inside mako_sample_desc is a DEVICE pointer; the host-pointer
- * convenience call stages through context-owned buffers.  The library never
- * writes the caller's logits, allocates nothing on the sampling path, and
- * reports failures as negative status codes (the reference throws
+ * convenience call stages through context-owned buffers, which it allocates
+ * on its first call.  The library never writes the caller's logits; the
+ * mako_sampler_sample_batch* calls allocate nothing (their scratch memory is
+ * allocated by mako_sampler_create, or is part of the library's image); and
+ * failures are reported as negative status codes (the reference throws
  * std::invalid_argument, src/gen/sampler.cpp:11-12).
  */
 #ifndef MAKO_SAMPLER_H
@@ -129,6 +131,20 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
  * top_k == 0 rows takes two launches instead of six).  The results never depend on it; null = the call above. */
 int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_desc* desc,
                                      const mako_sampling_params* params_host, void* stream);
+
+/* mako_sampler_sample_batch for callers that must not allocate device memory around the call and want none held per
+ * context: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  The kernels' scratch memory (candidate lists, histograms, sort buffers, work lists)
+ * is not the context's but an array of MAKO_STATIC_SCRATCH_MIB MiB inside the library's image, of which every GPU
+ * that the library runs on holds one copy until the process ends; mako_sampler_create() looks its address up once
+ * per device.  Batches of up to MAKO_STATIC_MAX_ROWS rows of up to MAKO_STATIC_MAX_VOCAB logits; anything larger is
+ * refused with MAKO_ERR_INVALID_ARG.  No hipMalloc, hipFree or other allocating call is made.  Results are those
+ * of mako_sampler_sample_batch, bit for bit.  All contexts of one GPU share that GPU's array: calls that overlap
+ * on one GPU (two streams, two threads) race; calls in stream order do not. */
+#define MAKO_STATIC_MAX_ROWS 16
+#define MAKO_STATIC_MAX_VOCAB 131072
+#define MAKO_STATIC_SCRATCH_MIB 52
+int mako_sampler_sample_batch_static(mako_sampler_ctx* ctx, const mako_sample_desc* desc, void* stream);
 
 /* Host-pointer convenience call with the reference's calling convention
  * (host logits, src/gen/session.cpp:443): copies the rows to the device,

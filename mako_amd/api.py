@@ -81,11 +81,14 @@ class Desc(C.Structure):
     ]
 
 
+STATIC_MAX_ROWS, STATIC_MAX_VOCAB = 16, 131072  # MAKO_STATIC_MAX_ROWS, MAKO_STATIC_MAX_VOCAB
+
 EXPORTS = [
     "mako_sampler_create",
     "mako_sampler_destroy",
     "mako_sampler_sample_batch",
     "mako_sampler_sample_batch_hinted",
+    "mako_sampler_sample_batch_static",
     "mako_sampler_sample_host",
     "mako_sampler_last_error",
     "mako_sampler_slices",
@@ -108,6 +111,7 @@ def load():
         lib.mako_sampler_destroy.argtypes = [C.c_void_p]
         lib.mako_sampler_sample_batch.argtypes = [C.c_void_p, C.POINTER(Desc), C.c_void_p]
         lib.mako_sampler_sample_batch_hinted.argtypes = [C.c_void_p, C.POINTER(Desc), C.c_void_p, C.c_void_p]
+        lib.mako_sampler_sample_batch_static.argtypes = [C.c_void_p, C.POINTER(Desc), C.c_void_p]
         lib.mako_sampler_last_error.restype = C.c_char_p
         lib.mako_sampler_last_error.argtypes = [C.c_void_p]
         lib.mako_sampler_set_profile.argtypes = [C.c_void_p, C.c_int]
@@ -178,6 +182,13 @@ class SamplerContext:
             rc = self.lib.mako_sampler_sample_batch(self.ptr, C.byref(desc), stream.ptr if stream else None)
         if rc != MAKO_OK:
             raise MakoError("mako_sampler_sample_batch: %d %s" % (rc, self.last_error()))
+
+    def sample_batch_static(self, desc, stream=None):
+        """mako_sampler_sample_batch_static: the same batch on the library's own scratch memory (STATIC_MAX_ROWS x
+        STATIC_MAX_VOCAB at most); allocates nothing."""
+        rc = self.lib.mako_sampler_sample_batch_static(self.ptr, C.byref(desc), stream.ptr if stream else None)
+        if rc != MAKO_OK:
+            raise MakoError("mako_sampler_sample_batch_static: %d %s" % (rc, self.last_error()))
 
 
 class Batch:

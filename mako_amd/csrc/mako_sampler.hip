@@ -6,6 +6,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
 #include <new>
 #include <string>
 
@@ -84,6 +85,122 @@ uint32_t slice_len_for(uint32_t n_vocab, uint32_t slices)
     return (len + 3u) & ~3u;
 }
 
+
+int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampling_params* params_host, void* stream,
+              const mako::Scratch& sc, const mako::Scratch* sc_dev, uint32_t max_rows, uint32_t max_vocab);
+
+#define MAKO_STR2(x) #x
+#define MAKO_STR(x) MAKO_STR2(x)
+
+// The kernels' scratch memory for batches of up to max_rows rows of up to max_vocab logits, every array taken from
+// `take` (256-byte aligned blocks); *sc_dev gets room for the device copy of the record itself.
+template <typename Take>
+hipError_t layout_scratch(mako::Scratch& sc, mako::Scratch** sc_dev, uint32_t max_rows, uint32_t max_vocab, Take take)
+{
+#define MAKO_TAKE(ptr, count)                                                                                      \
+    do {                                                                                                           \
+        hipError_t e_ = take(reinterpret_cast<void**>(&(ptr)), (size_t)(count) * sizeof(*(ptr)));                  \
+        if (e_ != hipSuccess)                                                                                      \
+            return e_;                                                                                             \
+    } while (0)
+    sc.vpad = ((uint64_t)max_vocab + 1023u) & ~1023ull;
+    const size_t rv = (size_t)max_rows * sc.vpad;
+    sc.slices_cap = mako_sampler_slices(max_vocab);
+    MAKO_TAKE(*sc_dev, 1);
+    MAKO_TAKE(sc.stats, (size_t)max_rows * mako::kMaxSlices);
+    MAKO_TAKE(sc.cand_w, (size_t)max_rows * sc.slices_cap * mako::kCap);
+    MAKO_TAKE(sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap);
+    MAKO_TAKE(sc.part_sum, (size_t)max_rows * mako::kMaxSlices);
+    MAKO_TAKE(sc.part_n, (size_t)max_rows * mako::kMaxSlices);
+    MAKO_TAKE(sc.plan, (size_t)max_rows);
+    MAKO_TAKE(sc.bins, (size_t)max_rows * mako::kBins);
+    MAKO_TAKE(sc.wbuf, rv);
+    MAKO_TAKE(sc.cnt, rv);
+    MAKO_TAKE(sc.key[0], rv);
+    MAKO_TAKE(sc.key[1], rv);
+    MAKO_TAKE(sc.idx[0], rv);
+    MAKO_TAKE(sc.idx[1], rv);
+    sc.g_cap = (uint32_t)(sc.vpad / mako::kGroup) + mako::kWorkers;
+    const size_t rg = (size_t)max_rows * sc.g_cap;
+    MAKO_TAKE(sc.gt.sum, rg);
+    MAKO_TAKE(sc.gt.d0, rg);
+    MAKO_TAKE(sc.gt.d1, rg);
+    MAKO_TAKE(sc.gt.cmax, rg);
+    MAKO_TAKE(sc.gt.start, rg);
+    MAKO_TAKE(sc.gt.pack, rg);
+    MAKO_TAKE(sc.gt.quarters, rg * 4);
+    MAKO_TAKE(sc.bin_worker, (size_t)max_rows * mako::kBins);
+    MAKO_TAKE(sc.work_n, 8);
+    MAKO_TAKE(sc.work_sort, (size_t)max_rows * mako::kWorkers);
+    MAKO_TAKE(sc.work_tail, (size_t)max_rows);
+#undef MAKO_TAKE
+    return hipSuccess;
+}
+
+// What the kernels expect to find zero before a context's first batch (they leave it zero after every batch).
+hipError_t zero_scratch(const mako::Scratch& sc, uint32_t max_rows)
+{
+    hipError_t e = hipMemset(sc.plan, 0, (size_t)max_rows * sizeof(mako::BigPlan));
+    if (e == hipSuccess)
+        e = hipMemset(sc.bins, 0, (size_t)max_rows * mako::kBins * sizeof(unsigned long long));
+    if (e == hipSuccess)
+        e = hipMemset(sc.cnt, 0, (size_t)max_rows * sc.vpad * sizeof(uint32_t));
+    if (e == hipSuccess)
+        e = hipMemset(sc.work_n, 0, 8 * sizeof(uint32_t));
+    return e;
+}
+
+// ---- scratch memory that is part of the library's image: mako_sampler_sample_batch_static() ----
+// One array per GPU (the loader places a copy on every device the library runs on, for the life of the process),
+// laid out once per device for MAKO_STATIC_MAX_ROWS rows of MAKO_STATIC_MAX_VOCAB logits.  `scratch` itself is only
+// a host-side handle: everything below works on the device address hipGetSymbolAddress() returns for the current
+// device.
+constexpr size_t kStaticBytes = (size_t)MAKO_STATIC_SCRATCH_MIB << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+constexpr int kStaticDevices = 64;
+struct StaticScratch {
+    bool ready = false;
+    hipError_t status = hipSuccess; // of the set-up, kept: a device whose set-up failed refuses every call
+    mako::Scratch sc{};
+    mako::Scratch* sc_dev = nullptr;
+};
+StaticScratch g_static[kStaticDevices];
+std::mutex g_static_mutex;
+
+// Once per device, with that device current (mako_sampler_create() calls it).
+hipError_t setup_static_scratch(int device)
+{
+    if (device < 0 || device >= kStaticDevices)
+        return hipSuccess; // (such a device's contexts refuse the static entry point)
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    StaticScratch& g = g_static[device];
+    if (g.ready)
+        return g.status;
+    unsigned char* base = nullptr;
+    hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&base), HIP_SYMBOL(scratch));
+    if (e == hipSuccess && (!base || (reinterpret_cast<uintptr_t>(base) & 255u)))
+        e = hipErrorInvalidSymbol;
+    size_t used = 0;
+    if (e == hipSuccess)
+        e = layout_scratch(g.sc, &g.sc_dev, MAKO_STATIC_MAX_ROWS, MAKO_STATIC_MAX_VOCAB, [&](void** p, size_t bytes) {
+            if (bytes > kStaticBytes - used)
+                return hipErrorOutOfMemory;
+            *p = base + used;
+            used += (bytes + 255u) & ~(size_t)255u;
+            return hipSuccess;
+        });
+    if (e == hipSuccess)
+        e = zero_scratch(g.sc, MAKO_STATIC_MAX_ROWS);
+    if (e == hipSuccess)
+        e = hipMemcpy(g.sc_dev, &g.sc, sizeof g.sc, hipMemcpyHostToDevice);
+    if (e == hipSuccess)
+        e = hipDeviceSynchronize();
+    g.status = e;
+    g.ready = true;
+    return e;
+}
+
 } // namespace
 
 extern "C" {
@@ -116,42 +233,10 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
         if (n > 0)
             ctx->cus = (uint32_t)n;
     }
-    mako::Scratch& sc = ctx->sc;
-    sc.vpad = ((uint64_t)max_vocab + 1023u) & ~1023ull;
-    const size_t rv = (size_t)max_rows * sc.vpad;
-    sc.slices_cap = mako_sampler_slices(max_vocab);
-    MAKO_HIP(ctx, dev_alloc(&sc.stats, (size_t)max_rows * mako::kMaxSlices));
-    MAKO_HIP(ctx, dev_alloc(&sc.cand_w, (size_t)max_rows * sc.slices_cap * mako::kCap));
-    MAKO_HIP(ctx, dev_alloc(&sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap));
-    MAKO_HIP(ctx, dev_alloc(&sc.part_sum, (size_t)max_rows * mako::kMaxSlices));
-    MAKO_HIP(ctx, dev_alloc(&sc.part_n, (size_t)max_rows * mako::kMaxSlices));
-    MAKO_HIP(ctx, dev_alloc(&sc.plan, (size_t)max_rows));
-    MAKO_HIP(ctx, hipMemset(sc.plan, 0, (size_t)max_rows * sizeof(mako::BigPlan)));
-    MAKO_HIP(ctx, dev_alloc(&sc.bins, (size_t)max_rows * mako::kBins));
-    MAKO_HIP(ctx, hipMemset(sc.bins, 0, (size_t)max_rows * mako::kBins * sizeof(unsigned long long)));
-    MAKO_HIP(ctx, dev_alloc(&sc.wbuf, rv));
-    MAKO_HIP(ctx, dev_alloc(&sc.cnt, rv));
-    MAKO_HIP(ctx, dev_alloc(&sc.key[0], rv));
-    MAKO_HIP(ctx, dev_alloc(&sc.key[1], rv));
-    MAKO_HIP(ctx, dev_alloc(&sc.idx[0], rv));
-    MAKO_HIP(ctx, dev_alloc(&sc.idx[1], rv));
-    MAKO_HIP(ctx, hipMemset(sc.cnt, 0, rv * sizeof(uint32_t)));
-    sc.g_cap = (uint32_t)(sc.vpad / mako::kGroup) + mako::kWorkers;
-    const size_t rg = (size_t)max_rows * sc.g_cap;
-    MAKO_HIP(ctx, dev_alloc(&sc.gt.sum, rg));
-    MAKO_HIP(ctx, dev_alloc(&sc.gt.d0, rg));
-    MAKO_HIP(ctx, dev_alloc(&sc.gt.d1, rg));
-    MAKO_HIP(ctx, dev_alloc(&sc.gt.cmax, rg));
-    MAKO_HIP(ctx, dev_alloc(&sc.gt.start, rg));
-    MAKO_HIP(ctx, dev_alloc(&sc.gt.pack, rg));
-    MAKO_HIP(ctx, dev_alloc(&sc.gt.quarters, rg * 4));
-    MAKO_HIP(ctx, dev_alloc(&sc.bin_worker, (size_t)max_rows * mako::kBins));
-    MAKO_HIP(ctx, dev_alloc(&sc.work_n, 8));
-    MAKO_HIP(ctx, hipMemset(sc.work_n, 0, 8 * sizeof(uint32_t)));
-    MAKO_HIP(ctx, dev_alloc(&sc.work_sort, (size_t)max_rows * mako::kWorkers));
-    MAKO_HIP(ctx, dev_alloc(&sc.work_tail, (size_t)max_rows));
-    MAKO_HIP(ctx, dev_alloc(&ctx->sc_dev, 1));
-    MAKO_HIP(ctx, hipMemcpy(ctx->sc_dev, &sc, sizeof sc, hipMemcpyHostToDevice));
+    MAKO_HIP(ctx, layout_scratch(ctx->sc, &ctx->sc_dev, max_rows, max_vocab, [](void** p, size_t bytes) { return hipMalloc(p, bytes); }));
+    MAKO_HIP(ctx, zero_scratch(ctx->sc, max_rows));
+    MAKO_HIP(ctx, hipMemcpy(ctx->sc_dev, &ctx->sc, sizeof ctx->sc, hipMemcpyHostToDevice));
+    MAKO_HIP(ctx, setup_static_scratch(device));
     MAKO_HIP(ctx, hipDeviceSynchronize());
     // the kernels overlay up to 64 KB of dynamic LDS (sort_kernel more) on a few KB of static LDS
     MAKO_HIP(ctx, mako::init_scan_kernels());
@@ -224,14 +309,41 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
 {
     if (!ctx || !desc)
         return MAKO_ERR_INVALID_ARG;
-    const mako_sample_desc& d = *desc;
+    MAKO_HIP(ctx, hipSetDevice(ctx->device));
+    return run_batch(ctx, *desc, params_host, stream, ctx->sc, ctx->sc_dev, ctx->max_rows, ctx->max_vocab);
+}
+
+int mako_sampler_sample_batch_static(mako_sampler_ctx* ctx, const mako_sample_desc* desc, void* stream)
+{
+    if (!ctx || !desc)
+        return MAKO_ERR_INVALID_ARG;
+    if (desc->n_rows > MAKO_STATIC_MAX_ROWS || desc->n_vocab > MAKO_STATIC_MAX_VOCAB)
+        return fail(ctx, MAKO_ERR_INVALID_ARG,
+                    "sampler: the library's own scratch memory holds batches of up to " MAKO_STR(MAKO_STATIC_MAX_ROWS)
+                    " rows of up to " MAKO_STR(MAKO_STATIC_MAX_VOCAB) " logits");
+    if (ctx->device < 0 || ctx->device >= kStaticDevices)
+        return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: no static scratch memory for this device ordinal");
+    const StaticScratch& g = g_static[ctx->device]; // (set up by mako_sampler_create(), never written afterwards)
+    if (!g.ready || g.status != hipSuccess)
+        return fail(ctx, MAKO_ERR_HIP, "sampler: the static scratch memory could not be set up on this device");
+    MAKO_HIP(ctx, hipSetDevice(ctx->device));
+    return run_batch(ctx, *desc, nullptr, stream, g.sc, g.sc_dev, MAKO_STATIC_MAX_ROWS, MAKO_STATIC_MAX_VOCAB);
+}
+
+} // extern "C"
+
+namespace {
+// One batch through the kernels, on scratch memory laid out for max_rows x max_vocab.  Allocates nothing.
+int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampling_params* params_host, void* stream,
+              const mako::Scratch& sc, const mako::Scratch* sc_dev, uint32_t max_rows, uint32_t max_vocab)
+{
     if (d.n_vocab == 0)
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: empty vocabulary"); // sampler.cpp:11-12
     if (d.n_rows == 0)
         return MAKO_OK;
     if (!d.logits || !d.params || !d.u || !d.out_tokens)
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: logits, params, u and out_tokens are required");
-    if (d.n_rows > ctx->max_rows || d.n_vocab > ctx->max_vocab)
+    if (d.n_rows > max_rows || d.n_vocab > max_vocab)
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: batch exceeds the context's max_rows/max_vocab");
     if (d.logits_stride < (int64_t)d.n_vocab)
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: logits_stride < n_vocab");
@@ -290,32 +402,35 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
     }
     const bool launch_sort = any_nucleus || any_general;
     MAKO_MARK(0);
-    mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, ctx->sc, slice_len, ctx->cus);
+    mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, sc, slice_len, ctx->cus);
     MAKO_MARK(1);
     if (any_nucleus)
-        mako::launch_finish(vec, kh, finish_wgs, st, d, ctx->sc_dev, slices);
+        mako::launch_finish(vec, kh, finish_wgs, st, d, sc_dev, slices);
     MAKO_MARK(2);
     // top_k == 0 rows: plan from the row's histogram, sort by the plan, cut and draw; the stages talk through
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  Other rows cost a load.
     if (launch_sort)
-        mako::launch_plan_for_sort(st, d, ctx->sc_dev, slices);
+        mako::launch_plan_for_sort(st, d, sc_dev, slices);
     else
-        mako::launch_plan_alone(st, d, ctx->sc_dev, slices);
+        mako::launch_plan_alone(st, d, sc_dev, slices);
     MAKO_MARK(3);
     if (any_nucleus)
-        mako::launch_partition(st, d, ctx->sc, list_rows);
+        mako::launch_partition(st, d, sc, list_rows);
     MAKO_MARK(4);
     if (launch_sort)
-        mako::launch_sort(st, d, ctx->sc, slices, list_rows);
+        mako::launch_sort(st, d, sc, slices, list_rows);
     MAKO_MARK(5);
     if (launch_sort) // (also finishes the top-k rows that plan_kernel<false> leaves)
-        mako::launch_tail(st, d, ctx->sc, slices, nucleus_rows);
+        mako::launch_tail(st, d, sc, slices, nucleus_rows);
     MAKO_MARK(6);
 #undef MAKO_MARK
     ctx->profiled = prof;
     MAKO_HIP(ctx, hipGetLastError());
     return MAKO_OK;
 }
+} // namespace
+
+extern "C" {
 
 int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t logits_stride, uint32_t n_rows,
                              uint32_t n_vocab, const mako_sampling_params* params, const float* u,
