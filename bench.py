@@ -23,8 +23,20 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per batch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
-# for a device-to-device copy of known size (see the traffic summary under profiles/)
-MEASURED_TRAFFIC_BYTES = {"config3": 74.8e6}
+# for a device-to-device copy of known size: records written by mako_amd/traffic_record.py, each tied to the kernel
+# sources it was measured on (null is reported once they have changed)
+TRAFFIC_RECORDS = {"config3": os.path.join(ROOT, "profiles", "config3_hbm_traffic.json")}
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return None
 
 
 def make_workload(name):
@@ -57,7 +69,7 @@ def cpu_baseline(w, budget_s):
     from oracle import pyoracle
     ref = pyoracle.reference()
     rows = w["logits"].shape[0]
-    cores = max(1, min(os.cpu_count() or 1, 16))
+    cores = os.cpu_count() or 1
     if ref is not None:
         kw = dict(hist=w.get("hist"), hist_len=w.get("hist_len"), mask=w.get("mask"))
         t1, tok = ref.sample_batch_timed(w["logits"], w["params"], w["seeds"], n_threads=1, **kw)
@@ -68,7 +80,7 @@ def cpu_baseline(w, budget_s):
             wall += time.perf_counter() - t0
             spent += wall / (reps + 1)
             reps += 1
-        return dict(value=rows * reps / wall, unit="rows/s", cores=cores, kind="reference",
+        return dict(value=rows * reps / wall, unit="rows/s", cores=cores, cpu_model=cpu_model(), kind="reference",
                     value_1thread=rows / t1,
                     sample="%d x the %d-row %s batch, one fresh Sampler per row, sample() only (history replay and "
                            "thread start included in the %d-thread wall time)" % (reps, rows, w["name"], cores)), tok
@@ -81,7 +93,7 @@ def cpu_baseline(w, budget_s):
         hist = w["hist"][r, : w["hist_len"][r]] if "hist" in w else None
         tok.append(o.sample(w["logits"][r], p, float(w["u"][r]), hist, w["mask"][r] if "mask" in w else None)[0])
     dt = time.perf_counter() - t0
-    return dict(value=n / dt, unit="rows/s", cores=1, kind="port",
+    return dict(value=n / dt, unit="rows/s", cores=1, cpu_model=cpu_model(), kind="port",
                 sample="first %d rows of the %s batch through the plain-C oracle" % (n, w["name"])), None
 
 
@@ -236,6 +248,8 @@ def main():
         parity = dict(rows=rows, mismatches=int((np.asarray(ref_tok) != tokens).sum()), against="reference sampler")
 
     achieved = batch_bytes / (ms_per_step * 1e-3) / 1e9
+    from mako_amd import traffic_record
+    traffic = traffic_record.load_record(TRAFFIC_RECORDS[a.workload], a.workload) if a.workload in TRAFFIC_RECORDS else None
     out = {
         "metric": "sampled rows/sec at B=64xV=129280 fp32; achieved HBM GB/s vs peak",
         "value": rows * a.steps / (ms * 1e-3),
@@ -253,7 +267,7 @@ def main():
                    "rows": rows, "vocab": vocab, "logit_copies_rotated": n_copies,
                    "host_wall_ms_per_step": wall * 1e3 / a.steps},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "bytes_per_launch": batch_bytes,
                      "kernel": "scan + finish + plan + partition + sort + tail kernels (the six launches of one batch)",
                      "launch_ms": ms_per_step,

@@ -8,8 +8,9 @@
 // uniform the reference would draw through uniform_real_distribution<float> is
 // drawn here with generate_canonical<float, 24> and handed to the device, so
 // with the same standard library the token stream is the reference's.
-// Logits are host pointers, as in src/gen/session.cpp:443; sample_device()
-// takes a device pointer instead.  Link with libmako_sampler.so.
+// Logits are host pointers, as in src/gen/session.cpp:443 (device-resident
+// logits go through mako_sampler_sample_batch of the C ABI instead).  Link with
+// libmako_sampler.so.
 #pragma once
 
 #include <cstdint>

@@ -159,6 +159,7 @@ constexpr size_t kStaticBytes = (size_t)MAKO_STATIC_SCRATCH_MIB << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticBytes];
 
 constexpr int kStaticDevices = 64;
+constexpr uint64_t kGridYMax = 65535; // workgroups in a grid's y dimension
 struct StaticScratch {
     bool ready = false;
     hipError_t status = hipSuccess; // of the set-up, kept: a device whose set-up failed refuses every call
@@ -365,6 +366,9 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uint32_t slices = mako_sampler_slices(d.n_vocab);
+    // (rows, and rows x slices, index the y dimension of the kernels' grids)
+    if ((uint64_t)d.n_rows * std::max(slices, 2u) > kGridYMax)
+        return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: n_rows x slices exceeds what one launch can index");
     const uint32_t slice_len = slice_len_for(d.n_vocab, slices);
     const bool vec = d.n_vocab % 4 == 0 && d.logits_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(d.logits) & 15u) == 0;
     const size_t lds = d.hist_tokens ? (size_t)slice_len * sizeof(uint32_t) : 0;
@@ -401,31 +405,37 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
         list_rows = std::max(n_nucleus + (n_other + mako::kWorkers - 1u) / mako::kWorkers, 1u);
     }
     const bool launch_sort = any_nucleus || any_general;
+    // (a launch that fails stops the batch there: the kernels after it would work on what it did not write)
+#define MAKO_LAUNCH(call)                                                                                          \
+    do {                                                                                                           \
+        call;                                                                                                      \
+        MAKO_HIP(ctx, hipGetLastError());                                                                          \
+    } while (0)
     MAKO_MARK(0);
-    mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, sc, slice_len, ctx->cus);
+    MAKO_LAUNCH(mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, sc, slice_len, ctx->cus));
     MAKO_MARK(1);
     if (any_nucleus)
-        mako::launch_finish(vec, kh, finish_wgs, st, d, sc_dev, slices);
+        MAKO_LAUNCH(mako::launch_finish(vec, kh, finish_wgs, st, d, sc_dev, slices));
     MAKO_MARK(2);
     // top_k == 0 rows: plan from the row's histogram, sort by the plan, cut and draw; the stages talk through
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  Other rows cost a load.
     if (launch_sort)
-        mako::launch_plan_for_sort(st, d, sc_dev, slices);
+        MAKO_LAUNCH(mako::launch_plan_for_sort(st, d, sc_dev, slices));
     else
-        mako::launch_plan_alone(st, d, sc_dev, slices);
+        MAKO_LAUNCH(mako::launch_plan_alone(st, d, sc_dev, slices));
     MAKO_MARK(3);
     if (any_nucleus)
-        mako::launch_partition(st, d, sc, list_rows);
+        MAKO_LAUNCH(mako::launch_partition(st, d, sc, list_rows));
     MAKO_MARK(4);
     if (launch_sort)
-        mako::launch_sort(st, d, sc, slices, list_rows);
+        MAKO_LAUNCH(mako::launch_sort(st, d, sc, slices, list_rows));
     MAKO_MARK(5);
     if (launch_sort) // (also finishes the top-k rows that plan_kernel<false> leaves)
-        mako::launch_tail(st, d, sc, slices, nucleus_rows);
+        MAKO_LAUNCH(mako::launch_tail(st, d, sc, slices, nucleus_rows));
     MAKO_MARK(6);
 #undef MAKO_MARK
+#undef MAKO_LAUNCH
     ctx->profiled = prof;
-    MAKO_HIP(ctx, hipGetLastError());
     return MAKO_OK;
 }
 } // namespace
@@ -450,6 +460,14 @@ int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: history exceeds the context's max_hist");
     if ((draft != nullptr) != (u2 != nullptr) || (draft != nullptr) != (out_accepted != nullptr))
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: draft, u2 and out_accepted go together");
+    if (logits_stride < (int64_t)n_vocab)
+        return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: logits_stride < n_vocab");
+    if (mask && mask_stride < (int64_t)(((uint64_t)n_vocab + 31) / 32))
+        return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: mask_stride < ceil(n_vocab / 32)");
+    if (hist_tokens && hist_stride > 0)
+        for (uint32_t r = 0; r < n_rows; ++r) // (columns beyond hist_stride of the staging rows hold older calls' ids)
+            if (hist_len[r] > (uint64_t)hist_stride)
+                return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: hist_len[r] > hist_stride");
     MAKO_HIP(ctx, hipSetDevice(ctx->device));
     const size_t R = ctx->max_rows;
     const size_t mwords = ((size_t)ctx->max_vocab + 31) / 32;

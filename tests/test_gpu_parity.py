@@ -409,6 +409,21 @@ def test_config5_masks(gpu_ctx):
         assert_parity(gpu_ctx, workloads.config5(rows=32, density=density))
 
 
+def test_config4_all_256_rows(gpu_ctx):
+    """The whole benchmark batch (128 heavy-tailed rows, 128 near-flat ones with ~133K-token nuclei) against the
+    oracle: the second pass's looped piece search, whole-slice pieces and sort_kernel's rounds of workgroups only
+    occur beyond 64 rows."""
+    g = assert_parity(gpu_ctx, workloads.config4(), cap=512)
+    _say("config4 (256 rows) paths: %s" % np.bincount(g["path"], minlength=6).tolist())
+
+
+@pytest.mark.parametrize("density", [0.01, 0.5])
+def test_config5_all_256_rows(gpu_ctx, density):
+    """The whole verify-shaped batch (32 x 8 rows under per-row bitmasks) against the oracle."""
+    g = assert_parity(gpu_ctx, workloads.config5(density=density), cap=64)
+    _say("config5 (256 rows, density %g) paths: %s" % (density, np.bincount(g["path"], minlength=6).tolist()))
+
+
 def test_wide_nucleus_walk_depths(gpu_ctx):
     """top_k = 0 rows whose nuclei hold tens of thousands of tokens, drawn at u from 0 to 1 - 2^-24: the walk
     ends anywhere between the first candidate and the last, crossing many binades of r on the way."""
@@ -588,3 +603,29 @@ def test_argument_errors(gpu_ctx):
     d.n_rows = 100000
     with pytest.raises(api.MakoError, match="exceeds"):
         gpu_ctx.sample_batch(d)
+
+
+def test_host_call_argument_errors(gpu_ctx):
+    """The host-pointer call refuses strides that do not cover a row and history lengths beyond the stride (the
+    staging rows' further columns hold older calls' ids) instead of sampling from them."""
+    v, rows = 4096, 2
+    w = workloads.config1(rows=rows, vocab=v)
+    lg = np.ascontiguousarray(w["logits"], np.float32)
+    pr = np.ascontiguousarray(w["params"])
+    uu = np.ascontiguousarray(w["u"], np.float32)
+    hist = np.zeros((rows, 8), np.int32)
+    mask = np.full((rows, v // 32), 0xffffffff, np.uint32)
+    tok = np.zeros(rows, np.int32)
+
+    def call(logits_stride=v, mask_stride=v // 32, hlen=(8, 8)):
+        hl = np.array(hlen, np.uint32)
+        return gpu_ctx.lib.mako_sampler_sample_host(
+            gpu_ctx.ptr, lg.ctypes.data, logits_stride, rows, v, pr.ctypes.data, uu.ctypes.data, mask.ctypes.data,
+            mask_stride, hist.ctypes.data, None, 8, hl.ctypes.data, None, None, None, tok.ctypes.data)
+
+    assert call() == api.MAKO_OK
+    good = tok.copy()
+    assert call(logits_stride=v - 1) == api.MAKO_ERR_INVALID_ARG and "logits_stride" in gpu_ctx.last_error()
+    assert call(mask_stride=v // 32 - 1) == api.MAKO_ERR_INVALID_ARG and "mask_stride" in gpu_ctx.last_error()
+    assert call(hlen=(8, 9)) == api.MAKO_ERR_INVALID_ARG and "hist_len" in gpu_ctx.last_error()
+    assert call() == api.MAKO_OK and np.array_equal(tok, good)

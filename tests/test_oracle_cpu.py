@@ -308,3 +308,28 @@ def test_close_forced_known_answers(oracle):
             continue
         want = int(np.sum(np.where(allowed, x, -np.inf) > x[t]))
         assert above == want and tok == (t if want < k else -1)
+
+
+SANITIZE = ["-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-static-libasan",
+            "-ffp-contract=off"]
+
+
+def test_oracle_under_sanitizers():
+    """oracle.c under AddressSanitizer and UndefinedBehaviorSanitizer on 1400 random calls (every parameter
+    combination, histories, masks, traces; tests/cpu/oracle_sanitized.c)."""
+    exe = os.path.join(HERE, "cpu", "oracle_sanitized")
+    subprocess.run(["gcc", "-std=c11", "-mfma", *SANITIZE, "-I", os.path.join(HERE, "..", "oracle"),
+                    os.path.join(HERE, "cpu", "oracle_sanitized.c"), os.path.join(HERE, "..", "oracle", "oracle.c"),
+                    "-o", exe, "-lm"], check=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and out.stdout.strip().endswith(" 0 failures"), out.stdout + out.stderr
+
+
+@pytest.mark.parametrize("name", ["seqfp_test", "gen_helpers_test"])
+def test_host_code_under_sanitizers(name):
+    """The host-side C++ the library shares with its kernels (seqfp.h) and ships (include/gen/), likewise."""
+    exe = os.path.join(HERE, "cpu", name + "_san")
+    subprocess.run(["g++", "-std=c++17", *SANITIZE, "-I", os.path.join(HERE, "..", "include"),
+                    os.path.join(HERE, "cpu", name + ".cpp"), "-o", exe], check=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and "0 failures" in out.stdout, out.stdout + out.stderr
