@@ -30,10 +30,15 @@ FLAGS = [
 # Every device function inlined into its kernel: no call stack, so the kernel needs no scratch memory (kernels
 # that use scratch run far fewer workgroups at a time on this chip).
 INLINE_ALL = ["-mllvm", "-amdgpu-function-calls=false"]
-# Per source.  tail_kernel calls the top-k row finisher out of line: few workgroups run it, and inlined it costs the
-# tails' own code registers and spills.
+# Per source (a source listed here is compiled WITHOUT INLINE_ALL): code that only rare rows reach is called, not
+# inlined, where it would cost a hot path registers and spills.  Such kernels use scratch memory for the calls, which
+# slows down the start of their workgroups: not for kernels that many workgroups run (sort_kernel: +15 %).
+RARE_CALLS = ["-DMAKO_RARE_CALL=__attribute__((noinline))"]
 SOURCE_FLAGS = {
-    "k_tail.hip": ["-DMAKO_ROWS_CALL=__attribute__((noinline))"],
+    # the late rows (top-k rows, the whole-row path, second looks at a cut) out of line beside the tails
+    "k_tail.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", *RARE_CALLS],
+    # the whole-row path and the second look at a cut that is too close to call, out of line beside the top-k rows
+    "k_plan_alone.hip": RARE_CALLS,
 }
 
 

@@ -387,24 +387,21 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
             MAKO_HIP(ctx, hipEventRecord(ctx->ev[i], st));                                                         \
     } while (0)
     // which kernels have work: all of them unless the caller's host copy of the parameters says otherwise
-    // and how long the finishing kernels' work lists can get: kWorkers entries per top_k == 0 row, one per other
-    // sampled row (whole-row rows, top-k rows that cannot be certified from their candidates)
-    bool any_nucleus = true, any_general = true;
-    uint32_t nucleus_rows = d.n_rows, list_rows = d.n_rows;
+    // (any_late: rows that are finished in tail_kernel's launch, after the plan)
+    bool any_nucleus = true, any_late = true;
+    uint32_t nucleus_rows = d.n_rows;
     if (params_host) {
-        any_nucleus = any_general = false;
-        uint32_t n_nucleus = 0, n_other = 0;
+        any_nucleus = any_late = false;
+        uint32_t n_nucleus = 0;
         for (uint32_t r = 0; r < d.n_rows; ++r) {
             const mako::RowClass c = mako::classify(params_host[r]);
             any_nucleus |= c == mako::kNucleus;
-            any_general |= c == mako::kGeneral;
+            any_late |= c == mako::kGeneral;
             n_nucleus += c == mako::kNucleus;
-            n_other += c == mako::kTopK || c == mako::kGeneral;
         }
         nucleus_rows = std::max(n_nucleus, 1u);
-        list_rows = std::max(n_nucleus + (n_other + mako::kWorkers - 1u) / mako::kWorkers, 1u);
     }
-    const bool launch_sort = any_nucleus || any_general;
+    const bool launch_sort = any_nucleus || any_late;
     // (a launch that fails stops the batch there: the kernels after it would work on what it did not write)
 #define MAKO_LAUNCH(call)                                                                                          \
     do {                                                                                                           \
@@ -425,12 +422,12 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
         MAKO_LAUNCH(mako::launch_plan_alone(st, d, sc_dev, slices));
     MAKO_MARK(3);
     if (any_nucleus)
-        MAKO_LAUNCH(mako::launch_partition(st, d, sc, list_rows));
+        MAKO_LAUNCH(mako::launch_partition(st, d, sc, nucleus_rows));
     MAKO_MARK(4);
-    if (launch_sort)
-        MAKO_LAUNCH(mako::launch_sort(st, d, sc, slices, list_rows));
+    if (any_nucleus)
+        MAKO_LAUNCH(mako::launch_sort(st, d, sc, slices, nucleus_rows));
     MAKO_MARK(5);
-    if (launch_sort) // (also finishes the top-k rows that plan_kernel<false> leaves)
+    if (launch_sort) // (also finishes the rows that plan_kernel<false> and sort_kernel leave: finish_late_row())
         MAKO_LAUNCH(mako::launch_tail(st, d, sc, slices, nucleus_rows));
     MAKO_MARK(6);
 #undef MAKO_MARK

@@ -11,7 +11,7 @@ namespace mako {
 // Returns n0, the number of weights to sort; the plan is written to `plan` (flag left untouched).
 __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, uint32_t c0, uint32_t c1,
                                  unsigned long long s0, unsigned long long s1, BigPlan* plan, uint8_t* bin_worker,
-                                 const FinishLds& L, uint32_t& thr_bits)
+                                 const FinishLds& L, uint32_t& thr_bits, uint32_t n_vocab)
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
@@ -22,7 +22,8 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
         return __longlong_as_double((long long)(1023ull + e - 150ull) << 52);
     };
     const double m0 = (double)s0 * scale(b0), m1 = (double)s1 * scale(b1);
-    const double want = (double)P.top_p * total64;
+    // (what the reference's sums can make of `want`, at most: see order_band())
+    const double want = (double)P.top_p * total64 + 2.0 * order_band(n_vocab, total64);
     uint32_t* w_hi = L.wcount;            // highest bin of each worker
     uint32_t* w_lo = L.wcount + kWorkers; // lowest bin
     uint32_t* w_off = L.wcount + 2 * kWorkers;
@@ -56,26 +57,26 @@ __device__ uint32_t plan_nucleus(const mako_sampling_params& P, double total64, 
     MAKO_STAMP(20);
     const double incl = pre_m + mass_w;
     const uint32_t above0 = pre_c + cnt_w - (c0 + c1), above1 = above0 + c0;
-    // The nucleus ends in the first bin (from the top) at which the running mass reaches `want`.  These sums
-    // associate differently from the sorted prefix sums that make the final decision, so one more non-empty
-    // bin is taken along: the list stops at the SECOND bin that satisfies the test.
+    // The nucleus ends by the first bin (from the top) at which the running mass reaches `want`: these sums
+    // associate differently from the sorted prefix sums that make the final decision and from the reference's, and
+    // `want` carries the band by which any of them can differ.
     const bool r0 = c0 && incl - m1 >= want, r1 = c1 && incl >= want;
     const uint32_t reached = (uint32_t)r0 + (uint32_t)r1;
     const uint32_t reached_w = __ockl_wfscan_add_u32(reached, true);
     if (lane_id() == kWave - 1)
         sm.hist[wave_id()] = reached_w;
     if (tid == 0) {
-        sm.ticket = 0;        // the lowest bin taken; not reached twice: every candidate is kept
+        sm.ticket = 0;        // the lowest bin taken; never reached: every candidate is kept
         sm.flag = count_all;  // the number of weights to sort
     }
     __syncthreads();
     uint32_t before = reached_w - reached;
     for (int w = 0; w < kWaves; ++w)
         before += w < wave_id() ? sm.hist[w] : 0u;
-    if (r0 && before + 1 == 2) {
+    if (r0 && before == 0) {
         sm.ticket = b0;
         sm.flag = above0 + c0;
-    } else if (r1 && before + (uint32_t)r0 + 1 == 2) {
+    } else if (r1 && before + (uint32_t)r0 == 0) {
         sm.ticket = b1;
         sm.flag = above1 + c1;
     }

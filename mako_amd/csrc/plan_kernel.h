@@ -6,39 +6,9 @@
 
 namespace mako {
 
-// A top-k row finished by one workgroup from the records and candidate lists scan_kernel left (all threads call;
-// sm.tab must hold the exp2 table): what plan_kernel<true> does for such a row, for tail_kernel's launch.  Rows that
-// plan_kernel<false> has dealt with (forced rows, rows it put on sort_kernel's whole-row list) are left alone.
-#ifndef MAKO_ROWS_CALL
-#define MAKO_ROWS_CALL __forceinline__
-#endif
-__device__ MAKO_ROWS_CALL void finish_topk_row(const mako_sample_desc& d, const Scratch& sc, const mako_sampling_params& P,
-                                               uint32_t row, uint32_t slices, const FinishLds& L)
-{
-    if (classify(P) != kTopK)
-        return;
-    if (d.force_token || d.close_token) { // uniform
-        int32_t ftok;
-        uint32_t above;
-        if (row_forced(d, sc, row, slices, ftok, above) != MAKO_FORCED_NONE)
-            return;
-    }
-    CandSlots pre;
-    const bool prefetched = !d.draft && slots_cover(slices); // uniform
-    if (prefetched)
-        fetch_candidate_slots(sc, row, slices, pre);
-    float m;
-    uint32_t argidx, n_cands, any_overflow;
-    SliceStat lane_stat;
-    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow, &lane_stat);
-    if (topk_takes_whole_row(kTopK, any_overflow, n_cands))
-        return;
-    topk_row<true>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
-}
-
 // grid = (1, rows), one workgroup per row.  Rows whose token is forced, greedy rows and (INLINE_GENERAL only: in a
-// batch that goes on to sort_kernel and tail_kernel the top-k rows are finished beside the tails) top-k rows are
-// finished here from the records scan_kernel left; a top_k == 0 row's exact total, candidate count and weight histogram (from
+// batch that goes on to sort_kernel and tail_kernel, top-k and whole-row rows are finished beside the tails) top-k
+// rows are finished here from the records scan_kernel left; a top_k == 0 row's exact total, candidate count and weight histogram (from
 // finish_kernel) are summed over its pieces and the row is planned: handed to sort_kernel's workers, or, when the
 // nucleus is narrow enough to end inside the candidate lists, to its worker 0 alone.
 // INLINE_GENERAL: sort_kernel will not be launched for this batch (the host saw no row that needs it), so a row
@@ -121,24 +91,14 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     }
 
     if (cls != kNucleus) {
-        if (topk_takes_whole_row(cls, any_overflow, n_cands)) {
-            if constexpr (inline_general) {
+        // (in a batch that goes on to sort_kernel and tail_kernel, tail_kernel's launch finishes these rows beside the
+        // tails: finish_late_row())
+        if constexpr (inline_general) {
+            if (topk_takes_whole_row(cls, any_overflow, n_cands))
                 general_row<1>(d, sc, row, P, m, argidx, L);
-                return;
-            }
-            if (tid == 0) {
-                sc.plan[row].total64 = (double)m; // carries the row maximum and its first index to the whole-row path
-                sc.plan[row].n0 = argidx;
-                sc.plan[row].flag = 2;
-                sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
-            }
-            return;
+            else
+                topk_row(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
         }
-
-        if constexpr (!inline_general)
-            return; // (tail_kernel's launch finishes the batch's top-k rows beside the tails: finish_topk_row())
-        else
-            topk_row<inline_general>(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
         return;
     }
 
@@ -165,7 +125,7 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         return;
     }
     uint32_t thr_bits = 0;
-    const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, sc.bin_worker + (size_t)row * kBins, L, thr_bits);
+    const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, sc.bin_worker + (size_t)row * kBins, L, thr_bits, d.n_vocab);
     MAKO_STAMP(16);
     const bool narrow = !d.draft && n0 <= kSmall && !any_overflow && n_cands <= kSortMax;
     // (a list too long for the workers' group records goes to the whole-row path)

@@ -138,6 +138,24 @@ struct Scratch {
     uint32_t g_cap;    // vpad / kGroup + kWorkers
 };
 
+// Device functions that only rare rows reach (the whole-row path, the second look at a cut that is too close to
+// call).  The sources whose kernels have a hot path beside them are compiled with MAKO_RARE_CALL=__attribute__((noinline)):
+// inlined, such code costs the hot path registers and spills.
+#ifndef MAKO_RARE_CALL
+#define MAKO_RARE_CALL
+#endif
+
+// The reference adds a row's weights one after the other in fp64 (src/gen/sampler.cpp:46-48 in candidate order,
+// :55-56 in sorted order); the sums here associate differently (per thread, wave and workgroup; bin masses).  An
+// fp64 sum of n fp32 addends in ANY order lies within n * 2^-53 * total of the exact sum, so two orders differ by at
+// most twice that; order_band() is that bound with room for the roundings of the product top_p * total and of the
+// tree sums themselves.  A cut whose two neighbouring prefix sums both clear `want` by more than the band is the
+// reference's cut; any other is decided by wave_sequential_sum() on the reference's own order.
+__device__ __forceinline__ double order_band(uint32_t n_addends, double total64)
+{
+    return (double)(n_addends + 64u) * 0x1p-51 * total64;
+}
+
 // Total order on floats as unsigned keys: -inf < ... < -0 = +0 < ... < +inf.  Never called on NaN.
 __device__ __forceinline__ uint32_t order_key(float f)
 {

@@ -31,4 +31,5 @@
 #include "second_pass.h"
 #include "plan_kernel.h"
 #include "sort_kernels.h"
+#include "late_rows.h"
 #include "tail_kernel.h"

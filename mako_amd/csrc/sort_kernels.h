@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     const uint32_t row = item >> 8, w = item & 255u, tid = threadIdx.x;
     MAKO_ROW(row);
     const uint32_t flag = sc_arg.plan[row].flag;
-    if (flag == 0 || (flag != 1 && w != 0)) // (never: the list holds exactly the flagged rows' pieces)
+    if ((flag != 1 && flag != 3) || (flag == 3 && w != 0)) // (never: the list holds exactly the flagged rows' pieces)
         return;
     stage_args(d_arg, sc_arg, row, s_args);
     const mako_sample_desc& d = s_args.d;
@@ -131,16 +131,6 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
     if (tid < 32)
         sm.tab[tid] = k_exp2_tab[tid];
-    if (flag == 2) {
-        // top_k > 128, no top-p, or a candidate list that could not be certified: the whole-row path
-        const float m = (float)plan->total64;
-        const uint32_t argidx = plan->n0;
-        __syncthreads();
-        if (tid == 0)
-            plan->flag = 0;
-        general_row<0>(d, sc, row, s_args.P, m, argidx, L);
-        return;
-    }
     const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
@@ -177,12 +167,9 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         if (n_list != kNone && n_list > 0 &&
             sorted_tail(d, row, P, kf, jf, n_list, true, total64, MAKO_PATH_NUCLEUS, L, true, q_bound))
             return;
-        // not certifiable from the candidates: the row's weights at or above the threshold, from its bits(q) array
-        if (!lds_sort_range(qk, d.n_vocab, thr_bits, 0x7f800001u, n0, key0, idx0, s_dyn64, sm)) {
-            gather_range(qk, d.n_vocab, thr_bits, 0x7f800001u, key0, idx0, n0, sm);
-            sort_segment(key0, idx0, key1, idx1, n0, L);
-        }
-        sorted_tail(d, row, P, key0, idx0, n0, true, total64, MAKO_PATH_GENERAL, L);
+        // not certifiable from the candidates: tail_kernel's launch takes a second look (narrow_second_look())
+        if (tid == 0)
+            plan->flag = 4;
         return;
     }
     uint32_t cnt = plan->cnt[w];

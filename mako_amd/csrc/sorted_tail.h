@@ -530,6 +530,70 @@ __device__ __forceinline__ ChainState sum_by_quarters(Keys kf, uint32_t st, uint
     return c;
 }
 
+// The band for a top-p cut in a sorted list of n weights q_at(0 .. n).  When total64 is the sum of
+// exactly these weights and the lightest one's last bit still lies within 53 bits of the total's first, no fp64
+// addition of any of these sums can round, whatever the order: all of them are exact, the reference's too, and the
+// comparison with `want` is the reference's (band 0).
+template <typename Get>
+__device__ __forceinline__ double cut_band(bool have_total, uint32_t n_vocab, uint32_t n, Get q_at, double total64)
+{
+    if (have_total)
+        return order_band(n_vocab, total64);
+    return total64 <= (double)q_at(n - 1u) * 0x1p29 ? 0.0 : order_band(n, total64);
+}
+
+// q_at(0) + q_at(1) + ... as the reference's loop adds them: one wave, one fp64 addition after the other, 256
+// entries per round (lane l brings entries 4l .. 4l+3, handed round lane by lane).  Stops after the round in which
+// the sum reaches `want` and returns in n_added how many entries the reference's `while (n < k && sum < want)` adds
+// (n, if the sum stays below `want`; pass +inf for a plain total).  Every lane returns the sum.  One wave calls it.
+template <typename Get>
+__device__ MAKO_RARE_CALL double wave_sequential_sum(Get q_at, uint32_t n, double want, uint32_t& n_added)
+{
+    double cum = 0.0;
+    n_added = n;
+    for (uint32_t base = 0; base < n; base += 4u * kWave) {
+        float q[4];
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t i = base + lane_id() * 4u + j;
+            q[j] = i < n ? q_at(i) : 0.0f;
+        }
+        const double before = cum;
+        for (uint32_t l = 0; l < kWave; ++l) {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                cum += (double)__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(q[j]), l));
+        }
+        if (cum >= want) { // (uniform) the reference stopped inside this round: again, entry by entry
+            cum = before;
+            uint32_t k = 0;
+            for (; k < 4u * kWave && base + k < n && cum < want; ++k)
+                cum += (double)__uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(q[k & 3u]), k >> 2));
+            n_added = base + k;
+            break;
+        }
+    }
+    return cum;
+}
+
+// The reference's `total` (src/gen/sampler.cpp:46-48) over n weights in the order q_at gives them.  All threads call,
+// all get it.
+template <typename Get>
+__device__ MAKO_RARE_CALL double reference_total(Get q_at, uint32_t n, FinishShared& sm)
+{
+    __syncthreads();
+    if (wave_id() == 0) {
+        uint32_t added;
+        const double t = wave_sequential_sum(q_at, n, (double)INFINITY, added);
+        if (lane_id() == 0)
+            sm.bs.f64[0] = t;
+    }
+    __syncthreads();
+    const double t = sm.bs.f64[0];
+    __syncthreads();
+    return t;
+}
+
 // Tail of every path that ends with a list sorted by (q desc, idx asc): kf[i] = ~bits(q_i), jf[i] = token id,
 // n1 entries (already cut to top_k).  Applies top-p (src/gen/sampler.cpp:44-61) against total64 (the fp64 sum over
 // the row's candidates; summed from the list when !have_total), then the exact fp32 total (:80-82) and walk
@@ -539,15 +603,22 @@ __device__ __forceinline__ ChainState sum_by_quarters(Keys kf, uint32_t st, uint
 // it weighs at most q_bound: the nucleus must then end inside the list, at an entry strictly heavier than
 // q_bound.  If it does not, nothing is written and false is returned (the caller widens the list).
 //
+// A cut that the sums here cannot tell from its neighbour with certainty (see order_band) is not made: nothing is
+// written and false is returned.  The caller then either widens (need_cut) or calls the EXACT instance with, as
+// total64, the reference's own total (reference_total() over the candidates in the reference's order): the cut is
+// then made by the reference's running sum, entry by entry.  EXACT on a whole list always succeeds.  (An instance of
+// its own, so that the usual one carries none of its code: sorted_tail_exact().)
+//
 // `T` (with `t_groups` records at `t_base`) describes a list whose groups were prepared by sort_kernel's workers;
 // without it the list is cut into groups of kGroup here.
 // SHORT_ONLY: the caller's lists never exceed kGroup entries; the code for longer ones is left out.
-template <bool PLANNED = false, bool SHORT_ONLY = false>
+template <bool PLANNED = false, bool SHORT_ONLY = false, bool EXACT = false>
 __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf_ptr,
                             const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
                             const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, const GroupTable& T = GroupTable{},
                             size_t t_base = 0, uint32_t t_groups = 0)
 {
+    constexpr bool exact = EXACT;
     using namespace seqfp;
     // (a planned row's list is in device memory; the other callers may hand over a list in LDS)
     const typename std::conditional<PLANNED, GlobalKeys, AnyKeys>::type kf{kf_ptr};
@@ -570,20 +641,39 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 total64 = block_sum_f64(part, sm.bs);
             }
             const double want = (double)P.top_p * total64;
-            double carry = 0;
             uint32_t keep = kNone;
-            for (uint32_t base = 0; base < n; base += kThreads) {
-                const uint32_t i = base + tid;
-                const double q = i < n ? (double)qat(i) : 0.0;
-                double tile;
-                const double incl = carry + block_incl_scan_f64(q, tile, sm.bs);
-                const uint32_t hit = (i < n && incl >= want) ? i : kNone;
-                const uint32_t first = block_min_u32(hit, sm.bs);
-                if (first != kNone) {
-                    keep = first + 1;
-                    break;
+            if (exact) {
+                if (wave_id() == 0) {
+                    uint32_t added;
+                    const double cum = wave_sequential_sum(qat, n, want, added);
+                    if (lane_id() == 0)
+                        sm.aux = cum >= want ? added : kNone;
                 }
-                carry += tile;
+                __syncthreads();
+                keep = sm.aux;
+            } else {
+                const double band = cut_band(have_total, d.n_vocab, n, qat, total64);
+                double carry = 0;
+                if (tid == 0)
+                    sm.aux = 0; // set: the cut is too close to `want` to call
+                for (uint32_t base = 0; base < n; base += kThreads) {
+                    const uint32_t i = base + tid;
+                    const double q = i < n ? (double)qat(i) : 0.0;
+                    double tile;
+                    const double incl = carry + block_incl_scan_f64(q, tile, sm.bs);
+                    const uint32_t hit = (i < n && incl >= want) ? i : kNone;
+                    const uint32_t first = block_min_u32(hit, sm.bs);
+                    if (first != kNone) {
+                        keep = first + 1;
+                        if (i == first && P.top_p > 0.0f && band != 0.0 && !(incl - want > band && want - (incl - q) > band))
+                            sm.aux = 1;
+                        break;
+                    }
+                    carry += tile;
+                }
+                __syncthreads();
+                if (sm.aux || keep == kNone) // (a list that never reaches `want`: the reference's sum might)
+                    return false;
             }
             if (need_cut && keep == kNone)
                 return false;
@@ -612,19 +702,34 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 total64 = readlane_f64(incl, kWave - 1);
             uint32_t n = n1;
             bool ok = true;
-            if (topp_active) {
+            if (topp_active && exact) {
                 const double want = (double)P.top_p * total64;
-                const double base = incl - p[3];
-                uint32_t hit = kNone;
-#pragma unroll
-                for (int j = 3; j >= 0; --j)
-                    if (base + p[j] >= want)
-                        hit = lane_id() * 4u + (uint32_t)j;
-                const unsigned long long bal = __ballot(hit != kNone && hit < n1);
-                if (bal)
-                    n = (uint32_t)__builtin_amdgcn_readlane((int)hit, __ffsll((long long)bal) - 1) + 1u;
+                uint32_t added;
+                const double cum = wave_sequential_sum(qat, n1, want, added);
+                if (cum >= want)
+                    n = max(added, 1u); // (sampler.cpp:58: never fewer than one)
                 else
                     ok = !need_cut;
+            } else if (topp_active) {
+                const double want = (double)P.top_p * total64;
+                const double band = cut_band(have_total, d.n_vocab, n1, qat, total64);
+                const double base = incl - p[3];
+                uint32_t hit = kNone;
+                bool clear = true; // both neighbours of the cut clear `want` by more than the band
+#pragma unroll
+                for (int j = 3; j >= 0; --j)
+                    if (base + p[j] >= want) {
+                        hit = lane_id() * 4u + (uint32_t)j;
+                        clear = !(P.top_p > 0.0f) || band == 0.0 || (base + p[j] - want > band && want - (j ? base + p[j - 1] : base) > band);
+                    }
+                const unsigned long long bal = __ballot(hit != kNone && hit < n1);
+                if (bal) {
+                    const int src = __ffsll((long long)bal) - 1;
+                    n = (uint32_t)__builtin_amdgcn_readlane((int)hit, src) + 1u;
+                    ok = __builtin_amdgcn_readlane((int)clear, src) != 0;
+                } else {
+                    ok = false; // (a list that never reaches `want`: the reference's sum might)
+                }
             }
             if (ok && need_cut && !(q_bound < qat(n - 1)))
                 ok = false;
@@ -751,11 +856,38 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     uint32_t n = n1, groups = uniform_u32(groups1);
     if (topp_active) {
         const double want = (double)P.top_p * total64;
-        const uint32_t hitg = (tid < groups1 && G.pg()[tid + 1] >= want) ? tid : kNone;
+        uint32_t hitg = (tid < groups1 && G.pg()[tid + 1] >= want) ? tid : kNone;
+        if (exact) {
+            // the reference's own running sum decides; the group it ends in follows from the entry
+            if (wave_id() == 0) {
+                uint32_t added;
+                const double cum = wave_sequential_sum(qat, n1, want, added);
+                if (lane_id() == 0)
+                    G.misc()[0] = cum >= want ? max(added, 1u) : kNone;
+            }
+            __syncthreads();
+            const uint32_t n_ref = G.misc()[0];
+            hitg = kNone;
+            if (n_ref != kNone && tid < groups1) {
+                const uint32_t st = G.start()[tid], len = G.pack()[tid] & kLenMask;
+                if (st < n_ref && n_ref <= st + len)
+                    hitg = tid;
+            }
+            __syncthreads();
+        }
         const uint32_t gs = block_min_u32(hitg, sm.bs);
-        if (need_cut && gs == kNone)
-            return false;
-        if (gs != kNone) {
+        if (gs == kNone && (need_cut || !exact))
+            return false; // (a list that never reaches `want`: a partial one is widened, a whole one decided exactly)
+        if (gs != kNone && exact) {
+            const uint32_t st = G.start()[gs], len = G.pack()[gs] & kLenMask, keep = G.misc()[0] - st;
+            __syncthreads();
+            if (tid == 0 && keep != len)
+                G.pack()[gs] = keep;
+            __syncthreads();
+            n = uniform_u32(G.misc()[0]);
+            groups = uniform_u32(gs + 1u);
+        } else if (gs != kNone) {
+            const double band = cut_band(have_total, d.n_vocab, n1, qat, total64);
             if (wave_id() == 0) {
                 const uint32_t st = G.start()[gs], len = G.pack()[gs] & kLenMask;
                 float q[4];
@@ -768,21 +900,30 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 const double incl = __ockl_wfscan_add_f64(p[3], true);
                 const double base = G.pg()[gs] + (incl - p[3]);
                 uint32_t hit = kNone;
+                bool clear = true; // both neighbours of the cut clear `want` by more than the band
 #pragma unroll
                 for (int j = 3; j >= 0; --j)
-                    if (base + p[j] >= want)
+                    if (base + p[j] >= want) {
                         hit = lane_id() * 4u + (uint32_t)j;
+                        clear = !(P.top_p > 0.0f) || band == 0.0 || (base + p[j] - want > band && want - (j ? base + p[j - 1] : base) > band);
+                    }
                 const unsigned long long bal = __ballot(hit != kNone && hit < len);
                 uint32_t keep = len;
-                if (bal)
-                    keep = (uint32_t)__builtin_amdgcn_readlane((int)hit, __ffsll((long long)bal) - 1) + 1u;
+                bool ok = false; // (no entry of the group reaches `want` although its sum does: too close to call)
+                if (bal) {
+                    const int src = __ffsll((long long)bal) - 1;
+                    keep = (uint32_t)__builtin_amdgcn_readlane((int)hit, src) + 1u;
+                    ok = __builtin_amdgcn_readlane((int)clear, src) != 0;
+                }
                 if (lane_id() == 0) {
-                    G.misc()[0] = st + keep;
-                    if (keep != len)
+                    G.misc()[0] = ok ? st + keep : kNone;
+                    if (ok && keep != len)
                         G.pack()[gs] = keep; // shortened: the prepared map no longer applies (exponent 0)
                 }
             }
             __syncthreads();
+            if (G.misc()[0] == kNone)
+                return false;
             n = uniform_u32(G.misc()[0]);
             groups = uniform_u32(gs + 1u);
         }
@@ -1083,6 +1224,16 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     MAKO_STAMP(9);
     emit(total, pos);
     return true;
+}
+
+// The EXACT instance, out of line where the source is compiled for it (see MAKO_RARE_CALL).
+template <bool PLANNED = false>
+__device__ MAKO_RARE_CALL void sorted_tail_exact(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P,
+                                                 const uint32_t* kf, const uint32_t* jf, uint32_t n1, double total64,
+                                                 uint32_t path, const FinishLds& L, const GroupTable& T = GroupTable{},
+                                                 size_t t_base = 0, uint32_t t_groups = 0)
+{
+    sorted_tail<PLANNED, false, true>(d, row, P, kf, jf, n1, true, total64, path, L, false, 0.0f, T, t_base, t_groups);
 }
 
 } // namespace mako

@@ -2,7 +2,7 @@
 #pragma once
 
 #include "sorted_tail.h"
-#include "plan_kernel.h"
+#include "late_rows.h"
 
 namespace mako {
 
@@ -12,9 +12,9 @@ namespace mako {
 // plan_kernel: 2.3 us less there, but this kernel's chains then compiled to slower code and lost twice that.)
 // (The context's record by value: with a pointer to it the first loads would have to wait for a trip to memory.  The
 // list's length and this workgroup's entry are asked for together, then everything the row's plan holds.)
-// Workgroups from tail_cap on: workgroup tail_cap + r finishes row r if it is a top-k row (finish_topk_row()), beside
-// the few long tails, on CUs that would otherwise idle.  (That code is kept out of line: inlined, it made this kernel's
-// chains compile to slower code.)
+// Workgroups from tail_cap on: workgroup tail_cap + r finishes what plan_kernel<false> and sort_kernel left of row r
+// (finish_late_row()), beside the few long tails, on CUs that would otherwise idle.  (That code is kept out of line:
+// inlined, it made this kernel's chains compile to slower code.)
 __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices,
                                                         uint32_t tail_cap)
 {
@@ -34,7 +34,7 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         Lr.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
         Lr.sortk = s_dyn64;
         Lr.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
-        finish_topk_row(s_args.d, s_args.sc, s_args.P, r, slices, Lr);
+        finish_late_row(s_args.d, s_args.sc, s_args.P, r, slices, Lr);
         return;
     }
     const uint32_t n_work = sc_arg.work_n[1];
@@ -63,8 +63,17 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     __syncthreads();
     if (tid == 0)
         plan->flag = 0;
-    sorted_tail<true>(d, row, s_args.P, sc.key[0] + (size_t)row * sc.vpad, sc.idx[0] + (size_t)row * sc.vpad, n0, true,
-                      total64, MAKO_PATH_GENERAL, L, false, 0.0f, sc.gt, (size_t)row * sc.g_cap, groups);
+    const uint32_t* kf = sc.key[0] + (size_t)row * sc.vpad;
+    const uint32_t* jf = sc.idx[0] + (size_t)row * sc.vpad;
+    if (sorted_tail<true>(d, row, s_args.P, kf, jf, n0, true, total64, MAKO_PATH_GENERAL, L, false, 0.0f, sc.gt,
+                          (size_t)row * sc.g_cap, groups))
+        return;
+    // too close to call: the reference's total, over the row's bits(q) array (index order; the zeros of the logits
+    // that are no candidates add nothing), decides (the list reaches far enough below the cut for it: plan_nucleus()
+    // takes the band along)
+    const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
+    const double total = reference_total([=](uint32_t i) { return __uint_as_float(qk[i]); }, d.n_vocab, sm);
+    sorted_tail_exact<true>(d, row, s_args.P, kf, jf, n0, total, MAKO_PATH_GENERAL, L, sc.gt, (size_t)row * sc.g_cap, groups);
 }
 #endif // MAKO_EMIT_TAIL_KERNEL
 

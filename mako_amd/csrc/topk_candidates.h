@@ -287,15 +287,15 @@ __device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t s
 // weight's neighbourhood ordered by (q desc, idx asc) in LDS, the certificate that nothing left behind in a slice can
 // reach the top_k-th weight, then top-p, total and draw by one wave.  A row that cannot be certified takes the
 // whole-row path: here and now (INLINE_GENERAL), or through sort_kernel's work list.
-template <bool INLINE_GENERAL>
+#ifndef MAKO_TOPK_GENERAL_SITE
+#define MAKO_TOPK_GENERAL_SITE 1 // (the general_row instance a top-k row falls back to: 0 where one exists anyway)
+#endif
 __device__ __forceinline__ void topk_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slices,
                                          const mako_sampling_params& P, float m, uint32_t argidx, uint32_t n_cands,
                                          const SliceStat& lane_stat, const FinishLds& L, bool have_pre = false,
                                          const CandSlots& pre = CandSlots{})
 {
-    constexpr bool inline_general = INLINE_GENERAL;
     FinishShared& sm = *L.sm;
-    const uint32_t tid = threadIdx.x;
     // ---- top-k rows: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
@@ -312,29 +312,18 @@ __device__ __forceinline__ void topk_row(const mako_sample_desc& d, const Scratc
                                    : sort_candidates<4>(sc, row, slices, n_cands, m, inv_t, floor_q, kf, jf, L);
     MAKO_STAMP(4);
     // top-k of the row = top-k of the candidates, provided nothing left behind can tie with or beat the k-th
-    const bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
-    if (!ok) {
-        if constexpr (inline_general) {
-            __syncthreads(); // (the lists in LDS are done with)
-            general_row<1>(d, sc, row, P, m, argidx, L);
-            return;
-        } else {
-            if (tid == 0) {
-                sc.plan[row].total64 = (double)m;
-                sc.plan[row].n0 = argidx;
-                sc.plan[row].flag = 2;
-                sc.work_sort[atomicAdd(&sc.work_n[0], 1u)] = row << 8;
-            }
-            return;
-        }
-    }
-    if (n_valid == 0) {
+    bool ok = n_valid >= P.top_k ? q_bound < __uint_as_float(~kf[P.top_k - 1]) : q_bound == 0.0f;
+    if (ok && n_valid == 0) {
         fallback_row(d, row, argidx);
         return;
     }
-    // (sampler.cpp:40-43; at most top_k <= kTopKFast <= kGroup entries)
+    // (sampler.cpp:40-43; at most top_k <= kTopKFast <= kGroup entries.  A top-p cut too close to call is left to the
+    // whole-row path, which can sum in the reference's order.)
     static_assert(kTopKFast <= kGroup, "top-k rows end in sorted_tail's short-list path");
-    sorted_tail<false, true>(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L);
+    if (ok && sorted_tail<false, true>(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L))
+        return;
+    __syncthreads(); // (the lists in LDS are done with)
+    general_row<MAKO_TOPK_GENERAL_SITE>(d, sc, row, P, m, argidx, L);
 }
 
 } // namespace mako

@@ -304,10 +304,44 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
     __syncthreads();
 }
 
+// key0 / idx0 <- the row's candidates in index order (~bits(q), token id), from its bits(q) array qb[0 .. V) (bits(q)
+// of every candidate at its index, 0 elsewhere), as general_row() first leaves them.  All threads call.  (Only for
+// the rare second look at a row: one entry per lane and round.)
+__device__ MAKO_RARE_CALL void compact_candidates(const uint32_t* qb, uint32_t V, uint32_t* key0, uint32_t* idx0, FinishShared& sm)
+{
+    const uint32_t lane = lane_id(), wave = wave_id();
+    const uint32_t chunk = (V + kWaves - 1u) / kWaves;
+    const uint32_t beg = min(V, wave * chunk), end = min(V, beg + chunk);
+    uint32_t mine = 0;
+    for (uint32_t i = beg + lane; i < end; i += kWave)
+        mine += qb[i] ? 1u : 0u;
+    mine = __ockl_wfred_add_u32(mine);
+    __syncthreads();
+    if (lane == 0)
+        sm.bs.u64[wave] = mine;
+    __syncthreads();
+    uint32_t at = 0;
+    for (uint32_t w = 0; w < wave; ++w)
+        at += (uint32_t)sm.bs.u64[w];
+    for (uint32_t base = beg; base < end; base += kWave) {
+        const uint32_t i = base + lane;
+        const uint32_t k = i < end ? qb[i] : 0u;
+        const unsigned long long bal = __ballot(k != 0u);
+        if (k) {
+            const uint32_t pos = at + (uint32_t)__popcll(bal & ((1ull << lane) - 1ull));
+            key0[pos] = ~k;
+            idx0[pos] = i;
+        }
+        at += (uint32_t)__popcll(bal);
+    }
+    __syncthreads();
+}
+
 // Common tail of the whole-row paths.  key[0]/idx[0] of the row hold n0 candidates (~bits(q), token id) in index
 // order.  Sorts them by (q desc, idx asc) when top-k or top-p is active, truncates (src/gen/sampler.cpp:39-61)
 // and draws.  `total64` (when have_total) is the fp64 sum of q over all candidates of the row, of which the list
-// may be only the heaviest part; otherwise it is summed from the list.
+// may be only the heaviest part; otherwise it is summed from the list.  The row's bits(q) array (sc.wbuf: bits(q) of
+// every candidate at its index, 0 elsewhere) must be in place.
 // (TOPK_ALONE = false leaves the top-k-without-top-p branch out of the instance inside plan_kernel<true>: that kernel is
 // only launched for batches whose host copy of the parameters shows a top-p on every sampled row, and the branch's
 // registers would be spilled around the top-k rows' fast path, +3.5 us on a 256-row batch.)
@@ -336,7 +370,22 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
     // (sorted_tail's one-wave path for lists of up to kGroup entries adds and walks them in the order given, whatever
     // it is, and without a top-p it cuts nothing: nth_element's survivors take it too)
     if (nth_order ? (!d.draft && n1 <= kGroup) : (topk_active || topp_active)) {
-        sorted_tail(d, row, P, ks, is, n1, have_total, total64, path, L);
+        if (sorted_tail(d, row, P, ks, is, n1, have_total, total64, path, L))
+            return;
+        // Too close to call (top-p rows only): the reference's total decides, summed in the order its candidates have
+        // at that point (sampler.cpp:40-48).
+        if (topk_active) {
+            // the order nth_element leaves the survivors in: from the candidates in index order again
+            compact_candidates(reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad), d.n_vocab, key0, idx0, sm);
+            nth_element_row(key0, idx0, n0, P.top_k, key1, idx1, L);
+            total64 = reference_total([=](uint32_t i) { return __uint_as_float(~key0[i]); }, n1, sm);
+            sort_segment(key0, idx0, key1, idx1, n1, L);
+        } else {
+            // index order: the row's bits(q) array (the zeros of the logits that are no candidates add nothing)
+            const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
+            total64 = reference_total([=](uint32_t i) { return __uint_as_float(qk[i]); }, d.n_vocab, sm);
+        }
+        sorted_tail_exact(d, row, P, ks, is, n1, total64, path, L);
         return;
     }
     // nth_element's order (long lists, verification), or neither top-k nor top-p: the candidates stay in index order
@@ -461,7 +510,7 @@ __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t*
 // (SITE: sort_kernel, its usual place, has an instance to itself, so that the compiler treats that kernel the same
 // whether or not the instances inside plan_kernel exist.)
 template <int SITE>
-__device__ void general_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
+__device__ MAKO_RARE_CALL void general_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
                             float m, uint32_t argidx, const FinishLds& L)
 {
     FinishShared& sm = *L.sm;

@@ -1,4 +1,7 @@
 """GPU parity tests: the HIP sampler, called through the C ABI, against the CPU oracle."""
+import os
+import sys
+
 import numpy as np
 import pytest
 
@@ -629,3 +632,32 @@ def test_host_call_argument_errors(gpu_ctx):
     assert call(mask_stride=v // 32 - 1) == api.MAKO_ERR_INVALID_ARG and "mask_stride" in gpu_ctx.last_error()
     assert call(hlen=(8, 9)) == api.MAKO_ERR_INVALID_ARG and "hist_len" in gpu_ctx.last_error()
     assert call() == api.MAKO_OK and np.array_equal(tok, good)
+
+
+def _topp_order_rows():
+    """The rows of tests/golden/topp_order_cases.json: on each the ORDER of the reference's fp64 additions decides the
+    nucleus (its sequential total and the exact total put top_p * total on different sides of a sorted prefix sum)."""
+    import json
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    import make_topp_order_cases as gen
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "topp_order_cases.json")) as f:
+        cases = json.load(f)["cases"]
+    logits = np.stack([gen.make_row(c["seed"], c["tiny_level"])[0] for c in cases])
+    p = api.make_params(len(cases), 1.0, 0, 0.9)
+    p["top_p"] = np.array([c["top_p_bits"] for c in cases], np.uint32).view(np.float32)
+    u = np.random.default_rng(77).random(len(cases)).astype(np.float32)
+    return dict(name="topp_order", logits=logits, params=p, u=u), cases
+
+
+def test_top_p_cut_follows_the_reference_addition_order(gpu_ctx):
+    """Twenty rows found by CPU brute force (tests/golden/make_topp_order_cases.py) whose nucleus has one entry more
+    or fewer depending on whether the fp64 total is added up one weight after the other in index order, as the
+    reference does (src/gen/sampler.cpp:46-48), or exactly: the device path must land on the reference's side."""
+    w, cases = _topp_order_rows()
+    g = assert_parity(gpu_ctx, w, cap=64)
+    assert [int(n) for n in g["n_cand"]] == [c["n_reference"] for c in cases]
+    assert all(c["n_reference"] != c["n_exact_total"] for c in cases)
+    # and as top-k + top-p rows over the same weights (top_k beyond the fast path: the whole-row path, where the
+    # reference's total runs over the top_k survivors in the order nth_element leaves them)
+    w["params"]["top_k"] = 60000
+    assert_parity(gpu_ctx, w, cap=64)

@@ -333,3 +333,32 @@ def test_host_code_under_sanitizers(name):
                     os.path.join(HERE, "cpu", name + ".cpp"), "-o", exe], check=True)
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0 and "0 failures" in out.stdout, out.stdout + out.stderr
+
+
+def test_topp_order_cases_fixture(oracle):
+    """tests/golden/topp_order_cases.json against the oracle: on these rows the nucleus size depends on the order of
+    the fp64 additions, and the oracle (sequential, like the reference) gives the recorded n_reference."""
+    import json
+    sys.path.insert(0, os.path.join(HERE, "golden"))
+    import make_topp_order_cases as gen
+    with open(os.path.join(HERE, "golden", "topp_order_cases.json")) as f:
+        cases = json.load(f)["cases"]
+    assert len(cases) >= 10
+    for c in cases[:6]:
+        logits, t = gen.make_row(c["seed"], c["tiny_level"])
+        top_p = float(np.array([c["top_p_bits"]], np.uint32).view(np.float32)[0])
+        _, tr = oracle.sample(logits, pyoracle.make_params(temperature=float(t), top_k=0, top_p=top_p), 0.5)
+        assert tr["n_cand"] == c["n_reference"] != c["n_exact_total"]
+
+
+def test_topp_order_cases_against_compiled_reference(reference):
+    """The same rows through the unmodified reference sampler (oracle/_ref): its nucleus sizes are the recorded ones."""
+    import json
+    import make_topp_order_cases as gen
+    with open(os.path.join(HERE, "golden", "topp_order_cases.json")) as f:
+        cases = json.load(f)["cases"]
+    for c in cases[:6]:
+        logits, t = gen.make_row(c["seed"], c["tiny_level"])
+        top_p = float(np.array([c["top_p_bits"]], np.uint32).view(np.float32)[0])
+        _, tr = reference.sample(logits, pyoracle.make_params(temperature=float(t), top_k=0, top_p=top_p), 1234, cap=0)
+        assert tr["n_cand"] == c["n_reference"]
