@@ -46,8 +46,18 @@ __device__ MAKO_RARE_CALL void finish_late_row(const mako_sample_desc& d, const 
     if (cls == kGreedy)
         return;
     if (cls == kNucleus) {
-        if (sc.plan[row].flag == 4) // (never set for a row whose token is forced: plan_kernel returns before planning)
+        // (the flag is never set for a row whose token is forced: plan_kernel returns before planning)
+        const uint32_t flag = sc.plan[row].flag;
+        if (flag == 4) {
             narrow_second_look(d, sc, P, row, L);
+        } else if (flag == 2) { // a nucleus too long for the workers' group records: the whole-row path
+            const float m = (float)sc.plan[row].total64;
+            const uint32_t argidx = sc.plan[row].n0;
+            __syncthreads();
+            if (threadIdx.x == 0)
+                sc.plan[row].flag = 0;
+            general_row<0>(d, sc, row, P, m, argidx, L);
+        }
         return;
     }
     if (d.force_token || d.close_token) { // uniform

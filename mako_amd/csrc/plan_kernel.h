@@ -138,14 +138,17 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         sc.plan[row].thr = thr_bits;
         sc.plan[row].flag = !fits ? 2 : (narrow ? 3 : 1);
     }
-    // the row's pieces of work for sort_kernel (all workers, or worker 0 alone) and tail_kernel
-    const uint32_t work = (fits && !narrow) ? kWorkers : 1u;
+    // the row's pieces of work for sort_kernel (all workers, or worker 0 alone) and tail_kernel; a row for the
+    // whole-row path is finished in tail_kernel's launch from its flag alone (finish_late_row())
+    if (!fits)
+        return;
+    const uint32_t work = !narrow ? kWorkers : 1u;
     if (tid == 0)
         sm.flag = atomicAdd(&sc.work_n[0], work);
     __syncthreads();
     if (tid < work)
         sc.work_sort[sm.flag + tid] = (row << 8) | tid;
-    if (tid == 0 && fits && !narrow)
+    if (tid == 0 && !narrow)
         sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
 }
 

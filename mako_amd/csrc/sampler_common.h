@@ -76,8 +76,9 @@ constexpr uint32_t kSortedCopyAt = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 
 // Work order for a top_k == 0 row whose nucleus is too wide for the per-slice candidate lists: the weights
 // with bits(q) >= key_lo (n0 of them) are split by value into kWorkers contiguous ranges of about equal size.
 struct BigPlan {
-    uint32_t flag;   // 1: the row waits for sort_kernel's workers; 2: for its whole-row path (worker 0 alone);
-                     // 3: a narrow nucleus, finished by worker 0 from the candidate lists
+    uint32_t flag;   // 1: the row waits for sort_kernel's workers and tail_kernel; 2: for the whole-row path (in
+                     // tail_kernel's launch); 3: a narrow nucleus, finished by worker 0 from the candidate lists;
+                     // 4: one that the lists could not certify (second look in tail_kernel's launch)
     uint32_t n0;     // entries to sort
     uint32_t pad0;
     uint32_t groups; // groups of the whole list: each worker's range is cut into groups of kGroup on its own

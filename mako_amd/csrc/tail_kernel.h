@@ -26,6 +26,7 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         const uint32_t r = blockIdx.y - tail_cap;
         if (r >= d_arg.n_rows)
             return;
+        MAKO_ROW(kNone);
         if (threadIdx.x < 32)
             sm.tab[threadIdx.x] = k_exp2_tab[threadIdx.x];
         stage_args(d_arg, sc_arg, r, s_args); // (its barrier publishes the table too)

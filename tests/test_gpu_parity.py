@@ -661,3 +661,20 @@ def test_top_p_cut_follows_the_reference_addition_order(gpu_ctx):
     # reference's total runs over the top_k survivors in the order nth_element leaves them)
     w["params"]["top_k"] = 60000
     assert_parity(gpu_ctx, w, cap=64)
+
+
+def test_nucleus_longer_than_the_group_records():
+    """A top-p row whose nucleus has more entries than the workers' group records hold (256 x 992): it takes the
+    whole-row path, in the last launch."""
+    v = 300000
+    rng = np.random.default_rng(4242)
+    logits = (rng.standard_normal((2, v)) * 0.05).astype(np.float32)
+    p = api.make_params(2, 1.0, 0, 0.99)
+    w = dict(name="long_nucleus", logits=logits, params=p, u=np.array([0.3, 0.97], np.float32))
+    ctx = api.SamplerContext(max_rows=2, max_vocab=v, max_hist=0)
+    try:
+        g = assert_parity(ctx, w, cap=256)
+        assert (g["n_cand"] > 256 * 992).all()
+        assert (g["path"] == 5).all()  # MAKO_PATH_GENERAL
+    finally:
+        ctx.close()
