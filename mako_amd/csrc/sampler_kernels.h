@@ -6,12 +6,15 @@
 //                     logits (a superset of what top-k can need) go to scratch.
 //   finish_kernel     the second, cache-resident pass over top_k == 0 rows: exact sums and the histogram of
 //                     q = expf((w - m) / T).
-//   plan_kernel       greedy and forced rows; top-k rows from the candidate lists, ordered by (q desc, idx asc) and
-//                     drawn from with the reference's exact fp32 rounding order; the plan of every top_k == 0 row.
-//   partition_kernel, sort_kernel, tail_kernel
-//                     the wide nuclei: weights handed to 32 workers per row, sorted, cut and drawn from.
-//   Whatever the candidate lists cannot certify falls to a whole-row path that is exact for every parameter
-//   combination.
+//   plan_kernel       greedy and forced rows; the plan of every top_k == 0 row; in a batch that ends here
+//                     (no top_k == 0 and no whole-row rows) also the top-k rows, from the candidate lists, ordered
+//                     by (q desc, idx asc) and drawn from with the reference's exact fp32 rounding order.
+//   partition_kernel, sort_kernel
+//                     the wide nuclei: weights handed to 32 workers per row and sorted; narrow nuclei from the
+//                     candidate lists.
+//   tail_kernel       the wide nuclei cut and drawn from; in the same launch, one workgroup per row, whatever the
+//                     earlier kernels left: top-k rows, rows on the whole-row path (exact for every parameter
+//                     combination), second looks at cuts too close to call.
 #pragma once
 
 #include "tuning_stamps.h"
