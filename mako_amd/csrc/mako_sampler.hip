@@ -372,7 +372,8 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     const uint32_t slice_len = slice_len_for(d.n_vocab, slices);
     const bool vec = d.n_vocab % 4 == 0 && d.logits_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(d.logits) & 15u) == 0;
     const size_t lds = d.hist_tokens ? (size_t)slice_len * sizeof(uint32_t) : 0;
-    const dim3 grid(slices, d.n_rows);
+    // (scan_kernel: with histories a row's slices share an XCD)
+    const dim3 grid = d.hist_tokens ? dim3((d.n_rows + 7u) & ~7u, slices) : dim3(slices, d.n_rows);
     // The second pass cuts top_k == 0 rows into pieces of one to four blocks of 4096 logits (decided on the device:
     // pieces finer than slices only while all of them fit one round of workgroups), so this many workgroups can
     // have work; the others leave after a look at the rows' parameters.

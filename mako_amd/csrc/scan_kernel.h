@@ -33,7 +33,6 @@ __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
     return prefix;
 }
 
-// grid = (slices, rows).
 // (ABOVE: the batch has close tokens, whose logits' ranks are counted on the way; a variant of its own because the
 // count takes sixteen more registers, up to the limit for two workgroups per CU, which no other batch should pay)
 template <bool VEC, int KH, bool ABOVE = false>
@@ -42,7 +41,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
 {
     // (scan_kernel takes the context's record by value: its first loads then need no trip to memory for a pointer)
     const Scratch& sc = sc_arg;
-    MAKO_ROW(blockIdx.y);
+    MAKO_ROW(d.hist_tokens ? blockIdx.x : blockIdx.y);
 #ifdef MAKO_TIMING_SCAN
     MAKO_WG_TIMER;
 #endif
@@ -50,7 +49,15 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
     extern __shared__ __align__(16) uint32_t s_dyn[]; // [slice_len] token counts when the row has penalties
     __shared__ ScanShared sm;
 
-    const uint32_t row = blockIdx.y, slice = blockIdx.x, tid = threadIdx.x;
+    // grid = (slices, rows), or, for a batch with histories, (rows rounded up to a multiple of 8, slices):
+    // workgroups go to the eight XCDs in turn, so with the row in x all slices of a row run on one XCD and its L2
+    // fetches the row's history from memory once, not eight times (-10 % of the kernel's fetches on a decode batch
+    // with 2048-token histories).  Without histories the first form is 2-4 % faster on batches of 256 rows.
+    const bool row_in_x = d.hist_tokens != nullptr; // uniform
+    const uint32_t row = row_in_x ? blockIdx.x : blockIdx.y, slice = row_in_x ? blockIdx.y : blockIdx.x, tid = threadIdx.x;
+    const uint32_t n_slices = row_in_x ? gridDim.y : gridDim.x;
+    if (row >= d.n_rows)
+        return;
     MAKO_STAMP(28);
     const uint32_t lo = slice * slice_len;
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
@@ -72,7 +79,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
     }
     if (row == 0 && slice == 0 && wave_id() == 1) { // how the second pass will be cut up
         uint32_t piece_len, busy;
-        const uint32_t pieces = second_pass_pieces(d, gridDim.x, slice_len, cus, piece_len, busy);
+        const uint32_t pieces = second_pass_pieces(d, n_slices, slice_len, cus, piece_len, busy);
         if (lane_id() == 0)
             *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(pieces, piece_len, busy, 0u);
     }
