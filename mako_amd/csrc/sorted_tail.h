@@ -776,31 +776,48 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         G.misc()[3] = 0;
     // The head of the list as floats in LDS (loads set out now, wanted after the cut): where the running sum and
     // the walk change binade every few entries, both go through it entry by entry.
-    constexpr uint32_t kHead = kWalkSeqGroups * kGroup;
-    {
-        uint32_t raw[kHead / kThreads];
+    constexpr uint32_t kHeadGroups = kWalkSeqGroups;
+    constexpr uint32_t kHead = kHeadGroups * kGroup;
+    float* const head = G.head();
+    uint32_t raw[kHead / kThreads];
 #pragma unroll
-        for (uint32_t t = 0; t < kHead / kThreads; ++t)
-            raw[t] = kf[min(t * kThreads + tid, n1 - 1u)];
-#pragma unroll
-        for (uint32_t t = 0; t < kHead / kThreads; ++t)
-            G.head()[t * kThreads + tid] = __uint_as_float(~raw[t] & (t * kThreads + tid < n1 ? 0xffffffffu : 0u));
-        if (tid < kWave)
-            G.head()[kHead + tid] = 0.0f;
-    }
-    __syncthreads();
+    for (uint32_t t = 0; t < kHead / kThreads; ++t)
+        raw[t] = kf[min(t * kThreads + tid, n1 - 1u)];
+    // (a planned list's group records are asked for in the same trip to memory: nothing below waits for the head's
+    // loads before these are out)
+    double r_sum = 0.0;
+    uint32_t r_d0 = 0, r_d1 = 0, r_cm = 0, r_st = 0, r_pk = 0;
+    uint4 qr0 = make_uint4(0, 0, 0, 0), qr1 = qr0, qr2 = qr0, qr3 = qr0;
     if constexpr (PLANNED) {
         if (tid < groups1) {
-            G.pg()[tid + 1] = T.sum[t_base + tid];
-            G.d0()[tid] = T.d0[t_base + tid];
-            G.d1()[tid] = T.d1[t_base + tid];
-            G.cmax()[tid] = T.cmax[t_base + tid];
-            // (clamped into the list: a record is only ever read, never trusted for addressing)
-            const uint32_t st = min(T.start[t_base + tid], n1), pk = T.pack[t_base + tid];
+            r_sum = T.sum[t_base + tid];
+            r_d0 = T.d0[t_base + tid];
+            r_d1 = T.d1[t_base + tid];
+            r_cm = T.cmax[t_base + tid];
+            r_st = T.start[t_base + tid];
+            r_pk = T.pack[t_base + tid];
             // (the quarter records are asked for together with the rest, whether or not the group has any: asking
             // only once `pk` is known would be one more trip to memory for every row)
             const uint4* tq = T.quarters + (t_base + tid) * 4u;
-            const uint4 qr0 = tq[0], qr1 = tq[1], qr2 = tq[2], qr3 = tq[3];
+            qr0 = tq[0], qr1 = tq[1], qr2 = tq[2], qr3 = tq[3];
+        }
+        lds_barrier(); // (misc[3] is published; the loads stay in flight)
+    } else {
+        __syncthreads();
+    }
+#pragma unroll
+    for (uint32_t t = 0; t < kHead / kThreads; ++t)
+        head[t * kThreads + tid] = __uint_as_float(~raw[t] & (t * kThreads + tid < n1 ? 0xffffffffu : 0u));
+    if (tid < kWave)
+        head[kHead + tid] = 0.0f;
+    if constexpr (PLANNED) {
+        if (tid < groups1) {
+            G.pg()[tid + 1] = r_sum;
+            G.d0()[tid] = r_d0;
+            G.d1()[tid] = r_d1;
+            G.cmax()[tid] = r_cm;
+            // (clamped into the list: a record is only ever read, never trusted for addressing)
+            const uint32_t st = min(r_st, n1), pk = r_pk;
             uint32_t slot = 0;
             if (pk & kHasQuarters) {
                 slot = atomicAdd(&G.misc()[3], 1u) + 1u;
@@ -961,7 +978,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         // A nucleus this short is copied to LDS and gone through entry by entry, once for the total and once for the
         // walk (three nanoseconds an entry each way): the group maps below only pay on longer lists.
         if (wave_id() == 0) {
-            const float S = sum_lds(G.head(), n, 0.0f);
+            const float S = sum_lds(head, n, 0.0f);
             const float span = S - 0.0f;
             const float prod = u_row * span;
             const float r0 = prod + 0.0f;
@@ -970,7 +987,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 at = 0;
             } else if (r0 == r0 && r0 != INFINITY) {
                 float r = r0;
-                walk_lds(G.head(), n, r, at);
+                walk_lds(head, n, r, at);
             }
             if (lane_id() == 0) {
                 G.misc()[1] = __float_as_uint(S);
@@ -1010,7 +1027,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 #endif
     // A walk that will end within a few groups goes through them entry by entry, from a copy in LDS: faster than
     // the groups' maps would be to build.
-    const bool head_walk = reach <= kWalkSeqGroups; // uniform
+    const bool head_walk = reach <= kHeadGroups; // uniform
     const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
     if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && !head_walk) {
         // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
@@ -1040,7 +1057,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             first = bal ? 64u - (uint32_t)__clzll((long long)bal) : 0u;
             if (first) {
                 const uint32_t hs = first == groups ? n : uniform_u32(G.start()[min(first, groups - 1u)]);
-                const float S = sum_lds(G.head(), min(hs, kHead), 0.0f);
+                const float S = sum_lds(head, min(hs, kHead), 0.0f);
                 uint32_t Mv;
                 int ev;
                 split(S, Mv, ev);
@@ -1129,7 +1146,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             uint32_t first = 0; // groups already walked
             if (head_walk && head_n) {
                 float r = r0;
-                stopped = walk_lds(G.head(), head_n, r, at);
+                stopped = walk_lds(head, head_n, r, at);
                 uint32_t Mv;
                 int ev;
                 split(r, Mv, ev);

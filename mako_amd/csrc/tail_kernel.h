@@ -22,10 +22,14 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
+#ifdef MAKO_TIMING_TAIL
+    MAKO_WG_TIMER;
+#endif
     if (blockIdx.y >= tail_cap) {
         const uint32_t r = blockIdx.y - tail_cap;
         if (r >= d_arg.n_rows)
             return;
+        MAKO_ROW(kNone);
         MAKO_ROW(kNone);
         if (threadIdx.x < 32)
             sm.tab[threadIdx.x] = k_exp2_tab[threadIdx.x];
@@ -42,9 +46,6 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     const uint32_t row = sc_arg.work_tail[blockIdx.y], tid = threadIdx.x; // (the list has room for every workgroup)
     if (blockIdx.y >= n_work)
         return;
-#ifdef MAKO_TIMING_TAIL
-    MAKO_WG_TIMER;
-#endif
     MAKO_ROW(row);
     const BigPlan* planned = sc_arg.plan + row;
     const uint32_t flag = planned->flag, plan_n0 = planned->n0, plan_groups = planned->groups;
