@@ -216,12 +216,68 @@ __device__ void build_quarters(const float (&q)[4], uint32_t len, double at_star
         out[quarter] = make_uint4(v.d0, v.d1, cm, (uint32_t)eg);
 }
 
-// Group maps of groups [0, groups) for epochs guessed from pg: of the running sum (walk == false, into G.d0 / d1 /
-// cmax / pack) or of the walk from r0 (into G.w_d0 / w_d1 / w_need / w_pack).  The calling wave is number `part` of
-// `parts` that share the work.
+// The same for the walk: a group inside which r is expected to change binade gets a record per quarter, each for
+// the binade guessed from r at the group's first entry minus the fp64 sum up to ITS first entry: (d0, d1, need,
+// exponent), `need` being the bound of group_sub_ok as one number (the state after the quarter must be at least the
+// quarter's first, largest weight, and inside the binade with room for one more decrement).  One wave.
+__device__ void build_walk_quarters(const float (&q)[4], uint32_t len, double r_start, uint4* out)
+{
+    using namespace seqfp;
+    const uint32_t lane = lane_id(), quarter = lane >> 4;
+    double rs = (((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3];
+    for (int o = 1; o < 16; o <<= 1)
+        rs += __shfl_xor(rs, o);
+    const double s0 = __shfl(rs, 0), s1 = __shfl(rs, 16), s2 = __shfl(rs, 32);
+    const double before = quarter == 0 ? 0.0 : (quarter == 1 ? s0 : (quarter == 2 ? s0 + s1 : (s0 + s1) + s2));
+    const double guess = r_start - before;
+    const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+    Step32 v = Step32{kSat, kSat, kSat};
+    if (eg > 0) {
+        v = identity32();
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (lane * 4u + j < len)
+                v = compose32(v, step32(q[j], eg));
+    }
+    uint32_t cm = v.cmax;
+    for (int o = 1; o < 16; o <<= 1)
+        cm = max(cm, (uint32_t)__shfl_xor((int)cm, o));
+#define MAKO_ROW_STEP(CTRL)                                                                                          \
+    {                                                                                                                \
+        const Step32 t = Step32{dpp_or_zero<CTRL, 0xf>(v.d0), dpp_or_zero<CTRL, 0xf>(v.d1), 0u};                     \
+        const Step32 r = compose32(t, Step32{v.d0, v.d1, 0u});                                                       \
+        v.d0 = r.d0;                                                                                                 \
+        v.d1 = r.d1;                                                                                                 \
+    }
+    MAKO_ROW_STEP(0x111)
+    MAKO_ROW_STEP(0x112)
+    MAKO_ROW_STEP(0x114)
+    MAKO_ROW_STEP(0x118)
+#undef MAKO_ROW_STEP
+    const float q_first = __shfl(q[0], (int)(quarter * 16u)); // the quarter's first, largest weight
+    uint32_t Mq;
+    int eq;
+    split(q_first, Mq, eq);
+    const int dl = eg - eq;
+    uint32_t need = 1u;
+    if (dl < 0)
+        need = 1u << 31;
+    else if (dl <= 25)
+        need = max(1u, (uint32_t)(((unsigned long long)Mq + (1ull << dl) - 1ull) >> dl));
+    if (eg > 1)
+        need = max(need, min(cm, 1u << 30) + (1u << 23) + 1u);
+    if (eg <= 0)
+        need = 1u << 31; // (no usable guess: the quarter is replayed)
+    if ((lane & 15u) == 15u)
+        out[quarter] = make_uint4(v.d0, v.d1, need, (uint32_t)eg);
+}
+
+// Group maps of groups [g_begin, groups) for epochs guessed from pg: of the running sum (walk == false, into G.d0 /
+// d1 / cmax / pack) or of the walk (into G.w_d0 / w_d1 / w_need / w_pack; r0 - pg[g] is the estimate of r at group
+// g).  The calling wave is number `part` of `parts` that share the work.
 template <typename Keys>
 __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0, const GroupLds G,
-                                 uint32_t part = wave_id(), uint32_t parts = kWaves)
+                                 uint32_t part = wave_id(), uint32_t parts = kWaves, uint32_t g_begin = 0)
 {
     using namespace seqfp;
     uint32_t* const o_d0 = walk ? G.w_d0() : G.d0();
@@ -230,7 +286,7 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
     uint32_t* const o_pack = walk ? G.w_pack() : G.pack();
     // Up to four groups per trip and wave, their loads issued together; a wave's groups lie `parts` apart, so that a
     // short list is spread over all the waves (a map costs a wave about a microsecond).
-    for (uint32_t g0 = part; g0 < groups; g0 += parts * 4u) {
+    for (uint32_t g0 = g_begin + part; g0 < groups; g0 += parts * 4u) {
         float q[4][4];
         uint32_t len[4];
 #pragma unroll
@@ -247,18 +303,20 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
             const double guess = g < groups ? (walk ? r0 - G.pg()[g] : G.pg()[g]) : 0.0;
             const int eg = guess > 0 ? exponent_of((float)guess) : 0;
             const Step32 st = span_map(q[u], len[u], eg);
-            // a group in which the running sum is expected to change binade (or starts from zero) gets quarter
-            // records; the walk replays such groups whole
+            // a group in which the running sum (or r) is expected to change binade, or which starts from zero, gets
+            // quarter records
             uint32_t slot = 0;
-            if (!walk && g < groups) { // uniform
-                const double at_end = G.pg()[g + 1];
+            if (g < groups) { // uniform
+                const double at_end = walk ? r0 - G.pg()[g + 1] : G.pg()[g + 1];
                 const int e_end = at_end > 0 ? exponent_of((float)at_end) : 0;
-                if (uniform_u32((uint32_t)(e_end != eg)) || g == 0) {
+                if (uniform_u32((uint32_t)(e_end != eg)) || (!walk && g == 0)) {
                     if (lane_id() == 0)
                         slot = atomicAdd(&G.misc()[3], 1u) + 1u;
                     slot = uniform_u32(slot);
                     if (slot > kQuarterSlots)
                         slot = 0;
+                    else if (walk)
+                        build_walk_quarters(q[u], len[u], guess, G.quarters() + (slot - 1u) * 4u);
                     else
                         build_quarters(q[u], len[u], G.pg()[g], G.quarters() + (slot - 1u) * 4u);
                 }
@@ -528,6 +586,67 @@ __device__ __forceinline__ ChainState sum_by_quarters(Keys kf, uint32_t st, uint
         }
     }
     return c;
+}
+
+// One block of at most 64 entries (x of lane l = entry l of the block, 0.0f past its end; the block starts at entry
+// `beg` of the list) subtracted from r one by one.  Returns true and the position when the walk stops inside the
+// block, else false and the new r.  One wave.  (walk_lanes() for a single block.)
+__device__ __forceinline__ bool walk_block(float cur, uint32_t n, uint32_t beg, float& r, uint32_t& pos)
+{
+    float v = r;
+    float r_in = r;
+    for (uint32_t b = 0; b < kWave && b < n; b += 16u) {
+#pragma unroll
+        for (uint32_t k = 0; k < 16; ++k)
+            v = ror_sub(v, cur);
+        const uint32_t o16 = (uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(v), (b + 15u) & 63u);
+        if (o16 >> 31) {
+            float rr = r_in;
+            for (uint32_t l = b; l < b + 16u; ++l) {
+                const float xv = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(cur), l & 63u));
+                if (__ballot(rr < xv) != 0ull) {
+                    pos = beg + l;
+                    return true;
+                }
+                rr -= xv;
+            }
+        }
+        r_in = __uint_as_float(o16);
+    }
+    r = r_in;
+    return false;
+}
+
+// One group of the walk quarter by quarter (records at `rec`, see build_walk_quarters(); the group's entries in x as
+// load_span_lanes() leaves them: x[k] of lane l is entry l of quarter k), replaying only the quarters whose map
+// does not apply.  Returns true (and c.pos) when the walk stops inside the group.  One wave.
+__device__ __forceinline__ bool walk_by_quarters(const float (&x)[4], uint32_t st, uint32_t len, const uint4* rec, ChainState& c)
+{
+    using namespace seqfp;
+#pragma unroll
+    for (uint32_t k = 0; k < 4u; ++k) {
+        if (k * kQuarter < len) { // uniform
+            const uint4 r = rec[k];
+            const uint32_t d0 = uniform_u32(r.x), d1 = uniform_u32(r.y), need = uniform_u32(r.z), eg = uniform_u32(r.w);
+            const uint32_t dd = (c.M & 1u) ? d1 : d0;
+            if ((uint32_t)c.e == eg && dd <= c.M && c.M - dd >= need) {
+                c.M -= dd;
+            } else {
+                float rr = join(c.M, c.e);
+                uint32_t at = 0;
+                if (walk_block(x[k], min(kQuarter, len - k * kQuarter), st + k * kQuarter, rr, at)) {
+                    c.pos = at;
+                    return true;
+                }
+                uint32_t Mv;
+                int ev;
+                split(rr, Mv, ev);
+                c.M = uniform_u32(Mv);
+                c.e = (int)uniform_u32((uint32_t)ev);
+            }
+        }
+    }
+    return false;
 }
 
 // The band for a top-p cut in a sorted list of n weights q_at(0 .. n).  When total64 is the sum of
@@ -1031,7 +1150,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
     if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && !head_walk) {
         // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
-        build_group_maps(kf, reach, true, r0_guess, G, (uint32_t)(wave_id() >> 2) * 3u + (uint32_t)(wave_id() & 3) - 1u,
+        build_group_maps(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)(wave_id() >> 2) * 3u + (uint32_t)(wave_id() & 3) - 1u,
                          3u * kWaves / 4u);
 #ifdef MAKO_TIMING
         if (tid == 64 && s_mako_row == 0)
@@ -1131,9 +1250,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         pos = 0;
     } else if (r0 == r0 && r0 != INFINITY) {
         MAKO_STAMP(14);
+        // The state of the walk (wave 0's, in scalar registers; between blocks of 64 groups in LDS).
+        uint32_t M = 0;
+        int e = 1;
+        uint32_t at = n - 1;
+        bool stopped = false;
+        uint32_t first = 0; // groups already walked
         if (wave_id() == 0) {
-            uint32_t M;
-            int e;
             {
                 uint32_t Mv;
                 int ev;
@@ -1141,9 +1264,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 M = uniform_u32(Mv);
                 e = (int)uniform_u32((uint32_t)ev);
             }
-            uint32_t at = n - 1;
-            bool stopped = false;
-            uint32_t first = 0; // groups already walked
             if (head_walk && head_n) {
                 float r = r0;
                 stopped = walk_lds(head, head_n, r, at);
@@ -1154,7 +1274,30 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 e = (int)uniform_u32((uint32_t)ev);
                 first = reach;
             }
-            for (uint32_t base = 0; base < groups && !stopped; base += kWave) {
+        }
+        // The groups are walked 64 at a time.  The first block's maps were built beside the running sum, for the
+        // binades guessed from u * (fp64 total); deep into a list r is a small difference of large numbers and
+        // that guess is worthless (every group would then go entry by entry: 140 us for a 245-group list at
+        // u = 0.999), so every later block's maps are built, by all the waves, when the walk gets there, from the
+        // exact r at the block's first group.
+        for (uint32_t base = 0; base < groups; base += kWave) {
+            if (base > 0) {
+                if (wave_id() == 0 && lane_id() == 0) {
+                    G.misc()[0] = M;
+                    G.misc()[1] = (uint32_t)e;
+                    sm.aux = stopped ? 1u : 0u;
+                }
+                __syncthreads();
+                if (sm.aux) // uniform
+                    break;
+                const double r_here = (double)join(G.misc()[0], (int)G.misc()[1]);
+                if (tid == 0)
+                    G.misc()[3] = 0; // (the quarter records so far are done with: their slots start over)
+                __syncthreads();
+                build_group_maps(kf, min(groups, base + (uint32_t)kWave), true, r_here + G.pg()[base], G, wave_id(), kWaves, base);
+                __syncthreads();
+            }
+            if (wave_id() == 0 && !stopped) {
                 const uint32_t gl = min(base + lane_id(), groups - 1u);
                 const uint32_t pk_l = G.w_pack()[gl], st_l = G.start()[gl];
                 const uint32_t d0_l = G.w_d0()[gl], d1_l = G.w_d1()[gl], need_l = G.w_need()[gl]; // (the bound, see build_group_maps)
@@ -1213,16 +1356,28 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         } else {
                             MAKO_COUNT(22, 1);
                             passed = 0;
-                            float r = join(M, e);
-                            if ((pk & kLenMask) && walk_lanes(xa, pk & kLenMask, st, r, at)) {
-                                stopped = true;
-                                break;
+                            const uint32_t slot = (pk >> 9) & 0x7fu;
+                            if (slot && (pk & kLenMask)) {
+                                ChainState c{M, e, kNone};
+                                if (walk_by_quarters(xa, st, pk & kLenMask, G.quarters() + (slot - 1u) * 4u, c)) {
+                                    at = c.pos;
+                                    stopped = true;
+                                    break;
+                                }
+                                M = c.M;
+                                e = c.e;
+                            } else {
+                                float r = join(M, e);
+                                if ((pk & kLenMask) && walk_lanes(xa, pk & kLenMask, st, r, at)) {
+                                    stopped = true;
+                                    break;
+                                }
+                                uint32_t Mv;
+                                int ev;
+                                split(r, Mv, ev);
+                                M = uniform_u32(Mv);
+                                e = (int)uniform_u32((uint32_t)ev);
                             }
-                            uint32_t Mv;
-                            int ev;
-                            split(r, Mv, ev);
-                            M = uniform_u32(Mv);
-                            e = (int)uniform_u32((uint32_t)ev);
                         }
                         ++g;
                     }
@@ -1231,9 +1386,9 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     done = g;
                 }
             }
-            if (lane_id() == 0)
-                G.misc()[2] = at;
         }
+        if (wave_id() == 0 && lane_id() == 0)
+            G.misc()[2] = at;
         __syncthreads();
         pos = G.misc()[2];
     }

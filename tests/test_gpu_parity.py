@@ -443,6 +443,16 @@ def test_wide_nucleus_walk_depths(gpu_ctx):
     assert g["n_cand"].min() > 5000
 
 
+@pytest.mark.parametrize("u", [0.9, 0.999, 1.0 - 2.0**-24])
+def test_config3_deep_walks(gpu_ctx, u):
+    """The decode batch drawn at one large u on every row: on its peaked wide rows (a few spikes, then tens of
+    thousands of small weights) the walk runs through several blocks of 64 groups, whose maps are rebuilt from the
+    exact r at each block's start, and r falls through many binades."""
+    w = workloads.config3()
+    w["u"] = np.full(64, u, np.float32)
+    assert_parity(gpu_ctx, w, cap=64)
+
+
 def test_tied_wide_nucleus(gpu_ctx):
     """Logits on a grid of 1/8: every weight is shared by hundreds of tokens, so candidates tie in q and the order
     inside a tie is by token id.  The workers' counting sort gives such rows to the stable radix sort."""
