@@ -168,28 +168,35 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
         }
         // w >= tau and w > -inf in one compare: -inf itself is below the most negative finite float
         const float tau = fmaxf(order_unkey(tau_key), -3.402823466e38f);
-        // slots in the slice's list: the wave counts its candidates, one lane reserves the wave's run with a single
-        // LDS atomic, and every thread fills its part of the run (one atomic per candidate cost a round trip each)
-        uint32_t mine = 0;
+        // Slots in the slice's list.  Candidates are few (a percent or three of the logits): for each of the sixteen
+        // positions j a ballot says which lanes hold one, the counts add up in scalar registers, one lane reserves
+        // the wave's run with a single LDS atomic, and only the positions with a candidate in some lane cost vector
+        // instructions at all (a lane's slot: the run's start, the candidates of earlier positions, and the set
+        // bits below the lane).  The order inside the list is by position, then lane; nobody depends on it.
+        unsigned long long takes[16];
+        uint32_t wave_total = 0;
 #pragma unroll
-        for (uint32_t j = 0; j < 16; ++j)
-            mine += wv[j] >= tau ? 1u : 0u;
-        const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
-        const uint32_t wave_total = (uint32_t)__builtin_amdgcn_readlane((int)upto, kWave - 1);
+        for (uint32_t j = 0; j < 16; ++j) {
+            takes[j] = __ballot(wv[j] >= tau);
+            wave_total += (uint32_t)__popcll(takes[j]);
+        }
         if (wave_total) { // uniform
             uint32_t base = 0;
             if (lane_id() == 0)
                 base = atomicAdd(&sm.emit_n, wave_total);
-            uint32_t pos = (uint32_t)__builtin_amdgcn_readfirstlane((int)base) + upto - mine;
+            uint32_t run = (uint32_t)__builtin_amdgcn_readfirstlane((int)base);
 #pragma unroll
             for (uint32_t j = 0; j < 16; ++j) {
-                const float w = wv[j];
-                const bool take = w >= tau;
-                if (take && pos < kCap) {
-                    sm.cw[pos] = w;
-                    sm.ci[pos] = elem_index<VEC>(lo, tid, j);
+                if (takes[j]) { // uniform
+                    const uint32_t pos =
+                        run + __builtin_amdgcn_mbcnt_hi((uint32_t)(takes[j] >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)takes[j], 0u));
+                    const float w = wv[j];
+                    if (w >= tau && pos < kCap) {
+                        sm.cw[pos] = w;
+                        sm.ci[pos] = elem_index<VEC>(lo, tid, j);
+                    }
+                    run += (uint32_t)__popcll(takes[j]);
                 }
-                pos += take ? 1u : 0u;
             }
         }
     }

@@ -132,14 +132,19 @@ __device__ __forceinline__ void finish_slice(const RawSlice<VEC>& r, uint32_t lo
             wv[4 * k + 3] = !inside ? nan : r.v[k].w;
         }
     } else if (VEC) {
+        // (a mask bit spread over a word, then one bit-field insert: the logit where the bit is set, -inf elsewhere)
         const float nan = __uint_as_float(0x7fc00000u);
+        auto pick = [](uint32_t bits, uint32_t c, float v) {
+            const uint32_t m = (uint32_t)((int32_t)(bits << (31u - c)) >> 31); // all ones if bit c is set
+            return __uint_as_float((__float_as_uint(v) & m) | (0xff800000u & ~m));
+        };
 #pragma unroll
         for (uint32_t k = 0; k < 4; ++k) {
             const bool inside = lo + k * 4096u + tid * 4u < hi;
-            wv[4 * k + 0] = !inside ? nan : ((r.bits[k] & 1u) ? r.v[k].x : -INFINITY);
-            wv[4 * k + 1] = !inside ? nan : ((r.bits[k] & 2u) ? r.v[k].y : -INFINITY);
-            wv[4 * k + 2] = !inside ? nan : ((r.bits[k] & 4u) ? r.v[k].z : -INFINITY);
-            wv[4 * k + 3] = !inside ? nan : ((r.bits[k] & 8u) ? r.v[k].w : -INFINITY);
+            wv[4 * k + 0] = !inside ? nan : pick(r.bits[k], 0, r.v[k].x);
+            wv[4 * k + 1] = !inside ? nan : pick(r.bits[k], 1, r.v[k].y);
+            wv[4 * k + 2] = !inside ? nan : pick(r.bits[k], 2, r.v[k].z);
+            wv[4 * k + 3] = !inside ? nan : pick(r.bits[k], 3, r.v[k].w);
         }
     } else {
         const float* f = reinterpret_cast<const float*>(r.v);
