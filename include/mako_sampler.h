@@ -51,6 +51,7 @@ typedef struct mako_sampling_params {
 #define MAKO_PATH_NUCLEUS 4u  /* top_k == 0: nucleus resolved from the per-slice candidates */
 #define MAKO_PATH_GENERAL 5u  /* whole-row sort path */
 #define MAKO_PATH_FORCED 6u   /* not sampled: force_token / close_token took the row */
+#define MAKO_PATH_SORTED 7u   /* top_k == 0: nucleus cut from the sorted list of the weights the row's plan kept */
 
 /* out_forced values */
 #define MAKO_FORCED_NONE 0u  /* the row was sampled (or verified) */

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libmako_sampler.so")
 MAKO_OK = 0
 MAKO_ERR_INVALID_ARG = -1
 MAKO_ERR_HIP = -2
-PATH_GREEDY, PATH_FALLBACK, PATH_TOPK, PATH_NUCLEUS, PATH_GENERAL, PATH_FORCED = 1, 2, 3, 4, 5, 6
+PATH_GREEDY, PATH_FALLBACK, PATH_TOPK, PATH_NUCLEUS, PATH_GENERAL, PATH_FORCED, PATH_SORTED = 1, 2, 3, 4, 5, 6, 7
 FORCED_NONE, FORCED_TOKEN, FORCED_CLOSE = 0, 1, 2
 
 # mako_sampling_params / SamplingParams (src/gen/sampler.hpp:11-20)

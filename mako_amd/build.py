@@ -7,8 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 # the C ABI, and one translation unit per kernel family (a kernel's register allocation then does not depend on
 # which other kernels exist; they also compile side by side)
-SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_for_sort.hip",
-           "k_plan_alone.hip", "k_sort.hip", "k_tail.hip"]
+SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_alone.hip", "k_sort.hip", "k_tail.hip"]
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 OUT = os.path.join(HERE, "libmako_sampler.so")
 

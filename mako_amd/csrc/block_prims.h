@@ -16,6 +16,7 @@ extern "C" __device__ unsigned long long __ockl_wfred_max_u64(unsigned long long
 extern "C" __device__ double __ockl_wfred_add_f64(double);
 extern "C" __device__ uint32_t __ockl_wfscan_add_u32(uint32_t, bool inclusive);
 extern "C" __device__ double __ockl_wfscan_add_f64(double, bool inclusive);
+extern "C" __device__ float __ockl_wfscan_add_f32(float, bool inclusive);
 
 namespace mako {
 

@@ -5,11 +5,6 @@
 #include "sampler_kernels.h"
 
 namespace mako {
-void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows)
-{
-    hipLaunchKernelGGL(partition_kernel, dim3(kWorkers, grid_rows), dim3(kThreads), 0, st, d, sc);
-}
-
 void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows)
 {
     hipLaunchKernelGGL(sort_kernel, dim3(kWorkers, grid_rows), dim3(kThreads), kSortLds, st, d, sc, slices);

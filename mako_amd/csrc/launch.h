@@ -13,29 +13,23 @@ struct Scratch;
 
 hipError_t init_scan_kernels();
 hipError_t init_finish_kernels();
-hipError_t init_plan_for_sort();
 hipError_t init_plan_alone();
 hipError_t init_sort_kernels();
 hipError_t init_tail_kernels();
 
 // scan_kernel<vec, kh, above>, grid = (slices, rows), `lds` bytes of dynamic LDS
-// (`sc`: the HOST copy of the context's record; scan, partition, sort and tail kernels take it by value, so that their
+// (`sc`: the HOST copy of the context's record; scan, sort and tail kernels take it by value, so that their
 // first loads need no trip to memory for the record itself; finish and plan kernels take the device copy's address)
 void launch_scan(bool vec, int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d,
                  const Scratch& sc, uint32_t slice_len, uint32_t cus);
 // finish_kernel<vec, kh> on `wgs` workgroups
 void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch* sc,
                    uint32_t slices);
-// plan_kernel, one workgroup per row: <false> when sort_kernel follows (it has the whole-row path), <true> when
-// plan_kernel is the last kernel of the batch
-void launch_plan_for_sort(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
 void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
-// partition_kernel and sort_kernel serve the same work list, workgroup i its entry i: `grid_rows` * kWorkers workgroups
-// must cover the longest list the batch can produce (kWorkers entries per top_k == 0 row, one per other sampled
-// row); tail_kernel takes one workgroup per possible wide row.  Workgroups beyond the lists leave at once, but each
+// sort_kernel's workgroup i serves entry i of the work list: `grid_rows` * kWorkers workgroups must cover the
+// longest list the batch can produce (kWorkers entries per top_k == 0 row); tail_kernel takes one workgroup per possible wide row.  Workgroups beyond the lists leave at once, but each
 // of them still has to be dispatched.
-void launch_partition(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t grid_rows); // (host copy, by value)
 void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows); // (host copy)
-// (tail_kernel: `tail_cap` workgroups for the possible wide rows, then one per row for the batch's top-k rows)
+// (tail_kernel: `tail_cap` workgroups for the possible wide rows, then one per row for what is left of every row)
 void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t tail_cap); // (host copy, by value)
 } // namespace mako

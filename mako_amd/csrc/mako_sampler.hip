@@ -113,7 +113,6 @@ hipError_t layout_scratch(mako::Scratch& sc, mako::Scratch** sc_dev, uint32_t ma
     MAKO_TAKE(sc.part_sum, (size_t)max_rows * mako::kMaxSlices);
     MAKO_TAKE(sc.part_n, (size_t)max_rows * mako::kMaxSlices);
     MAKO_TAKE(sc.plan, (size_t)max_rows);
-    MAKO_TAKE(sc.bins, (size_t)max_rows * mako::kBins);
     MAKO_TAKE(sc.wbuf, rv);
     MAKO_TAKE(sc.cnt, rv);
     MAKO_TAKE(sc.key[0], rv);
@@ -129,7 +128,7 @@ hipError_t layout_scratch(mako::Scratch& sc, mako::Scratch** sc_dev, uint32_t ma
     MAKO_TAKE(sc.gt.start, rg);
     MAKO_TAKE(sc.gt.pack, rg);
     MAKO_TAKE(sc.gt.quarters, rg * 4);
-    MAKO_TAKE(sc.bin_worker, (size_t)max_rows * mako::kBins);
+    MAKO_TAKE(sc.log_hist, (size_t)max_rows * sc.slices_cap * mako::kLogBins);
     MAKO_TAKE(sc.work_n, 8);
     MAKO_TAKE(sc.work_sort, (size_t)max_rows * mako::kWorkers);
     MAKO_TAKE(sc.work_tail, (size_t)max_rows);
@@ -141,8 +140,6 @@ hipError_t layout_scratch(mako::Scratch& sc, mako::Scratch** sc_dev, uint32_t ma
 hipError_t zero_scratch(const mako::Scratch& sc, uint32_t max_rows)
 {
     hipError_t e = hipMemset(sc.plan, 0, (size_t)max_rows * sizeof(mako::BigPlan));
-    if (e == hipSuccess)
-        e = hipMemset(sc.bins, 0, (size_t)max_rows * mako::kBins * sizeof(unsigned long long));
     if (e == hipSuccess)
         e = hipMemset(sc.cnt, 0, (size_t)max_rows * sc.vpad * sizeof(uint32_t));
     if (e == hipSuccess)
@@ -242,7 +239,6 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     // the kernels overlay up to 64 KB of dynamic LDS (sort_kernel more) on a few KB of static LDS
     MAKO_HIP(ctx, mako::init_scan_kernels());
     MAKO_HIP(ctx, mako::init_finish_kernels());
-    MAKO_HIP(ctx, mako::init_plan_for_sort());
     MAKO_HIP(ctx, mako::init_plan_alone());
     MAKO_HIP(ctx, mako::init_sort_kernels());
     MAKO_HIP(ctx, mako::init_tail_kernels());
@@ -255,8 +251,8 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {ctx->sc_dev, sc.bin_worker, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
-                    sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.bins, sc.plan,
+    void* ptrs[] = {ctx->sc_dev, sc.log_hist, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
+                    sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
                     ctx->st_hist,  ctx->st_hcnt, ctx->st_hlen,  ctx->st_draft, ctx->st_tokens, ctx->st_acc};
@@ -415,20 +411,17 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     if (any_nucleus)
         MAKO_LAUNCH(mako::launch_finish(vec, kh, finish_wgs, st, d, sc_dev, slices));
     MAKO_MARK(2);
-    // top_k == 0 rows: plan from the row's histogram, sort by the plan, cut and draw; the stages talk through
-    // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  Other rows cost a load.
-    if (launch_sort)
-        MAKO_LAUNCH(mako::launch_plan_for_sort(st, d, sc_dev, slices));
-    else
+    // top_k == 0 rows: planned and handed out by the second pass, sorted, cut and drawn from; the stages talk through
+    // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  A batch without such rows
+    // (and without rows for the whole-row path) ends with plan_kernel instead.
+    if (!launch_sort)
         MAKO_LAUNCH(mako::launch_plan_alone(st, d, sc_dev, slices));
     MAKO_MARK(3);
-    if (any_nucleus)
-        MAKO_LAUNCH(mako::launch_partition(st, d, sc, nucleus_rows));
     MAKO_MARK(4);
     if (any_nucleus)
         MAKO_LAUNCH(mako::launch_sort(st, d, sc, slices, nucleus_rows));
     MAKO_MARK(5);
-    if (launch_sort) // (also finishes the rows that plan_kernel<false> and sort_kernel leave: finish_late_row())
+    if (launch_sort) // (also finishes every row the kernels before it leave: finish_late_row())
         MAKO_LAUNCH(mako::launch_tail(st, d, sc, slices, nucleus_rows));
     MAKO_MARK(6);
 #undef MAKO_MARK

@@ -1,23 +1,17 @@
-// plan_kernel: one workgroup per row between the second pass and the sort.
+// plan_kernel: one workgroup per row of a batch that needs neither the second pass nor the sort.
 #pragma once
 
 #include "topk_candidates.h"
-#include "nucleus_plan.h"
 
 namespace mako {
 
-// grid = (1, rows), one workgroup per row.  Rows whose token is forced, greedy rows and (INLINE_GENERAL only: in a
-// batch that goes on to sort_kernel and tail_kernel, top-k and whole-row rows are finished beside the tails) top-k
-// rows are finished here from the records scan_kernel left; a top_k == 0 row's exact total, candidate count and weight histogram (from
-// finish_kernel) are summed over its pieces and the row is planned: handed to sort_kernel's workers, or, when the
-// nucleus is narrow enough to end inside the candidate lists, to its worker 0 alone.
-// INLINE_GENERAL: sort_kernel will not be launched for this batch (the host saw no row that needs it), so a row
-// that turns out to need the whole-row path after all is given it here.  (A variant of its own: the whole-row path
-// costs the kernel registers that the usual batches should not pay for.)
-template <bool INLINE_GENERAL>
+#ifdef MAKO_EMIT_PLAN_KERNEL // (not a template: defined by the one translation unit that launches it)
+// grid = (1, rows), one workgroup per row, for a batch without top_k == 0 rows and without rows that need the
+// whole-row path (the host saw none in its copy of the parameters): such a batch ends here.  Rows whose token is
+// forced, greedy rows and top-k rows are finished from the records scan_kernel left; a row that turns out to need
+// the whole-row path after all is given it here.
 __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
 {
-    constexpr bool inline_general = INLINE_GENERAL;
     const Scratch& sc_arg = *sc_dev;
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
@@ -67,7 +61,7 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     __syncthreads();
     // a top-k row's candidates are asked for together with the slices' records
     CandSlots pre;
-    const bool prefetched = inline_general && cls == kTopK && !d.draft && slots_cover(slices); // uniform
+    const bool prefetched = cls == kTopK && !d.draft && slots_cover(slices); // uniform
     if (prefetched)
         fetch_candidate_slots(sc, row, slices, pre);
     float m;
@@ -90,66 +84,13 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
         return;
     }
 
-    if (cls != kNucleus) {
-        // (in a batch that goes on to sort_kernel and tail_kernel, tail_kernel's launch finishes these rows beside the
-        // tails: finish_late_row())
-        if constexpr (inline_general) {
-            if (topk_takes_whole_row(cls, any_overflow, n_cands))
-                general_row<1>(d, sc, row, P, m, argidx, L);
-            else
-                topk_row(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
-        }
-        return;
-    }
-
-    MAKO_STAMP(2);
-    const uint32_t pieces = uniform_u32(sc.work_n[4]);
-    // this thread's two bins of the row's histogram (left zero for the next batch), the pieces' exact sums (one per
-    // lane, added up in the wave reduction's fixed order)
-    unsigned long long* bins = sc.bins + (size_t)row * kBins;
-    const unsigned long long rec0 = bins[kBins - 1u - 2u * tid], rec1 = bins[kBins - 2u - 2u * tid];
-    const uint32_t bin_c0 = (uint32_t)(rec0 >> kBinSumBits), bin_c1 = (uint32_t)(rec1 >> kBinSumBits);
-    const unsigned long long bin_s0 = rec0 & ((1ull << kBinSumBits) - 1ull), bin_s1 = rec1 & ((1ull << kBinSumBits) - 1ull);
-    const uint32_t pc = min((uint32_t)lane_id(), pieces - 1u); // pieces <= kMaxSlices = 64
-    const double ps = sc.part_sum[(size_t)row * kMaxSlices + pc];
-    const uint32_t pn = sc.part_n[(size_t)row * kMaxSlices + pc];
-    const double row_total = __ockl_wfred_add_f64((uint32_t)lane_id() < pieces ? ps : 0.0);
-    const uint32_t row_n0 = __ockl_wfred_add_u32((uint32_t)lane_id() < pieces ? pn : 0u);
-    if (rec0)
-        bins[kBins - 1u - 2u * tid] = 0;
-    if (rec1)
-        bins[kBins - 2u - 2u * tid] = 0;
-    MAKO_STAMP(15);
-    if (row_n0 == 0) {
-        fallback_row(d, row, argidx);
-        return;
-    }
-    uint32_t thr_bits = 0;
-    const uint32_t n0 = plan_nucleus(P, row_total, bin_c0, bin_c1, bin_s0, bin_s1, sc.plan + row, sc.bin_worker + (size_t)row * kBins, L, thr_bits, d.n_vocab);
-    MAKO_STAMP(16);
-    const bool narrow = !d.draft && n0 <= kSmall && !any_overflow && n_cands <= kSortMax;
-    // (a list too long for the workers' group records goes to the whole-row path)
-    const bool fits = n0 <= kGroup * (kMaxGroups - kWorkers);
-    if (tid == 0) {
-        if (!fits) {
-            sc.plan[row].total64 = (double)m;
-            sc.plan[row].n0 = argidx;
-        }
-        sc.plan[row].thr = thr_bits;
-        sc.plan[row].flag = !fits ? 2 : (narrow ? 3 : 1);
-    }
-    // the row's pieces of work for sort_kernel (all workers, or worker 0 alone) and tail_kernel; a row for the
-    // whole-row path is finished in tail_kernel's launch from its flag alone (finish_late_row())
-    if (!fits)
-        return;
-    const uint32_t work = !narrow ? kWorkers : 1u;
-    if (tid == 0)
-        sm.flag = atomicAdd(&sc.work_n[0], work);
-    __syncthreads();
-    if (tid < work)
-        sc.work_sort[sm.flag + tid] = (row << 8) | tid;
-    if (tid == 0 && !narrow)
-        sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
+    // (a top_k == 0 row has no business here; should the host's copy of the parameters have hidden one, the whole-row
+    // path serves it like any other)
+    if (cls == kNucleus || topk_takes_whole_row(cls, any_overflow, n_cands))
+        general_row<1>(d, sc, row, P, m, argidx, L);
+    else
+        topk_row(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
 }
+#endif // MAKO_EMIT_PLAN_KERNEL
 
 } // namespace mako

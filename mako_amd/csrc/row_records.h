@@ -7,14 +7,10 @@ namespace mako {
 
 // First maximum of the row (std::max_element semantics, NaNs never win unless at index 0) and the totals of the
 // slices' candidate lists, from the records scan_kernel left.
-__device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uint32_t slices, float& m, uint32_t& argidx,
-                                            uint32_t& n_cands, uint32_t& any_overflow, SliceStat* lane_stat = nullptr)
+// (`st`: the record of slice min(lane, slices - 1), already loaded)
+__device__ __forceinline__ void row_summary_of(const SliceStat& st, uint32_t slices, float& m, uint32_t& argidx,
+                                               uint32_t& n_cands, uint32_t& any_overflow)
 {
-    // lane s of every wave takes slice s (at most kMaxSlices = 64 of them): one load each, then wave reductions
-    const uint32_t s = min((uint32_t)lane_id(), slices - 1u);
-    const SliceStat st = sc.stats[(size_t)row * kMaxSlices + s];
-    if (lane_stat)
-        *lane_stat = st;
     const bool mine = (uint32_t)lane_id() < slices;
     const unsigned long long p =
         mine ? ((unsigned long long)order_key(st.wmax) << 32) | (unsigned long long)(kNone - st.argidx) : 0ull;
@@ -30,6 +26,15 @@ __device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uin
         m = __uint_as_float(0x7fc00000u);
         argidx = 0;
     }
+}
+__device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uint32_t slices, float& m, uint32_t& argidx,
+                                            uint32_t& n_cands, uint32_t& any_overflow, SliceStat* lane_stat = nullptr)
+{
+    // lane s of every wave takes slice s (at most kMaxSlices = 64 of them): one load each, then wave reductions
+    const SliceStat st = sc.stats[(size_t)row * kMaxSlices + min((uint32_t)lane_id(), slices - 1u)];
+    if (lane_stat)
+        *lane_stat = st;
+    row_summary_of(st, slices, m, argidx, n_cands, any_overflow);
 }
 
 // Where each slice's candidates start in the row's flattened candidate list (sm.soff), and the largest weight a

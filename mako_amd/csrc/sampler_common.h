@@ -21,6 +21,7 @@ constexpr uint32_t kMaxSlices = 64;
 constexpr uint32_t kCap = 512;       // candidates kept per slice
 constexpr uint32_t kTopKFast = 128;  // largest top_k resolved from the per-slice candidates
 constexpr uint32_t kSortMax = 4096;  // candidates the finisher sorts in LDS
+constexpr uint32_t kSmall = 256;     // lists of up to this many entries are ordered by counting ranks
 constexpr uint32_t kDynLds = 65536;  // dynamic LDS of both kernels
 constexpr uint32_t kBins = 2048;     // weight histogram of top_k == 0 rows, see weight_bin()
 constexpr uint32_t kBinSumBits = 44; // a bin's record: count << 44 | sum of 24-bit significands
@@ -63,6 +64,46 @@ struct SliceStat {
     uint32_t pad[2];
 };
 
+// A coarse view of a top_k == 0 row before its weights exist.  A logit's `unit` is floor(logit * scale) with
+// scale = kLogUnitsPerOctave * log2(e) / T: one unit is 1/kLogUnitsPerOctave of a factor of two of the weight the
+// logit will have, and the unit is a function of the logit and the row's temperature alone.  scan_kernel counts each
+// slice's penalised logits by unit, in the frame of the slice's own maximum: one bin per unit for the kLogFine units
+// at and below the maximum's (near-flat rows, whose weights all lie within a factor of two, still spread over a
+// hundred bins), one bin per aligned group of 2^kLogCoarseShift units below that (36 octaves in all; what lies
+// further down is not counted).  Units and groups are absolute, so the second pass can move every slice's counts
+// into the frame of the row's maximum with integer arithmetic alone, exactly, and size its work from them before it
+// has computed a single weight.  Nothing exact is ever decided from these counts: they balance work and size buffers,
+// and every list built from them is checked against the exact sums afterwards.
+constexpr uint32_t kLogBins = 1024;
+constexpr uint32_t kLogUnitsPerOctave = 128;
+constexpr uint32_t kLogFine = 512;
+constexpr uint32_t kLogCoarseShift = 3;
+__device__ __forceinline__ float log_unit_scale(const mako_sampling_params& P)
+{
+    return (1.0f / P.temperature) * (1.4426950408889634f * (float)kLogUnitsPerOctave);
+}
+__device__ __forceinline__ int32_t log_unit(float logit, float scale)
+{
+    // (NaN and whatever is out of range end up at the limits: the same for every kernel that asks)
+    return (int32_t)floorf(fminf(fmaxf(logit * scale, -1.0e9f), 1.0e9f));
+}
+// Bin of unit k in the frame of a maximum whose unit is k_top; kLogBins - 1 and above: not counted.
+__device__ __forceinline__ uint32_t log_bin_in_frame(int32_t k, int32_t k_top)
+{
+    const uint32_t d = (uint32_t)k_top - (uint32_t)k;
+    const uint32_t c = (uint32_t)(((k_top - (int32_t)kLogFine) >> kLogCoarseShift) - (k >> kLogCoarseShift));
+    return d < kLogFine ? d : (c < kLogBins ? kLogFine + c : kLogBins);
+}
+// How far below the maximum (its unit k_top) the middle of bin b lies, in units, counted from the maximum's unit's
+// lower edge.
+__device__ __forceinline__ float log_bin_middle(uint32_t b, int32_t k_top)
+{
+    if (b < kLogFine)
+        return (float)b - 0.5f;
+    const int32_t g = ((k_top - (int32_t)kLogFine) >> kLogCoarseShift) - (int32_t)(b - kLogFine);
+    return (float)(k_top - g * (1 << kLogCoarseShift) - (1 << (kLogCoarseShift - 1)));
+}
+
 constexpr uint32_t kWorkers = 32;  // workgroups that share the sort of one wide-nucleus row
 constexpr uint32_t kGroup = 256;      // a sorted list is processed in groups of one wave x four entries per lane
 constexpr uint32_t kMaxGroups = 1024; // groups per list
@@ -73,25 +114,28 @@ constexpr uint32_t kFine = 2048;      // value buckets of that sort
 constexpr uint32_t kSortLds = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u + kSegCap * 4u;
 constexpr uint32_t kSortedCopyAt = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u; // byte offset of that copy
 
-// Work order for a top_k == 0 row whose nucleus is too wide for the per-slice candidate lists: the weights
-// with bits(q) >= key_lo (n0 of them) are split by value into kWorkers contiguous ranges of about equal size.
+// Work order for a top_k == 0 row, written by the second pass (every workgroup of the row derives the same one from
+// scan_kernel's coarse counts, see coarse_plan(); the row's first piece stores it): the weights with bits(q) >= thr
+// are split by value into kWorkers contiguous ranges of about equal size, handed to the workers' shares as they are
+// computed, sorted by sort_kernel and cut and drawn from by tail_kernel.
 struct BigPlan {
     uint32_t flag;   // 1: the row waits for sort_kernel's workers and tail_kernel; 2: for the whole-row path (in
                      // tail_kernel's launch); 3: a narrow nucleus, finished by worker 0 from the candidate lists;
                      // 4: one that the lists could not certify (second look in tail_kernel's launch)
-    uint32_t n0;     // entries to sort
-    uint32_t pad0;
+    uint32_t n0;     // entries of the sorted list (sort_kernel's worker 0 adds up what the workers were handed)
+    uint32_t overflow; // set by the second pass when a worker's share did not fit its room (then flag 2 follows)
     uint32_t groups; // groups of the whole list: each worker's range is cut into groups of kGroup on its own
-    double total64;  // exact fp64 sum of q over the row's candidates
-    uint32_t thr;    // bits(q) below which the nucleus cannot reach
+    double total64;  // exact fp64 sum of q over the row's candidates (worker 0)
+    uint32_t thr;    // bits(q) from which weights are kept
+    uint32_t argidx; // first index of the row's maximum, and the maximum (for the whole-row path)
+    float m;
     uint32_t pad;
-    uint32_t key_lo[kWorkers]; // worker w takes bits(q) in [key_lo[w], key_hi[w])
-    uint32_t key_hi[kWorkers];
-    uint32_t off[kWorkers];    // and writes them from position off[w] of the sorted list
-    uint32_t cnt[kWorkers];
-    uint32_t gbase[kWorkers];  // first group of worker w
-    uint32_t cursor[kWorkers]; // entries partition_kernel has handed to worker w so far
-    double mass[kWorkers];     // sum of the weights above worker w's range
+    double mass_all; // the plan's estimate of the row's total, in the units of mass[]
+    uint32_t key_lo[kWorkers];    // worker w takes bits(q) in [key_lo[w], key_lo[w - 1]) (worker 0: up to 1.0)
+    uint32_t stage_off[kWorkers]; // where its share starts in the row's staging arrays (Scratch::key[1], idx[1])
+    uint32_t cap[kWorkers];       // and how many entries it has room for
+    uint32_t cursor[kWorkers];    // entries handed to worker w so far (zeroed by scan_kernel)
+    double mass[kWorkers];        // estimated sum of the weights above worker w's range
 };
 
 // Per-group records of a planned row's sorted list, written by the workers and read by the last of them.
@@ -112,18 +156,14 @@ struct Scratch {
     double* part_sum;  // [max_rows][kMaxSlices] exact fp64 sum of q over the slice (top_k == 0 rows)
     uint32_t* part_n;  // [max_rows][kMaxSlices] candidates (q > 0, q >= min_p) in the slice
     BigPlan* plan;     // [max_rows]; flag zero between calls
-    unsigned long long* bins; // [max_rows][kBins] weight histogram of top_k == 0 rows: candidates in the bin << 44 |
-                              // sum of their 24-bit significands (kBinSumBits: at most 2^20 - 1 logits per row).
-                              // A bin's exact mass is that sum * 2^(e - 150), e being the bin's exponent.  The
-                              // slices add with one atomic per non-empty bin; plan_kernel reads the row's bins
-                              // and leaves them zero
-    float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path; top_k == 0 rows keep
-                       // bits(q) of every logit here instead (0 where q is not a candidate)
+    float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path, then bits(q) of every logit
+                       // (0 where q is not a candidate)
     uint32_t* cnt;     // [max_rows][vpad] token counts; all zero between calls
     uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong; [1] also takes the workers' unsorted
-                       // shares (bits(q)) from partition_kernel
+                       // shares (bits(q)) from the second pass
     uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, likewise
-    uint8_t* bin_worker; // [max_rows][kBins] the worker that takes the weights of each histogram bin (0xff: none)
+    uint32_t* log_hist;  // [max_rows][slices_cap][kLogBins] top_k == 0 rows: logits of the slice by their distance
+                         // below the slice's own maximum (log_bin_of())
     GroupTable gt;     // [max_rows][g_cap] each
     // Work lists.  sort_kernel and tail_kernel are launched with one workgroup per POSSIBLE piece of work, but
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
@@ -132,8 +172,8 @@ struct Scratch {
     uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); then, 16-byte aligned at [4],
                            // the second pass's pieces per top_k == 0 row, their length and the number of workgroups
                            // with work (scan_kernel's first workgroup decides, see second_pass_pieces())
-    uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel and plan_kernel
-    uint32_t* work_tail;   // [max_rows] row; appended by plan_kernel
+    uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel
+    uint32_t* work_tail;   // [max_rows] row; appended by finish_kernel
     uint64_t vpad;
     uint32_t slices_cap;
     uint32_t g_cap;    // vpad / kGroup + kWorkers

@@ -15,6 +15,7 @@ struct alignas(16) ScanShared {
     uint32_t emit_flags;
     float cw[kCap];
     uint32_t ci[kCap];
+    uint32_t log_hist[kLogBins + kWave]; // top_k == 0 rows (and one slot per lane for what is not counted)
 };
 
 // A lower bound, tight to 2^-9 relative, of the j-th largest of the wavefront's 64 order keys (j >= 1): the largest
@@ -75,6 +76,16 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
         if (row == 0 && slice == 0) { // the lists finish_kernel and plan_kernel append to start empty
             sc.work_n[0] = 0;
             sc.work_n[1] = 0;
+        }
+    }
+    static_assert(kLogBins == (uint32_t)kThreads, "one bin per thread");
+    if (cls == kNucleus) {
+        sm.log_hist[tid] = 0;
+        if (slice == 0) { // what the second pass adds to starts at zero
+            if (tid < kWorkers)
+                sc.plan[row].cursor[tid] = 0;
+            if (tid == 0)
+                sc.plan[row].overflow = 0;
         }
     }
     if (row == 0 && slice == 0 && wave_id() == 1) { // how the second pass will be cut up
@@ -200,8 +211,22 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
             }
         }
     }
+    if (cls == kNucleus) {
+        // the slice's logits by unit, in the frame of the slice's maximum (log_bin_in_frame()); what the bins do not
+        // cover (and NaN) goes to a slot of the lane's own
+        const float scale = log_unit_scale(P);
+        const int32_t k_top = log_unit(st.wmax, scale);
+        const uint32_t dump = kLogBins + (uint32_t)lane_id();
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j) {
+            const uint32_t bin = log_bin_in_frame(log_unit(wv[j], scale), k_top);
+            atomicAdd(&sm.log_hist[bin < kLogBins - 1u ? bin : dump], 1u);
+        }
+    }
     __syncthreads();
     MAKO_STAMP(31);
+    if (cls == kNucleus)
+        sc.log_hist[((size_t)row * sc.slices_cap + slice) * kLogBins + tid] = sm.log_hist[tid];
     if (emits) {
         const uint32_t n = sm.emit_n;
         if (n > kCap)

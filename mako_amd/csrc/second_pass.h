@@ -4,40 +4,80 @@
 #include "slice_load.h"
 #include "work_split.h"
 #include "row_records.h"
+#include "coarse_plan.h"
 
 namespace mako {
 
-// Exact fp64 sum of q over one slice, and the number of candidates in it (q > 0 and q >= min_p).
+// One piece of a top_k == 0 row: the exact fp64 sum of q over it and the number of candidates in it (q > 0 and
+// q >= min_p), and every weight the row's plan keeps handed to the share of the worker that will sort it.
 // The summation order is fixed: each thread adds its logits in index order, then lanes, then waves.
+// The plan (coarse_plan()) is built while the piece's logits are on their way; every workgroup of the row arrives at
+// the same one, and the row's first piece stores it for the kernels that follow and enters the row in their lists.
 // (PEN: the row has penalties to apply; a compile-time fact so that each case gets straight-line code of its own.)
-// (`slices`: of scan_kernel, whose records give the row maximum; they are asked for behind the piece's own loads)
+// (`slices`: of scan_kernel, whose records give the row maximum)
 template <bool VEC, int KH, bool PEN>
 __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slice,
                               uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, uint32_t slices,
-                              const FinishLds& L)
+                              const FinishLds& L, CoarsePlan& pl)
 {
     FinishShared& sm = *L.sm;
+    const uint32_t tid = threadIdx.x;
     const uint32_t lo = slice * slice_len;
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
     constexpr bool pen = PEN;
     float wv[16];
     float m = 0.0f;
+    uint32_t argidx = 0;
+    PlanLoads pre;
+    issue_plan_loads(sc, row, slices, pre);
     load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, [&]() {
-        uint32_t argidx, n_cands, any_overflow;
-        row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
+        uint32_t n_cands, any_overflow;
+        row_summary_of(pre.st, slices, m, argidx, n_cands, any_overflow);
+        coarse_plan(sc, row, slices, P, m, pre, !d.draft && !any_overflow && n_cands <= kSortMax, pl, sm.tab);
     });
     MAKO_STAMP(1);
     MAKO_STAMP(24);
+    BigPlan* plan = sc.plan + row;
+    const uint32_t flag = pl.flag;
+    if (slice == 0) {
+        // the row's first piece stores the plan and enters the row in the lists of sort_kernel and tail_kernel
+        if (tid < kWorkers) {
+            plan->key_lo[tid] = pl.key_lo[tid];
+            plan->stage_off[tid] = pl.stage_off[tid];
+            plan->cap[tid] = pl.cap[tid];
+            plan->mass[tid] = pl.mass_above[tid];
+        }
+        if (tid == 0) {
+            plan->thr = pl.thr;
+            plan->argidx = argidx;
+            plan->m = m;
+            plan->mass_all = pl.mass_all;
+            plan->flag = flag;
+            if (flag == 1 || flag == 3) {
+                const uint32_t work = flag == 1 ? kWorkers : 1u;
+                const uint32_t at = atomicAdd(&sc.work_n[0], work);
+                for (uint32_t w = 0; w < work; ++w)
+                    sc.work_sort[at + w] = (row << 8) | w;
+                if (flag == 1)
+                    sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
+            }
+        }
+    }
+    if (flag == 2) // the whole-row path starts from the logits again
+        return;
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
+    const uint32_t thr = pl.thr;
     double sum = 0;
     uint32_t n = 0;
-    uint32_t qb[16]; // bits(q), 0 where q is not a candidate
+    uint32_t qb[16];   // bits(q), 0 where q is not a candidate
+    uint32_t slot[16]; // kept weights: worker << 16 | position among this workgroup's entries for that worker
     // (a piece may be shorter than the sixteen logits per thread: whole blocks past its end are skipped; the test is
     // the same for every thread)
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j) {
         qb[j] = 0u;
+        slot[j] = kNone;
         if (lo + (VEC ? (j / 4u) * 4096u : j * (uint32_t)kThreads) < hi) {
             const float q = weight_of(wv[j], m, inv_t, sm.tab);
             qb[j] = (q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
@@ -45,11 +85,19 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
                 sum += (double)q;
                 ++n;
             }
+            if (qb[j] >= thr && qb[j]) {
+                // the worker whose range of bits(q) holds the weight (equal weights always meet in one share): the
+                // number of workers whose lower edge lies above it, by bisection over the edges
+                uint32_t w = 0;
+#pragma unroll
+                for (uint32_t step = kWorkers / 2u; step; step >>= 1)
+                    w += qb[j] < pl.key_lo[w + step - 1u] ? step : 0u;
+                slot[j] = (w << 16) | atomicAdd(&pl.count[w], 1u);
+            }
         }
     }
     MAKO_STAMP(25);
-    // the piece's sum and count: wave reductions, one exchange of the sixteen waves' results for both (the barrier
-    // also retires every use of L.cnt above); they are stored at the very end, so that no barrier waits for the store
+    // the piece's sum and count: wave reductions, one exchange of the sixteen waves' results for both
     {
         const double sw = __ockl_wfred_add_f64(sum);
         const uint32_t nw = __ockl_wfred_add_u32(n);
@@ -59,44 +107,29 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
         }
     }
     lds_barrier();
-    // bits(q) of every logit of the slice (0 = not a candidate) and their histogram, for nucleus_big_row()
-    uint32_t* qk = reinterpret_cast<uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
-    unsigned long long* hist = reinterpret_cast<unsigned long long*>(L.cnt); // count << kBinSumBits | significands
-    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads)
-        hist[b] = 0;
-    lds_barrier();
     MAKO_STAMP(26);
-    // one candidate and the significand of a positive float (subnormals: no hidden bit, as seqfp::split)
-    auto record = [](uint32_t b) {
-        return (1ull << kBinSumBits) | (unsigned long long)((b & 0x7fffffu) | ((b >> 23) ? 0x800000u : 0u));
-    };
+    // one run per worker in its share of the row's staging arrays, reserved with a single atomic
+    if (tid < kWorkers)
+        pl.base[tid] = pl.count[tid] ? atomicAdd(&plan->cursor[tid], pl.count[tid]) : 0u;
+    __syncthreads();
+    MAKO_STAMP(27);
+    uint32_t* kstage = sc.key[1] + (size_t)row * sc.vpad;
+    uint32_t* istage = sc.idx[1] + (size_t)row * sc.vpad;
+    bool dropped = false;
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j)
-        if (qb[j])
-            atomicAdd(&hist[weight_bin(qb[j])], record(qb[j]));
-    if (VEC) {
-#pragma unroll
-        for (uint32_t k = 0; k < 4; ++k) {
-            const uint32_t i = lo + k * 4096u + threadIdx.x * 4u;
-            if (i < hi)
-                *reinterpret_cast<uint4*>(qk + i) = make_uint4(qb[4 * k], qb[4 * k + 1], qb[4 * k + 2], qb[4 * k + 3]);
+        if (slot[j] != kNone) {
+            const uint32_t w = slot[j] >> 16, at = pl.base[w] + (slot[j] & 0xffffu);
+            if (at < pl.cap[w]) {
+                kstage[pl.stage_off[w] + at] = qb[j];
+                istage[pl.stage_off[w] + at] = elem_index<VEC>(lo, tid, j);
+            } else {
+                dropped = true;
+            }
         }
-    } else {
-#pragma unroll
-        for (uint32_t j = 0; j < 16; ++j) {
-            const uint32_t i = lo + j * (uint32_t)kThreads + threadIdx.x;
-            if (i < hi)
-                qk[i] = qb[j];
-        }
-    }
-    lds_barrier(); // (the histogram is complete; nobody waits for the stores above)
-    MAKO_STAMP(27);
-    // the slice's non-empty bins are added to the row's histogram (a few hundred atomics per slice, none waited for)
-    unsigned long long* bins = sc.bins + (size_t)row * kBins;
-    for (uint32_t b = threadIdx.x; b < kBins; b += kThreads)
-        if (hist[b])
-            atomicAdd(&bins[b], hist[b]);
-    if (threadIdx.x == 0) {
+    if (dropped) // (more weights in a range than the counts promised: the row takes the whole-row path)
+        plan->overflow = 1;
+    if (tid == 0) {
         double total = 0;
         uint32_t count = 0;
         for (int w = 0; w < kWaves; ++w) { // waves in order: the same inputs always give the same bits
@@ -119,6 +152,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
+    __shared__ CoarsePlan s_plan;
 #ifdef MAKO_TIMING_FINISH
     MAKO_WG_TIMER;
 #endif
@@ -184,9 +218,9 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     // (a row without history entries takes the penalising variant too when it has penalties: it finds nothing to
     // penalise, and nothing here waits for the length)
     if (d.hist_tokens && !penalties_neutral(P))
-        slice_partial<VEC, KH, true>(d, sc, row, piece, piece_len, P, hl, slices, L);
+        slice_partial<VEC, KH, true>(d, sc, row, piece, piece_len, P, hl, slices, L, s_plan);
     else
-        slice_partial<VEC, KH, false>(d, sc, row, piece, piece_len, P, hl, slices, L);
+        slice_partial<VEC, KH, false>(d, sc, row, piece, piece_len, P, hl, slices, L, s_plan);
 }
 
 } // namespace mako

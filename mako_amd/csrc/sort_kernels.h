@@ -1,4 +1,4 @@
-// partition_kernel and sort_kernel.
+// sort_kernel.
 #pragma once
 
 #include "worker_sort.h"
@@ -7,98 +7,11 @@
 namespace mako {
 
 #ifdef MAKO_EMIT_SORT_KERNELS // (not templates: defined by the one translation unit that launches them)
-// grid = (kWorkers, rows) workgroups over the same work list as sort_kernel; only planned wide rows do anything.
-// Piece c of a row reads the c-th part of the row's bits(q) array once and hands every weight the plan wants to
-// the worker that will sort it: positions inside the workgroup from LDS counters, one global atomic per worker to
-// reserve the workgroup's run in that worker's share.  (Without this step each of the 32 workers would sweep the
-// whole row to find its own weights.)
-__global__ __launch_bounds__(kThreads) void partition_kernel(mako_sample_desc d, Scratch sc_arg)
-{
-    // (the context's record by value, and loads asked for in groups: a workgroup here lives four microseconds, and
-    // every dependent trip to memory is most of one)
-    const Scratch& sc = sc_arg;
-    __shared__ uint32_t s_count[kWorkers], s_base[kWorkers], s_off[kWorkers], s_cnt[kWorkers];
-    __shared__ uint32_t s_table[kBins / 4];
-    const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
-    // first trip: the list's length and this workgroup's entry of it (the list has room for every workgroup of the
-    // grid; what the entry says is looked at only if the length covers it)
-    const uint32_t n_work = sc.work_n[0];
-    const uint32_t item = sc.work_sort[piece];
-    if (piece >= n_work)
-        return;
-    const uint32_t row = item >> 8, c = item & 255u, tid = threadIdx.x;
-    MAKO_ROW(row);
-    BigPlan* plan = sc.plan + row;
-    const uint32_t V = d.n_vocab;
-    const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
-    uint32_t* kstage = sc.key[1] + (size_t)row * sc.vpad;
-    uint32_t* istage = sc.idx[1] + (size_t)row * sc.vpad;
-    const uint32_t part = (((V + kWorkers - 1u) / kWorkers) + 3u) & ~3u; // entries per piece, a multiple of 4
-    const uint32_t lo = min(V, c * part), hi = min(V, lo + part);
-    // second trip: the row's flag, the piece's first weights, the bin -> worker table and the workers' ranges
-    const uint32_t flag = plan->flag;
-    uint4 x = make_uint4(0, 0, 0, 0);
-    {
-        const uint32_t i = lo + tid * 4u;
-        if (i < hi)
-            x = *reinterpret_cast<const uint4*>(qk + i); // (the array is padded to a multiple of 1024 entries past V)
-    }
-    uint32_t table_word = 0, off_w = 0, cnt_w = 0;
-    if (tid < kBins / 4)
-        table_word = reinterpret_cast<const uint32_t*>(sc.bin_worker + (size_t)row * kBins)[tid];
-    if (tid < kWorkers) {
-        off_w = plan->off[tid];
-        cnt_w = plan->cnt[tid];
-    }
-    if (flag != 1)
-        return;
-    if (tid < kBins / 4)
-        s_table[tid] = table_word;
-    if (tid < kWorkers) {
-        s_count[tid] = 0;
-        s_off[tid] = off_w;
-        s_cnt[tid] = cnt_w;
-    }
-    __syncthreads();
-    const uint8_t* table = reinterpret_cast<const uint8_t*>(s_table);
-    for (uint32_t base = lo; base < hi; base += kThreads * 4u) {
-        const uint32_t i = base + tid * 4u;
-        if (base != lo) {
-            x = make_uint4(0, 0, 0, 0);
-            if (i < hi)
-                x = *reinterpret_cast<const uint4*>(qk + i);
-        }
-        const uint32_t k[4] = {x.x, x.y, x.z, x.w};
-        uint32_t dest[4], lpos[4];
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) {
-            dest[j] = (i + j < hi && k[j] != 0) ? table[weight_bin(k[j])] : 0xffu;
-            lpos[j] = 0;
-            if (dest[j] < kWorkers)
-                lpos[j] = atomicAdd(&s_count[dest[j]], 1u);
-        }
-        __syncthreads();
-        if (tid < kWorkers) {
-            s_base[tid] = s_count[tid] ? atomicAdd(&plan->cursor[tid], s_count[tid]) : 0u;
-            s_count[tid] = 0;
-        }
-        __syncthreads();
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            if (dest[j] < kWorkers) {
-                const uint32_t at = s_base[dest[j]] + lpos[j];
-                if (at < s_cnt[dest[j]] && s_off[dest[j]] + at < V) { // (always, when the plan is sound)
-                    kstage[s_off[dest[j]] + at] = k[j];
-                    istage[s_off[dest[j]] + at] = i + j;
-                }
-            }
-        __syncthreads();
-    }
-}
-
-// grid = (kWorkers, rows) workgroups, of which workgroup i serves entry i of the work list.  Worker w gathers its range of weights from
-// the row's bits(q) array, sorts it and stores it at its place in the row's sorted list; the last worker to
-// finish cuts the nucleus and draws.
+// grid = (kWorkers, rows) workgroups, of which workgroup i serves entry i of the work list.  Worker w sorts the share
+// of the row's weights that the second pass handed it and stores it at its place in the row's sorted list, with
+// the group records tail_kernel works from; worker 0 of a narrow row finishes the row from the candidate lists.
+// What the row's list looks like as a whole (the workers' counts, the exact total) every worker adds up for itself
+// from what the second pass left; worker 0 stores it for tail_kernel.
 __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
 {
     // (the context's record by value: its first loads, the list's length and this workgroup's entry, go out together
@@ -131,13 +44,26 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
     if (tid < 32)
         sm.tab[tid] = k_exp2_tab[tid];
-    const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
     uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
     uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
-    const uint32_t n0 = min(plan->n0, d.n_vocab), groups = min(plan->groups, kMaxGroups);
-    const double total64 = plan->total64;
+    // the row's exact total: the pieces' sums, one per lane, added up in the wave reduction's fixed order; the workers'
+    // counts, and from them this worker's place in the sorted list and in the group records
+    const uint32_t lane = (uint32_t)lane_id();
+    const uint32_t pieces = uniform_u32(sc.work_n[4]);
+    const uint32_t pc = min(lane, pieces - 1u); // pieces <= kMaxSlices = 64
+    const double ps = sc.part_sum[(size_t)row * kMaxSlices + pc];
+    const uint32_t wl = min(lane, kWorkers - 1u);
+    const uint32_t handed = plan->cursor[wl], room = plan->cap[wl];
+    const uint32_t overflow = plan->overflow;
+    const double total64 = __ockl_wfred_add_f64(lane < pieces ? ps : 0.0);
+    const uint32_t cnt_l = lane < kWorkers ? min(handed, room) : 0u;
+    const uint32_t grp_l = (cnt_l + kGroup - 1u) / kGroup;
+    const uint32_t cnt_upto = __ockl_wfscan_add_u32(cnt_l, true), grp_upto = __ockl_wfscan_add_u32(grp_l, true);
+    const uint32_t n0 = (uint32_t)__builtin_amdgcn_readlane((int)cnt_upto, kWave - 1);
+    const uint32_t groups = (uint32_t)__builtin_amdgcn_readlane((int)grp_upto, kWave - 1);
+    const bool spilled = __ballot(lane < kWorkers && handed > room) != 0ull || overflow != 0u;
     if (flag == 3) {
         // narrow nucleus: it should end inside the slices' candidate lists, strictly above everything they left out
         const uint32_t thr_bits = plan->thr;
@@ -168,37 +94,61 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
             sorted_tail(d, row, P, kf, jf, n_list, true, total64, MAKO_PATH_NUCLEUS, L, true, q_bound))
             return;
         // not certifiable from the candidates: tail_kernel's launch takes a second look (narrow_second_look())
-        if (tid == 0)
+        if (tid == 0) {
+            plan->total64 = total64;
             plan->flag = 4;
+        }
         return;
     }
-    uint32_t cnt = plan->cnt[w];
-    const uint32_t off = plan->off[w], gbase = plan->gbase[w];
-    // (a sound plan never trips these; they keep every store of this worker inside the row's arrays)
-    if (off > n0 || cnt > n0 - off || gbase + (cnt + kGroup - 1u) / kGroup > min(groups, sc.g_cap))
-        cnt = 0;
+    // a share that did not fit its room, or a list too long for the group records: the row takes the whole-row path
+    if (spilled || n0 > d.n_vocab || groups > min(kMaxGroups, sc.g_cap)) {
+        __syncthreads();
+        if (w == 0 && tid == 0)
+            plan->flag = 2;
+        return;
+    }
+    if (w == 0 && tid == 0) {
+        plan->n0 = n0;
+        plan->groups = groups;
+        plan->total64 = total64;
+    }
+    const uint32_t cnt = (uint32_t)__builtin_amdgcn_readlane((int)cnt_l, (int)w);
+    const uint32_t off = (uint32_t)__builtin_amdgcn_readlane((int)(cnt_upto - cnt_l), (int)w);
+    const uint32_t gbase = (uint32_t)__builtin_amdgcn_readlane((int)(grp_upto - grp_l), (int)w);
+    const uint32_t stage = plan->stage_off[w];
     const size_t t_row = (size_t)row * sc.g_cap;
     if (cnt) {
-        const uint32_t key_lo = plan->key_lo[w], key_hi = plan->key_hi[w];
+        const uint32_t key_lo = plan->key_lo[w], key_hi = w ? plan->key_lo[w - 1u] : 0x3f800001u; // (just above 1.0)
         MAKO_STAMP(10);
         MAKO_COUNT(31, threadIdx.x == 0 && cnt > kSegCap ? 1 : 0);
         MAKO_COUNT(21, threadIdx.x == 0 ? cnt : 0);
         uint32_t* sorted_copy = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(s_dyn64) + kSortedCopyAt);
         const bool in_lds = cnt <= kSegCap; // uniform
         const bool sorted = in_lds
-                                ? lds_sort_staged(key1 + off, idx1 + off, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm,
+                                ? lds_sort_staged(key1 + stage, idx1 + stage, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm,
                                                   sorted_copy)
-                                : lds_sort_staged_runs(key1 + off, idx1 + off, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm);
+                                : lds_sort_staged_runs(key1 + stage, idx1 + stage, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm);
         if (cnt > kSegCap)
             MAKO_STAMP(18);
         if (!sorted) {
+            // (crowded value buckets: the radix sort through device memory, on a copy of the share at its place in
+            // the list, with the share's own room in the staging arrays as the second buffer; stable, so the token
+            // ids are put in order first)
             MAKO_STAMP(17);
             MAKO_COUNT(23, threadIdx.x == 0 ? 1 : 0);
-            gather_range(qk, d.n_vocab, key_lo, key_hi, key0 + off, idx0 + off, cnt, sm);
-            sort_segment(key0 + off, idx0 + off, key1 + off, idx1 + off, cnt, L);
+            for (uint32_t i = tid; i < cnt; i += kThreads) {
+                key0[off + i] = ~key1[stage + i];
+                idx0[off + i] = idx1[stage + i];
+            }
+            __syncthreads();
+            sort_segment(idx0 + off, key0 + off, idx1 + stage, key1 + stage, cnt, L);
+            sort_segment(key0 + off, idx0 + off, key1 + stage, idx1 + stage, cnt, L);
         }
         MAKO_STAMP(11);
-        worker_groups(key0, off, cnt, t_row + gbase, plan->mass[w], sc.gt, L, (in_lds && sorted) ? sorted_copy : nullptr);
+        // (the guess of the running sum before the share: the plan's estimate, in the exact total's units)
+        const double mass_all = plan->mass_all;
+        worker_groups(key0, off, cnt, t_row + gbase, mass_all > 0.0 ? plan->mass[w] * (total64 / mass_all) : 0.0, sc.gt, L,
+                      (in_lds && sorted) ? sorted_copy : nullptr);
         MAKO_STAMP(12);
     }
 }

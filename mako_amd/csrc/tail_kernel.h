@@ -42,6 +42,8 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         finish_late_row(s_args.d, s_args.sc, s_args.P, r, slices, Lr);
         return;
     }
+    if (threadIdx.x < 32)
+        sm.tab[threadIdx.x] = k_exp2_tab[threadIdx.x]; // (for the whole-row path, should the row need it)
     const uint32_t n_work = sc_arg.work_n[1];
     const uint32_t row = sc_arg.work_tail[blockIdx.y], tid = threadIdx.x; // (the list has room for every workgroup)
     if (blockIdx.y >= n_work)
@@ -50,6 +52,8 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     const BigPlan* planned = sc_arg.plan + row;
     const uint32_t flag = planned->flag, plan_n0 = planned->n0, plan_groups = planned->groups;
     const double total64 = planned->total64;
+    const float plan_m = planned->m;
+    const uint32_t plan_argidx = planned->argidx;
     if (flag != 1)
         return;
     stage_args(d_arg, sc_arg, row, s_args);
@@ -67,15 +71,11 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         plan->flag = 0;
     const uint32_t* kf = sc.key[0] + (size_t)row * sc.vpad;
     const uint32_t* jf = sc.idx[0] + (size_t)row * sc.vpad;
-    if (sorted_tail<true>(d, row, s_args.P, kf, jf, n0, true, total64, MAKO_PATH_GENERAL, L, false, 0.0f, sc.gt,
+    if (sorted_tail<true>(d, row, s_args.P, kf, jf, n0, true, total64, MAKO_PATH_SORTED, L, false, 0.0f, sc.gt,
                           (size_t)row * sc.g_cap, groups))
         return;
-    // too close to call: the reference's total, over the row's bits(q) array (index order; the zeros of the logits
-    // that are no candidates add nothing), decides (the list reaches far enough below the cut for it: plan_nucleus()
-    // takes the band along)
-    const uint32_t* qk = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
-    const double total = reference_total([=](uint32_t i) { return __uint_as_float(qk[i]); }, d.n_vocab, sm);
-    sorted_tail_exact<true>(d, row, s_args.P, kf, jf, n0, total, MAKO_PATH_GENERAL, L, sc.gt, (size_t)row * sc.g_cap, groups);
+    // too close to call, or the list ends before the nucleus does: the whole-row path decides
+    general_row<0>(d, sc, row, s_args.P, plan_m, plan_argidx, L);
 }
 #endif // MAKO_EMIT_TAIL_KERNEL
 

@@ -152,7 +152,6 @@ __device__ uint32_t sort_candidates(const Scratch& sc, uint32_t row, uint32_t sl
     return block_sum_u32(nv, sm.bs); // (its barriers publish kf / jf)
 }
 
-constexpr uint32_t kSmall = 256; // lists of up to this many entries are ordered by counting ranks
 
 // Fast route for rows that need only a few of their candidates.  Every thread weights up to four candidates;
 // those at or above a weight threshold (at most kSmall of them) are ordered by (q desc, idx asc) by counting, for
