@@ -25,6 +25,7 @@ struct alignas(16) CoarsePlan {
     double mass_all;
     uint32_t count[kWorkers]; // hand-over: this workgroup's entries for each worker, and where its run starts
     uint32_t base[kWorkers];
+    uint32_t lbase[kWorkers + 1]; // and in the workgroup's own ordering of what it keeps
     uint32_t flag, thr, n0_est, pad;
 };
 

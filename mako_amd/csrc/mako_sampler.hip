@@ -370,11 +370,10 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     const size_t lds = d.hist_tokens ? (size_t)slice_len * sizeof(uint32_t) : 0;
     // (scan_kernel: with histories a row's slices share an XCD)
     const dim3 grid = d.hist_tokens ? dim3((d.n_rows + 7u) & ~7u, slices) : dim3(slices, d.n_rows);
-    // The second pass cuts top_k == 0 rows into pieces of one to four blocks of 4096 logits (decided on the device:
-    // pieces finer than slices only while all of them fit one round of workgroups), so this many workgroups can
-    // have work; the others leave after a look at the rows' parameters.
-    const uint32_t pieces_max = std::min<uint32_t>(mako::kMaxSlices, std::max(slices, (d.n_vocab + 4095u) / 4096u));
-    const uint32_t finish_wgs = std::max(d.n_rows * slices, std::min(ctx->cus, d.n_rows * pieces_max));
+    // The second pass's cut is decided on the device (SecondPassCut): at most one round of workgroups while the rows'
+    // pieces fit one, else one workgroup per row or a few; workgroups beyond those with work leave after a look at
+    // the cut.
+    const uint32_t finish_wgs = std::max(d.n_rows, ctx->cus);
     // histories of up to 2 (8) entries per thread stay in registers; longer ones take the generic route
     const int kh = !d.hist_tokens ? 2 : (d.hist_stride <= 2 * mako::kThreads ? 2 : (d.hist_stride <= 8 * mako::kThreads ? 8 : 0));
     const bool prof = ctx->profile;

@@ -68,16 +68,16 @@ struct SliceStat {
 // scale = kLogUnitsPerOctave * log2(e) / T: one unit is 1/kLogUnitsPerOctave of a factor of two of the weight the
 // logit will have, and the unit is a function of the logit and the row's temperature alone.  scan_kernel counts each
 // slice's penalised logits by unit, in the frame of the slice's own maximum: one bin per unit for the kLogFine units
-// at and below the maximum's (near-flat rows, whose weights all lie within a factor of two, still spread over a
-// hundred bins), one bin per aligned group of 2^kLogCoarseShift units below that (36 octaves in all; what lies
+// at and below the maximum's (near-flat rows, whose weights all lie within a factor of two, still spread over
+// hundreds of bins), one bin per aligned group of 2^kLogCoarseShift units below that (34 octaves in all; what lies
 // further down is not counted).  Units and groups are absolute, so the second pass can move every slice's counts
 // into the frame of the row's maximum with integer arithmetic alone, exactly, and size its work from them before it
 // has computed a single weight.  Nothing exact is ever decided from these counts: they balance work and size buffers,
 // and every list built from them is checked against the exact sums afterwards.
 constexpr uint32_t kLogBins = 1024;
-constexpr uint32_t kLogUnitsPerOctave = 128;
+constexpr uint32_t kLogUnitsPerOctave = 256;
 constexpr uint32_t kLogFine = 512;
-constexpr uint32_t kLogCoarseShift = 3;
+constexpr uint32_t kLogCoarseShift = 4;
 __device__ __forceinline__ float log_unit_scale(const mako_sampling_params& P)
 {
     return (1.0f / P.temperature) * (1.4426950408889634f * (float)kLogUnitsPerOctave);
@@ -170,8 +170,7 @@ struct Scratch {
     // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
     // (finish_kernel and plan_kernel get the same effect from find_piece().)
     uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); then, 16-byte aligned at [4],
-                           // the second pass's pieces per top_k == 0 row, their length and the number of workgroups
-                           // with work (scan_kernel's first workgroup decides, see second_pass_pieces())
+                           // how the second pass is cut up (SecondPassCut; scan_kernel's first workgroup decides)
     uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel
     uint32_t* work_tail;   // [max_rows] row; appended by finish_kernel
     uint64_t vpad;

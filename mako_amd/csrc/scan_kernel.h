@@ -89,10 +89,9 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
         }
     }
     if (row == 0 && slice == 0 && wave_id() == 1) { // how the second pass will be cut up
-        uint32_t piece_len, busy;
-        const uint32_t pieces = second_pass_pieces(d, n_slices, slice_len, cus, piece_len, busy);
+        const SecondPassCut cut = second_pass_cut(d, n_slices, slice_len, cus);
         if (lane_id() == 0)
-            *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(pieces, piece_len, busy, 0u);
+            *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(cut.per_row, cut.piece_len, cut.busy, cut.pieces);
     }
     // ReasoningBudget::forced's question (src/server/openai.cpp:598-602), answered in the same pass over the logits
     bool want_above = false;

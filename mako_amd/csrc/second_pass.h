@@ -8,38 +8,44 @@
 
 namespace mako {
 
-// One piece of a top_k == 0 row: the exact fp64 sum of q over it and the number of candidates in it (q > 0 and
-// q >= min_p), and every weight the row's plan keeps handed to the share of the worker that will sort it.
+// A workgroup's share of a top_k == 0 row's pieces, one after the other.  Of each piece: the exact fp64 sum of q over
+// it and the number of candidates in it (q > 0 and q >= min_p), and every weight the row's plan keeps handed to the
+// share of the worker that will sort it.
 // The summation order is fixed: each thread adds its logits in index order, then lanes, then waves.
-// The plan (coarse_plan()) is built while the piece's logits are on their way; every workgroup of the row arrives at
-// the same one, and the row's first piece stores it for the kernels that follow and enters the row in their lists.
+// The plan (coarse_plan()) is built while the first piece's logits are on their way; every workgroup of the row
+// arrives at the same one, and the one with the row's first piece stores it for the kernels that follow and enters
+// the row in their lists.
 // (PEN: the row has penalties to apply; a compile-time fact so that each case gets straight-line code of its own.)
 // (`slices`: of scan_kernel, whose records give the row maximum)
-template <bool VEC, int KH, bool PEN>
-__device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slice,
-                              uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, uint32_t slices,
-                              const FinishLds& L, CoarsePlan& pl)
+// (PLANNING: the workgroup's first piece, with which the plan is built; returns false when the row leaves for the
+// whole-row path and the pass has nothing more to do for it)
+template <bool VEC, int KH, bool PEN, bool PLANNING>
+__device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slice, uint32_t slice_len,
+                          const mako_sampling_params& P, uint32_t hl, uint32_t slices, const FinishLds& L, CoarsePlan& pl,
+                          float& m, uint32_t& argidx)
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
+    constexpr bool pen = PEN;
+    BigPlan* plan = sc.plan + row;
     const uint32_t lo = slice * slice_len;
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
-    constexpr bool pen = PEN;
     float wv[16];
-    float m = 0.0f;
-    uint32_t argidx = 0;
-    PlanLoads pre;
-    issue_plan_loads(sc, row, slices, pre);
-    load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, [&]() {
-        uint32_t n_cands, any_overflow;
-        row_summary_of(pre.st, slices, m, argidx, n_cands, any_overflow);
-        coarse_plan(sc, row, slices, P, m, pre, !d.draft && !any_overflow && n_cands <= kSortMax, pl, sm.tab);
-    });
+    if constexpr (PLANNING) {
+        PlanLoads pre;
+        issue_plan_loads(sc, row, slices, pre);
+        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, [&]() {
+            uint32_t n_cands, any_overflow;
+            row_summary_of(pre.st, slices, m, argidx, n_cands, any_overflow);
+            coarse_plan(sc, row, slices, P, m, pre, !d.draft && !any_overflow && n_cands <= kSortMax, pl, sm.tab);
+        });
+    } else {
+        load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv);
+    }
     MAKO_STAMP(1);
     MAKO_STAMP(24);
-    BigPlan* plan = sc.plan + row;
     const uint32_t flag = pl.flag;
-    if (slice == 0) {
+    if (PLANNING && slice == 0) {
         // the row's first piece stores the plan and enters the row in the lists of sort_kernel and tail_kernel
         if (tid < kWorkers) {
             plan->key_lo[tid] = pl.key_lo[tid];
@@ -64,7 +70,7 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
         }
     }
     if (flag == 2) // the whole-row path starts from the logits again
-        return;
+        return false;
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
     const uint32_t thr = pl.thr;
@@ -108,25 +114,59 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
     }
     lds_barrier();
     MAKO_STAMP(26);
-    // one run per worker in its share of the row's staging arrays, reserved with a single atomic
-    if (tid < kWorkers)
-        pl.base[tid] = pl.count[tid] ? atomicAdd(&plan->cursor[tid], pl.count[tid]) : 0u;
+    // One run per worker in its share of the row's staging arrays, reserved with a single atomic.  The kept weights
+    // are first put in LDS (the penalty table's block, free by now) in the order of their workers, so that the runs
+    // go out as contiguous stores.
+    if (wave_id() == 0) {
+        const uint32_t mine = tid < kWorkers ? pl.count[tid] : 0u;
+        const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
+        if (tid < kWorkers) {
+            pl.base[tid] = mine ? atomicAdd(&plan->cursor[tid], mine) : 0u;
+            pl.lbase[tid] = upto - mine;
+        }
+        if (tid == kWorkers - 1u)
+            pl.lbase[kWorkers] = upto;
+    }
     __syncthreads();
     MAKO_STAMP(27);
+    if (tid < kWorkers)
+        pl.count[tid] = 0; // (for the workgroup's next piece)
     uint32_t* kstage = sc.key[1] + (size_t)row * sc.vpad;
     uint32_t* istage = sc.idx[1] + (size_t)row * sc.vpad;
-    bool dropped = false;
+    uint2* buf = reinterpret_cast<uint2*>(L.cnt); // [kSliceMax / 2] (weight, token id)
+    constexpr uint32_t kHalf = kSliceMax / 2u;
+    const uint32_t kept = pl.lbase[kWorkers];
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j)
-        if (slot[j] != kNone) {
-            const uint32_t w = slot[j] >> 16, at = pl.base[w] + (slot[j] & 0xffffu);
-            if (at < pl.cap[w]) {
-                kstage[pl.stage_off[w] + at] = qb[j];
-                istage[pl.stage_off[w] + at] = elem_index<VEC>(lo, tid, j);
-            } else {
-                dropped = true;
+        if (slot[j] != kNone)
+            slot[j] = pl.lbase[slot[j] >> 16] + (slot[j] & 0xffffu); // (from here on: the entry's place in the order)
+    bool dropped = false;
+    for (uint32_t from = 0; from < kept; from += kHalf) { // (what fits the buffer at a time: usually everything)
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j)
+            if (slot[j] != kNone && slot[j] - from < kHalf)
+                buf[slot[j] - from] = make_uint2(qb[j], elem_index<VEC>(lo, tid, j));
+        lds_barrier();
+#pragma unroll
+        for (uint32_t t = 0; t < kHalf / kThreads; ++t) {
+            const uint32_t e = from + t * kThreads + tid;
+            if (e < kept) { // (uniform per wave but for the last one)
+                uint32_t w = 0; // the worker whose run holds entry e: the last one whose run starts at or before it
+#pragma unroll
+                for (uint32_t step = kWorkers / 2u; step; step >>= 1)
+                    w += pl.lbase[w + step] <= e ? step : 0u;
+                const uint32_t at = pl.base[w] + (e - pl.lbase[w]);
+                if (at < pl.cap[w]) {
+                    const uint2 x = buf[e - from];
+                    kstage[pl.stage_off[w] + at] = x.x;
+                    istage[pl.stage_off[w] + at] = x.y;
+                } else {
+                    dropped = true;
+                }
             }
         }
+        lds_barrier();
+    }
     if (dropped) // (more weights in a range than the counts promised: the row takes the whole-row path)
         plan->overflow = 1;
     if (tid == 0) {
@@ -139,10 +179,26 @@ __device__ void slice_partial(const mako_sample_desc& d, const Scratch& sc, uint
         sc.part_sum[(size_t)row * kMaxSlices + slice] = total;
         sc.part_n[(size_t)row * kMaxSlices + slice] = count;
     }
+    lds_barrier(); // (the waves' sums have been read before the next piece's replace them)
+    return true;
+}
+
+template <bool VEC, int KH, bool PEN>
+__device__ void row_pieces(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t first, uint32_t stride,
+                           uint32_t n_pieces, uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, uint32_t slices,
+                           const FinishLds& L, CoarsePlan& pl)
+{
+    // the workgroup's pieces in turn: first, first + stride, ...
+    float m = 0.0f;
+    uint32_t argidx = 0;
+    if (first >= n_pieces || !one_piece<VEC, KH, PEN, true>(d, sc, row, first, slice_len, P, hl, slices, L, pl, m, argidx))
+        return;
+    for (uint32_t slice = first + stride; slice < n_pieces; slice += stride)
+        one_piece<VEC, KH, PEN, false>(d, sc, row, slice, slice_len, P, hl, slices, L, pl, m, argidx);
 }
 
 // Second pass over the top_k == 0 rows.  grid = (most pieces a row can have, rows) workgroups, of which workgroup i
-// serves the i-th piece of work in row order, second_pass_pieces() per top_k == 0 row (find_piece): the busy
+// serves the i-th share of a row's pieces in row order, SecondPassCut::per_row per top_k == 0 row (find_piece): the busy
 // workgroups are then the first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the
 // mix of rows.
 template <bool VEC, int KH>
@@ -170,7 +226,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     const uint4 cut = *reinterpret_cast<const uint4*>(sc_arg.work_n + 4);
     if (wg >= cut.z)
         return;
-    const uint32_t pieces = cut.x, piece_len = cut.y;
+    const uint32_t pieces = cut.x, piece_len = cut.y, n_pieces = cut.w; // (pieces: workgroups per row)
     uint32_t row, piece;
     if (by_lane) {
         // find_piece() over the parameters already here: one row per lane, every wave for itself
@@ -218,9 +274,9 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     // (a row without history entries takes the penalising variant too when it has penalties: it finds nothing to
     // penalise, and nothing here waits for the length)
     if (d.hist_tokens && !penalties_neutral(P))
-        slice_partial<VEC, KH, true>(d, sc, row, piece, piece_len, P, hl, slices, L, s_plan);
+        row_pieces<VEC, KH, true>(d, sc, row, piece, pieces, n_pieces, piece_len, P, hl, slices, L, s_plan);
     else
-        slice_partial<VEC, KH, false>(d, sc, row, piece, piece_len, P, hl, slices, L, s_plan);
+        row_pieces<VEC, KH, false>(d, sc, row, piece, pieces, n_pieces, piece_len, P, hl, slices, L, s_plan);
 }
 
 } // namespace mako

@@ -51,7 +51,7 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     // the row's exact total: the pieces' sums, one per lane, added up in the wave reduction's fixed order; the workers'
     // counts, and from them this worker's place in the sorted list and in the group records
     const uint32_t lane = (uint32_t)lane_id();
-    const uint32_t pieces = uniform_u32(sc.work_n[4]);
+    const uint32_t pieces = uniform_u32(sc.work_n[7]);
     const uint32_t pc = min(lane, pieces - 1u); // pieces <= kMaxSlices = 64
     const double ps = sc.part_sum[(size_t)row * kMaxSlices + pc];
     const uint32_t wl = min(lane, kWorkers - 1u);

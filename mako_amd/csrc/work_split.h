@@ -5,32 +5,42 @@
 
 namespace mako {
 
-// Into how many pieces finish_kernel cuts each top_k == 0 row, and how long a piece is.  A piece is one to four
-// blocks of 4096 logits (a slice is four): as few blocks as keep all the pieces of the batch within one round of
-// workgroups (`cus` of them run at a time, one per CU), since the pass is bound by instruction issue and more
-// workgroups with less work each finish sooner.  Worked out from the rows' parameters by one wave of scan_kernel's
-// first workgroup and left in Scratch::work_n; batches of more than 64 rows take whole slices.
-__device__ __forceinline__ uint32_t second_pass_pieces(const mako_sample_desc& d, uint32_t slices, uint32_t slice_len,
-                                                       uint32_t cus, uint32_t& piece_len, uint32_t& busy)
+// How finish_kernel cuts each top_k == 0 row into pieces, and how many workgroups share a row's pieces.  A piece is
+// one to four blocks of 4096 logits (a slice is four): as few blocks as keep all the pieces of the batch within one
+// round of workgroups (`cus` of them run at a time, one per CU), since the pass is bound by instruction issue and
+// more workgroups with less work each finish sooner.  A batch with more pieces than that takes whole slices, and as
+// many workgroups per row as keeps it to one round; each of them goes through its share of the row's pieces in turn
+// (and builds the row's plan once, not once per piece).  Worked out from the rows' parameters by one wave of
+// scan_kernel's first workgroup and left in Scratch::work_n.
+struct SecondPassCut {
+    uint32_t per_row;   // workgroups per top_k == 0 row
+    uint32_t piece_len;
+    uint32_t busy;      // workgroups with work
+    uint32_t pieces;    // pieces per row: workgroup g of a row takes the pieces g, g + per_row, ...
+};
+__device__ __forceinline__ SecondPassCut second_pass_cut(const mako_sample_desc& d, uint32_t slices, uint32_t slice_len,
+                                                         uint32_t cus)
 {
-    piece_len = slice_len;
-    busy = d.n_rows * slices; // (no more than that)
-    if (d.n_rows > (uint32_t)kWave)
-        return slices;
-    const uint32_t r = lane_id();
-    const bool nucleus = r < d.n_rows && classify(d.params[r]) == kNucleus;
-    const uint32_t rows = (uint32_t)__popcll(__ballot(nucleus));
-    busy = rows * slices;
+    uint32_t rows = 0; // top_k == 0 rows of the batch (every lane ends up with the count)
+    for (uint32_t base = 0; base < d.n_rows; base += (uint32_t)kWave) {
+        const uint32_t r = base + (uint32_t)lane_id();
+        rows += (uint32_t)__popcll(__ballot(r < d.n_rows && classify(d.params[r]) == kNucleus));
+    }
+    SecondPassCut cut;
+    cut.piece_len = slice_len;
+    cut.pieces = slices;
     for (uint32_t blocks = 1; blocks < 4u; ++blocks) {
         const uint32_t len = blocks * 4096u;
         const uint32_t n = (d.n_vocab + len - 1u) / len;
         if (len < slice_len && n <= kMaxSlices && rows * n <= cus) {
-            piece_len = len;
-            busy = rows * n;
-            return n;
+            cut.piece_len = len;
+            cut.pieces = n;
+            break;
         }
     }
-    return slices;
+    cut.per_row = rows * cut.pieces <= cus ? cut.pieces : min(cut.pieces, max(1u, cus / max(rows, 1u)));
+    cut.busy = rows * cut.per_row;
+    return cut;
 }
 
 // Which piece of work does workgroup `piece` of finish_kernel (per_nucleus = slices, per_other = 1) or of plan_kernel
