@@ -167,7 +167,7 @@ def main():
 
     # per-kernel split of a batch: HIP events recorded by the library on the launch stream, a few extra steps
     ctx.set_profile(True)
-    split = np.zeros(6)
+    split = np.zeros(api.SAMPLER_KERNELS)
     n_split = min(a.steps, 50)
     for i in range(n_split):
         step(a.warmup + a.steps + i)
@@ -269,9 +269,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "bytes_per_launch": batch_bytes,
-                     "kernel": "scan + finish + plan + partition + sort + tail kernels (the six launches of one batch)",
+                     "kernel": "scan + finish + sort + tail kernels (the four launches of one batch)",
                      "launch_ms": ms_per_step,
-                     "kernel_ms": dict(zip(["scan_kernel", "finish_kernel", "plan_kernel", "partition_kernel", "sort_kernel", "tail_kernel"],
+                     "kernel_ms": dict(zip(["scan_kernel", "finish_kernel", "sort_kernel", "tail_kernel"],
                                            [float(x) for x in split])),
                      "scan_kernel_gbs": batch_bytes / (split[0] * 1e-3) / 1e9},
         "host_pointer_rows_per_s": host_rate,

@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libmako_sampler.so")
 MAKO_OK = 0
 MAKO_ERR_INVALID_ARG = -1
 MAKO_ERR_HIP = -2
+SAMPLER_KERNELS = 4  # MAKO_SAMPLER_KERNELS
 PATH_GREEDY, PATH_FALLBACK, PATH_TOPK, PATH_NUCLEUS, PATH_GENERAL, PATH_FORCED, PATH_SORTED = 1, 2, 3, 4, 5, 6, 7
 FORCED_NONE, FORCED_TOKEN, FORCED_CLOSE = 0, 1, 2
 
@@ -165,8 +166,8 @@ class SamplerContext:
             raise MakoError("mako_sampler_set_profile: %d %s" % (rc, self.last_error()))
 
     def kernel_times_ms(self):
-        """(scan, finish, plan, partition, sort, tail) kernel milliseconds of the last batch sampled while profiling was on."""
-        out = (C.c_float * 6)()
+        """(scan, finish, sort, tail) kernel milliseconds of the last batch sampled while profiling was on."""
+        out = (C.c_float * SAMPLER_KERNELS)()
         rc = self.lib.mako_sampler_kernel_times(self.ptr, out)
         if rc != MAKO_OK:
             raise MakoError("mako_sampler_kernel_times: %d %s" % (rc, self.last_error()))

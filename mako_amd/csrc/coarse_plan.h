@@ -74,8 +74,9 @@ __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, co
         if (!v)
             return;
         const int32_t ks = pl.slice_top[s];
-        const int32_t k = tid < kLogFine ? ks - (int32_t)tid
-                                         : (((ks - (int32_t)kLogFine) >> kLogCoarseShift) - (int32_t)(tid - kLogFine)) * (1 << kLogCoarseShift);
+        const int32_t k = tid < kLogFine
+                              ? (int32_t)((uint32_t)ks - tid)
+                              : (int32_t)((uint32_t)(((int32_t)((uint32_t)ks - kLogFine) >> kLogCoarseShift) - (int32_t)(tid - kLogFine)) << kLogCoarseShift);
         const uint32_t b = log_bin_in_frame(k, k_top);
         if (b < kLogBins - 1u)
             atomicAdd(&pl.cnt[b], v);

@@ -407,22 +407,20 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     MAKO_MARK(0);
     MAKO_LAUNCH(mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, sc, slice_len, ctx->cus));
     MAKO_MARK(1);
-    if (any_nucleus)
-        MAKO_LAUNCH(mako::launch_finish(vec, kh, finish_wgs, st, d, sc_dev, slices));
-    MAKO_MARK(2);
     // top_k == 0 rows: planned and handed out by the second pass, sorted, cut and drawn from; the stages talk through
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  A batch without such rows
     // (and without rows for the whole-row path) ends with plan_kernel instead.
+    if (any_nucleus)
+        MAKO_LAUNCH(mako::launch_finish(vec, kh, finish_wgs, st, d, sc_dev, slices));
     if (!launch_sort)
         MAKO_LAUNCH(mako::launch_plan_alone(st, d, sc_dev, slices));
-    MAKO_MARK(3);
-    MAKO_MARK(4);
+    MAKO_MARK(2);
     if (any_nucleus)
         MAKO_LAUNCH(mako::launch_sort(st, d, sc, slices, nucleus_rows));
-    MAKO_MARK(5);
+    MAKO_MARK(3);
     if (launch_sort) // (also finishes every row the kernels before it leave: finish_late_row())
         MAKO_LAUNCH(mako::launch_tail(st, d, sc, slices, nucleus_rows));
-    MAKO_MARK(6);
+    MAKO_MARK(4);
 #undef MAKO_MARK
 #undef MAKO_LAUNCH
     ctx->profiled = prof;

@@ -84,15 +84,19 @@ __device__ __forceinline__ float log_unit_scale(const mako_sampling_params& P)
 }
 __device__ __forceinline__ int32_t log_unit(float logit, float scale)
 {
-    // (NaN and whatever is out of range end up at the limits: the same for every kernel that asks)
-    return (int32_t)floorf(fminf(fmaxf(logit * scale, -1.0e9f), 1.0e9f));
+    // floor and conversion in one instruction that saturates at the limits and turns NaN into 0: the same for every
+    // kernel that asks, which is all that matters here
+    int32_t k;
+    asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(k) : "v"(logit * scale));
+    return k;
 }
 // Bin of unit k in the frame of a maximum whose unit is k_top; kLogBins - 1 and above: not counted.
+// (unsigned arithmetic: units at the limits wrap instead of overflowing, and end up "not counted")
 __device__ __forceinline__ uint32_t log_bin_in_frame(int32_t k, int32_t k_top)
 {
     const uint32_t d = (uint32_t)k_top - (uint32_t)k;
-    const uint32_t c = (uint32_t)(((k_top - (int32_t)kLogFine) >> kLogCoarseShift) - (k >> kLogCoarseShift));
-    return d < kLogFine ? d : (c < kLogBins ? kLogFine + c : kLogBins);
+    const uint32_t c = (uint32_t)(((int32_t)((uint32_t)k_top - kLogFine) >> kLogCoarseShift) - (k >> kLogCoarseShift));
+    return d < kLogFine ? d : (c < kLogBins - 1u - kLogFine ? kLogFine + c : kLogBins);
 }
 // How far below the maximum (its unit k_top) the middle of bin b lies, in units, counted from the maximum's unit's
 // lower edge.
@@ -100,7 +104,7 @@ __device__ __forceinline__ float log_bin_middle(uint32_t b, int32_t k_top)
 {
     if (b < kLogFine)
         return (float)b - 0.5f;
-    const int32_t g = ((k_top - (int32_t)kLogFine) >> kLogCoarseShift) - (int32_t)(b - kLogFine);
+    const int32_t g = ((int32_t)((uint32_t)k_top - kLogFine) >> kLogCoarseShift) - (int32_t)(b - kLogFine);
     return (float)(k_top - g * (1 << kLogCoarseShift) - (1 << (kLogCoarseShift - 1)));
 }
 
@@ -171,7 +175,8 @@ struct Scratch {
     // (finish_kernel and plan_kernel get the same effect from find_piece().)
     uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); then, 16-byte aligned at [4],
                            // how the second pass is cut up (SecondPassCut; scan_kernel's first workgroup decides)
-    uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel
+    uint4* work_sort;      // [max_rows * kWorkers] (row << 8 | plan flag << 5 | worker, where the worker's share starts in
+                           // the staging arrays, the room it has there, 0); appended by finish_kernel
     uint32_t* work_tail;   // [max_rows] row; appended by finish_kernel
     uint64_t vpad;
     uint32_t slices_cap;

@@ -36,8 +36,9 @@ __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 
 // (ABOVE: the batch has close tokens, whose logits' ranks are counted on the way; a variant of its own because the
 // count takes sixteen more registers, up to the limit for two workgroups per CU, which no other batch should pay)
+// (amdgpu_waves_per_eu: the vectorised variants are held to the 64 registers that let two workgroups share a CU)
 template <bool VEC, int KH, bool ABOVE = false>
-__global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scratch sc_arg, uint32_t slice_len,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 8 : 4))) void scan_kernel(mako_sample_desc d, Scratch sc_arg, uint32_t slice_len,
                                                         uint32_t cus)
 {
     // (scan_kernel takes the context's record by value: its first loads then need no trip to memory for a pointer)
@@ -219,7 +220,7 @@ __global__ __launch_bounds__(kThreads) void scan_kernel(mako_sample_desc d, Scra
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j) {
             const uint32_t bin = log_bin_in_frame(log_unit(wv[j], scale), k_top);
-            atomicAdd(&sm.log_hist[bin < kLogBins - 1u ? bin : dump], 1u);
+            atomicAdd(&sm.log_hist[bin < kLogBins ? bin : dump], 1u); // (kLogBins: "not counted")
         }
     }
     __syncthreads();

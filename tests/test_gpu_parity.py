@@ -491,6 +491,46 @@ def test_narrow_nucleus_inside_one_slice(gpu_ctx):
     assert (g["path"] == api.PATH_SORTED).any() and (g["path"] == api.PATH_NUCLEUS).any()
 
 
+def test_plan_with_logits_of_extreme_magnitude(gpu_ctx):
+    """The second pass plans a top_k == 0 row from counts of its logits by weight octave.  Logits so large that the
+    octave arithmetic saturates (everything lands in one bin, or far outside the bins), tiny ones (a near-flat row
+    inside a single bin), infinities and temperatures at the ends of the server's range still give the reference's
+    tokens: the plan only sizes the work, the weights decide."""
+    rng = np.random.default_rng(90210)
+    b, v = 12, 40000
+    base = rng.standard_normal((b, v)).astype(np.float32)
+    scales = np.array([1e9, 1e7, 1e5, 3e3, 1e-3, 1e-6, 1e-30, 3.0, 3.0, 3.0, 1e4, 1e-2], np.float32)
+    logits = (base * scales[:, None]).astype(np.float32)
+    logits[7, ::3] = -np.inf
+    logits[8, 5] = np.inf
+    logits[9] += np.float32(3e38)  # (+inf wherever the sum overflows)
+    p = api.make_params(b, 1.0, 0, 0.9)
+    p["temperature"] = np.array([1.0, 100.0, 1.0, 1.0, 1.0, 1e-3, 1.0, 0.5, 0.7, 1.0, 1e-3, 100.0], np.float32)
+    p["top_p"] = np.array([0.9, 0.5, 0.99, 0.9, 0.9, 0.9, 0.95, 0.9, 0.9, 0.9, 0.9, 0.999], np.float32)
+    w = dict(name="extreme_magnitudes", logits=logits, params=p, u=rng.random(b).astype(np.float32))
+    g = assert_parity(gpu_ctx, w, cap=256)
+    _say("extreme magnitudes: nuclei %s paths %s" % (g["n_cand"].tolist(), g["path"].tolist()))
+
+
+def test_big_batches_with_few_top_p_rows(gpu_ctx):
+    """Batches of more than 64 rows share the second pass's workgroups by the number of top_k == 0 rows: one round of
+    single pieces while they fit, else a few workgroups per row that take their pieces in turn."""
+    v = 40000
+    for b, n_nucleus in ((100, 5), (100, 60), (200, 200), (70, 1)):
+        rng = np.random.default_rng(7000 + b + n_nucleus)
+        w = _random_case(rng, v, b)
+        w["params"]["temperature"] = np.float32(0.9)
+        w["params"]["top_p"] = np.float32(0.97)
+        w["params"]["top_k"] = np.uint32(30)
+        w["params"]["top_k"][rng.permutation(b)[:n_nucleus]] = 0
+        _say("big batch b=%d nucleus rows=%d" % (b, n_nucleus))
+        ctx = api.SamplerContext(max_rows=b, max_vocab=v, max_hist=1024)
+        try:
+            assert_parity(ctx, w, cap=256)
+        finally:
+            ctx.close()
+
+
 @pytest.mark.parametrize("v", [40000, 129280])
 def test_second_pass_piece_sizes(gpu_ctx, v):
     """The second pass over top_k == 0 rows is cut into pieces of one to four 4096-logit blocks depending on how many
