@@ -35,7 +35,7 @@ INLINE_ALL = ["-mllvm", "-amdgpu-function-calls=false"]
 RARE_CALLS = ["-DMAKO_RARE_CALL=__attribute__((noinline))"]
 SOURCE_FLAGS = {
     # the late rows (top-k rows, the whole-row path, second looks at a cut) out of line beside the tails
-    "k_tail.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", *RARE_CALLS],
+    "k_tail.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", "-DMAKO_TOPK_PART=__attribute__((noinline))", *RARE_CALLS],
     # the whole-row path and the second look at a cut that is too close to call, out of line beside the top-k rows
     "k_plan_alone.hip": RARE_CALLS,
 }

@@ -46,12 +46,11 @@ __device__ MAKO_RARE_CALL void narrow_second_look(const mako_sample_desc& d, con
     general_row<0>(d, sc, row, P, m, argidx, L);
 }
 
-// What the earlier kernels leave of row `row`, by one workgroup (all threads call; sm.tab must hold the exp2 table):
-// rows whose token is forced, greedy rows, top-k rows, rows for the whole-row path, second looks.
-__device__ MAKO_RARE_CALL void finish_late_row(const mako_sample_desc& d, const Scratch& sc, const mako_sampling_params& P,
-                                               uint32_t row, uint32_t slices, const FinishLds& L)
+// Rows that need no sampling: a forced token, the argmax of a greedy row.  Returns whether the row was one.  (Out of
+// line: inlined beside the top-k rows' code it costs that code registers.)
+__device__ MAKO_RARE_CALL bool late_plain_row(const mako_sample_desc& d, const Scratch& sc, RowClass cls, uint32_t row,
+                                              uint32_t slices)
 {
-    const RowClass cls = classify(P);
     if (d.force_token || d.close_token) { // uniform
         int32_t ftok;
         uint32_t above;
@@ -71,9 +70,36 @@ __device__ MAKO_RARE_CALL void finish_late_row(const mako_sample_desc& d, const 
                 o.forced = kind;
                 write_row(d, row, o);
             }
-            return;
+            return true;
         }
     }
+    if (cls == kGreedy) { // sampler.cpp:77-78, 88-92
+        float m;
+        uint32_t argidx, n_cands, any_overflow;
+        row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
+        if (threadIdx.x == 0) {
+            RowOut o;
+            o.token = (int32_t)argidx;
+            o.n_cand = 0;
+            o.total = 0.0f;
+            o.q = 0.0f;
+            o.path = MAKO_PATH_GREEDY;
+            o.accepted = d.draft ? (d.draft[row] == (int32_t)argidx) : 0u;
+            write_row(d, row, o);
+        }
+        return true;
+    }
+    return false;
+}
+
+// What the earlier kernels leave of row `row`, by one workgroup (all threads call; sm.tab must hold the exp2 table):
+// rows whose token is forced, greedy rows, top-k rows, rows for the whole-row path, second looks.
+__device__ MAKO_RARE_CALL void finish_late_row(const mako_sample_desc& d, const Scratch& sc, const mako_sampling_params& P,
+                                               uint32_t row, uint32_t slices, const FinishLds& L)
+{
+    const RowClass cls = classify(P);
+    if ((d.force_token || d.close_token || cls == kGreedy) && late_plain_row(d, sc, cls, row, slices))
+        return;
     if (cls == kNucleus) {
         // (the flag is never set for a row whose token is forced: the second pass leaves such a row alone)
         const uint32_t flag = sc.plan[row].flag;
@@ -97,19 +123,6 @@ __device__ MAKO_RARE_CALL void finish_late_row(const mako_sample_desc& d, const 
     uint32_t argidx, n_cands, any_overflow;
     SliceStat lane_stat;
     row_summary(sc, row, slices, m, argidx, n_cands, any_overflow, &lane_stat);
-    if (cls == kGreedy) { // sampler.cpp:77-78, 88-92
-        if (threadIdx.x == 0) {
-            RowOut o;
-            o.token = (int32_t)argidx;
-            o.n_cand = 0;
-            o.total = 0.0f;
-            o.q = 0.0f;
-            o.path = MAKO_PATH_GREEDY;
-            o.accepted = d.draft ? (d.draft[row] == (int32_t)argidx) : 0u;
-            write_row(d, row, o);
-        }
-        return;
-    }
     if (topk_takes_whole_row(cls, any_overflow, n_cands))
         general_row<0>(d, sc, row, P, m, argidx, L);
     else

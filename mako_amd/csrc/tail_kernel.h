@@ -42,8 +42,6 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         finish_late_row(s_args.d, s_args.sc, s_args.P, r, slices, Lr);
         return;
     }
-    if (threadIdx.x < 32)
-        sm.tab[threadIdx.x] = k_exp2_tab[threadIdx.x]; // (for the whole-row path, should the row need it)
     const uint32_t n_work = sc_arg.work_n[1];
     const uint32_t row = sc_arg.work_tail[blockIdx.y], tid = threadIdx.x; // (the list has room for every workgroup)
     if (blockIdx.y >= n_work)
@@ -75,6 +73,10 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
                           (size_t)row * sc.g_cap, groups))
         return;
     // too close to call, or the list ends before the nucleus does: the whole-row path decides
+    __syncthreads();
+    if (tid < 32)
+        sm.tab[tid] = k_exp2_tab[tid];
+    __syncthreads();
     general_row<0>(d, sc, row, s_args.P, plan_m, plan_argidx, L);
 }
 #endif // MAKO_EMIT_TAIL_KERNEL

@@ -9,6 +9,11 @@ namespace mako {
 // Bitonic sort, descending, of 1024 * ITEMS keys held ITEMS per thread: key[t] is element t * 1024 + tid.
 // Partners 1024 or more apart are other registers of the same thread, partners less than 64 apart are lanes
 // of the same wave (shuffles); only the strides in between go through LDS (two barriers each).
+// (MAKO_TOPK_PART: __attribute__((noinline)) in a translation unit whose top-k code sits inside an out-of-line function:
+// each part then has the register file to itself instead of spilling inside its loops)
+#ifndef MAKO_TOPK_PART
+#define MAKO_TOPK_PART
+#endif
 template <int ITEMS>
 __device__ void bitonic_sort_regs(unsigned long long (&key)[ITEMS], unsigned long long* lds)
 {
@@ -134,7 +139,7 @@ __device__ __forceinline__ void keys_from_slots(const CandSlots& c, uint32_t sli
 // The row's candidates (all slices) weighted, sorted by (q desc, idx asc) and left in LDS as kf[i] = ~bits(q_i),
 // jf[i] = token id, invalid ones (q not a candidate) last.  Returns the number of valid candidates.
 template <int ITEMS>
-__device__ uint32_t sort_candidates(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_cands, float m, float inv_t,
+__device__ MAKO_TOPK_PART uint32_t sort_candidates(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_cands, float m, float inv_t,
                                     float floor_q, uint32_t* kf, uint32_t* jf, const FinishLds& L)
 {
     FinishShared& sm = *L.sm;
@@ -162,7 +167,7 @@ __device__ uint32_t sort_candidates(const Scratch& sc, uint32_t row, uint32_t sl
 // Returns the number of entries in the list, or kNone when they exceed kSmall (nothing is written then);
 // n_valid receives the number of candidates that have a weight at all.
 // `pre` (when have_pre): the row's candidate slots as fetch_candidate_slots() loaded them.
-__device__ uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_cands, float m, float inv_t,
+__device__ MAKO_TOPK_PART uint32_t small_candidates(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_cands, float m, float inv_t,
                                      float floor_q, uint32_t top_k, uint32_t thr_bits, uint32_t* kf, uint32_t* jf,
                                      uint32_t& n_valid, const FinishLds& L, bool have_pre = false,
                                      const CandSlots& pre = CandSlots{})
