@@ -175,8 +175,7 @@ struct Scratch {
     // (finish_kernel and plan_kernel get the same effect from find_piece().)
     uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); then, 16-byte aligned at [4],
                            // how the second pass is cut up (SecondPassCut; scan_kernel's first workgroup decides)
-    uint4* work_sort;      // [max_rows * kWorkers] (row << 8 | plan flag << 5 | worker, where the worker's share starts in
-                           // the staging arrays, the room it has there, 0); appended by finish_kernel
+    uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel
     uint32_t* work_tail;   // [max_rows] row; appended by finish_kernel
     uint64_t vpad;
     uint32_t slices_cap;

@@ -63,7 +63,7 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
                 const uint32_t work = flag == 1 ? kWorkers : 1u;
                 const uint32_t at = atomicAdd(&sc.work_n[0], work);
                 for (uint32_t w = 0; w < work; ++w)
-                    sc.work_sort[at + w] = make_uint4((row << 8) | (flag << 5) | w, pl.stage_off[w], pl.cap[w], 0u);
+                    sc.work_sort[at + w] = (row << 8) | w;
                 if (flag == 1)
                     sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
             }

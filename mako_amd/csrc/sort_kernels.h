@@ -22,33 +22,17 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     __shared__ ArgsLds s_args;
     const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
     const uint32_t n_work = sc_arg.work_n[0];
-    const uint4 item = sc_arg.work_sort[piece];
+    const uint32_t item = sc_arg.work_sort[piece];
     if (piece >= n_work)
         return;
 #ifdef MAKO_TIMING_SORT
     MAKO_WG_TIMER;
 #endif
-    const uint32_t row = item.x >> 8, flag = (item.x >> 5) & 7u, w = item.x & 31u, tid = threadIdx.x;
-    const uint32_t stage = item.y, room = item.z;
+    const uint32_t row = item >> 8, w = item & 255u, tid = threadIdx.x;
     MAKO_ROW(row);
+    const uint32_t flag = sc_arg.plan[row].flag;
     if ((flag != 1 && flag != 3) || (flag == 3 && w != 0)) // (never: the list holds exactly the flagged rows' pieces)
         return;
-    // Everything else the worker needs goes out in one trip: what the second pass left of the row as a whole (the
-    // pieces' sums, the workers' counts), the plan's entries for this worker, and the share itself, read up to the
-    // room it was given (how much of that counts is known when the counts arrive).
-    BigPlan* const plan_arg = sc_arg.plan + row;
-    const uint32_t lane = (uint32_t)lane_id();
-    const uint32_t wl = min(lane, kWorkers - 1u);
-    const uint32_t handed = plan_arg->cursor[wl], room_l = plan_arg->cap[wl];
-    const uint32_t overflow = plan_arg->overflow;
-    const uint32_t pieces_raw = sc_arg.work_n[7];
-    const double ps = sc_arg.part_sum[(size_t)row * kMaxSlices + lane]; // (kMaxSlices = 64 sums per row: one per lane)
-    const uint32_t key_lo = plan_arg->key_lo[w], key_hi = w ? plan_arg->key_lo[w - 1u] : 0x3f800001u; // (just above 1.0)
-    const double mass_above = plan_arg->mass[w], mass_all = plan_arg->mass_all;
-    ShareLoads share;
-    const bool share_ok = room <= sc_arg.vpad && stage <= sc_arg.vpad - room && room > 0; // (always, for a sound plan)
-    if (flag == 1 && share_ok)
-        issue_share_loads(sc_arg.key[1] + (size_t)row * sc_arg.vpad + stage, sc_arg.idx[1] + (size_t)row * sc_arg.vpad + stage, room, share);
     stage_args(d_arg, sc_arg, row, s_args);
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
@@ -64,16 +48,22 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
     uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
     uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
-    // the row's exact total: the pieces' sums added up in the wave reduction's fixed order; the workers' counts, and
-    // from them this worker's place in the sorted list and in the group records
+    // the row's exact total: the pieces' sums, one per lane, added up in the wave reduction's fixed order; the workers'
+    // counts, and from them this worker's place in the sorted list and in the group records
+    const uint32_t lane = (uint32_t)lane_id();
+    const uint32_t pieces_raw = sc.work_n[7];
+    const double ps = sc.part_sum[(size_t)row * kMaxSlices + lane]; // (kMaxSlices = 64 sums per row: one per lane)
     const uint32_t pieces = uniform_u32(pieces_raw);
+    const uint32_t wl = min(lane, kWorkers - 1u);
+    const uint32_t handed = plan->cursor[wl], room = plan->cap[wl];
+    const uint32_t overflow = plan->overflow;
     const double total64 = __ockl_wfred_add_f64(lane < pieces ? ps : 0.0);
-    const uint32_t cnt_l = lane < kWorkers ? min(handed, room_l) : 0u;
+    const uint32_t cnt_l = lane < kWorkers ? min(handed, room) : 0u;
     const uint32_t grp_l = (cnt_l + kGroup - 1u) / kGroup;
     const uint32_t cnt_upto = __ockl_wfscan_add_u32(cnt_l, true), grp_upto = __ockl_wfscan_add_u32(grp_l, true);
     const uint32_t n0 = (uint32_t)__builtin_amdgcn_readlane((int)cnt_upto, kWave - 1);
     const uint32_t groups = (uint32_t)__builtin_amdgcn_readlane((int)grp_upto, kWave - 1);
-    const bool spilled = __ballot(lane < kWorkers && handed > room_l) != 0ull || overflow != 0u;
+    const bool spilled = __ballot(lane < kWorkers && handed > room) != 0ull || overflow != 0u;
     if (flag == 3) {
         // narrow nucleus: it should end inside the slices' candidate lists, strictly above everything they left out
         const uint32_t thr_bits = plan->thr;
@@ -111,7 +101,7 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         return;
     }
     // a share that did not fit its room, or a list too long for the group records: the row takes the whole-row path
-    if (spilled || !share_ok || n0 > d.n_vocab || groups > min(kMaxGroups, sc.g_cap)) {
+    if (spilled || n0 > d.n_vocab || groups > min(kMaxGroups, sc.g_cap)) {
         __syncthreads();
         if (w == 0 && tid == 0)
             plan->flag = 2;
@@ -125,15 +115,18 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     const uint32_t cnt = (uint32_t)__builtin_amdgcn_readlane((int)cnt_l, (int)w);
     const uint32_t off = (uint32_t)__builtin_amdgcn_readlane((int)(cnt_upto - cnt_l), (int)w);
     const uint32_t gbase = (uint32_t)__builtin_amdgcn_readlane((int)(grp_upto - grp_l), (int)w);
+    const uint32_t stage = plan->stage_off[w];
     const size_t t_row = (size_t)row * sc.g_cap;
     if (cnt) {
+        const uint32_t key_lo = plan->key_lo[w], key_hi = w ? plan->key_lo[w - 1u] : 0x3f800001u; // (just above 1.0)
         MAKO_STAMP(10);
         MAKO_COUNT(31, threadIdx.x == 0 && cnt > kSegCap ? 1 : 0);
         MAKO_COUNT(21, threadIdx.x == 0 ? cnt : 0);
         uint32_t* sorted_copy = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(s_dyn64) + kSortedCopyAt);
         const bool in_lds = cnt <= kSegCap; // uniform
         const bool sorted = in_lds
-                                ? lds_sort_staged(share, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm, sorted_copy)
+                                ? lds_sort_staged(key1 + stage, idx1 + stage, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm,
+                                                  sorted_copy)
                                 : lds_sort_staged_runs(key1 + stage, idx1 + stage, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm);
         if (cnt > kSegCap)
             MAKO_STAMP(18);
@@ -153,7 +146,8 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         }
         MAKO_STAMP(11);
         // (the guess of the running sum before the share: the plan's estimate, in the exact total's units)
-        worker_groups(key0, off, cnt, t_row + gbase, mass_all > 0.0 ? mass_above * (total64 / mass_all) : 0.0, sc.gt, L,
+        const double mass_all = plan->mass_all;
+        worker_groups(key0, off, cnt, t_row + gbase, mass_all > 0.0 ? plan->mass[w] * (total64 / mass_all) : 0.0, sc.gt, L,
                       (in_lds && sorted) ? sorted_copy : nullptr);
         MAKO_STAMP(12);
     }

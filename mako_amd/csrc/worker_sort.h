@@ -156,25 +156,11 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
     return true;
 }
 
-// A worker's share as the second pass left it (bits(q) in ks and token ids in is, any order), asked for ahead of its
-// exact length: `room` entries may be read, the first `cnt` of them count.
-constexpr uint32_t kSharePer = kSegCap / kThreads;
-struct ShareLoads {
-    uint32_t k[kSharePer], id[kSharePer];
-};
-__device__ __forceinline__ void issue_share_loads(const uint32_t* ks, const uint32_t* is, uint32_t room, ShareLoads& x)
-{
-#pragma unroll
-    for (uint32_t t = 0; t < kSharePer; ++t) { // (all loads first, from clamped positions)
-        const uint32_t e = min(t * kThreads + threadIdx.x, room - 1u);
-        x.k[t] = ks[e];
-        x.id[t] = is[e];
-    }
-}
-
-// The share (cnt <= kSegCap entries, already on their way in `x`) sorted into kout / iout.
-__device__ bool lds_sort_staged(const ShareLoads& x, uint32_t key_lo, uint32_t key_hi, uint32_t cnt, uint32_t* kout,
-                                uint32_t* iout, unsigned long long* dyn, FinishShared& sm, uint32_t* sorted_lds = nullptr)
+// The worker's share as partition_kernel left it (cnt <= kSegCap entries, bits(q) in ks and token ids in is, any
+// order), sorted into kout / iout.
+__device__ bool lds_sort_staged(const uint32_t* ks, const uint32_t* is, uint32_t key_lo, uint32_t key_hi, uint32_t cnt,
+                                uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm,
+                                uint32_t* sorted_lds = nullptr)
 {
     uint2* A = reinterpret_cast<uint2*>(dyn);
     uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
@@ -184,11 +170,19 @@ __device__ bool lds_sort_staged(const ShareLoads& x, uint32_t key_lo, uint32_t k
         hist[b] = 0;
     if (tid == 0)
         sm.flag = 0;
+    constexpr uint32_t kPer = kSegCap / kThreads;
+    uint32_t k[kPer], id[kPer];
 #pragma unroll
-    for (uint32_t t = 0; t < kSharePer; ++t) {
+    for (uint32_t t = 0; t < kPer; ++t) { // (all loads first, from clamped positions)
+        const uint32_t e = min(t * kThreads + tid, cnt - 1u);
+        k[t] = ks[e];
+        id[t] = is[e];
+    }
+#pragma unroll
+    for (uint32_t t = 0; t < kPer; ++t) {
         const uint32_t e = t * kThreads + tid;
         if (e < cnt)
-            A[e] = make_uint2(min(max(x.k[t], key_lo), key_hi - 1u), x.id[t]); // (clamped: a bucket index is always valid)
+            A[e] = make_uint2(min(max(k[t], key_lo), key_hi - 1u), id[t]); // (clamped: a bucket index is always valid)
     }
     __syncthreads();
     return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm, sorted_lds);
