@@ -38,7 +38,7 @@ struct PlanLoads {
 __device__ __forceinline__ void issue_plan_loads(const Scratch& sc, uint32_t row, uint32_t slices, PlanLoads& pre)
 {
     pre.st = sc.stats[(size_t)row * kMaxSlices + min((uint32_t)lane_id(), slices - 1u)];
-    const uint32_t* lh = sc.log_hist + (size_t)row * sc.slices_cap * kLogBins + threadIdx.x;
+    const uint16_t* lh = sc.log_hist + (size_t)row * sc.slices_cap * kLogBins + threadIdx.x;
 #pragma unroll
     for (uint32_t t = 0; t < kPlanSlices; ++t)
         pre.v[t] = lh[(size_t)min(t, slices - 1u) * kLogBins]; // (clamped, not skipped: no branch between the loads)

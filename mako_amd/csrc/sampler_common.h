@@ -166,8 +166,8 @@ struct Scratch {
     uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong; [1] also takes the workers' unsorted
                        // shares (bits(q)) from the second pass
     uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, likewise
-    uint32_t* log_hist;  // [max_rows][slices_cap][kLogBins] top_k == 0 rows: logits of the slice by their distance
-                         // below the slice's own maximum (log_bin_of())
+    uint16_t* log_hist;  // [max_rows][slices_cap][kLogBins] top_k == 0 rows: logits of the slice per bin of the slice's
+                         // own frame (log_bin_in_frame(); a slice holds 16384 logits at most)
     GroupTable gt;     // [max_rows][g_cap] each
     // Work lists.  sort_kernel and tail_kernel are launched with one workgroup per POSSIBLE piece of work, but
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the

@@ -225,8 +225,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 
     }
     __syncthreads();
     MAKO_STAMP(31);
-    if (cls == kNucleus)
-        sc.log_hist[((size_t)row * sc.slices_cap + slice) * kLogBins + tid] = sm.log_hist[tid];
+    if (cls == kNucleus && tid < kLogBins / 2u) { // (two 16-bit counts per store)
+        static_assert(kSliceMax < 65536u, "a bin's count fits sixteen bits");
+        reinterpret_cast<uint32_t*>(sc.log_hist + ((size_t)row * sc.slices_cap + slice) * kLogBins)[tid] =
+            sm.log_hist[2u * tid] | (sm.log_hist[2u * tid + 1u] << 16);
+    }
     if (emits) {
         const uint32_t n = sm.emit_n;
         if (n > kCap)
