@@ -51,8 +51,8 @@ __device__ __forceinline__ void issue_plan_loads(const Scratch& sc, uint32_t row
 // under it falls to 1 - top_p of the estimated total, less a few percent.  The list that results is checked by the
 // exact sums later: a plan that keeps too little costs a second look at the row, never a wrong answer.
 // (Every instruction here is latency of the whole pass: a workgroup's sixteen waves share four SIMDs.)
-__device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, const mako_sampling_params& P, float m,
-                            const PlanLoads& pre, bool narrow_ok, CoarsePlan& pl, const uint64_t* tab)
+__device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_vocab, const mako_sampling_params& P,
+                            float m, const PlanLoads& pre, bool narrow_ok, CoarsePlan& pl, const uint64_t* tab)
 {
     const uint32_t tid = threadIdx.x, lane = (uint32_t)lane_id();
     MAKO_STAMP(10);
@@ -116,7 +116,9 @@ __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, co
     pl.incl[bin] = incl_c;
     // the nucleus ends where what lies below it is 1 - top_p of the total; the estimates of both are good to a few
     // percent of themselves (the bins' widths), whatever top_p is
-    const float tail_allowed = (1.0f - P.top_p) * all_m * 0.94f;
+    // (what the bins do not cover, masked and far-off logits alike, is taken at the weight where the bins end)
+    const float tail_allowed = (1.0f - P.top_p) * all_m * 0.94f -
+                               (float)(n_vocab - min(all_c, n_vocab)) * __builtin_amdgcn_exp2f((log_bin_middle(kLogBins - 2u, k_top) + top_frac) * kPerUnit);
     {
         const unsigned long long bal = __ballot(c != 0 && below_m <= tail_allowed);
         if (lane == 0) // (the highest such bin: the last such thread)

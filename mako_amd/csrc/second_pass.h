@@ -37,7 +37,7 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
         load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, [&]() {
             uint32_t n_cands, any_overflow;
             row_summary_of(pre.st, slices, m, argidx, n_cands, any_overflow);
-            coarse_plan(sc, row, slices, P, m, pre, !d.draft && !any_overflow && n_cands <= kSortMax, pl, sm.tab);
+            coarse_plan(sc, row, slices, d.n_vocab, P, m, pre, !d.draft && !any_overflow && n_cands <= kSortMax, pl, sm.tab);
         });
     } else {
         load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv);

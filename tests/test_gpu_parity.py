@@ -512,6 +512,26 @@ def test_plan_with_logits_of_extreme_magnitude(gpu_ctx):
     _say("extreme magnitudes: nuclei %s paths %s" % (g["n_cand"].tolist(), g["path"].tolist()))
 
 
+def test_plans_hold_for_top_p_close_to_one(gpu_ctx):
+    """The second pass's plan keeps what its coarse counts say the nucleus needs, with a margin on the mass that may be
+    left out.  For top_p up to 0.9999 and temperatures from 0.3 to 3 on Gaussian, spiked and near-flat rows the kept
+    list must reach the nucleus' end: every row is finished from the sorted list or the candidate lists, none by the
+    whole-row path."""
+    rng = np.random.default_rng(2718)
+    b, v = 24, 129280
+    logits = (rng.standard_normal((b, v)) * 3).astype(np.float32)
+    logits[8:16] = (logits[8:16] * 0.03).astype(np.float32)  # near-flat
+    for r in range(16, 24):  # spikes
+        logits[r, rng.integers(0, v, 1 + r)] += np.float32(8.0)
+    p = api.make_params(b, 1.0, 0, 0.9)
+    p["temperature"] = np.tile(np.array([0.3, 0.7, 1.0, 1.3, 2.0, 3.0, 1.0, 0.5], np.float32), 3)
+    p["top_p"] = np.tile(np.array([0.9999, 0.999, 0.99, 0.9999, 0.95, 0.9999, 0.999, 0.9], np.float32), 3)
+    w = dict(name="top_p_near_one", logits=logits, params=p, u=rng.random(b).astype(np.float32))
+    g = assert_parity(gpu_ctx, w, cap=256)
+    _say("top_p near one: nuclei %s paths %s" % (g["n_cand"].tolist(), g["path"].tolist()))
+    assert not (g["path"] == api.PATH_GENERAL).any()
+
+
 def test_big_batches_with_few_top_p_rows(gpu_ctx):
     """Batches of more than 64 rows share the second pass's workgroups by the number of top_k == 0 rows: one round of
     single pieces while they fit, else a few workgroups per row that take their pieces in turn."""
