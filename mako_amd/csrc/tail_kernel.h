@@ -39,6 +39,13 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         Lr.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
         Lr.sortk = s_dyn64;
         Lr.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
+        // (a top_k == 0 row that the workers and the tail above take care of needs nothing here: it leaves before the
+        // call, whose entry alone would store dozens of registers per thread)
+        if (classify(s_args.P) == kNucleus && !(d_arg.force_token || d_arg.close_token)) {
+            const uint32_t late_flag = sc_arg.plan[r].flag;
+            if (late_flag != 2 && late_flag != 4)
+                return;
+        }
         finish_late_row(s_args.d, s_args.sc, s_args.P, r, slices, Lr);
         return;
     }
