@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 #include <math.h>
+#include <stddef.h>
 #include <stdint.h>
 #include <type_traits>
 #include "../../include/mako_sampler.h"
@@ -166,9 +167,11 @@ struct Scratch {
     uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong; [1] also takes the workers' unsorted
                        // shares (bits(q)) from the second pass
     uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, likewise
+    GroupTable gt;     // [max_rows][g_cap] each
+                       // (kept at a multiple of 16 bytes: the kernels' LDS copies of this record are read with
+                       // 128-bit operations, which stall on anything less)
     uint16_t* log_hist;  // [max_rows][slices_cap][kLogBins] top_k == 0 rows: logits of the slice per bin of the slice's
                          // own frame (log_bin_in_frame(); a slice holds 16384 logits at most)
-    GroupTable gt;     // [max_rows][g_cap] each
     // Work lists.  sort_kernel and tail_kernel are launched with one workgroup per POSSIBLE piece of work, but
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
     // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
@@ -181,6 +184,8 @@ struct Scratch {
     uint32_t slices_cap;
     uint32_t g_cap;    // vpad / kGroup + kWorkers
 };
+
+static_assert(offsetof(Scratch, gt) % 16 == 0 && sizeof(mako_sample_desc) % 16 == 0, "128-bit LDS reads of the staged records");
 
 // Device functions that only rare rows reach (the whole-row path, the second look at a cut that is too close to
 // call).  The sources whose kernels have a hot path beside them are compiled with MAKO_RARE_CALL=__attribute__((noinline)):
