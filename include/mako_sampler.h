@@ -161,7 +161,7 @@ int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t
 const char* mako_sampler_last_error(const mako_sampler_ctx* ctx);
 
 /* Per-kernel timing for benchmarks (no counterpart in the reference).  While enabled, every
- * mako_sampler_sample_batch records HIP events on its stream around its six kernels;
+ * mako_sampler_sample_batch records HIP events on its stream around its kernels;
  * mako_sampler_kernel_times waits for the last recorded batch and returns the milliseconds of
  * scan_kernel, finish_kernel (plan_kernel, for a batch that ends with it), sort_kernel and
  * tail_kernel in out_ms[0..3].  Off by default. */

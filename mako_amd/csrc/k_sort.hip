@@ -1,5 +1,4 @@
-// partition_kernel and sort_kernel: the wide rows' weights handed to their workers and sorted; narrow and
-// whole-row rows finished by one worker.
+// sort_kernel: the wide rows' shares sorted by their workers; narrow nuclei finished by one worker.
 #define MAKO_EMIT_SORT_KERNELS
 #include "launch.h"
 #include "sampler_kernels.h"

@@ -213,8 +213,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
 {
     if (!out || max_rows == 0 || max_vocab == 0)
         return MAKO_ERR_INVALID_ARG;
-    // (kMaxSlices slices of kSliceMax logits; one logit fewer so that a histogram bin's count fits its 20 bits)
-    if (mako_sampler_slices(max_vocab) > mako::kMaxSlices || max_vocab >= (1u << (64 - mako::kBinSumBits)))
+    // (kMaxSlices slices of kSliceMax logits)
+    if (mako_sampler_slices(max_vocab) > mako::kMaxSlices)
         return MAKO_ERR_INVALID_ARG;
     mako_sampler_ctx* ctx = new (std::nothrow) mako_sampler_ctx;
     if (!ctx)

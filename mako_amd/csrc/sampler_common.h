@@ -23,34 +23,7 @@ constexpr uint32_t kCap = 512;       // candidates kept per slice
 constexpr uint32_t kTopKFast = 128;  // largest top_k resolved from the per-slice candidates
 constexpr uint32_t kSortMax = 4096;  // candidates the finisher sorts in LDS
 constexpr uint32_t kSmall = 256;     // lists of up to this many entries are ordered by counting ranks
-constexpr uint32_t kDynLds = 65536;  // dynamic LDS of both kernels
-constexpr uint32_t kBins = 2048;     // weight histogram of top_k == 0 rows, see weight_bin()
-constexpr uint32_t kBinSumBits = 44; // a bin's record: count << 44 | sum of 24-bit significands
-
-// Histogram bin of a weight q in (0, 1], by its bits: 128 bins per binade for the eight binades below 1.0 (bins
-// 1024..2047) and 8 per binade for everything smaller, subnormals included (bins 71..1023; bins below 71 stay
-// empty).  Bin edges include every binade boundary, so all weights of a bin share their exponent and the bin's
-// mass is exactly (sum of 24-bit significands) * 2^(exponent - 150).  The fine bins keep near-flat rows, whose
-// weights all lie within a factor of two, spread over all workers.
-constexpr uint32_t kFineFrom = 0x3b810000u; // bits(2^-8) + 0x10000: the top fine bin holds 1.0 alone
-constexpr uint32_t kCoarseShift = 20;       // 8 bins per binade
-constexpr uint32_t kCoarseBase = 1023u - ((kFineFrom - 1u) >> kCoarseShift); // 71
-__device__ __forceinline__ uint32_t weight_bin(uint32_t bits)
-{
-    return bits >= kFineFrom ? min(1024u + ((bits - kFineFrom) >> 16), kBins - 1u) : (bits >> kCoarseShift) + kCoarseBase;
-}
-// Smallest bits(q) of a bin, and one past the largest.
-__device__ __forceinline__ uint32_t bin_lo_key(uint32_t b)
-{
-    if (b >= 1024u)
-        return kFineFrom + ((b - 1024u) << 16);
-    return b > kCoarseBase ? (b - kCoarseBase) << kCoarseShift : 0u;
-}
-__device__ __forceinline__ uint32_t bin_hi_key(uint32_t b)
-{
-    return b + 1u < kBins ? bin_lo_key(b + 1u) : kFineFrom + (1024u << 16); // (just above bits(1.0f))
-}
-
+constexpr uint32_t kDynLds = 65536;  // dynamic LDS of the finishing kernels
 constexpr uint32_t kFlagFirstNan = 1u; // element 0 of the row is NaN (slice 0 only)
 constexpr uint32_t kFlagOverflow = 2u; // more than kCap logits reached the slice's threshold
 constexpr uint32_t kFlagComplete = 4u; // every logit above -inf was emitted

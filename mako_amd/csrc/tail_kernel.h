@@ -12,7 +12,7 @@ namespace mako {
 // plan_kernel: 2.3 us less there, but this kernel's chains then compiled to slower code and lost twice that.)
 // (The context's record by value: with a pointer to it the first loads would have to wait for a trip to memory.  The
 // list's length and this workgroup's entry are asked for together, then everything the row's plan holds.)
-// Workgroups from tail_cap on: workgroup tail_cap + r finishes what plan_kernel<false> and sort_kernel left of row r
+// Workgroups from tail_cap on: workgroup tail_cap + r finishes what the kernels before it left of row r
 // (finish_late_row()), beside the few long tails, on CUs that would otherwise idle.  (That code is kept out of line:
 // inlined, it made this kernel's chains compile to slower code.)
 __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices,

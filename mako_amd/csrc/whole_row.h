@@ -342,7 +342,7 @@ __device__ MAKO_RARE_CALL void compact_candidates(const uint32_t* qb, uint32_t V
 // and draws.  `total64` (when have_total) is the fp64 sum of q over all candidates of the row, of which the list
 // may be only the heaviest part; otherwise it is summed from the list.  The row's bits(q) array (sc.wbuf: bits(q) of
 // every candidate at its index, 0 elsewhere) must be in place.
-// (TOPK_ALONE = false leaves the top-k-without-top-p branch out of the instance inside plan_kernel<true>: that kernel is
+// (TOPK_ALONE = false leaves the top-k-without-top-p branch out of the instance inside plan_kernel: that kernel is
 // only launched for batches whose host copy of the parameters shows a top-p on every sampled row, and the branch's
 // registers would be spilled around the top-k rows' fast path, +3.5 us on a 256-row batch.)
 template <bool TOPK_ALONE>
@@ -393,88 +393,6 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
     const uint32_t* jf = is;
     draw_from_list(
         d, row, [=](uint32_t i) { return __uint_as_float(~kf[i]); }, [=](uint32_t i) { return jf[i]; }, n1, path, sm);
-}
-
-// Copies the weights of the row with key_lo <= bits(q) < key_hi, in index order, to kout / iout (as ~bits(q) and
-// token id).  Wave w owns a contiguous chunk of the row: a counting sweep, one exchange of the 16 wave totals,
-// then a writing sweep in which ranks come from ballots.  Lane l holds entries 4l..4l+3 of each 256-entry group.
-// Returns the number of entries written.
-__device__ uint32_t gather_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, uint32_t key_hi, uint32_t* kout,
-                                 uint32_t* iout, uint32_t cap, FinishShared& sm)
-{
-    const uint32_t lane = lane_id(), wave = wave_id();
-    const uint32_t chunk = ((V + kThreads * 4u - 1u) / (kThreads * 4u)) * kGroup; // per wave, a multiple of 256
-    const uint32_t beg = min(V, wave * chunk), end = min(V, beg + chunk);
-    auto fetch = [&](uint32_t i, uint32_t (&k)[4]) {
-        if (i + 3 < end) {
-            const uint4 x = *reinterpret_cast<const uint4*>(qk + i);
-            k[0] = x.x;
-            k[1] = x.y;
-            k[2] = x.z;
-            k[3] = x.w;
-        } else {
-#pragma unroll
-            for (uint32_t j = 0; j < 4; ++j)
-                k[j] = i + j < end ? qk[i + j] : 0u;
-        }
-#pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            if (k[j] < key_lo || k[j] >= key_hi)
-                k[j] = 0;
-    };
-    uint32_t mine = 0;
-    for (uint32_t base = beg; base < end; base += 4u * kGroup) {
-        uint32_t k[4][4];
-#pragma unroll
-        for (uint32_t u = 0; u < 4; ++u)
-            fetch(base + u * kGroup + lane * 4u, k[u]);
-#pragma unroll
-        for (uint32_t u = 0; u < 4; ++u)
-#pragma unroll
-            for (uint32_t j = 0; j < 4; ++j)
-                mine += k[u][j] != 0;
-    }
-    mine = __ockl_wfred_add_u32(mine);
-    __syncthreads();
-    if (lane == 0)
-        sm.bs.u64[wave] = mine;
-    __syncthreads();
-    uint32_t out = 0, n0 = 0;
-    for (int w = 0; w < kWaves; ++w) {
-        const uint32_t x = (uint32_t)sm.bs.u64[w];
-        if (w < (int)wave)
-            out += x;
-        n0 += x;
-    }
-    const unsigned long long lower = (1ull << lane) - 1ull;
-    for (uint32_t base = beg; base < end; base += 2u * kGroup) {
-        uint32_t k[2][4];
-        fetch(base + lane * 4u, k[0]);
-        fetch(base + kGroup + lane * 4u, k[1]);
-#pragma unroll
-        for (uint32_t u = 0; u < 2; ++u) {
-            uint32_t before = 0, total = 0;
-#pragma unroll
-            for (uint32_t j = 0; j < 4; ++j) {
-                const unsigned long long bal = __ballot(k[u][j] != 0);
-                before += (uint32_t)__popcll(bal & lower);
-                total += (uint32_t)__popcll(bal);
-            }
-            uint32_t pos = out + before;
-#pragma unroll
-            for (uint32_t j = 0; j < 4; ++j)
-                if (k[u][j]) {
-                    if (pos < cap) { // (the caller's count of the range; never exceeded when the plan is sound)
-                        kout[pos] = ~k[u][j];
-                        iout[pos] = base + u * kGroup + lane * 4u + j;
-                    }
-                    ++pos;
-                }
-            out += total;
-        }
-    }
-    __syncthreads();
-    return n0;
 }
 
 // Sorts n (key, id) pairs at (k0, i0) by key ascending, stably, with (k1, i1) as the second buffer; the result

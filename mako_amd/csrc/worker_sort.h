@@ -9,82 +9,10 @@ namespace mako {
 __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, uint32_t* kout, uint32_t* iout,
                                 unsigned long long* dyn, FinishShared& sm, uint32_t* sorted_lds = nullptr);
 
-// Worker's sort, LDS-resident: the weights of the row with key_lo <= bits(q) < key_hi (at most kSegCap of them)
-// are collected from the row's bits(q) array in one sweep, dropped into kFine value buckets (descending), and
-// every entry then finds its place by counting the entries of its own bucket that precede it under
-// (q desc, idx asc).  The sorted range is written to kout / iout as ~bits(q) and token id.  Returns false, having
-// written nothing, when the range does not fit or a bucket is too crowded to be ranked by counting.
-__device__ bool lds_sort_range(const uint32_t* qk, uint32_t V, uint32_t key_lo, uint32_t key_hi, uint32_t cnt, uint32_t* kout,
-                               uint32_t* iout, unsigned long long* dyn, FinishShared& sm)
-{
-    uint2* A = reinterpret_cast<uint2*>(dyn);                       // [kSegCap] (bits(q), idx), any order
-    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);         // [kSegCap] entry of A at each bucket-ordered slot
-    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap);      // [kFine + 1] bucket counts, then bucket starts
-    const uint32_t tid = threadIdx.x, lane = lane_id();
-    if (cnt > kSegCap)
-        return false;
-    for (uint32_t b = tid; b <= kFine; b += kThreads)
-        hist[b] = 0;
-    if (tid == 0) {
-        sm.ticket = 0;
-        sm.flag = 0;
-    }
-    __syncthreads();
-    // 1. collect: a slot range per wave and trip from one LDS atomic
-    for (uint32_t base = 0; base < V; base += 4u * kThreads * 4u) {
-        uint32_t k[4][4];
-#pragma unroll
-        for (uint32_t u = 0; u < 4; ++u) {
-            const uint32_t i = base + u * kThreads * 4u + tid * 4u;
-            if (i + 3 < V) {
-                const uint4 x = *reinterpret_cast<const uint4*>(qk + i);
-                k[u][0] = x.x;
-                k[u][1] = x.y;
-                k[u][2] = x.z;
-                k[u][3] = x.w;
-            } else {
-#pragma unroll
-                for (uint32_t j = 0; j < 4; ++j)
-                    k[u][j] = i + j < V ? qk[i + j] : 0u;
-            }
-        }
-#pragma unroll
-        for (uint32_t u = 0; u < 4; ++u) {
-            // ranks inside the wave from ballots (any order will do), one LDS atomic per wave for the slots
-            uint32_t before = 0, wave_total = 0;
-            const unsigned long long lower = (1ull << lane) - 1ull;
-#pragma unroll
-            for (uint32_t j = 0; j < 4; ++j) {
-                if (k[u][j] < key_lo || k[u][j] >= key_hi)
-                    k[u][j] = 0; // 0 is never a candidate's weight
-                const unsigned long long bal = __ballot(k[u][j] != 0);
-                before += (uint32_t)__popcll(bal & lower);
-                wave_total += (uint32_t)__popcll(bal);
-            }
-            if (wave_total) { // uniform
-                uint32_t slot = 0;
-                if (lane == 0)
-                    slot = atomicAdd(&sm.ticket, wave_total);
-                slot = uniform_u32(slot) + before;
-                const uint32_t i = base + u * kThreads * 4u + tid * 4u;
-#pragma unroll
-                for (uint32_t j = 0; j < 4; ++j)
-                    if (k[u][j]) {
-                        if (slot < kSegCap)
-                            A[slot] = make_uint2(k[u][j], i + j);
-                        ++slot;
-                    }
-            }
-        }
-    }
-    __syncthreads();
-    if (sm.ticket != cnt) // (cannot happen: the plan counted the same array)
-        return false;
-    return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm);
-}
-
-// Second half of the workers' sort: the n entries (bits(q), idx) in LDS at A, all with key_lo <= bits(q) < key_hi,
-// go to kout / iout ordered by (q desc, idx asc).  hist must be zero and sm.flag 0 on entry.
+// The workers' sort in LDS: the n entries (bits(q), idx) in LDS at A, all with key_lo <= bits(q) < key_hi,
+// are dropped into kFine value buckets (descending), and every entry finds its place by counting the entries of its
+// own bucket that precede it under (q desc, idx asc); they go to kout / iout as ~bits(q) and token id.  Returns false
+// when a bucket is too crowded to be ranked by counting.  hist must be zero and sm.flag 0 on entry.
 // sorted_lds (optional, n words of LDS outside the sort's own): receives the sorted ~bits(q) as well, and the
 // function then returns behind a barrier that orders LDS only: the caller goes on from the copy instead of waiting
 // for the stores to kout and reading them back.
@@ -156,7 +84,7 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
     return true;
 }
 
-// The worker's share as partition_kernel left it (cnt <= kSegCap entries, bits(q) in ks and token ids in is, any
+// The worker's share as the second pass left it (cnt <= kSegCap entries, bits(q) in ks and token ids in is, any
 // order), sorted into kout / iout.
 __device__ bool lds_sort_staged(const uint32_t* ks, const uint32_t* is, uint32_t key_lo, uint32_t key_hi, uint32_t cnt,
                                 uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm,

@@ -17,7 +17,7 @@ import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-KERNELS = ("scan_kernel", "finish_kernel", "plan_kernel", "partition_kernel", "sort_kernel", "tail_kernel")
+KERNELS = ("scan_kernel", "finish_kernel", "plan_kernel", "sort_kernel", "tail_kernel")
 
 
 def kernel_sources_digest():
