@@ -5,7 +5,6 @@
 
 namespace mako {
 
-constexpr uint32_t kStageSlack = 64; // room a worker's share gets beyond what the counts promise
 constexpr uint32_t kPlanSlices = 12; // slices whose counts are asked for ahead of the logits (the rest: one more trip)
 
 // Every workgroup of a row builds the same plan (same inputs, same instructions); LDS of its own, beside the
@@ -117,7 +116,7 @@ __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, ui
     // the nucleus ends where what lies below it is 1 - top_p of the total; the estimates of both are good to a few
     // percent of themselves (the bins' widths), whatever top_p is
     // (what the bins do not cover, masked and far-off logits alike, is taken at the weight where the bins end)
-    const float tail_allowed = (1.0f - P.top_p) * all_m * 0.94f -
+    const float tail_allowed = (1.0f - P.top_p) * all_m * 0.9f -
                                (float)(n_vocab - min(all_c, n_vocab)) * __builtin_amdgcn_exp2f((log_bin_middle(kLogBins - 2u, k_top) + top_frac) * kPerUnit);
     {
         const unsigned long long bal = __ballot(c != 0 && below_m <= tail_allowed);
@@ -162,8 +161,23 @@ __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, ui
             fb = (w == 0 || pl.first_bin[w]) ? pl.first_bin[w] : bins_end;
             nb = (w + 1u < kWorkers && pl.first_bin[w + 1u]) ? pl.first_bin[w + 1u] : bins_end;
         }
-        // the lower edge of the worker's weights: the logit at the upper edge of bin nb, as a weight
-        const float edge = m - (log_bin_middle(nb, k_top) + top_frac - 0.5f * (nb < kLogFine ? 1.0f : (float)(1 << kLogCoarseShift))) / scale;
+        // The lower edge of the worker's weights: the weight of the smallest logit whose unit lies above bin nb.
+        // Found exactly (a division, then a few steps from float to float with the very function that made the
+        // bins): the restated expf never falls as its argument rises, so every logit of the share's bins has a
+        // weight at or above this one and every logit of the bins below a weight at or below it; what the bins
+        // promised a worker and what its range of weights brings it then differ only by weights equal to an edge.
+        const int32_t k_edge =
+            nb <= kLogFine ? (int32_t)((uint32_t)k_top - nb + 1u)
+                           : (int32_t)((uint32_t)(((int32_t)((uint32_t)k_top - kLogFine) >> kLogCoarseShift) - (int32_t)(nb - kLogFine) + 1) << kLogCoarseShift);
+        float edge = (float)k_edge / scale;
+        for (int i = 0; i < 6 && log_unit(edge, scale) < k_edge; ++i)
+            edge = nextafterf(edge, INFINITY);
+        for (int i = 0; i < 6; ++i) {
+            const float below = nextafterf(edge, -INFINITY);
+            if (log_unit(below, scale) < k_edge)
+                break;
+            edge = below;
+        }
         const float qe = weight_of(edge, m, inv_t, tab);
         uint32_t key = qe == qe ? __float_as_uint(qe) : 0u; // (positive floats order like their bits)
         for (uint32_t o = 1; o < kWorkers; o <<= 1) { // the edges never rise from one worker to the next

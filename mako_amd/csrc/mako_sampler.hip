@@ -103,7 +103,8 @@ hipError_t layout_scratch(mako::Scratch& sc, mako::Scratch** sc_dev, uint32_t ma
         if (e_ != hipSuccess)                                                                                      \
             return e_;                                                                                             \
     } while (0)
-    sc.vpad = ((uint64_t)max_vocab + 1023u) & ~1023ull;
+    // (a row's arrays: the vocabulary, room for the slack of the workers' shares in the staging arrays, rounded up)
+    sc.vpad = ((uint64_t)max_vocab + max_vocab / 64u + mako::kWorkers * mako::kStageSlack + 1023u) & ~1023ull;
     const size_t rv = (size_t)max_rows * sc.vpad;
     sc.slices_cap = mako_sampler_slices(max_vocab);
     MAKO_TAKE(*sc_dev, 1);

@@ -83,6 +83,8 @@ __device__ __forceinline__ float log_bin_middle(uint32_t b, int32_t k_top)
 }
 
 constexpr uint32_t kWorkers = 32;  // workgroups that share the sort of one wide-nucleus row
+constexpr uint32_t kStageSlack = 64; // room a worker's share of the staging arrays gets beyond what the coarse counts
+                                     // promise (and 1/64 of that count); the rows' arrays are sized to hold it
 constexpr uint32_t kGroup = 256;      // a sorted list is processed in groups of one wave x four entries per lane
 constexpr uint32_t kMaxGroups = 1024; // groups per list
 constexpr uint32_t kSegCap = 6144;    // entries a worker sorts in LDS

@@ -532,6 +532,34 @@ def test_plans_hold_for_top_p_close_to_one(gpu_ctx):
     assert not (g["path"] == api.PATH_GENERAL).any()
 
 
+@pytest.mark.parametrize("v", [257, 4099, 20000])
+def test_shares_hold_what_their_bins_promise(v):
+    """The workers' shares get room for the logits their bins count (plus 1/64 and 64 entries).  Quantised logits
+    (thousands of equal weights per bin), near-flat rows of small vocabularies (where the slack is most of the row)
+    and logits far from zero (coarse float spacing) must not outgrow it: every top_k == 0 row takes the sorted list or
+    the candidate lists, none the whole-row path."""
+    rng = np.random.default_rng(4000 + v)
+    b = 70
+    logits = (rng.standard_normal((b, v)) * 3).astype(np.float32)
+    logits[:24] = (np.round(logits[:24] * 4) / 4).astype(np.float32)       # quantised: many equal weights
+    logits[24:40] = (logits[24:40] * 0.007).astype(np.float32)             # near-flat
+    logits[40:48] += np.float32(1000.0)                                    # coarse float spacing
+    logits[48:56] -= np.float32(50.0)
+    p = api.make_params(b, 1.0, 0, 0.9)
+    p["temperature"] = np.tile(np.array([2.0, 0.5, 1.0, 2.0, 0.3, 2.0, 1.3], np.float32), 10)
+    p["top_p"] = np.tile(np.array([0.999, 0.99, 0.9, 0.5, 0.95], np.float32), 14)
+    w = dict(name="shares_v%d" % v, logits=logits, params=p, u=rng.random(b).astype(np.float32))
+    w["hist"] = rng.integers(0, v, (b, 300)).astype(np.int32)
+    w["hist_len"] = rng.integers(0, 301, b).astype(np.uint32)
+    ctx = api.SamplerContext(max_rows=b, max_vocab=v, max_hist=300)
+    try:
+        g = assert_parity(ctx, w, cap=128)
+        _say("shares v=%d paths %s" % (v, np.bincount(g["path"], minlength=8).tolist()))
+        assert not (g["path"] == api.PATH_GENERAL).any()
+    finally:
+        ctx.close()
+
+
 def test_big_batches_with_few_top_p_rows(gpu_ctx):
     """Batches of more than 64 rows share the second pass's workgroups by the number of top_k == 0 rows: one round of
     single pieces while they fit, else a few workgroups per row that take their pieces in turn."""
