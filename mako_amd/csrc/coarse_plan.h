@@ -72,11 +72,7 @@ __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, ui
     auto add = [&](uint32_t s, uint32_t v) {
         if (!v)
             return;
-        const int32_t ks = pl.slice_top[s];
-        const int32_t k = tid < kLogFine
-                              ? (int32_t)((uint32_t)ks - tid)
-                              : (int32_t)((uint32_t)(((int32_t)((uint32_t)ks - kLogFine) >> kLogCoarseShift) - (int32_t)(tid - kLogFine)) << kLogCoarseShift);
-        const uint32_t b = log_bin_in_frame(k, k_top);
+        const uint32_t b = log_bin_in_frame(log_bin_unit(tid, pl.slice_top[s]), k_top);
         if (b < kLogBins - 1u)
             atomicAdd(&pl.cnt[b], v);
     };
@@ -166,9 +162,7 @@ __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, ui
         // bins): the restated expf never falls as its argument rises, so every logit of the share's bins has a
         // weight at or above this one and every logit of the bins below a weight at or below it; what the bins
         // promised a worker and what its range of weights brings it then differ only by weights equal to an edge.
-        const int32_t k_edge =
-            nb <= kLogFine ? (int32_t)((uint32_t)k_top - nb + 1u)
-                           : (int32_t)((uint32_t)(((int32_t)((uint32_t)k_top - kLogFine) >> kLogCoarseShift) - (int32_t)(nb - kLogFine) + 1) << kLogCoarseShift);
+        const int32_t k_edge = log_bin_upper_edge(nb, k_top);
         float edge = (float)k_edge / scale;
         for (int i = 0; i < 6 && log_unit(edge, scale) < k_edge; ++i)
             edge = nextafterf(edge, INFINITY);

@@ -11,6 +11,7 @@
 #include "block_prims.h"
 #include "device_math.h"
 #include "seqfp.h"
+#include "log_bins.h"
 #include "tuning_stamps.h"
 
 namespace mako {
@@ -38,20 +39,7 @@ struct SliceStat {
     uint32_t pad[2];
 };
 
-// A coarse view of a top_k == 0 row before its weights exist.  A logit's `unit` is floor(logit * scale) with
-// scale = kLogUnitsPerOctave * log2(e) / T: one unit is 1/kLogUnitsPerOctave of a factor of two of the weight the
-// logit will have, and the unit is a function of the logit and the row's temperature alone.  scan_kernel counts each
-// slice's penalised logits by unit, in the frame of the slice's own maximum: one bin per unit for the kLogFine units
-// at and below the maximum's (near-flat rows, whose weights all lie within a factor of two, still spread over
-// hundreds of bins), one bin per aligned group of 2^kLogCoarseShift units below that (34 octaves in all; what lies
-// further down is not counted).  Units and groups are absolute, so the second pass can move every slice's counts
-// into the frame of the row's maximum with integer arithmetic alone, exactly, and size its work from them before it
-// has computed a single weight.  Nothing exact is ever decided from these counts: they balance work and size buffers,
-// and every list built from them is checked against the exact sums afterwards.
-constexpr uint32_t kLogBins = 1024;
-constexpr uint32_t kLogUnitsPerOctave = 256;
-constexpr uint32_t kLogFine = 512;
-constexpr uint32_t kLogCoarseShift = 4;
+// A logit's unit for the coarse counts of log_bins.h.
 __device__ __forceinline__ float log_unit_scale(const mako_sampling_params& P)
 {
     return (1.0f / P.temperature) * (1.4426950408889634f * (float)kLogUnitsPerOctave);
@@ -63,23 +51,6 @@ __device__ __forceinline__ int32_t log_unit(float logit, float scale)
     int32_t k;
     asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(k) : "v"(logit * scale));
     return k;
-}
-// Bin of unit k in the frame of a maximum whose unit is k_top; kLogBins - 1 and above: not counted.
-// (unsigned arithmetic: units at the limits wrap instead of overflowing, and end up "not counted")
-__device__ __forceinline__ uint32_t log_bin_in_frame(int32_t k, int32_t k_top)
-{
-    const uint32_t d = (uint32_t)k_top - (uint32_t)k;
-    const uint32_t c = (uint32_t)(((int32_t)((uint32_t)k_top - kLogFine) >> kLogCoarseShift) - (k >> kLogCoarseShift));
-    return d < kLogFine ? d : (c < kLogBins - 1u - kLogFine ? kLogFine + c : kLogBins);
-}
-// How far below the maximum (its unit k_top) the middle of bin b lies, in units, counted from the maximum's unit's
-// lower edge.
-__device__ __forceinline__ float log_bin_middle(uint32_t b, int32_t k_top)
-{
-    if (b < kLogFine)
-        return (float)b - 0.5f;
-    const int32_t g = ((int32_t)((uint32_t)k_top - kLogFine) >> kLogCoarseShift) - (int32_t)(b - kLogFine);
-    return (float)(k_top - g * (1 << kLogCoarseShift) - (1 << (kLogCoarseShift - 1)));
 }
 
 constexpr uint32_t kWorkers = 32;  // workgroups that share the sort of one wide-nucleus row

@@ -220,7 +220,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j) {
             const uint32_t bin = log_bin_in_frame(log_unit(wv[j], scale), k_top);
-            atomicAdd(&sm.log_hist[bin < kLogBins ? bin : dump], 1u); // (kLogBins: "not counted")
+            atomicAdd(&sm.log_hist[bin != kLogNotCounted ? bin : dump], 1u);
         }
     }
     __syncthreads();

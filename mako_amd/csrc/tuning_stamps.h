@@ -18,11 +18,15 @@ __shared__ uint32_t s_mako_row; // the row this workgroup serves (set by MAKO_RO
         if (threadIdx.x == 0)                                                                                        \
             s_mako_row = (r);                                                                                        \
     } while (0)
+#ifdef MAKO_TIMING_NO_STAMPS // (workgroup timers only: the stamps themselves slow the chains they sit in)
+#define MAKO_STAMP(i) ((void)0)
+#else
 #define MAKO_STAMP(i)                                                                                                \
     do {                                                                                                             \
         if (threadIdx.x == 0 && s_mako_row == 0)                                                                     \
             g_mako_stamp[i] = wall_clock64();                                                                        \
     } while (0)
+#endif
 __device__ unsigned long long g_mako_wg[2][4096];
 struct WgTimer {
     __device__ WgTimer()

@@ -224,6 +224,15 @@ def test_seqfp_host():
     assert " 0 failures" in out, out
 
 
+def test_log_bins_host():
+    """The coarse-bin arithmetic scan_kernel and the second pass share (mako_amd/csrc/log_bins.h): a frame's bins tile
+    the units below its maximum, and a slice's counts move into the frame of the row's maximum exactly."""
+    exe = os.path.join(HERE, "cpu", "log_bins_test")
+    subprocess.run(["g++", "-O2", "-std=c++17", os.path.join(HERE, "cpu", "log_bins_test.cpp"), "-o", exe], check=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and " 0 failures" in out.stdout, out.stdout
+
+
 def test_generation_helpers_known_answers():
     """LoopGuard and LookupDrafter (include/gen/) on the scenarios and numbers of the reference's own tests
     (tests/loop_guard_test.cpp, tests/lookup_test.cpp), plus a brute-force restatement of the loop rule."""
@@ -325,7 +334,7 @@ def test_oracle_under_sanitizers():
     assert out.returncode == 0 and out.stdout.strip().endswith(" 0 failures"), out.stdout + out.stderr
 
 
-@pytest.mark.parametrize("name", ["seqfp_test", "gen_helpers_test"])
+@pytest.mark.parametrize("name", ["seqfp_test", "gen_helpers_test", "log_bins_test"])
 def test_host_code_under_sanitizers(name):
     """The host-side C++ the library shares with its kernels (seqfp.h) and ships (include/gen/), likewise."""
     exe = os.path.join(HERE, "cpu", name + "_san")
