@@ -251,6 +251,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
         stage_params(d_arg.params[row], s_args);
     }
     MAKO_ROW(row);
+    MAKO_WG_TAG((row << 8) | piece | 0x80000000u);
     if (tid < 32)
         sm.tab[tid] = k_exp2_tab[tid];
     __syncthreads(); // (publishes the arguments, the parameters and the table)

@@ -20,57 +20,80 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
-    const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x;
+    const uint32_t piece = blockIdx.y * gridDim.x + blockIdx.x, tid = threadIdx.x;
+    // A workgroup's time here is a chain of round trips to device memory, and each one left out shortens it by half
+    // a microsecond.  Three remain: the work list's entry (with the arguments' copy for LDS), everything of the row's
+    // record (a worker per lane), the worker's share.  (The empty asm statements keep each trip's loads together:
+    // the compiler would let those that only a later branch needs wait for that branch.)
+    ArgWords arg_words;
+    fetch_arg_words(d_arg, sc_arg, arg_words);
     const uint32_t n_work = sc_arg.work_n[0];
+    const uint32_t pieces_raw = sc_arg.work_n[7];
     const uint32_t item = sc_arg.work_sort[piece];
+    const uint64_t tab_word = k_exp2_tab[tid & 31u];
+    asm volatile("" ::"s"(item), "s"(n_work), "s"(pieces_raw), "v"(arg_words.d), "v"(arg_words.sc), "v"(tab_word));
     if (piece >= n_work)
         return;
 #ifdef MAKO_TIMING_SORT
     MAKO_WG_TIMER;
 #endif
-    const uint32_t row = item >> 8, w = item & 255u, tid = threadIdx.x;
+    const uint32_t row = item >> 8, w = item & 255u;
     MAKO_ROW(row);
-    const uint32_t flag = sc_arg.plan[row].flag;
+    const uint32_t lane = (uint32_t)lane_id();
+    const uint32_t wl = min(lane, kWorkers - 1u);
+    const BigPlan* rec = sc_arg.plan + row;
+    const uint32_t flag = rec->flag;
+    const uint32_t overflow = rec->overflow;
+    const uint32_t thr_bits = rec->thr;
+    const double mass_all = rec->mass_all;
+    const uint32_t handed = rec->cursor[wl], room = rec->cap[wl];
+    const uint32_t stage_l = rec->stage_off[wl], key_lo_l = rec->key_lo[wl];
+    const double mass_l = rec->mass[wl];
+    fetch_param_words(d_arg, row, arg_words);
+    const double ps = sc_arg.part_sum[(size_t)row * kMaxSlices + lane]; // (kMaxSlices = 64 sums per row: one per lane)
+    asm volatile("" ::"s"(flag), "s"(overflow), "s"(thr_bits), "v"(handed), "v"(room), "v"(stage_l), "v"(key_lo_l),
+                 "v"(mass_l), "v"(ps), "v"(arg_words.p));
     if ((flag != 1 && flag != 3) || (flag == 3 && w != 0)) // (never: the list holds exactly the flagged rows' pieces)
         return;
-    stage_args(d_arg, sc_arg, row, s_args);
+    // the worker's share sets out as soon as its place is known; the row's sums are added up under it
+    const uint32_t cnt_l = lane < kWorkers ? min(handed, room) : 0u;
+    const uint32_t cnt = flag == 1 ? (uint32_t)__builtin_amdgcn_readlane((int)cnt_l, (int)w) : 0u;
+    MAKO_WG_TAG(cnt | (flag == 1 ? 0x80000000u : 0u));
+    const uint32_t stage = (uint32_t)__builtin_amdgcn_readlane((int)stage_l, (int)w);
+    const uint32_t key_lo = (uint32_t)__builtin_amdgcn_readlane((int)key_lo_l, (int)w);
+    const uint32_t key_hi = w ? (uint32_t)__builtin_amdgcn_readlane((int)key_lo_l, (int)(w - 1u)) : 0x3f800001u; // (just above 1.0)
+    uint32_t* key1 = sc_arg.key[1] + (size_t)row * sc_arg.vpad;
+    uint32_t* idx1 = sc_arg.idx[1] + (size_t)row * sc_arg.vpad;
+    StagedShare share;
+    const bool in_lds = cnt <= kSegCap; // uniform
+    if (cnt && in_lds)
+        fetch_staged_share(key1 + stage, idx1 + stage, cnt, share);
+    place_arg_words(arg_words, s_args);
+    if (tid < 32)
+        sm.tab[tid] = tab_word;
+    lds_barrier(); // (not one that waits for the share)
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
     BigPlan* plan = sc.plan + row;
-    FinishLds L;
-    L.sm = &sm;
-    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
-    L.sortk = s_dyn64;
-    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
-    if (tid < 32)
-        sm.tab[tid] = k_exp2_tab[tid];
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
-    uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
-    uint32_t* idx1 = sc.idx[1] + (size_t)row * sc.vpad;
     // the row's exact total: the pieces' sums, one per lane, added up in the wave reduction's fixed order; the workers'
     // counts, and from them this worker's place in the sorted list and in the group records
-    const uint32_t lane = (uint32_t)lane_id();
-    const uint32_t pieces_raw = sc.work_n[7];
-    const double ps = sc.part_sum[(size_t)row * kMaxSlices + lane]; // (kMaxSlices = 64 sums per row: one per lane)
     const uint32_t pieces = uniform_u32(pieces_raw);
-    const uint32_t wl = min(lane, kWorkers - 1u);
-    const uint32_t handed = plan->cursor[wl], room = plan->cap[wl];
-    const uint32_t overflow = plan->overflow;
     const double total64 = __ockl_wfred_add_f64(lane < pieces ? ps : 0.0);
-    const uint32_t cnt_l = lane < kWorkers ? min(handed, room) : 0u;
     const uint32_t grp_l = (cnt_l + kGroup - 1u) / kGroup;
     const uint32_t cnt_upto = __ockl_wfscan_add_u32(cnt_l, true), grp_upto = __ockl_wfscan_add_u32(grp_l, true);
     const uint32_t n0 = (uint32_t)__builtin_amdgcn_readlane((int)cnt_upto, kWave - 1);
     const uint32_t groups = (uint32_t)__builtin_amdgcn_readlane((int)grp_upto, kWave - 1);
     const bool spilled = __ballot(lane < kWorkers && handed > room) != 0ull || overflow != 0u;
+    MAKO_STAMP(3);
     if (flag == 3) {
         // narrow nucleus: it should end inside the slices' candidate lists, strictly above everything they left out
-        const uint32_t thr_bits = plan->thr;
         __syncthreads();
         if (tid == 0)
             plan->flag = 0;
         const mako_sampling_params& P = s_args.P;
+        const FinishLds L = finish_lds_views(sm, s_dyn64);
         // (the candidate lists are asked for together with the slices' records, as for a top-k row)
         CandSlots pre;
         const bool prefetched = slots_cover(slices); // uniform
@@ -112,21 +135,17 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         plan->groups = groups;
         plan->total64 = total64;
     }
-    const uint32_t cnt = (uint32_t)__builtin_amdgcn_readlane((int)cnt_l, (int)w);
     const uint32_t off = (uint32_t)__builtin_amdgcn_readlane((int)(cnt_upto - cnt_l), (int)w);
     const uint32_t gbase = (uint32_t)__builtin_amdgcn_readlane((int)(grp_upto - grp_l), (int)w);
-    const uint32_t stage = plan->stage_off[w];
     const size_t t_row = (size_t)row * sc.g_cap;
     if (cnt) {
-        const uint32_t key_lo = plan->key_lo[w], key_hi = w ? plan->key_lo[w - 1u] : 0x3f800001u; // (just above 1.0)
         MAKO_STAMP(10);
         MAKO_COUNT(31, threadIdx.x == 0 && cnt > kSegCap ? 1 : 0);
         MAKO_COUNT(21, threadIdx.x == 0 ? cnt : 0);
         uint32_t* sorted_copy = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(s_dyn64) + kSortedCopyAt);
-        const bool in_lds = cnt <= kSegCap; // uniform
+        const FinishLds L = finish_lds_views(sm, s_dyn64);
         const bool sorted = in_lds
-                                ? lds_sort_staged(key1 + stage, idx1 + stage, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm,
-                                                  sorted_copy)
+                                ? lds_sort_staged(share, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm, sorted_copy)
                                 : lds_sort_staged_runs(key1 + stage, idx1 + stage, key_lo, key_hi, cnt, key0 + off, idx0 + off, s_dyn64, sm);
         if (cnt > kSegCap)
             MAKO_STAMP(18);
@@ -146,8 +165,8 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         }
         MAKO_STAMP(11);
         // (the guess of the running sum before the share: the plan's estimate, in the exact total's units)
-        const double mass_all = plan->mass_all;
-        worker_groups(key0, off, cnt, t_row + gbase, mass_all > 0.0 ? plan->mass[w] * (total64 / mass_all) : 0.0, sc.gt, L,
+        const double mass_w = readlane_f64(mass_l, w);
+        worker_groups(key0, off, cnt, t_row + gbase, mass_all > 0.0 ? mass_w * (total64 / mass_all) : 0.0, sc.gt, L,
                       (in_lds && sorted) ? sorted_copy : nullptr);
         MAKO_STAMP(12);
     }

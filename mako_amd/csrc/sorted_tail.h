@@ -487,31 +487,63 @@ __device__ bool exact_span_walk(Keys kf, uint32_t start, uint32_t len, float& r,
 // wave reads the same four entries with one broadcast load and subtracts them in turn, three nanoseconds an entry
 // (the travelling chain of walk_lanes() takes five).  Blocks of 64 blind, then of 16, then entry by entry, as there.
 // Returns true and the position when the walk stops, else false and the new r.
-__device__ __forceinline__ bool walk_lds(const float* sx, uint32_t n, float& r, uint32_t& pos)
+// (The list is read as LDS, not through the generic pointer: generic loads wait for one another in full, and the
+// first subtraction of a block would wait for the block's last entry.)
+typedef __attribute__((address_space(3))) const float LdsFloat;
+typedef float LdsFloat4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bool walk_lds(const float* sx_any, uint32_t n, float& r, uint32_t& pos)
 {
+    LdsFloat* sx = (LdsFloat*)sx_any;
+    typedef const __attribute__((address_space(3))) LdsFloat4* Vec4Ptr;
     float v = r;
     uint32_t base = 0;
+    // Blocks of 64 in two halves, each half's loads issued while the other half is subtracted (the scheduling
+    // barriers keep the loads where they are written: the compiler would otherwise issue each only just before its
+    // use, to save registers, and every fourth subtraction would wait for LDS).  The loads run up to 32 entries past
+    // the block; the staged list has a wave's worth of room behind it.
+    LdsFloat4 xa[8], xb[8];
+    if (kWave <= n) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; ++i)
+            xa[i] = ((Vec4Ptr)sx)[i];
+    }
     for (; base + kWave <= n; base += kWave) {
-        const float4* p = reinterpret_cast<const float4*>(sx + base);
+        Vec4Ptr p = (Vec4Ptr)(sx + base);
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; ++i)
+            xb[i] = p[8u + i];
+        __builtin_amdgcn_sched_barrier(0);
         float t = v;
 #pragma unroll
-        for (uint32_t i = 0; i < kWave / 4u; ++i) {
-            const float4 x = p[i];
-            t -= x.x;
-            t -= x.y;
-            t -= x.z;
-            t -= x.w;
+        for (uint32_t i = 0; i < 8u; ++i) {
+            t -= xa[i].x;
+            t -= xa[i].y;
+            t -= xa[i].z;
+            t -= xa[i].w;
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; ++i)
+            xa[i] = p[16u + i];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; ++i) {
+            t -= xb[i].x;
+            t -= xb[i].y;
+            t -= xb[i].z;
+            t -= xb[i].w;
+        }
+        __builtin_amdgcn_sched_barrier(0);
         if (__ballot(t < 0.0f) != 0ull)
             break; // the walk stops in this block: found below
         v = t;
     }
     for (; base + 16u <= n; base += 16u) {
-        const float4* p = reinterpret_cast<const float4*>(sx + base);
+        const __attribute__((address_space(3))) LdsFloat4* p = (const __attribute__((address_space(3))) LdsFloat4*)(sx + base);
         float t = v;
 #pragma unroll
         for (uint32_t i = 0; i < 4u; ++i) {
-            const float4 x = p[i];
+            const LdsFloat4 x = p[i];
             t -= x.x;
             t -= x.y;
             t -= x.z;
@@ -534,14 +566,50 @@ __device__ __forceinline__ bool walk_lds(const float* sx, uint32_t n, float& r, 
 }
 
 // S plus the first `n` entries of a list staged in LDS as for walk_lds(), added one by one in fp32.
-__device__ __forceinline__ float sum_lds(const float* sx, uint32_t n, float S)
+__device__ __forceinline__ float sum_lds(const float* sx_any, uint32_t n, float S)
 {
+    LdsFloat* sx = (LdsFloat*)sx_any;
+    typedef const __attribute__((address_space(3))) LdsFloat4* Vec4Ptr;
     uint32_t base = 0;
+    // (blocks of 64 in two halves, loads and additions interleaved as in walk_lds())
+    LdsFloat4 xa[8], xb[8];
+    if (kWave <= n) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; ++i)
+            xa[i] = ((Vec4Ptr)sx)[i];
+    }
+    for (; base + kWave <= n; base += kWave) {
+        Vec4Ptr p = (Vec4Ptr)(sx + base);
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; ++i)
+            xb[i] = p[8u + i];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; ++i) {
+            S += xa[i].x;
+            S += xa[i].y;
+            S += xa[i].z;
+            S += xa[i].w;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; ++i)
+            xa[i] = p[16u + i];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (uint32_t i = 0; i < 8u; ++i) {
+            S += xb[i].x;
+            S += xb[i].y;
+            S += xb[i].z;
+            S += xb[i].w;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
     for (; base + 16u <= n; base += 16u) {
-        const float4* p = reinterpret_cast<const float4*>(sx + base);
+        Vec4Ptr p = (Vec4Ptr)(sx + base);
 #pragma unroll
         for (uint32_t i = 0; i < 4u; ++i) {
-            const float4 x = p[i];
+            const LdsFloat4 x = p[i];
             S += x.x;
             S += x.y;
             S += x.z;
@@ -1146,7 +1214,10 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 #endif
     // A walk that will end within a few groups goes through them entry by entry, from a copy in LDS: faster than
     // the groups' maps would be to build.
-    const bool head_walk = reach <= kHeadGroups; // uniform
+#ifndef MAKO_HEAD_WALK_GROUPS
+#define MAKO_HEAD_WALK_GROUPS 8
+#endif
+    const bool head_walk = reach <= MAKO_HEAD_WALK_GROUPS; // uniform
     const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
     if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && !head_walk) {
         // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
@@ -1211,8 +1282,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
                     const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
 #ifdef MAKO_TIMING
-                    if (lane_id() == 0)
-                        g_mako_stamp[21] += 1;
+                    if (lane_id() == 0 && s_mako_row == 0)
+                        g_mako_stamp[24] += 1;
 #endif
                     const uint32_t slot = (pk >> 9) & 0x7fu;
                     if (slot) {
@@ -1294,8 +1365,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 if (tid == 0)
                     G.misc()[3] = 0; // (the quarter records so far are done with: their slots start over)
                 __syncthreads();
+                MAKO_TIC(2);
                 build_group_maps(kf, min(groups, base + (uint32_t)kWave), true, r_here + G.pg()[base], G, wave_id(), kWaves, base);
                 __syncthreads();
+                if (wave_id() == 0) {
+                    MAKO_TOC(2, 25);
+                    MAKO_COUNT(26, 1);
+                }
             }
             if (wave_id() == 0 && !stopped) {
                 const uint32_t gl = min(base + lane_id(), groups - 1u);

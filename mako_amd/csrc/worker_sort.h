@@ -51,6 +51,7 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
             hist[kFine] = total;
     }
     __syncthreads();
+    MAKO_STAMP(14);
     if (sm.flag)
         return false;
 #pragma unroll
@@ -58,6 +59,7 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
         if (bucket[t] != kNone)
             B[hist[bucket[t]] + pib[t]] = (uint16_t)(t * kThreads + tid);
     __syncthreads();
+    MAKO_STAMP(15);
     // 3. rank inside the bucket, and out
 #pragma unroll
     for (uint32_t t = 0; t < kPer; ++t) {
@@ -85,10 +87,24 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
 }
 
 // The worker's share as the second pass left it (cnt <= kSegCap entries, bits(q) in ks and token ids in is, any
-// order), sorted into kout / iout.
-__device__ bool lds_sort_staged(const uint32_t* ks, const uint32_t* is, uint32_t key_lo, uint32_t key_hi, uint32_t cnt,
-                                uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm,
-                                uint32_t* sorted_lds = nullptr)
+// order): asked for with fetch_staged_share() (the loads stay in flight while the caller goes on), sorted into
+// kout / iout by lds_sort_staged().
+struct StagedShare {
+    uint32_t k[kSegCap / kThreads], id[kSegCap / kThreads];
+};
+__device__ __forceinline__ void fetch_staged_share(const uint32_t* ks, const uint32_t* is, uint32_t cnt, StagedShare& s)
+{
+    const GlobalKeys gk{ks}, gi{is};
+#pragma unroll
+    for (uint32_t t = 0; t < kSegCap / kThreads; ++t) { // (all loads first, from clamped positions; cnt > 0)
+        const uint32_t e = min(t * kThreads + threadIdx.x, cnt - 1u);
+        s.k[t] = gk[e];
+        s.id[t] = gi[e];
+    }
+}
+__device__ __forceinline__ bool lds_sort_staged(const StagedShare& s, uint32_t key_lo, uint32_t key_hi, uint32_t cnt,
+                                                uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm,
+                                                uint32_t* sorted_lds = nullptr)
 {
     uint2* A = reinterpret_cast<uint2*>(dyn);
     uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
@@ -98,21 +114,16 @@ __device__ bool lds_sort_staged(const uint32_t* ks, const uint32_t* is, uint32_t
         hist[b] = 0;
     if (tid == 0)
         sm.flag = 0;
-    constexpr uint32_t kPer = kSegCap / kThreads;
-    uint32_t k[kPer], id[kPer];
 #pragma unroll
-    for (uint32_t t = 0; t < kPer; ++t) { // (all loads first, from clamped positions)
-        const uint32_t e = min(t * kThreads + tid, cnt - 1u);
-        k[t] = ks[e];
-        id[t] = is[e];
-    }
-#pragma unroll
-    for (uint32_t t = 0; t < kPer; ++t) {
+    for (uint32_t t = 0; t < kSegCap / kThreads; ++t) {
         const uint32_t e = t * kThreads + tid;
+        uint32_t k = s.k[t];
+        asm volatile("" : "+v"(k)); // (used here and not before: the loads are to be waited for no earlier)
         if (e < cnt)
-            A[e] = make_uint2(min(max(k[t], key_lo), key_hi - 1u), id[t]); // (clamped: a bucket index is always valid)
+            A[e] = make_uint2(min(max(k, key_lo), key_hi - 1u), s.id[t]); // (clamped: a bucket index is always valid)
     }
     __syncthreads();
+    MAKO_STAMP(13);
     return lds_bucket_sort(cnt, key_lo, key_hi, kout, iout, dyn, sm, sorted_lds);
 }
 
@@ -255,7 +266,7 @@ __device__ bool lds_sort_staged_runs(const uint32_t* ks, const uint32_t* is, uin
 // maps of the running fp32 sum for the epoch guessed from the mass above the range plus the sums before the group.
 // kf_lds (optional): the worker's cnt sorted weights in LDS (outside L.sortk's first 16 KB), read instead of kf + off.
 __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, size_t t_at, double mass, const GroupTable& T,
-                              const FinishLds& L, const uint32_t* kf_lds = nullptr)
+                              const FinishLds L, const uint32_t* kf_lds = nullptr)
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
@@ -274,29 +285,49 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
         if (lane_id() == 0)
             gs[g] = s;
     }
-    __syncthreads();
-    for (uint32_t g0 = 0; g0 < groups; g0 += kThreads) { // (one trip unless the range is the fallback's)
-        const uint32_t g = g0 + tid;
-        const double v = g < groups ? gs[g] : 0.0;
-        double all;
-        const double incl = block_incl_scan_f64(v, all, sm.bs);
-        if (g < groups) {
-            T.sum[t_at + g] = v;
-            gs[g] = mass + (incl - v);
-            ge[g] = mass + incl;
+    MAKO_STAMP(16);
+    // the sums before and after each group.  Up to a wave's worth of groups, every wave scans them for itself (the
+    // values are those of the workgroup's scan, whose first wave adds them up the same way) and goes on at once.
+    const bool few = groups <= (uint32_t)kWave; // uniform
+    double before_l = 0, after_l = 0; // (few: lane g holds group g's)
+    if (few) {
+        if (kf_lds)
+            lds_barrier();
+        else
+            __syncthreads();
+        const uint32_t gq = (uint32_t)lane_id();
+        const double v = gq < groups ? gs[gq] : 0.0;
+        const double incl = __ockl_wfscan_add_f64(v, true);
+        if (wave_id() == 0 && gq < groups)
+            T.sum[t_at + gq] = v;
+        before_l = mass + (incl - v);
+        after_l = mass + incl;
+    } else {
+        __syncthreads();
+        for (uint32_t g0 = 0; g0 < groups; g0 += kThreads) {
+            const uint32_t g = g0 + tid;
+            const double v = g < groups ? gs[g] : 0.0;
+            double all;
+            const double incl = block_incl_scan_f64(v, all, sm.bs);
+            if (g < groups) {
+                T.sum[t_at + g] = v;
+                gs[g] = mass + (incl - v);
+                ge[g] = mass + incl;
+            }
+            mass += all;
         }
-        mass += all;
+        __syncthreads();
     }
-    __syncthreads();
+    MAKO_STAMP(19);
     for (uint32_t g = wave_id(); g < groups; g += kWaves) {
         const uint32_t len = min(kGroup, cnt - g * kGroup);
         float q[4];
         load_span(src, g * kGroup, len, q);
-        const double guess = gs[g];
+        const double guess = few ? readlane_f64(before_l, g) : gs[g];
         const int eg = guess > 0 ? exponent_of((float)guess) : 0;
         const seqfp::Step32 st = span_map(q, len, eg);
         // the sum is expected to change binade inside the group (or starts at zero): records for its quarters
-        const double at_end = ge[g];
+        const double at_end = few ? readlane_f64(after_l, g) : ge[g];
         const bool split4 = uniform_u32((uint32_t)(eg == 0 || exponent_of((float)at_end) != eg)) != 0;
         if (split4)
             build_quarters(q, len, guess, T.quarters + (t_at + g) * 4u);
