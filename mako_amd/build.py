@@ -32,7 +32,7 @@ INLINE_ALL = ["-mllvm", "-amdgpu-function-calls=false"]
 # Per source (a source listed here is compiled WITHOUT INLINE_ALL): code that only rare rows reach is called, not
 # inlined, where it would cost a hot path registers and spills.  Such kernels use scratch memory for the calls, which
 # slows down the start of their workgroups: not for kernels that many workgroups run (sort_kernel: +15 %).
-RARE_CALLS = ["-DMAKO_RARE_CALL=__attribute__((noinline))"]
+RARE_CALLS = ["-DMAKO_RARE_CALL=__attribute__((noinline))", "-DMAKO_REAL_CALLS=1"]
 SOURCE_FLAGS = {
     # the late rows (top-k rows, the whole-row path, second looks at a cut) out of line beside the tails
     "k_tail.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", "-DMAKO_TOPK_PART=__attribute__((noinline))", *RARE_CALLS],

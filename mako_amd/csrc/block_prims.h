@@ -35,6 +35,21 @@ __device__ __forceinline__ int wave_id()
     return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 }
 
+// Pointers known to point to device memory, typed so.  A pointer that was itself loaded from memory (the finishing
+// kernels keep copies of their argument records in LDS) could point anywhere for all the compiler knows, and accesses
+// through it become "flat" instructions: those count as LDS traffic as well, so a barrier that orders LDS only
+// (lds_barrier()) would wait for every load from device memory still in flight, and the counters of the two kinds
+// of traffic can no longer be waited for one by one.
+template <typename T>
+using global_ptr = __attribute__((address_space(1))) T*;
+template <typename T>
+__device__ __forceinline__ global_ptr<T> as_global(T* p)
+{
+    return (global_ptr<T>)p;
+}
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4))); // (plain vector types: they load from any address space)
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
 // global load, which would serialise LDS set-up work behind the logits stream it is meant to overlap.
 __device__ __forceinline__ void lds_barrier()

@@ -36,8 +36,8 @@ struct PlanLoads {
 };
 __device__ __forceinline__ void issue_plan_loads(const Scratch& sc, uint32_t row, uint32_t slices, PlanLoads& pre)
 {
-    pre.st = sc.stats[(size_t)row * kMaxSlices + min((uint32_t)lane_id(), slices - 1u)];
-    const uint16_t* lh = sc.log_hist + (size_t)row * sc.slices_cap * kLogBins + threadIdx.x;
+    pre.st = load_slice_stat(sc.stats, (size_t)row * kMaxSlices + min((uint32_t)lane_id(), slices - 1u));
+    const global_ptr<const uint16_t> lh = as_global(sc.log_hist) + (size_t)row * sc.slices_cap * kLogBins + threadIdx.x;
 #pragma unroll
     for (uint32_t t = 0; t < kPlanSlices; ++t)
         pre.v[t] = lh[(size_t)min(t, slices - 1u) * kLogBins]; // (clamped, not skipped: no branch between the loads)
@@ -81,7 +81,7 @@ __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, ui
         if (t < slices)
             add(t, pre.v[t]);
     for (uint32_t s = kPlanSlices; s < slices; ++s)
-        add(s, sc.log_hist[((size_t)row * sc.slices_cap + s) * kLogBins + tid]);
+        add(s, as_global(sc.log_hist)[((size_t)row * sc.slices_cap + s) * kLogBins + tid]);
     lds_barrier();
     MAKO_STAMP(3);
     // Running mass and count from the LOWEST bin up (thread t takes bin kLogBins - 1 - t): the mass below a bin, which

@@ -15,6 +15,7 @@ namespace mako {
 __device__ MAKO_RARE_CALL void narrow_second_look(const mako_sample_desc& d, const Scratch& sc, const mako_sampling_params& P,
                                                   uint32_t row, const FinishLds& L)
 {
+    assume_lds(L);
     BigPlan* plan = sc.plan + row;
     const uint32_t handed = plan->cursor[0], room = plan->cap[0], overflow = plan->overflow;
     const double total = plan->total64;
@@ -97,6 +98,7 @@ __device__ MAKO_RARE_CALL bool late_plain_row(const mako_sample_desc& d, const S
 __device__ MAKO_RARE_CALL void finish_late_row(const mako_sample_desc& d, const Scratch& sc, const mako_sampling_params& P,
                                                uint32_t row, uint32_t slices, const FinishLds& L)
 {
+    assume_lds(L);
     const RowClass cls = classify(P);
     if ((d.force_token || d.close_token || cls == kGreedy) && late_plain_row(d, sc, cls, row, slices))
         return;

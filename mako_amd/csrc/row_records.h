@@ -31,7 +31,7 @@ __device__ __forceinline__ void row_summary(const Scratch& sc, uint32_t row, uin
                                             uint32_t& n_cands, uint32_t& any_overflow, SliceStat* lane_stat = nullptr)
 {
     // lane s of every wave takes slice s (at most kMaxSlices = 64 of them): one load each, then wave reductions
-    const SliceStat st = sc.stats[(size_t)row * kMaxSlices + min((uint32_t)lane_id(), slices - 1u)];
+    const SliceStat st = load_slice_stat(sc.stats, (size_t)row * kMaxSlices + min((uint32_t)lane_id(), slices - 1u));
     if (lane_stat)
         *lane_stat = st;
     row_summary_of(st, slices, m, argidx, n_cands, any_overflow);

@@ -39,6 +39,23 @@ struct SliceStat {
     uint32_t pad[2];
 };
 
+// A slice's record from device memory (two 128-bit loads through a pointer typed as device memory, see as_global()).
+__device__ __forceinline__ SliceStat load_slice_stat(const SliceStat* stats, size_t i)
+{
+    static_assert(sizeof(SliceStat) == 32, "two 128-bit loads");
+    const global_ptr<const u32x4> sp = (global_ptr<const u32x4>)(as_global(stats) + i);
+    const u32x4 s0 = sp[0], s1 = sp[1];
+    SliceStat st;
+    st.wmax = __uint_as_float(s0.x);
+    st.argidx = s0.y;
+    st.flags = s0.z;
+    st.n_emit = s0.w;
+    st.tau_key = s1.x;
+    st.above = s1.y;
+    st.pad[0] = st.pad[1] = 0;
+    return st;
+}
+
 // A logit's unit for the coarse counts of log_bins.h.
 __device__ __forceinline__ float log_unit_scale(const mako_sampling_params& P)
 {

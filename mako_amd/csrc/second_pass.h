@@ -24,6 +24,7 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
                           const mako_sampling_params& P, uint32_t hl, uint32_t slices, const FinishLds& L, CoarsePlan& pl,
                           float& m, uint32_t& argidx)
 {
+    assume_lds(L);
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
     constexpr bool pen = PEN;
@@ -131,8 +132,8 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
     MAKO_STAMP(27);
     if (tid < kWorkers)
         pl.count[tid] = 0; // (for the workgroup's next piece)
-    uint32_t* kstage = sc.key[1] + (size_t)row * sc.vpad;
-    uint32_t* istage = sc.idx[1] + (size_t)row * sc.vpad;
+    const global_ptr<uint32_t> kstage = as_global(sc.key[1]) + (size_t)row * sc.vpad;
+    const global_ptr<uint32_t> istage = as_global(sc.idx[1]) + (size_t)row * sc.vpad;
     uint2* buf = reinterpret_cast<uint2*>(L.cnt); // [kSliceMax / 2] (weight, token id)
     constexpr uint32_t kHalf = kSliceMax / 2u;
     const uint32_t kept = pl.lbase[kWorkers];
@@ -176,8 +177,8 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
             total += sm.bs.f64[w];
             count += (uint32_t)sm.bs.u64[w];
         }
-        sc.part_sum[(size_t)row * kMaxSlices + slice] = total;
-        sc.part_n[(size_t)row * kMaxSlices + slice] = count;
+        as_global(sc.part_sum)[(size_t)row * kMaxSlices + slice] = total;
+        as_global(sc.part_n)[(size_t)row * kMaxSlices + slice] = count;
     }
     lds_barrier(); // (the waves' sums have been read before the next piece's replace them)
     return true;
@@ -188,6 +189,7 @@ __device__ void row_pieces(const mako_sample_desc& d, const Scratch& sc, uint32_
                            uint32_t n_pieces, uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, uint32_t slices,
                            const FinishLds& L, CoarsePlan& pl)
 {
+    assume_lds(L);
     // the workgroup's pieces in turn: first, first + stride, ...
     float m = 0.0f;
     uint32_t argidx = 0;
@@ -271,7 +273,7 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
             return;
     }
     // (the history's length and, inside slice_partial, the history, the logits and the slices' records: one trip)
-    const uint32_t hl = d.hist_tokens ? min(d.hist_len[row], (uint32_t)d.hist_stride) : 0u;
+    const uint32_t hl = d.hist_tokens ? min(as_global(d.hist_len)[row], (uint32_t)d.hist_stride) : 0u;
     // (a row without history entries takes the penalising variant too when it has penalties: it finds nothing to
     // penalise, and nothing here waits for the length)
     if (d.hist_tokens && !penalties_neutral(P))

@@ -24,8 +24,8 @@ __device__ __forceinline__ void build_counts(const mako_sample_desc& d, uint32_t
     for (uint32_t i = tid; i < slice_len / 4; i += kThreads)
         z[i] = make_uint4(0, 0, 0, 0);
     __syncthreads();
-    const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
-    const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
+    const global_ptr<const int32_t> ht = as_global(d.hist_tokens) + (int64_t)row * d.hist_stride;
+    const global_ptr<const uint32_t> hc = d.hist_counts ? as_global(d.hist_counts) + (int64_t)row * d.hist_stride : nullptr;
     for (uint32_t h = tid; h < hl; h += kThreads) {
         const uint32_t t = (uint32_t)ht[h];
         if (t >= lo && t < hi)
@@ -46,8 +46,8 @@ template <bool VEC>
 __device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row, uint32_t lo, uint32_t hi, RawSlice<VEC>& r)
 {
     const uint32_t tid = threadIdx.x;
-    const float* lrow = d.logits + (int64_t)row * d.logits_stride;
-    const uint32_t* mrow = d.mask ? d.mask + (int64_t)row * d.mask_stride : nullptr;
+    const global_ptr<const float> lrow = as_global(d.logits) + (int64_t)row * d.logits_stride;
+    const global_ptr<const uint32_t> mrow = d.mask ? as_global(d.mask) + (int64_t)row * d.mask_stride : nullptr;
     const float nan = __uint_as_float(0x7fc00000u);
     if (VEC) {
         // all four loads go out back to back, from clamped addresses and without a branch between them (a branch
@@ -57,7 +57,8 @@ __device__ __forceinline__ void load_raw(const mako_sample_desc& d, uint32_t row
         for (uint32_t k = 0; k < 4; ++k) {
             const uint32_t i = lo + k * 4096u + tid * 4u;
             at[k] = i < hi ? i : hi - 4u; // hi - lo is a positive multiple of 4 in this mode
-            r.v[k] = *reinterpret_cast<const float4*>(lrow + at[k]);
+            const f32x4 x = *(global_ptr<const f32x4>)(lrow + at[k]);
+            r.v[k] = make_float4(x.x, x.y, x.z, x.w);
         }
         if (mrow) {
 #pragma unroll
@@ -215,8 +216,8 @@ __device__ __forceinline__ void load_penalised(const mako_sample_desc& d, uint32
     // Whether they are asked for depends on the kernel's arguments alone, not on the row's parameters or its history
     // length (`hl`, `pen`): a caller may still be waiting for those when these loads and the logits' go out.
     const bool may_penalise = KH > 0 && d.hist_tokens != nullptr && d.hist_stride > 0; // uniform
-    const int32_t* ht = d.hist_tokens + (int64_t)row * d.hist_stride;
-    const uint32_t* hc = d.hist_counts ? d.hist_counts + (int64_t)row * d.hist_stride : nullptr;
+    const global_ptr<const int32_t> ht = as_global(d.hist_tokens) + (int64_t)row * d.hist_stride;
+    const global_ptr<const uint32_t> hc = d.hist_counts ? as_global(d.hist_counts) + (int64_t)row * d.hist_stride : nullptr;
     uint32_t tok[KH > 0 ? KH : 1], cnt[KH > 0 ? KH : 1];
     bool have[KH > 0 ? KH : 1];
     if (may_penalise) {

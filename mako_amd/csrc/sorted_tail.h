@@ -35,6 +35,7 @@ constexpr uint32_t kSeqMax = 1024; // sorted lists up to this long get their tot
 
 __device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
 {
+    assume_lds(L);
     static_assert((kMaxGroups + 2) * 8 + 5 * kMaxGroups * 4 + 16 <= kSortMax * 8, "group records fit below the LDS lists");
     static_assert(kQuarterSlots * 16 == 1536 &&
                       kSortMax * 8 + 1536 * 4 + 4 * kMaxGroups * 4 + (kWalkSeqGroups * kGroup + kWave) * 4 <= kDynLds,
@@ -805,6 +806,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                             const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, const GroupTable& T = GroupTable{},
                             size_t t_base = 0, uint32_t t_groups = 0)
 {
+    assume_lds(L);
     constexpr bool exact = EXACT;
     using namespace seqfp;
     // (a planned row's list is in device memory; the other callers may hand over a list in LDS)
@@ -1481,6 +1483,7 @@ __device__ MAKO_RARE_CALL void sorted_tail_exact(const mako_sample_desc& d, uint
                                                  uint32_t path, const FinishLds& L, const GroupTable& T = GroupTable{},
                                                  size_t t_base = 0, uint32_t t_groups = 0)
 {
+    assume_lds(L);
     sorted_tail<PLANNED, false, true>(d, row, P, kf, jf, n1, true, total64, path, L, false, 0.0f, T, t_base, t_groups);
 }
 

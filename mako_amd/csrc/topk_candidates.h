@@ -80,12 +80,14 @@ __device__ __forceinline__ void candidate_keys(const Scratch& sc, uint32_t row, 
     }
     float w[ITEMS];
     uint32_t id[ITEMS];
+    const global_ptr<const float> cand_w = as_global(sc.cand_w);
+    const global_ptr<const uint32_t> cand_i = as_global(sc.cand_i);
 #pragma unroll
     for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t)
-        w[t] = sc.cand_w[at[t]];
+        w[t] = cand_w[at[t]];
 #pragma unroll
     for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t)
-        id[t] = sc.cand_i[at[t]];
+        id[t] = cand_i[at[t]];
 #pragma unroll
     for (uint32_t t = 0; t < (uint32_t)ITEMS; ++t) {
         key[t] = 0;
@@ -113,10 +115,12 @@ __device__ __forceinline__ void fetch_candidate_slots(const Scratch& sc, uint32_
     static_assert(kCap == (uint32_t)kPrefetchItems * 128u && kThreads == 1024, "eight slices of 128 threads, four entries each");
     const uint32_t sl = min(threadIdx.x >> 7, slices - 1u), i0 = threadIdx.x & 127u;
     const size_t base = ((size_t)row * sc.slices_cap + sl) * kCap + i0;
+    const global_ptr<const float> cand_w = as_global(sc.cand_w);
+    const global_ptr<const uint32_t> cand_i = as_global(sc.cand_i);
 #pragma unroll
     for (uint32_t t = 0; t < (uint32_t)kPrefetchItems; ++t) {
-        c.w[t] = sc.cand_w[base + 128u * t];
-        c.id[t] = sc.cand_i[base + 128u * t];
+        c.w[t] = cand_w[base + 128u * t];
+        c.id[t] = cand_i[base + 128u * t];
     }
 }
 // (sm.soff as candidate_bound() leaves it)
@@ -142,6 +146,7 @@ template <int ITEMS>
 __device__ MAKO_TOPK_PART uint32_t sort_candidates(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_cands, float m, float inv_t,
                                     float floor_q, uint32_t* kf, uint32_t* jf, const FinishLds& L)
 {
+    assume_lds(L);
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
     unsigned long long key[ITEMS];
@@ -172,6 +177,7 @@ __device__ MAKO_TOPK_PART uint32_t small_candidates(const Scratch& sc, uint32_t 
                                      uint32_t& n_valid, const FinishLds& L, bool have_pre = false,
                                      const CandSlots& pre = CandSlots{})
 {
+    assume_lds(L);
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
     uint32_t* hist = reinterpret_cast<uint32_t*>(L.sortk);             // [512]
@@ -299,6 +305,7 @@ __device__ __forceinline__ void topk_row(const mako_sample_desc& d, const Scratc
                                          const SliceStat& lane_stat, const FinishLds& L, bool have_pre = false,
                                          const CandSlots& pre = CandSlots{})
 {
+    assume_lds(L);
     FinishShared& sm = *L.sm;
     // ---- top-k rows: weights of the row's candidates, sorted by (q desc, idx asc) in LDS ----
     const float inv_t = 1.0f / P.temperature;

@@ -26,6 +26,7 @@ __device__ __forceinline__ unsigned long long match_digit(uint32_t digit, bool v
 __device__ bool radix_pass(const uint32_t* ksrc, const uint32_t* isrc, uint32_t* kdst, uint32_t* idst, uint32_t n,
                            uint32_t shift, const FinishLds& L)
 {
+    assume_lds(L);
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x, lane = lane_id(), wave = wave_id();
     const uint32_t chunk = ((n + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
@@ -275,6 +276,7 @@ __device__ bool introselect_rounds(Get get, Put put, uint32_t& first, uint32_t& 
 __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32_t nth, uint32_t* lsta, uint32_t* lstb,
                                 const FinishLds& L)
 {
+    assume_lds(L);
     typedef unsigned long long u64;
     const uint32_t tid = threadIdx.x;
     if (n == 0 || nth >= n)
@@ -349,6 +351,7 @@ template <bool TOPK_ALONE>
 __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
                                    uint32_t n0, bool have_total, double total64, uint32_t path, const FinishLds& L)
 {
+    assume_lds(L);
     FinishShared& sm = *L.sm;
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
     uint32_t* key1 = sc.key[1] + (size_t)row * sc.vpad;
@@ -399,6 +402,7 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
 // ends in (k0, i0).
 __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t* i1, uint32_t n, const FinishLds& L)
 {
+    assume_lds(L);
     if (n < 2)
         return;
     uint32_t *ks = k0, *is = i0, *kd = k1, *id = i1;
@@ -431,6 +435,7 @@ template <int SITE>
 __device__ MAKO_RARE_CALL void general_row(const mako_sample_desc& d, const Scratch& sc, uint32_t row, const mako_sampling_params& P,
                             float m, uint32_t argidx, const FinishLds& L)
 {
+    assume_lds(L);
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
     const uint32_t V = d.n_vocab;

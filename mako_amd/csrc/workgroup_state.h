@@ -25,6 +25,23 @@ struct FinishLds {
     uint32_t* wcount;           // [kWaves * 256]
 };
 
+// The views as a function that is really called (not inlined) received them by reference, said to the compiler to
+// point into LDS: through pointers that could point anywhere every access becomes a "flat" instruction, which takes
+// longer than an LDS one and counts as traffic to device memory as well, so that waiting for one kind means waiting
+// for both.  Only in sources compiled with calls (MAKO_REAL_CALLS): where everything is inlined the compiler sees
+// where the views come from, and the assumption's own loads would only keep the record in memory.
+__device__ __forceinline__ void assume_lds(const FinishLds& L)
+{
+#if defined(MAKO_REAL_CALLS) && defined(__HIP_DEVICE_COMPILE__)
+    __builtin_assume(__builtin_amdgcn_is_shared(L.sm));
+    __builtin_assume(__builtin_amdgcn_is_shared(L.cnt));
+    __builtin_assume(__builtin_amdgcn_is_shared(L.sortk));
+    __builtin_assume(__builtin_amdgcn_is_shared(L.wcount));
+#else
+    (void)L;
+#endif
+}
+
 __device__ __forceinline__ FinishLds finish_lds_views(FinishShared& sm, unsigned long long* dyn)
 {
     FinishLds L;
