@@ -212,23 +212,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 
         }
     }
     if (cls == kNucleus) {
-        // the slice's logits by unit, in the frame of the slice's maximum (log_bin_in_frame()); what the bins do not
-        // cover (and NaN) goes to a slot of the lane's own
+        // the slice's logits by unit, in the frame of the slice's maximum (log_slot_in_frame()); what the bins do not
+        // cover (and NaN) goes to slot kLogBins - 1, which is no bin, or to one of the spare slots up to the lane's own
         const float scale = log_unit_scale(P);
         const int32_t k_top = log_unit(st.wmax, scale);
-        const uint32_t dump = kLogBins + (uint32_t)lane_id();
+        const uint32_t spare_end = kLogBins + (uint32_t)lane_id();
 #pragma unroll
-        for (uint32_t j = 0; j < 16; ++j) {
-            const uint32_t bin = log_bin_in_frame(log_unit(wv[j], scale), k_top);
-            atomicAdd(&sm.log_hist[bin != kLogNotCounted ? bin : dump], 1u);
-        }
+        for (uint32_t j = 0; j < 16; ++j)
+            atomicAdd(&sm.log_hist[log_slot_in_frame(log_unit(wv[j], scale), k_top, spare_end)], 1u);
     }
     __syncthreads();
     MAKO_STAMP(31);
     if (cls == kNucleus && tid < kLogBins / 2u) { // (two 16-bit counts per store)
         static_assert(kSliceMax < 65536u, "a bin's count fits sixteen bits");
+        // (slot kLogBins - 1 took logits that no bin covers: it is stored as zero)
         reinterpret_cast<uint32_t*>(sc.log_hist + ((size_t)row * sc.slices_cap + slice) * kLogBins)[tid] =
-            sm.log_hist[2u * tid] | (sm.log_hist[2u * tid + 1u] << 16);
+            sm.log_hist[2u * tid] | (2u * tid + 1u < kLogBins - 1u ? sm.log_hist[2u * tid + 1u] << 16 : 0u);
     }
     if (emits) {
         const uint32_t n = sm.emit_n;

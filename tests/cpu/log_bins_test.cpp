@@ -31,6 +31,12 @@ static void check_frame(int32_t k_top)
     bool seen_uncounted = false;
     for (int32_t k = k_top; k > k_top - kUnitsCovered - 40; --k) {
         const uint32_t b = log_bin_in_frame(k, k_top);
+        {
+            // the counting form: the bin itself, or a slot from kLogBins - 1 to the end of the spare ones
+            const uint32_t spare_end = kLogBins + (uint32_t)(k & 63);
+            const uint32_t s = log_slot_in_frame(k, k_top, spare_end);
+            CHECK(b == kLogNotCounted ? (s >= kLogBins - 1u && s <= spare_end) : s == b, "top %d unit %d: slot %u, bin %u", k_top, k, s, b);
+        }
         if (b == kLogNotCounted) {
             if (!seen_uncounted)
                 first_uncounted = k;
