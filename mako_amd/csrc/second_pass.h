@@ -75,6 +75,7 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
     const uint32_t thr = pl.thr;
+    const uint32_t edge7 = uniform_u32(pl.key_lo[7]), edge15 = uniform_u32(pl.key_lo[15]), edge23 = uniform_u32(pl.key_lo[23]);
     double sum = 0;
     uint32_t n = 0;
     uint32_t qb[16];   // bits(q), 0 where q is not a candidate
@@ -95,9 +96,12 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
             if (qb[j] >= thr && qb[j]) {
                 // the worker whose range of bits(q) holds the weight (equal weights always meet in one share): the
                 // number of workers whose lower edge lies above it, by bisection over the edges
-                uint32_t w = 0;
+                // (the first two steps against edges held in scalar registers, the other three from LDS)
+                static_assert(kWorkers == 32, "five steps");
+                uint32_t w = qb[j] < edge15 ? 16u : 0u;
+                w += qb[j] < (w ? edge23 : edge7) ? 8u : 0u;
 #pragma unroll
-                for (uint32_t step = kWorkers / 2u; step; step >>= 1)
+                for (uint32_t step = 4u; step; step >>= 1)
                     w += qb[j] < pl.key_lo[w + step - 1u] ? step : 0u;
                 slot[j] = (w << 16) | atomicAdd(&pl.count[w], 1u);
             }
