@@ -7,11 +7,11 @@
 namespace mako {
 void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices)
 {
-    hipLaunchKernelGGL(plan_kernel, dim3(1, d.n_rows), dim3(kThreads), kDynLds, st, d, sc, slices);
+    hipLaunchKernelGGL(plan_kernel, dim3(1, d.n_rows), dim3(kThreads), kTailLds, st, d, sc, slices);
 }
 
 hipError_t init_plan_alone()
 {
-    return hipFuncSetAttribute((const void*)plan_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLds);
+    return hipFuncSetAttribute((const void*)plan_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTailLds);
 }
 } // namespace mako

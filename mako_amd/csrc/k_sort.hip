@@ -11,7 +11,7 @@ void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, u
 
 hipError_t init_sort_kernels()
 {
-    static_assert(kSortLds >= kDynLds, "sort_kernel's tail uses the finishing kernels' LDS layout");
+    static_assert(kSortLds >= kTailLds, "sort_kernel's tail uses the finishing kernels' LDS layout");
     return hipFuncSetAttribute((const void*)sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSortLds);
 }
 } // namespace mako

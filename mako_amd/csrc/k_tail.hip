@@ -6,11 +6,11 @@
 namespace mako {
 void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t tail_cap)
 {
-    hipLaunchKernelGGL(tail_kernel, dim3(1, tail_cap + d.n_rows), dim3(kThreads), kDynLds, st, d, sc, slices, tail_cap);
+    hipLaunchKernelGGL(tail_kernel, dim3(1, tail_cap + d.n_rows), dim3(kThreads), kTailLds, st, d, sc, slices, tail_cap);
 }
 
 hipError_t init_tail_kernels()
 {
-    return hipFuncSetAttribute((const void*)tail_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLds);
+    return hipFuncSetAttribute((const void*)tail_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTailLds);
 }
 } // namespace mako

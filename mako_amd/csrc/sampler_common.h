@@ -24,7 +24,9 @@ constexpr uint32_t kCap = 512;       // candidates kept per slice
 constexpr uint32_t kTopKFast = 128;  // largest top_k resolved from the per-slice candidates
 constexpr uint32_t kSortMax = 4096;  // candidates the finisher sorts in LDS
 constexpr uint32_t kSmall = 256;     // lists of up to this many entries are ordered by counting ranks
-constexpr uint32_t kDynLds = 65536;  // dynamic LDS of the finishing kernels
+constexpr uint32_t kDynLds = 65536;  // dynamic LDS of the second pass (and the most scan_kernel takes)
+constexpr uint32_t kHeadGroups = 32; // groups at the head of a sorted list that tail code keeps in LDS as floats
+constexpr uint32_t kTailLds = kDynLds + (kHeadGroups - 8u) * 1024u; // dynamic LDS of the kernels that cut and draw
 constexpr uint32_t kFlagFirstNan = 1u; // element 0 of the row is NaN (slice 0 only)
 constexpr uint32_t kFlagOverflow = 2u; // more than kCap logits reached the slice's threshold
 constexpr uint32_t kFlagComplete = 4u; // every logit above -inf was emitted

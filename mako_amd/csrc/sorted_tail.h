@@ -5,7 +5,9 @@
 
 namespace mako {
 
-constexpr uint32_t kWalkSeqGroups = 8; // a walk expected to end within this many groups goes entry by entry from LDS
+constexpr uint32_t kWalkSeqGroups = 8; // leading groups in which the running sum may be added entry by entry from LDS
+// (a walk expected to end within kHeadGroups groups goes entry by entry from LDS: two nanoseconds an entry, where a
+// group that is walked by its map costs the chain a fraction of that but every binade r falls through a microsecond)
 struct GroupLds { // carved from the dynamic LDS block once sorting is over; one pointer, the rest is offsets
     unsigned long long* base;
     __device__ __forceinline__ double* pg() const { return reinterpret_cast<double*>(base); } // [kMaxGroups + 2] fp64 sum of the entries before each group
@@ -24,7 +26,7 @@ struct GroupLds { // carved from the dynamic LDS block once sorting is over; one
     __device__ __forceinline__ uint32_t* w_d1() const { return w_d0() + kMaxGroups; }
     __device__ __forceinline__ uint32_t* w_need() const { return w_d1() + kMaxGroups; }
     __device__ __forceinline__ uint32_t* w_pack() const { return w_need() + kMaxGroups; }
-    // [kWalkSeqGroups * kGroup + kWave] the head of the list as floats, for a walk that ends within it
+    // [kHeadGroups * kGroup + kWave] the head of the list as floats, for a walk that ends within it
     __device__ __forceinline__ float* head() const { return reinterpret_cast<float*>(w_pack() + kMaxGroups); }
 };
 constexpr uint32_t kLenMask = 0x1ffu;
@@ -38,7 +40,7 @@ __device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
     assume_lds(L);
     static_assert((kMaxGroups + 2) * 8 + 5 * kMaxGroups * 4 + 16 <= kSortMax * 8, "group records fit below the LDS lists");
     static_assert(kQuarterSlots * 16 == 1536 &&
-                      kSortMax * 8 + 1536 * 4 + 4 * kMaxGroups * 4 + (kWalkSeqGroups * kGroup + kWave) * 4 <= kDynLds,
+                      kSortMax * 8 + 1536 * 4 + 4 * kMaxGroups * 4 + (kHeadGroups * kGroup + kWave) * 4 <= kTailLds,
                   "the walk's records sit behind the quarter records and fit the dynamic LDS block");
     return GroupLds{L.sortk};
 }
@@ -965,7 +967,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         G.misc()[3] = 0;
     // The head of the list as floats in LDS (loads set out now, wanted after the cut): where the running sum and
     // the walk change binade every few entries, both go through it entry by entry.
-    constexpr uint32_t kHeadGroups = kWalkSeqGroups;
     constexpr uint32_t kHead = kHeadGroups * kGroup;
     float* const head = G.head();
     uint32_t raw[kHead / kThreads];
@@ -1216,10 +1217,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
 #endif
     // A walk that will end within a few groups goes through them entry by entry, from a copy in LDS: faster than
     // the groups' maps would be to build.
-#ifndef MAKO_HEAD_WALK_GROUPS
-#define MAKO_HEAD_WALK_GROUPS 8
-#endif
-    const bool head_walk = reach <= MAKO_HEAD_WALK_GROUPS; // uniform
+    const bool head_walk = reach <= kHeadGroups; // uniform
     const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
     if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && !head_walk) {
         // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
