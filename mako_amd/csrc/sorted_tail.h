@@ -33,6 +33,9 @@ constexpr uint32_t kLenMask = 0x1ffu;
 constexpr uint32_t kHasQuarters = 1u << 31;
 constexpr uint32_t kQuarterSlots = 96;
 constexpr uint32_t kQuarter = kGroup / 4;
+#ifndef MAKO_WALK_PASSED
+#define MAKO_WALK_PASSED 1u
+#endif
 constexpr uint32_t kSeqMax = 1024; // sorted lists up to this long get their total and walk entry by entry
 
 __device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
@@ -1219,10 +1222,10 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     // the groups' maps would be to build.
     const bool head_walk = reach <= kHeadGroups; // uniform
     const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
-    if (wave_id() != 0 && (wave_id() & 3) != 0 && r0_guess == r0_guess && !head_walk) {
-        // (the waves that do not share a SIMD with the chaining wave: 1, 2, 3, 5, 6, 7, ...)
-        build_group_maps(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)(wave_id() >> 2) * 3u + (uint32_t)(wave_id() & 3) - 1u,
-                         3u * kWaves / 4u);
+    if (wave_id() != 0 && r0_guess == r0_guess && !head_walk) {
+        // (all the other waves: with more than kHeadGroups maps to build they take longer than the chain, even
+        // though three of them share its SIMD)
+        build_group_maps(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u);
 #ifdef MAKO_TIMING
         if (tid == 64 && s_mako_row == 0)
             g_mako_stamp[23] = wall_clock64() - tb0;
@@ -1396,7 +1399,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     // Group f goes entry by entry.  Where one group does, its neighbours tend to follow (r is down
                     // among the weights and changes binade every few entries), so the groups behind it are tried one
                     // at a time with a few scalar operations each, the next one's entries already on their way,
-                    // and the scan takes over again once four in a row have gone through as maps.
+                    // and the scan takes over again as soon as one has gone through as a map.
                     uint32_t g = f, passed = 0;
                     uint32_t raw[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu}; // the entries of group g
                     {
@@ -1405,7 +1408,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         if (pk & kLenMask)
                             fetch_span_lanes(kf, st, pk & kLenMask, raw);
                     }
-                    while (g < cnt && passed < 4u) {
+                    while (g < cnt && passed < MAKO_WALK_PASSED) {
                         const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g);
                         const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g);
                         float xa[4];
