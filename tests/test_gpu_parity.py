@@ -597,12 +597,13 @@ def test_second_pass_piece_sizes(gpu_ctx, v):
 
 def test_nucleus_sizes_around_path_boundaries(gpu_ctx):
     """Nuclei just below and above the sizes at which the sorted tail changes its route (one wave up to 256 entries,
-    total and walk from LDS up to 1024, the list's head in LDS up to 2048, group maps beyond), each drawn at the
-    first entry, deep inside and at the very end."""
+    total and walk from LDS up to 1024; a walk that ends within the 8192 entries staged in LDS goes entry by entry,
+    group maps beyond), each drawn at the first entry, deep inside and at the very end."""
     v = 129280
     rng = np.random.default_rng(2024)
-    targets = [200, 256, 257, 300, 1000, 1024, 1025, 1100, 2040, 2048, 2049, 2100, 4096, 5000, 20000]
-    us = [0.0, 1e-7, 0.3, 0.9, 0.99999994]
+    targets = [200, 256, 257, 300, 1000, 1024, 1025, 1100, 2040, 2048, 2049, 2100, 4096, 5000, 8100, 8192, 8193, 8300,
+               9000, 16500, 20000]
+    us = [0.0, 1e-7, 0.3, 0.9, 0.97, 0.99999994]
     base = -np.arange(v, dtype=np.float64) * 2e-4  # distinct, slowly falling weights
     q = np.exp(base)
     csum = np.cumsum(q)
@@ -619,8 +620,8 @@ def test_nucleus_sizes_around_path_boundaries(gpu_ctx):
     g = assert_parity(gpu_ctx, w, cap=64)
     sizes = sorted(set(int(x) for x in g["n_cand"]))
     _say("nucleus sizes: %s" % sizes)
-    assert min(sizes) <= 256 and any(256 < x <= 1024 for x in sizes) and any(1024 < x <= 2048 for x in sizes) \
-        and any(x > 2048 for x in sizes)
+    assert min(sizes) <= 256 and any(256 < x <= 1024 for x in sizes) and any(1024 < x <= 8192 for x in sizes) \
+        and any(x > 8192 for x in sizes)
 
 
 def test_host_parameter_copy_only_skips_work(gpu_ctx):
