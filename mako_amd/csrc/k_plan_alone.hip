@@ -5,7 +5,7 @@
 #include "sampler_kernels.h"
 
 namespace mako {
-void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices)
+void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices)
 {
     hipLaunchKernelGGL(plan_kernel, dim3(1, d.n_rows), dim3(kThreads), kTailLds, st, d, sc, slices);
 }

@@ -25,7 +25,7 @@ void launch_scan(bool vec, int kh, bool above, dim3 grid, size_t lds, hipStream_
 // finish_kernel<vec, kh> on `wgs` workgroups
 void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch* sc,
                    uint32_t slices);
-void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices);
+void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices); // (host copy, by value)
 // sort_kernel's workgroup i serves entry i of the work list: `grid_rows` * kWorkers workgroups must cover the
 // longest list the batch can produce (kWorkers entries per top_k == 0 row); tail_kernel takes one workgroup per possible wide row.  Workgroups beyond the lists leave at once, but each
 // of them still has to be dispatched.

@@ -414,7 +414,7 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     if (any_nucleus)
         MAKO_LAUNCH(mako::launch_finish(vec, kh, finish_wgs, st, d, sc_dev, slices));
     if (!launch_sort)
-        MAKO_LAUNCH(mako::launch_plan_alone(st, d, sc_dev, slices));
+        MAKO_LAUNCH(mako::launch_plan_alone(st, d, sc, slices));
     MAKO_MARK(2);
     if (any_nucleus)
         MAKO_LAUNCH(mako::launch_sort(st, d, sc, slices, nucleus_rows));

@@ -10,9 +10,9 @@ namespace mako {
 // whole-row path (the host saw none in its copy of the parameters): such a batch ends here.  Rows whose token is
 // forced, greedy rows and top-k rows are finished from the records scan_kernel left; a row that turns out to need
 // the whole-row path after all is given it here.
-__global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
+__global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
 {
-    const Scratch& sc_arg = *sc_dev;
+    const Scratch& sc_arg = sc_val; // (by value: where the row's records are is known without a trip to memory)
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
@@ -22,7 +22,23 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     MAKO_WG_TIMER;
 #endif
     MAKO_ROW(row);
-    stage_args(d_arg, sc_arg, row, s_args);
+    // Two trips to memory before the row's candidates are here, not three: the arguments' copy for LDS, the row's
+    // parameters and the exp2 table go out first; the candidate slots and the slices' records as soon as the context's
+    // record says where they are (whatever the row turns out to be: a greedy row's are never looked at); the copy is
+    // put in LDS under them.
+    const uint64_t tab_word = k_exp2_tab[tid & 31u];
+    ArgWords arg_words;
+    fetch_arg_words(d_arg, sc_arg, arg_words);
+    fetch_param_words(d_arg, row, arg_words);
+    CandSlots pre;
+    const bool covered = slots_cover(slices); // uniform
+    if (covered)
+        fetch_candidate_slots(sc_arg, row, slices, pre);
+    const SliceStat lane_stat = load_slice_stat(sc_arg.stats, (size_t)row * kMaxSlices + min((uint32_t)lane_id(), slices - 1u));
+    place_arg_words(arg_words, s_args);
+    if (tid < 32)
+        sm.tab[tid] = tab_word;
+    lds_barrier(); // (publishes the copy and the table; the loads above stay in flight)
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
     const mako_sampling_params& P = s_args.P;
@@ -56,18 +72,10 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
             return;
         }
     }
-    if (tid < 32)
-        sm.tab[tid] = k_exp2_tab[tid];
-    __syncthreads();
-    // a top-k row's candidates are asked for together with the slices' records
-    CandSlots pre;
-    const bool prefetched = cls == kTopK && !d.draft && slots_cover(slices); // uniform
-    if (prefetched)
-        fetch_candidate_slots(sc, row, slices, pre);
+    const bool prefetched = covered && cls == kTopK && !d.draft; // uniform
     float m;
     uint32_t argidx, n_cands, any_overflow;
-    SliceStat lane_stat;
-    row_summary(sc, row, slices, m, argidx, n_cands, any_overflow, &lane_stat);
+    row_summary_of(lane_stat, slices, m, argidx, n_cands, any_overflow);
     if (cls != kNucleus)
         MAKO_STAMP(1);
     if (cls == kGreedy) { // sampler.cpp:77-78, 88-92
