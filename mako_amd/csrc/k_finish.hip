@@ -5,12 +5,12 @@
 namespace mako {
 namespace {
 template <bool VEC, int KH>
-void launch_one(uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices)
+void launch_one(uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices)
 {
     hipLaunchKernelGGL((finish_kernel<VEC, KH>), dim3(1, wgs), dim3(kThreads), kDynLds, st, d, sc, slices);
 }
 template <bool VEC>
-void launch_vec(int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch* sc, uint32_t slices)
+void launch_vec(int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices)
 {
     if (kh == 2)
         launch_one<VEC, 2>(wgs, st, d, sc, slices);
@@ -21,7 +21,7 @@ void launch_vec(int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d,
 }
 } // namespace
 
-void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch* sc,
+void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc,
                    uint32_t slices)
 {
     if (vec)

@@ -18,13 +18,13 @@ hipError_t init_sort_kernels();
 hipError_t init_tail_kernels();
 
 // scan_kernel<vec, kh, above>, grid = (slices, rows), `lds` bytes of dynamic LDS
-// (`sc`: the HOST copy of the context's record; scan, sort and tail kernels take it by value, so that their
-// first loads need no trip to memory for the record itself; finish and plan kernels take the device copy's address)
+// (`sc`: the HOST copy of the context's record; the kernels take it by value, so that their first loads need no
+// trip to memory for the record itself)
 void launch_scan(bool vec, int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d,
                  const Scratch& sc, uint32_t slice_len, uint32_t cus);
 // finish_kernel<vec, kh> on `wgs` workgroups
-void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch* sc,
-                   uint32_t slices);
+void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc,
+                   uint32_t slices); // (host copy, by value)
 void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices); // (host copy, by value)
 // sort_kernel's workgroup i serves entry i of the work list: `grid_rows` * kWorkers workgroups must cover the
 // longest list the batch can produce (kWorkers entries per top_k == 0 row); tail_kernel takes one workgroup per possible wide row.  Workgroups beyond the lists leave at once, but each

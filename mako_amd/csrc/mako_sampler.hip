@@ -38,7 +38,6 @@ struct mako_sampler_ctx {
     int device = 0;
     uint32_t max_rows = 0, max_vocab = 0, max_hist = 0;
     mako::Scratch sc{};
-    mako::Scratch* sc_dev = nullptr; // the same record in device memory: the kernels take a pointer to it
     // staging for the host-pointer call
     float* st_logits = nullptr;
     mako_sampling_params* st_params = nullptr;
@@ -87,15 +86,15 @@ uint32_t slice_len_for(uint32_t n_vocab, uint32_t slices)
 
 
 int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampling_params* params_host, void* stream,
-              const mako::Scratch& sc, const mako::Scratch* sc_dev, uint32_t max_rows, uint32_t max_vocab);
+              const mako::Scratch& sc, uint32_t max_rows, uint32_t max_vocab);
 
 #define MAKO_STR2(x) #x
 #define MAKO_STR(x) MAKO_STR2(x)
 
 // The kernels' scratch memory for batches of up to max_rows rows of up to max_vocab logits, every array taken from
-// `take` (256-byte aligned blocks); *sc_dev gets room for the device copy of the record itself.
+// `take` (256-byte aligned blocks).  (The kernels take the record by value.)
 template <typename Take>
-hipError_t layout_scratch(mako::Scratch& sc, mako::Scratch** sc_dev, uint32_t max_rows, uint32_t max_vocab, Take take)
+hipError_t layout_scratch(mako::Scratch& sc, uint32_t max_rows, uint32_t max_vocab, Take take)
 {
 #define MAKO_TAKE(ptr, count)                                                                                      \
     do {                                                                                                           \
@@ -107,7 +106,6 @@ hipError_t layout_scratch(mako::Scratch& sc, mako::Scratch** sc_dev, uint32_t ma
     sc.vpad = ((uint64_t)max_vocab + max_vocab / 64u + mako::kWorkers * mako::kStageSlack + 1023u) & ~1023ull;
     const size_t rv = (size_t)max_rows * sc.vpad;
     sc.slices_cap = mako_sampler_slices(max_vocab);
-    MAKO_TAKE(*sc_dev, 1);
     MAKO_TAKE(sc.stats, (size_t)max_rows * mako::kMaxSlices);
     MAKO_TAKE(sc.cand_w, (size_t)max_rows * sc.slices_cap * mako::kCap);
     MAKO_TAKE(sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap);
@@ -162,7 +160,6 @@ struct StaticScratch {
     bool ready = false;
     hipError_t status = hipSuccess; // of the set-up, kept: a device whose set-up failed refuses every call
     mako::Scratch sc{};
-    mako::Scratch* sc_dev = nullptr;
 };
 StaticScratch g_static[kStaticDevices];
 std::mutex g_static_mutex;
@@ -182,7 +179,7 @@ hipError_t setup_static_scratch(int device)
         e = hipErrorInvalidSymbol;
     size_t used = 0;
     if (e == hipSuccess)
-        e = layout_scratch(g.sc, &g.sc_dev, MAKO_STATIC_MAX_ROWS, MAKO_STATIC_MAX_VOCAB, [&](void** p, size_t bytes) {
+        e = layout_scratch(g.sc, MAKO_STATIC_MAX_ROWS, MAKO_STATIC_MAX_VOCAB, [&](void** p, size_t bytes) {
             if (bytes > kStaticBytes - used)
                 return hipErrorOutOfMemory;
             *p = base + used;
@@ -191,8 +188,6 @@ hipError_t setup_static_scratch(int device)
         });
     if (e == hipSuccess)
         e = zero_scratch(g.sc, MAKO_STATIC_MAX_ROWS);
-    if (e == hipSuccess)
-        e = hipMemcpy(g.sc_dev, &g.sc, sizeof g.sc, hipMemcpyHostToDevice);
     if (e == hipSuccess)
         e = hipDeviceSynchronize();
     g.status = e;
@@ -232,9 +227,8 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
         if (n > 0)
             ctx->cus = (uint32_t)n;
     }
-    MAKO_HIP(ctx, layout_scratch(ctx->sc, &ctx->sc_dev, max_rows, max_vocab, [](void** p, size_t bytes) { return hipMalloc(p, bytes); }));
+    MAKO_HIP(ctx, layout_scratch(ctx->sc, max_rows, max_vocab, [](void** p, size_t bytes) { return hipMalloc(p, bytes); }));
     MAKO_HIP(ctx, zero_scratch(ctx->sc, max_rows));
-    MAKO_HIP(ctx, hipMemcpy(ctx->sc_dev, &ctx->sc, sizeof ctx->sc, hipMemcpyHostToDevice));
     MAKO_HIP(ctx, setup_static_scratch(device));
     MAKO_HIP(ctx, hipDeviceSynchronize());
     // the kernels overlay up to 64 KB of dynamic LDS (sort_kernel more) on a few KB of static LDS
@@ -252,7 +246,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {ctx->sc_dev, sc.log_hist, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
+    void* ptrs[] = {sc.log_hist, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
                     sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
@@ -308,7 +302,7 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
     if (!ctx || !desc)
         return MAKO_ERR_INVALID_ARG;
     MAKO_HIP(ctx, hipSetDevice(ctx->device));
-    return run_batch(ctx, *desc, params_host, stream, ctx->sc, ctx->sc_dev, ctx->max_rows, ctx->max_vocab);
+    return run_batch(ctx, *desc, params_host, stream, ctx->sc, ctx->max_rows, ctx->max_vocab);
 }
 
 int mako_sampler_sample_batch_static(mako_sampler_ctx* ctx, const mako_sample_desc* desc, void* stream)
@@ -325,7 +319,7 @@ int mako_sampler_sample_batch_static(mako_sampler_ctx* ctx, const mako_sample_de
     if (!g.ready || g.status != hipSuccess)
         return fail(ctx, MAKO_ERR_HIP, "sampler: the static scratch memory could not be set up on this device");
     MAKO_HIP(ctx, hipSetDevice(ctx->device));
-    return run_batch(ctx, *desc, nullptr, stream, g.sc, g.sc_dev, MAKO_STATIC_MAX_ROWS, MAKO_STATIC_MAX_VOCAB);
+    return run_batch(ctx, *desc, nullptr, stream, g.sc, MAKO_STATIC_MAX_ROWS, MAKO_STATIC_MAX_VOCAB);
 }
 
 } // extern "C"
@@ -333,7 +327,7 @@ int mako_sampler_sample_batch_static(mako_sampler_ctx* ctx, const mako_sample_de
 namespace {
 // One batch through the kernels, on scratch memory laid out for max_rows x max_vocab.  Allocates nothing.
 int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampling_params* params_host, void* stream,
-              const mako::Scratch& sc, const mako::Scratch* sc_dev, uint32_t max_rows, uint32_t max_vocab)
+              const mako::Scratch& sc, uint32_t max_rows, uint32_t max_vocab)
 {
     if (d.n_vocab == 0)
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: empty vocabulary"); // sampler.cpp:11-12
@@ -412,7 +406,7 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  A batch without such rows
     // (and without rows for the whole-row path) ends with plan_kernel instead.
     if (any_nucleus)
-        MAKO_LAUNCH(mako::launch_finish(vec, kh, finish_wgs, st, d, sc_dev, slices));
+        MAKO_LAUNCH(mako::launch_finish(vec, kh, finish_wgs, st, d, sc, slices));
     if (!launch_sort)
         MAKO_LAUNCH(mako::launch_plan_alone(st, d, sc, slices));
     MAKO_MARK(2);

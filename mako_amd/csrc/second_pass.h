@@ -208,9 +208,9 @@ __device__ void row_pieces(const mako_sample_desc& d, const Scratch& sc, uint32_
 // workgroups are then the first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the
 // mix of rows.
 template <bool VEC, int KH>
-__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, const Scratch* sc_dev, uint32_t slices)
+__global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
 {
-    const Scratch& sc_arg = *sc_dev;
+    const Scratch& sc_arg = sc_val; // (by value: the cut is one trip to memory away, not two)
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
