@@ -49,8 +49,14 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         finish_late_row(s_args.d, s_args.sc, s_args.P, r, slices, Lr);
         return;
     }
+    // (two trips to memory before the list's records are asked for: the work list's entry with the arguments' copy
+    // for LDS, then the row's plan with its parameters; the empty asm statements keep each trip's loads together)
+    const uint32_t tid = threadIdx.x;
+    ArgWords arg_words;
+    fetch_arg_words(d_arg, sc_arg, arg_words);
     const uint32_t n_work = sc_arg.work_n[1];
-    const uint32_t row = sc_arg.work_tail[blockIdx.y], tid = threadIdx.x; // (the list has room for every workgroup)
+    const uint32_t row = sc_arg.work_tail[blockIdx.y]; // (the list has room for every workgroup)
+    asm volatile("" ::"s"(row), "s"(n_work), "v"(arg_words.d), "v"(arg_words.sc));
     if (blockIdx.y >= n_work)
         return;
     MAKO_ROW(row);
@@ -59,9 +65,12 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     const double total64 = planned->total64;
     const float plan_m = planned->m;
     const uint32_t plan_argidx = planned->argidx;
+    fetch_param_words(d_arg, row, arg_words);
+    asm volatile("" ::"s"(flag), "s"(plan_n0), "s"(plan_groups), "v"(arg_words.p));
     if (flag != 1)
         return;
-    stage_args(d_arg, sc_arg, row, s_args);
+    place_arg_words(arg_words, s_args);
+    __syncthreads();
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
     BigPlan* plan = sc.plan + row;
