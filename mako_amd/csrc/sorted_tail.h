@@ -490,7 +490,7 @@ __device__ bool exact_span_walk(Keys kf, uint32_t start, uint32_t len, float& r,
 }
 
 // The walk over the first `n` entries of the list, staged in LDS as floats (16-byte aligned): every lane of the
-// wave reads the same four entries with one broadcast load and subtracts them in turn, three nanoseconds an entry
+// wave reads the same four entries with one broadcast load and subtracts them in turn, two nanoseconds an entry
 // (the travelling chain of walk_lanes() takes five).  Blocks of 64 blind, then of 16, then entry by entry, as there.
 // Returns true and the position when the walk stops, else false and the new r.
 // (The list is read as LDS, not through the generic pointer: generic loads wait for one another in full, and the
@@ -1169,7 +1169,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     MAKO_STAMP(7);
     if (n <= kSeqMax) {
         // A nucleus this short is copied to LDS and gone through entry by entry, once for the total and once for the
-        // walk (three nanoseconds an entry each way): the group maps below only pay on longer lists.
+        // walk (two nanoseconds an entry each way): the group maps below only pay on longer lists.
         if (wave_id() == 0) {
             const float S = sum_lds(head, n, 0.0f);
             const float span = S - 0.0f;
