@@ -72,7 +72,8 @@ __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, ui
     auto add = [&](uint32_t s, uint32_t v) {
         if (!v)
             return;
-        const uint32_t b = log_bin_in_frame(log_bin_unit(tid, pl.slice_top[s]), k_top);
+        // (the slice's maximum in a scalar register: what depends on it alone is scalar arithmetic)
+        const uint32_t b = log_bin_moved(tid, (int32_t)__builtin_amdgcn_readfirstlane(pl.slice_top[s]), k_top);
         if (b < kLogBins - 1u)
             atomicAdd(&pl.cnt[b], v);
     };

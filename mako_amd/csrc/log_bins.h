@@ -69,6 +69,20 @@ LOGBINS_HD int32_t log_bin_unit(uint32_t b, int32_t k_top)
                         : (int32_t)((uint32_t)(log_first_group(k_top) - (int32_t)(b - kLogFine)) << kLogCoarseShift);
 }
 
+// Where the logits of bin b of a slice's frame (maximum k_slice) belong in the frame of the row's maximum k_top
+// (>= k_slice): log_bin_in_frame(log_bin_unit(b, k_slice), k_top) with less arithmetic.  A coarse bin is a group of
+// units and stays one: only its number changes, by the distance between the two frames' first groups.
+// (Equal to that composition for units within +-2^30, which is what the host test checks; beyond, where the units
+// of log_unit() saturate anyway, the two may name different bins, which costs balance and nothing else.)
+LOGBINS_HD uint32_t log_bin_moved(uint32_t b, int32_t k_slice, int32_t k_top)
+{
+    if (b >= kLogFine) {
+        const uint32_t c = b + (uint32_t)(log_first_group(k_top) - log_first_group(k_slice));
+        return c < kLogBins - 1u ? c : kLogNotCounted;
+    }
+    return log_bin_in_frame((int32_t)((uint32_t)k_slice - b), k_top);
+}
+
 // The lowest unit that lies above every unit of bin b (b >= 1) in the frame of k_top: logits whose unit is at
 // least this one are in the bins before b.
 LOGBINS_HD int32_t log_bin_upper_edge(uint32_t b, int32_t k_top)

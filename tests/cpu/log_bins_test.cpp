@@ -84,6 +84,12 @@ static void check_merge(int32_t k_row, int32_t k_slice, std::mt19937& rng)
         const uint32_t moved = log_bin_in_frame(log_bin_unit(sb, k_slice), k_row);
         CHECK(direct == moved, "row top %d slice top %d unit %d: slice bin %u -> row bin %u, its own %u", k_row, k_slice, k, sb, moved, direct);
     }
+    // the short form of the move, for every bin of the slice's frame
+    for (uint32_t b = 0; b < kLogBins - 1u; ++b) {
+        const uint32_t composed = log_bin_in_frame(log_bin_unit(b, k_slice), k_row);
+        const uint32_t moved = log_bin_moved(b, k_slice, k_row);
+        CHECK(composed == moved, "row top %d slice top %d bin %u: moved to %u, composition says %u", k_row, k_slice, b, moved, composed);
+    }
 }
 
 int main()
