@@ -126,8 +126,11 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
         const uint32_t mine = tid < kWorkers ? pl.count[tid] : 0u;
         const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
         if (tid < kWorkers) {
-            pl.base[tid] = mine ? atomicAdd(&plan->cursor[tid], mine) : 0u;
+            const uint32_t base = mine ? atomicAdd(&plan->cursor[tid], mine) : 0u, room = pl.cap[tid];
+            pl.base[tid] = base;
             pl.lbase[tid] = upto - mine;
+            pl.goff[tid] = pl.stage_off[tid] + base - (upto - mine);
+            pl.lim[tid] = (upto - mine) + (room > base ? room - base : 0u);
         }
         if (tid == kWorkers - 1u)
             pl.lbase[kWorkers] = upto;
@@ -141,30 +144,33 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
     uint2* buf = reinterpret_cast<uint2*>(L.cnt); // [kSliceMax / 2] (weight, token id)
     constexpr uint32_t kHalf = kSliceMax / 2u;
     const uint32_t kept = pl.lbase[kWorkers];
+    // (the entries' workers travel beside them, a byte each, in the plan's count arrays, which are done with)
+    static_assert(offsetof(CoarsePlan, incl) == offsetof(CoarsePlan, cnt) + sizeof(uint32_t) * kLogBins && 2u * sizeof(uint32_t) * kLogBins >= kHalf &&
+                      kSliceMax <= 0x10000u && kWorkers <= 256u,
+                  "a byte per buffered entry; an entry's place fits sixteen bits beside its worker");
+    uint8_t* wbuf = reinterpret_cast<uint8_t*>(pl.cnt);
 #pragma unroll
     for (uint32_t j = 0; j < 16; ++j)
-        if (slot[j] != kNone)
-            slot[j] = pl.lbase[slot[j] >> 16] + (slot[j] & 0xffffu); // (from here on: the entry's place in the order)
+        if (slot[j] != kNone) // (from here on: worker << 16 | the entry's place in the workgroup's order)
+            slot[j] = (slot[j] & 0xffff0000u) | (pl.lbase[slot[j] >> 16] + (slot[j] & 0xffffu));
     bool dropped = false;
     for (uint32_t from = 0; from < kept; from += kHalf) { // (what fits the buffer at a time: usually everything)
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j)
-            if (slot[j] != kNone && slot[j] - from < kHalf)
-                buf[slot[j] - from] = make_uint2(qb[j], elem_index<VEC>(lo, tid, j));
+            if (slot[j] != kNone && (slot[j] & 0xffffu) - from < kHalf) {
+                buf[(slot[j] & 0xffffu) - from] = make_uint2(qb[j], elem_index<VEC>(lo, tid, j));
+                wbuf[(slot[j] & 0xffffu) - from] = (uint8_t)(slot[j] >> 16);
+            }
         lds_barrier();
-#pragma unroll
+#pragma unroll 4 // (fully unrolled, the unaligned variants spill dozens of registers for no gain)
         for (uint32_t t = 0; t < kHalf / kThreads; ++t) {
             const uint32_t e = from + t * kThreads + tid;
             if (e < kept) { // (uniform per wave but for the last one)
-                uint32_t w = 0; // the worker whose run holds entry e: the last one whose run starts at or before it
-#pragma unroll
-                for (uint32_t step = kWorkers / 2u; step; step >>= 1)
-                    w += pl.lbase[w + step] <= e ? step : 0u;
-                const uint32_t at = pl.base[w] + (e - pl.lbase[w]);
-                if (at < pl.cap[w]) {
+                const uint32_t w = wbuf[e - from];
+                if (e < pl.lim[w]) {
                     const uint2 x = buf[e - from];
-                    kstage[pl.stage_off[w] + at] = x.x;
-                    istage[pl.stage_off[w] + at] = x.y;
+                    kstage[pl.goff[w] + e] = x.x;
+                    istage[pl.goff[w] + e] = x.y;
                 } else {
                     dropped = true;
                 }
