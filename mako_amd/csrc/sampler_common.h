@@ -79,10 +79,10 @@ constexpr uint32_t kGroup = 256;      // a sorted list is processed in groups of
 constexpr uint32_t kMaxGroups = 1024; // groups per list
 constexpr uint32_t kSegCap = 6144;    // entries a worker sorts in LDS
 constexpr uint32_t kFine = 2048;      // value buckets of that sort
-// dynamic LDS of sort_kernel: the entries, their order, the buckets, and a copy of the sorted weights for the group
-// records
-constexpr uint32_t kSortLds = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u + kSegCap * 4u;
-constexpr uint32_t kSortedCopyAt = kSegCap * 8u + kSegCap * 2u + (kFine + 4u) * 4u; // byte offset of that copy
+// dynamic LDS of sort_kernel: the entries, the entries again in the order of their buckets, the buckets, and a copy
+// of the sorted weights for the group records
+constexpr uint32_t kSortLds = kSegCap * 8u + kSegCap * 8u + (kFine + 4u) * 4u + kSegCap * 4u;
+constexpr uint32_t kSortedCopyAt = kSegCap * 8u + kSegCap * 8u + (kFine + 4u) * 4u; // byte offset of that copy
 
 // Work order for a top_k == 0 row, written by the second pass (every workgroup of the row derives the same one from
 // scan_kernel's coarse counts, see coarse_plan(); the row's first piece stores it): the weights with bits(q) >= thr

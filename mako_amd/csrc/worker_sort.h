@@ -20,8 +20,8 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
                                 unsigned long long* dyn, FinishShared& sm, uint32_t* sorted_lds)
 {
     uint2* A = reinterpret_cast<uint2*>(dyn);
-    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
-    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap);
+    uint2* A2 = A + kSegCap; // the entries again, bucket after bucket (any order inside a bucket)
+    uint32_t* hist = reinterpret_cast<uint32_t*>(A2 + kSegCap);
     const uint32_t tid = threadIdx.x;
     // 2. buckets by value, heaviest first
     const uint32_t range = key_hi - key_lo; // > 0
@@ -54,10 +54,12 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
     MAKO_STAMP(14);
     if (sm.flag)
         return false;
+    // (the entries themselves move, not their numbers: whoever ranks an entry reads its bucket's entries in one
+    // trip to LDS each instead of two)
 #pragma unroll
     for (uint32_t t = 0; t < kPer; ++t)
         if (bucket[t] != kNone)
-            B[hist[bucket[t]] + pib[t]] = (uint16_t)(t * kThreads + tid);
+            A2[hist[bucket[t]] + pib[t]] = A[t * kThreads + tid];
     __syncthreads();
     MAKO_STAMP(15);
     // 3. rank inside the bucket, and out
@@ -65,12 +67,12 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
     for (uint32_t t = 0; t < kPer; ++t) {
         const uint32_t s = t * kThreads + tid;
         if (s < n) {
-            const uint2 me = A[B[s]];
+            const uint2 me = A2[s];
             const uint32_t b = (key_hi - 1u - me.x) >> shift;
             const uint32_t lo = hist[b], hi = hist[b + 1u];
             uint32_t r = 0;
             for (uint32_t x = lo; x < hi; ++x) {
-                const uint2 o = A[B[x]];
+                const uint2 o = A2[x];
                 r += (o.x > me.x) || (o.x == me.x && o.y < me.y);
             }
             kout[lo + r] = ~me.x;
@@ -107,8 +109,7 @@ __device__ __forceinline__ bool lds_sort_staged(const StagedShare& s, uint32_t k
                                                 uint32_t* sorted_lds = nullptr)
 {
     uint2* A = reinterpret_cast<uint2*>(dyn);
-    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
-    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap);
+    uint32_t* hist = reinterpret_cast<uint32_t*>(A + 2u * kSegCap); // (behind lds_bucket_sort()'s second copy)
     const uint32_t tid = threadIdx.x;
     for (uint32_t b = tid; b <= kFine; b += kThreads)
         hist[b] = 0;
@@ -135,8 +136,7 @@ __device__ bool lds_sort_staged_runs(const uint32_t* ks, const uint32_t* is, uin
                                      uint32_t* kout, uint32_t* iout, unsigned long long* dyn, FinishShared& sm)
 {
     uint2* A = reinterpret_cast<uint2*>(dyn);
-    uint16_t* B = reinterpret_cast<uint16_t*>(A + kSegCap);
-    uint32_t* hist = reinterpret_cast<uint32_t*>(B + kSegCap); // [kFine + 1]
+    uint32_t* hist = reinterpret_cast<uint32_t*>(A + 2u * kSegCap); // (behind lds_bucket_sort()'s second copy) // [kFine + 1]
     const uint32_t tid = threadIdx.x, lane = lane_id();
     const uint32_t range = key_hi - key_lo;
     const uint32_t shift = range > kFine ? 32u - (uint32_t)__clz((range - 1u) >> 11) : 0u;
