@@ -70,10 +70,16 @@ __device__ bool lds_bucket_sort(uint32_t n, uint32_t key_lo, uint32_t key_hi, ui
             const uint2 me = A2[s];
             const uint32_t b = (key_hi - 1u - me.x) >> shift;
             const uint32_t lo = hist[b], hi = hist[b + 1u];
+            // (four of the bucket's entries per trip, from clamped positions: a bucket rarely holds more)
             uint32_t r = 0;
-            for (uint32_t x = lo; x < hi; ++x) {
-                const uint2 o = A2[x];
-                r += (o.x > me.x) || (o.x == me.x && o.y < me.y);
+            for (uint32_t x = lo; x < hi; x += 4u) {
+                uint2 o[4];
+#pragma unroll
+                for (uint32_t u = 0; u < 4; ++u)
+                    o[u] = A2[min(x + u, hi - 1u)];
+#pragma unroll
+                for (uint32_t u = 0; u < 4; ++u)
+                    r += (x + u < hi && ((o[u].x > me.x) || (o[u].x == me.x && o[u].y < me.y))) ? 1u : 0u;
             }
             kout[lo + r] = ~me.x;
             iout[lo + r] = me.y;
