@@ -231,7 +231,7 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, zero_scratch(ctx->sc, max_rows));
     MAKO_HIP(ctx, setup_static_scratch(device));
     MAKO_HIP(ctx, hipDeviceSynchronize());
-    // the kernels overlay up to 64 KB of dynamic LDS (sort_kernel more) on a few KB of static LDS
+    // the kernels overlay 64 to 128 KB of dynamic LDS (kDynLds, kTailLds, kSortLds) on a few KB of static LDS
     MAKO_HIP(ctx, mako::init_scan_kernels());
     MAKO_HIP(ctx, mako::init_finish_kernels());
     MAKO_HIP(ctx, mako::init_plan_alone());

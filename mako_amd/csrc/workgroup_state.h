@@ -17,7 +17,7 @@ struct alignas(16) FinishShared {
     uint32_t soff[kMaxSlices + 1]; // first candidate of each slice in the row's flattened candidate list
 };
 
-// Views into the 64 KB dynamic LDS block; `cnt` (first pass) overlaps the two others (second pass).
+// Views into the first 64 KB of the dynamic LDS block; `cnt` (first pass) overlaps the two others (second pass).
 struct FinishLds {
     FinishShared* sm;
     uint32_t* cnt;              // [kSliceMax]
