@@ -110,7 +110,6 @@ hipError_t layout_scratch(mako::Scratch& sc, uint32_t max_rows, uint32_t max_voc
     MAKO_TAKE(sc.cand_w, (size_t)max_rows * sc.slices_cap * mako::kCap);
     MAKO_TAKE(sc.cand_i, (size_t)max_rows * sc.slices_cap * mako::kCap);
     MAKO_TAKE(sc.part_sum, (size_t)max_rows * mako::kMaxSlices);
-    MAKO_TAKE(sc.part_n, (size_t)max_rows * mako::kMaxSlices);
     MAKO_TAKE(sc.plan, (size_t)max_rows);
     MAKO_TAKE(sc.wbuf, rv);
     MAKO_TAKE(sc.cnt, rv);
@@ -247,7 +246,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
     void* ptrs[] = {sc.log_hist, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
-                    sc.cand_w, sc.cand_i, sc.part_sum, sc.part_n, sc.plan,
+                    sc.cand_w, sc.cand_i, sc.part_sum, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,
                     ctx->st_hist,  ctx->st_hcnt, ctx->st_hlen,  ctx->st_draft, ctx->st_tokens, ctx->st_acc};

@@ -124,7 +124,6 @@ struct Scratch {
     float* cand_w;     // [max_rows][slices_cap][kCap] penalised logits of the slice's candidates
     uint32_t* cand_i;  // [max_rows][slices_cap][kCap] their token ids
     double* part_sum;  // [max_rows][kMaxSlices] exact fp64 sum of q over the slice (top_k == 0 rows)
-    uint32_t* part_n;  // [max_rows][kMaxSlices] candidates (q > 0, q >= min_p) in the slice
     BigPlan* plan;     // [max_rows]; flag zero between calls
     float* wbuf;       // [max_rows][vpad] penalised logits of rows on the whole-row path, then bits(q) of every logit
                        // (0 where q is not a candidate)
@@ -132,11 +131,11 @@ struct Scratch {
     uint32_t* key[2];  // [max_rows][vpad] candidate keys (~bits(q)), ping-pong; [1] also takes the workers' unsorted
                        // shares (bits(q)) from the second pass
     uint32_t* idx[2];  // [max_rows][vpad] candidate token ids, likewise
+    uint16_t* log_hist;  // [max_rows][slices_cap][kLogBins] top_k == 0 rows: logits of the slice per bin of the slice's
+                         // own frame (log_bin_in_frame(); a slice holds 16384 logits at most)
     GroupTable gt;     // [max_rows][g_cap] each
                        // (kept at a multiple of 16 bytes: the kernels' LDS copies of this record are read with
                        // 128-bit operations, which stall on anything less)
-    uint16_t* log_hist;  // [max_rows][slices_cap][kLogBins] top_k == 0 rows: logits of the slice per bin of the slice's
-                         // own frame (log_bin_in_frame(); a slice holds 16384 logits at most)
     // Work lists.  sort_kernel and tail_kernel are launched with one workgroup per POSSIBLE piece of work, but
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
     // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.

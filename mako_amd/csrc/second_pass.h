@@ -9,8 +9,7 @@
 namespace mako {
 
 // A workgroup's share of a top_k == 0 row's pieces, one after the other.  Of each piece: the exact fp64 sum of q over
-// it and the number of candidates in it (q > 0 and q >= min_p), and every weight the row's plan keeps handed to the
-// share of the worker that will sort it.
+// it, and every weight the row's plan keeps handed to the share of the worker that will sort it.
 // The summation order is fixed: each thread adds its logits in index order, then lanes, then waves.
 // The plan (coarse_plan()) is built while the first piece's logits are on their way; every workgroup of the row
 // arrives at the same one, and the one with the row's first piece stores it for the kernels that follow and enters
@@ -77,7 +76,6 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
     const uint32_t thr = pl.thr;
     const uint32_t edge7 = uniform_u32(pl.key_lo[7]), edge15 = uniform_u32(pl.key_lo[15]), edge23 = uniform_u32(pl.key_lo[23]);
     double sum = 0;
-    uint32_t n = 0;
     uint32_t qb[16];   // bits(q), 0 where q is not a candidate
     uint32_t slot[16]; // kept weights: worker << 16 | position among this workgroup's entries for that worker
     // (a piece may be shorter than the sixteen logits per thread: whole blocks past its end are skipped; the test is
@@ -89,10 +87,8 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
         if (lo + (VEC ? (j / 4u) * 4096u : j * (uint32_t)kThreads) < hi) {
             const float q = weight_of(wv[j], m, inv_t, sm.tab);
             qb[j] = (q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
-            if (qb[j]) {
+            if (qb[j])
                 sum += (double)q;
-                ++n;
-            }
             if (qb[j] >= thr && qb[j]) {
                 // the worker whose range of bits(q) holds the weight (equal weights always meet in one share): the
                 // number of workers whose lower edge lies above it, by bisection over the edges
@@ -108,14 +104,11 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
         }
     }
     MAKO_STAMP(25);
-    // the piece's sum and count: wave reductions, one exchange of the sixteen waves' results for both
+    // the piece's sum: wave reductions, then the sixteen waves' results in order
     {
         const double sw = __ockl_wfred_add_f64(sum);
-        const uint32_t nw = __ockl_wfred_add_u32(n);
-        if (lane_id() == 0) {
+        if (lane_id() == 0)
             sm.bs.f64[wave_id()] = sw;
-            sm.bs.u64[wave_id()] = nw;
-        }
     }
     lds_barrier();
     MAKO_STAMP(26);
@@ -182,13 +175,9 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
         plan->overflow = 1;
     if (tid == 0) {
         double total = 0;
-        uint32_t count = 0;
-        for (int w = 0; w < kWaves; ++w) { // waves in order: the same inputs always give the same bits
+        for (int w = 0; w < kWaves; ++w) // waves in order: the same inputs always give the same bits
             total += sm.bs.f64[w];
-            count += (uint32_t)sm.bs.u64[w];
-        }
         as_global(sc.part_sum)[(size_t)row * kMaxSlices + slice] = total;
-        as_global(sc.part_n)[(size_t)row * kMaxSlices + slice] = count;
     }
     lds_barrier(); // (the waves' sums have been read before the next piece's replace them)
     return true;
