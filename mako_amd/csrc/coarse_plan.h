@@ -22,9 +22,8 @@ struct alignas(16) CoarsePlan {
     uint32_t stage_off[kWorkers];
     double mass_above[kWorkers];
     double mass_all;
-    uint32_t count[kWorkers]; // hand-over: this workgroup's entries for each worker, and where its run starts
-    uint32_t base[kWorkers];
-    uint32_t lbase[kWorkers + 1]; // and in the workgroup's own ordering of what it keeps
+    uint32_t count[kWorkers]; // hand-over: this workgroup's entries for each worker
+    uint32_t lbase[kWorkers + 1]; // where its run starts in the workgroup's own ordering of what it keeps
     uint32_t goff[kWorkers];      // entry e of that ordering, if worker w's, goes to goff[w] + e of the row's staging arrays
     uint32_t lim[kWorkers];       // if e < lim[w] (the share's room allows it)
     uint32_t flag, thr, n0_est, pad;

@@ -115,20 +115,21 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
     // One run per worker in its share of the row's staging arrays, reserved with a single atomic.  The kept weights
     // are first put in LDS (the penalty table's block, free by now) in the order of their workers, so that the runs
     // go out as contiguous stores.
+    // (the reservations' answers take a trip to device memory: the entries are put in LDS order under it)
+    uint32_t mine = 0, lbase_mine = 0, base_mine = 0;
     if (wave_id() == 0) {
-        const uint32_t mine = tid < kWorkers ? pl.count[tid] : 0u;
+        mine = tid < kWorkers ? pl.count[tid] : 0u;
         const uint32_t upto = __ockl_wfscan_add_u32(mine, true);
+        lbase_mine = upto - mine;
         if (tid < kWorkers) {
-            const uint32_t base = mine ? atomicAdd(&plan->cursor[tid], mine) : 0u, room = pl.cap[tid];
-            pl.base[tid] = base;
-            pl.lbase[tid] = upto - mine;
-            pl.goff[tid] = pl.stage_off[tid] + base - (upto - mine);
-            pl.lim[tid] = (upto - mine) + (room > base ? room - base : 0u);
+            pl.lbase[tid] = lbase_mine;
+            if (mine)
+                base_mine = __hip_atomic_fetch_add(as_global(&plan->cursor[tid]), mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         if (tid == kWorkers - 1u)
             pl.lbase[kWorkers] = upto;
     }
-    __syncthreads();
+    lds_barrier(); // (not one that waits for the reservations)
     MAKO_STAMP(27);
     if (tid < kWorkers)
         pl.count[tid] = 0; // (for the workgroup's next piece)
@@ -142,10 +143,18 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
                       kSliceMax <= 0x10000u && kWorkers <= 256u,
                   "a byte per buffered entry; an entry's place fits sixteen bits beside its worker");
     uint8_t* wbuf = reinterpret_cast<uint8_t*>(pl.cnt);
+    // (from here on: worker << 16 | the entry's place in the workgroup's order.  The runs' starts are read for all
+    // sixteen at once, kept or not: behind sixteen branches each read would be a wait of its own.)
+    {
+        uint32_t start[16];
 #pragma unroll
-    for (uint32_t j = 0; j < 16; ++j)
-        if (slot[j] != kNone) // (from here on: worker << 16 | the entry's place in the workgroup's order)
-            slot[j] = (slot[j] & 0xffff0000u) | (pl.lbase[slot[j] >> 16] + (slot[j] & 0xffffu));
+        for (uint32_t j = 0; j < 16; ++j)
+            start[j] = pl.lbase[(slot[j] >> 16) & (kWorkers - 1u)];
+#pragma unroll
+        for (uint32_t j = 0; j < 16; ++j)
+            if (slot[j] != kNone)
+                slot[j] = (slot[j] & 0xffff0000u) | (start[j] + (slot[j] & 0xffffu));
+    }
     bool dropped = false;
     for (uint32_t from = 0; from < kept; from += kHalf) { // (what fits the buffer at a time: usually everything)
 #pragma unroll
@@ -154,6 +163,12 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
                 buf[(slot[j] & 0xffffu) - from] = make_uint2(qb[j], elem_index<VEC>(lo, tid, j));
                 wbuf[(slot[j] & 0xffffu) - from] = (uint8_t)(slot[j] >> 16);
             }
+        if (from == 0 && tid < kWorkers) { // (wave 0: where each worker's run goes and where its room ends, in the
+                                           // workgroup's order)
+            const uint32_t room = pl.cap[tid];
+            pl.goff[tid] = pl.stage_off[tid] + base_mine - lbase_mine;
+            pl.lim[tid] = lbase_mine + (room > base_mine ? room - base_mine : 0u);
+        }
         lds_barrier();
 #pragma unroll 4 // (fully unrolled, the unaligned variants spill dozens of registers for no gain)
         for (uint32_t t = 0; t < kHalf / kThreads; ++t) {
