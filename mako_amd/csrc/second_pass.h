@@ -232,7 +232,8 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     // (each costs most of a microsecond here, and the pass starts with nothing else to do): the rows' parameters
     // for find_piece() and the arguments' copy go out together with the cut, and the row's own parameters are then
     // taken from the lane that loaded them.
-    const uint32_t wg = blockIdx.y * gridDim.x + blockIdx.x, tid = threadIdx.x;
+    uint32_t wg = blockIdx.y * gridDim.x + blockIdx.x;
+    const uint32_t tid = threadIdx.x;
     const bool by_lane = d_arg.n_rows <= (uint32_t)kWave; // uniform
     mako_sampling_params P_lane = mako_sampling_params{};
     if (by_lane)
@@ -240,6 +241,17 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     stage_args_only(d_arg, sc_arg, s_args);
     // (pieces per row, their length, workgroups with work: the others leave at once)
     const uint4 cut = *reinterpret_cast<const uint4*>(sc_arg.work_n + 4);
+    // Workgroups go to the eight XCDs in turn.  The shares are dealt so that an XCD's workgroups serve consecutive
+    // ones: the workgroups of a row then sit on one XCD (two where a row straddles), whose L2 fetches the row's
+    // coarse counts and history once for all of them.  (Only if the grid holds every workgroup the deal names.)
+    {
+        const uint32_t per_xcd = (cut.z + 7u) / 8u;
+        if (per_xcd * 8u <= gridDim.x * gridDim.y) {
+            if ((wg >> 3) >= per_xcd)
+                return;
+            wg = (wg & 7u) * per_xcd + (wg >> 3);
+        }
+    }
     if (wg >= cut.z)
         return;
     const uint32_t pieces = cut.x, piece_len = cut.y, n_pieces = cut.w; // (pieces: workgroups per row)
