@@ -8,13 +8,13 @@ namespace mako {
 
 #ifdef MAKO_EMIT_TAIL_KERNEL
 // grid = (1, rows).  Rows whose sorted list sort_kernel's workers have prepared: top-p cut, exact total, draw.
-// (The batch's top-k rows were tried here too, beside the few long tails instead of ahead of the planning in
-// plan_kernel: 2.3 us less there, but this kernel's chains then compiled to slower code and lost twice that.)
 // (The context's record by value: with a pointer to it the first loads would have to wait for a trip to memory.  The
 // list's length and this workgroup's entry are asked for together, then everything the row's plan holds.)
-// Workgroups from tail_cap on: workgroup tail_cap + r finishes what the kernels before it left of row r
-// (finish_late_row()), beside the few long tails, on CUs that would otherwise idle.  (That code is kept out of line:
-// inlined, it made this kernel's chains compile to slower code.)
+// Workgroups from tail_cap on: workgroup tail_cap + r finishes what the kernels before it left of row r, beside the
+// few long tails, on CUs that would otherwise idle.  Top-k rows are finished in line; everything rarer
+// (finish_late_row()) is called out of line: inlined as well, it made this kernel's chains compile to slower code.
+// (With the top-k rows in line the compiler would make a called function of the wide rows' sorted tail instead,
+// which costs them 2 us: that call is forced in line below.)
 __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices,
                                                         uint32_t tail_cap)
 {
@@ -30,21 +30,47 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         if (r >= d_arg.n_rows)
             return;
         MAKO_ROW(kNone);
-        MAKO_ROW(kNone);
+        // (the arguments' copy for LDS, the row's parameters, the exp2 table, the candidate slots and the slices'
+        // records are asked for before anything is waited for)
+        const uint64_t tab_word = k_exp2_tab[threadIdx.x & 31u];
+        ArgWords late_words;
+        fetch_arg_words(d_arg, sc_arg, late_words);
+        fetch_param_words(d_arg, r, late_words);
+        // (a top_k == 0 row has no use for its candidate slots: a look at the row's top_k first, which costs the
+        // others a trip they have time for beside the long tails)
+        CandSlots pre;
+        const bool covered = slots_cover(slices) && d_arg.params[r].top_k != 0u; // uniform
+        if (covered)
+            fetch_candidate_slots(sc_arg, r, slices, pre);
+        const SliceStat lane_stat = load_slice_stat(sc_arg.stats, (size_t)r * kMaxSlices + min((uint32_t)lane_id(), slices - 1u));
+        place_arg_words(late_words, s_args);
         if (threadIdx.x < 32)
-            sm.tab[threadIdx.x] = k_exp2_tab[threadIdx.x];
-        stage_args(d_arg, sc_arg, r, s_args); // (its barrier publishes the table too)
+            sm.tab[threadIdx.x] = tab_word;
+        lds_barrier(); // (publishes the copy and the table; the loads above stay in flight)
         FinishLds Lr;
         Lr.sm = &sm;
         Lr.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
         Lr.sortk = s_dyn64;
         Lr.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
-        // (a top_k == 0 row that the workers and the tail above take care of needs nothing here: it leaves before the
-        // call, whose entry alone would store dozens of registers per thread)
-        if (classify(s_args.P) == kNucleus && !(d_arg.force_token || d_arg.close_token)) {
+        const RowClass late_cls = classify(s_args.P);
+        const bool plain = d_arg.force_token || d_arg.close_token; // uniform
+        // (a top_k == 0 row that the workers and the tail above take care of needs nothing here)
+        if (late_cls == kNucleus && !plain) {
             const uint32_t late_flag = sc_arg.plan[r].flag;
             if (late_flag != 2 && late_flag != 4)
                 return;
+        }
+        // A top-k row is finished here, in line: there are dozens of them beside a few long tails, and through the
+        // call below (whose entry and the entries of what it calls store dozens of registers per thread) each took
+        // longer than the longest tail.
+        if (late_cls == kTopK && !plain && !d_arg.draft && covered) {
+            float m;
+            uint32_t argidx, n_cands, any_overflow;
+            row_summary_of(lane_stat, slices, m, argidx, n_cands, any_overflow);
+            if (!topk_takes_whole_row(late_cls, any_overflow, n_cands)) {
+                topk_row(s_args.d, s_args.sc, r, slices, s_args.P, m, argidx, n_cands, lane_stat, Lr, true, pre);
+                return;
+            }
         }
         finish_late_row(s_args.d, s_args.sc, s_args.P, r, slices, Lr);
         return;
@@ -85,8 +111,12 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         plan->flag = 0;
     const uint32_t* kf = sc.key[0] + (size_t)row * sc.vpad;
     const uint32_t* jf = sc.idx[0] + (size_t)row * sc.vpad;
-    if (sorted_tail<true>(d, row, s_args.P, kf, jf, n0, true, total64, MAKO_PATH_SORTED, L, false, 0.0f, sc.gt,
-                          (size_t)row * sc.g_cap, groups))
+    // (in line whatever the compiler makes of the kernel's size: as a called function the wide rows' chains would
+    // start by storing registers)
+    bool done;
+    [[clang::always_inline]] done = sorted_tail<true>(d, row, s_args.P, kf, jf, n0, true, total64, MAKO_PATH_SORTED, L, false, 0.0f,
+                                                      sc.gt, (size_t)row * sc.g_cap, groups);
+    if (done)
         return;
     // too close to call, or the list ends before the nucleus does: the whole-row path decides
     __syncthreads();
