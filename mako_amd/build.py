@@ -34,8 +34,8 @@ INLINE_ALL = ["-mllvm", "-amdgpu-function-calls=false"]
 # slows down the start of their workgroups: not for kernels that many workgroups run (sort_kernel: +15 %).
 RARE_CALLS = ["-DMAKO_RARE_CALL=__attribute__((noinline))", "-DMAKO_REAL_CALLS=1"]
 SOURCE_FLAGS = {
-    # the late rows (top-k rows, the whole-row path, second looks at a cut) out of line beside the tails
-    "k_tail.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", "-DMAKO_TOPK_PART=__attribute__((noinline))", *RARE_CALLS],
+    # the rare late rows (the whole-row path, second looks at a cut) out of line beside the tails and the top-k rows
+    "k_tail.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", *RARE_CALLS],
     # the whole-row path and the second look at a cut that is too close to call, out of line beside the top-k rows
     "k_plan_alone.hip": RARE_CALLS,
 }

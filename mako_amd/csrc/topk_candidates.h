@@ -9,8 +9,9 @@ namespace mako {
 // Bitonic sort, descending, of 1024 * ITEMS keys held ITEMS per thread: key[t] is element t * 1024 + tid.
 // Partners 1024 or more apart are other registers of the same thread, partners less than 64 apart are lanes
 // of the same wave (shuffles); only the strides in between go through LDS (two barriers each).
-// (MAKO_TOPK_PART: __attribute__((noinline)) in a translation unit whose top-k code sits inside an out-of-line function:
-// each part then has the register file to itself instead of spilling inside its loops)
+// (MAKO_TOPK_PART: __attribute__((noinline)) for a translation unit whose top-k code sits inside an out-of-line
+// function: each part then has the register file to itself instead of spilling inside its loops.  No source sets it
+// today: every kernel has its top-k rows in line.)
 #ifndef MAKO_TOPK_PART
 #define MAKO_TOPK_PART
 #endif
