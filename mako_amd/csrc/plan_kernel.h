@@ -42,11 +42,6 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
     const mako_sampling_params& P = s_args.P;
-    FinishLds L;
-    L.sm = &sm;
-    L.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
-    L.sortk = s_dyn64;
-    L.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
     const RowClass cls = classify(P);
     if (cls != kNucleus)
         MAKO_STAMP(0);
@@ -94,10 +89,14 @@ __global__ __launch_bounds__(kThreads) void plan_kernel(mako_sample_desc d_arg, 
 
     // (a top_k == 0 row has no business here; should the host's copy of the parameters have hidden one, the whole-row
     // path serves it like any other)
-    if (cls == kNucleus || topk_takes_whole_row(cls, any_overflow, n_cands))
-        general_row<1>(d, sc, row, P, m, argidx, L);
-    else
-        topk_row(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, L, prefetched, pre);
+    // (the views of the dynamic LDS block are made where they are handed on: those that a called function receives
+    // by reference live in scratch memory, 32 bytes per thread, and only the rows that take the call should store them)
+    if (cls == kNucleus || topk_takes_whole_row(cls, any_overflow, n_cands)) {
+        const FinishLds views = finish_lds_views(sm, s_dyn64);
+        general_row<1>(d, sc, row, P, m, argidx, views);
+    } else {
+        topk_row(d, sc, row, slices, P, m, argidx, n_cands, lane_stat, finish_lds_views(sm, s_dyn64), prefetched, pre);
+    }
 }
 #endif // MAKO_EMIT_PLAN_KERNEL
 

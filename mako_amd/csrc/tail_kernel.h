@@ -47,11 +47,6 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
         if (threadIdx.x < 32)
             sm.tab[threadIdx.x] = tab_word;
         lds_barrier(); // (publishes the copy and the table; the loads above stay in flight)
-        FinishLds Lr;
-        Lr.sm = &sm;
-        Lr.cnt = reinterpret_cast<uint32_t*>(s_dyn64);
-        Lr.sortk = s_dyn64;
-        Lr.wcount = reinterpret_cast<uint32_t*>(s_dyn64 + kSortMax);
         const RowClass late_cls = classify(s_args.P);
         const bool plain = d_arg.force_token || d_arg.close_token; // uniform
         // (a top_k == 0 row that the workers and the tail above take care of needs nothing here)
@@ -68,11 +63,15 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
             uint32_t argidx, n_cands, any_overflow;
             row_summary_of(lane_stat, slices, m, argidx, n_cands, any_overflow);
             if (!topk_takes_whole_row(late_cls, any_overflow, n_cands)) {
-                topk_row(s_args.d, s_args.sc, r, slices, s_args.P, m, argidx, n_cands, lane_stat, Lr, true, pre);
+                topk_row(s_args.d, s_args.sc, r, slices, s_args.P, m, argidx, n_cands, lane_stat,
+                         finish_lds_views(sm, s_dyn64), true, pre);
                 return;
             }
         }
-        finish_late_row(s_args.d, s_args.sc, s_args.P, r, slices, Lr);
+        // (the views handed on by reference live in scratch memory, 32 bytes per thread: made here, where only the
+        // rows that take the call store them)
+        const FinishLds late_views = finish_lds_views(sm, s_dyn64);
+        finish_late_row(s_args.d, s_args.sc, s_args.P, r, slices, late_views);
         return;
     }
     // (two trips to memory before the list's records are asked for: the work list's entry with the arguments' copy

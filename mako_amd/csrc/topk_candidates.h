@@ -335,7 +335,10 @@ __device__ __forceinline__ void topk_row(const mako_sample_desc& d, const Scratc
     if (ok && sorted_tail<false, true>(d, row, P, kf, jf, min(P.top_k, n_valid), false, 0.0, MAKO_PATH_TOPK, L))
         return;
     __syncthreads(); // (the lists in LDS are done with)
-    general_row<MAKO_TOPK_GENERAL_SITE>(d, sc, row, P, m, argidx, L);
+    // (where the whole-row path is a called function the views it receives by reference live in scratch memory: a copy
+    // made here, so that only the rows that come this way store one)
+    const FinishLds views = L;
+    general_row<MAKO_TOPK_GENERAL_SITE>(d, sc, row, P, m, argidx, views);
 }
 
 } // namespace mako
