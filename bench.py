@@ -97,6 +97,55 @@ def cpu_baseline(w, budget_s):
                 sample="first %d rows of the %s batch through the plain-C oracle" % (n, w["name"])), None
 
 
+def time_other(w, steps, warmup, pool_mb, orc, stream):
+    """One more workload through the same timed loop: ms per batch, rows/s, roofline fraction, parity with the reference."""
+    from mako_amd import api, hip, workloads
+    from oracle import pyoracle
+    rows, vocab = w["logits"].shape
+    w["u"] = np.array([orc.uniforms(int(s), 1)[0] for s in w["seeds"]], np.float32)
+    ctx = api.SamplerContext(max_rows=rows, max_vocab=vocab, max_hist=w["hist"].shape[1] if "hist" in w else 0)
+    batch = api.Batch(w["logits"], w["params"], w["u"], mask=w.get("mask"), hist=w.get("hist"),
+                      hist_len=w.get("hist_len"), diagnostics=False, params_host=True)
+    n_copies = max(2, -(-pool_mb * (1 << 20) // (rows * vocab * 4)))
+    pool = [batch.d_logits] + [hip.DeviceArray.from_host(w["logits"]) for _ in range(n_copies - 1)]
+
+    def step(i):
+        batch.desc.logits = pool[i % n_copies].ptr
+        ctx.sample_batch(batch.desc, stream, params_host=batch.params_host)
+
+    for i in range(warmup):
+        step(i)
+    stream.synchronize()
+    e0, e1 = hip.Event(), hip.Event()
+    e0.record(stream)
+    for i in range(steps):
+        step(warmup + i)
+    e1.record(stream)
+    e1.synchronize()
+    ms = e0.elapsed_ms(e1) / steps
+    tokens = batch.o_tokens.download()
+    ctx.set_profile(True)
+    split = np.zeros(api.SAMPLER_KERNELS)
+    for i in range(min(steps, 10)):
+        step(warmup + steps + i)
+        split += np.array(ctx.kernel_times_ms())
+    split /= min(steps, 10)
+    ctx.close()
+    mism = None
+    ref = pyoracle.reference()
+    if ref is not None:
+        kw = dict(hist=w.get("hist"), hist_len=w.get("hist_len"), mask=w.get("mask"))
+        _, tok = ref.sample_batch_timed(w["logits"], w["params"], w["seeds"], n_threads=os.cpu_count() or 1, **kw)
+        mism = int((np.asarray(tok) != tokens).sum())
+    nbytes = rows * workloads.bytes_per_row(w)
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return dict(workload="%s: B=%d x V=%d" % (w["name"], rows, vocab), steps=steps, ms_per_batch=ms,
+                rows_per_s=rows / (ms * 1e-3), bytes_per_batch=nbytes, achieved_gbs=gbs, roofline_frac=gbs / HBM_PEAK_GBS,
+                kernel_ms=dict(zip(["scan_kernel", "finish_or_plan_kernel", "sort_kernel", "tail_kernel"],
+                                   [float(x) for x in split])),
+                parity_mismatches=mism)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -109,6 +158,9 @@ def main():
                     help="also time this many calls of the host-pointer entry point (PCIe-inclusive rate; 0 = skip)")
     ap.add_argument("--overlap-steps", type=int, default=400,
                     help="batches of the several-contexts-on-their-own-streams measurement (0 = skip)")
+    ap.add_argument("--other-steps", type=int, default=20,
+                    help="with the default workload: also time configs 4 and 5 for this many batches each and report "
+                         "them under other_configs (0 = skip)")
     ap.add_argument("--calibrate-copy-mb", type=int, default=0,
                     help="also run one device-to-device copy of this many MB (a kernel of known traffic, to scale "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -247,6 +299,15 @@ def main():
     if ref_tok is not None:
         parity = dict(rows=rows, mismatches=int((np.asarray(ref_tok) != tokens).sum()), against="reference sampler")
 
+    # BASELINE's two 256-row configurations, event-timed on the same stream with the logits rotated the same way and
+    # their tokens checked against the reference CPU sampler (untimed): beside the headline value, never part of it
+    others = None
+    if a.workload == "config3" and a.other_steps > 0:
+        others = {}
+        ctx.close()
+        for key, name in (("config4", "config4"), ("config5_0.5", "config5")):
+            others[key] = time_other(make_workload(name), a.other_steps, max(2, a.other_steps // 4), a.pool_mb, orc, stream)
+
     achieved = batch_bytes / (ms_per_step * 1e-3) / 1e9
     from mako_amd import traffic_record
     traffic = traffic_record.load_record(TRAFFIC_RECORDS[a.workload], a.workload) if a.workload in TRAFFIC_RECORDS else None
@@ -276,6 +337,7 @@ def main():
                      "scan_kernel_gbs": batch_bytes / (split[0] * 1e-3) / 1e9},
         "host_pointer_rows_per_s": host_rate,
         "overlapped_batches": overlapped,
+        "other_configs": others,
         "cpu_baseline": base,
         "parity": parity,
     }

@@ -123,19 +123,23 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx);
 
 /* Enqueues one batch on `stream` (a hipStream_t, or null for the default
  * stream) and returns without waiting: Sampler::sample / Sampler::verify
- * (src/gen/sampler.cpp:75-107) for every row.  One batch at a time per context. */
+ * (src/gen/sampler.cpp:75-107) for every row.  One batch at a time per context.
+ * If a kernel launch fails the call returns MAKO_ERR_HIP at once and the batch's outputs are undefined; the next
+ * call on the same context (for the static call: on the same GPU) first waits for the device and clears the
+ * kernels' scratch memory again, which it cannot do under stream capture (it then returns MAKO_ERR_HIP). */
 int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* desc, void* stream);
 
 /* The same call for a caller that still has the batch's parameters in HOST memory (the SamplingParams originate
  * there, src/gen/session.hpp:19-21): params_host[n_rows] must hold the same values as desc->params.  The call
  * looks at them on the calling thread and leaves out the kernels that no row of the batch needs (a batch without
- * top_k == 0 rows takes two launches instead of six).  The results never depend on it; null = the call above. */
+ * top_k == 0 rows takes two launches instead of four).  The results never depend on it; null = the call above. */
 int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_desc* desc,
                                      const mako_sampling_params* params_host, void* stream);
 
-/* mako_sampler_sample_batch for callers that must not allocate device memory around the call and want none held per
- * context: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
- * counterpart in the reference.  The kernels' scratch memory (candidate lists, histograms, sort buffers, work lists)
+/* mako_sampler_sample_batch for callers that must not allocate device memory around the call: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  (The
+ * context it is given still holds the scratch memory mako_sampler_create() allocated for it; a context made only for
+ * this call can be created with max_rows = 1 and a small max_vocab.)  The kernels' scratch memory (candidate lists, histograms, sort buffers, work lists)
  * is not the context's but an array of MAKO_STATIC_SCRATCH_MIB MiB inside the library's image, of which every GPU
  * that the library runs on holds one copy until the process ends; mako_sampler_create() looks its address up once
  * per device.  Batches of up to MAKO_STATIC_MAX_ROWS rows of up to MAKO_STATIC_MAX_VOCAB logits; anything larger is

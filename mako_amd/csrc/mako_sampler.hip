@@ -52,6 +52,7 @@ struct mako_sampler_ctx {
     uint8_t* st_acc = nullptr;
     std::string err = "";
     bool profile = false, profiled = false;
+    bool dirty = false; // a launch of the last batch failed: the scratch memory is cleared again before the next one
     uint32_t cus = 256; // compute units: workgroups of the finishing kernels that run at a time
     hipEvent_t ev[MAKO_SAMPLER_KERNELS + 1] = {};
 };
@@ -86,7 +87,7 @@ uint32_t slice_len_for(uint32_t n_vocab, uint32_t slices)
 
 
 int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampling_params* params_host, void* stream,
-              const mako::Scratch& sc, uint32_t max_rows, uint32_t max_vocab);
+              const mako::Scratch& sc, uint32_t max_rows, uint32_t max_vocab, bool* dirty);
 
 #define MAKO_STR2(x) #x
 #define MAKO_STR(x) MAKO_STR2(x)
@@ -157,7 +158,8 @@ constexpr int kStaticDevices = 64;
 constexpr uint64_t kGridYMax = 65535; // workgroups in a grid's y dimension
 struct StaticScratch {
     bool ready = false;
-    hipError_t status = hipSuccess; // of the set-up, kept: a device whose set-up failed refuses every call
+    hipError_t status = hipSuccess; // of the set-up, kept: a device whose set-up failed refuses every static call
+    bool dirty = false;             // as mako_sampler_ctx::dirty, for the device's array (under g_static_mutex)
     mako::Scratch sc{};
 };
 StaticScratch g_static[kStaticDevices];
@@ -211,6 +213,9 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     // (kMaxSlices slices of kSliceMax logits)
     if (mako_sampler_slices(max_vocab) > mako::kMaxSlices)
         return MAKO_ERR_INVALID_ARG;
+    // (the largest grid, tail_kernel's, has two workgroups per row in its y dimension)
+    if (2ull * max_rows > kGridYMax)
+        return MAKO_ERR_INVALID_ARG;
     mako_sampler_ctx* ctx = new (std::nothrow) mako_sampler_ctx;
     if (!ctx)
         return MAKO_ERR_NO_MEMORY;
@@ -228,7 +233,10 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     }
     MAKO_HIP(ctx, layout_scratch(ctx->sc, max_rows, max_vocab, [](void** p, size_t bytes) { return hipMalloc(p, bytes); }));
     MAKO_HIP(ctx, zero_scratch(ctx->sc, max_rows));
-    MAKO_HIP(ctx, setup_static_scratch(device));
+    // (a device on which the library's own array cannot be set up only refuses mako_sampler_sample_batch_static,
+    // which checks the kept status itself)
+    (void)setup_static_scratch(device);
+    (void)hipGetLastError();
     MAKO_HIP(ctx, hipDeviceSynchronize());
     // the kernels overlay 64 to 128 KB of dynamic LDS (kDynLds, kTailLds, kSortLds) on a few KB of static LDS
     MAKO_HIP(ctx, mako::init_scan_kernels());
@@ -301,7 +309,7 @@ int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_de
     if (!ctx || !desc)
         return MAKO_ERR_INVALID_ARG;
     MAKO_HIP(ctx, hipSetDevice(ctx->device));
-    return run_batch(ctx, *desc, params_host, stream, ctx->sc, ctx->max_rows, ctx->max_vocab);
+    return run_batch(ctx, *desc, params_host, stream, ctx->sc, ctx->max_rows, ctx->max_vocab, &ctx->dirty);
 }
 
 int mako_sampler_sample_batch_static(mako_sampler_ctx* ctx, const mako_sample_desc* desc, void* stream)
@@ -314,19 +322,22 @@ int mako_sampler_sample_batch_static(mako_sampler_ctx* ctx, const mako_sample_de
                     " rows of up to " MAKO_STR(MAKO_STATIC_MAX_VOCAB) " logits");
     if (ctx->device < 0 || ctx->device >= kStaticDevices)
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: no static scratch memory for this device ordinal");
-    const StaticScratch& g = g_static[ctx->device]; // (set up by mako_sampler_create(), never written afterwards)
+    StaticScratch& g = g_static[ctx->device]; // (set up by mako_sampler_create(); only `dirty` is written afterwards)
     if (!g.ready || g.status != hipSuccess)
         return fail(ctx, MAKO_ERR_HIP, "sampler: the static scratch memory could not be set up on this device");
     MAKO_HIP(ctx, hipSetDevice(ctx->device));
-    return run_batch(ctx, *desc, nullptr, stream, g.sc, MAKO_STATIC_MAX_ROWS, MAKO_STATIC_MAX_VOCAB);
+    return run_batch(ctx, *desc, nullptr, stream, g.sc, MAKO_STATIC_MAX_ROWS, MAKO_STATIC_MAX_VOCAB, &g.dirty);
 }
 
 } // extern "C"
 
 namespace {
 // One batch through the kernels, on scratch memory laid out for max_rows x max_vocab.  Allocates nothing.
+// (`dirty`: of the scratch memory the batch runs on.  The kernels rely on what the last kernels of a batch leave zero
+// (BigPlan::flag, the token counts, the work lists' lengths); a batch that stopped at a failed launch may not have
+// left it so, and the next batch on that memory clears it again first.)
 int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampling_params* params_host, void* stream,
-              const mako::Scratch& sc, uint32_t max_rows, uint32_t max_vocab)
+              const mako::Scratch& sc, uint32_t max_rows, uint32_t max_vocab, bool* dirty)
 {
     if (d.n_vocab == 0)
         return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: empty vocabulary"); // sampler.cpp:11-12
@@ -355,10 +366,23 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
                     "sampler: append_history needs hist_tokens and hist_len, and neither hist_counts nor draft");
 
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (*dirty) {
+        // an earlier batch on this scratch memory stopped at a failed launch: clear what the kernels expect to find
+        // zero, which cannot be recorded into a stream capture
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        MAKO_HIP(ctx, hipStreamIsCapturing(st, &capturing));
+        if (capturing != hipStreamCaptureStatusNone)
+            return fail(ctx, MAKO_ERR_HIP,
+                        "sampler: an earlier batch failed at a launch; the next call must come outside stream capture");
+        MAKO_HIP(ctx, hipDeviceSynchronize());
+        MAKO_HIP(ctx, zero_scratch(sc, max_rows));
+        MAKO_HIP(ctx, hipDeviceSynchronize());
+        *dirty = false;
+    }
     const uint32_t slices = mako_sampler_slices(d.n_vocab);
-    // (rows, and rows x slices, index the y dimension of the kernels' grids)
-    if ((uint64_t)d.n_rows * std::max(slices, 2u) > kGridYMax)
-        return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: n_rows x slices exceeds what one launch can index");
+    // (the largest grid, tail_kernel's, has two workgroups per row in its y dimension)
+    if (2ull * d.n_rows > kGridYMax)
+        return fail(ctx, MAKO_ERR_INVALID_ARG, "sampler: more rows than one launch can index (32767)");
     const uint32_t slice_len = slice_len_for(d.n_vocab, slices);
     const bool vec = d.n_vocab % 4 == 0 && d.logits_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(d.logits) & 15u) == 0;
     const size_t lds = d.hist_tokens ? (size_t)slice_len * sizeof(uint32_t) : 0;
@@ -396,7 +420,11 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
 #define MAKO_LAUNCH(call)                                                                                          \
     do {                                                                                                           \
         call;                                                                                                      \
-        MAKO_HIP(ctx, hipGetLastError());                                                                          \
+        const hipError_t e_launch_ = hipGetLastError();                                                            \
+        if (e_launch_ != hipSuccess) {                                                                             \
+            *dirty = true;                                                                                         \
+            return fail(ctx, MAKO_ERR_HIP, std::string(#call) + ": " + hipGetErrorString(e_launch_));             \
+        }                                                                                                          \
     } while (0)
     MAKO_MARK(0);
     MAKO_LAUNCH(mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, sc, slice_len, ctx->cus));

@@ -1210,14 +1210,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             G.w_pack()[tid] = G.pack()[tid] & kLenMask;
         __syncthreads();
     }
-#ifdef MAKO_TIMING
-    if (tid == 0 && s_mako_row == 0) {
-        g_mako_stamp[20] = groups;
-        g_mako_stamp[21] = reach;
-        g_mako_stamp[22] = n;
-    }
-    const unsigned long long tb0 = wall_clock64();
-#endif
     // A walk that will end within a few groups goes through them entry by entry, from a copy in LDS: faster than
     // the groups' maps would be to build.
     const bool head_walk = reach <= kHeadGroups; // uniform
@@ -1226,10 +1218,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         // (all the other waves: with more than kHeadGroups maps to build they take longer than the chain, even
         // though three of them share its SIMD)
         build_group_maps(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u);
-#ifdef MAKO_TIMING
-        if (tid == 64 && s_mako_row == 0)
-            g_mako_stamp[23] = wall_clock64() - tb0;
-#endif
     }
     if (wave_id() == 0) {
         // 64 groups at a time, one per lane.  A scan composes the lanes' maps; every lane then knows the state after
@@ -1259,10 +1247,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             }
         }
         MAKO_TOC(0, 17);
-#ifdef MAKO_TIMING
-        if (lane_id() == 0)
-            g_mako_stamp[19] = first;
-#endif
         MAKO_TIC(1);
         for (uint32_t base = 0; base < groups; base += kWave) {
             const uint32_t gl = min(base + lane_id(), groups - 1u);
@@ -1284,10 +1268,6 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 if (f < cnt) {
                     const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
                     const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
-#ifdef MAKO_TIMING
-                    if (lane_id() == 0 && s_mako_row == 0)
-                        g_mako_stamp[24] += 1;
-#endif
                     const uint32_t slot = (pk >> 9) & 0x7fu;
                     if (slot) {
                         const ChainState c = sum_by_quarters(kf, st, pk & kLenMask, G.quarters() + (slot - 1u) * 4u,

@@ -64,6 +64,13 @@ def synchronize():
     check(lib().hipDeviceSynchronize(), "hipDeviceSynchronize")
 
 
+def mem_get_info():
+    """(free, total) bytes of device memory on the current device."""
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    check(lib().hipMemGetInfo(C.byref(free), C.byref(total)), "hipMemGetInfo")
+    return free.value, total.value
+
+
 class DeviceArray:
     """A typed device allocation; freed with the object."""
 

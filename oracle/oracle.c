@@ -67,6 +67,13 @@ float or_expf(float x)
     return (float)(y * s);
 }
 
+/* or_expf over an array (for tests that compare millions of device results). */
+void or_expf_array(const float* x, float* y, size_t n)
+{
+    for (size_t i = 0; i < n; ++i)
+        y[i] = or_expf(x[i]);
+}
+
 /* ------------------------------------------------------------- uniforms */
 
 /* std::mt19937_64 (ISO C++ [rand.predef]) followed by libstdc++ 11.4

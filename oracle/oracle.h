@@ -19,6 +19,7 @@
 #ifndef MAKO_ORACLE_H
 #define MAKO_ORACLE_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -49,6 +50,7 @@ typedef struct {
 
 /* glibc 2.35 expf restated (FMA variant). */
 float or_expf(float x);
+void or_expf_array(const float* x, float* y, size_t n);
 
 /* n draws of generate_canonical<float,24>(mt19937_64(seed)). */
 void or_uniforms(uint64_t seed, uint32_t n, float* out);

@@ -85,6 +85,8 @@ class _Oracle:
         self.lib = lib = C.CDLL(os.path.join(_HERE, "liboracle.so"))
         lib.or_expf.restype = C.c_float
         lib.or_expf.argtypes = [C.c_float]
+        lib.or_expf_array.restype = None
+        lib.or_expf_array.argtypes = [C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_size_t]
         lib.or_uniforms.argtypes = [C.c_uint64, C.c_uint32, C.POINTER(C.c_float)]
         lib.or_sample.restype = C.c_int32
         lib.or_sample.argtypes = [C.POINTER(C.c_float), C.c_uint32, C.POINTER(Params), C.POINTER(C.c_int32),
@@ -113,6 +115,12 @@ class _Oracle:
 
     def expf(self, x):
         return self.lib.or_expf(float(x))
+
+    def expf_array(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        y = np.empty_like(x)
+        self.lib.or_expf_array(_fp(x), _fp(y), x.size)
+        return y
 
     def uniforms(self, seed, n):
         out = np.empty(n, np.float32)

@@ -30,6 +30,10 @@ def test_host_only_entry_points():
     assert lib.mako_sampler_create(None, 0, 1, 1, 0) == api.MAKO_ERR_INVALID_ARG
     p = ctypes.c_void_p()
     assert lib.mako_sampler_create(ctypes.byref(p), 0, 0, 8, 0) == api.MAKO_ERR_INVALID_ARG
+    # more rows than the kernels' grids can index (two workgroups per row in a y dimension of at most 65535), and a
+    # vocabulary of more than 64 slices: refused before anything is allocated
+    assert lib.mako_sampler_create(ctypes.byref(p), 0, 32768, 8, 0) == api.MAKO_ERR_INVALID_ARG
+    assert lib.mako_sampler_create(ctypes.byref(p), 0, 1, 64 * 16384 + 1, 0) == api.MAKO_ERR_INVALID_ARG
 
 
 def test_params_layout():

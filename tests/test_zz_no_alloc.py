@@ -4,7 +4,7 @@ second one smaller."""
 import numpy as np
 import pytest
 
-from mako_amd import api, workloads
+from mako_amd import api, hip, workloads
 from parity import oracle_rows
 
 pytestmark = pytest.mark.gpu
@@ -59,6 +59,32 @@ def test_static_scratch_matches_context_scratch(gpu_ctx, oracle):
     # and the first again: what the small call left behind does not leak into a larger one
     ref, got = _both(gpu_ctx, big)
     _same(ref, got, "16 x 129280 again")
+
+
+def test_static_call_allocates_no_device_memory(gpu_ctx):
+    """What the entry point is for: the device's free memory is the same before the first and after the last of a
+    run of static calls, of different sizes and with the per-kernel events of set_profile() recorded around them
+    (inputs and outputs are allocated before the first reading)."""
+    big = _mixed(api.STATIC_MAX_ROWS, workloads.V_DEEPSEEK, 2048, seed=7103)
+    small = _mixed(5, 32000, 300, seed=7104)
+    batches = [api.Batch(w["logits"], w["params"], w["u"], hist=w.get("hist"), hist_len=w.get("hist_len"), cand_cap=64)
+               for w in (big, small, big)]
+    gpu_ctx.set_profile(True)  # (the events are created here, not inside a call)
+    try:
+        gpu_ctx.sample_batch_static(batches[1].desc)  # (first use of every kernel: code objects are loaded by now)
+        hip.synchronize()
+        free_before, _ = hip.mem_get_info()
+        for b in batches:
+            gpu_ctx.sample_batch_static(b.desc)
+            hip.synchronize()
+            assert len(gpu_ctx.kernel_times_ms()) == api.SAMPLER_KERNELS
+        free_after, _ = hip.mem_get_info()
+    finally:
+        gpu_ctx.set_profile(False)
+    assert free_after == free_before, (free_before, free_after)
+    for b, w in zip(batches, (big, small, big)):
+        for r, (t, _) in enumerate(oracle_rows(w)):
+            assert b.results()["tokens"][r] == t
 
 
 def test_static_scratch_rejects_what_does_not_fit(gpu_ctx):
