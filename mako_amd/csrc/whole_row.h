@@ -101,6 +101,109 @@ __device__ bool radix_pass(const uint32_t* ksrc, const uint32_t* isrc, uint32_t*
 
 __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t* i1, uint32_t n, const FinishLds& L);
 
+// libstdc++'s __heap_select(first, nth + 1, last) followed by iter_swap(first, nth) (bits/stl_algo.h:1956-1960,
+// stl_heap.h): where introselect ends up when its depth limit is spent.  The arrangement it leaves is the library's,
+// entry for entry, but the time is bounded:
+//  * __make_heap sifts the parents from the last one down to the root.  A sift only touches the subtree of its
+//    node and the subtrees of one level are disjoint, so a level's sifts run side by side, one thread each, level
+//    after level from the bottom: the heap's depth in rounds instead of its size in dependent steps.
+//  * the sweep `for (i = middle; i < last; ++i) if (comp(i, first)) __pop_heap(...)` is done by one wave, 64 entries
+//    per ballot against the current root: entries that do not beat the root cost nothing, the first that does is
+//    popped in (a sequential sift from the root), the lanes behind it are asked again (the root only ever moves
+//    towards the heavy end, so whoever failed before fails again).
+//  * the heap's first `cache_cap` entries (its upper levels, or all of it) live in LDS while this runs.
+// get / put: the range in device memory or LDS, as introselect_rounds() has it.  cache: room for cache_cap values in
+// LDS (0: the range is in LDS already).  All threads call.
+template <typename Get, typename Put>
+__device__ void heap_select_rest(Get get, Put put, uint32_t first, uint32_t last, uint32_t nth, unsigned long long* cache,
+                                 uint32_t cache_cap)
+{
+    typedef unsigned long long u64;
+    const uint32_t tid = threadIdx.x, lane = lane_id();
+    const uint32_t middle = nth + 1u - first, len = last - first;
+    const uint32_t cached = min(middle, cache_cap);
+    for (uint32_t i = tid; i < cached; i += kThreads)
+        cache[i] = get(first + i);
+    __syncthreads();
+    auto hget = [&](uint32_t j) -> u64 { return j < cached ? cache[j] : get(first + j); };
+    auto hput = [&](uint32_t j, u64 v) {
+        if (j < cached)
+            cache[j] = v;
+        else
+            put(first + j, v);
+    };
+    auto sift = [&](uint32_t hole, u64 v) { // __adjust_heap: the hole sinks to a leaf, v rises from there
+        const uint32_t top = hole;
+        uint32_t child = hole;
+        while (child < (middle - 1u) / 2u) {
+            child = 2u * (child + 1u);
+            if (hget(child) < hget(child - 1u))
+                --child;
+            hput(hole, hget(child));
+            hole = child;
+        }
+        if ((middle & 1u) == 0 && middle >= 2u && child == (middle - 2u) / 2u) {
+            child = 2u * (child + 1u);
+            hput(hole, hget(child - 1u));
+            hole = child - 1u;
+        }
+        while (hole > top) {
+            const uint32_t parent = (hole - 1u) / 2u;
+            if (!(hget(parent) < v))
+                break;
+            hput(hole, hget(parent));
+            hole = parent;
+        }
+        hput(hole, v);
+    };
+    if (middle >= 2u) {
+        const uint32_t last_parent = (middle - 2u) / 2u;
+        // (node p sits on level floor(log2(p + 1)), which holds the nodes 2^level - 1 .. 2^(level + 1) - 2)
+        for (int level = 31 - __clz((int)(last_parent + 1u)); level >= 0; --level) {
+            const uint32_t lo = (1u << level) - 1u, hi = min(last_parent, (2u << level) - 2u);
+            for (uint32_t p = lo + tid; p <= hi; p += kThreads)
+                sift(p, hget(p));
+            __syncthreads();
+        }
+    }
+    if (wave_id() == 0 && middle < len) {
+        constexpr uint32_t kTrip = 4;
+        u64 root = hget(0u); // (the same in every lane)
+        for (uint32_t base = middle; base < len; base += kWave * kTrip) {
+            u64 v[kTrip];
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u)
+                v[u] = get(first + min(base + u * kWave + lane, len - 1u));
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u) {
+                const bool in = base + u * kWave + lane < len;
+                u64 bal = __ballot(in && v[u] < root);
+                while (bal) { // uniform
+                    const int l = __ffsll((long long)bal) - 1;
+                    const u64 hit = ((u64)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v[u] >> 32), l) << 32) |
+                                    (u64)(uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v[u], l);
+                    // __pop_heap(first, middle, i): the root goes to the entry's place, the entry sinks in from the root
+                    // (every lane does the same stores and loads: each then reads back what it wrote itself)
+                    put(first + base + u * kWave + (uint32_t)l, root);
+                    sift(0u, hit);
+                    root = hget(0u);
+                    bal = __ballot(in && v[u] < root) & ~((2ull << l) - 1ull);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < cached; i += kThreads)
+        put(first + i, cache[i]);
+    __syncthreads();
+    if (tid == 0) {
+        const u64 a = get(first), b = get(nth);
+        put(first, b);
+        put(nth, a);
+    }
+    __syncthreads();
+}
+
 // std::ranges::nth_element(cand, cand + nth, desc) of src/gen/sampler.cpp:41 as libstdc++ 11 runs it (introselect,
 // bits/stl_algo.h:1964), leaving the candidates in exactly the arrangement that library leaves: the reference sums
 // and walks the top_k survivors in that order when no top-p follows.  key/idx hold n candidates (~bits(q), token
@@ -109,65 +212,22 @@ __device__ void sort_segment(uint32_t* k0, uint32_t* i0, uint32_t* k1, uint32_t*
 // partition swaps the t-th entry from the left that belongs right with the t-th entry from the right that belongs
 // left for as long as the former lies before the latter, and cuts behind the entries that belong left: the two
 // position lists come from ballots (wave w owns the w-th sixteenth of the range), the swaps are independent.
-// The depth limit's heap select and the last insertion sort (at most three entries) are sequential code on one
-// thread.
+// The depth limit's heap select is heap_select_rest() above; the last insertion sort (at most three entries) is one
+// thread's.
 //
 // introselect_rounds runs the rounds on [first, last) through get(i) / put(i, v) until the range is no longer than
-// `until` (3 = to the end, insertion sort included).  lsta / lstb: room for last - first positions each.  Returns
-// true when nothing is left to do.
+// `until` (3 = to the end, insertion sort included).  lsta / lstb: room for last - first positions each.  cache /
+// cache_cap: LDS for heap_select_rest().  Returns true when nothing is left to do.
 template <typename Get, typename Put>
 __device__ bool introselect_rounds(Get get, Put put, uint32_t& first, uint32_t& last, uint32_t nth, uint32_t& depth,
-                                   uint32_t until, uint32_t* lsta, uint32_t* lstb, FinishShared& sm)
+                                   uint32_t until, uint32_t* lsta, uint32_t* lstb, FinishShared& sm,
+                                   unsigned long long* cache, uint32_t cache_cap)
 {
     typedef unsigned long long u64;
     const uint32_t tid = threadIdx.x, lane = lane_id(), wave = wave_id();
     while (last - first > until) {
         if (depth == 0) {
-            // __heap_select(first, nth + 1, last) and iter_swap(first, nth): bits/stl_algo.h:1956-1960, stl_heap.h
-            if (tid == 0) {
-                const uint32_t middle = nth + 1u - first, len = last - first;
-                auto sift = [&](uint32_t hole, u64 v) { // __adjust_heap: the hole sinks to a leaf, v rises from there
-                    const uint32_t top = hole;
-                    uint32_t child = hole;
-                    while (child < (middle - 1u) / 2u) {
-                        child = 2u * (child + 1u);
-                        if (get(first + child) < get(first + child - 1u))
-                            --child;
-                        put(first + hole, get(first + child));
-                        hole = child;
-                    }
-                    if ((middle & 1u) == 0 && middle >= 2u && child == (middle - 2u) / 2u) {
-                        child = 2u * (child + 1u);
-                        put(first + hole, get(first + child - 1u));
-                        hole = child - 1u;
-                    }
-                    while (hole > top) {
-                        const uint32_t parent = (hole - 1u) / 2u;
-                        if (!(get(first + parent) < v))
-                            break;
-                        put(first + hole, get(first + parent));
-                        hole = parent;
-                    }
-                    put(first + hole, v);
-                };
-                if (middle >= 2u)
-                    for (uint32_t parent = (middle - 2u) / 2u;; --parent) {
-                        sift(parent, get(first + parent));
-                        if (parent == 0)
-                            break;
-                    }
-                for (uint32_t i = middle; i < len; ++i) {
-                    const u64 v = get(first + i);
-                    if (v < get(first)) {
-                        put(first + i, get(first));
-                        sift(0u, v);
-                    }
-                }
-                const u64 a = get(first), b = get(nth);
-                put(first, b);
-                put(nth, a);
-            }
-            __syncthreads();
+            heap_select_rest(get, put, first, last, nth, cache, cache_cap);
             return true;
         }
         --depth;
@@ -289,7 +349,9 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
         key[i] = (uint32_t)(v >> 32);
         idx[i] = (uint32_t)v;
     };
-    if (introselect_rounds(get, put, first, last, nth, depth, kSortMax, lsta, lstb, *L.sm))
+    // (the rounds in device memory use no LDS of their own: the whole block holds the heap's upper levels if the
+    // depth limit is reached here)
+    if (introselect_rounds(get, put, first, last, nth, depth, kSortMax, lsta, lstb, *L.sm, L.sortk, kDynLds / 8u))
         return;
     u64* lds = L.sortk;
     uint32_t* la = reinterpret_cast<uint32_t*>(L.sortk + kSortMax);
@@ -300,7 +362,7 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
         lds[i] = get(base + i);
     __syncthreads();
     introselect_rounds([=](uint32_t i) { return lds[i - base]; }, [=](uint32_t i, u64 v) { lds[i - base] = v; }, first, last,
-                       nth, depth, 3u, la, lb, *L.sm);
+                       nth, depth, 3u, la, lb, *L.sm, nullptr, 0u);
     for (uint32_t i = tid; i < len; i += kThreads)
         put(base + i, lds[i]);
     __syncthreads();

@@ -196,6 +196,33 @@ def test_topk_alone_depth_limit(gpu_ctx, oracle):
         assert oracle.heap_selects() > before, "the case no longer reaches the depth limit"
 
 
+@pytest.mark.parametrize("nth", [3000, 20000, 100000])
+def test_topk_alone_depth_limit_whole_row(gpu_ctx, oracle, reference, nth):
+    """The same at full size: an adversary (McIlroy's, run against std::nth_element itself by the reference build's
+    shim) orders a 129 280-entry row so that introselect spends its depth limit while the range is still the whole row
+    in device memory, and the heap select that follows has to pop nearly every entry.  The heap holds nth + 1 entries:
+    inside LDS (3000) or only its upper levels there (20000, 100000).  The call must stay short (the sweep goes 64 entries
+    per ballot, the heap is built level by level) and leave the library's arrangement."""
+    import time
+    n = workloads.V_DEEPSEEK
+    q, _ = reference.make_nth_killer(n, nth)
+    ranks = np.unique(-q, return_inverse=True)[1]  # 0 = heaviest; equal weights keep equal logits
+    logits = (-(ranks.astype(np.float32)) * np.float32(0.0007)).reshape(1, -1)  # (every weight stays above zero)
+    p = api.make_params(1, 1.0, top_k=nth)
+    w = dict(name="nth_killer_%d_%d" % (n, nth), logits=logits, params=p, u=np.array([0.61], np.float32))
+    before = oracle.heap_selects()
+    _say("depth limit case n=%d nth=%d" % (n, nth))
+    cap = min(nth, 4096)
+    t0 = time.perf_counter()
+    g = gpu_rows(gpu_ctx, w, cap=cap)
+    dt = time.perf_counter() - t0
+    _say("  the call took %.1f ms" % (dt * 1e3))
+    assert_parity(gpu_ctx, w, cap=cap)
+    assert g["n_cand"][0] == nth
+    assert oracle.heap_selects() > before, "the case no longer reaches the depth limit"
+    assert dt < 2.0, "the depth limit's heap select took %.2f s" % dt
+
+
 def test_special_values(gpu_ctx):
     """NaN/inf logits, all-masked rows, NaN parameters: the fallbacks of src/gen/sampler.cpp:37-38."""
     v = 5000

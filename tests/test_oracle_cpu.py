@@ -233,6 +233,17 @@ def test_log_bins_host():
     assert out.returncode == 0 and " 0 failures" in out.stdout, out.stdout
 
 
+def test_heap_select_host():
+    """The depth-limit branch of the kernels' nth_element (heap_select_rest, mako_amd/csrc/whole_row.h) restated on
+    the host: libstdc++'s __make_heap level by level and its sweep 64 entries per ballot leave exactly what
+    std::__heap_select leaves (1296 cases), and the dependent steps on a whole 129 280-entry row stay within
+    ballots <= entries / 64 + pops, sift steps <= 2 x depth per pop."""
+    exe = os.path.join(HERE, "cpu", "heap_select_test")
+    subprocess.run(["g++", "-O2", "-std=c++17", os.path.join(HERE, "cpu", "heap_select_test.cpp"), "-o", exe], check=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and ": 0 failures" in out.stdout and out.stdout.strip().endswith("ok"), out.stdout
+
+
 def test_generation_helpers_known_answers():
     """LoopGuard and LookupDrafter (include/gen/) on the scenarios and numbers of the reference's own tests
     (tests/loop_guard_test.cpp, tests/lookup_test.cpp), plus a brute-force restatement of the loop rule."""
