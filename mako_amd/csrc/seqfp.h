@@ -245,6 +245,28 @@ SEQFP_HD Step32 step32(float q, int e)
     return Step32{ce, co, ce > co ? ce : co};
 }
 
+// step32() in straight-line form (the same map for every weight q >= 0 and every exponent e >= 1): no branches for a
+// GPU compiler to keep or to execute both sides of.  The host test compares the two.
+SEQFP_HD Step32 step32_flat(float q, int e)
+{
+    const uint32_t b = f2u(q);
+    const uint32_t ex = b >> 23; // (q is a weight: no sign bit)
+    const uint32_t Mq = (b & 0x7fffffu) | (ex ? 0x800000u : 0u);
+    const int d = e - int(ex ? ex : 1u);
+    const uint32_t sh = uint32_t(d < 0 ? 0 : (d > 31 ? 31 : d));
+    const uint32_t a = Mq >> sh;
+    const uint32_t rem = Mq - (a << sh);
+    const uint32_t half = (1u << sh) >> 1; // (0 when d == 0: nothing is rounded away, and rem is 0 too)
+    const uint32_t up = rem > half ? 1u : 0u;
+    const uint32_t tie = (rem == half && sh != 0u) ? 1u : 0u;
+    uint32_t ce = a + (up | (tie & a)), co = a + (up | (tie & ~a));
+    if (d > 25) // (the weight is below half a unit of the epoch's last place)
+        ce = co = 0u;
+    if (d < 0) // (a weight from a higher binade cannot be expressed)
+        ce = co = kSat;
+    return Step32{ce, co, ce > co ? ce : co};
+}
+
 // May a group's map g (built for exponent e) be applied to the running sum m * ulp(e)?  Sufficient: the state
 // after the group, plus one more of its largest increments, still lies inside the binade.
 SEQFP_HD bool group_add_ok(long long m, const Step32& g)

@@ -163,36 +163,86 @@ __device__ __forceinline__ seqfp::Step32 wave_compose_step32(seqfp::Step32 v)
 }
 
 // The map of one span for the epoch with exponent eg (eg == 0: no usable guess, the map is marked unusable).
+// An entry's map depends on the parity of the state only when the entry is an exact tie (its bits below the epoch's
+// last place are exactly one half), which is rare once the running value is far above the entries.  A span without
+// ties is a span of constant increments, and their composition is their sum (saturated like compose32()): one wave
+// reduction of one number instead of a six-step scan of two.
 __device__ __forceinline__ seqfp::Step32 span_map(const float (&q)[4], uint32_t len, int eg)
 {
     using namespace seqfp;
     Step32 st = Step32{kSat, kSat, kSat};
     if (eg > 0) { // uniform per wave
+        Step32 e[4];
+        bool tie = false;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+            e[j] = lane_id() * 4u + j < len ? seqfp::step32_flat(q[j], eg) : identity32();
+            tie |= e[j].d0 != e[j].d1;
+        }
+        if (__ballot(tie) == 0ull) {
+            // (a lane's four increments: below 2^26, or marked unusable; clamped so that 64 of them cannot wrap)
+            const uint32_t mine = min(e[0].d0 + e[1].d0 + e[2].d0 + e[3].d0, 1u << 25);
+            // (a total of 2^24 or more can never be applied, whatever its value: marked like an unusable map)
+            const uint32_t all = __ockl_wfred_add_u32(mine);
+            st.d0 = st.d1 = all < (1u << 24) ? all : kSat;
+            st.cmax = __ockl_wfred_max_u32(max(max(e[0].cmax, e[1].cmax), max(e[2].cmax, e[3].cmax)));
+            return st;
+        }
         st = identity32();
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
-            if (lane_id() * 4u + j < len)
-                st = compose32(st, step32(q[j], eg));
+            st = compose32(st, e[j]);
         st = wave_compose_step32(st);
     }
     return st;
+}
+
+// Sums and maxima inside the rows of sixteen lanes (a group's quarters), on the VALU data path: lane 15 of each row
+// ends up with its row's result (inclusive scans: row_shr 1, 2, 4, 8; lanes without a source lane add 0).
+__device__ __forceinline__ double row_scan_add_f64(double v)
+{
+#define MAKO_ROW_ADD(CTRL)                                                                                           \
+    {                                                                                                                \
+        const unsigned long long b = (unsigned long long)__double_as_longlong(v);                                    \
+        const unsigned long long t = ((unsigned long long)dpp_or_zero<CTRL, 0xf>((uint32_t)(b >> 32)) << 32) |       \
+                                     (unsigned long long)dpp_or_zero<CTRL, 0xf>((uint32_t)b);                        \
+        v += __longlong_as_double((long long)t);                                                                     \
+    }
+    MAKO_ROW_ADD(0x111)
+    MAKO_ROW_ADD(0x112)
+    MAKO_ROW_ADD(0x114)
+    MAKO_ROW_ADD(0x118)
+#undef MAKO_ROW_ADD
+    return v;
+}
+__device__ __forceinline__ uint32_t row_scan_max_u32(uint32_t v)
+{
+    v = max(v, dpp_or_zero<0x111, 0xf>(v));
+    v = max(v, dpp_or_zero<0x112, 0xf>(v));
+    v = max(v, dpp_or_zero<0x114, 0xf>(v));
+    v = max(v, dpp_or_zero<0x118, 0xf>(v));
+    return v;
+}
+// The estimate of the sum in front of each quarter of a group (quarter k = the 16 lanes of row k, four entries per lane):
+// every lane receives its own quarter's.
+__device__ __forceinline__ double sum_before_quarter(const float (&q)[4])
+{
+    const double rs = row_scan_add_f64((((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3]);
+    const double s0 = readlane_f64(rs, 15), s1 = readlane_f64(rs, 31), s2 = readlane_f64(rs, 47);
+    const uint32_t quarter = lane_id() >> 4;
+    return quarter == 0 ? 0.0 : (quarter == 1 ? s0 : (quarter == 2 ? s0 + s1 : (s0 + s1) + s2));
 }
 
 // A group inside which the running sum is expected to change binade cannot be applied as one map.  Its four
 // quarters (64 entries = the 16 lanes of one DPP row each) get maps of their own, each for the binade guessed from
 // the fp64 sum up to ITS first entry: the chain then replays only the quarter in which the change happens.
 // `at_start` is the estimate of the sum at the group's first entry.  One wave; the four records (d0, d1, cmax,
-// exponent) go to out[0..3].
+// exponent) go to out[0..3].  (No trip through LDS: the waves that meet such a group are the ones everybody waits for.)
 __device__ void build_quarters(const float (&q)[4], uint32_t len, double at_start, uint4* out)
 {
     using namespace seqfp;
     const uint32_t lane = lane_id(), quarter = lane >> 4;
-    double rs = (((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3];
-    for (int o = 1; o < 16; o <<= 1)
-        rs += __shfl_xor(rs, o);
-    const double s0 = __shfl(rs, 0), s1 = __shfl(rs, 16), s2 = __shfl(rs, 32);
-    const double before = quarter == 0 ? 0.0 : (quarter == 1 ? s0 : (quarter == 2 ? s0 + s1 : (s0 + s1) + s2));
-    const double guess = at_start + before;
+    const double guess = at_start + sum_before_quarter(q);
     const int eg = guess > 0 ? exponent_of((float)guess) : 0;
     Step32 v = Step32{kSat, kSat, kSat};
     if (eg > 0) {
@@ -200,11 +250,9 @@ __device__ void build_quarters(const float (&q)[4], uint32_t len, double at_star
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
             if (lane * 4u + j < len)
-                v = compose32(v, step32(q[j], eg));
+                v = compose32(v, step32_flat(q[j], eg));
     }
-    uint32_t cm = v.cmax;
-    for (int o = 1; o < 16; o <<= 1)
-        cm = max(cm, (uint32_t)__shfl_xor((int)cm, o));
+    const uint32_t cm = row_scan_max_u32(v.cmax);
     // inclusive scan inside the row of 16 lanes
 #define MAKO_ROW_STEP(CTRL)                                                                                          \
     {                                                                                                                \
@@ -230,12 +278,7 @@ __device__ void build_walk_quarters(const float (&q)[4], uint32_t len, double r_
 {
     using namespace seqfp;
     const uint32_t lane = lane_id(), quarter = lane >> 4;
-    double rs = (((double)q[0] + (double)q[1]) + (double)q[2]) + (double)q[3];
-    for (int o = 1; o < 16; o <<= 1)
-        rs += __shfl_xor(rs, o);
-    const double s0 = __shfl(rs, 0), s1 = __shfl(rs, 16), s2 = __shfl(rs, 32);
-    const double before = quarter == 0 ? 0.0 : (quarter == 1 ? s0 : (quarter == 2 ? s0 + s1 : (s0 + s1) + s2));
-    const double guess = r_start - before;
+    const double guess = r_start - sum_before_quarter(q);
     const int eg = guess > 0 ? exponent_of((float)guess) : 0;
     Step32 v = Step32{kSat, kSat, kSat};
     if (eg > 0) {
@@ -243,11 +286,9 @@ __device__ void build_walk_quarters(const float (&q)[4], uint32_t len, double r_
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
             if (lane * 4u + j < len)
-                v = compose32(v, step32(q[j], eg));
+                v = compose32(v, step32_flat(q[j], eg));
     }
-    uint32_t cm = v.cmax;
-    for (int o = 1; o < 16; o <<= 1)
-        cm = max(cm, (uint32_t)__shfl_xor((int)cm, o));
+    const uint32_t cm = row_scan_max_u32(v.cmax);
 #define MAKO_ROW_STEP(CTRL)                                                                                          \
     {                                                                                                                \
         const Step32 t = Step32{dpp_or_zero<CTRL, 0xf>(v.d0), dpp_or_zero<CTRL, 0xf>(v.d1), 0u};                     \
@@ -260,7 +301,11 @@ __device__ void build_walk_quarters(const float (&q)[4], uint32_t len, double r_
     MAKO_ROW_STEP(0x114)
     MAKO_ROW_STEP(0x118)
 #undef MAKO_ROW_STEP
-    const float q_first = __shfl(q[0], (int)(quarter * 16u)); // the quarter's first, largest weight
+    // the quarter's first, largest weight (lane 16 * quarter's first entry), wanted by the row's last lane
+    const uint32_t qb = __float_as_uint(q[0]);
+    const uint32_t f0 = (uint32_t)__builtin_amdgcn_readlane((int)qb, 0), f1 = (uint32_t)__builtin_amdgcn_readlane((int)qb, 16);
+    const uint32_t f2 = (uint32_t)__builtin_amdgcn_readlane((int)qb, 32), f3 = (uint32_t)__builtin_amdgcn_readlane((int)qb, 48);
+    const float q_first = __uint_as_float(quarter == 0 ? f0 : (quarter == 1 ? f1 : (quarter == 2 ? f2 : f3)));
     uint32_t Mq;
     int eq;
     split(q_first, Mq, eq);

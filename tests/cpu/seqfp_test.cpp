@@ -227,6 +227,26 @@ int main()
     std::uniform_real_distribution<float> U(0.0f, 1.0f);
     std::normal_distribution<float> N(0.0f, 1.0f);
     long fails = 0, cases = 0, rounds = 0;
+    // step32_flat() against step32(): every exponent pair, weights with ties, halves just missed, zero and subnormals
+    for (int it = 0; it < 2000000; ++it) {
+        uint32_t bits = uint32_t(rng()) & 0x7fffffffu;
+        if (it % 4 == 1)
+            bits &= ~((1u << (rng() % 24)) - 1u); // trailing zeros: exact ties at some shift
+        if (it % 4 == 2)
+            bits = (bits & 0x7f800000u) | ((1u << (rng() % 23)) + (rng() % 3) - 1u); // around a half
+        if (it % 97 == 0)
+            bits = uint32_t(rng() % 16); // zero and the smallest subnormals
+        if (bits >= 0x7f800000u)
+            continue;
+        const float q = seqfp::u2f(bits);
+        const int e = 1 + int(rng() % 254);
+        const seqfp::Step32 x = seqfp::step32(q, e), y = seqfp::step32_flat(q, e);
+        ++cases;
+        if (x.d0 != y.d0 || x.d1 != y.d1 || x.cmax != y.cmax) {
+            if (++fails < 10)
+                printf("step32_flat differs: q bits %08x e %d: %u %u %u vs %u %u %u\n", bits, e, x.d0, x.d1, x.cmax, y.d0, y.d1, y.cmax);
+        }
+    }
     for (int it = 0; it < 4000; ++it) {
         const int kind = it % 8;
         size_t n = 1 + rng() % (it % 50 == 0 ? 200000 : 3000);
