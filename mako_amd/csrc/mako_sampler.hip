@@ -127,6 +127,7 @@ hipError_t layout_scratch(mako::Scratch& sc, uint32_t max_rows, uint32_t max_voc
     MAKO_TAKE(sc.gt.start, rg);
     MAKO_TAKE(sc.gt.pack, rg);
     MAKO_TAKE(sc.gt.quarters, rg * 4);
+    MAKO_TAKE(sc.gt.walk, rg);
     MAKO_TAKE(sc.log_hist, (size_t)max_rows * sc.slices_cap * mako::kLogBins);
     MAKO_TAKE(sc.work_n, 8);
     MAKO_TAKE(sc.work_sort, (size_t)max_rows * mako::kWorkers);
@@ -253,7 +254,7 @@ void mako_sampler_destroy(mako_sampler_ctx* ctx)
         return;
     (void)hipSetDevice(ctx->device);
     mako::Scratch& sc = ctx->sc;
-    void* ptrs[] = {sc.log_hist, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters,
+    void* ptrs[] = {sc.log_hist, sc.work_n, sc.work_sort, sc.work_tail, sc.gt.sum, sc.gt.d0, sc.gt.d1, sc.gt.cmax, sc.gt.start, sc.gt.pack, sc.gt.quarters, sc.gt.walk,
                     sc.cand_w, sc.cand_i, sc.part_sum, sc.plan,
                     sc.stats,      sc.wbuf,      sc.cnt,        sc.key[0],     sc.key[1],     sc.idx[0],
                     sc.idx[1],     ctx->st_logits, ctx->st_params, ctx->st_u,   ctx->st_u2,    ctx->st_mask,

@@ -117,6 +117,8 @@ struct GroupTable {
     uint32_t* start; // first entry of the group in the sorted list
     uint32_t* pack;  // entries | guessed exponent << 16 | kHasQuarters if `quarters` holds records for the group
     uint4* quarters; // [4] per group: the maps of the group's four quarters (see build_quarters)
+    uint4* walk;     // the group's map for the walk (d0, d1, the bound of group_sub_ok, exponent) in the epoch guessed
+                     // for r at the group; exponent 0: none
 };
 
 struct Scratch {

@@ -51,6 +51,7 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     const double mass_l = rec->mass[wl];
     fetch_param_words(d_arg, row, arg_words);
     const double ps = sc_arg.part_sum[(size_t)row * kMaxSlices + lane]; // (kMaxSlices = 64 sums per row: one per lane)
+    const float u_row = d_arg.u[row]; // (for the estimate of where the row's walk starts)
     asm volatile("" ::"s"(flag), "s"(overflow), "s"(thr_bits), "v"(handed), "v"(room), "v"(stage_l), "v"(key_lo_l),
                  "v"(mass_l), "v"(ps), "v"(arg_words.p));
     if ((flag != 1 && flag != 3) || (flag == 3 && w != 0)) // (never: the list holds exactly the flagged rows' pieces)
@@ -166,8 +167,11 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         MAKO_STAMP(11);
         // (the guess of the running sum before the share: the plan's estimate, in the exact total's units)
         const double mass_w = readlane_f64(mass_l, w);
+        // (the walk starts from u * (the nucleus' fp32 total), which is top_p * total64 and at most one weight more;
+        // a verification row's walk is replayed by other code)
+        const double r0 = d.draft ? 0.0 : (double)u_row * ((double)s_args.P.top_p * total64);
         worker_groups(key0, off, cnt, t_row + gbase, mass_all > 0.0 ? mass_w * (total64 / mass_all) : 0.0, sc.gt, L,
-                      (in_lds && sorted) ? sorted_copy : nullptr);
+                      (in_lds && sorted) ? sorted_copy : nullptr, r0 == r0 ? r0 : 0.0);
         MAKO_STAMP(12);
     }
 }

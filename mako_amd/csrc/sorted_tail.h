@@ -151,22 +151,13 @@ __device__ __forceinline__ void load_span(const uint32_t* kf, uint32_t start, ui
     load_span(AnyKeys{kf}, start, len, q);
 }
 
-// Composition of the 64 lanes' maps in lane order; every lane receives the result.
-__device__ __forceinline__ seqfp::Step32 wave_compose_step32(seqfp::Step32 v)
-{
-    wave_scan_maps(v.d0, v.d1);
-    seqfp::Step32 r;
-    r.d0 = (uint32_t)__builtin_amdgcn_readlane((int)v.d0, kWave - 1);
-    r.d1 = (uint32_t)__builtin_amdgcn_readlane((int)v.d1, kWave - 1);
-    r.cmax = __ockl_wfred_max_u32(v.cmax);
-    return r;
-}
-
-// The map of one span for the epoch with exponent eg (eg == 0: no usable guess, the map is marked unusable).
+// The map of one span OF A DESCENDING LIST for the epoch with exponent eg (eg == 0: no usable guess, the map is marked
+// unusable).
 // An entry's map depends on the parity of the state only when the entry is an exact tie (its bits below the epoch's
 // last place are exactly one half), which is rare once the running value is far above the entries.  A span without
 // ties is a span of constant increments, and their composition is their sum (saturated like compose32()): one wave
-// reduction of one number instead of a six-step scan of two.
+// reduction of one number instead of a six-step scan of two.  The largest single step is the first entry's (a weight's
+// step never grows as the weight falls): no reduction at all.
 __device__ __forceinline__ seqfp::Step32 span_map(const float (&q)[4], uint32_t len, int eg)
 {
     using namespace seqfp;
@@ -176,23 +167,27 @@ __device__ __forceinline__ seqfp::Step32 span_map(const float (&q)[4], uint32_t 
         bool tie = false;
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            e[j] = lane_id() * 4u + j < len ? seqfp::step32_flat(q[j], eg) : identity32();
+            e[j] = lane_id() * 4u + j < len ? step32_flat(q[j], eg) : identity32();
             tie |= e[j].d0 != e[j].d1;
         }
+        const uint32_t cmax = (uint32_t)__builtin_amdgcn_readfirstlane((int)e[0].cmax);
         if (__ballot(tie) == 0ull) {
             // (a lane's four increments: below 2^26, or marked unusable; clamped so that 64 of them cannot wrap)
             const uint32_t mine = min(e[0].d0 + e[1].d0 + e[2].d0 + e[3].d0, 1u << 25);
             // (a total of 2^24 or more can never be applied, whatever its value: marked like an unusable map)
             const uint32_t all = __ockl_wfred_add_u32(mine);
             st.d0 = st.d1 = all < (1u << 24) ? all : kSat;
-            st.cmax = __ockl_wfred_max_u32(max(max(e[0].cmax, e[1].cmax), max(e[2].cmax, e[3].cmax)));
+            st.cmax = cmax;
             return st;
         }
         st = identity32();
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
             st = compose32(st, e[j]);
-        st = wave_compose_step32(st);
+        wave_scan_maps(st.d0, st.d1);
+        st.d0 = (uint32_t)__builtin_amdgcn_readlane((int)st.d0, kWave - 1);
+        st.d1 = (uint32_t)__builtin_amdgcn_readlane((int)st.d1, kWave - 1);
+        st.cmax = cmax;
     }
     return st;
 }
@@ -323,6 +318,26 @@ __device__ void build_walk_quarters(const float (&q)[4], uint32_t len, double r_
         out[quarter] = make_uint4(v.d0, v.d1, need, (uint32_t)eg);
 }
 
+// group_sub_ok() as one bound, for a span of a descending list whose first (largest) weight is q_first and whose map
+// for the epoch with exponent eg has the largest single step cmax: the state after the span must be at least the
+// bound, which keeps it inside the binade with room for one more decrement and at or above that weight, so that
+// nothing in the span stopped the walk.
+__device__ __forceinline__ uint32_t walk_need(float q_first, int eg, uint32_t cmax)
+{
+    uint32_t Mq;
+    int eq;
+    seqfp::split(q_first, Mq, eq);
+    const int dl = eg - eq;
+    uint32_t need = 1u;
+    if (dl < 0)
+        need = 1u << 31;
+    else if (dl <= 25)
+        need = max(1u, (uint32_t)(((unsigned long long)Mq + (1ull << dl) - 1ull) >> dl));
+    if (eg > 1)
+        need = max(need, min(cmax, 1u << 30) + (1u << 23) + 1u);
+    return need;
+}
+
 // Group maps of groups [g_begin, groups) for epochs guessed from pg: of the running sum (walk == false, into G.d0 /
 // d1 / cmax / pack) or of the walk (into G.w_d0 / w_d1 / w_need / w_pack; r0 - pg[g] is the estimate of r at group
 // g).  The calling wave is number `part` of `parts` that share the work.
@@ -340,60 +355,50 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
     for (uint32_t g0 = g_begin + part; g0 < groups; g0 += parts * 4u) {
         float q[4][4];
         uint32_t len[4];
+        double guess[4];
+        int eg[4];
+        bool crossing[4], keep[4];
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
             const uint32_t g = min(g0 + u * parts, groups - 1u);
+            guess[u] = walk ? r0 - G.pg()[g] : G.pg()[g];
+            eg[u] = guess[u] > 0 ? exponent_of((float)guess[u]) : 0;
+            // a group in which the running sum (or r) is expected to change binade, or which starts from zero, gets
+            // quarter records
+            const double at_end = walk ? r0 - G.pg()[g + 1] : G.pg()[g + 1];
+            const int e_end = at_end > 0 ? exponent_of((float)at_end) : 0;
+            crossing[u] = uniform_u32((uint32_t)(e_end != eg[u])) != 0 || (!walk && g == 0);
+            // (a walk's map that a worker of sort_kernel has left for this very epoch is the map built here: kept)
+            keep[u] = walk && !crossing[u] && eg[u] > 0 && uniform_u32(o_pack[g] >> 16) == (uint32_t)eg[u];
             len[u] = uniform_u32(G.pack()[g] & kLenMask);
-            load_span(kf, uniform_u32(G.start()[g]), len[u], q[u]);
+            load_span(kf, uniform_u32(G.start()[g]), keep[u] ? 0u : len[u], q[u]);
         }
 #pragma unroll
         for (uint32_t u = 0; u < 4; ++u) {
             const uint32_t g = g0 + u * parts;
             if (g >= groups) // uniform
                 break;
-            const double guess = g < groups ? (walk ? r0 - G.pg()[g] : G.pg()[g]) : 0.0;
-            const int eg = guess > 0 ? exponent_of((float)guess) : 0;
-            const Step32 st = span_map(q[u], len[u], eg);
-            // a group in which the running sum (or r) is expected to change binade, or which starts from zero, gets
-            // quarter records
+            if (keep[u]) // uniform
+                continue;
+            const Step32 st = span_map(q[u], len[u], eg[u]);
             uint32_t slot = 0;
-            if (g < groups) { // uniform
-                const double at_end = walk ? r0 - G.pg()[g + 1] : G.pg()[g + 1];
-                const int e_end = at_end > 0 ? exponent_of((float)at_end) : 0;
-                if (uniform_u32((uint32_t)(e_end != eg)) || (!walk && g == 0)) {
-                    if (lane_id() == 0)
-                        slot = atomicAdd(&G.misc()[3], 1u) + 1u;
-                    slot = uniform_u32(slot);
-                    if (slot > kQuarterSlots)
-                        slot = 0;
-                    else if (walk)
-                        build_walk_quarters(q[u], len[u], guess, G.quarters() + (slot - 1u) * 4u);
-                    else
-                        build_quarters(q[u], len[u], G.pg()[g], G.quarters() + (slot - 1u) * 4u);
-                }
+            if (crossing[u]) {
+                if (lane_id() == 0)
+                    slot = atomicAdd(&G.misc()[3], 1u) + 1u;
+                slot = uniform_u32(slot);
+                if (slot > kQuarterSlots)
+                    slot = 0;
+                else if (walk)
+                    build_walk_quarters(q[u], len[u], guess[u], G.quarters() + (slot - 1u) * 4u);
+                else
+                    build_quarters(q[u], len[u], G.pg()[g], G.quarters() + (slot - 1u) * 4u);
             }
-            if (lane_id() == 0 && g < groups) {
-                uint32_t third = st.cmax;
-                if (walk) {
-                    // group_sub_ok as one bound (lane 0 holds the group's first, largest weight): the state after
-                    // the group must be at least `third`, which keeps it inside the binade with room for one
-                    // more decrement and at or above that weight, so that nothing in the group stopped the walk
-                    uint32_t Mq;
-                    int eq;
-                    split(q[u][0], Mq, eq);
-                    const int dl = eg - eq;
-                    third = 1u;
-                    if (dl < 0)
-                        third = 1u << 31;
-                    else if (dl <= 25)
-                        third = max(1u, (uint32_t)(((unsigned long long)Mq + (1ull << dl) - 1ull) >> dl));
-                    if (eg > 1)
-                        third = max(third, min(st.cmax, 1u << 30) + (1u << 23) + 1u);
-                }
+            if (lane_id() == 0) {
+                // (walk: lane 0 holds the group's first, largest weight)
                 o_d0[g] = st.d0;
                 o_d1[g] = st.d1;
-                o_c[g] = third;
-                o_pack[g] = len[u] | (slot << 9) | ((uint32_t)eg << 16);
+                o_c[g] = walk ? walk_need(q[u][0], eg[u], st.cmax) : st.cmax;
+                o_pack[g] = len[u] | (slot << 9) | ((uint32_t)eg[u] << 16);
             }
         }
     }
@@ -1025,9 +1030,10 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     // loads before these are out)
     double r_sum = 0.0;
     uint32_t r_d0 = 0, r_d1 = 0, r_cm = 0, r_st = 0, r_pk = 0;
-    uint4 qr0 = make_uint4(0, 0, 0, 0), qr1 = qr0, qr2 = qr0, qr3 = qr0;
+    uint4 qr0 = make_uint4(0, 0, 0, 0), qr1 = qr0, qr2 = qr0, qr3 = qr0, r_walk = qr0;
     if constexpr (PLANNED) {
         if (tid < groups1) {
+            r_walk = T.walk[t_base + tid];
             r_sum = T.sum[t_base + tid];
             r_d0 = T.d0[t_base + tid];
             r_d1 = T.d1[t_base + tid];
@@ -1071,6 +1077,11 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             }
             G.start()[tid] = st;
             G.pack()[tid] = min(pk & kLenMask, min(kGroup, n1 - st)) | (slot << 9) | (pk & 0x00ff0000u);
+            // (the worker's map for the walk, for the length the worker saw; see the walk's w_pack below)
+            G.w_d0()[tid] = r_walk.x;
+            G.w_d1()[tid] = r_walk.y;
+            G.w_need()[tid] = r_walk.z;
+            G.w_pack()[tid] = (pk & kLenMask) | ((r_walk.w & 0xffu) << 16);
         }
     } else {
         if (tid < groups1) {
@@ -1251,8 +1262,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     {
         const uint32_t beyond = (tid < groups && !(r0_guess * 1.001 - G.pg()[tid] > 0)) ? tid : kNone;
         reach = min(groups, block_min_u32(beyond, sm.bs));
-        if (tid < groups)
-            G.w_pack()[tid] = G.pack()[tid] & kLenMask;
+        if (tid < groups) {
+            // (a planned list's groups come with the workers' maps for the walk: one that was made for the length the
+            // group has after the cut stays, with its exponent; the others are built when the walk gets to them)
+            const uint32_t len = G.pack()[tid] & kLenMask;
+            const uint32_t left = PLANNED ? G.w_pack()[tid] : 0u;
+            G.w_pack()[tid] = (PLANNED && (left & kLenMask) == len) ? (left & (0x00ff0000u | kLenMask)) : len;
+        }
         __syncthreads();
     }
     // A walk that will end within a few groups goes through them entry by entry, from a copy in LDS: faster than

@@ -271,8 +271,10 @@ __device__ bool lds_sort_staged_runs(const uint32_t* ks, const uint32_t* is, uin
 // Group records of a worker's sorted range (cnt entries from position off of the list kf): fp64 sums, and the
 // maps of the running fp32 sum for the epoch guessed from the mass above the range plus the sums before the group.
 // kf_lds (optional): the worker's cnt sorted weights in LDS (outside L.sortk's first 16 KB), read instead of kf + off.
+// r0: the estimate of where the walk starts, u * top_p * (the row's total): the groups that r can reach also get their
+// map for the walk, for the epoch guessed from r0 less the mass before the group (0 or less: none).
 __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, size_t t_at, double mass, const GroupTable& T,
-                              const FinishLds L, const uint32_t* kf_lds = nullptr)
+                              const FinishLds L, const uint32_t* kf_lds = nullptr, double r0 = 0.0)
 {
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
@@ -337,12 +339,21 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
         const bool split4 = uniform_u32((uint32_t)(eg == 0 || exponent_of((float)at_end) != eg)) != 0;
         if (split4)
             build_quarters(q, len, guess, T.quarters + (t_at + g) * 4u);
+        // the walk's map, where the walk is expected to pass the group without changing binade in it
+        const double r_here = r0 - guess, r_after = r0 - at_end;
+        const int ew = (r0 > 0.0 && r_after > 0.0) ? exponent_of((float)r_here) : 0;
+        uint4 wrec = make_uint4(0u, 0u, 0u, 0u);
+        if (ew > 0 && uniform_u32((uint32_t)(exponent_of((float)r_after) == ew)) != 0) {
+            const seqfp::Step32 sw = span_map(q, len, ew);
+            wrec = make_uint4(sw.d0, sw.d1, walk_need(q[0], ew, sw.cmax), (uint32_t)ew); // (lane 0: the group's first weight)
+        }
         if (lane_id() == 0) {
             T.d0[t_at + g] = st.d0;
             T.d1[t_at + g] = st.d1;
             T.cmax[t_at + g] = st.cmax;
             T.start[t_at + g] = off + g * kGroup;
             T.pack[t_at + g] = len | ((uint32_t)eg << 16) | (split4 ? kHasQuarters : 0u);
+            T.walk[t_at + g] = wrec;
         }
     }
 }
