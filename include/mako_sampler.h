@@ -181,6 +181,13 @@ uint32_t mako_sampler_slices(uint32_t n_vocab);
 int mako_sampler_debug_expf(const float* x_dev, float* y_dev, uint32_t n, void* stream);
 int mako_sampler_debug_div(const float* a_dev, const float* b_dev, float* y_dev, uint32_t n, void* stream);
 
+/* Checked builds of the library (libmako_sampler_checked.so, -DMAKO_CHECKED) compare every index their kernels
+ * compute into the context's scratch arrays with the array's bound and record failures instead of trapping: this call
+ * waits for the device, returns the failed checks of all batches since the last call as a bit set in *out_bits and
+ * clears them.  Bit 31 is set by every batch of a checked build (the checks are there); the other bits name checks that
+ * failed.  The shipped library has no checks compiled in and always reports 0. */
+int mako_sampler_debug_checks(mako_sampler_ctx* ctx, uint32_t* out_bits);
+
 #ifdef __cplusplus
 }
 #endif

@@ -97,17 +97,21 @@ EXPORTS = [
     "mako_sampler_kernel_times",
     "mako_sampler_debug_expf",
     "mako_sampler_debug_div",
+    "mako_sampler_debug_checks",
 ]
 
-_lib = None
+_libs = {}
+# the library with the kernels' index checks compiled in (mako_amd/build.py, checked=True): tests only
+CHECKED_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmako_sampler_checked.so")
 
 
-def load():
-    global _lib
-    if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            raise RuntimeError("libmako_sampler.so is not built: run `python -m mako_amd.build` (needs hipcc)")
-        lib = C.CDLL(LIB_PATH)
+def load(path=None):
+    """The C-ABI library (LIB_PATH unless another build of it is named), loaded once per path."""
+    path = path or LIB_PATH
+    if path not in _libs:
+        if not os.path.exists(path):
+            raise RuntimeError("%s is not built: run `python -m mako_amd.build` (needs hipcc)" % os.path.basename(path))
+        lib = C.CDLL(path)
         lib.mako_sampler_create.argtypes = [C.POINTER(C.c_void_p), C.c_int, C.c_uint32, C.c_uint32, C.c_uint32]
         lib.mako_sampler_destroy.argtypes = [C.c_void_p]
         lib.mako_sampler_sample_batch.argtypes = [C.c_void_p, C.POINTER(Desc), C.c_void_p]
@@ -124,8 +128,9 @@ def load():
         lib.mako_sampler_sample_host.argtypes = [
             C.c_void_p, C.c_void_p, C.c_int64, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
             C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
-        _lib = lib
-    return _lib
+        lib.mako_sampler_debug_checks.argtypes = [C.c_void_p, C.POINTER(C.c_uint32)]
+        _libs[path] = lib
+    return _libs[path]
 
 
 class MakoError(RuntimeError):
@@ -135,8 +140,8 @@ class MakoError(RuntimeError):
 class SamplerContext:
     """Owner of a mako_sampler_ctx."""
 
-    def __init__(self, max_rows, max_vocab, max_hist=0, device=0):
-        self.lib = load()
+    def __init__(self, max_rows, max_vocab, max_hist=0, device=0, lib_path=None):
+        self.lib = load(lib_path)
         p = C.c_void_p()
         rc = self.lib.mako_sampler_create(C.byref(p), device, max_rows, max_vocab, max_hist)
         self.ptr = p.value
@@ -159,6 +164,14 @@ class SamplerContext:
 
     def last_error(self):
         return self.lib.mako_sampler_last_error(self.ptr).decode()
+
+    def failed_checks(self):
+        """Bit set of the index checks that failed since the last call (always 0 unless the library is the checked build)."""
+        bits = C.c_uint32(0)
+        rc = self.lib.mako_sampler_debug_checks(self.ptr, C.byref(bits))
+        if rc != MAKO_OK:
+            raise MakoError("mako_sampler_debug_checks: %d %s" % (rc, self.last_error()))
+        return int(bits.value)
 
     def set_profile(self, enabled):
         rc = self.lib.mako_sampler_set_profile(self.ptr, 1 if enabled else 0)

@@ -10,6 +10,9 @@ CSRC = os.path.join(HERE, "csrc")
 SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_alone.hip", "k_sort.hip", "k_tail.hip"]
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 OUT = os.path.join(HERE, "libmako_sampler.so")
+# the same library with the kernels' index checks compiled in (-DMAKO_CHECKED): for the test that runs the workloads
+# under it and expects no check to fail; never the library that is benchmarked
+OUT_CHECKED = os.path.join(HERE, "libmako_sampler_checked.so")
 
 # Bit-exactness against the host toolchain needs: no FMA contraction, IEEE fp32
 # division, subnormals kept.  Packed-fp32 instructions stay off.
@@ -41,12 +44,14 @@ SOURCE_FLAGS = {
 }
 
 
-def build(verbose=False, extra=(), jobs=8):
+def build(verbose=False, extra=(), jobs=8, checked=False):
     from concurrent.futures import ThreadPoolExecutor
     os.makedirs(OBJ_DIR, exist_ok=True)
+    if checked:
+        extra = (*extra, "-DMAKO_CHECKED=1")
 
     def compile_one(name):
-        obj = os.path.join(OBJ_DIR, os.path.splitext(name)[0] + ".o")
+        obj = os.path.join(OBJ_DIR, os.path.splitext(name)[0] + ("_checked.o" if checked else ".o"))
         cmd = ["hipcc", *FLAGS, *SOURCE_FLAGS.get(name, INLINE_ALL), *extra, "-c", os.path.join(CSRC, name), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -55,12 +60,14 @@ def build(verbose=False, extra=(), jobs=8):
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(compile_one, SOURCES))
-    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", OUT]
+    out = OUT_CHECKED if checked else OUT
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    return OUT
+    return out
 
 
 if __name__ == "__main__":
     build(verbose=True, extra=sys.argv[1:])
+    build(verbose=True, extra=sys.argv[1:], checked=True)

@@ -547,6 +547,17 @@ int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t
     return MAKO_OK;
 }
 
+int mako_sampler_debug_checks(mako_sampler_ctx* ctx, uint32_t* out_bits)
+{
+    if (!ctx || !out_bits)
+        return MAKO_ERR_INVALID_ARG;
+    MAKO_HIP(ctx, hipSetDevice(ctx->device));
+    MAKO_HIP(ctx, hipDeviceSynchronize());
+    MAKO_HIP(ctx, hipMemcpy(out_bits, ctx->sc.work_n + 2, sizeof(uint32_t), hipMemcpyDeviceToHost));
+    MAKO_HIP(ctx, hipMemset(ctx->sc.work_n + 2, 0, sizeof(uint32_t)));
+    return MAKO_OK;
+}
+
 int mako_sampler_debug_expf(const float* x_dev, float* y_dev, uint32_t n, void* stream)
 {
     if (!x_dev || !y_dev)

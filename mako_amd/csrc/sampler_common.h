@@ -142,8 +142,9 @@ struct Scratch {
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
     // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
     // (finish_kernel and plan_kernel get the same effect from find_piece().)
-    uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); then, 16-byte aligned at [4],
-                           // how the second pass is cut up (SecondPassCut; scan_kernel's first workgroup decides)
+    uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); [2]: failed checks of a checked
+                           // build (MAKO_CHECK); then, 16-byte aligned at [4], how the second pass is cut up
+                           // (SecondPassCut; scan_kernel's first workgroup decides)
     uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel
     uint32_t* work_tail;   // [max_rows] row; appended by finish_kernel
     uint64_t vpad;
@@ -152,6 +153,29 @@ struct Scratch {
 };
 
 static_assert(offsetof(Scratch, gt) % 16 == 0 && sizeof(mako_sample_desc) % 16 == 0, "128-bit LDS reads of the staged records");
+
+// Checked builds (-DMAKO_CHECKED, libmako_sampler_checked.so): every index a kernel computes into the context's scratch
+// arrays from counts that other kernels left is compared with the array's bound before it is used, and a failed
+// comparison sets a bit of Scratch::work_n[2] (nothing traps; mako_sampler_debug_checks() reads and clears the word).
+// The shipped library compiles the checks to nothing: its hot code clamps where it must and assumes the rest.
+enum CheckBit {
+    kCheckCandSlot = 0,   // scan_kernel: a candidate's slot in its slice's list
+    kCheckStage = 1,      // second pass: an entry's place in the row's staging arrays
+    kCheckShare = 2,      // sort_kernel: a worker's share and its place in the sorted list
+    kCheckGroups = 3,     // sort_kernel: a worker's group records
+    kCheckTailGroup = 4,  // tail_kernel: the list's length and group count as sort_kernel left them
+    kCheckCompact = 5,    // the whole-row path: a candidate's place in the compacted list
+    kCheckAlive = 31,     // set by every batch of a checked build: the checks are compiled in and their word is read
+};
+#ifdef MAKO_CHECKED
+#define MAKO_CHECK(sc, bit, cond)                                                                                    \
+    do {                                                                                                             \
+        if (!(cond))                                                                                                 \
+            atomicOr(&(sc).work_n[2], 1u << (bit));                                                                  \
+    } while (0)
+#else
+#define MAKO_CHECK(sc, bit, cond) ((void)0)
+#endif
 
 // Device functions that only rare rows reach (the whole-row path, the second look at a cut that is too close to
 // call).  The sources whose kernels have a hot path beside them are compiled with MAKO_RARE_CALL=__attribute__((noinline)):

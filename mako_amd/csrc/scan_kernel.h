@@ -77,6 +77,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 
         if (row == 0 && slice == 0) { // the lists finish_kernel and plan_kernel append to start empty
             sc.work_n[0] = 0;
             sc.work_n[1] = 0;
+            MAKO_CHECK(sc, kCheckAlive, false);
         }
     }
     static_assert(kLogBins == (uint32_t)kThreads, "one bin per thread");
@@ -236,6 +237,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 
         st.n_emit = min(n, kCap);
         st.tau_key = tau_key;
         const size_t base = ((size_t)row * sc.slices_cap + slice) * kCap;
+        MAKO_CHECK(sc, kCheckCandSlot, st.n_emit <= kCap && slice < sc.slices_cap);
         if (tid < st.n_emit) {
             sc.cand_w[base + tid] = sm.cw[tid];
             sc.cand_i[base + tid] = sm.ci[tid];

@@ -177,6 +177,8 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
                 const uint32_t w = wbuf[e - from];
                 if (e < pl.lim[w]) {
                     const uint2 x = buf[e - from];
+                    MAKO_CHECK(sc, kCheckStage, (uint64_t)(pl.goff[w] + e) < sc.vpad && pl.goff[w] + e >= pl.stage_off[w] &&
+                                                    pl.goff[w] + e < pl.stage_off[w] + pl.cap[w]);
                     kstage[pl.goff[w] + e] = x.x;
                     istage[pl.goff[w] + e] = x.y;
                 } else {

@@ -131,6 +131,8 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
             plan->flag = 2;
         return;
     }
+    MAKO_CHECK(sc, kCheckShare, (uint64_t)stage + cnt <= sc.vpad && (uint64_t)(cnt_upto - cnt_l) + cnt_l <= sc.vpad && n0 <= d.n_vocab);
+    MAKO_CHECK(sc, kCheckGroups, grp_upto <= sc.g_cap);
     if (w == 0 && tid == 0) {
         plan->n0 = n0;
         plan->groups = groups;

@@ -112,6 +112,7 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     const uint32_t* jf = sc.idx[0] + (size_t)row * sc.vpad;
     // (in line whatever the compiler makes of the kernel's size: as a called function the wide rows' chains would
     // start by storing registers)
+    MAKO_CHECK(sc, kCheckTailGroup, plan_n0 <= d.n_vocab && plan_groups <= min(kMaxGroups, sc.g_cap));
     bool done;
     [[clang::always_inline]] done = sorted_tail<true>(d, row, s_args.P, kf, jf, n0, true, total64, MAKO_PATH_SORTED, L, false, 0.0f,
                                                       sc.gt, (size_t)row * sc.g_cap, groups);

@@ -606,6 +606,7 @@ __device__ MAKO_RARE_CALL void general_row(const mako_sample_desc& d, const Scra
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j)
             if (k[j]) {
+                MAKO_CHECK(sc, kCheckCompact, pos < n0 && (uint64_t)pos < sc.vpad);
                 key0[pos] = ~k[j];
                 idx0[pos] = i + j;
                 ++pos;
