@@ -1076,17 +1076,20 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 gq[3] = qr3;
             }
             G.start()[tid] = st;
-            G.pack()[tid] = min(pk & kLenMask, min(kGroup, n1 - st)) | (slot << 9) | (pk & 0x00ff0000u);
-            // (the worker's map for the walk, for the length the worker saw; see the walk's w_pack below)
+            const uint32_t len = min(pk & kLenMask, min(kGroup, n1 - st));
+            G.pack()[tid] = len | (slot << 9) | (pk & 0x00ff0000u);
+            // (the worker's map for the walk, if it was made for the length the group has here: with its exponent;
+            // the cut takes the exponent away again from the group it shortens, and the walk builds what is missing)
             G.w_d0()[tid] = r_walk.x;
             G.w_d1()[tid] = r_walk.y;
             G.w_need()[tid] = r_walk.z;
-            G.w_pack()[tid] = (pk & kLenMask) | ((r_walk.w & 0xffu) << 16);
+            G.w_pack()[tid] = (pk & kLenMask) == len ? (len | ((r_walk.w & 0xffu) << 16)) : len;
         }
     } else {
         if (tid < groups1) {
             G.start()[tid] = tid * kGroup;
             G.pack()[tid] = min(kGroup, n1 - tid * kGroup);
+            G.w_pack()[tid] = min(kGroup, n1 - tid * kGroup); // (no exponent: the walk's maps are built when it gets there)
         }
         for (uint32_t g0 = wave_id() * 4u; g0 < groups1; g0 += kWaves * 4u) {
             float q[4][4];
@@ -1147,8 +1150,10 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         if (gs != kNone && exact) {
             const uint32_t st = G.start()[gs], len = G.pack()[gs] & kLenMask, keep = G.misc()[0] - st;
             __syncthreads();
-            if (tid == 0 && keep != len)
+            if (tid == 0 && keep != len) {
                 G.pack()[gs] = keep;
+                G.w_pack()[gs] = keep;
+            }
             __syncthreads();
             n = uniform_u32(G.misc()[0]);
             groups = uniform_u32(gs + 1u);
@@ -1183,8 +1188,10 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 }
                 if (lane_id() == 0) {
                     G.misc()[0] = ok ? st + keep : kNone;
-                    if (ok && keep != len)
-                        G.pack()[gs] = keep; // shortened: the prepared map no longer applies (exponent 0)
+                    if (ok && keep != len) {
+                        G.pack()[gs] = keep; // shortened: the prepared maps no longer apply (exponent 0)
+                        G.w_pack()[gs] = keep;
+                    }
                 }
             }
             __syncthreads();
@@ -1250,26 +1257,24 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     }
 
     // exact fp32 total: group maps in parallel (here, or already by the workers), then one wave chains them
-    if (!PLANNED)
+    if (!PLANNED) {
         build_group_maps(kf, groups, false, 0.0, G);
-    __syncthreads();
+        __syncthreads();
+    }
     MAKO_STAMP(13);
     // While one wave chains the running sum, the others already prepare the walk: its maps only need the binade r is
     // expected to be in at each group, and the fp64 sums give that (a wrong guess costs a replay, never the result).
-    // Groups that start after the mass r0 could have is used up get no map.
+    // Groups that start after the mass r0 could have is used up get no map.  (Every wave finds that group for itself,
+    // 64 groups per ballot: no barrier stands between the cut and the chain.)
     const double r0_guess = (double)u_row * G.pg()[groups];
-    uint32_t reach;
-    {
-        const uint32_t beyond = (tid < groups && !(r0_guess * 1.001 - G.pg()[tid] > 0)) ? tid : kNone;
-        reach = min(groups, block_min_u32(beyond, sm.bs));
-        if (tid < groups) {
-            // (a planned list's groups come with the workers' maps for the walk: one that was made for the length the
-            // group has after the cut stays, with its exponent; the others are built when the walk gets to them)
-            const uint32_t len = G.pack()[tid] & kLenMask;
-            const uint32_t left = PLANNED ? G.w_pack()[tid] : 0u;
-            G.w_pack()[tid] = (PLANNED && (left & kLenMask) == len) ? (left & (0x00ff0000u | kLenMask)) : len;
+    uint32_t reach = groups;
+    for (uint32_t g0 = 0; g0 < groups; g0 += kWave) {
+        const uint32_t g = g0 + lane_id();
+        const unsigned long long beyond = __ballot(g < groups && !(r0_guess * 1.001 - G.pg()[min(g, groups - 1u)] > 0));
+        if (beyond) { // uniform
+            reach = g0 + (uint32_t)__ffsll((long long)beyond) - 1u;
+            break;
         }
-        __syncthreads();
     }
     // A walk that will end within a few groups goes through them entry by entry, from a copy in LDS: faster than
     // the groups' maps would be to build.
