@@ -52,6 +52,8 @@ typedef struct mako_sampling_params {
 #define MAKO_PATH_GENERAL 5u  /* whole-row sort path */
 #define MAKO_PATH_FORCED 6u   /* not sampled: force_token / close_token took the row */
 #define MAKO_PATH_SORTED 7u   /* top_k == 0: nucleus cut from the sorted list of the weights the row's plan kept */
+#define MAKO_PATH_SUMMED 8u   /* the same on a batch of many such rows: the parts of the list whose order cannot matter to the
+                                 fp32 total and walk were summed, not sorted */
 
 /* out_forced values */
 #define MAKO_FORCED_NONE 0u  /* the row was sampled (or verified) */

@@ -17,7 +17,7 @@ MAKO_OK = 0
 MAKO_ERR_INVALID_ARG = -1
 MAKO_ERR_HIP = -2
 SAMPLER_KERNELS = 4  # MAKO_SAMPLER_KERNELS
-PATH_GREEDY, PATH_FALLBACK, PATH_TOPK, PATH_NUCLEUS, PATH_GENERAL, PATH_FORCED, PATH_SORTED = 1, 2, 3, 4, 5, 6, 7
+PATH_GREEDY, PATH_FALLBACK, PATH_TOPK, PATH_NUCLEUS, PATH_GENERAL, PATH_FORCED, PATH_SORTED, PATH_SUMMED = 1, 2, 3, 4, 5, 6, 7, 8
 FORCED_NONE, FORCED_TOKEN, FORCED_CLOSE = 0, 1, 2
 
 # mako_sampling_params / SamplingParams (src/gen/sampler.hpp:11-20)
@@ -103,6 +103,8 @@ EXPORTS = [
 _libs = {}
 # the library with the kernels' index checks compiled in (mako_amd/build.py, checked=True): tests only
 CHECKED_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmako_sampler_checked.so")
+# the checked library whose plans for large batches leave shares unsorted that they should not (rash=True): tests only
+RASH_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libmako_sampler_rash.so")
 
 
 def load(path=None):

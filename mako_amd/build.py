@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 # the C ABI, and one translation unit per kernel family (a kernel's register allocation then does not depend on
 # which other kernels exist; they also compile side by side)
-SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_alone.hip", "k_sort.hip", "k_tail.hip"]
+SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_alone.hip", "k_sort.hip", "k_sort_unsorted.hip", "k_tail.hip", "k_tail_unsorted.hip"]
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 OUT = os.path.join(HERE, "libmako_sampler.so")
 # the same library with the kernels' index checks compiled in (-DMAKO_CHECKED): for the test that runs the workloads
@@ -39,20 +39,33 @@ RARE_CALLS = ["-DMAKO_RARE_CALL=__attribute__((noinline))", "-DMAKO_REAL_CALLS=1
 SOURCE_FLAGS = {
     # the rare late rows (the whole-row path, second looks at a cut) out of line beside the tails and the top-k rows
     "k_tail.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", *RARE_CALLS],
+    "k_tail_unsorted.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", *RARE_CALLS],
     # the whole-row path and the second look at a cut that is too close to call, out of line beside the top-k rows
     "k_plan_alone.hip": RARE_CALLS,
 }
 
 
-def build(verbose=False, extra=(), jobs=8, checked=False):
+# and the checked library with plans that leave shares unsorted which they should not (-DMAKO_RASH_PLANS, only
+# finish_kernel differs): for the test that expects the oracle's results all the same, through rows given up to the
+# whole-row path
+OUT_RASH = os.path.join(HERE, "libmako_sampler_rash.so")
+
+
+def build(verbose=False, extra=(), jobs=8, checked=False, rash=False):
+    """rash=True needs the checked build's objects (build(checked=True) first)."""
     from concurrent.futures import ThreadPoolExecutor
     os.makedirs(OBJ_DIR, exist_ok=True)
-    if checked:
+    if checked or rash:
         extra = (*extra, "-DMAKO_CHECKED=1")
 
     def compile_one(name):
-        obj = os.path.join(OBJ_DIR, os.path.splitext(name)[0] + ("_checked.o" if checked else ".o"))
-        cmd = ["hipcc", *FLAGS, *SOURCE_FLAGS.get(name, INLINE_ALL), *extra, "-c", os.path.join(CSRC, name), "-o", obj]
+        mine = rash and name == "k_finish.hip"
+        suffix = "_rash.o" if mine else ("_checked.o" if checked or rash else ".o")
+        obj = os.path.join(OBJ_DIR, os.path.splitext(name)[0] + suffix)
+        if rash and not mine:
+            return obj # (the checked build's)
+        cmd = ["hipcc", *FLAGS, *SOURCE_FLAGS.get(name, INLINE_ALL), *extra, *(["-DMAKO_RASH_PLANS=1"] if mine else []), "-c",
+               os.path.join(CSRC, name), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)
@@ -60,7 +73,7 @@ def build(verbose=False, extra=(), jobs=8, checked=False):
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(compile_one, SOURCES))
-    out = OUT_CHECKED if checked else OUT
+    out = OUT_RASH if rash else (OUT_CHECKED if checked else OUT)
     cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
@@ -71,3 +84,4 @@ def build(verbose=False, extra=(), jobs=8, checked=False):
 if __name__ == "__main__":
     build(verbose=True, extra=sys.argv[1:])
     build(verbose=True, extra=sys.argv[1:], checked=True)
+    build(verbose=True, extra=sys.argv[1:], rash=True)

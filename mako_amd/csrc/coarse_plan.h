@@ -2,6 +2,7 @@
 #pragma once
 
 #include "row_records.h"
+#include "unsorted_shares.h"
 
 namespace mako {
 
@@ -26,7 +27,8 @@ struct alignas(16) CoarsePlan {
     uint32_t lbase[kWorkers + 1]; // where its run starts in the workgroup's own ordering of what it keeps
     uint32_t goff[kWorkers];      // entry e of that ordering, if worker w's, goes to goff[w] + e of the row's staging arrays
     uint32_t lim[kWorkers];       // if e < lim[w] (the share's room allows it)
-    uint32_t flag, thr, n0_est, pad;
+    uint32_t flag, thr, n0_est;
+    uint32_t opq_mask; // workers whose shares are left unsorted (opaque_guess())
 };
 
 // What coarse_plan() needs from device memory, asked for before the logits so that the plan can be built while they
@@ -34,9 +36,12 @@ struct alignas(16) CoarsePlan {
 struct PlanLoads {
     SliceStat st; // the record of slice min(lane, slices - 1)
     uint32_t v[kPlanSlices];
+    float u; // the row's uniform draw (for the estimate of where its walk ends)
 };
-__device__ __forceinline__ void issue_plan_loads(const Scratch& sc, uint32_t row, uint32_t slices, PlanLoads& pre)
+template <bool WITH_U>
+__device__ __forceinline__ void issue_plan_loads(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slices, PlanLoads& pre)
 {
+    pre.u = WITH_U ? as_global(d.u)[row] : 0.0f;
     pre.st = load_slice_stat(sc.stats, (size_t)row * kMaxSlices + min((uint32_t)lane_id(), slices - 1u));
     const global_ptr<const uint16_t> lh = as_global(sc.log_hist) + (size_t)row * sc.slices_cap * kLogBins + threadIdx.x;
 #pragma unroll
@@ -51,8 +56,9 @@ __device__ __forceinline__ void issue_plan_loads(const Scratch& sc, uint32_t row
 // under it falls to 1 - top_p of the estimated total, less a few percent.  The list that results is checked by the
 // exact sums later: a plan that keeps too little costs a second look at the row, never a wrong answer.
 // (Every instruction here is latency of the whole pass: a workgroup's sixteen waves share four SIMDs.)
+// opaque_first: the first position of the list from which a share may be left unsorted (kNone: none may).
 __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, uint32_t n_vocab, const mako_sampling_params& P,
-                            float m, const PlanLoads& pre, bool narrow_ok, CoarsePlan& pl, const uint64_t* tab)
+                            float m, const PlanLoads& pre, bool narrow_ok, uint32_t opaque_first, CoarsePlan& pl, const uint64_t* tab)
 {
     const uint32_t tid = threadIdx.x, lane = (uint32_t)lane_id();
     MAKO_STAMP(10);
@@ -191,11 +197,35 @@ __device__ void coarse_plan(const Scratch& sc, uint32_t row, uint32_t slices, ui
             pl.cap[w] = cap;
             pl.stage_off[w] = upto - cap;
         }
+        // which shares are left unsorted (positions from the counts the bins promise, with an eighth to spare: the
+        // tail checks the records' real positions); and a valid mass for every worker
+        const uint32_t expect_w = w < kWorkers ? expect : 0u;
+        const unsigned long long filled = __ballot(expect_w != 0u);
+        const unsigned long long above = w + 1u < (uint32_t)kWave ? filled >> (w + 1u) : 0ull;
+        const uint32_t nx = above ? w + 1u + (uint32_t)__ffsll((long long)above) - 1u : kWorkers; // the next share with entries
+        const double before = w < kWorkers ? pl.mass_above[w] : 0.0, after = nx < kWorkers ? pl.mass_above[nx] : -1.0;
+        if (w > 0u && w < kWorkers && expect_w == 0u)
+            pl.mass_above[w] = after; // (a worker without bins: the mass above the next one that has some, or none)
+        bool unsorted = false;
+        if (opaque_first != kNone) { // (uniform; only batches of many such rows)
+            const uint32_t off_est = __ockl_wfscan_add_u32(expect_w, true) - expect_w;
+            const uint32_t key_hi = w ? (uint32_t)__shfl_up((int)key, 1) : 0x3f800001u; // (just above 1.0)
+            const double r0 = (double)pre.u * ((double)P.top_p * (double)all_m);
+#ifdef MAKO_RASH_PLANS // (a test build: plans that leave unsorted what they should not; the results must not change)
+            const uint32_t rash = 1u << (row & 3u);
+#else
+            constexpr uint32_t rash = 0u;
+#endif
+            unsorted = opaque_guess(flag == 1u && w < kWorkers && nx < kWorkers, expect_w, off_est, opaque_first + opaque_first / 8u,
+                                    before, after, (double)all_m, P.top_p, r0, key_hi, rash);
+        }
+        const uint32_t opq_mask = (uint32_t)__ballot(unsorted);
         if (w == kWorkers - 1u) {
             pl.thr = key;
             pl.n0_est = n0_est;
             pl.mass_all = (double)all_m;
             pl.flag = (sane && upto > sc.vpad) ? 2u : flag;
+            pl.opq_mask = opq_mask;
         }
     }
     lds_barrier();

@@ -23,13 +23,15 @@ hipError_t init_tail_kernels();
 void launch_scan(bool vec, int kh, bool above, dim3 grid, size_t lds, hipStream_t st, const mako_sample_desc& d,
                  const Scratch& sc, uint32_t slice_len, uint32_t cus);
 // finish_kernel<vec, kh> on `wgs` workgroups
-void launch_finish(bool vec, int kh, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc,
+// (unsorted: the instances for batches of many top_k == 0 rows, whose plans leave shares unsorted; the kernels
+// of one batch must agree on it)
+void launch_finish(bool vec, int kh, bool unsorted, uint32_t wgs, hipStream_t st, const mako_sample_desc& d, const Scratch& sc,
                    uint32_t slices); // (host copy, by value)
 void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices); // (host copy, by value)
 // sort_kernel's workgroup i serves entry i of the work list: `grid_rows` * kWorkers workgroups must cover the
 // longest list the batch can produce (kWorkers entries per top_k == 0 row); tail_kernel takes one workgroup per possible wide row.  Workgroups beyond the lists leave at once, but each
 // of them still has to be dispatched.
-void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows); // (host copy)
+void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows, bool unsorted); // (host copy)
 // (tail_kernel: `tail_cap` workgroups for the possible wide rows, then one per row for what is left of every row)
-void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t tail_cap); // (host copy, by value)
+void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t tail_cap, bool unsorted); // (host copy, by value)
 } // namespace mako

@@ -417,6 +417,12 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
         nucleus_rows = std::max(n_nucleus, 1u);
     }
     const bool launch_sort = any_nucleus || any_late;
+    // Batches with many top_k == 0 rows leave the shares of their sorted lists that need no order unsorted
+    // (unsorted_shares.h): there sort_kernel is bound by the number of its workgroups, one per CU at a time, and not, as
+    // on a small batch, by its slowest worker.  More than four rounds of workers; without the caller's copy of the
+    // parameters, from twice as many rows.
+    const bool unsorted = params_host ? (uint64_t)nucleus_rows * mako::kWorkers > 4ull * ctx->cus
+                                      : (uint64_t)d.n_rows * mako::kWorkers > 8ull * ctx->cus;
     // (a launch that fails stops the batch there: the kernels after it would work on what it did not write)
 #define MAKO_LAUNCH(call)                                                                                          \
     do {                                                                                                           \
@@ -434,15 +440,15 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  A batch without such rows
     // (and without rows for the whole-row path) ends with plan_kernel instead.
     if (any_nucleus)
-        MAKO_LAUNCH(mako::launch_finish(vec, kh, finish_wgs, st, d, sc, slices));
+        MAKO_LAUNCH(mako::launch_finish(vec, kh, unsorted, finish_wgs, st, d, sc, slices));
     if (!launch_sort)
         MAKO_LAUNCH(mako::launch_plan_alone(st, d, sc, slices));
     MAKO_MARK(2);
     if (any_nucleus)
-        MAKO_LAUNCH(mako::launch_sort(st, d, sc, slices, nucleus_rows));
+        MAKO_LAUNCH(mako::launch_sort(st, d, sc, slices, nucleus_rows, unsorted));
     MAKO_MARK(3);
     if (launch_sort) // (also finishes every row the kernels before it leave: finish_late_row())
-        MAKO_LAUNCH(mako::launch_tail(st, d, sc, slices, nucleus_rows));
+        MAKO_LAUNCH(mako::launch_tail(st, d, sc, slices, nucleus_rows, unsorted));
     MAKO_MARK(4);
 #undef MAKO_MARK
 #undef MAKO_LAUNCH

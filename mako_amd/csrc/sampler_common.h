@@ -99,7 +99,7 @@ struct BigPlan {
     uint32_t thr;    // bits(q) from which weights are kept
     uint32_t argidx; // first index of the row's maximum, and the maximum (for the whole-row path)
     float m;
-    uint32_t pad;
+    uint32_t opq_mask; // workers whose shares are left unsorted, as one record each (unsorted_shares.h)
     double mass_all; // the plan's estimate of the row's total, in the units of mass[]
     uint32_t key_lo[kWorkers];    // worker w takes bits(q) in [key_lo[w], key_lo[w - 1]) (worker 0: up to 1.0)
     uint32_t stage_off[kWorkers]; // where its share starts in the row's staging arrays (Scratch::key[1], idx[1])

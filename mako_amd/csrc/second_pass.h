@@ -18,10 +18,10 @@ namespace mako {
 // (`slices`: of scan_kernel, whose records give the row maximum)
 // (PLANNING: the workgroup's first piece, with which the plan is built; returns false when the row leaves for the
 // whole-row path and the pass has nothing more to do for it)
-template <bool VEC, int KH, bool PEN, bool PLANNING>
+template <bool VEC, int KH, bool PEN, bool PLANNING, bool UNSORTED = false>
 __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t slice, uint32_t slice_len,
                           const mako_sampling_params& P, uint32_t hl, uint32_t slices, const FinishLds& L, CoarsePlan& pl,
-                          float& m, uint32_t& argidx)
+                          float& m, uint32_t& argidx, uint32_t opaque_first = kNone)
 {
     assume_lds(L);
     FinishShared& sm = *L.sm;
@@ -33,11 +33,11 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
     float wv[16];
     if constexpr (PLANNING) {
         PlanLoads pre;
-        issue_plan_loads(sc, row, slices, pre);
+        issue_plan_loads<UNSORTED>(d, sc, row, slices, pre);
         load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv, [&]() {
             uint32_t n_cands, any_overflow;
             row_summary_of(pre.st, slices, m, argidx, n_cands, any_overflow);
-            coarse_plan(sc, row, slices, d.n_vocab, P, m, pre, !d.draft && !any_overflow && n_cands <= kSortMax, pl, sm.tab);
+            coarse_plan(sc, row, slices, d.n_vocab, P, m, pre, !d.draft && !any_overflow && n_cands <= kSortMax, UNSORTED ? opaque_first : kNone, pl, sm.tab);
         });
     } else {
         load_penalised<VEC, KH>(d, row, lo, hi, slice_len, P, hl, pen, L.cnt, wv);
@@ -59,11 +59,19 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
             plan->m = m;
             plan->mass_all = pl.mass_all;
             plan->flag = flag;
+            const uint32_t unsorted = (UNSORTED && flag == 1) ? pl.opq_mask : 0u;
+            plan->opq_mask = unsorted;
             if (flag == 1 || flag == 3) {
-                const uint32_t work = flag == 1 ? kWorkers : 1u;
-                const uint32_t at = atomicAdd(&sc.work_n[0], work);
-                for (uint32_t w = 0; w < work; ++w)
-                    sc.work_sort[at + w] = (row << 8) | w;
+                // sort_kernel's work: a workgroup per worker that sorts, and up to kCollectors that share the row's
+                // unsorted shares between them (work items kWorkers + c)
+                const uint32_t n_unsorted = (uint32_t)__popc(unsorted), collectors = min(n_unsorted, kCollectors);
+                const uint32_t work = flag == 1 ? kWorkers - n_unsorted + collectors : 1u;
+                uint32_t at = atomicAdd(&sc.work_n[0], work);
+                for (uint32_t c = 0; c < collectors; ++c)
+                    sc.work_sort[at++] = (row << 8) | (kWorkers + c);
+                for (uint32_t w = 0; w < (flag == 1 ? kWorkers : 1u); ++w)
+                    if (!((unsorted >> w) & 1u))
+                        sc.work_sort[at++] = (row << 8) | w;
                 if (flag == 1)
                     sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
             }
@@ -200,16 +208,16 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
     return true;
 }
 
-template <bool VEC, int KH, bool PEN>
+template <bool VEC, int KH, bool PEN, bool UNSORTED>
 __device__ void row_pieces(const mako_sample_desc& d, const Scratch& sc, uint32_t row, uint32_t first, uint32_t stride,
                            uint32_t n_pieces, uint32_t slice_len, const mako_sampling_params& P, uint32_t hl, uint32_t slices,
-                           const FinishLds& L, CoarsePlan& pl)
+                           const FinishLds& L, CoarsePlan& pl, uint32_t opaque_first)
 {
     assume_lds(L);
     // the workgroup's pieces in turn: first, first + stride, ...
     float m = 0.0f;
     uint32_t argidx = 0;
-    if (first >= n_pieces || !one_piece<VEC, KH, PEN, true>(d, sc, row, first, slice_len, P, hl, slices, L, pl, m, argidx))
+    if (first >= n_pieces || !one_piece<VEC, KH, PEN, true, UNSORTED>(d, sc, row, first, slice_len, P, hl, slices, L, pl, m, argidx, opaque_first))
         return;
     for (uint32_t slice = first + stride; slice < n_pieces; slice += stride)
         one_piece<VEC, KH, PEN, false>(d, sc, row, slice, slice_len, P, hl, slices, L, pl, m, argidx);
@@ -219,7 +227,8 @@ __device__ void row_pieces(const mako_sample_desc& d, const Scratch& sc, uint32_
 // serves the i-th share of a row's pieces in row order, SecondPassCut::per_row per top_k == 0 row (find_piece): the busy
 // workgroups are then the first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the
 // mix of rows.
-template <bool VEC, int KH>
+// (UNSORTED: the instance for batches of many such rows, whose plans leave shares unsorted: unsorted_shares.h)
+template <bool VEC, int KH, bool UNSORTED>
 __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
 {
     const Scratch& sc_arg = sc_val; // (by value: the cut is one trip to memory away, not two)
@@ -304,10 +313,13 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     const uint32_t hl = d.hist_tokens ? min(as_global(d.hist_len)[row], (uint32_t)d.hist_stride) : 0u;
     // (a row without history entries takes the penalising variant too when it has penalties: it finds nothing to
     // penalise, and nothing here waits for the length)
+    // (shares may be left unsorted from the first position that the tail neither keeps in LDS nor writes out; never on
+    // verification rows, whose replay reads the list itself)
+    const uint32_t opaque_first = (UNSORTED && !d.draft) ? max(kHeadGroups * kGroup, (d.out_cand_idx && d.out_cand_q) ? d.cand_cap : 0u) : kNone;
     if (d.hist_tokens && !penalties_neutral(P))
-        row_pieces<VEC, KH, true>(d, sc, row, piece, pieces, n_pieces, piece_len, P, hl, slices, L, s_plan);
+        row_pieces<VEC, KH, true, UNSORTED>(d, sc, row, piece, pieces, n_pieces, piece_len, P, hl, slices, L, s_plan, opaque_first);
     else
-        row_pieces<VEC, KH, false>(d, sc, row, piece, pieces, n_pieces, piece_len, P, hl, slices, L, s_plan);
+        row_pieces<VEC, KH, false, UNSORTED>(d, sc, row, piece, pieces, n_pieces, piece_len, P, hl, slices, L, s_plan, opaque_first);
 }
 
 } // namespace mako

@@ -12,7 +12,10 @@ namespace mako {
 // the group records tail_kernel works from; worker 0 of a narrow row finishes the row from the candidate lists.
 // What the row's list looks like as a whole (the workers' counts, the exact total) every worker adds up for itself
 // from what the second pass left; worker 0 stores it for tail_kernel.
-__global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
+// UNSORTED: the instance for batches whose plans leave shares unsorted (unsorted_shares.h; a translation unit of its own,
+// k_sort_unsorted.hip): it knows the rows' collectors and that an unsorted share is one record.
+template <bool UNSORTED>
+__device__ __forceinline__ void sort_body(const mako_sample_desc& d_arg, const Scratch& sc_val, uint32_t slices)
 {
     // (the context's record by value: its first loads, the list's length and this workgroup's entry, go out together
     // and at once; the list has room for every workgroup of the grid)
@@ -46,13 +49,14 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     const uint32_t overflow = rec->overflow;
     const uint32_t thr_bits = rec->thr;
     const double mass_all = rec->mass_all;
+    const uint32_t opq_mask = UNSORTED ? rec->opq_mask : 0u; // workers whose shares stay unsorted (unsorted_shares.h)
     const uint32_t handed = rec->cursor[wl], room = rec->cap[wl];
     const uint32_t stage_l = rec->stage_off[wl], key_lo_l = rec->key_lo[wl];
     const double mass_l = rec->mass[wl];
     fetch_param_words(d_arg, row, arg_words);
     const double ps = sc_arg.part_sum[(size_t)row * kMaxSlices + lane]; // (kMaxSlices = 64 sums per row: one per lane)
     const float u_row = d_arg.u[row]; // (for the estimate of where the row's walk starts)
-    asm volatile("" ::"s"(flag), "s"(overflow), "s"(thr_bits), "v"(handed), "v"(room), "v"(stage_l), "v"(key_lo_l),
+    asm volatile("" ::"s"(flag), "s"(overflow), "s"(thr_bits), "s"(opq_mask), "v"(handed), "v"(room), "v"(stage_l), "v"(key_lo_l),
                  "v"(mass_l), "v"(ps), "v"(arg_words.p));
     if ((flag != 1 && flag != 3) || (flag == 3 && w != 0)) // (never: the list holds exactly the flagged rows' pieces)
         return;
@@ -82,7 +86,9 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     // counts, and from them this worker's place in the sorted list and in the group records
     const uint32_t pieces = uniform_u32(pieces_raw);
     const double total64 = __ockl_wfred_add_f64(lane < pieces ? ps : 0.0);
-    const uint32_t grp_l = (cnt_l + kGroup - 1u) / kGroup;
+    // (a share that is left unsorted is one record, whatever it holds)
+    const bool unsorted_l = UNSORTED && flag == 1 && lane < kWorkers && ((opq_mask >> lane) & 1u) != 0u;
+    const uint32_t grp_l = unsorted_l ? 1u : (cnt_l + kGroup - 1u) / kGroup;
     const uint32_t cnt_upto = __ockl_wfscan_add_u32(cnt_l, true), grp_upto = __ockl_wfscan_add_u32(grp_l, true);
     const uint32_t n0 = (uint32_t)__builtin_amdgcn_readlane((int)cnt_upto, kWave - 1);
     const uint32_t groups = (uint32_t)__builtin_amdgcn_readlane((int)grp_upto, kWave - 1);
@@ -141,6 +147,47 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
     const uint32_t off = (uint32_t)__builtin_amdgcn_readlane((int)(cnt_upto - cnt_l), (int)w);
     const uint32_t gbase = (uint32_t)__builtin_amdgcn_readlane((int)(grp_upto - grp_l), (int)w);
     const size_t t_row = (size_t)row * sc.g_cap;
+    if (UNSORTED && w >= kWorkers) {
+        // One of the row's collectors: every kCollectors-th of the shares that are left unsorted, one after the other.
+        // (The binades of their maps from the plan's estimates in the exact total's units; any guess is safe, the tail
+        // tests what it applies.  A verification row has no such shares.)
+        MAKO_WG_TAG(0xc0000000u);
+        const double r0_raw = (double)u_row * ((double)s_args.P.top_p * total64);
+        const double r0 = r0_raw == r0_raw ? r0_raw : 0.0, scale = mass_all > 0.0 ? total64 / mass_all : 0.0;
+        uint32_t rank = 0;
+        for (uint32_t v = 0; v + 1u < kWorkers; ++v) { // (uniform)
+            if (!((opq_mask >> v) & 1u) || (rank++ % kCollectors) != w - kWorkers)
+                continue;
+            const uint32_t cnt_v = (uint32_t)__builtin_amdgcn_readlane((int)cnt_l, (int)v);
+            const uint32_t stage_v = (uint32_t)__builtin_amdgcn_readlane((int)stage_l, (int)v);
+            const uint32_t off_v = (uint32_t)__builtin_amdgcn_readlane((int)(cnt_upto - cnt_l), (int)v);
+            const size_t t_at = t_row + (uint32_t)__builtin_amdgcn_readlane((int)(grp_upto - grp_l), (int)v);
+            const double before = readlane_f64(mass_l, v) * scale, after_raw = readlane_f64(mass_l, v + 1u) * scale;
+            bool same_tot, same_walk;
+            const OpaqueGuess og = opaque_epochs(before, after_raw > before ? after_raw : before, r0, same_tot, same_walk);
+            if (cnt_v == 0u || cnt_v > kSegCap) {
+                // (nothing came: an empty group; more than a thread's registers hold: a record nothing can apply)
+                if (tid == 0) {
+                    sc.gt.sum[t_at] = cnt_v ? after_raw - before : 0.0;
+                    sc.gt.d0[t_at] = sc.gt.d1[t_at] = sc.gt.cmax[t_at] = cnt_v ? seqfp::kSat : 0u;
+                    sc.gt.start[t_at] = off_v;
+                    sc.gt.pack[t_at] = cnt_v ? kOpaque : 0u;
+                    sc.gt.walk[t_at] = make_uint4(0u, 0u, 0u, 0u);
+                }
+                continue;
+            }
+            StagedKeys keys;
+            {
+                const GlobalKeys gk{key1 + stage_v};
+#pragma unroll
+                for (uint32_t t = 0; t < kSegCap / kThreads; ++t) // (all loads first, from clamped positions)
+                    keys.k[t] = gk[min(t * kThreads + tid, cnt_v - 1u)];
+            }
+            opaque_share(keys, cnt_v, off_v, og.e_tot, og.e_walk, t_at, sc.gt, s_dyn64, sm);
+        }
+        MAKO_STAMP(12);
+        return;
+    }
     if (cnt) {
         MAKO_STAMP(10);
         MAKO_COUNT(31, threadIdx.x == 0 && cnt > kSegCap ? 1 : 0);
@@ -177,6 +224,17 @@ __global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, 
         MAKO_STAMP(12);
     }
 }
+#ifdef MAKO_SORT_UNSORTED
+__global__ __launch_bounds__(kThreads) void sort_kernel_unsorted(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
+{
+    sort_body<true>(d_arg, sc_val, slices);
+}
+#else
+__global__ __launch_bounds__(kThreads) void sort_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
+{
+    sort_body<false>(d_arg, sc_val, slices);
+}
+#endif
 #endif // MAKO_EMIT_SORT_KERNELS
 
 } // namespace mako

@@ -2,6 +2,7 @@
 #pragma once
 
 #include "generic_replay.h"
+#include "unsorted_shares.h"
 
 namespace mako {
 
@@ -341,7 +342,8 @@ __device__ __forceinline__ uint32_t walk_need(float q_first, int eg, uint32_t cm
 // Group maps of groups [g_begin, groups) for epochs guessed from pg: of the running sum (walk == false, into G.d0 /
 // d1 / cmax / pack) or of the walk (into G.w_d0 / w_d1 / w_need / w_pack; r0 - pg[g] is the estimate of r at group
 // g).  The calling wave is number `part` of `parts` that share the work.
-template <typename Keys>
+// (UNSORTED: the list may hold records of unsorted shares, see unsorted_shares.h)
+template <bool UNSORTED = false, typename Keys>
 __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0, const GroupLds G,
                                  uint32_t part = wave_id(), uint32_t parts = kWaves, uint32_t g_begin = 0)
 {
@@ -369,7 +371,12 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
             const int e_end = at_end > 0 ? exponent_of((float)at_end) : 0;
             crossing[u] = uniform_u32((uint32_t)(e_end != eg[u])) != 0 || (!walk && g == 0);
             // (a walk's map that a worker of sort_kernel has left for this very epoch is the map built here: kept)
-            keep[u] = walk && !crossing[u] && eg[u] > 0 && uniform_u32(o_pack[g] >> 16) == (uint32_t)eg[u];
+            // (and so is the record of a share that was left unsorted, whatever it is for: there is nothing to build from)
+            if constexpr (UNSORTED)
+                keep[u] = walk && ((!crossing[u] && eg[u] > 0 && (uniform_u32(o_pack[g] >> 16) & 0xffu) == (uint32_t)eg[u]) ||
+                                   (uniform_u32(o_pack[g]) & kOpaque) != 0u);
+            else
+                keep[u] = walk && !crossing[u] && eg[u] > 0 && uniform_u32(o_pack[g] >> 16) == (uint32_t)eg[u];
             len[u] = uniform_u32(G.pack()[g] & kLenMask);
             load_span(kf, uniform_u32(G.start()[g]), keep[u] ? 0u : len[u], q[u]);
         }
@@ -855,7 +862,9 @@ __device__ MAKO_RARE_CALL double reference_total(Get q_at, uint32_t n, FinishSha
 // `T` (with `t_groups` records at `t_base`) describes a list whose groups were prepared by sort_kernel's workers;
 // without it the list is cut into groups of kGroup here.
 // SHORT_ONLY: the caller's lists never exceed kGroup entries; the code for longer ones is left out.
-template <bool PLANNED = false, bool SHORT_ONLY = false, bool EXACT = false>
+// UNSORTED (with PLANNED): some of the workers' shares may have been left unsorted, as one record each
+// (unsorted_shares.h); a row whose records of that kind cannot all be applied is given up (false).
+template <bool PLANNED = false, bool SHORT_ONLY = false, bool EXACT = false, bool UNSORTED = false>
 __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf_ptr,
                             const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
                             const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, const GroupTable& T = GroupTable{},
@@ -874,6 +883,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     auto idat = [=](uint32_t i) { return jf[i]; };
     const GroupLds G = group_lds(L);
     const bool topp_active = P.top_p < 1.0f;
+    constexpr uint32_t kEpochBits = UNSORTED ? 0xffu : ~0u; // (of a pack's upper half)
     if (d.draft || (!PLANNED && n1 > kGroup * kMaxGroups)) {
         // verification and oversized lists take the generic windowed replay
         uint32_t n = n1;
@@ -1016,8 +1026,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     // group records: fp64 sums (and, from the workers, the maps of the running sum)
     MAKO_STAMP(5);
     const uint32_t groups1 = PLANNED ? t_groups : (n1 + kGroup - 1) / kGroup;
-    if (tid == 0)
+    if (tid == 0) {
         G.misc()[3] = 0;
+        if (UNSORTED) {
+            sm.ticket = 0; // set: a record of an unsorted share where the code below needs the list itself
+            sm.flag = 0;   // set: the list has such records
+        }
+    }
     // The head of the list as floats in LDS (loads set out now, wanted after the cut): where the running sum and
     // the walk change binade every few entries, both go through it entry by entry.
     constexpr uint32_t kHead = kHeadGroups * kGroup;
@@ -1077,13 +1092,20 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             }
             G.start()[tid] = st;
             const uint32_t len = min(pk & kLenMask, min(kGroup, n1 - st));
-            G.pack()[tid] = len | (slot << 9) | (pk & 0x00ff0000u);
+            G.pack()[tid] = len | (slot << 9) | (pk & (0x00ff0000u | (UNSORTED ? kOpaque : 0u)));
             // (the worker's map for the walk, if it was made for the length the group has here: with its exponent;
             // the cut takes the exponent away again from the group it shortens, and the walk builds what is missing)
             G.w_d0()[tid] = r_walk.x;
             G.w_d1()[tid] = r_walk.y;
             G.w_need()[tid] = r_walk.z;
-            G.w_pack()[tid] = (pk & kLenMask) == len ? (len | ((r_walk.w & 0xffu) << 16)) : len;
+            G.w_pack()[tid] = ((pk & kLenMask) == len ? (len | ((r_walk.w & 0xffu) << 16)) : len) | (UNSORTED ? pk & kOpaque : 0u);
+            // (the staged head and the candidates written out are read entry by entry: no unsorted share may lie there,
+            // wherever the plan expected it to lie)
+            if (UNSORTED && (pk & kOpaque)) {
+                sm.flag = 1;
+                if (tid < kHeadGroups || st < kHead || (d.out_cand_idx && d.out_cand_q && st < d.cand_cap))
+                    sm.ticket = 1;
+            }
         }
     } else {
         if (tid < groups1) {
@@ -1107,6 +1129,9 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         }
     }
     __syncthreads();
+    if (UNSORTED && sm.ticket)
+        return false;
+    const uint32_t path_out = (UNSORTED && path == MAKO_PATH_SORTED && sm.flag) ? MAKO_PATH_SUMMED : path;
     {
         const double v = tid < groups1 ? G.pg()[tid + 1] : 0.0;
         double all;
@@ -1147,6 +1172,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         const uint32_t gs = block_min_u32(hitg, sm.bs);
         if (gs == kNone && (need_cut || !exact))
             return false; // (a list that never reaches `want`: a partial one is widened, a whole one decided exactly)
+        if (UNSORTED && gs != kNone && (G.pack()[gs] & kOpaque))
+            return false; // (the cut falls into a share that was left unsorted)
         if (gs != kNone && exact) {
             const uint32_t st = G.start()[gs], len = G.pack()[gs] & kLenMask, keep = G.misc()[0] - st;
             __syncthreads();
@@ -1223,7 +1250,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             o.n_cand = n;
             o.total = total;
             o.q = qat(pos);
-            o.path = path;
+            o.path = path_out;
             o.accepted = 0;
             write_row(d, row, o);
         }
@@ -1278,12 +1305,14 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     }
     // A walk that will end within a few groups goes through them entry by entry, from a copy in LDS: faster than
     // the groups' maps would be to build.
-    const bool head_walk = reach <= kHeadGroups; // uniform
+    bool head_walk = reach <= kHeadGroups; // uniform
     const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
+    if (UNSORTED) // (no unsorted share lies in front of an entry of the staged head: see kOpaque)
+        head_walk = head_walk && head_n <= kHead;
     if (wave_id() != 0 && r0_guess == r0_guess && !head_walk) {
         // (all the other waves: with more than kHeadGroups maps to build they take longer than the chain, even
         // though three of them share its SIMD)
-        build_group_maps(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u);
+        build_group_maps<UNSORTED>(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u);
     }
     if (wave_id() == 0) {
         // 64 groups at a time, one per lane.  A scan composes the lanes' maps; every lane then knows the state after
@@ -1314,7 +1343,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         }
         MAKO_TOC(0, 17);
         MAKO_TIC(1);
-        for (uint32_t base = 0; base < groups; base += kWave) {
+        bool gave_up = false;
+        for (uint32_t base = 0; base < groups && !(UNSORTED && gave_up); base += kWave) {
             const uint32_t gl = min(base + lane_id(), groups - 1u);
             const uint32_t pk_l = G.pack()[gl], st_l = G.start()[gl];
             const uint32_t d0_l = G.d0()[gl], d1_l = G.d1()[gl], cm_l = G.cmax()[gl];
@@ -1322,7 +1352,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             uint32_t done = base == 0 ? first : 0u; // (first <= kWalkSeqGroups)
             while (done < cnt) {
                 const bool live = lane_id() >= done && lane_id() < cnt;
-                const bool same = live && (pk_l >> 16) == (uint32_t)e;
+                const bool same = live && ((pk_l >> 16) & kEpochBits) == (uint32_t)e;
                 Step32 v = lane_id() < done ? identity32() : (same ? Step32{d0_l, d1_l, 0u} : Step32{kSat, kSat, 0u});
                 wave_scan_maps(v.d0, v.d1);
                 const uint32_t after = M + ((M & 1u) ? v.d1 : v.d0); // < 2^29: no wrap
@@ -1335,6 +1365,10 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     const uint32_t st = (uint32_t)__builtin_amdgcn_readlane((int)st_l, f);
                     const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, f);
                     const uint32_t slot = (pk >> 9) & 0x7fu;
+                    if (UNSORTED && (pk & kOpaque)) { // (a share left unsorted whose record does not apply: the row is given up)
+                        gave_up = true;
+                        break;
+                    }
                     if (slot) {
                         const ChainState c = sum_by_quarters(kf, st, pk & kLenMask, G.quarters() + (slot - 1u) * 4u,
                                                              ChainState{M, e, kNone});
@@ -1354,10 +1388,12 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         }
         MAKO_TOC(1, 18);
         if (lane_id() == 0)
-            G.misc()[1] = __float_as_uint(join(M, e));
+            G.misc()[1] = (UNSORTED && gave_up) ? 0xffffffffu : __float_as_uint(join(M, e)); // (a sum of weights is never a NaN)
     }
     __syncthreads();
     MAKO_STAMP(8);
+    if (UNSORTED && G.misc()[1] == 0xffffffffu)
+        return false;
     const float total = __uint_as_float(G.misc()[1]);
     const float span = total - 0.0f;
     const float prod = u_row * span;
@@ -1415,7 +1451,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     G.misc()[3] = 0; // (the quarter records so far are done with: their slots start over)
                 __syncthreads();
                 MAKO_TIC(2);
-                build_group_maps(kf, min(groups, base + (uint32_t)kWave), true, r_here + G.pg()[base], G, wave_id(), kWaves, base);
+                build_group_maps<UNSORTED>(kf, min(groups, base + (uint32_t)kWave), true, r_here + G.pg()[base], G, wave_id(), kWaves, base);
                 __syncthreads();
                 if (wave_id() == 0) {
                     MAKO_TOC(2, 25);
@@ -1431,7 +1467,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 while (done < cnt) {
                     MAKO_COUNT(30, 1);
                     const bool live = lane_id() >= done && lane_id() < cnt;
-                    const bool same = live && (pk_l >> 16) == (uint32_t)e;
+                    const bool same = live && ((pk_l >> 16) & kEpochBits) == (uint32_t)e;
                     Step32 v = lane_id() < done ? identity32() : (same ? Step32{d0_l, d1_l, 0u} : Step32{kSat, kSat, 0u});
                     wave_scan_maps(v.d0, v.d1);
                     const uint32_t dd = (M & 1u) ? v.d1 : v.d0;
@@ -1466,7 +1502,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         if (pk1 & kLenMask)
                             fetch_span_lanes(kf, st1, pk1 & kLenMask, raw);
                         bool by_map = false;
-                        if (g != f && (pk >> 16) == (uint32_t)e) {
+                        if (g != f && ((pk >> 16) & kEpochBits) == (uint32_t)e) {
                             const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d0_l, g);
                             const uint32_t d1 = (uint32_t)__builtin_amdgcn_readlane((int)d1_l, g);
                             const uint32_t need = (uint32_t)__builtin_amdgcn_readlane((int)need_l, g);
@@ -1478,6 +1514,11 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         }
                         if (by_map) {
                             ++passed;
+                        } else if (UNSORTED && (pk & kOpaque)) {
+                            // (a share left unsorted whose record does not apply: the row is given up)
+                            at = kNone;
+                            stopped = true;
+                            break;
                         } else {
                             MAKO_COUNT(22, 1);
                             passed = 0;
@@ -1516,6 +1557,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             G.misc()[2] = at;
         __syncthreads();
         pos = G.misc()[2];
+        if (UNSORTED && pos == kNone)
+            return false;
     }
 
     MAKO_STAMP(9);

@@ -15,8 +15,10 @@ namespace mako {
 // (finish_late_row()) is called out of line: inlined as well, it made this kernel's chains compile to slower code.
 // (With the top-k rows in line the compiler would make a called function of the wide rows' sorted tail instead,
 // which costs them 2 us: that call is forced in line below.)
-__global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices,
-                                                        uint32_t tail_cap)
+// UNSORTED: the instance for batches whose plans may have left shares unsorted (unsorted_shares.h; a translation unit of its
+// own, k_tail_unsorted.hip).
+template <bool UNSORTED>
+__device__ __forceinline__ void tail_body(const mako_sample_desc& d_arg, const Scratch& sc_val, uint32_t slices, uint32_t tail_cap)
 {
     const Scratch& sc_arg = sc_val;
     extern __shared__ __align__(16) unsigned long long s_dyn64[]; // (128-bit LDS operations need the alignment)
@@ -114,8 +116,8 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     // start by storing registers)
     MAKO_CHECK(sc, kCheckTailGroup, plan_n0 <= d.n_vocab && plan_groups <= min(kMaxGroups, sc.g_cap));
     bool done;
-    [[clang::always_inline]] done = sorted_tail<true>(d, row, s_args.P, kf, jf, n0, true, total64, MAKO_PATH_SORTED, L, false, 0.0f,
-                                                      sc.gt, (size_t)row * sc.g_cap, groups);
+    [[clang::always_inline]] done = sorted_tail<true, false, false, UNSORTED>(d, row, s_args.P, kf, jf, n0, true, total64, MAKO_PATH_SORTED,
+                                                                              L, false, 0.0f, sc.gt, (size_t)row * sc.g_cap, groups);
     if (done)
         return;
     // too close to call, or the list ends before the nucleus does: the whole-row path decides
@@ -125,6 +127,17 @@ __global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, 
     __syncthreads();
     general_row<0>(d, sc, row, s_args.P, plan_m, plan_argidx, L);
 }
+#ifdef MAKO_TAIL_UNSORTED
+__global__ __launch_bounds__(kThreads) void tail_kernel_unsorted(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices, uint32_t tail_cap)
+{
+    tail_body<true>(d_arg, sc_val, slices, tail_cap);
+}
+#else
+__global__ __launch_bounds__(kThreads) void tail_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices, uint32_t tail_cap)
+{
+    tail_body<false>(d_arg, sc_val, slices, tail_cap);
+}
+#endif
 #endif // MAKO_EMIT_TAIL_KERNEL
 
 } // namespace mako

@@ -3,7 +3,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 import numpy as np
 
-from mako_amd import api
+from mako_amd import api, workloads
 from oracle import pyoracle
 
 
@@ -61,3 +61,16 @@ def assert_parity(ctx, w, cap=256, rel_tol=1e-5):
             bad.append((r, "prob", float(pg), float(po)))
     assert not bad, "%s: %d rows differ from the oracle: %s" % (w.get("name", "?"), len(bad), bad[:8])
     return g
+
+
+def nucleus_batch(rows, vocab, seed, sigmas, temps, top_ps, us=None, name="unsorted"):
+    """top_k = 0 rows: row r is N(0, sigma^2) logits with sigma, temperature and top_p taken in turn from the lists."""
+    rng = np.random.Generator(np.random.PCG64([seed, 77]))
+    logits = np.empty((rows, vocab), np.float32)
+    p = workloads.make_params(rows, 1.0, 0, 0.9)
+    for r in range(rows):
+        logits[r] = (rng.standard_normal(vocab) * sigmas[r % len(sigmas)]).astype(np.float32)
+        p["temperature"][r] = temps[(r // len(sigmas)) % len(temps)]
+        p["top_p"][r] = top_ps[(r // (len(sigmas) * len(temps))) % len(top_ps)]
+    u = workloads._uniforms(rng, rows) if us is None else np.asarray([us[r % len(us)] for r in range(rows)], np.float32)
+    return dict(name=name, logits=logits, params=p, u=u)

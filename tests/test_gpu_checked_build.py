@@ -50,3 +50,20 @@ def test_no_index_check_fails(gpu_ctx, checked_ctx, name):
     assert np.array_equal(got["tokens"], ref["tokens"])
     assert np.array_equal(got["n_cand"], ref["n_cand"])
     assert gpu_ctx.failed_checks() == 0  # (the shipped library has no checks: always 0)
+
+
+def test_no_index_check_fails_on_a_large_batch(gpu_ctx):
+    """config 4 whole (256 rows: the second pass's looped pieces, sort_kernel's collectors of unsorted shares and the
+    instance of tail_kernel that applies their records only occur on large batches)."""
+    ctx = api.SamplerContext(max_rows=256, max_vocab=151552, max_hist=0, lib_path=api.CHECKED_LIB_PATH)
+    try:
+        w = workloads.config4()
+        ctx.failed_checks()
+        got = gpu_rows(ctx, w, cap=64)
+        bits = ctx.failed_checks()
+        assert bits == 1 << 31, "index checks failed: bit set 0x%x" % bits
+        ref = gpu_rows(gpu_ctx, w, cap=64)
+        assert np.array_equal(got["tokens"], ref["tokens"]) and np.array_equal(got["n_cand"], ref["n_cand"])
+        assert (got["path"] == api.PATH_SUMMED).any()
+    finally:
+        ctx.close()
