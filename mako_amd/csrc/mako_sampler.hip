@@ -392,7 +392,6 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     // The second pass's cut is decided on the device (SecondPassCut): at most one round of workgroups while the rows'
     // pieces fit one, else one workgroup per row or a few; workgroups beyond those with work leave after a look at
     // the cut.
-    const uint32_t finish_wgs = std::max(d.n_rows, ctx->cus);
     // histories of up to 2 (8) entries per thread stay in registers; longer ones take the generic route
     const int kh = !d.hist_tokens ? 2 : (d.hist_stride <= 2 * mako::kThreads ? 2 : (d.hist_stride <= 8 * mako::kThreads ? 8 : 0));
     const bool prof = ctx->profile;
@@ -417,6 +416,8 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
         nucleus_rows = std::max(n_nucleus, 1u);
     }
     const bool launch_sort = any_nucleus || any_late;
+    // (finish_kernel's grid: scan_kernel, which cuts the second pass up, is told of it)
+    const uint32_t finish_wgs = mako::second_pass_grid(d.n_rows, nucleus_rows, ctx->cus);
     // Batches with many top_k == 0 rows leave the shares of their sorted lists that need no order unsorted
     // (unsorted_shares.h): there sort_kernel is bound by the number of its workgroups, one per CU at a time, and not, as
     // on a small batch, by its slowest worker.  More than four rounds of workers; without the caller's copy of the
@@ -434,7 +435,7 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
         }                                                                                                          \
     } while (0)
     MAKO_MARK(0);
-    MAKO_LAUNCH(mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, sc, slice_len, ctx->cus));
+    MAKO_LAUNCH(mako::launch_scan(vec, kh, d.close_token != nullptr, grid, lds, st, d, sc, slice_len, (ctx->cus & 0xffffu) | ((finish_wgs / 8u) << 16)));
     MAKO_MARK(1);
     // top_k == 0 rows: planned and handed out by the second pass, sorted, cut and drawn from; the stages talk through
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  A batch without such rows

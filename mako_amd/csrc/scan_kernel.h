@@ -39,8 +39,9 @@ __device__ __forceinline__ uint32_t wave_kth_largest(uint32_t key, uint32_t j)
 // (amdgpu_waves_per_eu: the vectorised variants are held to the 64 registers that let two workgroups share a CU)
 template <bool VEC, int KH, bool ABOVE = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 8 : 4))) void scan_kernel(mako_sample_desc d, Scratch sc_arg, uint32_t slice_len,
-                                                        uint32_t cus)
+                                                        uint32_t cus_and_grid)
 {
+    // (cus_and_grid: the CUs of the device, and in the upper half an eighth of finish_kernel's grid: second_pass_cut())
     // (scan_kernel takes the context's record by value: its first loads then need no trip to memory for a pointer)
     const Scratch& sc = sc_arg;
     MAKO_ROW(d.hist_tokens ? blockIdx.x : blockIdx.y);
@@ -91,7 +92,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 
         }
     }
     if (row == 0 && slice == 0 && wave_id() == 1) { // how the second pass will be cut up
-        const SecondPassCut cut = second_pass_cut(d, n_slices, slice_len, cus);
+        const SecondPassCut cut = second_pass_cut(d, n_slices, slice_len, cus_and_grid & 0xffffu, (cus_and_grid >> 16) * 8u);
         if (lane_id() == 0)
             *reinterpret_cast<uint4*>(sc.work_n + 4) = make_uint4(cut.per_row, cut.piece_len, cut.busy, cut.pieces);
     }

@@ -62,9 +62,9 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
             const uint32_t unsorted = (UNSORTED && flag == 1) ? pl.opq_mask : 0u;
             plan->opq_mask = unsorted;
             if (flag == 1 || flag == 3) {
-                // sort_kernel's work: a workgroup per worker that sorts, and up to kCollectors that share the row's
-                // unsorted shares between them (work items kWorkers + c)
-                const uint32_t n_unsorted = (uint32_t)__popc(unsorted), collectors = min(n_unsorted, kCollectors);
+                // sort_kernel's work: a workgroup per worker that sorts, and up to kCollectors whose waves take one of the
+                // row's unsorted shares each (work items kWorkers + c)
+                const uint32_t n_unsorted = (uint32_t)__popc(unsorted), collectors = (n_unsorted + (uint32_t)kWaves - 1u) / (uint32_t)kWaves;
                 const uint32_t work = flag == 1 ? kWorkers - n_unsorted + collectors : 1u;
                 uint32_t at = atomicAdd(&sc.work_n[0], work);
                 for (uint32_t c = 0; c < collectors; ++c)
@@ -255,7 +255,16 @@ __global__ __launch_bounds__(kThreads) void finish_kernel(mako_sample_desc d_arg
     // Workgroups go to the eight XCDs in turn.  The shares are dealt so that an XCD's workgroups serve consecutive
     // ones: the workgroups of a row then sit on one XCD (two where a row straddles), whose L2 fetches the row's
     // coarse counts and history once for all of them.  (Only if the grid holds every workgroup the deal names.)
-    {
+    if (cut.x < cut.w) {
+        // More pieces than one round of workgroups, so a row's workgroups go through several pieces each and rows that
+        // need little are done long before rows that need much (a near-flat row takes twice as long as a peaked one).
+        // The rows go round-robin to the XCDs (an XCD's workgroups are dispatched in order onto whichever of its CUs
+        // is free, but which XCD a workgroup goes to is fixed by its number), a row's workgroups to one XCD.
+        const uint32_t rowrank = (wg & 7u) + 8u * ((wg >> 3) / cut.x);
+        wg = rowrank * cut.x + (wg >> 3) % cut.x;
+        if (rowrank * cut.x >= cut.z)
+            return;
+    } else {
         const uint32_t per_xcd = (cut.z + 7u) / 8u;
         if (per_xcd * 8u <= gridDim.x * gridDim.y) {
             if ((wg >> 3) >= per_xcd)

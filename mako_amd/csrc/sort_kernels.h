@@ -148,15 +148,18 @@ __device__ __forceinline__ void sort_body(const mako_sample_desc& d_arg, const S
     const uint32_t gbase = (uint32_t)__builtin_amdgcn_readlane((int)(grp_upto - grp_l), (int)w);
     const size_t t_row = (size_t)row * sc.g_cap;
     if (UNSORTED && w >= kWorkers) {
-        // One of the row's collectors: every kCollectors-th of the shares that are left unsorted, one after the other.
-        // (The binades of their maps from the plan's estimates in the exact total's units; any guess is safe, the tail
-        // tests what it applies.  A verification row has no such shares.)
+        // One of the row's collectors: each of its waves takes one of the shares that are left unsorted (collector c the
+        // shares 16 c .. 16 c + 15 of them) and leaves its record.  (The binades of the maps from the plan's estimates in
+        // the exact total's units; any guess is safe, the tail tests what it applies.  A verification row has no such
+        // shares.)
         MAKO_WG_TAG(0xc0000000u);
         const double r0_raw = (double)u_row * ((double)s_args.P.top_p * total64);
         const double r0 = r0_raw == r0_raw ? r0_raw : 0.0, scale = mass_all > 0.0 ? total64 / mass_all : 0.0;
+        uint32_t* wave_lds = reinterpret_cast<uint32_t*>(s_dyn64) + (uint32_t)wave_id() * (kOpaqueLdsWords + 2u);
+        const uint32_t mine = (w - kWorkers) * (uint32_t)kWaves + (uint32_t)wave_id();
         uint32_t rank = 0;
         for (uint32_t v = 0; v + 1u < kWorkers; ++v) { // (uniform)
-            if (!((opq_mask >> v) & 1u) || (rank++ % kCollectors) != w - kWorkers)
+            if (!((opq_mask >> v) & 1u) || rank++ != mine)
                 continue;
             const uint32_t cnt_v = (uint32_t)__builtin_amdgcn_readlane((int)cnt_l, (int)v);
             const uint32_t stage_v = (uint32_t)__builtin_amdgcn_readlane((int)stage_l, (int)v);
@@ -165,25 +168,17 @@ __device__ __forceinline__ void sort_body(const mako_sample_desc& d_arg, const S
             const double before = readlane_f64(mass_l, v) * scale, after_raw = readlane_f64(mass_l, v + 1u) * scale;
             bool same_tot, same_walk;
             const OpaqueGuess og = opaque_epochs(before, after_raw > before ? after_raw : before, r0, same_tot, same_walk);
-            if (cnt_v == 0u || cnt_v > kSegCap) {
-                // (nothing came: an empty group; more than a thread's registers hold: a record nothing can apply)
-                if (tid == 0) {
-                    sc.gt.sum[t_at] = cnt_v ? after_raw - before : 0.0;
-                    sc.gt.d0[t_at] = sc.gt.d1[t_at] = sc.gt.cmax[t_at] = cnt_v ? seqfp::kSat : 0u;
+            if (cnt_v == 0u) { // (nothing came: an empty group)
+                if (lane == 0u) {
+                    sc.gt.sum[t_at] = 0.0;
+                    sc.gt.d0[t_at] = sc.gt.d1[t_at] = sc.gt.cmax[t_at] = 0u;
                     sc.gt.start[t_at] = off_v;
-                    sc.gt.pack[t_at] = cnt_v ? kOpaque : 0u;
+                    sc.gt.pack[t_at] = 0u;
                     sc.gt.walk[t_at] = make_uint4(0u, 0u, 0u, 0u);
                 }
-                continue;
+            } else {
+                opaque_share(key1 + stage_v, cnt_v, off_v, og.e_tot, og.e_walk, t_at, sc.gt, wave_lds);
             }
-            StagedKeys keys;
-            {
-                const GlobalKeys gk{key1 + stage_v};
-#pragma unroll
-                for (uint32_t t = 0; t < kSegCap / kThreads; ++t) // (all loads first, from clamped positions)
-                    keys.k[t] = gk[min(t * kThreads + tid, cnt_v - 1u)];
-            }
-            opaque_share(keys, cnt_v, off_v, og.e_tot, og.e_walk, t_at, sc.gt, s_dyn64, sm);
         }
         MAKO_STAMP(12);
         return;

@@ -385,8 +385,10 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
             const uint32_t g = g0 + u * parts;
             if (g >= groups) // uniform
                 break;
+            MAKO_COUNT(walk ? 23 : 24, 1);
             if (keep[u]) // uniform
                 continue;
+            MAKO_COUNT(walk ? 27 : 28, 1);
             const Step32 st = span_map(q[u], len[u], eg[u]);
             uint32_t slot = 0;
             if (crossing[u]) {

@@ -28,7 +28,8 @@ namespace mako {
 constexpr uint32_t kOpaque = 1u << 30;
 constexpr int kOpaqueShift = 11;     // the share's largest weight lies at least this many binades below the sum and r
 constexpr uint32_t kOpaqueTies = 16; // exact ties a share may hold (expected: entries * 2^-kOpaqueShift <= 3)
-constexpr uint32_t kCollectors = 4;  // workgroups of sort_kernel that share a row's unsorted shares (work items kWorkers + c)
+constexpr uint32_t kCollectors = 2;  // workgroups of sort_kernel that take a row's unsorted shares, one share per wave (work items kWorkers + c)
+static_assert(kCollectors * (uint32_t)kWaves + 1u >= kWorkers, "a wave for every share but the last, which is never left unsorted");
 constexpr double kOpaqueMu = 0.01;   // what the estimates of the mass above a share are trusted to ...
 constexpr double kOpaqueMuCut = 0.03; // ... and of the mass below it
 
@@ -82,7 +83,7 @@ __device__ __forceinline__ bool opaque_guess(bool allowed, uint32_t cnt, uint32_
     bool same_tot, same_walk;
     const OpaqueGuess g = opaque_epochs(before, after, r0, same_tot, same_walk);
     const int e_q = binade_of((double)__uint_as_float(key_hi - 1u));
-    bool ok = allowed && cnt > 0u && cnt <= kSegCap - kSegCap / 16u && after < mass_all;
+    bool ok = allowed && cnt > 0u && cnt <= 2u * kSegCap && after < mass_all;
     ok = ok && ((rash & 1u) || off >= first_free);
     ok = ok && ((rash & 2u) || (same_tot && g.e_tot >= e_q + kOpaqueShift));
     ok = ok && ((rash & 8u) || (same_walk && (g.e_walk == 0 || g.e_walk >= e_q + kOpaqueShift)));

@@ -18,8 +18,9 @@ struct SecondPassCut {
     uint32_t busy;      // workgroups with work
     uint32_t pieces;    // pieces per row: workgroup g of a row takes the pieces g, g + per_row, ...
 };
+// finish_grid: the workgroups finish_kernel is launched with (second_pass_grid()).
 __device__ __forceinline__ SecondPassCut second_pass_cut(const mako_sample_desc& d, uint32_t slices, uint32_t slice_len,
-                                                         uint32_t cus)
+                                                         uint32_t cus, uint32_t finish_grid)
 {
     uint32_t rows = 0; // top_k == 0 rows of the batch (every lane ends up with the count)
     for (uint32_t base = 0; base < d.n_rows; base += (uint32_t)kWave) {
@@ -38,9 +39,21 @@ __device__ __forceinline__ SecondPassCut second_pass_cut(const mako_sample_desc&
             break;
         }
     }
-    cut.per_row = rows * cut.pieces <= cus ? cut.pieces : min(cut.pieces, max(1u, cus / max(rows, 1u)));
+    // (more pieces than one round of workgroups: as many workgroups per row as the grid allows when the rows are dealt
+    // to the XCDs eight at a time, see finish_kernel)
+    cut.per_row = rows * cut.pieces <= cus ? cut.pieces : min(cut.pieces, max(1u, finish_grid / ((max(rows, 1u) + 7u) & ~7u)));
     cut.busy = rows * cut.per_row;
     return cut;
+}
+
+// Workgroups finish_kernel is launched with (a multiple of eight, at least a workgroup per row): one round's worth, or
+// two where the batch is expected to have more top_k == 0 rows than half a round: the CUs whose rows need little then
+// take on the second halves of those that need much (a near-flat row takes twice as long as a peaked one).  On small
+// batches the workgroups without work, which can only start once a CU is free, would lengthen the kernel instead.
+__host__ __device__ inline uint32_t second_pass_grid(uint32_t n_rows, uint32_t nucleus_rows, uint32_t cus)
+{
+    const uint32_t rows8 = (n_rows + 7u) & ~7u, rounds = 2u * nucleus_rows >= cus ? 2u : 1u;
+    return rows8 > rounds * cus ? rows8 : (rounds * cus + 7u) & ~7u;
 }
 
 // Which piece of work does workgroup `piece` of finish_kernel (per_nucleus = slices, per_other = 1) or of plan_kernel

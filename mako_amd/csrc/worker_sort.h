@@ -271,121 +271,139 @@ __device__ bool lds_sort_staged_runs(const uint32_t* ks, const uint32_t* is, uin
 
 // ---- shares that need no sorting (unsorted_shares.h) ---------------------------------------------------------------
 //
-// The record of an unsorted share.  share.k: the share's cnt <= kSegCap weights as bits(q), any order, asked
-// for by the caller (kSegCap / kThreads per thread, clamped positions: a StagedShare).  All threads call.
-template <typename Share>
-__device__ __forceinline__ void opaque_share(const Share& share, uint32_t cnt, uint32_t off, int e_tot, int e_walk,
-                             size_t t_at, const GroupTable& T, unsigned long long* dyn, FinishShared& sm)
+// The record of an unsorted share, by ONE wave (a collector workgroup's sixteen waves take a share each: no barrier,
+// nothing shared).  ks: the share's cnt weights as bits(q), in device memory, any order.  `lds`: kOpaqueLdsWords words
+// of LDS of the wave's own.  The share is streamed once (sixteen loads per lane in flight): its fp64 sum, its largest
+// weight, the sums of the increments of the weights that are no exact ties, and the ties themselves (kept apart, up
+// to kOpaqueTies of either kind); only a share with ties is streamed again, for the sums between neighbouring ties.
+constexpr uint32_t kOpaqueLdsWords = 4u * kOpaqueTies + 4u * (kOpaqueTies + 1u);
+__device__ void opaque_share(const uint32_t* ks, uint32_t cnt, uint32_t off, int e_tot, int e_walk, size_t t_at,
+                             const GroupTable& T, uint32_t* lds)
 {
     using namespace seqfp;
-    constexpr uint32_t kPer = kSegCap / kThreads, kSegs = kOpaqueTies + 1u;
-    unsigned long long* seg = dyn;                                      // [2][kSegs] sums of increments between ties
-    uint32_t* tie_n = reinterpret_cast<uint32_t*>(seg + 2u * kSegs);    // [2]
-    uint32_t* tie_key = tie_n + 2u;                                     // [2][kOpaqueTies] as found
-    uint32_t* tie_sorted = tie_key + 2u * kOpaqueTies;                  // [2][kOpaqueTies] heaviest first
-    const uint32_t tid = threadIdx.x, lane = (uint32_t)lane_id();
-    if (tid < 2u * kSegs)
-        seg[tid] = 0ull;
-    if (tid < 2u)
-        tie_n[tid] = 0u;
-    lds_barrier();
-    uint32_t k[kPer], dt[kPer], dw[kPer];
+    constexpr uint32_t kTrip = 16, kSegs = kOpaqueTies + 1u;
+    uint32_t* tie_key = lds;                          // [2][kOpaqueTies] as found
+    uint32_t* tie_sorted = lds + 2u * kOpaqueTies;    // [2][kOpaqueTies] heaviest first
+    unsigned long long* seg = reinterpret_cast<unsigned long long*>(lds + 4u * kOpaqueTies); // [2][kSegs]
+    const GlobalKeys gk{ks};
+    const uint32_t lane = (uint32_t)lane_id();
+    const unsigned long long lower = (1ull << lane) - 1ull;
     double sum = 0.0;
-    uint32_t kmax = 0u;
+    uint32_t kmax = 0u, n_t = 0u, n_w = 0u; // (the counts: uniform)
+    uint32_t acc_t = 0u, acc_w = 0u;        // a lane's increments: at most 250 of them, 2^24 at most each
+    const bool sat = cnt > (250u << 6);     // (more than that many per lane: no map)
+    for (uint32_t base = 0; base < cnt; base += kTrip * kWave) {
+        uint32_t k[kTrip];
 #pragma unroll
-    for (uint32_t t = 0; t < kPer; ++t) {
-        const bool valid = t * kThreads + tid < cnt;
-        k[t] = share.k[t];
-        asm volatile("" : "+v"(k[t])); // (used here and not before: the loads are waited for no earlier)
-        k[t] = valid ? k[t] : 0u;
-        const float q = __uint_as_float(k[t]);
-        sum += (double)q;
-        kmax = max(kmax, k[t]);
-        const Step32 st = step32_flat(q, e_tot);
-        dt[t] = valid ? st.d0 : 0u;
-        if (valid && st.d0 != st.d1) {
-            const uint32_t slot = atomicAdd(&tie_n[0], 1u);
-            if (slot < kOpaqueTies)
-                tie_key[slot] = k[t];
-            dt[t] = kNone; // (its step is composed in at its place)
-        }
-        dw[t] = 0u;
-        if (e_walk > 0) { // uniform
-            const Step32 sw = step32_flat(q, e_walk);
-            dw[t] = valid ? sw.d0 : 0u;
-            if (valid && sw.d0 != sw.d1) {
-                const uint32_t slot = atomicAdd(&tie_n[1], 1u);
-                if (slot < kOpaqueTies)
-                    tie_key[kOpaqueTies + slot] = k[t];
-                dw[t] = kNone;
+        for (uint32_t u = 0; u < kTrip; ++u)
+            k[u] = gk[min(base + u * kWave + lane, cnt - 1u)];
+#pragma unroll
+        for (uint32_t u = 0; u < kTrip; ++u) {
+            const bool valid = base + u * kWave + lane < cnt;
+            const uint32_t kv = valid ? k[u] : 0u;
+            const float q = __uint_as_float(kv);
+            sum += (double)q;
+            kmax = max(kmax, kv);
+            const Step32 st = step32_flat(q, e_tot);
+            const bool tie_t = valid && st.d0 != st.d1;
+            acc_t += (valid && !tie_t) ? min(st.d0, 1u << 24) : 0u;
+            const unsigned long long bal_t = __ballot(tie_t);
+            if (bal_t) { // (uniform, rare)
+                const uint32_t slot = n_t + (uint32_t)__popcll(bal_t & lower);
+                if (tie_t && slot < kOpaqueTies)
+                    tie_key[slot] = kv;
+                n_t += (uint32_t)__popcll(bal_t);
+            }
+            if (e_walk > 0) { // uniform
+                const Step32 sw = step32_flat(q, e_walk);
+                const bool tie_w = valid && sw.d0 != sw.d1;
+                acc_w += (valid && !tie_w) ? min(sw.d0, 1u << 24) : 0u;
+                const unsigned long long bal_w = __ballot(tie_w);
+                if (bal_w) {
+                    const uint32_t slot = n_w + (uint32_t)__popcll(bal_w & lower);
+                    if (tie_w && slot < kOpaqueTies)
+                        tie_key[kOpaqueTies + slot] = kv;
+                    n_w += (uint32_t)__popcll(bal_w);
+                }
             }
         }
     }
-    const double sum64 = block_sum_f64(sum, sm.bs); // (its barriers publish the ties)
-    kmax = ~block_min_u32(~kmax, sm.bs);
-    const uint32_t n_t = tie_n[0], n_w = tie_n[1];
-    // the ties of each kind by weight, heaviest first (equal ones in any order: they are the same step)
-    auto order_ties = [&](uint32_t which, uint32_t n_raw) {
-        const uint32_t n = min(n_raw, kOpaqueTies);
-        const uint32_t mine = lane < n ? tie_key[which * kOpaqueTies + lane] : 0u;
-        uint32_t rank = 0;
-        for (uint32_t j = 0; j < n; ++j) {
-            const uint32_t other = (uint32_t)__builtin_amdgcn_readlane((int)mine, (int)j);
-            rank += (other > mine || (other == mine && j < lane)) ? 1u : 0u;
-        }
-        if (lane < n)
-            tie_sorted[which * kOpaqueTies + rank] = mine;
+    const double sum64 = __ockl_wfred_add_f64(sum);
+    kmax = __ockl_wfred_max_u32(kmax);
+    // (a sum of 64 numbers below 2^31: in two halves)
+    auto wave_total = [](uint32_t v) {
+        return ((unsigned long long)__ockl_wfred_add_u32(v >> 16) << 16) + (unsigned long long)__ockl_wfred_add_u32(v & 0xffffu);
     };
-    if (wave_id() == 0) {
-        order_ties(0u, n_t);
-        order_ties(1u, n_w);
-    }
-    lds_barrier();
-    // the increments between neighbouring ties: a weight's segment is the number of ties heavier than it
-    auto segment_sums = [&](uint32_t which, uint32_t n_raw, const uint32_t (&dv)[kPer]) {
-        const uint32_t n = uniform_u32(min(n_raw, kOpaqueTies));
-        uint32_t sg[kPer];
-#pragma unroll
-        for (uint32_t t = 0; t < kPer; ++t)
-            sg[t] = 0u;
-        for (uint32_t i = 0; i < n; ++i) {
-            const uint32_t tk = tie_sorted[which * kOpaqueTies + i];
-#pragma unroll
-            for (uint32_t t = 0; t < kPer; ++t)
-                sg[t] += tk > k[t] ? 1u : 0u;
-        }
-        for (uint32_t s = 0; s <= n; ++s) {
-            uint32_t part = 0u; // (six increments below 2^24 each; clamped so that 64 lanes cannot wrap: a clamped sum
-                                // is 2^24 or more either way, and marked unusable below)
-#pragma unroll
-            for (uint32_t t = 0; t < kPer; ++t)
-                part += (dv[t] != kNone && sg[t] == s) ? min(dv[t], 1u << 24) : 0u;
-            const uint32_t all = __ockl_wfred_add_u32(min(part, 1u << 25));
-            if (lane == 0u && all)
-                atomicAdd(&seg[which * kSegs + s], (unsigned long long)all);
-        }
-    };
-    segment_sums(0u, n_t, dt);
-    if (e_walk > 0) // uniform
-        segment_sums(1u, n_w, dw);
-    lds_barrier();
-    if (tid == 0) {
-        auto share_map = [&](uint32_t which, uint32_t n_raw, int e) {
-            const uint32_t n = min(n_raw, kOpaqueTies);
-            Step32 v = identity32();
-            for (uint32_t s = 0; s <= n; ++s) {
-                const unsigned long long S = seg[which * kSegs + s];
+    // One kind of map: the sums of the increments between neighbouring ties (heaviest first), with each tie's own
+    // two-valued step composed in at its place.
+    auto share_map = [&](uint32_t which, uint32_t n_raw, int e, uint32_t acc) {
+        Step32 v = Step32{kSat, kSat, 0u};
+        if (e > 0 && n_raw <= kOpaqueTies && !sat) { // uniform
+            const uint32_t n = n_raw;
+            if (n == 0u) {
+                const unsigned long long S = wave_total(acc);
                 const uint32_t add = S < (1ull << 24) ? (uint32_t)S : kSat;
-                v = compose32(v, Step32{add, add, 0u});
-                if (s < n)
-                    v = compose32(v, step32_flat(__uint_as_float(tie_sorted[which * kOpaqueTies + s]), e));
+                v = Step32{add, add, 0u};
+            } else {
+                // the ties by weight, heaviest first (equal ones in any order: they are the same step)
+                __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): the wave's own writes of the ties
+                const uint32_t mine = lane < n ? tie_key[which * kOpaqueTies + lane] : 0u;
+                uint32_t rank = 0;
+                for (uint32_t j = 0; j < n; ++j) {
+                    const uint32_t other = (uint32_t)__builtin_amdgcn_readlane((int)mine, (int)j);
+                    rank += (other > mine || (other == mine && j < lane)) ? 1u : 0u;
+                }
+                if (lane < n)
+                    tie_sorted[which * kOpaqueTies + rank] = mine;
+                if (lane <= n)
+                    seg[which * kSegs + lane] = 0ull;
+                __builtin_amdgcn_s_waitcnt(0xc07f);
+                // the share again: a weight's segment is the number of ties heavier than it
+                for (uint32_t base = 0; base < cnt; base += kTrip * kWave) {
+                    uint32_t k[kTrip], sg[kTrip], dv[kTrip];
+#pragma unroll
+                    for (uint32_t u = 0; u < kTrip; ++u)
+                        k[u] = gk[min(base + u * kWave + lane, cnt - 1u)];
+#pragma unroll
+                    for (uint32_t u = 0; u < kTrip; ++u) {
+                        const bool valid = base + u * kWave + lane < cnt;
+                        const Step32 st = step32_flat(__uint_as_float(k[u]), e);
+                        dv[u] = (valid && st.d0 == st.d1) ? min(st.d0, 1u << 24) : 0u;
+                        sg[u] = 0u;
+                    }
+                    for (uint32_t i = 0; i < n; ++i) {
+                        const uint32_t tk = uniform_u32(tie_sorted[which * kOpaqueTies + i]);
+#pragma unroll
+                        for (uint32_t u = 0; u < kTrip; ++u)
+                            sg[u] += tk > k[u] ? 1u : 0u;
+                    }
+                    for (uint32_t s = 0; s <= n; ++s) {
+                        uint32_t part = 0u; // (sixteen increments below 2^24 + 1 each: below 2^29)
+#pragma unroll
+                        for (uint32_t u = 0; u < kTrip; ++u)
+                            part += sg[u] == s ? dv[u] : 0u;
+                        const unsigned long long all = wave_total(part);
+                        if (lane == 0u && all)
+                            seg[which * kSegs + s] += all;
+                    }
+                }
+                __builtin_amdgcn_s_waitcnt(0xc07f);
+                v = identity32();
+                for (uint32_t s = 0; s <= n; ++s) {
+                    const unsigned long long S = seg[which * kSegs + s];
+                    const uint32_t add = S < (1ull << 24) ? (uint32_t)S : kSat;
+                    v = compose32(v, Step32{add, add, 0u});
+                    if (s < n)
+                        v = compose32(v, step32_flat(__uint_as_float(tie_sorted[which * kOpaqueTies + s]), e));
+                }
             }
-            if (n_raw > kOpaqueTies || e <= 0)
-                v = Step32{kSat, kSat, 0u};
-            v.cmax = e > 0 ? step32_flat(__uint_as_float(kmax), e).cmax : kSat; // (a weight's step never grows as the weight falls)
-            return v;
-        };
-        const Step32 m0 = share_map(0u, n_t, e_tot), m1 = share_map(1u, n_w, e_walk);
+        }
+        v.cmax = e > 0 ? step32_flat(__uint_as_float(kmax), e).cmax : kSat; // (a weight's step never grows as the weight falls)
+        return v;
+    };
+    const Step32 m0 = share_map(0u, n_t, e_tot, acc_t);
+    const Step32 m1 = e_walk > 0 ? share_map(1u, n_w, e_walk, acc_w) : Step32{kSat, kSat, kSat};
+    if (lane == 0u) {
         T.sum[t_at] = sum64;
         T.d0[t_at] = m0.d0;
         T.d1[t_at] = m0.d1;
@@ -395,12 +413,7 @@ __device__ __forceinline__ void opaque_share(const Share& share, uint32_t cnt, u
         T.walk[t_at] = e_walk > 0 ? make_uint4(m1.d0, m1.d1, walk_need(__uint_as_float(kmax), e_walk, m1.cmax), (uint32_t)e_walk)
                                   : make_uint4(0u, 0u, 0u, 0u);
     }
-    lds_barrier(); // (the caller may come back with the next share)
 }
-
-struct StagedKeys { // (a share's weights alone, as fetch_staged_share() would leave them in a StagedShare)
-    uint32_t k[kSegCap / kThreads];
-};
 
 // Group records of a worker's sorted range (cnt entries from position off of the list kf): fp64 sums, and the
 // maps of the running fp32 sum for the epoch guessed from the mass above the range plus the sums before the group.
