@@ -224,6 +224,18 @@ def test_seqfp_host():
     assert " 0 failures" in out, out
 
 
+def test_unsorted_share_host():
+    """The record that stands for an unsorted share of a sorted list (opaque_share, mako_amd/csrc/worker_sort.h)
+    restated on the host: sums of the increments between neighbouring exact ties, the ties' own steps composed in
+    between.  Wherever it passes the tests under which tail_kernel applies it, it gives the state that adding
+    (subtracting) the sorted weights one by one with real fp32 operations gives: 60000 shares."""
+    exe = os.path.join(HERE, "cpu", "unsorted_share_test")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-I", os.path.join(HERE, "..", "mako_amd", "csrc"),
+                    os.path.join(HERE, "cpu", "unsorted_share_test.cpp"), "-o", exe], check=True)
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and ": 0 failures" in out.stdout, out.stdout
+
+
 def test_log_bins_host():
     """The coarse-bin arithmetic scan_kernel and the second pass share (mako_amd/csrc/log_bins.h): a frame's bins tile
     the units below its maximum, and a slice's counts move into the frame of the row's maximum exactly."""
@@ -345,12 +357,12 @@ def test_oracle_under_sanitizers():
     assert out.returncode == 0 and out.stdout.strip().endswith(" 0 failures"), out.stdout + out.stderr
 
 
-@pytest.mark.parametrize("name", ["seqfp_test", "gen_helpers_test", "log_bins_test"])
+@pytest.mark.parametrize("name", ["seqfp_test", "gen_helpers_test", "log_bins_test", "unsorted_share_test"])
 def test_host_code_under_sanitizers(name):
     """The host-side C++ the library shares with its kernels (seqfp.h) and ships (include/gen/), likewise."""
     exe = os.path.join(HERE, "cpu", name + "_san")
-    subprocess.run(["g++", "-std=c++17", *SANITIZE, "-I", os.path.join(HERE, "..", "include"),
-                    os.path.join(HERE, "cpu", name + ".cpp"), "-o", exe], check=True)
+    subprocess.run(["g++", "-std=c++17", *SANITIZE, "-I", os.path.join(HERE, "..", "include"), "-I",
+                    os.path.join(HERE, "..", "mako_amd", "csrc"), os.path.join(HERE, "cpu", name + ".cpp"), "-o", exe], check=True)
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0 and "0 failures" in out.stdout, out.stdout + out.stderr
 
