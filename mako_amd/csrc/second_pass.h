@@ -31,6 +31,7 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
     const uint32_t lo = slice * slice_len;
     const uint32_t hi = min(d.n_vocab, lo + slice_len);
     float wv[16];
+    MAKO_STAMP(28);
     if constexpr (PLANNING) {
         PlanLoads pre;
         issue_plan_loads<UNSORTED>(d, sc, row, slices, pre);
@@ -93,7 +94,11 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
         qb[j] = 0u;
         slot[j] = kNone;
         if (lo + (VEC ? (j / 4u) * 4096u : j * (uint32_t)kThreads) < hi) {
-            const float q = weight_of(wv[j], m, inv_t, sm.tab);
+            // (the large batches' instance: a wave whose weights all underflow to zero, as those of a peaked row far
+            // below its maximum do, skips the arithmetic that would tell it so; expf_glibc() returns 0 below that bound)
+            float q = 0.0f;
+            if (!UNSORTED || __ballot(!((wv[j] - m) * inv_t < -0x1.9fe368p6f)) != 0ull)
+                q = weight_of(wv[j], m, inv_t, sm.tab);
             qb[j] = (q >= floor_q && q > 0.0f) ? __float_as_uint(q) : 0u;
             if (qb[j])
                 sum += (double)q;
@@ -196,6 +201,7 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
         }
         lds_barrier();
     }
+    MAKO_STAMP(29);
     if (dropped) // (more weights in a range than the counts promised: the row takes the whole-row path)
         plan->overflow = 1;
     if (tid == 0) {
@@ -205,6 +211,7 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
         as_global(sc.part_sum)[(size_t)row * kMaxSlices + slice] = total;
     }
     lds_barrier(); // (the waves' sums have been read before the next piece's replace them)
+    MAKO_STAMP(30);
     return true;
 }
 
