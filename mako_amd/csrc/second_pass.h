@@ -169,6 +169,7 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
                 slot[j] = (slot[j] & 0xffff0000u) | (start[j] + (slot[j] & 0xffffu));
     }
     bool dropped = false;
+    const uint32_t unsorted_mask = UNSORTED ? uniform_u32(pl.opq_mask) : 0u;
     for (uint32_t from = 0; from < kept; from += kHalf) { // (what fits the buffer at a time: usually everything)
 #pragma unroll
         for (uint32_t j = 0; j < 16; ++j)
@@ -193,7 +194,8 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
                     MAKO_CHECK(sc, kCheckStage, (uint64_t)(pl.goff[w] + e) < sc.vpad && pl.goff[w] + e >= pl.stage_off[w] &&
                                                     pl.goff[w] + e < pl.stage_off[w] + pl.cap[w]);
                     kstage[pl.goff[w] + e] = x.x;
-                    istage[pl.goff[w] + e] = x.y;
+                    if (!UNSORTED || !((unsorted_mask >> w) & 1u)) // (a share that is only summed has no use for the token ids)
+                        istage[pl.goff[w] + e] = x.y;
                 } else {
                     dropped = true;
                 }
