@@ -74,3 +74,45 @@ def nucleus_batch(rows, vocab, seed, sigmas, temps, top_ps, us=None, name="unsor
         p["top_p"][r] = top_ps[(r // (len(sigmas) * len(temps))) % len(top_ps)]
     u = workloads._uniforms(rng, rows) if us is None else np.asarray([us[r % len(us)] for r in range(rows)], np.float32)
     return dict(name=name, logits=logits, params=p, u=u)
+
+
+def random_large_batch(seed):
+    """A batch of 65-256 rows of every kind a top_k = 0 row comes in (wide and narrow, on grids of few distinct values,
+    offset by hundreds, spiked, partly at -inf), a few top-k rows among them, with or without penalties, histories and
+    masks; the number of candidates the caller wants written out varies too.  Returns (workload, cand_cap)."""
+    rng = np.random.default_rng(seed)
+    v = int(rng.choice([4099, 20000, 40000, 65537, 129280, 151552]))
+    b = int(rng.choice([65, 100, 130, 200, 256])) if v < 100000 else int(rng.choice([65, 72, 96]))
+    logits = np.empty((b, v), np.float32)
+    kinds = rng.integers(0, 7, b)
+    for r in range(b):
+        kind = kinds[r]
+        row = (rng.standard_normal(v) * [3.0, 3.0, 0.1, 0.02, 1.0, 6.0, 0.3][kind]).astype(np.float32)
+        if kind == 1:
+            row = (np.round(row * 4) / 4).astype(np.float32)
+        if kind == 4:
+            row += np.float32(rng.choice([0.0, 50.0, -50.0, 1000.0]))
+        if kind == 5:
+            row[rng.integers(0, v, rng.integers(1, 40))] += np.float32(rng.uniform(3, 15))
+        logits[r] = row
+    if rng.integers(0, 4) == 0:
+        logits[:, rng.integers(0, v, max(1, v // 50))] = -np.inf
+    p = workloads.make_params(b)
+    p["temperature"] = rng.choice(np.array([0.3, 0.5, 0.8, 1.0, 1.3, 2.0, 5.0], np.float32), b)
+    p["top_k"] = rng.choice(np.array([0, 0, 0, 0, 0, 0, 40], np.uint32), b)
+    p["top_p"] = rng.choice(np.array([0.5, 0.8, 0.9, 0.95, 0.99, 0.999, 0.99999, 0.3], np.float32), b)
+    p["min_p"] = rng.choice(np.array([0.0, 0.0, 0.0, 0.0, 1e-4, 0.02], np.float32), b)
+    if rng.integers(0, 2):
+        p["repetition_penalty"] = np.float32(1.1)
+        p["frequency_penalty"] = np.float32(0.2)
+        p["presence_penalty"] = np.float32(0.3)
+    u = rng.random(b).astype(np.float32)
+    u[rng.integers(0, b, 4)] = np.array([0.0, 1.0 - 2.0**-24, 0.5, 0.999999], np.float32)
+    w = dict(name="random large batch %d" % seed, logits=logits, params=p, u=u)
+    if rng.integers(0, 2):
+        hl = int(rng.choice([5, 300, 2048]))
+        w["hist"] = rng.integers(0, v, (b, hl)).astype(np.int32)
+        w["hist_len"] = rng.integers(0, hl + 1, b).astype(np.uint32)
+    if rng.integers(0, 4) == 0:
+        w["mask"] = rng.integers(0, 2**32, (b, (v + 31) // 32), dtype=np.uint64).astype(np.uint32)
+    return w, int(rng.choice([1, 64, 128, 3000, 12000]))

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from mako_amd import api, hip, workloads
-from parity import assert_parity, nucleus_batch
+from parity import assert_parity, nucleus_batch, random_large_batch
 
 pytestmark = pytest.mark.gpu
 
@@ -50,3 +50,17 @@ def test_rash_plans_walk_depths(rash_ctx):
     us = [0.0, 1e-4, 0.01, 0.1, 0.25, 0.5, 0.6, 0.7, 0.8, 0.9, 0.95, 0.99, 0.999, 0.9999, 1.0 - 2.0**-24, 0.3333333, 0.6666667]
     w = nucleus_batch(136, 129280, 12, sigmas=[0.1, 1.0], temps=[1.0], top_ps=[0.9, 0.97], us=us, name="rash, walk depths")
     _run(rash_ctx, w, 64)
+
+
+def test_rash_plans_random_large_batches():
+    total = np.zeros(9, np.int64)
+    for seed in range(9100, 9110):
+        w, cap = random_large_batch(seed)
+        b, v = w["logits"].shape
+        ctx = api.SamplerContext(max_rows=b, max_vocab=v, max_hist=2048, lib_path=api.RASH_LIB_PATH)
+        try:
+            g = _run(ctx, w, cap)
+        finally:
+            ctx.close()
+        total += np.bincount(g["path"], minlength=9)[:9]
+    assert total[api.PATH_GENERAL] > 50

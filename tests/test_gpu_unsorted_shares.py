@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from mako_amd import api, workloads
-from parity import assert_parity, gpu_rows, nucleus_batch as _batch, oracle_rows
+from parity import assert_parity, gpu_rows, nucleus_batch as _batch, oracle_rows, random_large_batch
 
 pytestmark = pytest.mark.gpu
 
@@ -115,3 +115,19 @@ def test_hinted_and_unhinted_calls_agree(gpu_ctx):
     assert np.array_equal(h["tokens"], g["tokens"]) and np.array_equal(h["n_cand"], g["n_cand"])
     assert np.array_equal(h["total"].view(np.uint32), g["total"].view(np.uint32))
     assert (h["path"] == PATH_SUMMED).any()
+
+
+def test_random_large_batches():
+    """Sixteen batches of random shape and content (random_large_batch), each with a context of its own size."""
+    total = np.zeros(9, np.int64)
+    for seed in range(9000, 9016):
+        w, cap = random_large_batch(seed)
+        b, v = w["logits"].shape
+        ctx = api.SamplerContext(max_rows=b, max_vocab=v, max_hist=2048)
+        try:
+            g = assert_parity(ctx, w, cap=cap)
+        finally:
+            ctx.close()
+        total += np.bincount(g["path"], minlength=9)[:9]
+    _say("random large batches, rows by path: %s" % total.tolist())
+    assert total[PATH_SUMMED] > 200
