@@ -1215,11 +1215,22 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     keep = (uint32_t)__builtin_amdgcn_readlane((int)hit, src) + 1u;
                     ok = __builtin_amdgcn_readlane((int)clear, src) != 0;
                 }
+                // (the shortened group's map for the running sum is made again from the entries at hand, for the binade
+                // its old map was for: the chain then need not add its entries one by one; the walk's is not, exponent 0)
+                const uint32_t eg_cut = PLANNED ? (uniform_u32(G.pack()[gs]) >> 16) & 0xffu : 0u;
+                Step32 cut_map = Step32{kSat, kSat, kSat};
+                if (ok && keep != len && eg_cut) // uniform
+                    cut_map = span_map(q, keep, (int)eg_cut);
                 if (lane_id() == 0) {
                     G.misc()[0] = ok ? st + keep : kNone;
                     if (ok && keep != len) {
-                        G.pack()[gs] = keep; // shortened: the prepared maps no longer apply (exponent 0)
+                        G.pack()[gs] = keep | (eg_cut << 16);
                         G.w_pack()[gs] = keep;
+                        if (eg_cut) {
+                            G.d0()[gs] = cut_map.d0;
+                            G.d1()[gs] = cut_map.d1;
+                            G.cmax()[gs] = cut_map.cmax;
+                        }
                     }
                 }
             }
