@@ -8,7 +8,9 @@
 namespace mako {
 void launch_sort_unsorted(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows)
 {
-    hipLaunchKernelGGL(sort_kernel_unsorted, dim3(kWorkers, grid_rows), dim3(kThreads), kSortLds, st, d, sc, slices);
+    // (the three regions of large_batch_lists() are sized by the batch's rows)
+    (void)grid_rows;
+    hipLaunchKernelGGL(sort_kernel_unsorted, dim3(kSortItemsPerRow, d.n_rows), dim3(kThreads), kSortLds, st, d, sc, slices);
 }
 
 hipError_t init_sort_unsorted()

@@ -121,6 +121,20 @@ struct GroupTable {
                      // for r at the group; exponent 0: none
 };
 
+// The large batches' work lists of sort_kernel.  Workgroups are dispatched in the order of their numbers, to the XCDs
+// in turn, and the next one waits for a CU of ITS XCD: with entries of unequal cost in row order the XCDs fall out of
+// step and CUs idle (a quarter of the time on config 4).  So the entries are kept by kind, the costliest first, each
+// kind in a region of workgroup numbers of its own: the collectors of unsorted shares (up to two per row, ~19 us),
+// the workers that sort (up to kWorkers per row, ~13 us), the narrow rows (one per row, ~10 us).
+constexpr uint32_t kSortItemsPerRow = kWorkers + 3u;
+struct SortLists {
+    uint32_t collectors_at, sorted_at, narrow_at; // first workgroup number (= first entry of work_sort) of each region
+};
+__host__ __device__ inline SortLists large_batch_lists(uint32_t n_rows)
+{
+    return SortLists{0u, 2u * n_rows, (kWorkers + 2u) * n_rows};
+}
+
 struct Scratch {
     SliceStat* stats;  // [max_rows][kMaxSlices]
     float* cand_w;     // [max_rows][slices_cap][kCap] penalised logits of the slice's candidates
@@ -142,10 +156,11 @@ struct Scratch {
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
     // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
     // (finish_kernel and plan_kernel get the same effect from find_piece().)
-    uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); [2]: failed checks of a checked
+    uint32_t* work_n;      // [16] entries in work_sort, work_tail (zeroed by scan_kernel); [3], [8]: large batches' lists (below); [2]: failed checks of a checked
                            // build (MAKO_CHECK); then, 16-byte aligned at [4], how the second pass is cut up
                            // (SecondPassCut; scan_kernel's first workgroup decides)
-    uint32_t* work_sort;   // [max_rows * kWorkers] row << 8 | worker; appended by finish_kernel
+    uint32_t* work_sort;   // [max_rows * kSortItemsPerRow] row << 8 | worker; appended by finish_kernel.  The large batches'
+                           // instances keep three lists in it, by what an entry costs (large_batch_lists())
     uint32_t* work_tail;   // [max_rows] row; appended by finish_kernel
     uint64_t vpad;
     uint32_t slices_cap;

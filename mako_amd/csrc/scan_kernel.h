@@ -78,6 +78,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 
         if (row == 0 && slice == 0) { // the lists finish_kernel and plan_kernel append to start empty
             sc.work_n[0] = 0;
             sc.work_n[1] = 0;
+            sc.work_n[3] = 0;
+            sc.work_n[8] = 0;
             MAKO_CHECK(sc, kCheckAlive, false);
         }
     }

@@ -66,13 +66,26 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
                 // sort_kernel's work: a workgroup per worker that sorts, and up to kCollectors whose waves take one of the
                 // row's unsorted shares each (work items kWorkers + c)
                 const uint32_t n_unsorted = (uint32_t)__popc(unsorted), collectors = (n_unsorted + (uint32_t)kWaves - 1u) / (uint32_t)kWaves;
-                const uint32_t work = flag == 1 ? kWorkers - n_unsorted + collectors : 1u;
-                uint32_t at = atomicAdd(&sc.work_n[0], work);
-                for (uint32_t c = 0; c < collectors; ++c)
-                    sc.work_sort[at++] = (row << 8) | (kWorkers + c);
-                for (uint32_t w = 0; w < (flag == 1 ? kWorkers : 1u); ++w)
-                    if (!((unsorted >> w) & 1u))
+                if constexpr (UNSORTED) {
+                    // (three lists, by what an entry costs: large_batch_lists())
+                    const SortLists lists = large_batch_lists(d.n_rows);
+                    if (flag == 3) {
+                        sc.work_sort[lists.narrow_at + atomicAdd(&sc.work_n[8], 1u)] = row << 8;
+                    } else {
+                        uint32_t at = lists.collectors_at + atomicAdd(&sc.work_n[3], collectors);
+                        for (uint32_t c = 0; c < collectors; ++c)
+                            sc.work_sort[at++] = (row << 8) | (kWorkers + c);
+                        at = lists.sorted_at + atomicAdd(&sc.work_n[0], kWorkers - n_unsorted);
+                        for (uint32_t w = 0; w < kWorkers; ++w)
+                            if (!((unsorted >> w) & 1u))
+                                sc.work_sort[at++] = (row << 8) | w;
+                    }
+                } else {
+                    const uint32_t work = flag == 1 ? kWorkers : 1u;
+                    uint32_t at = atomicAdd(&sc.work_n[0], work);
+                    for (uint32_t w = 0; w < work; ++w)
                         sc.work_sort[at++] = (row << 8) | w;
+                }
                 if (flag == 1)
                     sc.work_tail[atomicAdd(&sc.work_n[1], 1u)] = row;
             }
