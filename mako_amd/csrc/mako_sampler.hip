@@ -129,7 +129,7 @@ hipError_t layout_scratch(mako::Scratch& sc, uint32_t max_rows, uint32_t max_voc
     MAKO_TAKE(sc.gt.quarters, rg * 4);
     MAKO_TAKE(sc.gt.walk, rg);
     MAKO_TAKE(sc.log_hist, (size_t)max_rows * sc.slices_cap * mako::kLogBins);
-    MAKO_TAKE(sc.work_n, 16);
+    MAKO_TAKE(sc.work_n, 8);
     MAKO_TAKE(sc.work_sort, (size_t)max_rows * mako::kSortItemsPerRow);
     MAKO_TAKE(sc.work_tail, (size_t)max_rows);
 #undef MAKO_TAKE
@@ -143,7 +143,7 @@ hipError_t zero_scratch(const mako::Scratch& sc, uint32_t max_rows)
     if (e == hipSuccess)
         e = hipMemset(sc.cnt, 0, (size_t)max_rows * sc.vpad * sizeof(uint32_t));
     if (e == hipSuccess)
-        e = hipMemset(sc.work_n, 0, 16 * sizeof(uint32_t));
+        e = hipMemset(sc.work_n, 0, 8 * sizeof(uint32_t));
     return e;
 }
 

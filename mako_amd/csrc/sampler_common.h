@@ -123,16 +123,18 @@ struct GroupTable {
 
 // The large batches' work lists of sort_kernel.  Workgroups are dispatched in the order of their numbers, to the XCDs
 // in turn, and the next one waits for a CU of ITS XCD: with entries of unequal cost in row order the XCDs fall out of
-// step and CUs idle (a quarter of the time on config 4).  So the entries are kept by kind, the costliest first, each
-// kind in a region of workgroup numbers of its own: the collectors of unsorted shares (up to two per row, ~19 us),
-// the workers that sort (up to kWorkers per row, ~13 us), the narrow rows (one per row, ~10 us).
-constexpr uint32_t kSortItemsPerRow = kWorkers + 3u;
+// step and CUs idle (a quarter of the time on config 4).  So the costliest entries, the collectors of unsorted shares
+// (up to two per row, ~19 us), come first and together, then the workers that sort (~13 us) and the narrow rows
+// (~10 us).  A workgroup without an entry costs nothing behind the last one with work, but between two of them it
+// waits for a CU like any other: the collectors' list is filled from its end backwards (work_n[3] of them, the last at
+// workgroup number sorted_at - 1), the others' forwards from sorted_at (work_n[0]), so that no gap lies between.
+constexpr uint32_t kSortItemsPerRow = kWorkers + 2u;
 struct SortLists {
-    uint32_t collectors_at, sorted_at, narrow_at; // first workgroup number (= first entry of work_sort) of each region
+    uint32_t sorted_at; // first workgroup number (= entry of work_sort) of the workers that sort and the narrow rows
 };
 __host__ __device__ inline SortLists large_batch_lists(uint32_t n_rows)
 {
-    return SortLists{0u, 2u * n_rows, (kWorkers + 2u) * n_rows};
+    return SortLists{2u * n_rows};
 }
 
 struct Scratch {
@@ -156,7 +158,7 @@ struct Scratch {
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
     // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
     // (finish_kernel and plan_kernel get the same effect from find_piece().)
-    uint32_t* work_n;      // [16] entries in work_sort, work_tail (zeroed by scan_kernel); [3], [8]: large batches' lists (below); [2]: failed checks of a checked
+    uint32_t* work_n;      // [16] entries in work_sort, work_tail (zeroed by scan_kernel); [3]: large batches' lists (below); [2]: failed checks of a checked
                            // build (MAKO_CHECK); then, 16-byte aligned at [4], how the second pass is cut up
                            // (SecondPassCut; scan_kernel's first workgroup decides)
     uint32_t* work_sort;   // [max_rows * kSortItemsPerRow] row << 8 | worker; appended by finish_kernel.  The large batches'

@@ -79,7 +79,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(VEC ? 
             sc.work_n[0] = 0;
             sc.work_n[1] = 0;
             sc.work_n[3] = 0;
-            sc.work_n[8] = 0;
             MAKO_CHECK(sc, kCheckAlive, false);
         }
     }

@@ -67,12 +67,12 @@ __device__ bool one_piece(const mako_sample_desc& d, const Scratch& sc, uint32_t
                 // row's unsorted shares each (work items kWorkers + c)
                 const uint32_t n_unsorted = (uint32_t)__popc(unsorted), collectors = (n_unsorted + (uint32_t)kWaves - 1u) / (uint32_t)kWaves;
                 if constexpr (UNSORTED) {
-                    // (three lists, by what an entry costs: large_batch_lists())
+                    // (two lists, the costly entries in front: large_batch_lists())
                     const SortLists lists = large_batch_lists(d.n_rows);
                     if (flag == 3) {
-                        sc.work_sort[lists.narrow_at + atomicAdd(&sc.work_n[8], 1u)] = row << 8;
+                        sc.work_sort[lists.sorted_at + atomicAdd(&sc.work_n[0], 1u)] = row << 8;
                     } else {
-                        uint32_t at = lists.collectors_at + atomicAdd(&sc.work_n[3], collectors);
+                        uint32_t at = lists.sorted_at - atomicAdd(&sc.work_n[3], collectors) - collectors;
                         for (uint32_t c = 0; c < collectors; ++c)
                             sc.work_sort[at++] = (row << 8) | (kWorkers + c);
                         at = lists.sorted_at + atomicAdd(&sc.work_n[0], kWorkers - n_unsorted);

@@ -35,12 +35,11 @@ __device__ __forceinline__ void sort_body(const mako_sample_desc& d_arg, const S
     const uint32_t item = sc_arg.work_sort[piece];
     const uint64_t tab_word = k_exp2_tab[tid & 31u];
     if constexpr (UNSORTED) {
-        // (three lists, each in a region of workgroup numbers of its own: large_batch_lists())
-        const uint32_t n_collectors = sc_arg.work_n[3], n_narrow = sc_arg.work_n[8];
-        asm volatile("" ::"s"(item), "s"(n_work), "s"(n_collectors), "s"(n_narrow), "s"(pieces_raw), "v"(arg_words.d), "v"(arg_words.sc), "v"(tab_word));
+        // (two lists that meet at workgroup number sorted_at: large_batch_lists())
+        const uint32_t n_collectors = sc_arg.work_n[3];
+        asm volatile("" ::"s"(item), "s"(n_work), "s"(n_collectors), "s"(pieces_raw), "v"(arg_words.d), "v"(arg_words.sc), "v"(tab_word));
         const SortLists lists = large_batch_lists(d_arg.n_rows);
-        const bool with_work = piece < lists.sorted_at ? piece - lists.collectors_at < n_collectors
-                                                       : (piece < lists.narrow_at ? piece - lists.sorted_at < n_work : piece - lists.narrow_at < n_narrow);
+        const bool with_work = piece < lists.sorted_at ? lists.sorted_at - piece <= n_collectors : piece - lists.sorted_at < n_work;
         if (!with_work)
             return;
     } else {
