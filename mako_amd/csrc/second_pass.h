@@ -242,7 +242,7 @@ __device__ void row_pieces(const mako_sample_desc& d, const Scratch& sc, uint32_
     if (first >= n_pieces || !one_piece<VEC, KH, PEN, true, UNSORTED>(d, sc, row, first, slice_len, P, hl, slices, L, pl, m, argidx, opaque_first))
         return;
     for (uint32_t slice = first + stride; slice < n_pieces; slice += stride)
-        one_piece<VEC, KH, PEN, false>(d, sc, row, slice, slice_len, P, hl, slices, L, pl, m, argidx);
+        one_piece<VEC, KH, PEN, false, UNSORTED>(d, sc, row, slice, slice_len, P, hl, slices, L, pl, m, argidx);
 }
 
 // Second pass over the top_k == 0 rows.  grid = (most pieces a row can have, rows) workgroups, of which workgroup i
