@@ -18,7 +18,7 @@ struct GroupLds { // carved from the dynamic LDS block once sorting is over; one
     __device__ __forceinline__ uint32_t* start() const { return cmax() + kMaxGroups; } // first entry of the group
     // entries (bits 0-8) | quarter-record slot + 1 (bits 9-15) | guessed exponent << 16
     __device__ __forceinline__ uint32_t* pack() const { return start() + kMaxGroups; }
-    __device__ __forceinline__ uint32_t* misc() const { return pack() + kMaxGroups; } // [4]; misc[3] counts the quarter-record slots in use
+    __device__ __forceinline__ uint32_t* misc() const { return pack() + kMaxGroups; } // [8]; misc[3] (and [4]: QuarterSlots) count the quarter-record slots in use
     // [kQuarterSlots][4], in the upper half of the dynamic LDS block
     __device__ __forceinline__ uint4* quarters() const { return reinterpret_cast<uint4*>(base + kSortMax); }
     // the walk's maps, bounds and packs ([kMaxGroups] each, behind the quarter records): built while the running
@@ -33,6 +33,12 @@ struct GroupLds { // carved from the dynamic LDS block once sorting is over; one
 constexpr uint32_t kLenMask = 0x1ffu;
 constexpr uint32_t kHasQuarters = 1u << 31;
 constexpr uint32_t kQuarterSlots = 96;
+// Where a builder of group maps takes its quarter-record slots from: G.misc()[counter] counts those handed out of
+// [first, first + slots).  (All of them from one counter, or, for long lists whose maps for the walk are built a block
+// of groups ahead of the walk, the two halves in turn.)
+struct QuarterSlots {
+    uint32_t counter = 3, first = 0, slots = kQuarterSlots;
+};
 constexpr uint32_t kQuarter = kGroup / 4;
 #ifndef MAKO_WALK_PASSED
 #define MAKO_WALK_PASSED 1u
@@ -42,7 +48,7 @@ constexpr uint32_t kSeqMax = 1024; // sorted lists up to this long get their tot
 __device__ __forceinline__ GroupLds group_lds(const FinishLds& L)
 {
     assume_lds(L);
-    static_assert((kMaxGroups + 2) * 8 + 5 * kMaxGroups * 4 + 16 <= kSortMax * 8, "group records fit below the LDS lists");
+    static_assert((kMaxGroups + 2) * 8 + 5 * kMaxGroups * 4 + 32 <= kSortMax * 8, "group records fit below the LDS lists");
     static_assert(kQuarterSlots * 16 == 1536 &&
                       kSortMax * 8 + 1536 * 4 + 4 * kMaxGroups * 4 + (kHeadGroups * kGroup + kWave) * 4 <= kTailLds,
                   "the walk's records sit behind the quarter records and fit the dynamic LDS block");
@@ -345,7 +351,8 @@ __device__ __forceinline__ uint32_t walk_need(float q_first, int eg, uint32_t cm
 // (UNSORTED: the list may hold records of unsorted shares, see unsorted_shares.h)
 template <bool UNSORTED = false, typename Keys>
 __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0, const GroupLds G,
-                                 uint32_t part = wave_id(), uint32_t parts = kWaves, uint32_t g_begin = 0)
+                                 uint32_t part = wave_id(), uint32_t parts = kWaves, uint32_t g_begin = 0,
+                                 const QuarterSlots qs = QuarterSlots{})
 {
     using namespace seqfp;
     uint32_t* const o_d0 = walk ? G.w_d0() : G.d0();
@@ -393,8 +400,10 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
             uint32_t slot = 0;
             if (crossing[u]) {
                 if (lane_id() == 0)
-                    slot = atomicAdd(&G.misc()[3], 1u) + 1u;
+                    slot = atomicAdd(&G.misc()[UNSORTED ? qs.counter : 3u], 1u) + 1u;
                 slot = uniform_u32(slot);
+                if constexpr (UNSORTED)
+                    slot = slot > qs.slots ? kQuarterSlots + 1u : slot + qs.first;
                 if (slot > kQuarterSlots)
                     slot = 0;
                 else if (walk)
@@ -1028,9 +1037,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     // group records: fp64 sums (and, from the workers, the maps of the running sum)
     MAKO_STAMP(5);
     const uint32_t groups1 = PLANNED ? t_groups : (n1 + kGroup - 1) / kGroup;
+    // (UNSORTED: the running sum and the walk's first block of groups share the first half of the quarter-record slots;
+    // the other half is for the maps of the walk's second block, built while the first is walked)
+    constexpr uint32_t kFirstSlots = UNSORTED ? kQuarterSlots / 2u : kQuarterSlots;
     if (tid == 0) {
         G.misc()[3] = 0;
         if (UNSORTED) {
+            G.misc()[4] = 0;
             sm.ticket = 0; // set: a record of an unsorted share where the code below needs the list itself
             sm.flag = 0;   // set: the list has such records
         }
@@ -1082,7 +1095,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             uint32_t slot = 0;
             if (pk & kHasQuarters) {
                 slot = atomicAdd(&G.misc()[3], 1u) + 1u;
-                if (slot > kQuarterSlots)
+                if (slot > kFirstSlots)
                     slot = 0;
             }
             if (slot) {
@@ -1325,7 +1338,11 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     if (wave_id() != 0 && r0_guess == r0_guess && !head_walk) {
         // (all the other waves: with more than kHeadGroups maps to build they take longer than the chain, even
         // though three of them share its SIMD)
-        build_group_maps<UNSORTED>(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u);
+        if constexpr (UNSORTED)
+            build_group_maps<UNSORTED>(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u, 0u,
+                                       QuarterSlots{3u, 0u, kFirstSlots});
+        else
+            build_group_maps(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u);
     }
     if (wave_id() == 0) {
         // 64 groups at a time, one per lane.  A scan composes the lanes' maps; every lane then knows the state after
@@ -1449,26 +1466,54 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         // that guess is worthless (every group would then go entry by entry: 140 us for a 245-group list at
         // u = 0.999), so every later block's maps are built, by all the waves, when the walk gets there, from the
         // exact r at the block's first group.
+        // (UNSORTED, the instance for lists of hundreds of groups: the maps of the NEXT block are built by the other
+        // waves while wave 0 walks this one, from the exact r at this block's first group less the fp64 sums up to the
+        // group, which is as good a guess as the exact r at the next block's first group unless the walk is about to
+        // end; then nothing is built, so that a walk that has ended does not wait for maps nobody needs.  The two
+        // blocks' quarter records take the halves of the slots in turn.)
         for (uint32_t base = 0; base < groups; base += kWave) {
-            if (base > 0) {
-                if (wave_id() == 0 && lane_id() == 0) {
-                    G.misc()[0] = M;
-                    G.misc()[1] = (uint32_t)e;
-                    sm.aux = stopped ? 1u : 0u;
+            if constexpr (!UNSORTED) {
+                if (base > 0) {
+                    if (wave_id() == 0 && lane_id() == 0) {
+                        G.misc()[0] = M;
+                        G.misc()[1] = (uint32_t)e;
+                        sm.aux = stopped ? 1u : 0u;
+                    }
+                    __syncthreads();
+                    if (sm.aux) // uniform
+                        break;
+                    const double r_here = (double)join(G.misc()[0], (int)G.misc()[1]);
+                    if (tid == 0)
+                        G.misc()[3] = 0; // (the quarter records so far are done with: their slots start over)
+                    __syncthreads();
+                    MAKO_TIC(2);
+                    build_group_maps(kf, min(groups, base + (uint32_t)kWave), true, r_here + G.pg()[base], G, wave_id(), kWaves, base);
+                    __syncthreads();
+                    if (wave_id() == 0) {
+                        MAKO_TOC(2, 25);
+                        MAKO_COUNT(26, 1);
+                    }
                 }
-                __syncthreads();
-                if (sm.aux) // uniform
-                    break;
-                const double r_here = (double)join(G.misc()[0], (int)G.misc()[1]);
-                if (tid == 0)
-                    G.misc()[3] = 0; // (the quarter records so far are done with: their slots start over)
-                __syncthreads();
-                MAKO_TIC(2);
-                build_group_maps<UNSORTED>(kf, min(groups, base + (uint32_t)kWave), true, r_here + G.pg()[base], G, wave_id(), kWaves, base);
-                __syncthreads();
-                if (wave_id() == 0) {
-                    MAKO_TOC(2, 25);
-                    MAKO_COUNT(26, 1);
+            } else {
+                double r_here = (double)r0;
+                if (base > 0) {
+                    if (wave_id() == 0 && lane_id() == 0) {
+                        G.misc()[0] = M;
+                        G.misc()[1] = (uint32_t)e;
+                        sm.aux = stopped ? 1u : 0u;
+                        // (the slots of the block before this one are done with: the next block's start over)
+                        G.misc()[3u + (((base / (uint32_t)kWave) + 1u) & 1u)] = 0;
+                    }
+                    __syncthreads();
+                    if (sm.aux) // uniform
+                        break;
+                    r_here = (double)join(G.misc()[0], (int)G.misc()[1]);
+                }
+                const uint32_t next = base + (uint32_t)kWave;
+                if (wave_id() != 0 && next < groups && r_here - (G.pg()[next] - G.pg()[base]) > r_here * -0x1p-6) { // uniform
+                    const uint32_t half = ((next / (uint32_t)kWave) & 1u);
+                    build_group_maps<UNSORTED>(kf, min(groups, next + (uint32_t)kWave), true, r_here + G.pg()[base], G, (uint32_t)wave_id() - 1u,
+                                               (uint32_t)kWaves - 1u, next, QuarterSlots{3u + half, half * (kQuarterSlots / 2u), kQuarterSlots / 2u});
                 }
             }
             if (wave_id() == 0 && !stopped) {
