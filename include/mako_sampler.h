@@ -52,6 +52,7 @@ typedef struct mako_sampling_params {
 #define MAKO_PATH_GENERAL 5u  /* whole-row sort path */
 #define MAKO_PATH_FORCED 6u   /* not sampled: force_token / close_token took the row */
 #define MAKO_PATH_SORTED 7u   /* top_k == 0: nucleus cut from the sorted list of the weights the row's plan kept */
+#define MAKO_PATH_INDEXED 9u  /* neither top-k nor top-p: total and walk in token order over the whole row, by group maps */
 #define MAKO_PATH_SUMMED 8u   /* the same on a batch of many such rows: the parts of the list whose order cannot matter to the
                                  fp32 total and walk were summed, not sorted */
 

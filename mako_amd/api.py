@@ -17,7 +17,7 @@ MAKO_OK = 0
 MAKO_ERR_INVALID_ARG = -1
 MAKO_ERR_HIP = -2
 SAMPLER_KERNELS = 4  # MAKO_SAMPLER_KERNELS
-PATH_GREEDY, PATH_FALLBACK, PATH_TOPK, PATH_NUCLEUS, PATH_GENERAL, PATH_FORCED, PATH_SORTED, PATH_SUMMED = 1, 2, 3, 4, 5, 6, 7, 8
+PATH_GREEDY, PATH_FALLBACK, PATH_TOPK, PATH_NUCLEUS, PATH_GENERAL, PATH_FORCED, PATH_SORTED, PATH_SUMMED, PATH_INDEXED = 1, 2, 3, 4, 5, 6, 7, 8, 9
 FORCED_NONE, FORCED_TOKEN, FORCED_CLOSE = 0, 1, 2
 
 # mako_sampling_params / SamplingParams (src/gen/sampler.hpp:11-20)

@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 # the C ABI, and one translation unit per kernel family (a kernel's register allocation then does not depend on
 # which other kernels exist; they also compile side by side)
-SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_alone.hip", "k_sort.hip", "k_sort_unsorted.hip", "k_tail.hip", "k_tail_unsorted.hip"]
+SOURCES = ["mako_sampler.hip", "k_scan.hip", "k_finish.hip", "k_plan_alone.hip", "k_sort.hip", "k_sort_unsorted.hip", "k_tail.hip", "k_tail_unsorted.hip", "k_index.hip"]
 OBJ_DIR = os.path.join(HERE, "csrc", "_obj")
 OUT = os.path.join(HERE, "libmako_sampler.so")
 # the same library with the kernels' index checks compiled in (-DMAKO_CHECKED): for the test that runs the workloads
@@ -40,6 +40,7 @@ SOURCE_FLAGS = {
     # the rare late rows (the whole-row path, second looks at a cut) out of line beside the tails and the top-k rows
     "k_tail.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", *RARE_CALLS],
     "k_tail_unsorted.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", *RARE_CALLS],
+    "k_index.hip": ["-DMAKO_TOPK_GENERAL_SITE=0", *RARE_CALLS],
     # the whole-row path and the second look at a cut that is too close to call, out of line beside the top-k rows
     "k_plan_alone.hip": RARE_CALLS,
 }

@@ -1,0 +1,35 @@
+// The kernels of the rows whose candidates stay in token order (index_rows.h): a translation unit of their own.
+#define MAKO_EMIT_INDEX_KERNELS
+#include "launch.h"
+#include "sampler_kernels.h"
+
+namespace mako {
+void launch_index_weights(int kh, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices)
+{
+    const dim3 grid((d.n_vocab + kSliceMax - 1u) / kSliceMax, d.n_rows);
+    if (kh == 2)
+        hipLaunchKernelGGL(index_weights_kernel<2>, grid, dim3(kThreads), kDynLds, st, d, sc, slices);
+    else if (kh == 8)
+        hipLaunchKernelGGL(index_weights_kernel<8>, grid, dim3(kThreads), kDynLds, st, d, sc, slices);
+    else
+        hipLaunchKernelGGL(index_weights_kernel<0>, grid, dim3(kThreads), kDynLds, st, d, sc, slices);
+}
+
+void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratch& sc)
+{
+    hipLaunchKernelGGL(index_groups_kernel, dim3((d.n_vocab + kIndexBlock - 1u) / kIndexBlock, d.n_rows), dim3(kThreads), kDynLds, st, d, sc);
+    hipLaunchKernelGGL(index_tail_kernel, dim3(1, d.n_rows), dim3(kThreads), kTailLds, st, d, sc);
+}
+
+hipError_t init_index_kernels()
+{
+    const void* kernels[] = {(const void*)index_weights_kernel<0>, (const void*)index_weights_kernel<2>, (const void*)index_weights_kernel<8>,
+                             (const void*)index_groups_kernel};
+    for (const void* k : kernels) {
+        const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLds);
+        if (e != hipSuccess)
+            return e;
+    }
+    return hipFuncSetAttribute((const void*)index_tail_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTailLds);
+}
+} // namespace mako

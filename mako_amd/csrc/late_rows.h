@@ -102,6 +102,8 @@ __device__ MAKO_RARE_CALL void finish_late_row(const mako_sample_desc& d, const 
     const RowClass cls = classify(P);
     if ((d.force_token || d.close_token || cls == kGreedy) && late_plain_row(d, sc, cls, row, slices))
         return;
+    if (cls == kGeneral && sc.plan[row].flag == kIndexClaimed) // (a row in token order that the kernels of index_rows.h finish)
+        return;
     if (cls == kNucleus) {
         // (the flag is never set for a row whose token is forced: the second pass leaves such a row alone)
         const uint32_t flag = sc.plan[row].flag;

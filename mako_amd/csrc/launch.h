@@ -34,4 +34,9 @@ void launch_plan_alone(hipStream_t st, const mako_sample_desc& d, const Scratch&
 void launch_sort(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t grid_rows, bool unsorted); // (host copy)
 // (tail_kernel: `tail_cap` workgroups for the possible wide rows, then one per row for what is left of every row)
 void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices, uint32_t tail_cap, bool unsorted); // (host copy, by value)
+// the three kernels of the rows whose candidates stay in token order (index_rows.h): the weights (before tail_kernel's
+// launch, which then leaves such rows alone), the group records, the total and the draw (behind it)
+hipError_t init_index_kernels();
+void launch_index_weights(int kh, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices);
+void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratch& sc);
 } // namespace mako

@@ -245,6 +245,7 @@ int mako_sampler_create(mako_sampler_ctx** out, int device, uint32_t max_rows, u
     MAKO_HIP(ctx, mako::init_plan_alone());
     MAKO_HIP(ctx, mako::init_sort_kernels());
     MAKO_HIP(ctx, mako::init_tail_kernels());
+    MAKO_HIP(ctx, mako::init_index_kernels());
     return MAKO_OK;
 }
 
@@ -402,15 +403,21 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     } while (0)
     // which kernels have work: all of them unless the caller's host copy of the parameters says otherwise
     // (any_late: rows that are finished in tail_kernel's launch, after the plan)
-    bool any_nucleus = true, any_late = true;
+    // (any_index: rows cut neither to a top-k nor to a nucleus, whose candidates stay in token order; known only from
+    // the caller's copy of the parameters, they get the kernels of index_rows.h instead of a workgroup each on the
+    // whole-row path, unless the batch is one those kernels do not serve: verification, forced tokens, rows that are
+    // not aligned for 128-bit loads, a vocabulary beyond 262 144)
+    bool any_nucleus = true, any_late = true, any_index = false;
     uint32_t nucleus_rows = d.n_rows;
     if (params_host) {
         any_nucleus = any_late = false;
         uint32_t n_nucleus = 0;
+        const bool index_served = vec && !d.draft && !d.force_token && !d.close_token && d.n_vocab <= mako::kIndexMaxVocab;
         for (uint32_t r = 0; r < d.n_rows; ++r) {
             const mako::RowClass c = mako::classify(params_host[r]);
             any_nucleus |= c == mako::kNucleus;
             any_late |= c == mako::kGeneral;
+            any_index |= index_served && mako::index_order_row(params_host[r]);
             n_nucleus += c == mako::kNucleus;
         }
         nucleus_rows = std::max(n_nucleus, 1u);
@@ -440,6 +447,8 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     // top_k == 0 rows: planned and handed out by the second pass, sorted, cut and drawn from; the stages talk through
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  A batch without such rows
     // (and without rows for the whole-row path) ends with plan_kernel instead.
+    if (any_index) // (before the launch that finishes late rows: it leaves alone what this one has claimed)
+        MAKO_LAUNCH(mako::launch_index_weights(kh, st, d, sc, slices));
     if (any_nucleus)
         MAKO_LAUNCH(mako::launch_finish(vec, kh, unsorted, finish_wgs, st, d, sc, slices));
     if (!launch_sort)
@@ -450,6 +459,8 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     MAKO_MARK(3);
     if (launch_sort) // (also finishes every row the kernels before it leave: finish_late_row())
         MAKO_LAUNCH(mako::launch_tail(st, d, sc, slices, nucleus_rows, unsorted));
+    if (any_index)
+        MAKO_LAUNCH(mako::launch_index_finish(st, d, sc));
     MAKO_MARK(4);
 #undef MAKO_MARK
 #undef MAKO_LAUNCH

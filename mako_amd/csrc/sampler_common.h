@@ -238,6 +238,17 @@ __host__ __device__ __forceinline__ RowClass classify(const mako_sampling_params
     return p.top_k <= kTopKFast ? kTopK : kGeneral;
 }
 
+// Rows that are cut neither to a top-k nor to a nucleus: their candidates stay in token order.  With the caller's host
+// copy of the parameters such rows get kernels of their own (index_rows.h), which hand a row on through BigPlan::flag:
+__host__ __device__ __forceinline__ bool index_order_row(const mako_sampling_params& p)
+{
+    return p.temperature > 0.0f && !(p.top_p < 1.0f) && p.top_k == 0u;
+}
+constexpr uint32_t kIndexClaimed = 6; // index_weights_kernel has the row: the kernels that finish late rows leave it alone
+constexpr uint32_t kIndexReady = 7;   // the group records are in place
+constexpr uint32_t kIndexWhole = 8;   // the whole-row path is wanted (candidates to be written out from a list with gaps)
+constexpr uint32_t kIndexEmpty = 9;   // no candidate survived
+
 __device__ __forceinline__ bool penalties_neutral(const mako_sampling_params& p)
 {
     return p.repetition_penalty == 1.0f && p.presence_penalty == 0.0f && p.frequency_penalty == 0.0f;

@@ -34,3 +34,4 @@
 #include "sort_kernels.h"
 #include "late_rows.h"
 #include "tail_kernel.h"
+#include "index_rows.h"

@@ -165,6 +165,9 @@ __device__ __forceinline__ void load_span(const uint32_t* kf, uint32_t start, ui
 // ties is a span of constant increments, and their composition is their sum (saturated like compose32()): one wave
 // reduction of one number instead of a six-step scan of two.  The largest single step is the first entry's (a weight's
 // step never grows as the weight falls): no reduction at all.
+// (UNORDERED: the span's entries come in any order, as those of a list in token order do: the composition is the same,
+// in the order given, but the largest single step has to be looked for.)
+template <bool UNORDERED = false>
 __device__ __forceinline__ seqfp::Step32 span_map(const float (&q)[4], uint32_t len, int eg)
 {
     using namespace seqfp;
@@ -177,7 +180,11 @@ __device__ __forceinline__ seqfp::Step32 span_map(const float (&q)[4], uint32_t 
             e[j] = lane_id() * 4u + j < len ? step32_flat(q[j], eg) : identity32();
             tie |= e[j].d0 != e[j].d1;
         }
-        const uint32_t cmax = (uint32_t)__builtin_amdgcn_readfirstlane((int)e[0].cmax);
+        uint32_t cmax;
+        if constexpr (UNORDERED)
+            cmax = __ockl_wfred_max_u32(max(max(e[0].cmax, e[1].cmax), max(e[2].cmax, e[3].cmax)));
+        else
+            cmax = (uint32_t)__builtin_amdgcn_readfirstlane((int)e[0].cmax);
         if (__ballot(tie) == 0ull) {
             // (a lane's four increments: below 2^26, or marked unusable; clamped so that 64 of them cannot wrap)
             const uint32_t mine = min(e[0].d0 + e[1].d0 + e[2].d0 + e[3].d0, 1u << 25);
@@ -276,6 +283,7 @@ __device__ void build_quarters(const float (&q)[4], uint32_t len, double at_star
 // the binade guessed from r at the group's first entry minus the fp64 sum up to ITS first entry: (d0, d1, need,
 // exponent), `need` being the bound of group_sub_ok as one number (the state after the quarter must be at least the
 // quarter's first, largest weight, and inside the binade with room for one more decrement).  One wave.
+template <bool UNORDERED = false>
 __device__ void build_walk_quarters(const float (&q)[4], uint32_t len, double r_start, uint4* out)
 {
     using namespace seqfp;
@@ -307,7 +315,9 @@ __device__ void build_walk_quarters(const float (&q)[4], uint32_t len, double r_
     const uint32_t qb = __float_as_uint(q[0]);
     const uint32_t f0 = (uint32_t)__builtin_amdgcn_readlane((int)qb, 0), f1 = (uint32_t)__builtin_amdgcn_readlane((int)qb, 16);
     const uint32_t f2 = (uint32_t)__builtin_amdgcn_readlane((int)qb, 32), f3 = (uint32_t)__builtin_amdgcn_readlane((int)qb, 48);
-    const float q_first = __uint_as_float(quarter == 0 ? f0 : (quarter == 1 ? f1 : (quarter == 2 ? f2 : f3)));
+    float q_first = __uint_as_float(quarter == 0 ? f0 : (quarter == 1 ? f1 : (quarter == 2 ? f2 : f3)));
+    if constexpr (UNORDERED) // (the quarter's largest weight, wherever it is: positive floats order like their bits)
+        q_first = __uint_as_float(row_scan_max_u32(max(max(__float_as_uint(q[0]), __float_as_uint(q[1])), max(__float_as_uint(q[2]), __float_as_uint(q[3])))));
     uint32_t Mq;
     int eq;
     split(q_first, Mq, eq);
@@ -349,7 +359,8 @@ __device__ __forceinline__ uint32_t walk_need(float q_first, int eg, uint32_t cm
 // d1 / cmax / pack) or of the walk (into G.w_d0 / w_d1 / w_need / w_pack; r0 - pg[g] is the estimate of r at group
 // g).  The calling wave is number `part` of `parts` that share the work.
 // (UNSORTED: the list may hold records of unsorted shares, see unsorted_shares.h)
-template <bool UNSORTED = false, typename Keys>
+// (UNORDERED: a list in any order; see span_map)
+template <bool UNSORTED = false, bool UNORDERED = false, typename Keys>
 __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0, const GroupLds G,
                                  uint32_t part = wave_id(), uint32_t parts = kWaves, uint32_t g_begin = 0,
                                  const QuarterSlots qs = QuarterSlots{})
@@ -396,7 +407,7 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
             if (keep[u]) // uniform
                 continue;
             MAKO_COUNT(walk ? 27 : 28, 1);
-            const Step32 st = span_map(q[u], len[u], eg[u]);
+            const Step32 st = span_map<UNORDERED>(q[u], len[u], eg[u]);
             uint32_t slot = 0;
             if (crossing[u]) {
                 if (lane_id() == 0)
@@ -407,15 +418,18 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
                 if (slot > kQuarterSlots)
                     slot = 0;
                 else if (walk)
-                    build_walk_quarters(q[u], len[u], guess[u], G.quarters() + (slot - 1u) * 4u);
+                    build_walk_quarters<UNORDERED>(q[u], len[u], guess[u], G.quarters() + (slot - 1u) * 4u);
                 else
                     build_quarters(q[u], len[u], G.pg()[g], G.quarters() + (slot - 1u) * 4u);
             }
+            float q_top = q[u][0]; // (lane 0 holds the group's first, largest weight)
+            if constexpr (UNORDERED)
+                q_top = __uint_as_float(__ockl_wfred_max_u32(max(max(__float_as_uint(q[u][0]), __float_as_uint(q[u][1])),
+                                                                 max(__float_as_uint(q[u][2]), __float_as_uint(q[u][3])))));
             if (lane_id() == 0) {
-                // (walk: lane 0 holds the group's first, largest weight)
                 o_d0[g] = st.d0;
                 o_d1[g] = st.d1;
-                o_c[g] = walk ? walk_need(q[u][0], eg[u], st.cmax) : st.cmax;
+                o_c[g] = walk ? walk_need(q_top, eg[u], st.cmax) : st.cmax;
                 o_pack[g] = len[u] | (slot << 9) | ((uint32_t)eg[u] << 16);
             }
         }
@@ -875,7 +889,10 @@ __device__ MAKO_RARE_CALL double reference_total(Get q_at, uint32_t n, FinishSha
 // SHORT_ONLY: the caller's lists never exceed kGroup entries; the code for longer ones is left out.
 // UNSORTED (with PLANNED): some of the workers' shares may have been left unsorted, as one record each
 // (unsorted_shares.h); a row whose records of that kind cannot all be applied is given up (false).
-template <bool PLANNED = false, bool SHORT_ONLY = false, bool EXACT = false, bool UNSORTED = false>
+// UNORDERED (with PLANNED, without a top-p): the list is in token order, not sorted (a row that is neither cut to a
+// top-k nor to a nucleus: src/gen/sampler.cpp:79-83 and :64-72 over the candidates as they come); nothing here needs
+// the order except the bounds that stand for "the largest weight of a span", which are then looked for.
+template <bool PLANNED = false, bool SHORT_ONLY = false, bool EXACT = false, bool UNSORTED = false, bool UNORDERED = false>
 __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf_ptr,
                             const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
                             const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, const GroupTable& T = GroupTable{},
@@ -1342,7 +1359,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             build_group_maps<UNSORTED>(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u, 0u,
                                        QuarterSlots{3u, 0u, kFirstSlots});
         else
-            build_group_maps(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u);
+            build_group_maps<false, UNORDERED>(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u);
     }
     if (wave_id() == 0) {
         // 64 groups at a time, one per lane.  A scan composes the lanes' maps; every lane then knows the state after
@@ -1487,7 +1504,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         G.misc()[3] = 0; // (the quarter records so far are done with: their slots start over)
                     __syncthreads();
                     MAKO_TIC(2);
-                    build_group_maps(kf, min(groups, base + (uint32_t)kWave), true, r_here + G.pg()[base], G, wave_id(), kWaves, base);
+                    build_group_maps<false, UNORDERED>(kf, min(groups, base + (uint32_t)kWave), true, r_here + G.pg()[base], G, wave_id(), kWaves, base);
                     __syncthreads();
                     if (wave_id() == 0) {
                         MAKO_TOC(2, 25);

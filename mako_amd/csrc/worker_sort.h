@@ -420,6 +420,8 @@ __device__ void opaque_share(const uint32_t* ks, uint32_t cnt, uint32_t off, int
 // kf_lds (optional): the worker's cnt sorted weights in LDS (outside L.sortk's first 16 KB), read instead of kf + off.
 // r0: the estimate of where the walk starts, u * top_p * (the row's total): the groups that r can reach also get their
 // map for the walk, for the epoch guessed from r0 less the mass before the group (0 or less: none).
+// (UNORDERED: the entries are in any order, e.g. a stretch of a row in token order: see span_map)
+template <bool UNORDERED = false>
 __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, size_t t_at, double mass, const GroupTable& T,
                               const FinishLds L, const uint32_t* kf_lds = nullptr, double r0 = 0.0)
 {
@@ -480,7 +482,7 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
         load_span(src, g * kGroup, len, q);
         const double guess = few ? readlane_f64(before_l, g) : gs[g];
         const int eg = guess > 0 ? exponent_of((float)guess) : 0;
-        const seqfp::Step32 st = span_map(q, len, eg);
+        const seqfp::Step32 st = span_map<UNORDERED>(q, len, eg);
         // the sum is expected to change binade inside the group (or starts at zero): records for its quarters
         const double at_end = few ? readlane_f64(after_l, g) : ge[g];
         const bool split4 = uniform_u32((uint32_t)(eg == 0 || exponent_of((float)at_end) != eg)) != 0;
@@ -491,8 +493,11 @@ __device__ void worker_groups(const uint32_t* kf, uint32_t off, uint32_t cnt, si
         const int ew = (r0 > 0.0 && r_after > 0.0) ? exponent_of((float)r_here) : 0;
         uint4 wrec = make_uint4(0u, 0u, 0u, 0u);
         if (ew > 0 && uniform_u32((uint32_t)(exponent_of((float)r_after) == ew)) != 0) {
-            const seqfp::Step32 sw = span_map(q, len, ew);
-            wrec = make_uint4(sw.d0, sw.d1, walk_need(q[0], ew, sw.cmax), (uint32_t)ew); // (lane 0: the group's first weight)
+            const seqfp::Step32 sw = span_map<UNORDERED>(q, len, ew);
+            float q_top = q[0]; // (lane 0: the group's first, largest weight)
+            if constexpr (UNORDERED)
+                q_top = __uint_as_float(__ockl_wfred_max_u32(max(max(__float_as_uint(q[0]), __float_as_uint(q[1])), max(__float_as_uint(q[2]), __float_as_uint(q[3])))));
+            wrec = make_uint4(sw.d0, sw.d1, walk_need(q_top, ew, sw.cmax), (uint32_t)ew);
         }
         if (lane_id() == 0) {
             T.d0[t_at + g] = st.d0;

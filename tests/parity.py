@@ -25,15 +25,17 @@ def oracle_rows(w, rows=None, cap=0, order_mode=0, draft=None, u2=None):
         return list(ex.map(one, rows))
 
 
-def gpu_rows(ctx, w, cap=0, draft=None, u2=None, hist_counts=None):
+def gpu_rows(ctx, w, cap=0, draft=None, u2=None, hist_counts=None, hinted=False):
+    """(hinted: the call also gets the host copy of the parameters, from which the library learns the rows' kinds)"""
     return api.sample(ctx, w["logits"], w["params"], w["u"], mask=w.get("mask"), hist=w.get("hist"),
-                      hist_len=w.get("hist_len"), hist_counts=hist_counts, draft=draft, u2=u2, cand_cap=cap)
+                      hist_len=w.get("hist_len"), hist_counts=hist_counts, draft=draft, u2=u2, cand_cap=cap,
+                      params_host=hinted)
 
 
-def assert_parity(ctx, w, cap=256, rel_tol=1e-5):
+def assert_parity(ctx, w, cap=256, rel_tol=1e-5, hinted=False):
     """Token ids, candidate counts, candidate id lists and weights must match the oracle exactly;
     probabilities q/total within rel_tol (they are in fact bit-identical)."""
-    g = gpu_rows(ctx, w, cap=cap)
+    g = gpu_rows(ctx, w, cap=cap, hinted=hinted)
     ref = oracle_rows(w, cap=cap)
     bad = []
     for r, (t, tr) in enumerate(ref):
@@ -47,10 +49,10 @@ def assert_parity(ctx, w, cap=256, rel_tol=1e-5):
             bad.append((r, "n_cand", int(g["n_cand"][r]), tr["n_cand"]))
             continue
         n = min(cap, tr["n_cand"])
-        if not np.array_equal(g["cand_idx"][r, :n], tr["cand_idx"][:n]):
+        if n and not np.array_equal(g["cand_idx"][r, :n], tr["cand_idx"][:n]):
             bad.append((r, "cand_idx"))
             continue
-        if not np.array_equal(g["cand_q"][r, :n].view(np.uint32), tr["cand_q"][:n].view(np.uint32)):
+        if n and not np.array_equal(g["cand_q"][r, :n].view(np.uint32), tr["cand_q"][:n].view(np.uint32)):
             bad.append((r, "cand_q"))
             continue
         if np.float32(g["total"][r]).view(np.uint32) != np.float32(tr["total"]).view(np.uint32):

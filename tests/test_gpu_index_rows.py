@@ -1,0 +1,137 @@
+"""GPU parity of rows that are cut neither to a top-k nor to a nucleus (temperature only: top_k = 0, top_p = 1), whose
+candidates the reference adds up and walks in token order (src/gen/sampler.cpp:79-83, :64-72).  With the caller's host
+copy of the parameters such rows take kernels of their own (mako_amd/csrc/index_rows.h: weights in place, group records,
+exact fp32 total and walk by group maps over the unsorted list); tokens, candidate counts, candidate lists and fp32
+totals must be the oracle's bit for bit, with gaps in the list (masks, min_p, underflow), at both ends of u, beside rows
+of every other kind, and the results must equal those of the call without the host copy (the whole-row path)."""
+import numpy as np
+import pytest
+
+from mako_amd import api, workloads
+from parity import assert_parity, gpu_rows
+
+pytestmark = pytest.mark.gpu
+
+PATH_INDEXED, PATH_GENERAL = api.PATH_INDEXED, api.PATH_GENERAL
+
+
+def _say(msg):
+    print(msg, flush=True)
+
+
+def _plain_batch(rows, vocab, seed, sigmas=(3.0,), temps=(0.7,), us=None, spikes=True):
+    rng = np.random.Generator(np.random.PCG64([seed, 91]))
+    logits = np.empty((rows, vocab), np.float32)
+    p = workloads.make_params(rows, 1.0, 0, 1.0)
+    for r in range(rows):
+        row = (rng.standard_normal(vocab) * sigmas[r % len(sigmas)]).astype(np.float32)
+        if spikes:
+            row[rng.integers(0, vocab, 20)] += np.float32(10.0)
+        logits[r] = row
+        p["temperature"][r] = temps[(r // len(sigmas)) % len(temps)]
+    u = workloads._uniforms(rng, rows) if us is None else np.asarray([us[r % len(us)] for r in range(rows)], np.float32)
+    return dict(name="temperature only %d" % seed, logits=logits, params=p, u=u)
+
+
+def _paths(g):
+    return np.bincount(g["path"], minlength=10).tolist()
+
+
+def test_temperature_only_rows(gpu_ctx):
+    w = _plain_batch(64, 129280, 1, sigmas=(3.0, 1.0, 0.1, 6.0), temps=(0.7, 1.0, 1.5))
+    g = assert_parity(gpu_ctx, w, cap=300, hinted=True)
+    _say("temperature only paths: %s" % _paths(g))
+    assert (g["path"] == PATH_INDEXED).all()
+
+
+def test_walk_ends_everywhere(gpu_ctx):
+    us = [0.0, 2.0**-24, 1e-6, 1e-3, 0.1, 0.25, 0.4999999, 0.5, 0.5000001, 0.75, 0.9, 0.99, 0.999, 0.99999,
+          1.0 - 2.0**-23, 1.0 - 2.0**-24]
+    w = _plain_batch(64, 151552, 2, sigmas=(3.0, 0.05), temps=(1.0, 0.8), us=us)
+    g = assert_parity(gpu_ctx, w, cap=64, hinted=True)
+    _say("walk ends paths: %s" % _paths(g))
+    assert (g["path"] == PATH_INDEXED).all()
+
+
+def test_gaps_in_the_list(gpu_ctx):
+    """Masks, a min_p floor and a cold temperature (weights that underflow to zero) leave logits that are no
+    candidates: with no candidate list asked for the rows stay on the new path, with one they take the whole-row
+    path; either way the oracle's results."""
+    rng = np.random.Generator(np.random.PCG64([3, 92]))
+    rows, vocab = 48, 129280
+    w = _plain_batch(rows, vocab, 3, sigmas=(3.0, 8.0), temps=(0.3, 1.0, 0.1))
+    w["params"]["min_p"][::3] = np.float32(1e-3)
+    words = (vocab + 31) // 32
+    bits = rng.random((rows, words * 32)) < 0.6
+    bits[:, vocab:] = False
+    bits[1::4] = True
+    bits[:, vocab:] = False
+    w["mask"] = np.ascontiguousarray(np.packbits(bits.reshape(rows, words, 32), axis=2, bitorder="little").view(np.uint32).reshape(rows, words))
+    g0 = assert_parity(gpu_ctx, w, cap=0, hinted=True)
+    _say("gaps, no candidate lists, paths: %s" % _paths(g0))
+    assert (g0["path"] == PATH_INDEXED).sum() >= rows - 2
+    g1 = assert_parity(gpu_ctx, w, cap=500, hinted=True)
+    _say("gaps, candidate lists, paths: %s" % _paths(g1))
+    assert np.array_equal(g0["tokens"], g1["tokens"])
+
+
+def test_penalties_and_histories(gpu_ctx):
+    rng = np.random.Generator(np.random.PCG64([4, 93]))
+    rows, vocab, hl = 40, 129280, 2048
+    w = _plain_batch(rows, vocab, 4, sigmas=(3.0,), temps=(0.9, 1.2))
+    w["params"]["repetition_penalty"] = 1.1
+    w["params"]["frequency_penalty"] = 0.2
+    w["params"]["presence_penalty"] = 0.3
+    w["hist"] = workloads.zipf_history(rng, workloads._zipf_cdf(vocab), rows, hl)
+    w["hist_len"] = rng.integers(0, hl + 1, rows).astype(np.uint32)
+    g = assert_parity(gpu_ctx, w, cap=128, hinted=True)
+    _say("penalties paths: %s" % _paths(g))
+    assert (g["path"] == PATH_INDEXED).all()
+
+
+def test_beside_rows_of_every_kind(gpu_ctx):
+    """config 3's batch with every fourth row made a temperature-only row."""
+    w = workloads.config3()
+    w["params"]["top_p"][::4] = np.float32(1.0)
+    w["params"]["top_k"][::4] = 0
+    g = assert_parity(gpu_ctx, w, cap=256, hinted=True)
+    _say("mixed batch paths: %s" % _paths(g))
+    # (cold rows have weights that underflow: with candidate lists asked for they take the whole-row path)
+    assert np.isin(g["path"][::4], [PATH_INDEXED, PATH_GENERAL]).all() and (g["path"][::4] == PATH_INDEXED).sum() >= 4
+    assert not (np.delete(g["path"], np.s_[::4]) == PATH_INDEXED).any()
+    h = gpu_rows(gpu_ctx, w, cap=256)
+    assert (h["path"][::4] == PATH_GENERAL).all()
+    assert np.array_equal(h["tokens"], g["tokens"]) and np.array_equal(h["total"].view(np.uint32), g["total"].view(np.uint32))
+    assert np.array_equal(h["n_cand"], g["n_cand"])
+
+
+@pytest.mark.parametrize("vocab", [4, 252, 260, 4096, 4100, 20000, 65536])
+def test_small_and_odd_vocabularies(vocab):
+    ctx = api.SamplerContext(max_rows=24, max_vocab=vocab, max_hist=0)
+    try:
+        w = _plain_batch(24, vocab, 100 + vocab, sigmas=(2.0, 0.2), temps=(0.6, 1.0), spikes=False)
+        g = assert_parity(ctx, w, cap=64, hinted=True)
+    finally:
+        ctx.close()
+    _say("V = %d paths: %s" % (vocab, _paths(g)))
+    assert (g["path"] == PATH_INDEXED).all()
+
+
+def test_rows_the_kernels_do_not_serve():
+    """A vocabulary that is no multiple of four: the rows take the whole-row path as before."""
+    ctx = api.SamplerContext(max_rows=8, max_vocab=4099, max_hist=0)
+    try:
+        w = _plain_batch(8, 4099, 7, spikes=False)
+        g = assert_parity(ctx, w, cap=64, hinted=True)
+    finally:
+        ctx.close()
+    assert (g["path"] == PATH_GENERAL).all()
+
+
+def test_no_candidate_survives(gpu_ctx):
+    """Every logit masked out but for NaNs' sake nothing survives: the fallback token (sampler.cpp:37-38)."""
+    w = _plain_batch(8, 129280, 8)
+    w["logits"][0:4] = -np.inf
+    w["logits"][4:6] = np.nan
+    g = assert_parity(gpu_ctx, w, cap=16, hinted=True)
+    _say("empty rows paths: %s" % _paths(g))
