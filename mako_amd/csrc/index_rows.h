@@ -4,9 +4,9 @@
 // of their own instead of one workgroup per row on the whole-row path:
 //   index_weights_kernel  a workgroup per 16 384 logits: masks and penalties as everywhere, q = expf((w - m) / T), and
 //                         ~bits(q) (0.0f for a logit that is no candidate) stored at the token's own position;
-//   index_groups_kernel   a workgroup per 4 096 entries: the group records of its sixteen groups of 256 (fp64 sums, the
-//                         maps of the running fp32 sum and of the walk for the binades guessed from the sums before
-//                         them), as sort_kernel's workers leave them for a sorted list;
+//   index_groups_kernel   a workgroup per 16 384 entries: the group records of its 64 groups of 256 (fp64 sums, the maps
+//                         of the running fp32 sum and of the walk for the binades guessed from the sums before them),
+//                         as sort_kernel's workers leave them for a sorted list;
 //   index_tail_kernel     a workgroup per row: the exact fp32 total and the walk over the group records
 //                         (sorted_tail's planned instance for lists in any order).
 // A logit that is no candidate stays in the list as a weight of 0.0f: adding it changes no sum, and the walk's
@@ -20,9 +20,9 @@
 
 namespace mako {
 
-constexpr uint32_t kIndexBlock = 4096;                       // entries per workgroup of index_groups_kernel
-constexpr uint32_t kIndexMaxVocab = kMaxSlices * kIndexBlock; // a sum per block in Scratch::part_sum's row
-static_assert(kIndexMaxVocab <= kMaxGroups * kGroup && kSliceMax == 4u * kIndexBlock && kIndexBlock % kGroup == 0, "blocks, groups");
+constexpr uint32_t kIndexMaxVocab = kMaxGroups * kGroup; // the group records of a row
+static_assert(kIndexMaxVocab / kSliceMax <= kWorkers && kIndexMaxVocab / kSliceMax <= kMaxSlices && kSliceMax == (uint32_t)kWave * kGroup,
+              "a piece's count, last candidate and sum travel in the plan's per-worker words and the row's part_sum; a lane per group");
 #ifdef MAKO_EMIT_INDEX_KERNELS
 // grid = (ceil(V / 16384), rows); rows of other kinds leave at once.  V % 4 == 0 and aligned rows (the host checks).
 template <int KH>
@@ -60,8 +60,8 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
 #pragma unroll
     for (uint32_t b = 0; b < 4; ++b) {
         bsum[b] = 0.0;
-        const uint32_t base = lo + b * kIndexBlock + tid * 4u;
-        if (lo + b * kIndexBlock < hi) { // uniform
+        const uint32_t base = lo + b * 4096u + tid * 4u;
+        if (lo + b * 4096u < hi) { // uniform
             uint32_t k[4];
 #pragma unroll
             for (uint32_t c = 0; c < 4; ++c) {
@@ -84,40 +84,40 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
                     }
             }
         }
+        // (four weights at a time: with all sixteen in flight the kernel needs twice the registers, and two workgroups
+        // no longer share a CU)
+        __builtin_amdgcn_sched_barrier(0);
     }
-    // the blocks' fp64 sums (estimates for the binades only: any order of addition will do), the piece's candidates
-    // and its last one
-    double* wsum = reinterpret_cast<double*>(s_dyn64); // [4][kWaves] (the penalty table is done with)
-    uint32_t* wcnt = reinterpret_cast<uint32_t*>(wsum + 4 * kWaves);
+    // the piece's fp64 sum (an estimate for the binades only: any order of addition will do), its candidates and its
+    // last one
+    double* wsum = reinterpret_cast<double*>(s_dyn64); // [kWaves] (the penalty table is done with)
+    uint32_t* wcnt = reinterpret_cast<uint32_t*>(wsum + kWaves);
     __syncthreads();
-#pragma unroll
-    for (uint32_t b = 0; b < 4; ++b) {
-        const double s = __ockl_wfred_add_f64(bsum[b]);
-        if (lane_id() == 0)
-            wsum[b * kWaves + wave_id()] = s;
-    }
-    cnt = __ockl_wfred_add_u32(cnt);
-    last = __ockl_wfred_max_u32(last);
-    if (lane_id() == 0) {
-        wcnt[wave_id()] = cnt;
-        wcnt[kWaves + wave_id()] = last;
+    {
+        const double s = __ockl_wfred_add_f64((bsum[0] + bsum[1]) + (bsum[2] + bsum[3]));
+        cnt = __ockl_wfred_add_u32(cnt);
+        last = __ockl_wfred_max_u32(last);
+        if (lane_id() == 0) {
+            wsum[wave_id()] = s;
+            wcnt[wave_id()] = cnt;
+            wcnt[kWaves + wave_id()] = last;
+        }
     }
     __syncthreads();
-    if (tid < 4 && lo + tid * kIndexBlock < hi) {
-        double s = 0.0;
-        for (int w = 0; w < kWaves; ++w)
-            s += wsum[tid * kWaves + w];
-        sc.part_sum[(size_t)row * kMaxSlices + piece * 4u + tid] = s;
+    double sum = 0.0;
+    if (tid == 0) {
+        cnt = last = 0;
+        for (int w = 0; w < kWaves; ++w) {
+            sum += wsum[w];
+            cnt += wcnt[w];
+            last = max(last, wcnt[kWaves + w]);
+        }
     }
     if (tid == 0) {
-        uint32_t c = 0, l = 0;
-        for (int w = 0; w < kWaves; ++w) {
-            c += wcnt[w];
-            l = max(l, wcnt[kWaves + w]);
-        }
         BigPlan* plan = sc.plan + row;
-        plan->cursor[piece] = c; // (the pieces' counts and last candidates travel in the plan's per-worker words)
-        plan->key_lo[piece] = l;
+        sc.part_sum[(size_t)row * kMaxSlices + piece] = sum;
+        plan->cursor[piece] = cnt; // (the pieces' counts and last candidates travel in the plan's per-worker words)
+        plan->key_lo[piece] = last;
         if (piece == 0) {
             plan->flag = kIndexClaimed;
             plan->m = m;
@@ -126,25 +126,26 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
     }
 }
 
-// grid = (ceil(V / 4096), rows).
+// grid = (ceil(V / 16384), rows): workgroup p leaves the records of the groups of entries [16384 p, 16384 (p + 1)).
+// Wave w takes the groups w, w + 16, w + 32 and w + 48 of those: their entries in one trip to memory, their fp64 sums to
+// LDS, and once every wave has the sums before each group, the maps from the entries it still holds.
 __global__ __launch_bounds__(kThreads) void index_groups_kernel(mako_sample_desc d_arg, Scratch sc_val)
 {
-    extern __shared__ __align__(16) unsigned long long s_dyn64[];
-    __shared__ FinishShared sm;
-    const uint32_t row = blockIdx.y, b = blockIdx.x, tid = threadIdx.x, lane = lane_id();
+    __shared__ double s_gs[kWave];
+    const uint32_t row = blockIdx.y, p = blockIdx.x, tid = threadIdx.x, lane = lane_id(), wave = wave_id();
     const mako_sampling_params P0 = d_arg.params[row];
     if (!index_order_row(P0)) // uniform
         return;
     BigPlan* plan = sc_val.plan + row;
-    const uint32_t pieces = (d_arg.n_vocab + kSliceMax - 1u) / kSliceMax, blocks = (d_arg.n_vocab + kIndexBlock - 1u) / kIndexBlock;
+    const uint32_t pieces = (d_arg.n_vocab + kSliceMax - 1u) / kSliceMax;
     const uint32_t cnt_l = lane < pieces ? plan->cursor[min(lane, kWorkers - 1u)] : 0u;
     const uint32_t last_l = lane < pieces ? plan->key_lo[min(lane, kWorkers - 1u)] : 0u;
-    const double ps = lane < blocks ? sc_val.part_sum[(size_t)row * kMaxSlices + lane] : 0.0;
+    const double ps = lane < pieces ? sc_val.part_sum[(size_t)row * kMaxSlices + lane] : 0.0;
     const float u_row = d_arg.u[row];
     const uint32_t n_cand = __ockl_wfred_add_u32(cnt_l), n_list = __ockl_wfred_max_u32(last_l);
     const double incl = __ockl_wfscan_add_f64(ps, true);
-    const double total64 = readlane_f64(incl, kWave - 1), mass = readlane_f64(incl - ps, b);
-    if (b == 0 && tid == 0) {
+    const double total64 = readlane_f64(incl, kWave - 1), mass = readlane_f64(incl - ps, p);
+    if (p == 0 && tid == 0) {
         plan->n0 = n_list;
         plan->groups = (n_list + kGroup - 1u) / kGroup;
         plan->total64 = total64;
@@ -152,13 +153,65 @@ __global__ __launch_bounds__(kThreads) void index_groups_kernel(mako_sample_desc
         const bool gaps_matter = n_cand < n_list && d_arg.out_cand_idx && d_arg.out_cand_q && d_arg.cand_cap;
         plan->flag = n_cand == 0u ? kIndexEmpty : (gaps_matter ? kIndexWhole : kIndexReady);
     }
-    if (n_cand == 0u || b * kIndexBlock >= n_list) // uniform
+    if (n_cand == 0u || p * kSliceMax >= n_list) // uniform
         return;
-    const FinishLds L = finish_lds_views(sm, s_dyn64);
-    const double r0_raw = (double)u_row * total64;
-    const uint32_t* key0 = sc_val.key[0] + (size_t)row * sc_val.vpad;
-    worker_groups<true>(key0, b * kIndexBlock, min(kIndexBlock, n_list - b * kIndexBlock),
-                        (size_t)row * sc_val.g_cap + b * (kIndexBlock / kGroup), mass, sc_val.gt, L, nullptr, r0_raw == r0_raw ? r0_raw : 0.0);
+    const uint32_t off = p * kSliceMax, cnt = min(kSliceMax, n_list - off);
+    const uint32_t groups = (cnt + kGroup - 1u) / kGroup; // <= 64
+    const GlobalKeys kf{sc_val.key[0] + (size_t)row * sc_val.vpad};
+    const GroupTable& T = sc_val.gt;
+    const size_t t_at = (size_t)row * sc_val.g_cap + p * (kSliceMax / kGroup);
+    float q[4][4];
+    uint32_t len[4];
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t g = wave + k * (uint32_t)kWaves;
+        len[k] = g < groups ? min(kGroup, cnt - g * kGroup) : 0u; // uniform per wave
+        load_span(kf, off + min(g, groups - 1u) * kGroup, len[k], q[k]);
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k) {
+        const double s = __ockl_wfred_add_f64((((double)q[k][0] + (double)q[k][1]) + (double)q[k][2]) + (double)q[k][3]);
+        if (lane == 0)
+            s_gs[wave + k * (uint32_t)kWaves] = len[k] ? s : 0.0;
+    }
+    __syncthreads();
+    // the sums before and behind each group: lane g holds group g's
+    const double v = s_gs[lane];
+    const double upto = __ockl_wfscan_add_f64(v, true);
+    const double before_l = mass + (upto - v), after_l = mass + upto;
+    const double r0_raw = (double)u_row * total64, r0 = r0_raw == r0_raw ? r0_raw : 0.0;
+#pragma unroll
+    for (uint32_t k = 0; k < 4; ++k) {
+        const uint32_t g = uniform_u32(wave + k * (uint32_t)kWaves);
+        if (g >= groups) // uniform per wave
+            break;
+        const double guess = readlane_f64(before_l, g), at_end = readlane_f64(after_l, g);
+        const int eg = guess > 0 ? exponent_of((float)guess) : 0;
+        const seqfp::Step32 st = span_map<true>(q[k], len[k], eg);
+        // the sum is expected to change binade inside the group (or starts at zero): records for its quarters
+        const bool split4 = uniform_u32((uint32_t)(eg == 0 || exponent_of((float)at_end) != eg)) != 0;
+        if (split4)
+            build_quarters(q[k], len[k], guess, T.quarters + (t_at + g) * 4u);
+        // the walk's map, where the walk is expected to pass the group without changing binade in it
+        const double r_here = r0 - guess, r_after = r0 - at_end;
+        const int ew = (r0 > 0.0 && r_after > 0.0) ? exponent_of((float)r_here) : 0;
+        uint4 wrec = make_uint4(0u, 0u, 0u, 0u);
+        if (ew > 0 && uniform_u32((uint32_t)(exponent_of((float)r_after) == ew)) != 0) {
+            const seqfp::Step32 sw = span_map<true>(q[k], len[k], ew);
+            const float q_top = __uint_as_float(__ockl_wfred_max_u32(max(max(__float_as_uint(q[k][0]), __float_as_uint(q[k][1])),
+                                                                         max(__float_as_uint(q[k][2]), __float_as_uint(q[k][3])))));
+            wrec = make_uint4(sw.d0, sw.d1, walk_need(q_top, ew, sw.cmax), (uint32_t)ew);
+        }
+        if (lane == 0) {
+            T.sum[t_at + g] = s_gs[g];
+            T.d0[t_at + g] = st.d0;
+            T.d1[t_at + g] = st.d1;
+            T.cmax[t_at + g] = st.cmax;
+            T.start[t_at + g] = off + g * kGroup;
+            T.pack[t_at + g] = len[k] | ((uint32_t)eg << 16) | (split4 ? kHasQuarters : 0u);
+            T.walk[t_at + g] = wrec;
+        }
+    }
 }
 
 // grid = (1, rows).

@@ -17,14 +17,13 @@ void launch_index_weights(int kh, hipStream_t st, const mako_sample_desc& d, con
 
 void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratch& sc)
 {
-    hipLaunchKernelGGL(index_groups_kernel, dim3((d.n_vocab + kIndexBlock - 1u) / kIndexBlock, d.n_rows), dim3(kThreads), kDynLds, st, d, sc);
+    hipLaunchKernelGGL(index_groups_kernel, dim3((d.n_vocab + kSliceMax - 1u) / kSliceMax, d.n_rows), dim3(kThreads), 0, st, d, sc);
     hipLaunchKernelGGL(index_tail_kernel, dim3(1, d.n_rows), dim3(kThreads), kTailLds, st, d, sc);
 }
 
 hipError_t init_index_kernels()
 {
-    const void* kernels[] = {(const void*)index_weights_kernel<0>, (const void*)index_weights_kernel<2>, (const void*)index_weights_kernel<8>,
-                             (const void*)index_groups_kernel};
+    const void* kernels[] = {(const void*)index_weights_kernel<0>, (const void*)index_weights_kernel<2>, (const void*)index_weights_kernel<8>};
     for (const void* k : kernels) {
         const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLds);
         if (e != hipSuccess)

@@ -407,20 +407,26 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     // the caller's copy of the parameters, they get the kernels of index_rows.h instead of a workgroup each on the
     // whole-row path, unless the batch is one those kernels do not serve: verification, forced tokens, rows that are
     // not aligned for 128-bit loads, a vocabulary beyond 262 144)
-    bool any_nucleus = true, any_late = true, any_index = false;
+    bool any_nucleus = true, any_late = true, any_index = false, only_index = false;
     uint32_t nucleus_rows = d.n_rows;
     if (params_host) {
         any_nucleus = any_late = false;
-        uint32_t n_nucleus = 0;
+        uint32_t n_nucleus = 0, n_index = 0;
         const bool index_served = vec && !d.draft && !d.force_token && !d.close_token && d.n_vocab <= mako::kIndexMaxVocab;
         for (uint32_t r = 0; r < d.n_rows; ++r) {
             const mako::RowClass c = mako::classify(params_host[r]);
+            const bool index_row = index_served && mako::index_order_row(params_host[r]);
             any_nucleus |= c == mako::kNucleus;
-            any_late |= c == mako::kGeneral;
-            any_index |= index_served && mako::index_order_row(params_host[r]);
+            any_late |= c == mako::kGeneral && !index_row;
+            n_index += index_row;
             n_nucleus += c == mako::kNucleus;
         }
         nucleus_rows = std::max(n_nucleus, 1u);
+        any_index = n_index != 0;
+        only_index = n_index == d.n_rows;
+        // (rows of other kinds beside them are finished in tail_kernel's launch, which leaves alone what the index
+        // kernels have claimed; plan_kernel would not)
+        any_late |= any_index && !only_index;
     }
     const bool launch_sort = any_nucleus || any_late;
     // (finish_kernel's grid: scan_kernel, which cuts the second pass up, is told of it)
@@ -451,7 +457,7 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
         MAKO_LAUNCH(mako::launch_index_weights(kh, st, d, sc, slices));
     if (any_nucleus)
         MAKO_LAUNCH(mako::launch_finish(vec, kh, unsorted, finish_wgs, st, d, sc, slices));
-    if (!launch_sort)
+    if (!launch_sort && !only_index)
         MAKO_LAUNCH(mako::launch_plan_alone(st, d, sc, slices));
     MAKO_MARK(2);
     if (any_nucleus)

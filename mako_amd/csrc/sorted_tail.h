@@ -411,9 +411,9 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
             uint32_t slot = 0;
             if (crossing[u]) {
                 if (lane_id() == 0)
-                    slot = atomicAdd(&G.misc()[UNSORTED ? qs.counter : 3u], 1u) + 1u;
+                    slot = atomicAdd(&G.misc()[(UNSORTED || UNORDERED) ? qs.counter : 3u], 1u) + 1u;
                 slot = uniform_u32(slot);
-                if constexpr (UNSORTED)
+                if constexpr (UNSORTED || UNORDERED) // (the instances whose walk builds its maps a block ahead)
                     slot = slot > qs.slots ? kQuarterSlots + 1u : slot + qs.first;
                 if (slot > kQuarterSlots)
                     slot = 0;
@@ -1056,11 +1056,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     const uint32_t groups1 = PLANNED ? t_groups : (n1 + kGroup - 1) / kGroup;
     // (UNSORTED: the running sum and the walk's first block of groups share the first half of the quarter-record slots;
     // the other half is for the maps of the walk's second block, built while the first is walked)
-    constexpr uint32_t kFirstSlots = UNSORTED ? kQuarterSlots / 2u : kQuarterSlots;
+    constexpr bool kAhead = UNSORTED || UNORDERED; // (the instances for lists of hundreds of groups)
+    constexpr uint32_t kFirstSlots = kAhead ? kQuarterSlots / 2u : kQuarterSlots;
     if (tid == 0) {
         G.misc()[3] = 0;
-        if (UNSORTED) {
+        if (kAhead)
             G.misc()[4] = 0;
+        if (UNSORTED) {
             sm.ticket = 0; // set: a record of an unsorted share where the code below needs the list itself
             sm.flag = 0;   // set: the list has such records
         }
@@ -1355,8 +1357,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     if (wave_id() != 0 && r0_guess == r0_guess && !head_walk) {
         // (all the other waves: with more than kHeadGroups maps to build they take longer than the chain, even
         // though three of them share its SIMD)
-        if constexpr (UNSORTED)
-            build_group_maps<UNSORTED>(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u, 0u,
+        if constexpr (kAhead)
+            build_group_maps<UNSORTED, UNORDERED>(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u, 0u,
                                        QuarterSlots{3u, 0u, kFirstSlots});
         else
             build_group_maps<false, UNORDERED>(kf, min(reach, (uint32_t)kWave), true, r0_guess, G, (uint32_t)wave_id() - 1u, (uint32_t)kWaves - 1u);
@@ -1483,13 +1485,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         // that guess is worthless (every group would then go entry by entry: 140 us for a 245-group list at
         // u = 0.999), so every later block's maps are built, by all the waves, when the walk gets there, from the
         // exact r at the block's first group.
-        // (UNSORTED, the instance for lists of hundreds of groups: the maps of the NEXT block are built by the other
+        // (UNSORTED and UNORDERED, the instances for lists of hundreds of groups: the maps of the NEXT block are built by the other
         // waves while wave 0 walks this one, from the exact r at this block's first group less the fp64 sums up to the
         // group, which is as good a guess as the exact r at the next block's first group unless the walk is about to
         // end; then nothing is built, so that a walk that has ended does not wait for maps nobody needs.  The two
         // blocks' quarter records take the halves of the slots in turn.)
         for (uint32_t base = 0; base < groups; base += kWave) {
-            if constexpr (!UNSORTED) {
+            if constexpr (!kAhead) {
                 if (base > 0) {
                     if (wave_id() == 0 && lane_id() == 0) {
                         G.misc()[0] = M;
@@ -1529,7 +1531,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 const uint32_t next = base + (uint32_t)kWave;
                 if (wave_id() != 0 && next < groups && r_here - (G.pg()[next] - G.pg()[base]) > r_here * -0x1p-6) { // uniform
                     const uint32_t half = ((next / (uint32_t)kWave) & 1u);
-                    build_group_maps<UNSORTED>(kf, min(groups, next + (uint32_t)kWave), true, r_here + G.pg()[base], G, (uint32_t)wave_id() - 1u,
+                    build_group_maps<UNSORTED, UNORDERED>(kf, min(groups, next + (uint32_t)kWave), true, r_here + G.pg()[base], G, (uint32_t)wave_id() - 1u,
                                                (uint32_t)kWaves - 1u, next, QuarterSlots{3u + half, half * (kQuarterSlots / 2u), kQuarterSlots / 2u});
                 }
             }
