@@ -135,7 +135,11 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
 /* The same call for a caller that still has the batch's parameters in HOST memory (the SamplingParams originate
  * there, src/gen/session.hpp:19-21): params_host[n_rows] must hold the same values as desc->params.  The call
  * looks at them on the calling thread and leaves out the kernels that no row of the batch needs (a batch without
- * top_k == 0 rows takes two launches instead of four).  The results never depend on it; null = the call above. */
+ * top_k == 0 rows takes two launches instead of four).  Rows that are cut neither to a top-k nor to a nucleus
+ * (temperature only: top_k == 0, top_p >= 1), whose candidates stay in token order, get three launches of their own
+ * instead of one workgroup each for the whole row (not when verifying, with force_token / close_token, with rows that
+ * are not 16-byte aligned multiples of four logits, or beyond 262 144 logits).  The results never depend on it;
+ * null = the call above. */
 int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_desc* desc,
                                      const mako_sampling_params* params_host, void* stream);
 

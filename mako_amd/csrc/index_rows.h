@@ -55,6 +55,7 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
+    MAKO_CHECK(sc, kCheckStage, (uint64_t)hi <= sc.vpad);
     uint32_t cnt = 0, last = 0;
     double bsum[4];
 #pragma unroll
@@ -160,6 +161,7 @@ __global__ __launch_bounds__(kThreads) void index_groups_kernel(mako_sample_desc
     const GlobalKeys kf{sc_val.key[0] + (size_t)row * sc_val.vpad};
     const GroupTable& T = sc_val.gt;
     const size_t t_at = (size_t)row * sc_val.g_cap + p * (kSliceMax / kGroup);
+    MAKO_CHECK(sc_val, kCheckGroups, p * (kSliceMax / kGroup) + groups <= sc_val.g_cap && (uint64_t)off + cnt <= sc_val.vpad);
     float q[4][4];
     uint32_t len[4];
 #pragma unroll

@@ -562,7 +562,8 @@ int mako_sampler_sample_host(mako_sampler_ctx* ctx, const float* logits, int64_t
         d.out_accepted = ctx->st_acc;
     }
     d.out_tokens = ctx->st_tokens;
-    const int rc = mako_sampler_sample_batch(ctx, &d, nullptr);
+    // (the caller's parameters are in host memory: the call looks at them and leaves out what no row needs)
+    const int rc = mako_sampler_sample_batch_hinted(ctx, &d, params, nullptr);
     if (rc != MAKO_OK)
         return rc;
     MAKO_HIP(ctx, hipMemcpy(out_tokens, ctx->st_tokens, n_rows * 4, hipMemcpyDeviceToHost));

@@ -31,6 +31,20 @@ def _mixed_paths(rows, vocab, seed):
     return w
 
 
+def test_no_index_check_fails_on_rows_in_token_order(gpu_ctx, checked_ctx):
+    """Temperature-only rows beside the others, with the host copy of the parameters: the kernels of index_rows.h."""
+    w = _mixed_paths(24, workloads.V_DEEPSEEK, 9108)
+    w["params"]["top_k"][4::3] = 0
+    w["params"]["top_p"][4::3] = 1.0
+    checked_ctx.failed_checks()
+    got = gpu_rows(checked_ctx, w, cap=0, hinted=True)
+    bits = checked_ctx.failed_checks()
+    assert bits == 1 << 31, "index checks failed: bit set 0x%x" % bits
+    ref = gpu_rows(gpu_ctx, w, cap=0, hinted=True)
+    assert np.array_equal(got["tokens"], ref["tokens"]) and np.array_equal(got["n_cand"], ref["n_cand"])
+    assert (got["path"][4::3] == api.PATH_INDEXED).all()
+
+
 @pytest.mark.parametrize("name", ["config3", "config4", "config5", "mixed"])
 def test_no_index_check_fails(gpu_ctx, checked_ctx, name):
     if name == "config3":
