@@ -3,7 +3,8 @@
 // the caller's host copy of the parameters the library knows that a batch has such rows and gives them three launches
 // of their own instead of one workgroup per row on the whole-row path:
 //   index_weights_kernel  a workgroup per 16 384 logits: masks and penalties as everywhere, q = expf((w - m) / T), and
-//                         ~bits(q) (0.0f for a logit that is no candidate) stored at the token's own position;
+//                         ~bits(q) (0.0f for a logit that is no candidate) stored at the token's own position (entry i
+//                         of the list is token i: no array of token ids);
 //   index_groups_kernel   a workgroup per 16 384 entries: the group records of its 64 groups of 256 (fp64 sums, the maps
 //                         of the running fp32 sum and of the walk for the binades guessed from the sums before them),
 //                         as sort_kernel's workers leave them for a sorted list;
@@ -54,7 +55,6 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
-    uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
     MAKO_CHECK(sc, kCheckStage, (uint64_t)hi <= sc.vpad);
     uint32_t cnt = 0, last = 0;
     double bsum[4];
@@ -75,14 +75,11 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
             }
             if (base + 3u < hi) {
                 *reinterpret_cast<uint4*>(key0 + base) = make_uint4(~k[0], ~k[1], ~k[2], ~k[3]);
-                *reinterpret_cast<uint4*>(idx0 + base) = make_uint4(base, base + 1u, base + 2u, base + 3u);
             } else {
 #pragma unroll
                 for (uint32_t c = 0; c < 4; ++c)
-                    if (base + c < hi) {
+                    if (base + c < hi)
                         key0[base + c] = ~k[c];
-                        idx0[base + c] = base + c;
-                    }
             }
         }
         // (four weights at a time: with all sixteen in flight the kernel needs twice the registers, and two workgroups
@@ -245,8 +242,8 @@ __global__ __launch_bounds__(kThreads) void index_tail_kernel(mako_sample_desc d
     }
     if (flag == kIndexReady) {
         const uint32_t* kf = sc.key[0] + (size_t)row * sc.vpad;
-        const uint32_t* jf = sc.idx[0] + (size_t)row * sc.vpad;
-        if (sorted_tail<true, false, false, false, true>(d, row, s_args.P, kf, jf, n0, true, total64, MAKO_PATH_INDEXED, L, false, 0.0f,
+        // (entry i of the list is token i: no array of token ids)
+        if (sorted_tail<true, false, false, false, true>(d, row, s_args.P, kf, nullptr, n0, true, total64, MAKO_PATH_INDEXED, L, false, 0.0f,
                                                          sc.gt, (size_t)row * sc.g_cap, groups)) {
             // (the list's length counts the gaps; the candidates are what the reference counts)
             if (tid == 0 && d.out_n_cand)

@@ -908,7 +908,13 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     FinishShared& sm = *L.sm;
     const uint32_t tid = threadIdx.x;
     auto qat = [=](uint32_t i) { return __uint_as_float(~kf[i]); };
-    auto idat = [=](uint32_t i) { return jf[i]; };
+    // (UNORDERED: a list in token order, whose entry i is token i: jf is not read)
+    auto idat = [=](uint32_t i) {
+        if constexpr (UNORDERED)
+            return i;
+        else
+            return jf[i];
+    };
     const GroupLds G = group_lds(L);
     const bool topp_active = P.top_p < 1.0f;
     constexpr uint32_t kEpochBits = UNSORTED ? 0xffu : ~0u; // (of a pack's upper half)
