@@ -2,7 +2,7 @@
 """Headline benchmark: sampled rows/s of the HIP sampler on the decode batch B=64 x V=129280 fp32
 (penalties over 2048-token histories, per-row temperature / top-k / top-p), one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config4|config5|config1|config2b|config1_topk_alone|topk_alone_64|temperature_only_64|temperature_only_256]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config3|config4|config5|config1|config2b|config1_topk_alone|topk_alone_64|temperature_only_1|temperature_only_64|temperature_only_256]
 
 A step is one batch through the whole sampling pipeline with every input already resident in HBM.
 The logits are rotated through a pool of copies larger than the 256 MB Infinity Cache so each step
@@ -53,7 +53,7 @@ def make_workload(name):
         w["params"]["top_p"] = np.float32(1.0)
         w["name"] = name
         return w
-    if name in ("temperature_only_64", "temperature_only_256"):  # rows with neither top-k nor top-p: the whole vocabulary in token order
+    if name in ("temperature_only_1", "temperature_only_64", "temperature_only_256"):  # rows with neither top-k nor top-p: the whole vocabulary in token order
         w = workloads.config1(rows=int(name.rsplit("_", 1)[1]))
         w["params"]["top_p"] = np.float32(1.0)
         w["params"]["top_k"] = np.uint32(0)

@@ -21,9 +21,11 @@
 
 namespace mako {
 
+constexpr uint32_t kIndexBlock = 4096;                   // entries whose fp64 sum index_weights_kernel leaves as one number
 constexpr uint32_t kIndexMaxVocab = kMaxGroups * kGroup; // the group records of a row
-static_assert(kIndexMaxVocab / kSliceMax <= kWorkers && kIndexMaxVocab / kSliceMax <= kMaxSlices && kSliceMax == (uint32_t)kWave * kGroup,
-              "a piece's count, last candidate and sum travel in the plan's per-worker words and the row's part_sum; a lane per group");
+static_assert(kIndexMaxVocab / kSliceMax <= kWorkers && kIndexMaxVocab / kIndexBlock <= kMaxSlices && kIndexMaxVocab / kIndexBlock <= (uint32_t)kWave &&
+                  kSliceMax == 4u * kIndexBlock && kIndexBlock == (uint32_t)kWaves * kGroup,
+              "a piece's count and last candidate travel in the plan's per-worker words, the blocks' sums in the row's part_sum, a lane each");
 #ifdef MAKO_EMIT_INDEX_KERNELS
 // grid = (ceil(V / 16384), rows); rows of other kinds leave at once.  V % 4 == 0 and aligned rows (the host checks).
 template <int KH>
@@ -61,8 +63,8 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
 #pragma unroll
     for (uint32_t b = 0; b < 4; ++b) {
         bsum[b] = 0.0;
-        const uint32_t base = lo + b * 4096u + tid * 4u;
-        if (lo + b * 4096u < hi) { // uniform
+        const uint32_t base = lo + b * kIndexBlock + tid * 4u;
+        if (lo + b * kIndexBlock < hi) { // uniform
             uint32_t k[4];
 #pragma unroll
             for (uint32_t c = 0; c < 4; ++c) {
@@ -88,32 +90,37 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
     }
     // the piece's fp64 sum (an estimate for the binades only: any order of addition will do), its candidates and its
     // last one
-    double* wsum = reinterpret_cast<double*>(s_dyn64); // [kWaves] (the penalty table is done with)
-    uint32_t* wcnt = reinterpret_cast<uint32_t*>(wsum + kWaves);
+    double* wsum = reinterpret_cast<double*>(s_dyn64); // [4][kWaves] (the penalty table is done with)
+    uint32_t* wcnt = reinterpret_cast<uint32_t*>(wsum + 4 * kWaves);
     __syncthreads();
-    {
-        const double s = __ockl_wfred_add_f64((bsum[0] + bsum[1]) + (bsum[2] + bsum[3]));
-        cnt = __ockl_wfred_add_u32(cnt);
-        last = __ockl_wfred_max_u32(last);
-        if (lane_id() == 0) {
-            wsum[wave_id()] = s;
-            wcnt[wave_id()] = cnt;
-            wcnt[kWaves + wave_id()] = last;
-        }
+#pragma unroll
+    for (uint32_t b = 0; b < 4; ++b) {
+        const double s = __ockl_wfred_add_f64(bsum[b]);
+        if (lane_id() == 0)
+            wsum[b * kWaves + wave_id()] = s;
+    }
+    cnt = __ockl_wfred_add_u32(cnt);
+    last = __ockl_wfred_max_u32(last);
+    if (lane_id() == 0) {
+        wcnt[wave_id()] = cnt;
+        wcnt[kWaves + wave_id()] = last;
     }
     __syncthreads();
-    double sum = 0.0;
+    if (tid < 4u && lo + tid * kIndexBlock < hi) { // (a sum per 4 096 entries: index_groups_kernel's workgroups may be that small)
+        double s = 0.0;
+        for (int w = 0; w < kWaves; ++w)
+            s += wsum[tid * kWaves + w];
+        sc.part_sum[(size_t)row * kMaxSlices + piece * 4u + tid] = s;
+    }
     if (tid == 0) {
         cnt = last = 0;
         for (int w = 0; w < kWaves; ++w) {
-            sum += wsum[w];
             cnt += wcnt[w];
             last = max(last, wcnt[kWaves + w]);
         }
     }
     if (tid == 0) {
         BigPlan* plan = sc.plan + row;
-        sc.part_sum[(size_t)row * kMaxSlices + piece] = sum;
         plan->cursor[piece] = cnt; // (the pieces' counts and last candidates travel in the plan's per-worker words)
         plan->key_lo[piece] = last;
         if (piece == 0) {
@@ -124,25 +131,28 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
     }
 }
 
-// grid = (ceil(V / 16384), rows): workgroup p leaves the records of the groups of entries [16384 p, 16384 (p + 1)).
-// Wave w takes the groups w, w + 16, w + 32 and w + 48 of those: their entries in one trip to memory, their fp64 sums to
-// LDS, and once every wave has the sums before each group, the maps from the entries it still holds.
+// grid = (ceil(V / (4096 GPW)), rows): workgroup p leaves the records of the groups of its 4096 GPW entries.  Wave w
+// takes the groups w, w + 16, ... (GPW of them): their entries in one trip to memory, their fp64 sums to LDS, and once
+// every wave has the sums before each group, the maps from the entries it still holds.  (GPW = 4 where there are rows
+// enough to fill the chip, 1 on a small batch, which waits for one workgroup's chain of dependent steps.)
+template <uint32_t GPW>
 __global__ __launch_bounds__(kThreads) void index_groups_kernel(mako_sample_desc d_arg, Scratch sc_val)
 {
     __shared__ double s_gs[kWave];
+    constexpr uint32_t kSpan = kIndexBlock * GPW; // entries per workgroup
     const uint32_t row = blockIdx.y, p = blockIdx.x, tid = threadIdx.x, lane = lane_id(), wave = wave_id();
     const mako_sampling_params P0 = d_arg.params[row];
     if (!index_order_row(P0)) // uniform
         return;
     BigPlan* plan = sc_val.plan + row;
-    const uint32_t pieces = (d_arg.n_vocab + kSliceMax - 1u) / kSliceMax;
+    const uint32_t pieces = (d_arg.n_vocab + kSliceMax - 1u) / kSliceMax, blocks = (d_arg.n_vocab + kIndexBlock - 1u) / kIndexBlock;
     const uint32_t cnt_l = lane < pieces ? plan->cursor[min(lane, kWorkers - 1u)] : 0u;
     const uint32_t last_l = lane < pieces ? plan->key_lo[min(lane, kWorkers - 1u)] : 0u;
-    const double ps = lane < pieces ? sc_val.part_sum[(size_t)row * kMaxSlices + lane] : 0.0;
+    const double ps = lane < blocks ? sc_val.part_sum[(size_t)row * kMaxSlices + lane] : 0.0;
     const float u_row = d_arg.u[row];
     const uint32_t n_cand = __ockl_wfred_add_u32(cnt_l), n_list = __ockl_wfred_max_u32(last_l);
     const double incl = __ockl_wfscan_add_f64(ps, true);
-    const double total64 = readlane_f64(incl, kWave - 1), mass = readlane_f64(incl - ps, p);
+    const double total64 = readlane_f64(incl, kWave - 1), mass = readlane_f64(incl - ps, p * GPW);
     if (p == 0 && tid == 0) {
         plan->n0 = n_list;
         plan->groups = (n_list + kGroup - 1u) / kGroup;
@@ -151,24 +161,28 @@ __global__ __launch_bounds__(kThreads) void index_groups_kernel(mako_sample_desc
         const bool gaps_matter = n_cand < n_list && d_arg.out_cand_idx && d_arg.out_cand_q && d_arg.cand_cap;
         plan->flag = n_cand == 0u ? kIndexEmpty : (gaps_matter ? kIndexWhole : kIndexReady);
     }
-    if (n_cand == 0u || p * kSliceMax >= n_list) // uniform
+    if (n_cand == 0u || p * kSpan >= n_list) // uniform
         return;
-    const uint32_t off = p * kSliceMax, cnt = min(kSliceMax, n_list - off);
-    const uint32_t groups = (cnt + kGroup - 1u) / kGroup; // <= 64
+    const uint32_t off = p * kSpan, cnt = min(kSpan, n_list - off);
+    const uint32_t groups = (cnt + kGroup - 1u) / kGroup; // <= 16 GPW <= 64
     const GlobalKeys kf{sc_val.key[0] + (size_t)row * sc_val.vpad};
     const GroupTable& T = sc_val.gt;
-    const size_t t_at = (size_t)row * sc_val.g_cap + p * (kSliceMax / kGroup);
-    MAKO_CHECK(sc_val, kCheckGroups, p * (kSliceMax / kGroup) + groups <= sc_val.g_cap && (uint64_t)off + cnt <= sc_val.vpad);
-    float q[4][4];
-    uint32_t len[4];
+    const size_t t_at = (size_t)row * sc_val.g_cap + p * (kSpan / kGroup);
+    MAKO_CHECK(sc_val, kCheckGroups, p * (kSpan / kGroup) + groups <= sc_val.g_cap && (uint64_t)off + cnt <= sc_val.vpad);
+    float q[GPW][4];
+    uint32_t len[GPW];
 #pragma unroll
-    for (uint32_t k = 0; k < 4; ++k) {
+    for (uint32_t k = 0; k < GPW; ++k) {
         const uint32_t g = wave + k * (uint32_t)kWaves;
         len[k] = g < groups ? min(kGroup, cnt - g * kGroup) : 0u; // uniform per wave
         load_span(kf, off + min(g, groups - 1u) * kGroup, len[k], q[k]);
     }
+    if (GPW < 4u && tid < (uint32_t)kWave)
+        s_gs[tid] = 0.0;
+    if (GPW < 4u)
+        __syncthreads();
 #pragma unroll
-    for (uint32_t k = 0; k < 4; ++k) {
+    for (uint32_t k = 0; k < GPW; ++k) {
         const double s = __ockl_wfred_add_f64((((double)q[k][0] + (double)q[k][1]) + (double)q[k][2]) + (double)q[k][3]);
         if (lane == 0)
             s_gs[wave + k * (uint32_t)kWaves] = len[k] ? s : 0.0;
@@ -180,7 +194,7 @@ __global__ __launch_bounds__(kThreads) void index_groups_kernel(mako_sample_desc
     const double before_l = mass + (upto - v), after_l = mass + upto;
     const double r0_raw = (double)u_row * total64, r0 = r0_raw == r0_raw ? r0_raw : 0.0;
 #pragma unroll
-    for (uint32_t k = 0; k < 4; ++k) {
+    for (uint32_t k = 0; k < GPW; ++k) {
         const uint32_t g = uniform_u32(wave + k * (uint32_t)kWaves);
         if (g >= groups) // uniform per wave
             break;
@@ -228,6 +242,7 @@ __global__ __launch_bounds__(kThreads) void index_tail_kernel(mako_sample_desc d
     const double total64 = planned->total64;
     const float m = planned->m;
     const uint32_t argidx = planned->argidx;
+    MAKO_ROW(row);
     stage_args(d_arg, sc_val, row, s_args); // (with a barrier: the plan has been read)
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
