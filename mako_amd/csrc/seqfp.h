@@ -19,6 +19,7 @@
 // share one implementation.
 #pragma once
 
+#include <math.h>
 #include <stdint.h>
 #include <string.h>
 
@@ -263,6 +264,27 @@ SEQFP_HD Step32 step32_flat(float q, int e)
     if (d > 25) // (the weight is below half a unit of the epoch's last place)
         ce = co = 0u;
     if (d < 0) // (a weight from a higher binade cannot be expressed)
+        ce = co = kSat;
+    return Step32{ce, co, ce > co ? ce : co};
+}
+
+// The same map taken from the adder itself: in the epoch with exponent e the states 2^23 (even) and 2^23 + 1 (odd) are
+// the floats R0 and R1, and for a weight below 2^23 units R + q stays inside the binade, so (R + q) - R is, exactly, the
+// increment that round-to-nearest-even gives a state of R's parity: two additions, two subtractions and two exact
+// scalings instead of the integer arithmetic above.  A weight of 2^23 units or more gets the "unusable" mark (its
+// map could never be applied to a state of a binade of 2^23 states; in the subnormal binade, whose states start at
+// zero, that gives up maps step32_flat() would allow, which costs a replay and nothing else).  Compiled without
+// contraction or reassociation, like every fp32 operation that stands for one of the reference's.
+SEQFP_HD Step32 step32_fp(float q, int e)
+{
+    const float R0 = u2f(uint32_t(e) << 23), R1 = u2f((uint32_t(e) << 23) | 1u);
+    const float t0 = (R0 + q) - R0, t1 = (R1 + q) - R1;
+#if defined(__HIP_DEVICE_COMPILE__)
+    uint32_t ce = (uint32_t)__builtin_ldexpf(t0, 150 - e), co = (uint32_t)__builtin_ldexpf(t1, 150 - e);
+#else
+    uint32_t ce = (uint32_t)ldexpf(t0, 150 - e), co = (uint32_t)ldexpf(t1, 150 - e);
+#endif
+    if (!(q < R0) || e > 253) // (in the last binade R + q may overflow: no maps there, running sums of weights never get near it)
         ce = co = kSat;
     return Step32{ce, co, ce > co ? ce : co};
 }

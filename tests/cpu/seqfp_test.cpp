@@ -247,6 +247,41 @@ int main()
                 printf("step32_flat differs: q bits %08x e %d: %u %u %u vs %u %u %u\n", bits, e, x.d0, x.d1, x.cmax, y.d0, y.d1, y.cmax);
         }
     }
+    // step32_fp() (the map taken from real additions) against step32_flat(): equal wherever the weight is below 2^23
+    // units of the epoch, the "unusable" mark from there on; weights around every tie and around the limits
+    long fp_cases = 0, fp_marked = 0;
+    for (int it = 0; it < 6000000; ++it) {
+        const int e = 1 + int(rng() % 254);
+        uint32_t bits;
+        switch (it % 6) {
+        case 0: bits = uint32_t(rng()) & 0x7fffffffu; break;
+        case 1: { // an exponent close to the epoch's, any significand
+            const int ex = std::max(0, std::min(254, e - 27 + int(rng() % 30)));
+            bits = (uint32_t(ex) << 23) | (uint32_t(rng()) & 0x7fffffu);
+            break;
+        }
+        case 2: { // exact ties and their neighbours at a shift the epoch makes relevant
+            const int ex = std::max(0, std::min(254, e - int(rng() % 26)));
+            const uint32_t low = 1u << (rng() % 23);
+            bits = (uint32_t(ex) << 23) | (((uint32_t(rng()) & 0x7fffffu) & ~(2u * low - 1u)) + low + uint32_t(rng() % 3) - 1u);
+            break;
+        }
+        case 3: bits = uint32_t(rng() % 64); break;                                                  // zero and subnormals
+        case 4: bits = (uint32_t(e) << 23) + uint32_t(rng() % 5) - 2u; break;                         // around 2^23 units
+        default: bits = (uint32_t(std::max(0, e - 24 - int(rng() % 3))) << 23) | (rng() % 2 ? 0u : uint32_t(rng()) & 0x7fffffu); // around half a unit
+        }
+        if (bits >= 0x7f800000u)
+            continue;
+        const float q = seqfp::u2f(bits);
+        const seqfp::Step32 x = seqfp::step32_flat(q, e), y = seqfp::step32_fp(q, e);
+        ++fp_cases;
+        const bool big = !(q < seqfp::u2f(uint32_t(e) << 23)) || e > 253; // (and the last binade, where R + q may overflow)
+        fp_marked += big;
+        const bool same = big ? (y.d0 == seqfp::kSat && y.d1 == seqfp::kSat) : (x.d0 == y.d0 && x.d1 == y.d1 && x.cmax == y.cmax);
+        if (!same && ++fails < 10)
+            printf("step32_fp differs: q bits %08x e %d: %u %u %u vs %u %u %u\n", bits, e, x.d0, x.d1, x.cmax, y.d0, y.d1, y.cmax);
+    }
+    printf("step32_fp: %ld cases (%ld of them at or above 2^23 units)\n", fp_cases, fp_marked);
     for (int it = 0; it < 4000; ++it) {
         const int kind = it % 8;
         size_t n = 1 + rng() % (it % 50 == 0 ? 200000 : 3000);
