@@ -177,12 +177,9 @@ __device__ __forceinline__ seqfp::Step32 span_map(const float (&q)[4], uint32_t 
         bool tie = false;
 #pragma unroll
         for (uint32_t j = 0; j < 4; ++j) {
-            // (UNORDERED, which builds a map for every group of a whole row: the step from the adder itself, half the
-            // instructions; it marks a weight of 2^23 units or more unusable, which such a map would be anyway)
-            if constexpr (UNORDERED)
-                e[j] = lane_id() * 4u + j < len ? step32_fp(q[j], eg) : identity32();
-            else
-                e[j] = lane_id() * 4u + j < len ? step32_flat(q[j], eg) : identity32();
+            // (the step from the adder itself, half the instructions of the integer form; it marks a weight of 2^23 units
+            // or more unusable, which a map that holds one is anyway)
+            e[j] = lane_id() * 4u + j < len ? step32_fp(q[j], eg) : identity32();
             tie |= e[j].d0 != e[j].d1;
         }
         uint32_t cmax;
