@@ -304,7 +304,7 @@ __device__ void opaque_share(const uint32_t* ks, uint32_t cnt, uint32_t off, int
             const float q = __uint_as_float(kv);
             sum += (double)q;
             kmax = max(kmax, kv);
-            const Step32 st = step32_flat(q, e_tot);
+            const Step32 st = step32_fp(q, e_tot); // (the weights of such a share lie binades below the epochs: never the mark)
             const bool tie_t = valid && st.d0 != st.d1;
             acc_t += (valid && !tie_t) ? min(st.d0, 1u << 24) : 0u;
             const unsigned long long bal_t = __ballot(tie_t);
@@ -315,7 +315,7 @@ __device__ void opaque_share(const uint32_t* ks, uint32_t cnt, uint32_t off, int
                 n_t += (uint32_t)__popcll(bal_t);
             }
             if (e_walk > 0) { // uniform
-                const Step32 sw = step32_flat(q, e_walk);
+                const Step32 sw = step32_fp(q, e_walk);
                 const bool tie_w = valid && sw.d0 != sw.d1;
                 acc_w += (valid && !tie_w) ? min(sw.d0, 1u << 24) : 0u;
                 const unsigned long long bal_w = __ballot(tie_w);
@@ -367,7 +367,7 @@ __device__ void opaque_share(const uint32_t* ks, uint32_t cnt, uint32_t off, int
 #pragma unroll
                     for (uint32_t u = 0; u < kTrip; ++u) {
                         const bool valid = base + u * kWave + lane < cnt;
-                        const Step32 st = step32_flat(__uint_as_float(k[u]), e);
+                        const Step32 st = step32_fp(__uint_as_float(k[u]), e);
                         dv[u] = (valid && st.d0 == st.d1) ? min(st.d0, 1u << 24) : 0u;
                         sg[u] = 0u;
                     }
