@@ -13,6 +13,9 @@
 // A logit that is no candidate stays in the list as a weight of 0.0f: adding it changes no sum, and the walk's
 // `r < q` is never true for it.  The list ends behind the row's last candidate, which is where the reference's walk
 // ends when it runs off its list.
+// The other rows of the whole-row class (top-k without top-p, top-k beyond the candidate lists) only get their weights
+// here (index_weights_kernel, into the array general_row_from_weights() starts from) and one workgroup each in
+// index_tail_kernel's launch for the rest of the whole-row path.
 #pragma once
 
 #include "sorted_tail.h"
@@ -36,8 +39,12 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
     __shared__ ArgsLds s_args;
     const uint32_t row = blockIdx.y, piece = blockIdx.x, tid = threadIdx.x;
     const mako_sampling_params P0 = d_arg.params[row];
-    if (!index_order_row(P0)) // uniform
+    if (classify(P0) != kGeneral) // uniform
         return;
+    // (a row that is cut to a top-k without a top-p, or to a top-k beyond the candidate lists, is still finished by one
+    // workgroup on the whole-row path, in index_tail_kernel's launch; its weights, a third of that path's time, are left
+    // here where general_row_from_weights() expects them)
+    const bool in_order = index_order_row(P0);
     stage_args_only(d_arg, sc_val, s_args);
     stage_params(P0, s_args);
     if (tid < 32)
@@ -56,7 +63,9 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
     load_penalised<true, KH>(d, row, lo, hi, kSliceMax, P, hl, pen, reinterpret_cast<uint32_t*>(s_dyn64), wv);
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
-    uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
+    // (~bits(q) into the row's list, or bits(q) into the whole-row path's array)
+    uint32_t* key0 = in_order ? sc.key[0] + (size_t)row * sc.vpad : reinterpret_cast<uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
+    const uint32_t flip = in_order ? ~0u : 0u;
     MAKO_CHECK(sc, kCheckStage, (uint64_t)hi <= sc.vpad);
     uint32_t cnt = 0, last = 0;
     double bsum[4];
@@ -76,12 +85,12 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
                 bsum[b] += ok ? (double)q : 0.0;
             }
             if (base + 3u < hi) {
-                *reinterpret_cast<uint4*>(key0 + base) = make_uint4(~k[0], ~k[1], ~k[2], ~k[3]);
+                *reinterpret_cast<uint4*>(key0 + base) = make_uint4(k[0] ^ flip, k[1] ^ flip, k[2] ^ flip, k[3] ^ flip);
             } else {
 #pragma unroll
                 for (uint32_t c = 0; c < 4; ++c)
                     if (base + c < hi)
-                        key0[base + c] = ~k[c];
+                        key0[base + c] = k[c] ^ flip;
             }
         }
         // (four weights at a time: with all sixteen in flight the kernel needs twice the registers, and two workgroups
@@ -234,8 +243,10 @@ __global__ __launch_bounds__(kThreads) void index_tail_kernel(mako_sample_desc d
     __shared__ FinishShared sm;
     __shared__ ArgsLds s_args;
     const uint32_t row = blockIdx.y, tid = threadIdx.x;
-    if (!index_order_row(d_arg.params[row])) // uniform
+    const mako_sampling_params P0 = d_arg.params[row];
+    if (classify(P0) != kGeneral) // uniform
         return;
+    const bool in_order = index_order_row(P0);
     const BigPlan* planned = sc_val.plan + row;
     const uint32_t flag = planned->flag, n0 = min(planned->n0, d_arg.n_vocab), n_cand = planned->thr;
     const uint32_t groups = min(planned->groups, min(kMaxGroups, sc_val.g_cap));
@@ -248,9 +259,20 @@ __global__ __launch_bounds__(kThreads) void index_tail_kernel(mako_sample_desc d
     const Scratch& sc = s_args.sc;
     if (tid == 0)
         sc.plan[row].flag = 0;
+    const FinishLds L = finish_lds_views(sm, s_dyn64);
+    if (!in_order) {
+        // the whole-row path from the weights index_weights_kernel left (the group records' kernel has not touched the row)
+        if (flag != kIndexClaimed) // (never)
+            return;
+        __syncthreads();
+        if (tid < 32)
+            sm.tab[tid] = k_exp2_tab[tid];
+        __syncthreads();
+        general_row_from_weights<0>(d, sc, row, s_args.P, argidx, L);
+        return;
+    }
     if (flag != kIndexReady && flag != kIndexWhole && flag != kIndexEmpty) // (never)
         return;
-    const FinishLds L = finish_lds_views(sm, s_dyn64);
     if (flag == kIndexEmpty) {
         fallback_row(d, row, argidx);
         return;

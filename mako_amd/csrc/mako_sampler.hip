@@ -415,7 +415,8 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
         const bool index_served = vec && !d.draft && !d.force_token && !d.close_token && d.n_vocab <= mako::kIndexMaxVocab;
         for (uint32_t r = 0; r < d.n_rows; ++r) {
             const mako::RowClass c = mako::classify(params_host[r]);
-            const bool index_row = index_served && mako::index_order_row(params_host[r]);
+            // (with them every other row of the whole-row class, whose weights the first of those kernels leaves too)
+            const bool index_row = index_served && c == mako::kGeneral;
             any_nucleus |= c == mako::kNucleus;
             any_late |= c == mako::kGeneral && !index_row;
             n_index += index_row;

@@ -622,4 +622,78 @@ __device__ MAKO_RARE_CALL void general_row(const mako_sample_desc& d, const Scra
     sort_truncate_draw<SITE == 0>(d, sc, row, P, n0, false, 0.0, MAKO_PATH_GENERAL, L);
 }
 
+// The whole-row path for a row whose weights are already in place: sc.wbuf of the row holds bits(q) of every candidate at
+// its index and 0 elsewhere, as general_row()'s first sweep leaves it (index_weights_kernel writes the same array with a
+// workgroup per 16 384 logits instead of one for the row).  Counts and compacts the candidates in index order and goes
+// on like general_row().  All threads call; `argidx`: the row's first maximum, for a row without candidates.
+template <int SITE>
+__device__ MAKO_RARE_CALL void general_row_from_weights(const mako_sample_desc& d, const Scratch& sc, uint32_t row,
+                                                        const mako_sampling_params& P, uint32_t argidx, const FinishLds& L)
+{
+    assume_lds(L);
+    FinishShared& sm = *L.sm;
+    const uint32_t V = d.n_vocab;
+    const uint32_t* qb = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
+    uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
+    uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
+    const uint32_t lane = lane_id(), wave = wave_id();
+    // (wave w owns the w-th sixteenth of the row, a multiple of 256 logits, lane l entries 4l..4l+3 of each 256)
+    const uint32_t chunk = ((V + kThreads * 4u - 1u) / (kThreads * 4u)) * kGroup;
+    const uint32_t beg = min(V, wave * chunk), end = min(V, beg + chunk);
+    auto four = [&](uint32_t i, uint32_t (&k)[4]) {
+        k[0] = k[1] = k[2] = k[3] = 0u;
+        if (i + 3u < end) {
+            const uint4 x = *reinterpret_cast<const uint4*>(qb + i);
+            k[0] = x.x, k[1] = x.y, k[2] = x.z, k[3] = x.w;
+        } else {
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j)
+                if (i + j < end)
+                    k[j] = qb[i + j];
+        }
+    };
+    uint32_t mine = 0;
+    for (uint32_t base = beg; base < end; base += kGroup) {
+        uint32_t k[4];
+        four(base + lane * 4u, k);
+        mine += (k[0] ? 1u : 0u) + (k[1] ? 1u : 0u) + (k[2] ? 1u : 0u) + (k[3] ? 1u : 0u);
+    }
+    mine = __ockl_wfred_add_u32(mine);
+    __syncthreads();
+    if (lane == 0)
+        sm.bs.u64[wave] = mine;
+    __syncthreads();
+    uint32_t n0 = 0, at = 0;
+    for (int w = 0; w < kWaves; ++w) {
+        const uint32_t x = (uint32_t)sm.bs.u64[w];
+        if (w < (int)wave)
+            at += x;
+        n0 += x;
+    }
+    for (uint32_t base = beg; base < end; base += kGroup) {
+        const uint32_t i = base + lane * 4u;
+        uint32_t k[4];
+        four(i, k);
+        const uint32_t c = (k[0] ? 1u : 0u) + (k[1] ? 1u : 0u) + (k[2] ? 1u : 0u) + (k[3] ? 1u : 0u);
+        const uint32_t incl = __ockl_wfscan_add_u32(c, true);
+        uint32_t pos = at + incl - c;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j)
+            if (k[j]) {
+                MAKO_CHECK(sc, kCheckCompact, pos < n0 && (uint64_t)pos < sc.vpad);
+                key0[pos] = ~k[j];
+                idx0[pos] = i + j;
+                ++pos;
+            }
+        at += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+    }
+    __syncthreads();
+    if (n0 == 0) {
+        fallback_row(d, row, argidx);
+        return;
+    }
+    sort_truncate_draw<SITE == 0>(d, sc, row, P, n0, false, 0.0, MAKO_PATH_GENERAL, L);
+}
+
+
 } // namespace mako

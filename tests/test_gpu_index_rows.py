@@ -135,3 +135,33 @@ def test_no_candidate_survives(gpu_ctx):
     w["logits"][4:6] = np.nan
     g = assert_parity(gpu_ctx, w, cap=16, hinted=True)
     _say("empty rows paths: %s" % _paths(g))
+
+
+def test_other_rows_of_the_whole_row_path_get_their_weights_there_too(gpu_ctx):
+    """Rows cut to a top-k without a top-p (the order nth_element leaves) and to a top-k beyond the candidate lists:
+    with the host copy of the parameters their weights come from the same kernel as the rows' in token order, a
+    workgroup per 16 384 logits, and the whole-row path goes on from there."""
+    rng = np.random.Generator(np.random.PCG64([9, 94]))
+    rows, vocab, hl = 36, 129280, 512
+    w = _plain_batch(rows, vocab, 9, sigmas=(3.0, 1.0), temps=(0.7, 1.1))
+    p = w["params"]
+    p["top_k"][0::3], p["top_p"][0::3] = 40, 1.0
+    p["top_k"][1::3], p["top_p"][1::3] = 700, 0.9
+    p["top_k"][4], p["top_p"][4] = 5000, 1.0
+    p["min_p"][::5] = np.float32(1e-4)
+    p["repetition_penalty"] = 1.1
+    p["frequency_penalty"] = 0.2
+    p["presence_penalty"] = 0.3
+    w["hist"] = workloads.zipf_history(rng, workloads._zipf_cdf(vocab), rows, hl)
+    w["hist_len"] = rng.integers(0, hl + 1, rows).astype(np.uint32)
+    words = (vocab + 31) // 32
+    bits = rng.random((rows, words * 32)) < 0.8
+    bits[::2] = True
+    bits[:, vocab:] = False
+    w["mask"] = np.ascontiguousarray(np.packbits(bits.reshape(rows, words, 32), axis=2, bitorder="little").view(np.uint32).reshape(rows, words))
+    g = assert_parity(gpu_ctx, w, cap=128, hinted=True)
+    _say("whole-row rows with the host copy, paths: %s" % _paths(g))
+    assert (g["path"][0::3] == PATH_GENERAL).all() and (g["path"][1::3] == PATH_GENERAL).all()
+    h = gpu_rows(gpu_ctx, w, cap=128)
+    assert np.array_equal(h["tokens"], g["tokens"]) and np.array_equal(h["total"].view(np.uint32), g["total"].view(np.uint32))
+    assert np.array_equal(h["cand_idx"], g["cand_idx"])
