@@ -15,12 +15,13 @@ void launch_index_weights(int kh, hipStream_t st, const mako_sample_desc& d, con
         hipLaunchKernelGGL(index_weights_kernel<0>, grid, dim3(kThreads), kDynLds, st, d, sc, slices);
 }
 
-void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratch& sc)
+void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, bool in_order_rows)
 {
-    // (a workgroup per 16 384 entries where the rows fill the chip anyway, per 4 096 on a small batch)
-    if ((uint64_t)d.n_rows * ((d.n_vocab + kSliceMax - 1u) / kSliceMax) >= 256u)
+    // (the group records are for rows in token order only: a workgroup per 16 384 entries where the rows fill the chip
+    // anyway, per 4 096 on a small batch)
+    if (in_order_rows && (uint64_t)d.n_rows * ((d.n_vocab + kSliceMax - 1u) / kSliceMax) >= 256u)
         hipLaunchKernelGGL(index_groups_kernel<4u>, dim3((d.n_vocab + kSliceMax - 1u) / kSliceMax, d.n_rows), dim3(kThreads), 0, st, d, sc);
-    else
+    else if (in_order_rows)
         hipLaunchKernelGGL(index_groups_kernel<1u>, dim3((d.n_vocab + kIndexBlock - 1u) / kIndexBlock, d.n_rows), dim3(kThreads), 0, st, d, sc);
     hipLaunchKernelGGL(index_tail_kernel, dim3(1, d.n_rows), dim3(kThreads), kTailLds, st, d, sc);
 }

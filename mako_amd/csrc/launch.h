@@ -38,5 +38,5 @@ void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, u
 // launch, which then leaves such rows alone), the group records, the total and the draw (behind it)
 hipError_t init_index_kernels();
 void launch_index_weights(int kh, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices);
-void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratch& sc);
+void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, bool in_order_rows);
 } // namespace mako

@@ -407,7 +407,7 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     // the caller's copy of the parameters, they get the kernels of index_rows.h instead of a workgroup each on the
     // whole-row path, unless the batch is one those kernels do not serve: verification, forced tokens, rows that are
     // not aligned for 128-bit loads, a vocabulary beyond 262 144)
-    bool any_nucleus = true, any_late = true, any_index = false, only_index = false;
+    bool any_nucleus = true, any_late = true, any_index = false, only_index = false, any_in_order = false;
     uint32_t nucleus_rows = d.n_rows;
     if (params_host) {
         any_nucleus = any_late = false;
@@ -420,6 +420,7 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
             any_nucleus |= c == mako::kNucleus;
             any_late |= c == mako::kGeneral && !index_row;
             n_index += index_row;
+            any_in_order |= index_row && mako::index_order_row(params_host[r]);
             n_nucleus += c == mako::kNucleus;
         }
         nucleus_rows = std::max(n_nucleus, 1u);
@@ -467,7 +468,7 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     if (launch_sort) // (also finishes every row the kernels before it leave: finish_late_row())
         MAKO_LAUNCH(mako::launch_tail(st, d, sc, slices, nucleus_rows, unsorted));
     if (any_index)
-        MAKO_LAUNCH(mako::launch_index_finish(st, d, sc));
+        MAKO_LAUNCH(mako::launch_index_finish(st, d, sc, any_in_order));
     MAKO_MARK(4);
 #undef MAKO_MARK
 #undef MAKO_LAUNCH
