@@ -920,7 +920,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     const GroupLds G = group_lds(L);
     const bool topp_active = P.top_p < 1.0f;
     constexpr uint32_t kEpochBits = UNSORTED ? 0xffu : ~0u; // (of a pack's upper half)
-    if (d.draft || (!PLANNED && n1 > kGroup * kMaxGroups)) {
+    // (UNORDERED: verification takes the running sum's chain below and, only if the draft is rejected, the generic walk)
+    if ((d.draft && !UNORDERED) || (!PLANNED && n1 > kGroup * kMaxGroups)) {
         // verification and oversized lists take the generic windowed replay
         uint32_t n = n1;
         if (topp_active) {
@@ -1310,7 +1311,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     };
 
     MAKO_STAMP(7);
-    if (n <= kSeqMax) {
+    if (n <= kSeqMax && !(UNORDERED && d.draft)) {
         // A nucleus this short is copied to LDS and gone through entry by entry, once for the total and once for the
         // walk (two nanoseconds an entry each way): the group maps below only pay on longer lists.
         if (wave_id() == 0) {
@@ -1456,6 +1457,48 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     const float prod = u_row * span;
     const float r0 = prod + 0.0f;
     __syncthreads();
+
+    if constexpr (UNORDERED) {
+        if (d.draft) {
+            // Verification (src/gen/sampler.cpp:93-106) of a row in token order: entry i is token i, so the draft's weight is
+            // read off the list (0.0f if it is no candidate).  A rejected draft leaves the list for the redraw: as a weight of
+            // 0.0f it can neither stop the walk nor change r; only where the reference's walk would run off its list onto the
+            // last candidate, and that was the draft, the last one before it has to be looked for.
+            const uint32_t dr = (uint32_t)d.draft[row];
+            const float q_draft = dr < n ? qat(dr) : 0.0f;
+            RowOut o;
+            o.n_cand = n;
+            o.total = total;
+            o.path = path_out;
+            o.accepted = r0 < q_draft;
+            o.token = (int32_t)dr;
+            o.q = q_draft;
+            if (!o.accepted) {
+                const float rest = total - q_draft;
+                const float span2 = rest - 0.0f;
+                const float prod2 = d.u2[row] * span2;
+                auto qat2 = [&](uint32_t i) { return i == dr ? 0.0f : qat(i); };
+                uint32_t at = emulate_walk(qat2, n, prod2 + 0.0f, sm);
+                if (at == dr) { // (only as the end of the list: a weight of 0.0f stops nothing)
+                    uint32_t before = 0; // (index + 1 of the last candidate in front of it)
+                    for (uint32_t i = tid; i < dr; i += kThreads)
+                        before = qat(i) > 0.0f ? i + 1u : before;
+                    before = kNone - block_min_u32(kNone - before, sm.bs);
+                    at = before ? before - 1u : dr; // (no other candidate: the draft, src/gen/sampler.cpp:104-105)
+                }
+                o.token = (int32_t)at;
+                o.q = at == dr ? q_draft : qat(at);
+            }
+            if (d.out_cand_idx && d.out_cand_q)
+                for (uint32_t j = tid; j < n && j < d.cand_cap; j += kThreads) {
+                    d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
+                    d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
+                }
+            if (tid == 0)
+                write_row(d, row, o);
+            return true;
+        }
+    }
 
     // exact walk
     uint32_t pos = n - 1;

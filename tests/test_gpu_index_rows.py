@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from mako_amd import api, workloads
-from parity import assert_parity, gpu_rows
+from parity import assert_parity, gpu_rows, oracle_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -165,3 +165,41 @@ def test_other_rows_of_the_whole_row_path_get_their_weights_there_too(gpu_ctx):
     h = gpu_rows(gpu_ctx, w, cap=128)
     assert np.array_equal(h["tokens"], g["tokens"]) and np.array_equal(h["total"].view(np.uint32), g["total"].view(np.uint32))
     assert np.array_equal(h["cand_idx"], g["cand_idx"])
+
+
+def test_verification_of_rows_in_token_order(gpu_ctx):
+    """Sampler::verify (src/gen/sampler.cpp:86-107) on temperature-only rows: the draft's weight read off the list,
+    the total by the chain of group maps, and for a rejected draft the walk over the list without it.  Drafts that
+    are likely and unlikely tokens, no candidates (masked), the row's last candidate, and beyond the vocabulary's
+    candidates; both uniforms from 0 to 1 - 2^-24."""
+    rng = np.random.Generator(np.random.PCG64([10, 95]))
+    rows, vocab = 64, 129280
+    w = _plain_batch(rows, vocab, 10, sigmas=(3.0, 0.3), temps=(0.7, 1.0, 0.4))
+    words = (vocab + 31) // 32
+    bits = np.ones((rows, words * 32), bool)
+    bits[::4] = rng.random((rows // 4, words * 32)) < 0.7
+    bits[:, vocab:] = False
+    bits[5, vocab - 3000:] = False  # (the row's last candidates masked out: the list ends early)
+    w["mask"] = np.ascontiguousarray(np.packbits(bits.reshape(rows, words, 32), axis=2, bitorder="little").view(np.uint32).reshape(rows, words))
+    masked = np.where(bits[:, :vocab], w["logits"], -np.inf)
+    draft = rng.integers(0, vocab, rows).astype(np.int32)
+    draft[0::3] = masked[0::3].argmax(axis=1)           # the most likely token: mostly accepted
+    draft[7] = vocab - 1                                 # the row's last candidate
+    draft[5] = vocab - 10                                # masked out: no candidate
+    draft[9] = np.nonzero(bits[9, :vocab])[0][-1]        # the last candidate of a masked row
+    u2 = workloads._uniforms(rng, rows)
+    w["u"][11], u2[11] = np.float32(1.0 - 2.0**-24), np.float32(1.0 - 2.0**-24)  # rejected, and the redraw runs to the end
+    w["u"][7], u2[7] = np.float32(1.0 - 2.0**-24), np.float32(1.0 - 2.0**-24)
+    w["u"][9], u2[9] = np.float32(1.0 - 2.0**-24), np.float32(1.0 - 2.0**-24)
+    w["u"][13], u2[13] = np.float32(0.0), np.float32(0.0)
+    for cap in (0, 64):
+        g = gpu_rows(gpu_ctx, w, cap=cap, draft=draft, u2=u2, hinted=True)
+        ref = oracle_rows(w, draft=draft, u2=u2)
+        bad = [(r, int(g["tokens"][r]), t, bool(g["accepted"][r]), bool(tr["accepted"])) for r, (t, tr) in enumerate(ref)
+               if g["tokens"][r] != t or bool(g["accepted"][r]) != bool(tr["accepted"])]
+        assert not bad, bad[:8]
+        _say("verification (cap %d): %d accepted, paths %s" % (cap, int(g["accepted"].sum()), _paths(g)))
+        assert (g["path"] == PATH_INDEXED).sum() >= rows // 2
+        h = gpu_rows(gpu_ctx, w, cap=cap, draft=draft, u2=u2)
+        assert np.array_equal(h["tokens"], g["tokens"]) and np.array_equal(h["accepted"], g["accepted"])
+        assert np.array_equal(h["total"].view(np.uint32), g["total"].view(np.uint32))
