@@ -12,7 +12,8 @@
 //                         (sorted_tail's planned instance for lists in any order).
 // A logit that is no candidate stays in the list as a weight of 0.0f: adding it changes no sum, and the walk's
 // `r < q` is never true for it.  The list ends behind the row's last candidate, which is where the reference's walk
-// ends when it runs off its list.
+// ends when it runs off its list.  Verification works on the same list: the draft's weight is entry `draft`, and a
+// rejected draft is redrawn with that entry taken as 0.0f (sorted_tail's UNORDERED instance).
 // The other rows of the whole-row class (top-k without top-p, top-k beyond the candidate lists) only get their weights
 // here (index_weights_kernel, into the array general_row_from_weights() starts from) and one workgroup each in
 // index_tail_kernel's launch for the rest of the whole-row path.
@@ -280,8 +281,12 @@ __global__ __launch_bounds__(kThreads) void index_tail_kernel(mako_sample_desc d
     if (flag == kIndexReady) {
         const uint32_t* kf = sc.key[0] + (size_t)row * sc.vpad;
         // (entry i of the list is token i: no array of token ids)
-        if (sorted_tail<true, false, false, false, true>(d, row, s_args.P, kf, nullptr, n0, true, total64, MAKO_PATH_INDEXED, L, false, 0.0f,
-                                                         sc.gt, (size_t)row * sc.g_cap, groups)) {
+        // (verification has an instance of its own: its code costs the plain one registers)
+        const bool done = d.draft ? sorted_tail<true, false, false, false, true, true>(d, row, s_args.P, kf, nullptr, n0, true, total64, MAKO_PATH_INDEXED,
+                                                                                        L, false, 0.0f, sc.gt, (size_t)row * sc.g_cap, groups)
+                                  : sorted_tail<true, false, false, false, true, false>(d, row, s_args.P, kf, nullptr, n0, true, total64, MAKO_PATH_INDEXED,
+                                                                                         L, false, 0.0f, sc.gt, (size_t)row * sc.g_cap, groups);
+        if (done) {
             // (the list's length counts the gaps; the candidates are what the reference counts)
             if (tid == 0 && d.out_n_cand)
                 d.out_n_cand[row] = n_cand;

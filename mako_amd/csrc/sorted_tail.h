@@ -362,7 +362,8 @@ __device__ __forceinline__ uint32_t walk_need(float q_first, int eg, uint32_t cm
 // g).  The calling wave is number `part` of `parts` that share the work.
 // (UNSORTED: the list may hold records of unsorted shares, see unsorted_shares.h)
 // (UNORDERED: a list in any order; see span_map)
-template <bool UNSORTED = false, bool UNORDERED = false, typename Keys>
+// (LEAVE: G.misc()[5] may name a group that is to be left alone)
+template <bool UNSORTED = false, bool UNORDERED = false, bool LEAVE = false, typename Keys>
 __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0, const GroupLds G,
                                  uint32_t part = wave_id(), uint32_t parts = kWaves, uint32_t g_begin = 0,
                                  const QuarterSlots qs = QuarterSlots{})
@@ -397,6 +398,8 @@ __device__ void build_group_maps(Keys kf, uint32_t groups, bool walk, double r0,
                                    (uniform_u32(o_pack[g]) & kOpaque) != 0u);
             else
                 keep[u] = walk && !crossing[u] && eg[u] > 0 && uniform_u32(o_pack[g] >> 16) == (uint32_t)eg[u];
+            if constexpr (LEAVE) // (the group of a rejected draft during its redraw: it has no map, see sorted_tail)
+                keep[u] = keep[u] || g == uniform_u32(G.misc()[5]);
             len[u] = uniform_u32(G.pack()[g] & kLenMask);
             load_span(kf, uniform_u32(G.start()[g]), keep[u] ? 0u : len[u], q[u]);
         }
@@ -894,7 +897,8 @@ __device__ MAKO_RARE_CALL double reference_total(Get q_at, uint32_t n, FinishSha
 // UNORDERED (with PLANNED, without a top-p): the list is in token order, not sorted (a row that is neither cut to a
 // top-k nor to a nucleus: src/gen/sampler.cpp:79-83 and :64-72 over the candidates as they come); nothing here needs
 // the order except the bounds that stand for "the largest weight of a span", which are then looked for.
-template <bool PLANNED = false, bool SHORT_ONLY = false, bool EXACT = false, bool UNSORTED = false, bool UNORDERED = false>
+// VERIFY (with UNORDERED): the instance for verification (d.draft given); the plain one is then never asked to verify.
+template <bool PLANNED = false, bool SHORT_ONLY = false, bool EXACT = false, bool UNSORTED = false, bool UNORDERED = false, bool VERIFY = false>
 __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_sampling_params& P, const uint32_t* kf_ptr,
                             const uint32_t* jf, uint32_t n1_arg, bool have_total, double total64, uint32_t path,
                             const FinishLds& L, bool need_cut = false, float q_bound = 0.0f, const GroupTable& T = GroupTable{},
@@ -1071,6 +1075,8 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         G.misc()[3] = 0;
         if (kAhead)
             G.misc()[4] = 0;
+        if (UNORDERED && VERIFY)
+            G.misc()[5] = kNone; // (set: the group that is to get no map for the walk)
         if (UNSORTED) {
             sm.ticket = 0; // set: a record of an unsorted share where the code below needs the list itself
             sm.flag = 0;   // set: the list has such records
@@ -1311,7 +1317,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     };
 
     MAKO_STAMP(7);
-    if (n <= kSeqMax && !(UNORDERED && d.draft)) {
+    if (n <= kSeqMax && !(UNORDERED && VERIFY)) {
         // A nucleus this short is copied to LDS and gone through entry by entry, once for the total and once for the
         // walk (two nanoseconds an entry each way): the group maps below only pay on longer lists.
         if (wave_id() == 0) {
@@ -1363,7 +1369,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     const uint32_t head_n = !head_walk ? 0u : (reach == groups ? n : uniform_u32(G.start()[reach]));
     if (UNSORTED) // (no unsorted share lies in front of an entry of the staged head: see kOpaque)
         head_walk = head_walk && head_n <= kHead;
-    if (wave_id() != 0 && r0_guess == r0_guess && !head_walk) {
+    if (wave_id() != 0 && r0_guess == r0_guess && !head_walk && !(UNORDERED && VERIFY)) {
         // (all the other waves: with more than kHeadGroups maps to build they take longer than the chain, even
         // though three of them share its SIMD)
         if constexpr (kAhead)
@@ -1458,53 +1464,83 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
     const float r0 = prod + 0.0f;
     __syncthreads();
 
-    if constexpr (UNORDERED) {
-        if (d.draft) {
+    // What the walk starts from (other than r0, the maps' reach and the staged head only when a rejected draft is redrawn)
+    float r_begin = r0;
+    uint32_t reach_w = reach, head_n_w = head_n;
+    bool head_walk_w = head_walk;
+    uint32_t redraw_g = kNone, redraw_at = kNone; // the rejected draft's group and position
+    float redraw_q = 0.0f;
+    if constexpr (UNORDERED && VERIFY) {
+        {
             // Verification (src/gen/sampler.cpp:93-106) of a row in token order: entry i is token i, so the draft's weight is
             // read off the list (0.0f if it is no candidate).  A rejected draft leaves the list for the redraw: as a weight of
-            // 0.0f it can neither stop the walk nor change r; only where the reference's walk would run off its list onto the
-            // last candidate, and that was the draft, the last one before it has to be looked for.
+            // 0.0f it can neither stop the walk nor change r.  Its group gets no map (it is gone through entry by entry,
+            // the draft's entry zeroed in the registers), the staged head and the fp64 sums behind it lose its weight,
+            // and the first block's maps are built now, from the redraw's own r.  Only where the reference's walk would
+            // run off its list onto the last candidate, and that was the draft, the last one before it is looked for.
             const uint32_t dr = (uint32_t)d.draft[row];
             const float q_draft = dr < n ? qat(dr) : 0.0f;
-            RowOut o;
-            o.n_cand = n;
-            o.total = total;
-            o.path = path_out;
-            o.accepted = r0 < q_draft;
-            o.token = (int32_t)dr;
-            o.q = q_draft;
-            if (!o.accepted) {
-                const float rest = total - q_draft;
-                const float span2 = rest - 0.0f;
-                const float prod2 = d.u2[row] * span2;
-                auto qat2 = [&](uint32_t i) { return i == dr ? 0.0f : qat(i); };
-                uint32_t at = emulate_walk(qat2, n, prod2 + 0.0f, sm);
-                if (at == dr) { // (only as the end of the list: a weight of 0.0f stops nothing)
-                    uint32_t before = 0; // (index + 1 of the last candidate in front of it)
-                    for (uint32_t i = tid; i < dr; i += kThreads)
-                        before = qat(i) > 0.0f ? i + 1u : before;
-                    before = kNone - block_min_u32(kNone - before, sm.bs);
-                    at = before ? before - 1u : dr; // (no other candidate: the draft, src/gen/sampler.cpp:104-105)
+            if (r0 < q_draft) { // accepted
+                if (d.out_cand_idx && d.out_cand_q)
+                    for (uint32_t j = tid; j < n && j < d.cand_cap; j += kThreads) {
+                        d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
+                        d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
+                    }
+                if (tid == 0) {
+                    RowOut o;
+                    o.token = (int32_t)dr;
+                    o.n_cand = n;
+                    o.total = total;
+                    o.q = q_draft;
+                    o.path = path_out;
+                    o.accepted = 1;
+                    write_row(d, row, o);
                 }
-                o.token = (int32_t)at;
-                o.q = at == dr ? q_draft : qat(at);
+                return true;
             }
-            if (d.out_cand_idx && d.out_cand_q)
-                for (uint32_t j = tid; j < n && j < d.cand_cap; j += kThreads) {
-                    d.out_cand_idx[(size_t)row * d.cand_cap + j] = (int32_t)idat(j);
-                    d.out_cand_q[(size_t)row * d.cand_cap + j] = qat(j);
+            const float rest = total - q_draft;
+            const float span2 = rest - 0.0f;
+            const float prod2 = d.u2[row] * span2;
+            r_begin = prod2 + 0.0f;
+            if (q_draft > 0.0f) { // (the draft is a candidate, at dr < n)
+                redraw_at = dr;
+                redraw_q = q_draft;
+                redraw_g = dr / kGroup; // (a list in token order: every group but the last holds kGroup entries)
+                for (uint32_t g = redraw_g + 1u + tid; g <= groups; g += kThreads)
+                    G.pg()[g] -= (double)q_draft;
+                if (tid == 0) {
+                    G.misc()[5] = redraw_g;
+                    G.w_pack()[redraw_g] = G.w_pack()[redraw_g] & kLenMask; // (no binade, no quarter records)
+                    if (dr < kHead)
+                        head[dr] = 0.0f;
                 }
-            if (tid == 0)
-                write_row(d, row, o);
-            return true;
+            }
+            __syncthreads();
+            const double rg = (double)r_begin;
+            reach_w = groups;
+            for (uint32_t g0 = 0; g0 < groups; g0 += kWave) {
+                const uint32_t g = g0 + lane_id();
+                const unsigned long long beyond = __ballot(g < groups && !(rg * 1.001 - G.pg()[min(g, groups - 1u)] > 0));
+                if (beyond) { // uniform
+                    reach_w = g0 + (uint32_t)__ffsll((long long)beyond) - 1u;
+                    break;
+                }
+            }
+            head_walk_w = reach_w <= kHeadGroups;
+            head_n_w = !head_walk_w ? 0u : (reach_w == groups ? n : uniform_u32(G.start()[reach_w]));
+            head_walk_w = head_walk_w && head_n_w <= kHead;
+            if (rg == rg && !head_walk_w)
+                build_group_maps<false, true, true>(kf, min(reach_w, (uint32_t)kWave), true, rg, G, wave_id(), kWaves, 0u,
+                                                    QuarterSlots{3u, 0u, kFirstSlots});
+            __syncthreads();
         }
     }
 
     // exact walk
     uint32_t pos = n - 1;
-    if (r0 < 0.0f) {
+    if (r_begin < 0.0f) {
         pos = 0;
-    } else if (r0 == r0 && r0 != INFINITY) {
+    } else if (r_begin == r_begin && r_begin != INFINITY) {
         MAKO_STAMP(14);
         // The state of the walk (wave 0's, in scalar registers; between blocks of 64 groups in LDS).
         uint32_t M = 0;
@@ -1516,19 +1552,19 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
             {
                 uint32_t Mv;
                 int ev;
-                split(r0, Mv, ev);
+                split(r_begin, Mv, ev);
                 M = uniform_u32(Mv);
                 e = (int)uniform_u32((uint32_t)ev);
             }
-            if (head_walk && head_n) {
-                float r = r0;
-                stopped = walk_lds(head, head_n, r, at);
+            if (head_walk_w && head_n_w) {
+                float r = r_begin;
+                stopped = walk_lds(head, head_n_w, r, at);
                 uint32_t Mv;
                 int ev;
                 split(r, Mv, ev);
                 M = uniform_u32(Mv);
                 e = (int)uniform_u32((uint32_t)ev);
-                first = reach;
+                first = reach_w;
             }
         }
         // The groups are walked 64 at a time.  The first block's maps were built beside the running sum, for the
@@ -1565,7 +1601,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                     }
                 }
             } else {
-                double r_here = (double)r0;
+                double r_here = (double)r_begin;
                 if (base > 0) {
                     if (wave_id() == 0 && lane_id() == 0) {
                         G.misc()[0] = M;
@@ -1582,7 +1618,7 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                 const uint32_t next = base + (uint32_t)kWave;
                 if (wave_id() != 0 && next < groups && r_here - (G.pg()[next] - G.pg()[base]) > r_here * -0x1p-6) { // uniform
                     const uint32_t half = ((next / (uint32_t)kWave) & 1u);
-                    build_group_maps<UNSORTED, UNORDERED>(kf, min(groups, next + (uint32_t)kWave), true, r_here + G.pg()[base], G, (uint32_t)wave_id() - 1u,
+                    build_group_maps<UNSORTED, UNORDERED, UNORDERED && VERIFY>(kf, min(groups, next + (uint32_t)kWave), true, r_here + G.pg()[base], G, (uint32_t)wave_id() - 1u,
                                                (uint32_t)kWaves - 1u, next, QuarterSlots{3u + half, half * (kQuarterSlots / 2u), kQuarterSlots / 2u});
                 }
             }
@@ -1623,6 +1659,17 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
                         const uint32_t pk = (uint32_t)__builtin_amdgcn_readlane((int)pk_l, g);
                         float xa[4];
                         take_span_lanes(raw, pk & kLenMask, xa);
+                        if constexpr (UNORDERED && VERIFY) {
+                            if (base + g == redraw_g) { // (the rejected draft's own entry, out of the list: entry 64 j + lane is xa[j])
+                                const uint32_t in_g = redraw_at % kGroup;
+                                if ((uint32_t)lane_id() == (in_g & 63u)) {
+                                    xa[0] = (in_g >> 6) == 0u ? 0.0f : xa[0];
+                                    xa[1] = (in_g >> 6) == 1u ? 0.0f : xa[1];
+                                    xa[2] = (in_g >> 6) == 2u ? 0.0f : xa[2];
+                                    xa[3] = (in_g >> 6) == 3u ? 0.0f : xa[3];
+                                }
+                            }
+                        }
                         // (the next group's entries set out now; they are used only if that group is replayed too)
                         const uint32_t g1 = min(g + 1u, cnt - 1u);
                         const uint32_t st1 = (uint32_t)__builtin_amdgcn_readlane((int)st_l, g1);
@@ -1687,6 +1734,15 @@ __device__ bool sorted_tail(const mako_sample_desc& d, uint32_t row, const mako_
         pos = G.misc()[2];
         if (UNSORTED && pos == kNone)
             return false;
+    }
+    if constexpr (UNORDERED && VERIFY) {
+        if (pos == redraw_at) { // (only as the end of the list: a weight of 0.0f stops nothing)
+            uint32_t before = 0; // (index + 1 of the last candidate in front of it)
+            for (uint32_t i = tid; i < redraw_at; i += kThreads)
+                before = qat(i) > 0.0f ? i + 1u : before;
+            before = kNone - block_min_u32(kNone - before, sm.bs);
+            pos = before ? before - 1u : redraw_at; // (no other candidate: the draft, src/gen/sampler.cpp:104-105)
+        }
     }
 
     MAKO_STAMP(9);
