@@ -54,6 +54,13 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
     const mako_sample_desc& d = s_args.d;
     const Scratch& sc = s_args.sc;
     const mako_sampling_params& P = s_args.P;
+    if (d.force_token || d.close_token) { // a forced row needs no weights: it is not claimed, and the launch that
+                                          // finishes the late rows writes its token
+        int32_t ftok;
+        uint32_t above;
+        if (row_forced(d, sc, row, slices, ftok, above) != MAKO_FORCED_NONE)
+            return;
+    }
     float m;
     uint32_t argidx, n_cands, any_overflow;
     row_summary(sc, row, slices, m, argidx, n_cands, any_overflow);
@@ -155,6 +162,10 @@ __global__ __launch_bounds__(kThreads) void index_groups_kernel(mako_sample_desc
     if (!index_order_row(P0)) // uniform
         return;
     BigPlan* plan = sc_val.plan + row;
+    // (zero: index_weights_kernel left the row alone, its token is forced; a workgroup that starts late may already see
+    // what this kernel's first workgroup has made of the flag)
+    if (plan->flag == 0u) // uniform
+        return;
     const uint32_t pieces = (d_arg.n_vocab + kSliceMax - 1u) / kSliceMax, blocks = (d_arg.n_vocab + kIndexBlock - 1u) / kIndexBlock;
     const uint32_t cnt_l = lane < pieces ? plan->cursor[min(lane, kWorkers - 1u)] : 0u;
     const uint32_t last_l = lane < pieces ? plan->key_lo[min(lane, kWorkers - 1u)] : 0u;

@@ -203,3 +203,30 @@ def test_verification_of_rows_in_token_order(gpu_ctx):
         h = gpu_rows(gpu_ctx, w, cap=cap, draft=draft, u2=u2)
         assert np.array_equal(h["tokens"], g["tokens"]) and np.array_equal(h["accepted"], g["accepted"])
         assert np.array_equal(h["total"].view(np.uint32), g["total"].view(np.uint32))
+
+
+def test_forced_and_close_tokens_beside_rows_in_token_order(gpu_ctx):
+    """The decode loop's hooks (force_token, close_token) on a batch of temperature-only rows: a forced row is left to
+    the launch that writes forced tokens, the others take the kernels of their own; the results are those of the call
+    without the host copy of the parameters."""
+    rng = np.random.Generator(np.random.PCG64([11, 96]))
+    rows, vocab = 48, 129280
+    w = _plain_batch(rows, vocab, 11, sigmas=(3.0, 1.0), temps=(0.8, 1.1))
+    force = np.full(rows, -1, np.int32)
+    force[::5] = rng.integers(0, vocab, len(force[::5]))
+    close = np.full(rows, -1, np.int32)
+    order = np.argsort(-w["logits"], axis=1, kind="stable")
+    close[1::3] = order[1::3, 1]   # the second most likely token: taken (fewer than three logits above it)
+    close[2::6] = order[2::6, 40]  # an unlikely one: not taken
+    kw = dict(force_token=force, close_token=close, close_max_above=3, cand_cap=32)
+    g = api.sample(gpu_ctx, w["logits"], w["params"], w["u"], params_host=True, **kw)
+    h = api.sample(gpu_ctx, w["logits"], w["params"], w["u"], **kw)
+    _say("forced beside rows in token order, paths: %s" % _paths(g))
+    for key in ("tokens", "forced", "above", "n_cand"):
+        assert np.array_equal(g[key], h[key]), key
+    assert np.array_equal(g["total"].view(np.uint32), h["total"].view(np.uint32))
+    forced = g["forced"] != api.FORCED_NONE
+    assert forced.sum() >= 10 and (g["path"][forced] == api.PATH_FORCED).all() and (g["path"][~forced] == PATH_INDEXED).all()
+    assert (g["tokens"][::5] == force[::5]).all()
+    ref = oracle_rows(w)
+    assert all(g["tokens"][r] == ref[r][0] for r in range(rows) if not forced[r])
