@@ -137,11 +137,9 @@ int mako_sampler_sample_batch(mako_sampler_ctx* ctx, const mako_sample_desc* des
  * looks at them on the calling thread and leaves out the kernels that no row of the batch needs (a batch without
  * top_k == 0 rows takes two launches instead of four).  Rows that are cut neither to a top-k nor to a nucleus
  * (temperature only: top_k == 0, top_p >= 1), whose candidates stay in token order, get three launches of their own
- * instead of one workgroup each for the whole row (not with rows that
- * are not 16-byte aligned multiples of four logits, or beyond 262 144 logits); under the same conditions the other rows of
- * the whole-row path (a top-k without a top-p, a top-k beyond 128) get their weights from many workgroups instead of
- * one.  The results never depend on it;
- * null = the call above. */
+ * instead of one workgroup each for the whole row (up to 262 144 logits per row), verification and the decode loop's
+ * hooks included; the other rows of the whole-row path (a top-k without a top-p, a top-k beyond 128) then get their
+ * weights from many workgroups instead of one.  The results never depend on it; null = the call above. */
 int mako_sampler_sample_batch_hinted(mako_sampler_ctx* ctx, const mako_sample_desc* desc,
                                      const mako_sampling_params* params_host, void* stream);
 

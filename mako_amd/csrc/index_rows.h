@@ -31,8 +31,9 @@ static_assert(kIndexMaxVocab / kSliceMax <= kWorkers && kIndexMaxVocab / kIndexB
                   kSliceMax == 4u * kIndexBlock && kIndexBlock == (uint32_t)kWaves * kGroup,
               "a piece's count and last candidate travel in the plan's per-worker words, the blocks' sums in the row's part_sum, a lane each");
 #ifdef MAKO_EMIT_INDEX_KERNELS
-// grid = (ceil(V / 16384), rows); rows of other kinds leave at once.  V % 4 == 0 and aligned rows (the host checks).
-template <int KH>
+// grid = (ceil(V / 16384), rows); rows of other kinds leave at once.  (VEC: V % 4 == 0 and 16-byte aligned rows, whose
+// logits are loaded four at a time; the layout of a thread's sixteen logits is slice_load.h's either way.)
+template <bool VEC, int KH>
 __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_desc d_arg, Scratch sc_val, uint32_t slices)
 {
     extern __shared__ __align__(16) unsigned long long s_dyn64[];
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
     const bool pen = d.hist_tokens && !penalties_neutral(P);
     const uint32_t lo = piece * kSliceMax, hi = min(d.n_vocab, lo + kSliceMax);
     float wv[16];
-    load_penalised<true, KH>(d, row, lo, hi, kSliceMax, P, hl, pen, reinterpret_cast<uint32_t*>(s_dyn64), wv);
+    load_penalised<VEC, KH>(d, row, lo, hi, kSliceMax, P, hl, pen, reinterpret_cast<uint32_t*>(s_dyn64), wv);
     const float inv_t = 1.0f / P.temperature;
     const float floor_q = (1.0f < P.min_p) ? 1.0f : P.min_p;
     // (~bits(q) into the row's list, or bits(q) into the whole-row path's array)
@@ -80,25 +81,27 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
 #pragma unroll
     for (uint32_t b = 0; b < 4; ++b) {
         bsum[b] = 0.0;
-        const uint32_t base = lo + b * kIndexBlock + tid * 4u;
+        // (the thread's logits 4b .. 4b+3 lie in the piece's b-th 4 096: four in a row, or 1 024 apart)
+        const uint32_t base = elem_index<VEC>(lo, tid, 4u * b);
         if (lo + b * kIndexBlock < hi) { // uniform
             uint32_t k[4];
 #pragma unroll
             for (uint32_t c = 0; c < 4; ++c) {
+                const uint32_t at = elem_index<VEC>(lo, tid, 4u * b + c);
                 const float q = weight_of(wv[4u * b + c], m, inv_t, sm.tab);
-                const bool ok = base + c < hi && q >= floor_q && q > 0.0f; // src/gen/sampler.cpp:34-35
+                const bool ok = at < hi && q >= floor_q && q > 0.0f; // src/gen/sampler.cpp:34-35
                 k[c] = ok ? __float_as_uint(q) : 0u;
                 cnt += ok ? 1u : 0u;
-                last = ok ? base + c + 1u : last;
+                last = ok ? max(last, at + 1u) : last;
                 bsum[b] += ok ? (double)q : 0.0;
             }
-            if (base + 3u < hi) {
+            if (VEC && base + 3u < hi) {
                 *reinterpret_cast<uint4*>(key0 + base) = make_uint4(k[0] ^ flip, k[1] ^ flip, k[2] ^ flip, k[3] ^ flip);
             } else {
 #pragma unroll
                 for (uint32_t c = 0; c < 4; ++c)
-                    if (base + c < hi)
-                        key0[base + c] = k[c] ^ flip;
+                    if (elem_index<VEC>(lo, tid, 4u * b + c) < hi)
+                        key0[elem_index<VEC>(lo, tid, 4u * b + c)] = k[c] ^ flip;
             }
         }
         // (four weights at a time: with all sixteen in flight the kernel needs twice the registers, and two workgroups

@@ -4,15 +4,26 @@
 #include "sampler_kernels.h"
 
 namespace mako {
-void launch_index_weights(int kh, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices)
+namespace {
+template <bool VEC>
+void launch_weights(int kh, dim3 grid, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices)
+{
+    if (kh == 2)
+        hipLaunchKernelGGL((index_weights_kernel<VEC, 2>), grid, dim3(kThreads), kDynLds, st, d, sc, slices);
+    else if (kh == 8)
+        hipLaunchKernelGGL((index_weights_kernel<VEC, 8>), grid, dim3(kThreads), kDynLds, st, d, sc, slices);
+    else
+        hipLaunchKernelGGL((index_weights_kernel<VEC, 0>), grid, dim3(kThreads), kDynLds, st, d, sc, slices);
+}
+} // namespace
+
+void launch_index_weights(bool vec, int kh, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices)
 {
     const dim3 grid((d.n_vocab + kSliceMax - 1u) / kSliceMax, d.n_rows);
-    if (kh == 2)
-        hipLaunchKernelGGL(index_weights_kernel<2>, grid, dim3(kThreads), kDynLds, st, d, sc, slices);
-    else if (kh == 8)
-        hipLaunchKernelGGL(index_weights_kernel<8>, grid, dim3(kThreads), kDynLds, st, d, sc, slices);
+    if (vec)
+        launch_weights<true>(kh, grid, st, d, sc, slices);
     else
-        hipLaunchKernelGGL(index_weights_kernel<0>, grid, dim3(kThreads), kDynLds, st, d, sc, slices);
+        launch_weights<false>(kh, grid, st, d, sc, slices);
 }
 
 void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, bool in_order_rows)
@@ -28,7 +39,9 @@ void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratc
 
 hipError_t init_index_kernels()
 {
-    const void* kernels[] = {(const void*)index_weights_kernel<0>, (const void*)index_weights_kernel<2>, (const void*)index_weights_kernel<8>};
+    const void* kernels[] = {(const void*)index_weights_kernel<true, 0>,  (const void*)index_weights_kernel<true, 2>,
+                             (const void*)index_weights_kernel<true, 8>,  (const void*)index_weights_kernel<false, 0>,
+                             (const void*)index_weights_kernel<false, 2>, (const void*)index_weights_kernel<false, 8>};
     for (const void* k : kernels) {
         const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDynLds);
         if (e != hipSuccess)

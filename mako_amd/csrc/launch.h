@@ -37,6 +37,6 @@ void launch_tail(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, u
 // the three kernels of the rows whose candidates stay in token order (index_rows.h): the weights (before tail_kernel's
 // launch, which then leaves such rows alone), the group records, the total and the draw (behind it)
 hipError_t init_index_kernels();
-void launch_index_weights(int kh, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices);
+void launch_index_weights(bool vec, int kh, hipStream_t st, const mako_sample_desc& d, const Scratch& sc, uint32_t slices);
 void launch_index_finish(hipStream_t st, const mako_sample_desc& d, const Scratch& sc, bool in_order_rows);
 } // namespace mako

@@ -405,14 +405,13 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     // (any_late: rows that are finished in tail_kernel's launch, after the plan)
     // (any_index: rows cut neither to a top-k nor to a nucleus, whose candidates stay in token order; known only from
     // the caller's copy of the parameters, they get the kernels of index_rows.h instead of a workgroup each on the
-    // whole-row path, unless the batch is one those kernels do not serve: rows that are not aligned for 128-bit loads, a
-    // vocabulary beyond 262 144)
+    // whole-row path, unless the vocabulary is beyond 262 144)
     bool any_nucleus = true, any_late = true, any_index = false, only_index = false, any_in_order = false;
     uint32_t nucleus_rows = d.n_rows;
     if (params_host) {
         any_nucleus = any_late = false;
         uint32_t n_nucleus = 0, n_index = 0;
-        const bool index_served = vec && d.n_vocab <= mako::kIndexMaxVocab;
+        const bool index_served = d.n_vocab <= mako::kIndexMaxVocab;
         for (uint32_t r = 0; r < d.n_rows; ++r) {
             const mako::RowClass c = mako::classify(params_host[r]);
             // (with them every other row of the whole-row class, whose weights the first of those kernels leaves too)
@@ -456,7 +455,7 @@ int run_batch(mako_sampler_ctx* ctx, const mako_sample_desc& d, const mako_sampl
     // kernel boundaries (device-wide fences inside a kernel cost far more on this chip).  A batch without such rows
     // (and without rows for the whole-row path) ends with plan_kernel instead.
     if (any_index) // (before the launch that finishes late rows: it leaves alone what this one has claimed)
-        MAKO_LAUNCH(mako::launch_index_weights(kh, st, d, sc, slices));
+        MAKO_LAUNCH(mako::launch_index_weights(vec, kh, st, d, sc, slices));
     if (any_nucleus)
         MAKO_LAUNCH(mako::launch_finish(vec, kh, unsorted, finish_wgs, st, d, sc, slices));
     if (!launch_sort && !only_index)

@@ -117,12 +117,27 @@ def test_small_and_odd_vocabularies(vocab):
     assert (g["path"] == PATH_INDEXED).all()
 
 
-def test_rows_the_kernels_do_not_serve():
-    """A vocabulary that is no multiple of four: the rows take the whole-row path as before."""
-    ctx = api.SamplerContext(max_rows=8, max_vocab=4099, max_hist=0)
+@pytest.mark.parametrize("vocab", [4099, 50257])
+def test_vocabularies_that_are_no_multiple_of_four(vocab):
+    """The logits are then loaded one at a time (rows cannot be 16-byte aligned): the same kernels, the same results."""
+    ctx = api.SamplerContext(max_rows=12, max_vocab=vocab, max_hist=0)
     try:
-        w = _plain_batch(8, 4099, 7, spikes=False)
-        g = assert_parity(ctx, w, cap=64, hinted=True)
+        w = _plain_batch(12, vocab, 7 + vocab, sigmas=(2.0, 0.5), temps=(0.7, 1.0))
+        w["params"]["min_p"][::4] = np.float32(1e-3)
+        g = assert_parity(ctx, w, cap=0, hinted=True)
+        assert (g["path"] == PATH_INDEXED).all()
+        assert_parity(ctx, w, cap=64, hinted=True)
+    finally:
+        ctx.close()
+
+
+def test_rows_the_kernels_do_not_serve():
+    """More logits than a row's group records cover (262 144): the rows take the whole-row path as before."""
+    vocab = 262148
+    ctx = api.SamplerContext(max_rows=2, max_vocab=vocab, max_hist=0)
+    try:
+        w = _plain_batch(2, vocab, 7, spikes=False)
+        g = assert_parity(ctx, w, cap=16, hinted=True)
     finally:
         ctx.close()
     assert (g["path"] == PATH_GENERAL).all()
