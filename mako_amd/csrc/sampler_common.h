@@ -158,11 +158,11 @@ struct Scratch {
     // workgroup i serves entry i of its kernel's list and exits if there is none: the busy workgroups are then the
     // first ones dispatched and land evenly on the XCDs, shader engines and CUs, whatever the mix of rows.
     // (finish_kernel and plan_kernel get the same effect from find_piece().)
-    uint32_t* work_n;      // [16] entries in work_sort, work_tail (zeroed by scan_kernel); [3]: large batches' lists (below); [2]: failed checks of a checked
+    uint32_t* work_n;      // [8] entries in work_sort, work_tail (zeroed by scan_kernel); [3]: the large batches' collectors; [2]: failed checks of a checked
                            // build (MAKO_CHECK); then, 16-byte aligned at [4], how the second pass is cut up
                            // (SecondPassCut; scan_kernel's first workgroup decides)
     uint32_t* work_sort;   // [max_rows * kSortItemsPerRow] row << 8 | worker; appended by finish_kernel.  The large batches'
-                           // instances keep three lists in it, by what an entry costs (large_batch_lists())
+                           // instances keep two lists in it that meet, the costliest entries in front (large_batch_lists())
     uint32_t* work_tail;   // [max_rows] row; appended by finish_kernel
     uint64_t vpad;
     uint32_t slices_cap;

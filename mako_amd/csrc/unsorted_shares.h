@@ -19,9 +19,9 @@ namespace mako {
 // tail_kernel applies such a record under the same exact tests as a group's map, and gives the row to the whole-row
 // path if one fails (the share's order would be needed then and does not exist).
 //
-// Only batches with many top_k == 0 rows do this (scan_kernel decides, Scratch::work_n[3]): there sort_kernel is bound
-// by the number of its workgroups, one per CU at a time, and a share that needs no sorting is summed by a workgroup that
-// takes several of them; on a small batch every worker has a CU to itself and the batch waits for the slowest anyway.
+// Only batches with many top_k == 0 rows do this (the host decides and launches the kernels' instances for it): there
+// sort_kernel is bound by the number of its workgroups, one per CU at a time, and a share that needs no sorting is summed
+// by one wave of a collector workgroup that takes sixteen of them; on a small batch every worker has a CU to itself and the batch waits for the slowest anyway.
 
 // A record that stands for a whole unsorted share (in GroupTable::pack): its maps are all there is.  Never among the
 // first kHeadGroups groups of a list, and the list's entries at its positions are not written.
