@@ -637,26 +637,34 @@ __device__ MAKO_RARE_CALL void general_row_from_weights(const mako_sample_desc& 
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
     const uint32_t lane = lane_id(), wave = wave_id();
-    // (wave w owns the w-th sixteenth of the row, a multiple of 256 logits, lane l entries 4l..4l+3 of each 256)
+    // (wave w owns the w-th sixteenth of the row, a multiple of 256 logits, lane l entries 4l..4l+3 of each 256; eight
+    // such blocks' loads are in flight per trip, from clamped addresses and masked afterwards: one round trip to memory
+    // per 2 048 entries of the wave instead of one per 256)
     const uint32_t chunk = ((V + kThreads * 4u - 1u) / (kThreads * 4u)) * kGroup;
     const uint32_t beg = min(V, wave * chunk), end = min(V, beg + chunk);
-    auto four = [&](uint32_t i, uint32_t (&k)[4]) {
-        k[0] = k[1] = k[2] = k[3] = 0u;
-        if (i + 3u < end) {
-            const uint4 x = *reinterpret_cast<const uint4*>(qb + i);
-            k[0] = x.x, k[1] = x.y, k[2] = x.z, k[3] = x.w;
-        } else {
+    const uint32_t last_vec = (uint32_t)sc.vpad - 4u; // (vpad is a multiple of 1024)
+    constexpr uint32_t kTrip = 8;
+    auto load_trip = [&](uint32_t base, uint32_t (&k)[kTrip][4]) {
+        uint4 x[kTrip];
 #pragma unroll
-            for (uint32_t j = 0; j < 4; ++j)
-                if (i + j < end)
-                    k[j] = qb[i + j];
+        for (uint32_t u = 0; u < kTrip; ++u)
+            x[u] = *reinterpret_cast<const uint4*>(qb + min(base + u * kGroup + lane * 4u, last_vec));
+#pragma unroll
+        for (uint32_t u = 0; u < kTrip; ++u) {
+            const uint32_t i = base + u * kGroup + lane * 4u;
+            k[u][0] = i < end ? x[u].x : 0u;
+            k[u][1] = i + 1u < end ? x[u].y : 0u;
+            k[u][2] = i + 2u < end ? x[u].z : 0u;
+            k[u][3] = i + 3u < end ? x[u].w : 0u;
         }
     };
     uint32_t mine = 0;
-    for (uint32_t base = beg; base < end; base += kGroup) {
-        uint32_t k[4];
-        four(base + lane * 4u, k);
-        mine += (k[0] ? 1u : 0u) + (k[1] ? 1u : 0u) + (k[2] ? 1u : 0u) + (k[3] ? 1u : 0u);
+    for (uint32_t base = beg; base < end; base += kGroup * kTrip) {
+        uint32_t k[kTrip][4];
+        load_trip(base, k);
+#pragma unroll
+        for (uint32_t u = 0; u < kTrip; ++u)
+            mine += (k[u][0] ? 1u : 0u) + (k[u][1] ? 1u : 0u) + (k[u][2] ? 1u : 0u) + (k[u][3] ? 1u : 0u);
     }
     mine = __ockl_wfred_add_u32(mine);
     __syncthreads();
@@ -670,22 +678,49 @@ __device__ MAKO_RARE_CALL void general_row_from_weights(const mako_sample_desc& 
             at += x;
         n0 += x;
     }
-    for (uint32_t base = beg; base < end; base += kGroup) {
-        const uint32_t i = base + lane * 4u;
-        uint32_t k[4];
-        four(i, k);
-        const uint32_t c = (k[0] ? 1u : 0u) + (k[1] ? 1u : 0u) + (k[2] ? 1u : 0u) + (k[3] ? 1u : 0u);
-        const uint32_t incl = __ockl_wfscan_add_u32(c, true);
-        uint32_t pos = at + incl - c;
+    if (n0 == V) {
+        // every logit is a candidate (no mask, no floor, no underflow: the usual row): the list is the array itself,
+        // written four entries per lane and store
+        for (uint32_t base = beg; base < end; base += kGroup * kTrip) {
+            uint32_t k[kTrip][4];
+            load_trip(base, k);
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j)
-            if (k[j]) {
-                MAKO_CHECK(sc, kCheckCompact, pos < n0 && (uint64_t)pos < sc.vpad);
-                key0[pos] = ~k[j];
-                idx0[pos] = i + j;
-                ++pos;
+            for (uint32_t u = 0; u < kTrip; ++u) {
+                const uint32_t i = base + u * kGroup + lane * 4u;
+                if (i + 3u < end) {
+                    *reinterpret_cast<uint4*>(key0 + i) = make_uint4(~k[u][0], ~k[u][1], ~k[u][2], ~k[u][3]);
+                    *reinterpret_cast<uint4*>(idx0 + i) = make_uint4(i, i + 1u, i + 2u, i + 3u);
+                } else {
+#pragma unroll
+                    for (uint32_t j = 0; j < 4; ++j)
+                        if (i + j < end) {
+                            key0[i + j] = ~k[u][j];
+                            idx0[i + j] = i + j;
+                        }
+                }
             }
-        at += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+        }
+    } else {
+        for (uint32_t base = beg; base < end; base += kGroup * kTrip) {
+            uint32_t k[kTrip][4];
+            load_trip(base, k);
+#pragma unroll
+            for (uint32_t u = 0; u < kTrip; ++u) {
+                const uint32_t i = base + u * kGroup + lane * 4u;
+                const uint32_t c = (k[u][0] ? 1u : 0u) + (k[u][1] ? 1u : 0u) + (k[u][2] ? 1u : 0u) + (k[u][3] ? 1u : 0u);
+                const uint32_t incl = __ockl_wfscan_add_u32(c, true);
+                uint32_t pos = at + incl - c;
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j)
+                    if (k[u][j]) {
+                        MAKO_CHECK(sc, kCheckCompact, pos < n0 && (uint64_t)pos < sc.vpad);
+                        key0[pos] = ~k[u][j];
+                        idx0[pos] = i + j;
+                        ++pos;
+                    }
+                at += (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+            }
+        }
     }
     __syncthreads();
     if (n0 == 0) {
