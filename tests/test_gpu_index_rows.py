@@ -245,3 +245,18 @@ def test_forced_and_close_tokens_beside_rows_in_token_order(gpu_ctx):
     assert (g["tokens"][::5] == force[::5]).all()
     ref = oracle_rows(w)
     assert all(g["tokens"][r] == ref[r][0] for r in range(rows) if not forced[r])
+
+
+def test_beside_a_large_batch_of_nucleus_rows():
+    """config 4's 256 rows (the large batches' instances of the kernels, unsorted shares included) with every eighth
+    row made a temperature-only row."""
+    w = workloads.config4()
+    rows, vocab = w["logits"].shape
+    w["params"]["top_p"][::8] = np.float32(1.0)
+    ctx = api.SamplerContext(max_rows=rows, max_vocab=vocab, max_hist=0)
+    try:
+        g = assert_parity(ctx, w, cap=0, hinted=True)
+    finally:
+        ctx.close()
+    _say("large mixed batch paths: %s" % _paths(g))
+    assert (g["path"][::8] == PATH_INDEXED).all() and (g["path"] == api.PATH_SUMMED).sum() >= 80
