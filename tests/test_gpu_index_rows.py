@@ -260,3 +260,34 @@ def test_beside_a_large_batch_of_nucleus_rows():
         ctx.close()
     _say("large mixed batch paths: %s" % _paths(g))
     assert (g["path"][::8] == PATH_INDEXED).all() and (g["path"] == api.PATH_SUMMED).sum() >= 80
+
+
+@pytest.mark.parametrize("hist_len", [5000, 10000])
+def test_long_histories(hist_len):
+    """Histories beyond two (eight) entries per thread take the weights kernel's other instances."""
+    rng = np.random.Generator(np.random.PCG64([12, hist_len]))
+    rows, vocab = 12, 65536
+    w = _plain_batch(rows, vocab, 12, sigmas=(2.0,), temps=(0.8, 1.1))
+    w["params"]["repetition_penalty"] = 1.2
+    w["params"]["frequency_penalty"] = 0.1
+    w["params"]["presence_penalty"] = 0.4
+    w["hist"] = rng.integers(0, vocab, (rows, hist_len)).astype(np.int32)
+    w["hist_len"] = rng.integers(hist_len // 2, hist_len + 1, rows).astype(np.uint32)
+    ctx = api.SamplerContext(max_rows=rows, max_vocab=vocab, max_hist=hist_len)
+    try:
+        g = assert_parity(ctx, w, cap=32, hinted=True)
+    finally:
+        ctx.close()
+    assert (g["path"] == PATH_INDEXED).all()
+
+
+def test_more_rows_than_a_workgroup_has_threads():
+    ctx = api.SamplerContext(max_rows=1100, max_vocab=320, max_hist=0)
+    try:
+        w = _plain_batch(1100, 320, 13, sigmas=(2.0, 0.3), temps=(0.7, 1.3), spikes=False)
+        w["params"]["top_p"][::3] = np.float32(0.9)
+        w["params"]["top_k"][1::5] = 7
+        g = assert_parity(ctx, w, cap=8, hinted=True)
+    finally:
+        ctx.close()
+    assert (g["path"] == PATH_INDEXED).sum() >= 400
