@@ -205,9 +205,10 @@ __device__ void heap_select_rest(Get get, Put put, uint32_t first, uint32_t last
 }
 
 // std::ranges::nth_element(cand, cand + nth, desc) of src/gen/sampler.cpp:41 as libstdc++ 11 runs it (introselect,
-// bits/stl_algo.h:1964), leaving the candidates in exactly the arrangement that library leaves: the reference sums
-// and walks the top_k survivors in that order when no top-p follows.  key/idx hold n candidates (~bits(q), token
-// id); `desc` is the order of the 64-bit values key << 32 | idx, all distinct.
+// bits/stl_algo.h:1964), leaving the first nth candidates in exactly the arrangement that library leaves: the
+// reference keeps those (sampler.cpp:42) and sums and walks them in that order when no top-p follows.  What lies behind
+// a cut that the rounds leave behind them is not kept up.  key/idx hold n candidates (~bits(q), token id); `desc` is
+// the order of the 64-bit values key << 32 | idx, all distinct.
 // One round = median of three to the front, then the unguarded Hoare partition of the rest around it.  That
 // partition swaps the t-th entry from the left that belongs right with the t-th entry from the right that belongs
 // left for as long as the former lies before the latter, and cuts behind the entries that belong left: the two
@@ -215,11 +216,11 @@ __device__ void heap_select_rest(Get get, Put put, uint32_t first, uint32_t last
 // The depth limit's heap select is heap_select_rest() above; the last insertion sort (at most three entries) is one
 // thread's.
 //
-// introselect_rounds runs the rounds on [first, last) through get(i) / put(i, v) until the range is no longer than
+// introselect_rounds runs the rounds on [first, last) through get(i) / get_key(i) (the high half alone) / put(i, v) until the range is no longer than
 // `until` (3 = to the end, insertion sort included).  lsta / lstb: room for last - first positions each.  cache /
 // cache_cap: LDS for heap_select_rest().  Returns true when nothing is left to do.
-template <typename Get, typename Put>
-__device__ bool introselect_rounds(Get get, Put put, uint32_t& first, uint32_t& last, uint32_t nth, uint32_t& depth,
+template <typename Get, typename GetKey, typename Put>
+__device__ bool introselect_rounds(Get get, GetKey get_key, Put put, uint32_t& first, uint32_t& last, uint32_t nth, uint32_t& depth,
                                    uint32_t until, uint32_t* lsta, uint32_t* lstb, FinishShared& sm,
                                    unsigned long long* cache, uint32_t cache_cap)
 {
@@ -242,24 +243,66 @@ __device__ bool introselect_rounds(Get get, Put put, uint32_t& first, uint32_t& 
             const u64 r = get(first), med = get(im);
             put(first, med);
             put(im, r);
+            sm.bs.bcast = 0; // the pairs that change places, counted below
         }
         __syncthreads();
         const u64 pivot = get(first);
-        const uint32_t lo0 = first + 1u, len = last - lo0;
+        const uint32_t lo0 = uniform_u32(first + 1u), last_s = uniform_u32(last), len = last_s - lo0; // (scalars, like all
+                                                                                                      // of a wave's bounds and counts below)
         const uint32_t chunk = ((len + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
-        const uint32_t beg = min(last, lo0 + wave * chunk), end = min(last, beg + chunk);
+        const uint32_t beg = uniform_u32(min(last_s, lo0 + wave * chunk)), end = min(last_s, beg + chunk);
         // entries of the wave's chunk that belong left of the cut
-        // (kTrip loads in flight per lane: a trip costs one round trip to memory, not kTrip)
-        constexpr uint32_t kTrip = 4;
+        // (kTrip loads in flight per lane: a trip costs one round trip to memory, not kTrip; the high halves decide
+        // but for an entry whose weight is the pivot's; one workgroup's instruction issue bounds these passes, so they
+        // keep what they can in wave masks: per entry one compare, the masks' scalar arithmetic, and for an entry
+        // that is listed its rank among the mask's lanes)
+        constexpr uint32_t kTrip = 8;
+        const uint32_t pivot_key = uniform_u32((uint32_t)(pivot >> 32));
+        // left[u] / in[u]: the lanes whose entry base + 64 u + lane belongs left / lies in the chunk
+        auto trip_masks = [&](uint32_t base, u64 (&left)[kTrip], u64 (&in)[kTrip]) {
+            uint32_t k[kTrip];
+            u64 ties = 0;
+            if (base + kWave * kTrip <= end) { // (uniform)
+                const size_t at = (size_t)base + lane;
+#pragma unroll
+                for (uint32_t u = 0; u < kTrip; ++u)
+                    k[u] = get_key(at + u * kWave);
+#pragma unroll
+                for (uint32_t u = 0; u < kTrip; ++u) {
+                    in[u] = ~0ull;
+                    left[u] = __builtin_amdgcn_ballot_w64(k[u] < pivot_key);
+                    ties |= __builtin_amdgcn_ballot_w64(k[u] == pivot_key);
+                }
+            } else {
+#pragma unroll
+                for (uint32_t u = 0; u < kTrip; ++u)
+                    k[u] = get_key((size_t)min(base + u * kWave + lane, last_s - 1u));
+#pragma unroll
+                for (uint32_t u = 0; u < kTrip; ++u) {
+                    in[u] = __builtin_amdgcn_ballot_w64(base + u * kWave + lane < end);
+                    left[u] = __builtin_amdgcn_ballot_w64(k[u] < pivot_key) & in[u];
+                    ties |= __builtin_amdgcn_ballot_w64(k[u] == pivot_key) & in[u];
+                }
+            }
+            if (ties) { // (rare)
+#pragma unroll
+                for (uint32_t u = 0; u < kTrip; ++u) {
+                    const uint32_t pos = base + u * kWave + lane;
+                    bool l = false;
+                    if (pos < end && k[u] == pivot_key)
+                        l = get(pos) < pivot;
+                    left[u] |= __builtin_amdgcn_ballot_w64(l);
+                }
+            }
+        };
+        auto rank_in = [](u64 m) { return __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u)); };
         uint32_t mine = 0;
         for (uint32_t base = beg; base < end; base += kWave * kTrip) {
-            u64 v[kTrip];
+            u64 left[kTrip], in[kTrip];
+            trip_masks(base, left, in);
 #pragma unroll
             for (uint32_t u = 0; u < kTrip; ++u)
-                v[u] = get(min(base + u * kWave + lane, last - 1u));
-#pragma unroll
-            for (uint32_t u = 0; u < kTrip; ++u)
-                mine += (uint32_t)__popcll(__ballot(base + u * kWave + lane < end && v[u] < pivot));
+                mine += (uint32_t)__popcll(left[u]);
         }
         if (lane == 0)
             sm.bs.u64[wave] = mine;
@@ -271,42 +314,69 @@ __device__ bool introselect_rounds(Get get, Put put, uint32_t& first, uint32_t& 
                 small_before += x;
             smalls += x;
         }
-        const uint32_t bigs = len - smalls;
+        small_before = uniform_u32(small_before);
+        smalls = uniform_u32(smalls);
+        const uint32_t cut = lo0 + smalls;
+        // Only the big entries before the cut and the small ones behind it change places, the t-th of the former
+        // with the t-th of the latter counted from the right: as many of one kind as of the other.  When the rounds go
+        // on in the left part (cut > nth), what lies behind the cut is never read again (nth_element's caller keeps the
+        // first nth entries only): the big entries need not be moved there.
+        const bool right_kept = cut <= nth;
         uint32_t big_before = (beg - lo0) - small_before;
-        // position lists: lsta[t] = the t-th big entry from the left, lstb[t] = the t-th small entry from the left
-        const u64 lower = (1ull << lane) - 1ull;
+        // position lists: lsta[t] = the t-th big entry from the left (those before the cut), lstb[t] = the t-th small
+        // entry from the left (those behind it)
+        uint32_t moving = 0; // big entries of the wave's chunk before the cut
         for (uint32_t base = beg; base < end; base += kWave * kTrip) {
-            u64 v[kTrip];
+            u64 left[kTrip], in[kTrip];
+            trip_masks(base, left, in);
+            if (base + kWave * kTrip <= cut) { // (uniform; all but one of the chunks' trips lie on one side of the cut)
 #pragma unroll
-            for (uint32_t u = 0; u < kTrip; ++u)
-                v[u] = get(min(base + u * kWave + lane, last - 1u));
+                for (uint32_t u = 0; u < kTrip; ++u) {
+                    const u64 big = in[u] & ~left[u];
+                    if ((big >> lane) & 1ull)
+                        lsta[big_before + rank_in(big)] = base + u * kWave + lane;
+                    const uint32_t nb = (uint32_t)__popcll(big);
+                    big_before += nb;
+                    moving += nb;
+                    small_before += (uint32_t)__popcll(left[u]);
+                }
+            } else if (base >= cut) {
 #pragma unroll
-            for (uint32_t u = 0; u < kTrip; ++u) {
-                const uint32_t pos = base + u * kWave + lane;
-                const bool in = pos < end;
-                const bool small = in && v[u] < pivot;
-                const u64 bs = __ballot(small), bb = __ballot(in && !small);
-                if (small)
-                    lstb[small_before + (uint32_t)__popcll(bs & lower)] = pos;
-                else if (in)
-                    lsta[big_before + (uint32_t)__popcll(bb & lower)] = pos;
-                small_before += (uint32_t)__popcll(bs);
-                big_before += (uint32_t)__popcll(bb);
+                for (uint32_t u = 0; u < kTrip; ++u) {
+                    if ((left[u] >> lane) & 1ull)
+                        lstb[small_before + rank_in(left[u])] = base + u * kWave + lane;
+                    small_before += (uint32_t)__popcll(left[u]);
+                }
+            } else {
+#pragma unroll
+                for (uint32_t u = 0; u < kTrip; ++u) {
+                    const uint32_t pos = base + u * kWave + lane;
+                    const u64 big = in[u] & ~left[u];
+                    const u64 before = __builtin_amdgcn_ballot_w64(pos < cut);
+                    if ((left[u] >> lane) & 1ull) {
+                        if (pos >= cut)
+                            lstb[small_before + rank_in(left[u])] = pos;
+                    } else if (((big >> lane) & 1ull) && pos < cut)
+                        lsta[big_before + rank_in(big)] = pos;
+                    big_before += (uint32_t)__popcll(big);
+                    moving += (uint32_t)__popcll(big & before);
+                    small_before += (uint32_t)__popcll(left[u]);
+                }
             }
         }
+        if (lane == 0 && moving)
+            atomicAdd(&sm.bs.bcast, (u64)moving);
         __syncthreads();
-        const uint32_t pairs = min(bigs, smalls);
+        const uint32_t pairs = (uint32_t)sm.bs.bcast;
         for (uint32_t t = tid; t < pairs; t += kThreads) {
             const uint32_t a = lsta[t], b = lstb[smalls - 1u - t];
-            if (a < b) {
-                const u64 va = get(a), vb = get(b);
-                put(a, vb);
-                put(b, va);
-            }
+            const u64 vb = get(b);
+            if (right_kept)
+                put(b, get(a));
+            put(a, vb);
         }
         __syncthreads();
-        const uint32_t cut = lo0 + smalls;
-        if (cut <= nth)
+        if (right_kept)
             first = cut;
         else
             last = cut;
@@ -351,7 +421,8 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
     };
     // (the rounds in device memory use no LDS of their own: the whole block holds the heap's upper levels if the
     // depth limit is reached here)
-    if (introselect_rounds(get, put, first, last, nth, depth, kSortMax, lsta, lstb, *L.sm, L.sortk, kDynLds / 8u))
+    if (introselect_rounds(get, [=](size_t i) { return key[i]; }, put, first, last, nth, depth, kSortMax, lsta, lstb, *L.sm, L.sortk,
+                           kDynLds / 8u))
         return;
     u64* lds = L.sortk;
     uint32_t* la = reinterpret_cast<uint32_t*>(L.sortk + kSortMax);
@@ -361,8 +432,8 @@ __device__ void nth_element_row(uint32_t* key, uint32_t* idx, uint32_t n, uint32
     for (uint32_t i = tid; i < len; i += kThreads)
         lds[i] = get(base + i);
     __syncthreads();
-    introselect_rounds([=](uint32_t i) { return lds[i - base]; }, [=](uint32_t i, u64 v) { lds[i - base] = v; }, first, last,
-                       nth, depth, 3u, la, lb, *L.sm, nullptr, 0u);
+    introselect_rounds([=](uint32_t i) { return lds[i - base]; }, [=](size_t i) { return (uint32_t)(lds[i - base] >> 32); },
+                       [=](uint32_t i, u64 v) { lds[i - base] = v; }, first, last, nth, depth, 3u, la, lb, *L.sm, nullptr, 0u);
     for (uint32_t i = tid; i < len; i += kThreads)
         put(base + i, lds[i]);
     __syncthreads();
