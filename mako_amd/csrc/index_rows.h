@@ -103,6 +103,25 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
                     if (elem_index<VEC>(lo, tid, 4u * b + c) < hi)
                         key0[elem_index<VEC>(lo, tid, 4u * b + c)] = k[c] ^ flip;
             }
+            if (VEC && !in_order) { // uniform
+                // the whole-row path's list as well, (~bits(q), token) at the token's position: it is the row's list
+                // of candidates when every logit turns out to be one, as the pieces' counts will tell.  (Not from
+                // the instances for rows that are loaded a logit at a time: they would need more registers than
+                // two workgroups on a CU have.)
+                uint32_t* lk = sc.key[0] + (size_t)row * sc.vpad;
+                uint32_t* li = sc.idx[0] + (size_t)row * sc.vpad;
+                if (base + 3u < hi) {
+                    *reinterpret_cast<uint4*>(lk + base) = make_uint4(~k[0], ~k[1], ~k[2], ~k[3]);
+                    *reinterpret_cast<uint4*>(li + base) = make_uint4(base, base + 1u, base + 2u, base + 3u);
+                } else {
+#pragma unroll
+                    for (uint32_t c = 0; c < 4; ++c)
+                        if (base + c < hi) {
+                            lk[base + c] = ~k[c];
+                            li[base + c] = base + c;
+                        }
+                }
+            }
         }
         // (four weights at a time: with all sixteen in flight the kernel needs twice the registers, and two workgroups
         // no longer share a CU)
@@ -147,6 +166,7 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
             plan->flag = kIndexClaimed;
             plan->m = m;
             plan->argidx = argidx;
+            plan->n0 = VEC && !in_order ? 1u : 0u; // (the whole-row path's list is there as well)
         }
     }
 }
@@ -283,7 +303,12 @@ __global__ __launch_bounds__(kThreads) void index_tail_kernel(mako_sample_desc d
         if (tid < 32)
             sm.tab[tid] = k_exp2_tab[tid];
         __syncthreads();
-        general_row_from_weights<0>(d, sc, row, s_args.P, argidx, L);
+        // (the pieces' counts of candidates: when every logit is one, index_weights_kernel's list is the row's list)
+        const uint32_t pieces = (d.n_vocab + kSliceMax - 1u) / kSliceMax;
+        uint32_t counted = 0;
+        for (uint32_t p = 0; p < pieces; ++p)
+            counted += sc.plan[row].cursor[p];
+        general_row_from_weights<0>(d, sc, row, s_args.P, argidx, sc.plan[row].n0 == 1u && uniform_u32(counted) == d.n_vocab, L);
         return;
     }
     if (flag != kIndexReady && flag != kIndexWhole && flag != kIndexEmpty) // (never)

@@ -697,13 +697,20 @@ __device__ MAKO_RARE_CALL void general_row(const mako_sample_desc& d, const Scra
 // its index and 0 elsewhere, as general_row()'s first sweep leaves it (index_weights_kernel writes the same array with a
 // workgroup per 16 384 logits instead of one for the row).  Counts and compacts the candidates in index order and goes
 // on like general_row().  All threads call; `argidx`: the row's first maximum, for a row without candidates.
+// `listed`: true when that kernel found every logit a candidate (no mask, no floor, no underflow: the usual row) and
+// has left the list itself as well, (~bits(q), i) at i in key[0] / idx[0] of the row: nothing to count or to compact.
 template <int SITE>
 __device__ MAKO_RARE_CALL void general_row_from_weights(const mako_sample_desc& d, const Scratch& sc, uint32_t row,
-                                                        const mako_sampling_params& P, uint32_t argidx, const FinishLds& L)
+                                                        const mako_sampling_params& P, uint32_t argidx, bool listed,
+                                                        const FinishLds& L)
 {
     assume_lds(L);
     FinishShared& sm = *L.sm;
     const uint32_t V = d.n_vocab;
+    if (listed) { // uniform
+        sort_truncate_draw<SITE == 0>(d, sc, row, P, V, false, 0.0, MAKO_PATH_GENERAL, L);
+        return;
+    }
     const uint32_t* qb = reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad);
     uint32_t* key0 = sc.key[0] + (size_t)row * sc.vpad;
     uint32_t* idx0 = sc.idx[0] + (size_t)row * sc.vpad;
