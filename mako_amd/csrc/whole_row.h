@@ -234,19 +234,23 @@ __device__ bool introselect_rounds(Get get, GetKey get_key, Put put, uint32_t& f
         --depth;
         if (tid == 0) { // __move_median_to_first(first, first + 1, mid, last - 1)
             const uint32_t ix = first + 1u, iy = first + (last - first) / 2u, iz = last - 1u;
-            const u64 x = get(ix), y = get(iy), z = get(iz);
+            const u64 x = get(ix), y = get(iy), z = get(iz), r = get(first); // (one trip to memory)
             uint32_t im;
-            if (x < y)
+            u64 med;
+            if (x < y) {
                 im = y < z ? iy : (x < z ? iz : ix);
-            else
+                med = y < z ? y : (x < z ? z : x);
+            } else {
                 im = x < z ? ix : (y < z ? iz : iy);
-            const u64 r = get(first), med = get(im);
+                med = x < z ? x : (y < z ? z : y);
+            }
             put(first, med);
             put(im, r);
-            sm.bs.bcast = 0; // the pairs that change places, counted below
+            sm.bs.f64[0] = __longlong_as_double((long long)med); // (the pivot, for everyone)
+            sm.bs.bcast = 0;                                     // the pairs that change places, counted below
         }
         __syncthreads();
-        const u64 pivot = get(first);
+        const u64 pivot = (u64)__double_as_longlong(sm.bs.f64[0]);
         const uint32_t lo0 = uniform_u32(first + 1u), last_s = uniform_u32(last), len = last_s - lo0; // (scalars, like all
                                                                                                       // of a wave's bounds and counts below)
         const uint32_t chunk = ((len + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
