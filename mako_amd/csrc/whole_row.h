@@ -502,7 +502,14 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
     const bool nth_order = TOPK_ALONE && topk_active && !topp_active;
     if (nth_order)
         nth_element_row(key0, idx0, n0, P.top_k, key1, idx1, L);
-    else if (topk_active || topp_active)
+    else if (topk_active) {
+        // a top-p follows: the survivors are sorted, so only which candidates they are matters, and `desc` is a total
+        // order: nth_element's first top_k entries are the top_k first of the sorted list, in some order.  The
+        // partitions and a sort of top_k entries cost a quarter of the sort of all candidates.
+        nth_element_row(key0, idx0, n0, P.top_k, key1, idx1, L);
+        sort_segment(idx0, key0, idx1, key1, P.top_k, L); // (stable sorts: token ids first, then the weights)
+        sort_segment(key0, idx0, key1, idx1, P.top_k, L);
+    } else if (topp_active)
         sort_segment(key0, idx0, key1, idx1, n0, L);
     const uint32_t *ks = key0, *is = idx0;
     MAKO_STAMP(12);
@@ -519,6 +526,7 @@ __device__ void sort_truncate_draw(const mako_sample_desc& d, const Scratch& sc,
             compact_candidates(reinterpret_cast<const uint32_t*>(sc.wbuf + (size_t)row * sc.vpad), d.n_vocab, key0, idx0, sm);
             nth_element_row(key0, idx0, n0, P.top_k, key1, idx1, L);
             total64 = reference_total([=](uint32_t i) { return __uint_as_float(~key0[i]); }, n1, sm);
+            sort_segment(idx0, key0, idx1, key1, n1, L); // (equal weights by token id, as in the list of all candidates)
             sort_segment(key0, idx0, key1, idx1, n1, L);
         } else {
             // index order: the row's bits(q) array (the zeros of the logits that are no candidates add nothing)

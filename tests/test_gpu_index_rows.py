@@ -182,6 +182,30 @@ def test_other_rows_of_the_whole_row_path_get_their_weights_there_too(gpu_ctx):
     assert np.array_equal(h["cand_idx"], g["cand_idx"])
 
 
+@pytest.mark.parametrize("vocab", [40000, 129280])
+def test_wide_top_k_before_a_top_p_with_many_equal_weights(gpu_ctx, vocab):
+    """A top-k beyond the candidate lists followed by a top-p: the library partitions the candidates as nth_element
+    does and sorts the survivors only.  With logits on a coarse grid many candidates share a weight, at the top-k's edge
+    and among the survivors: which of them survive, and their order (equal weights by token id), must be the
+    reference's, on rows with and without gaps in the list, with and without the host copy of the parameters."""
+    rng = np.random.Generator(np.random.PCG64([vocab, 97]))
+    rows = 24
+    logits = (np.round(rng.standard_normal((rows, vocab)) * 3.0 * 2.0) / 2.0).astype(np.float32)
+    logits[1::4] = (np.round(rng.standard_normal((rows // 4, vocab)) * 0.5 * 8.0) / 8.0).astype(np.float32)
+    logits[2::4, ::7] = -np.inf
+    p = workloads.make_params(rows, 1.0, 0, 1.0)
+    p["temperature"] = rng.choice(np.array([0.5, 1.0, 2.5], np.float32), rows)
+    p["top_k"] = rng.choice(np.array([129, 200, 1000, 5000, 20000], np.uint32), rows)
+    p["top_p"] = rng.choice(np.array([0.5, 0.9, 0.95, 0.999], np.float32), rows)
+    p["min_p"][::6] = np.float32(0.01)
+    u = workloads._uniforms(rng, rows)
+    w = dict(name="wide top-k, equal weights, V=%d" % vocab, logits=logits, params=p, u=u)
+    for hinted in (False, True):
+        _say("wide top-k before a top-p, V=%d hinted=%s" % (vocab, hinted))
+        g = assert_parity(gpu_ctx, w, cap=512, hinted=hinted)
+        assert (g["path"] == PATH_GENERAL).all()
+
+
 def test_verification_of_rows_in_token_order(gpu_ctx):
     """Sampler::verify (src/gen/sampler.cpp:86-107) on temperature-only rows: the draft's weight read off the list,
     the total by the chain of group maps, and for a rejected draft the walk over the list without it.  Drafts that
