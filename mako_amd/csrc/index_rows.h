@@ -166,7 +166,7 @@ __global__ __launch_bounds__(kThreads) void index_weights_kernel(mako_sample_des
             plan->flag = kIndexClaimed;
             plan->m = m;
             plan->argidx = argidx;
-            plan->n0 = VEC && !in_order ? 1u : 0u; // (the whole-row path's list is there as well)
+            plan->n0 = VEC && !in_order ? kIndexListed : 0u;
         }
     }
 }
@@ -308,7 +308,7 @@ __global__ __launch_bounds__(kThreads) void index_tail_kernel(mako_sample_desc d
         uint32_t counted = 0;
         for (uint32_t p = 0; p < pieces; ++p)
             counted += sc.plan[row].cursor[p];
-        general_row_from_weights<0>(d, sc, row, s_args.P, argidx, sc.plan[row].n0 == 1u && uniform_u32(counted) == d.n_vocab, L);
+        general_row_from_weights<0>(d, sc, row, s_args.P, argidx, sc.plan[row].n0 == kIndexListed && uniform_u32(counted) == d.n_vocab, L);
         return;
     }
     if (flag != kIndexReady && flag != kIndexWhole && flag != kIndexEmpty) // (never)

@@ -248,6 +248,9 @@ constexpr uint32_t kIndexClaimed = 6; // index_weights_kernel has the row: the k
 constexpr uint32_t kIndexReady = 7;   // the group records are in place
 constexpr uint32_t kIndexWhole = 8;   // the whole-row path is wanted (candidates to be written out from a list with gaps)
 constexpr uint32_t kIndexEmpty = 9;   // no candidate survived
+// (BigPlan::n0 of a claimed row of another kind, from index_weights_kernel to index_tail_kernel: the whole-row path's
+// list was written beside the weights, and is the row's list of candidates if every logit turns out to be one)
+constexpr uint32_t kIndexListed = 1;
 
 __device__ __forceinline__ bool penalties_neutral(const mako_sampling_params& p)
 {
