@@ -216,9 +216,10 @@ __device__ void heap_select_rest(Get get, Put put, uint32_t first, uint32_t last
 // The depth limit's heap select is heap_select_rest() above; the last insertion sort (at most three entries) is one
 // thread's.
 //
-// introselect_rounds runs the rounds on [first, last) through get(i) / get_key(i) (the high half alone) / put(i, v) until the range is no longer than
-// `until` (3 = to the end, insertion sort included).  lsta / lstb: room for last - first positions each.  cache /
-// cache_cap: LDS for heap_select_rest().  Returns true when nothing is left to do.
+// introselect_rounds runs the rounds on [first, last) through get(i) / get_key(i) (the high half alone) / put(i, v)
+// until the range is no longer than `until` (3 = to the end, insertion sort included).  lsta / lstb: room for
+// last - first positions each.  cache / cache_cap: LDS for heap_select_rest().  Returns true when nothing is left to
+// do.
 template <typename Get, typename GetKey, typename Put>
 __device__ bool introselect_rounds(Get get, GetKey get_key, Put put, uint32_t& first, uint32_t& last, uint32_t nth, uint32_t& depth,
                                    uint32_t until, uint32_t* lsta, uint32_t* lstb, FinishShared& sm,
@@ -251,8 +252,8 @@ __device__ bool introselect_rounds(Get get, GetKey get_key, Put put, uint32_t& f
         }
         __syncthreads();
         const u64 pivot = (u64)__double_as_longlong(sm.bs.f64[0]);
-        const uint32_t lo0 = uniform_u32(first + 1u), last_s = uniform_u32(last), len = last_s - lo0; // (scalars, like all
-                                                                                                      // of a wave's bounds and counts below)
+        // (scalars, like all of a wave's bounds and counts below)
+        const uint32_t lo0 = uniform_u32(first + 1u), last_s = uniform_u32(last), len = last_s - lo0;
         const uint32_t chunk = ((len + kThreads - 1u) / kThreads) * kWave; // per wave, a multiple of 64
         const uint32_t beg = uniform_u32(min(last_s, lo0 + wave * chunk)), end = min(last_s, beg + chunk);
         // entries of the wave's chunk that belong left of the cut
