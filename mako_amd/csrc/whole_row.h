@@ -279,19 +279,29 @@ __device__ bool introselect_rounds(Get get, GetKey get_key, Put put, uint32_t& f
                     ties |= __builtin_amdgcn_ballot_w64(k[u] == pivot_key);
                 }
             } else {
-#pragma unroll
-                for (uint32_t u = 0; u < kTrip; ++u)
-                    k[u] = get_key((size_t)min(base + u * kWave + lane, last_s - 1u));
+                // (the chunk's last trip: only its loads that reach into the chunk, which on the short ranges of the
+                // rounds in LDS is one in eight; scalar branches)
 #pragma unroll
                 for (uint32_t u = 0; u < kTrip; ++u) {
-                    in[u] = __builtin_amdgcn_ballot_w64(base + u * kWave + lane < end);
-                    left[u] = __builtin_amdgcn_ballot_w64(k[u] < pivot_key) & in[u];
-                    ties |= __builtin_amdgcn_ballot_w64(k[u] == pivot_key) & in[u];
+                    k[u] = 0u;
+                    if (base + u * kWave < end)
+                        k[u] = get_key((size_t)min(base + u * kWave + lane, last_s - 1u));
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < kTrip; ++u) {
+                    in[u] = left[u] = 0ull;
+                    if (base + u * kWave < end) {
+                        in[u] = __builtin_amdgcn_ballot_w64(base + u * kWave + lane < end);
+                        left[u] = __builtin_amdgcn_ballot_w64(k[u] < pivot_key) & in[u];
+                        ties |= __builtin_amdgcn_ballot_w64(k[u] == pivot_key) & in[u];
+                    }
                 }
             }
             if (ties) { // (rare)
 #pragma unroll
                 for (uint32_t u = 0; u < kTrip; ++u) {
+                    if (!in[u])
+                        continue;
                     const uint32_t pos = base + u * kWave + lane;
                     bool l = false;
                     if (pos < end && k[u] == pivot_key)
@@ -337,6 +347,8 @@ __device__ bool introselect_rounds(Get get, GetKey get_key, Put put, uint32_t& f
             if (base + kWave * kTrip <= cut) { // (uniform; all but one of the chunks' trips lie on one side of the cut)
 #pragma unroll
                 for (uint32_t u = 0; u < kTrip; ++u) {
+                    if (!in[u]) // (scalar: a trip's part beyond the chunk)
+                        continue;
                     const u64 big = in[u] & ~left[u];
                     if ((big >> lane) & 1ull)
                         lsta[big_before + rank_in(big)] = base + u * kWave + lane;
@@ -348,6 +360,8 @@ __device__ bool introselect_rounds(Get get, GetKey get_key, Put put, uint32_t& f
             } else if (base >= cut) {
 #pragma unroll
                 for (uint32_t u = 0; u < kTrip; ++u) {
+                    if (!left[u])
+                        continue;
                     if ((left[u] >> lane) & 1ull)
                         lstb[small_before + rank_in(left[u])] = base + u * kWave + lane;
                     small_before += (uint32_t)__popcll(left[u]);
@@ -355,6 +369,8 @@ __device__ bool introselect_rounds(Get get, GetKey get_key, Put put, uint32_t& f
             } else {
 #pragma unroll
                 for (uint32_t u = 0; u < kTrip; ++u) {
+                    if (!in[u])
+                        continue;
                     const uint32_t pos = base + u * kWave + lane;
                     const u64 big = in[u] & ~left[u];
                     const u64 before = __builtin_amdgcn_ballot_w64(pos < cut);
