@@ -307,13 +307,15 @@ def main():
 
     # BASELINE's two 256-row configurations, event-timed on the same stream with the logits rotated the same way and
     # their tokens checked against the reference CPU sampler (untimed): beside the headline value, never part of it.
-    # (And a batch of rows with a temperature only, what an API request without top_k / top_p asks for: no BASELINE
-    # configuration, but the kind of row that takes kernels of its own.)
+    # (And a batch of rows with a temperature only, what an API request without top_k / top_p asks for, and one of rows
+    # cut to a top-k without a top-p, whose survivors keep nth_element's order: no BASELINE configurations, but the
+    # kinds of row that take kernels of their own and the whole-row path.)
     others = None
     if a.workload == "config3" and a.other_steps > 0:
         others = {}
         ctx.close()
-        for key, name in (("config4", "config4"), ("config5_0.5", "config5"), ("temperature_only_64", "temperature_only_64")):
+        for key, name in (("config4", "config4"), ("config5_0.5", "config5"), ("temperature_only_64", "temperature_only_64"),
+                          ("topk_alone_64", "topk_alone_64")):
             others[key] = time_other(make_workload(name), a.other_steps, max(2, a.other_steps // 4), a.pool_mb, orc, stream)
 
     achieved = batch_bytes / (ms_per_step * 1e-3) / 1e9
