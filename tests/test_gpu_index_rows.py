@@ -182,12 +182,13 @@ def test_other_rows_of_the_whole_row_path_get_their_weights_there_too(gpu_ctx):
     assert np.array_equal(h["cand_idx"], g["cand_idx"])
 
 
-@pytest.mark.parametrize("vocab", [40000, 129280])
+@pytest.mark.parametrize("vocab", [4099, 40000, 129280])
 def test_wide_top_k_before_a_top_p_with_many_equal_weights(gpu_ctx, vocab):
     """A top-k beyond the candidate lists followed by a top-p: the library partitions the candidates as nth_element
     does and sorts the survivors only.  With logits on a coarse grid many candidates share a weight, at the top-k's edge
     and among the survivors: which of them survive, and their order (equal weights by token id), must be the
-    reference's, on rows with and without gaps in the list, with and without the host copy of the parameters."""
+    reference's, on rows with and without gaps in the list, with and without the host copy of the parameters, also
+    where the rows' length is no multiple of four (the weights kernel then leaves no list of its own)."""
     rng = np.random.Generator(np.random.PCG64([vocab, 97]))
     rows = 24
     logits = (np.round(rng.standard_normal((rows, vocab)) * 3.0 * 2.0) / 2.0).astype(np.float32)
@@ -197,6 +198,7 @@ def test_wide_top_k_before_a_top_p_with_many_equal_weights(gpu_ctx, vocab):
     p["temperature"] = rng.choice(np.array([0.5, 1.0, 2.5], np.float32), rows)
     p["top_k"] = rng.choice(np.array([129, 200, 1000, 5000, 20000], np.uint32), rows)
     p["top_p"] = rng.choice(np.array([0.5, 0.9, 0.95, 0.999], np.float32), rows)
+    p["top_p"][5::8] = 1.0  # (and a few rows whose survivors keep the partitions' order)
     p["min_p"][::6] = np.float32(0.01)
     u = workloads._uniforms(rng, rows)
     w = dict(name="wide top-k, equal weights, V=%d" % vocab, logits=logits, params=p, u=u)
